@@ -1,0 +1,188 @@
+/* lyraquant.h -- C ABI of the MI355X (gfx950) quantized-linear library `liblyraquant.so`.
+ *
+ * Every entry point enqueues HIP kernels on the caller's stream and returns immediately
+ * (stream-ordered, no implicit synchronisation, no host-side allocation unless stated).
+ * All pointers are DEVICE pointers unless the parameter name starts with `host_`.
+ * Return value: LQ_OK (0) or a negative lq_status_t; lq_last_error() gives the message of the
+ * last failure on the calling thread.  Nothing throws across this boundary.
+ *
+ * Each declaration cites the interface of the lyraDiff reference that it replaces
+ * (paths relative to the reference's src/lyradiff/).  The reference's C++ templates on
+ * T in {float, half, __nv_bfloat16} become an lq_dtype_t argument.
+ *
+ * Conventions: activations row-major [M,K]; weights row-major [N,K] before repacking; outputs
+ * row-major [M,N].  "rows32 layout" = the byte matrix [N, Kb] re-ordered as
+ * [N/32][Kb/16][32][16] (see lq_repack_rows32).
+ */
+#ifndef LYRAQUANT_H_
+#define LYRAQUANT_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* lq_stream_t; /* a hipStream_t; NULL selects the null stream */
+
+typedef enum { LQ_F32 = 0, LQ_F16 = 1, LQ_BF16 = 2, LQ_I32 = 3 } lq_dtype_t;
+
+typedef enum {
+    LQ_OK = 0,
+    LQ_ERR_ARG = -1,         /* null pointer, bad enum */
+    LQ_ERR_SHAPE = -2,       /* shape not supported by the kernels (message says which rule) */
+    LQ_ERR_HIP = -3,         /* a HIP runtime call failed */
+    LQ_ERR_UNSUPPORTED = -4  /* dtype combination not built */
+} lq_status_t;
+
+typedef enum { LQ_W_INT8 = 0, LQ_W_FP8 = 1, LQ_W_INT4 = 2 } lq_weight_kind_t;
+
+/* Message of the last failing call on this thread ("" if none).  No reference counterpart:
+ * the reference throws std::runtime_error / LyraException (utils/cuda_utils.h:128-147). */
+const char* lq_last_error(void);
+
+/* Library version, major*10000 + minor*100 + patch. */
+int lq_version(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * INT8 SmoothQuant activation quantisation
+ * ------------------------------------------------------------------------------------------- */
+
+/* q[r,k] = sat_s8(rne((f32(src[r,k]) * pre[k]) / s)), s = in_scale[0] or in_scale[r] when
+ * per_token != 0.  pre may be NULL (treated as all ones).
+ * Replaces invokeSqInputQuant<T> (kernels/quant_kernels/quant_kernels.h:8-17, kernels
+ * sqInputQuant / sqPerTokenInputQuant quant_kernels.cu:51-115); rows = batch_size*seq_len.
+ * Lifts the reference's limits (dim even; per-token only for dim <= 2048). */
+int lq_sq_input_quant(int8_t* dst, const void* src, lq_dtype_t src_dtype, const float* pre_quant_scale,
+                      const float* input_quant_scale, int per_token, size_t rows, size_t dim,
+                      lq_stream_t stream);
+
+/* Dynamic per-token variant: scale_out[r] = max_k|f32(src)*pre[k]| / 127 (1 when the row is all
+ * zero) and q as above with that scale, in one pass.  The reference has only the consumer of a
+ * per-token scale (quant_kernels.cu:93-115); the amax formula is that of its weight path
+ * (quant_kernels.cu:207). */
+int lq_sq_dynamic_quant(int8_t* dst, float* scale_out, const void* src, lq_dtype_t src_dtype,
+                        const float* pre_quant_scale, size_t rows, size_t dim, lq_stream_t stream);
+
+/* y[r,n] = T(f32(acc[r,n]) * s_in * s_w[n]).  Replaces invokeSqOutputDequant<T>
+ * (quant_kernels.h:19-28, quant_kernels.cu:117-171). */
+int lq_sq_output_dequant(void* dst, lq_dtype_t dst_dtype, const int32_t* src, const float* input_quant_scale,
+                         const float* weight_quant_scale, int per_token, size_t rows, size_t dim,
+                         lq_stream_t stream);
+
+/* Per-output-channel weight quantisation on device: w' = w/pre[k], scale_out[n] = max_k|w'|/127,
+ * q = sat_s8(rne(w'/scale)).  Replaces invokeGetINT8WeightScale<T> (quant_kernels.h:30-37,
+ * quant_kernels.cu:173-223,270-312).  Output q is plain row-major [d_out, d_in]. */
+int lq_int8_weight_quant(float* scale_out, int8_t* q_out, const void* weight, lq_dtype_t w_dtype,
+                         const float* pre_quant_scale, size_t d_out, size_t d_in, lq_stream_t stream);
+
+/* hidden [rows, 2*dim] -> q [rows, dim]:  h = x[:, :dim] + b[:dim]; g = gelu_tanh(x[:, dim:] + b[dim:]);
+ * q = sat_s8(rne(f32(h*g) * pre[k] / in_scale[0])); adds and products rounded to T as the
+ * reference does.  bias may be NULL.  Replaces invokeFusedAddBiasGegluInt8O<T>
+ * (kernels/quant_kernels/ffn_kernels_int8.h:12-21, ffn_kernels_int8.cu:102-237); lifts its
+ * dim in {1280,2560,5120} limit to any dim % 8 == 0.  T in {F16, BF16, F32}. */
+int lq_geglu_int8(int8_t* dst, const void* hidden, const void* bias, lq_dtype_t dtype,
+                  const float* pre_quant_scale, const float* input_quant_scale, size_t rows, size_t dim,
+                  lq_stream_t stream);
+
+/* Same with the dynamic per-token scale of lq_sq_dynamic_quant (scale_out[rows]). */
+int lq_geglu_int8_dynamic(int8_t* dst, float* scale_out, const void* hidden, const void* bias,
+                          lq_dtype_t dtype, const float* pre_quant_scale, size_t rows, size_t dim,
+                          lq_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * FP8 e4m3 (OCP e4m3fn) per-tensor quantisation
+ * ------------------------------------------------------------------------------------------- */
+
+/* *scale = max(*scale, max_i |f32(x_i)| / 448); the caller zero-initialises *scale, as the
+ * reference's callers do (utils/common_macro_def.h:68).  Replaces invokeGetFP8WeightScale<T>
+ * (kernels/lora/load_lora.h:30-31, load_lora.cu:16-23,48-54,108-112). */
+int lq_fp8_amax_scale(float* scale, const void* x, lq_dtype_t dtype, size_t n, lq_stream_t stream);
+
+/* dst[i] = e4m3_satfinite_rne(f32(src[i]) * (invert ? 1.0f/scale[0] : scale[0])).
+ * Replaces invokeCudaD2DScaleCpyConvert<T_IN, __nv_fp8_e4m3> (utils/memory_utils.cu:431-446). */
+int lq_fp8_scale_cast(uint8_t* dst, const void* src, lq_dtype_t dtype, const float* scale, int invert,
+                      size_t n, lq_stream_t stream);
+
+/* Dynamic per-tensor activation quant in one call: scale_out[0] = max|x|/448, then the cast
+ * above with invert = 1.  No single reference counterpart (its activation scales are static,
+ * layers/flux_attention_processor/FluxAttentionFP8Processor.cc:165-192); the two formulas are
+ * those of the two functions above.  Overwrites scale_out (no zero-init needed). */
+int lq_fp8_amax_cast(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t n,
+                     lq_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * W4A4 group-wise INT4 activation quantisation
+ * ------------------------------------------------------------------------------------------- */
+
+/* v = f32(x[m,k]) / smooth[k] (smooth may be NULL); scales[m,g] = max_{k in group g}|v| / 7;
+ * q = clamp(rne(v / scales[m,g]), -8, 7); q_words[m, k/8] packs 8 values per uint32, element i
+ * of the word in bits [4i, 4i+3].  scale_dtype F32 (as the reference stores) or F16 (scale is
+ * rounded to fp16 first and the rounded value quantises).  group must be 64, k % 64 == 0.
+ * Replaces the quantisation half of invokeFusedQuantizeAndLoraDownSimple
+ * (kernels/w4a4_gemm/w4a4_gemm.h:6-16, w4a4_gemm.cu:206-214,769-954) without the LoRA-down
+ * branch; lifts its m % 256 == 0 limit. */
+int lq_w4a4_quantize(uint32_t* q_words, void* scales, lq_dtype_t scale_dtype, const void* x,
+                     lq_dtype_t x_dtype, const float* smooth, int m, int k, int group, lq_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Offline weight repack (MFMA-friendly tiled layout)
+ * ------------------------------------------------------------------------------------------- */
+
+/* Bytes per weight row: k for INT8/FP8, k/2 for INT4. */
+size_t lq_weight_row_bytes(lq_weight_kind_t kind, size_t k);
+
+/* dst = rows32 layout of the row-major byte matrix src [n, row_bytes]:
+ *   dst[((nb*(row_bytes/16) + kc)*32 + r)*16 + b] = src[(nb*32 + r)*row_bytes + kc*16 + b].
+ * A pure permutation (same byte count); n % 32 == 0, row_bytes % 16 == 0; dst != src.
+ * Plays the role of preprocess_weights_for_mixed_gemm (kernels/cutlass_kernels/
+ * cutlass_preprocessors.cpp:484-530): one-time re-ordering of a quantized weight for the
+ * matrix-core operand layout -- here gfx950 MFMA instead of NVIDIA mma. */
+int lq_repack_rows32(uint8_t* dst, const uint8_t* src, size_t n, size_t row_bytes, lq_stream_t stream);
+
+/* Inverse permutation (for tests and for exporting a weight back to [N,K]). */
+int lq_unpack_rows32(uint8_t* dst, const uint8_t* src, size_t n, size_t row_bytes, lq_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Quantized GEMMs with fused dequant / bias / cast epilogue.  B is always the rows32 layout.
+ * ------------------------------------------------------------------------------------------- */
+
+/* C[m,n] = T( f32(sum_k A[m,k]*B[n,k]) * (alpha_col[n] * alpha_row[per_token ? m : 0]) [+ f32(bias[n])] )
+ * with an exact int32 accumulator.  out_dtype F16/BF16/F32, or I32 (raw accumulator; scales and
+ * bias ignored and may be NULL).  bias (nullable) has the output dtype.  n % 32 == 0, k % 64 == 0.
+ * Replaces CutlassInt8GemmRunner<T>::gemm (kernels/cutlass_kernels/int8_gemm/int8_gemm.h:16-90,
+ * int8_gemm_template.h:45-189,644-672) with EpilogueVisitorPerRowPerCol
+ * (kernels/cutlass_extensions/include/cutlass_extensions/epilogue/threadblock/
+ * epilogue_per_row_per_col_scale.h:239-305), as reached through cublasMMWrapper::runGemmInt8
+ * (utils/cublasMMWrapper.h:368-385); the bias add replaces the separate bias kernels that
+ * follow it (layers/basic_transformer/BasicTransformerInt8Block.cc:452,838). */
+int lq_gemm_int8(void* C, lq_dtype_t out_dtype, const int8_t* A, const int8_t* B_rows32,
+                 const float* alpha_col, const float* alpha_row, int per_token, const void* bias,
+                 int m, int n, int k, lq_stream_t stream);
+
+/* C[m,n] = T( act( (a_scale[0]*b_scale[0]) * sum_k A[m,k]*B[n,k] + f32(bias[n]) ) + beta*f32(residual[m,n]) )
+ * on e4m3 operands with fp32 accumulation; act = tanh-GELU when gelu != 0.  bias and residual are
+ * nullable and have the output dtype (F16/BF16/F32).  n % 32 == 0, k % 64 == 0.
+ * Replaces the FP8 overload of cublasMMWrapper::GemmWithResidualAndBias
+ * (utils/cublasMMWrapper.h:299-318, cublasMMWrapper.cc:1104-1274), whose (transa=T, weight as
+ * "A", m/n swapped) column-major call is this row-major product. */
+int lq_gemm_fp8(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32,
+                const float* a_scale, const float* b_scale, const void* bias, int gelu,
+                const void* residual, float beta, int m, int n, int k, lq_stream_t stream);
+
+/* C[m,n] = T( fold_{g=0..k/64-1} r = fmaf( f32(sum_{k in g} a*b) * sA[m,g], sB[n,g], r ) [+ f32(bias[n])] )
+ * on nibble-packed int4 operands (A: uint32 words [m, k/8]; B: rows32 layout of the byte matrix
+ * [n, k/2]), exact int32 group sums on the int8 MFMA.  Scales F32 or F16; out F16/BF16/F32.
+ * n % 32 == 0, k % 128 == 0, group == 64.
+ * Replaces the GEMM half of invokeFusedW4A4GemmAndLoraUp (kernels/w4a4_gemm/w4a4_gemm.h:18-30,
+ * w4a4_gemm.cu:227-512,665-767) without the LoRA-up branch; the bias add replaces invokeAddBias
+ * (layers/flux_attention_processor/FluxAttentionInt4Processor.cc:216-230). */
+int lq_gemm_w4a4(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const uint8_t* B_rows32,
+                 const void* sA, const void* sB, lq_dtype_t scale_dtype, const void* bias,
+                 int m, int n, int k, int group, lq_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LYRAQUANT_H_ */

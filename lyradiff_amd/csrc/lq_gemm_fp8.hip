@@ -1,0 +1,43 @@
+// FP8 e4m3 GEMM entry point (fp32 accumulation on v_mfma_f32_32x32x64_f8f6f4) with the fused
+// per-tensor scale, bias, optional tanh-GELU and residual epilogue.  Reference contract:
+// utils/cublasMMWrapper.cc:1104-1274 of lyraDiff (cuBLASLt FP8 matmul with A/B scale pointers and
+// BIAS / GELU_BIAS epilogues).
+#include "lq_gemm_core.h"
+
+namespace lq {
+
+template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
+    const long t256 = (long)((p.m + 255) / 256) * ((p.n + 255) / 256);
+    const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
+    if (t256 >= 192) return launch_gemm<K_FP8, OutTag, 256, 256, 64, 2, 4>(p, st);
+    if (t128 >= 192) return launch_gemm<K_FP8, OutTag, 128, 128, 64, 2, 2>(p, st);
+    return launch_gemm<K_FP8, OutTag, 64, 64, 64, 2, 2>(p, st);
+}
+
+}  // namespace lq
+
+using namespace lq;
+
+extern "C" int lq_gemm_fp8(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32,
+                           const float* a_scale, const float* b_scale, const void* bias, int gelu,
+                           const void* residual, float beta, int m, int n, int k, lq_stream_t stream) {
+    LQ_REQUIRE(C && A && B_rows32 && a_scale && b_scale, LQ_ERR_ARG, "lq_gemm_fp8: null pointer");
+    LQ_REQUIRE(m >= 0 && n > 0 && k > 0 && n % 32 == 0 && k % 64 == 0, LQ_ERR_SHAPE,
+               "lq_gemm_fp8: need n %% 32 == 0 and k %% 64 == 0 (m=%d n=%d k=%d)", m, n, k);
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B_rows32) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(C) % 16 == 0 && reinterpret_cast<uintptr_t>(bias) % 8 == 0 &&
+                   reinterpret_cast<uintptr_t>(residual) % 16 == 0,
+               LQ_ERR_ARG, "lq_gemm_fp8: A, B, C, residual must be 16-byte aligned and bias 8-byte aligned");
+    if (m == 0) return LQ_OK;
+    GemmParams p = {};
+    p.C = C; p.A = A; p.B = B_rows32; p.bias = bias; p.a_scale = a_scale; p.b_scale = b_scale;
+    p.gelu = gelu; p.residual = (beta != 0.0f) ? residual : nullptr; p.beta = beta;
+    p.m = m; p.n = n; p.k = k; p.kb = k;
+    hipStream_t st = as_stream(stream);
+    switch (out_dtype) {
+        case LQ_F16: return run_fp8<F16Tag>(p, st);
+        case LQ_BF16: return run_fp8<BF16Tag>(p, st);
+        case LQ_F32: return run_fp8<F32Tag>(p, st);
+        default: set_error("lq_gemm_fp8: unsupported output dtype %d", (int)out_dtype); return LQ_ERR_UNSUPPORTED;
+    }
+}

@@ -1,0 +1,47 @@
+// INT8 W8A8 GEMM entry point (exact int32 accumulation on v_mfma_i32_32x32x32_i8) with the fused
+// per-token x per-channel dequant (+ bias) epilogue.  Reference semantics:
+// kernels/cutlass_kernels/int8_gemm/int8_gemm_template.h:45-189 and
+// kernels/cutlass_extensions/.../epilogue_per_row_per_col_scale.h:239-305 of lyraDiff.
+#include "lq_gemm_core.h"
+
+namespace lq {
+
+template <typename OutTag> static int run_int8(GemmParams p, hipStream_t st) {
+    // static tile table in place of the reference's run-time tactic profiler
+    // (layers/gemm_utils/GemmProfiler.cc:78-127): largest tile that still fills the 256 CUs.
+    const long t256 = (long)((p.m + 255) / 256) * ((p.n + 255) / 256);
+    const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
+    if (t256 >= 192) return launch_gemm<K_INT8, OutTag, 256, 256, 64, 2, 4>(p, st);
+    if (t128 >= 192) return launch_gemm<K_INT8, OutTag, 128, 128, 64, 2, 2>(p, st);
+    return launch_gemm<K_INT8, OutTag, 64, 64, 64, 2, 2>(p, st);
+}
+
+}  // namespace lq
+
+using namespace lq;
+
+extern "C" int lq_gemm_int8(void* C, lq_dtype_t out_dtype, const int8_t* A, const int8_t* B_rows32,
+                            const float* alpha_col, const float* alpha_row, int per_token, const void* bias, int m,
+                            int n, int k, lq_stream_t stream) {
+    LQ_REQUIRE(C && A && B_rows32, LQ_ERR_ARG, "lq_gemm_int8: null pointer");
+    LQ_REQUIRE(out_dtype == LQ_I32 || (alpha_col && alpha_row), LQ_ERR_ARG, "lq_gemm_int8: scale pointers are required");
+    LQ_REQUIRE(m >= 0 && n > 0 && k > 0 && n % 32 == 0 && k % 64 == 0, LQ_ERR_SHAPE,
+               "lq_gemm_int8: need n %% 32 == 0 and k %% 64 == 0 (m=%d n=%d k=%d)", m, n, k);
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B_rows32) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(C) % 16 == 0 && reinterpret_cast<uintptr_t>(alpha_col) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(bias) % 8 == 0,
+               LQ_ERR_ARG, "lq_gemm_int8: A, B, C, alpha_col must be 16-byte aligned and bias 8-byte aligned");
+    if (m == 0) return LQ_OK;
+    GemmParams p = {};
+    p.C = C; p.A = reinterpret_cast<const uint8_t*>(A); p.B = reinterpret_cast<const uint8_t*>(B_rows32);
+    p.bias = bias; p.alpha_col = alpha_col; p.alpha_row = alpha_row; p.per_token = per_token;
+    p.m = m; p.n = n; p.k = k; p.kb = k;
+    hipStream_t st = as_stream(stream);
+    switch (out_dtype) {
+        case LQ_F16: return run_int8<F16Tag>(p, st);
+        case LQ_BF16: return run_int8<BF16Tag>(p, st);
+        case LQ_F32: return run_int8<F32Tag>(p, st);
+        case LQ_I32: p.bias = nullptr; return run_int8<I32Tag>(p, st);
+        default: set_error("lq_gemm_int8: unsupported output dtype %d", (int)out_dtype); return LQ_ERR_UNSUPPORTED;
+    }
+}

@@ -1,0 +1,43 @@
+// W4A4 (group-64 INT4 x INT4) GEMM entry point: nibbles widened to int8 in registers, exact
+// int32 group sums on v_mfma_i32_32x32x32_i8, fp32 group-scale accumulation in ascending group
+// order.  Reference semantics: kernels/w4a4_gemm/w4a4_gemm.cu:227-512 (group loop :473-506) of
+// lyraDiff, without the low-rank branch.
+#include "lq_gemm_core.h"
+
+namespace lq {
+
+template <typename OutTag> static int run_w4a4(GemmParams p, hipStream_t st) {
+    const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
+    if (t128 >= 192) return launch_gemm<K_W4A4, OutTag, 128, 128, 64, 2, 2>(p, st);
+    return launch_gemm<K_W4A4, OutTag, 64, 64, 64, 2, 2>(p, st);
+}
+
+}  // namespace lq
+
+using namespace lq;
+
+extern "C" int lq_gemm_w4a4(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const uint8_t* B_rows32,
+                            const void* sA, const void* sB, lq_dtype_t scale_dtype, const void* bias, int m, int n,
+                            int k, int group, lq_stream_t stream) {
+    LQ_REQUIRE(C && A_words && B_rows32 && sA && sB, LQ_ERR_ARG, "lq_gemm_w4a4: null pointer");
+    LQ_REQUIRE(group == 64, LQ_ERR_SHAPE, "lq_gemm_w4a4: group=%d, only 64 is supported", group);
+    LQ_REQUIRE(scale_dtype == LQ_F32 || scale_dtype == LQ_F16, LQ_ERR_UNSUPPORTED,
+               "lq_gemm_w4a4: scale dtype must be F32 or F16");
+    LQ_REQUIRE(m >= 0 && n > 0 && k > 0 && n % 32 == 0 && k % 128 == 0, LQ_ERR_SHAPE,
+               "lq_gemm_w4a4: need n %% 32 == 0 and k %% 128 == 0 (m=%d n=%d k=%d)", m, n, k);
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(A_words) % 16 == 0 && reinterpret_cast<uintptr_t>(B_rows32) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(C) % 16 == 0 && reinterpret_cast<uintptr_t>(bias) % 8 == 0,
+               LQ_ERR_ARG, "lq_gemm_w4a4: A, B, C must be 16-byte aligned and bias 8-byte aligned");
+    if (m == 0) return LQ_OK;
+    GemmParams p = {};
+    p.C = C; p.A = reinterpret_cast<const uint8_t*>(A_words); p.B = B_rows32; p.bias = bias;
+    p.sA = sA; p.sB = sB; p.scale_f16 = scale_dtype == LQ_F16;
+    p.m = m; p.n = n; p.k = k; p.kb = k / 2;
+    hipStream_t st = as_stream(stream);
+    switch (out_dtype) {
+        case LQ_F16: return run_w4a4<F16Tag>(p, st);
+        case LQ_BF16: return run_w4a4<BF16Tag>(p, st);
+        case LQ_F32: return run_w4a4<F32Tag>(p, st);
+        default: set_error("lq_gemm_w4a4: unsupported output dtype %d", (int)out_dtype); return LQ_ERR_UNSUPPORTED;
+    }
+}

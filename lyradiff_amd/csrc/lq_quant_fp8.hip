@@ -1,0 +1,196 @@
+// FP8 e4m3 (OCP e4m3fn on gfx950) per-tensor quantisation: amax -> scale, and scale-cast.
+//
+// Formulas follow the lyraDiff reference: kernels/lora/load_lora.cu:16-23,48-54 (scale =
+// max|x| / 448 through an integer-punned atomic max) and utils/memory_utils.cu:431-446
+// (dst = e4m3(float(src) * (invert ? 1/scale : scale)), saturating to +-448, RNE).
+// Unlike the reference (one atomic per element, 65 536 threads, byte stores) the amax kernel
+// reduces in registers -> wavefront shuffles -> LDS and issues one atomic per workgroup, and
+// the cast kernel moves 32 B in / 16 B out per lane per step.
+#include "lq_common.h"
+
+namespace lq {
+
+template <typename Tag> struct Chunk16 {  // 16 consecutive elements of a 16-bit type, or 8 of fp32
+    static constexpr int elems = Elem<Tag>::bytes == 2 ? 16 : 8;
+};
+
+template <typename Tag>
+__device__ __forceinline__ void load_elems(const void* base, size_t idx, float* o) {
+    if constexpr (Elem<Tag>::bytes == 2) {
+        const uint4* p = reinterpret_cast<const uint4*>(static_cast<const char*>(base) + idx * 2);
+        uint4 a = p[0], b = p[1];
+        unpack8<Tag>(a, o);
+        unpack8<Tag>(b, o + 8);
+    } else {
+        const float4* p = reinterpret_cast<const float4*>(static_cast<const char*>(base) + idx * 4);
+        float4 a = p[0], b = p[1];
+        o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+        o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+    }
+}
+template <typename Tag> __device__ __forceinline__ float load_one(const void* base, size_t idx) {
+    if constexpr (Elem<Tag>::bytes == 2) return Elem<Tag>::load(static_cast<const unsigned short*>(base)[idx]);
+    else return static_cast<const float*>(base)[idx];
+}
+
+// saturate-to-finite RNE conversion of two floats into the low or high half of a dword
+__device__ __forceinline__ u32 cvt2_e4m3(float a, float b, u32 old, bool hi) {
+    float ca = __builtin_amdgcn_fmed3f(a, 448.0f, -448.0f);
+    float cb = __builtin_amdgcn_fmed3f(b, 448.0f, -448.0f);
+    ca = (a != a) ? a : ca;  // keep NaN (-> 0x7F)
+    cb = (b != b) ? b : cb;
+    return hi ? (u32)__builtin_amdgcn_cvt_pk_fp8_f32(ca, cb, (int)old, true)
+              : (u32)__builtin_amdgcn_cvt_pk_fp8_f32(ca, cb, (int)old, false);
+}
+__device__ __forceinline__ u32 cvt4_e4m3(float a, float b, float c, float d) {
+    u32 w = cvt2_e4m3(a, b, 0u, false);
+    return cvt2_e4m3(c, d, w, true);
+}
+
+// Non-negative floats order like their bit patterns, so an integer atomic max works.  Thousands of
+// same-address atomics serialise in L2, so a workgroup first looks at the current value and only
+// issues the atomic when it would raise it (after the first few workgroups almost none do).
+__device__ __forceinline__ void publish_scale(float* scale, float v) {
+    int cur = __hip_atomic_load(reinterpret_cast<int*>(scale), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (__float_as_int(v) > cur) atomicMax(reinterpret_cast<int*>(scale), __float_as_int(v));
+}
+
+template <typename Tag>
+__global__ __launch_bounds__(256) void fp8_amax_kernel(float* __restrict__ scale, const void* __restrict__ x, size_t n) {
+    constexpr int E = Chunk16<Tag>::elems;
+    const size_t nchunks = n / E;
+    float amax = 0.0f;
+    for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < nchunks; c += (size_t)gridDim.x * blockDim.x) {
+        float v[16];
+        load_elems<Tag>(x, c * E, v);
+#pragma unroll
+        for (int i = 0; i < E; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    }
+    // tail elements (fewer than E) handled by the first threads of block 0
+    if (blockIdx.x == 0) {
+        size_t i = nchunks * E + threadIdx.x;
+        if (i < n) amax = fmaxf(amax, fabsf(load_one<Tag>(x, i)));
+    }
+    __shared__ float red[4];
+    amax = wave_max(amax);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        // non-negative floats order like their bit patterns
+        publish_scale(scale, amax / 448.0f);
+    }
+}
+
+template <typename Tag>
+__global__ __launch_bounds__(256) void fp8_cast_kernel(uint8_t* __restrict__ dst, const void* __restrict__ src,
+                                                       const float* __restrict__ scale, int invert, size_t n) {
+    constexpr int E = Chunk16<Tag>::elems;
+    const float s = scale[0];
+    const float r = invert ? 1.0f / s : s;
+    const size_t nchunks = n / E;
+    for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < nchunks; c += (size_t)gridDim.x * blockDim.x) {
+        float v[16];
+        load_elems<Tag>(src, c * E, v);
+        u32 w[4];
+#pragma unroll
+        for (int i = 0; i < E / 4; ++i)
+            w[i] = cvt4_e4m3(v[4 * i] * r, v[4 * i + 1] * r, v[4 * i + 2] * r, v[4 * i + 3] * r);
+        if constexpr (E == 16) *reinterpret_cast<uint4*>(dst + c * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+        else *reinterpret_cast<uint2*>(dst + c * 8) = make_uint2(w[0], w[1]);
+    }
+    if (blockIdx.x == 0) {
+        size_t i = nchunks * E + threadIdx.x;
+        if (i < n) dst[i] = (uint8_t)(cvt2_e4m3(load_one<Tag>(src, i) * r, 0.0f, 0u, false) & 0xFFu);
+    }
+}
+
+// scalar fallback for unaligned buffers
+template <typename Tag>
+__global__ __launch_bounds__(256) void fp8_cast_scalar_kernel(uint8_t* __restrict__ dst, const void* __restrict__ src,
+                                                              const float* __restrict__ scale, int invert, size_t n) {
+    const float s = scale[0];
+    const float r = invert ? 1.0f / s : s;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = (uint8_t)(cvt2_e4m3(load_one<Tag>(src, i) * r, 0.0f, 0u, false) & 0xFFu);
+}
+template <typename Tag>
+__global__ __launch_bounds__(256) void fp8_amax_scalar_kernel(float* __restrict__ scale, const void* __restrict__ x, size_t n) {
+    float amax = 0.0f;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        amax = fmaxf(amax, fabsf(load_one<Tag>(x, i)));
+    __shared__ float red[4];
+    amax = wave_max(amax);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        publish_scale(scale, amax / 448.0f);
+    }
+}
+
+__global__ void fill_f32_kernel(float* p, float v) { p[0] = v; }
+
+static unsigned stream_grid(size_t n, int elems_per_thread) {
+    size_t blocks = (n / elems_per_thread + 255) / 256;
+    const size_t cap = 256 * 8;  // 8 workgroups of 4 wavefronts per CU keep HBM busy
+    if (blocks > cap) blocks = cap;
+    if (blocks == 0) blocks = 1;
+    return (unsigned)blocks;
+}
+
+template <typename Tag> static int launch_amax(float* scale, const void* x, size_t n, hipStream_t st) {
+    if (reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+        hipLaunchKernelGGL((fp8_amax_kernel<Tag>), dim3(stream_grid(n, Chunk16<Tag>::elems)), dim3(256), 0, st, scale, x, n);
+    } else {
+        hipLaunchKernelGGL((fp8_amax_scalar_kernel<Tag>), dim3(stream_grid(n, 4)), dim3(256), 0, st, scale, x, n);
+    }
+    return check_launch("fp8_amax");
+}
+template <typename Tag>
+static int launch_cast(uint8_t* dst, const void* src, const float* scale, int invert, size_t n, hipStream_t st) {
+    if (reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0) {
+        hipLaunchKernelGGL((fp8_cast_kernel<Tag>), dim3(stream_grid(n, Chunk16<Tag>::elems)), dim3(256), 0, st, dst, src, scale, invert, n);
+    } else {
+        hipLaunchKernelGGL((fp8_cast_scalar_kernel<Tag>), dim3(stream_grid(n, 4)), dim3(256), 0, st, dst, src, scale, invert, n);
+    }
+    return check_launch("fp8_cast");
+}
+
+}  // namespace lq
+
+using namespace lq;
+
+extern "C" int lq_fp8_amax_scale(float* scale, const void* x, lq_dtype_t dtype, size_t n, lq_stream_t stream) {
+    LQ_REQUIRE(scale && (x || n == 0), LQ_ERR_ARG, "lq_fp8_amax_scale: null pointer");
+    if (n == 0) return LQ_OK;
+    switch (dtype) {
+        case LQ_F16: return launch_amax<F16Tag>(scale, x, n, as_stream(stream));
+        case LQ_BF16: return launch_amax<BF16Tag>(scale, x, n, as_stream(stream));
+        case LQ_F32: return launch_amax<F32Tag>(scale, x, n, as_stream(stream));
+        default: set_error("lq_fp8_amax_scale: unsupported dtype %d", (int)dtype); return LQ_ERR_UNSUPPORTED;
+    }
+}
+
+extern "C" int lq_fp8_scale_cast(uint8_t* dst, const void* src, lq_dtype_t dtype, const float* scale, int invert,
+                                 size_t n, lq_stream_t stream) {
+    LQ_REQUIRE(scale && ((dst && src) || n == 0), LQ_ERR_ARG, "lq_fp8_scale_cast: null pointer");
+    if (n == 0) return LQ_OK;
+    switch (dtype) {
+        case LQ_F16: return launch_cast<F16Tag>(dst, src, scale, invert, n, as_stream(stream));
+        case LQ_BF16: return launch_cast<BF16Tag>(dst, src, scale, invert, n, as_stream(stream));
+        case LQ_F32: return launch_cast<F32Tag>(dst, src, scale, invert, n, as_stream(stream));
+        default: set_error("lq_fp8_scale_cast: unsupported dtype %d", (int)dtype); return LQ_ERR_UNSUPPORTED;
+    }
+}
+
+extern "C" int lq_fp8_amax_cast(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t n,
+                                lq_stream_t stream) {
+    LQ_REQUIRE(scale_out && ((dst && src) || n == 0), LQ_ERR_ARG, "lq_fp8_amax_cast: null pointer");
+    hipLaunchKernelGGL(fill_f32_kernel, dim3(1), dim3(1), 0, as_stream(stream), scale_out, 0.0f);
+    int rc = check_launch("fp8_amax_cast(fill)");
+    if (rc != LQ_OK || n == 0) return rc;
+    rc = lq_fp8_amax_scale(scale_out, src, dtype, n, stream);
+    if (rc != LQ_OK) return rc;
+    return lq_fp8_scale_cast(dst, src, dtype, scale_out, 1, n, stream);
+}

@@ -1,0 +1,452 @@
+// INT8 SmoothQuant activation / weight quantisation kernels for gfx950.
+//
+// Row kernels: one 64-lane wavefront owns one row at a time and keeps the whole row in
+// registers (NP passes of 64 lanes x 8 elements), so the dynamic per-token variant reads the
+// activation from HBM exactly once: 128-bit loads, wavefront max by cross-lane shuffles,
+// 64-bit packed int8 stores.  The per-channel smoothing vector is loaded once per wavefront
+// and reused for all of its rows when it fits in registers.
+//
+// Formulas follow the lyraDiff reference: kernels/quant_kernels/quant_kernels.cu:51-115
+// (activation), :173-223 (weights), :117-171 (dequant), kernels/quant_kernels/
+// ffn_kernels_int8.cu:102-147 (bias + GEGLU), kernels/quant_kernels/int8_utils.cuh:23-28.
+#include "lq_common.h"
+
+namespace lq {
+
+// q = sat_s8(rne(t / s)) with the IEEE quotient, computed from r = 1/s whenever that provably
+// gives the same integer: |t*r - t/s| <= 1.5*2^-23*|t/s| and |fl(t/s) - t/s| <= 2^-24*|t/s|, so for
+// |t*r| < 512 both lie within 1e-4 of the true quotient; unless t*r is that close to a half
+// integer the two round to the same integer.  Beyond 512 both saturate.  Otherwise divide.
+__device__ __forceinline__ int quant_div_s8(float t, float s, float r, bool slow_row) {
+    float qa = t * r;
+    float fr = __builtin_amdgcn_fractf(qa);
+    bool risky = slow_row || (fabsf(fr - 0.5f) < 2e-4f && fabsf(qa) < 512.0f);
+    if (__builtin_expect(risky, 0)) qa = t / s;
+    return rne_sat_s8(qa);
+}
+__device__ __forceinline__ bool recip_unsafe(float s, float r) {
+    return !(fabsf(s) >= 1e-30f && fabsf(r) < 1e30f && fabsf(r) >= 1e-30f);
+}
+
+__device__ __forceinline__ u32 pack4_s8(int a, int b, int c, int d) {
+    return (u32)(a & 0xFF) | ((u32)(b & 0xFF) << 8) | ((u32)(c & 0xFF) << 16) | ((u32)d << 24);
+}
+
+// Load 8 consecutive elements (element offset `col` inside the row) as floats.
+template <typename Tag> __device__ __forceinline__ void load8(const void* row_base, int col, float* o) {
+    if constexpr (Elem<Tag>::bytes == 2) {
+        uint4 v = *reinterpret_cast<const uint4*>(static_cast<const char*>(row_base) + (size_t)col * 2);
+        unpack8<Tag>(v, o);
+    } else {
+        const float4* p = reinterpret_cast<const float4*>(static_cast<const char*>(row_base) + (size_t)col * 4);
+        float4 a = p[0], b = p[1];
+        o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+        o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+    }
+}
+
+// MODE 0: static per-tensor scale, 1: given per-token scale, 2: dynamic per-token scale.
+template <typename Tag, int NP, int MODE, bool PRE_REGS>
+__global__ __launch_bounds__(256) void sq_quant_rows_kernel(int8_t* __restrict__ dst,
+                                                            float* __restrict__ scale_out,
+                                                            const void* __restrict__ src,
+                                                            const float* __restrict__ pre,
+                                                            const float* __restrict__ in_scale,
+                                                            size_t rows, int dim) {
+    const int lane = threadIdx.x & 63;
+    const size_t wave = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const size_t nwaves = (size_t)gridDim.x * 4;
+    const size_t row_bytes = (size_t)dim * Elem<Tag>::bytes;
+
+    float pr[PRE_REGS ? NP : 1][8];
+    if constexpr (PRE_REGS) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            int col = (p * 64 + lane) * 8;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) pr[p][i] = 1.0f;
+            if (pre != nullptr && col < dim) load8<F32Tag>(pre, col, pr[p]);
+        }
+    }
+
+    for (size_t row = wave; row < rows; row += nwaves) {
+        const char* rb = static_cast<const char*>(src) + row * row_bytes;
+        float t[NP][8];
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            int col = (p * 64 + lane) * 8;
+            if (col < dim) {
+                load8<Tag>(rb, col, t[p]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) t[p][i] = 0.0f;
+            }
+        }
+        float amax = 0.0f;
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            int col = (p * 64 + lane) * 8;
+            if constexpr (PRE_REGS) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) t[p][i] = t[p][i] * pr[p][i];
+            } else {
+                if (pre != nullptr && col < dim) {
+                    float pv[8];
+                    load8<F32Tag>(pre, col, pv);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) t[p][i] = t[p][i] * pv[i];
+                }
+            }
+            if constexpr (MODE == 2) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(t[p][i]));
+            }
+        }
+        float s;
+        if constexpr (MODE == 2) {
+            amax = wave_max(amax);
+            s = (amax <= 5.9604644775390625e-08f) ? 1.0f : amax / 127.0f;
+            if (lane == 0) scale_out[row] = s;
+        } else if constexpr (MODE == 1) {
+            s = in_scale[row];
+        } else {
+            s = in_scale[0];
+        }
+        const float r = 1.0f / s;
+        const bool slow = recip_unsafe(s, r);
+        int8_t* ob = dst + row * (size_t)dim;
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            int col = (p * 64 + lane) * 8;
+            if (col < dim) {
+                int q[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) q[i] = quant_div_s8(t[p][i], s, r, slow);
+                uint2 o;
+                o.x = pack4_s8(q[0], q[1], q[2], q[3]);
+                o.y = pack4_s8(q[4], q[5], q[6], q[7]);
+                *reinterpret_cast<uint2*>(ob + col) = o;
+            }
+        }
+    }
+}
+
+// Generic (any dim, any alignment) fallback: one workgroup per row, scalar accesses.
+template <typename Tag, int MODE>
+__global__ __launch_bounds__(256) void sq_quant_generic_kernel(int8_t* __restrict__ dst, float* __restrict__ scale_out,
+                                                               const void* __restrict__ src,
+                                                               const float* __restrict__ pre,
+                                                               const float* __restrict__ in_scale, size_t rows,
+                                                               size_t dim) {
+    __shared__ float red[4];
+    for (size_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const char* rb = static_cast<const char*>(src) + row * dim * Elem<Tag>::bytes;
+        auto ld = [&](size_t c) -> float {
+            u32 bits;
+            if constexpr (Elem<Tag>::bytes == 2) bits = reinterpret_cast<const unsigned short*>(rb)[c];
+            else bits = reinterpret_cast<const u32*>(rb)[c];
+            float v = Elem<Tag>::load(bits);
+            return pre ? v * pre[c] : v;
+        };
+        float s;
+        if constexpr (MODE == 2) {
+            float amax = 0.0f;
+            for (size_t c = threadIdx.x; c < dim; c += blockDim.x) amax = fmaxf(amax, fabsf(ld(c)));
+            amax = wave_max(amax);
+            __syncthreads();
+            if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+            __syncthreads();
+            amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+            s = (amax <= 5.9604644775390625e-08f) ? 1.0f : amax / 127.0f;
+            if (threadIdx.x == 0) scale_out[row] = s;
+        } else if constexpr (MODE == 1) {
+            s = in_scale[row];
+        } else {
+            s = in_scale[0];
+        }
+        for (size_t c = threadIdx.x; c < dim; c += blockDim.x) dst[row * dim + c] = (int8_t)rne_sat_s8(ld(c) / s);
+    }
+}
+
+template <typename Tag, int MODE>
+static int launch_sq_quant(int8_t* dst, float* scale_out, const void* src, const float* pre, const float* in_scale,
+                           size_t rows, size_t dim, hipStream_t st) {
+    const bool fast = (dim % 8 == 0) && dim <= 16384 && (reinterpret_cast<uintptr_t>(src) % 16 == 0) &&
+                      (reinterpret_cast<uintptr_t>(dst) % 8 == 0) &&
+                      (pre == nullptr || reinterpret_cast<uintptr_t>(pre) % 16 == 0);
+    if (!fast) {
+        unsigned grid = (unsigned)(rows < 65536 ? rows : 65536);
+        hipLaunchKernelGGL((sq_quant_generic_kernel<Tag, MODE>), dim3(grid), dim3(256), 0, st, dst, scale_out, src, pre,
+                           in_scale, rows, dim);
+        return check_launch("sq_quant_generic");
+    }
+    const int np = (int)((dim + 511) / 512);
+    // each wavefront walks several rows so that the smoothing vector is fetched once per wavefront
+    size_t blocks = (rows + 3) / 4;
+    const size_t max_blocks = 256 * 8;
+    if (blocks > max_blocks) blocks = max_blocks;
+    dim3 grid((unsigned)blocks), block(256);
+    int d = (int)dim;
+#define LQ_SQ_CASE(NPV, PREREG)                                                                                  \
+    hipLaunchKernelGGL((sq_quant_rows_kernel<Tag, NPV, MODE, PREREG>), grid, block, 0, st, dst, scale_out, src, pre, \
+                       in_scale, rows, d)
+    if (np <= 1) LQ_SQ_CASE(1, true);
+    else if (np <= 2) LQ_SQ_CASE(2, true);
+    else if (np <= 3) LQ_SQ_CASE(3, true);
+    else if (np <= 4) LQ_SQ_CASE(4, true);
+    else if (np <= 6) LQ_SQ_CASE(6, true);
+    else if (np <= 8) LQ_SQ_CASE(8, true);
+    else if (np <= 12) LQ_SQ_CASE(12, false);
+    else if (np <= 16) LQ_SQ_CASE(16, false);
+    else if (np <= 24) LQ_SQ_CASE(24, false);
+    else LQ_SQ_CASE(32, false);
+#undef LQ_SQ_CASE
+    return check_launch("sq_quant_rows");
+}
+
+template <int MODE>
+static int dispatch_sq_quant(int8_t* dst, float* scale_out, const void* src, lq_dtype_t dt, const float* pre,
+                             const float* in_scale, size_t rows, size_t dim, hipStream_t st) {
+    switch (dt) {
+        case LQ_F16: return launch_sq_quant<F16Tag, MODE>(dst, scale_out, src, pre, in_scale, rows, dim, st);
+        case LQ_BF16: return launch_sq_quant<BF16Tag, MODE>(dst, scale_out, src, pre, in_scale, rows, dim, st);
+        case LQ_F32: return launch_sq_quant<F32Tag, MODE>(dst, scale_out, src, pre, in_scale, rows, dim, st);
+        default: set_error("sq_quant: unsupported source dtype %d", (int)dt); return LQ_ERR_UNSUPPORTED;
+    }
+}
+
+// ---- unfused dequant (quant_kernels.cu:117-171) -------------------------------------------------
+template <typename Tag, bool PER_TOKEN>
+__global__ __launch_bounds__(256) void sq_dequant_kernel(void* __restrict__ dst, const int32_t* __restrict__ src,
+                                                         const float* __restrict__ in_scale,
+                                                         const float* __restrict__ w_scale, size_t rows, size_t dim) {
+    size_t total = rows * dim;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        size_t r = i / dim, c = i - r * dim;
+        float y = ((float)src[i] * in_scale[PER_TOKEN ? r : 0]) * w_scale[c];
+        u32 b = Elem<Tag>::store(y);
+        if constexpr (Elem<Tag>::bytes == 2) static_cast<unsigned short*>(dst)[i] = (unsigned short)b;
+        else static_cast<u32*>(dst)[i] = b;
+    }
+}
+
+// ---- per-output-channel weight quantisation (quant_kernels.cu:173-223) -----------------------------
+template <typename Tag>
+__global__ __launch_bounds__(256) void int8_weight_quant_kernel(float* __restrict__ scale_out, int8_t* __restrict__ q,
+                                                                const void* __restrict__ w,
+                                                                const float* __restrict__ pre, size_t d_out,
+                                                                size_t d_in) {
+    __shared__ float red[4];
+    for (size_t row = blockIdx.x; row < d_out; row += gridDim.x) {
+        const char* rb = static_cast<const char*>(w) + row * d_in * Elem<Tag>::bytes;
+        auto ld = [&](size_t c) -> float {
+            u32 bits;
+            if constexpr (Elem<Tag>::bytes == 2) bits = reinterpret_cast<const unsigned short*>(rb)[c];
+            else bits = reinterpret_cast<const u32*>(rb)[c];
+            float v = Elem<Tag>::load(bits);
+            return pre ? v / pre[c] : v;
+        };
+        float amax = 0.0f;
+        for (size_t c = threadIdx.x; c < d_in; c += blockDim.x) amax = fmaxf(amax, fabsf(ld(c)));
+        amax = wave_max(amax);
+        __syncthreads();
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+        __syncthreads();
+        amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        float s = amax / 127.0f;
+        if (threadIdx.x == 0) scale_out[row] = s;
+        for (size_t c = threadIdx.x; c < d_in; c += blockDim.x) q[row * d_in + c] = (int8_t)rne_sat_s8(ld(c) / s);
+    }
+}
+
+// ---- bias + GEGLU -> INT8 (ffn_kernels_int8.cu:102-147) ----------------------------------------------
+// One wavefront per row; the row of `dim` products h*g stays in registers (NP passes of 512).
+template <typename Tag, int NP, bool DYNAMIC>
+__global__ __launch_bounds__(256) void geglu_int8_kernel(int8_t* __restrict__ dst, float* __restrict__ scale_out,
+                                                         const void* __restrict__ hidden,
+                                                         const void* __restrict__ bias,
+                                                         const float* __restrict__ pre,
+                                                         const float* __restrict__ in_scale, size_t rows, int dim) {
+    const int lane = threadIdx.x & 63;
+    const size_t wave = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const size_t nwaves = (size_t)gridDim.x * 4;
+    for (size_t row = wave; row < rows; row += nwaves) {
+        const char* rb = static_cast<const char*>(hidden) + row * (size_t)dim * 2 * Elem<Tag>::bytes;
+        float t[NP][8];
+        float amax = 0.0f;
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            int col = (p * 64 + lane) * 8;
+            if (col < dim) {
+                float h[8], g[8], pv[8];
+                load8<Tag>(rb, col, h);
+                load8<Tag>(rb, col + dim, g);
+                if (bias != nullptr) {
+                    float bh[8], bg[8];
+                    load8<Tag>(bias, col, bh);
+                    load8<Tag>(bias, col + dim, bg);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        h[i] = round_through<Tag>(h[i] + bh[i]);
+                        g[i] = round_through<Tag>(g[i] + bg[i]);
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) pv[i] = 1.0f;
+                if (pre != nullptr) load8<F32Tag>(pre, col, pv);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    float cube = round_through<Tag>(g[i] * round_through<Tag>(g[i] * g[i]));
+                    float cdf = 0.5f * (1.0f + tanh_basic(0.7978845608028654f * (g[i] + 0.044715f * cube)));
+                    float gel = round_through<Tag>(g[i] * round_through<Tag>(cdf));
+                    float prod = round_through<Tag>(h[i] * gel);
+                    t[p][i] = prod * pv[i];
+                    amax = fmaxf(amax, fabsf(t[p][i]));
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) t[p][i] = 0.0f;
+            }
+        }
+        float s;
+        if constexpr (DYNAMIC) {
+            amax = wave_max(amax);
+            s = (amax <= 5.9604644775390625e-08f) ? 1.0f : amax / 127.0f;
+            if (lane == 0) scale_out[row] = s;
+        } else {
+            s = in_scale[0];
+        }
+        const float r = 1.0f / s;
+        const bool slow = recip_unsafe(s, r);
+        int8_t* ob = dst + row * (size_t)dim;
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            int col = (p * 64 + lane) * 8;
+            if (col < dim) {
+                int q[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) q[i] = quant_div_s8(t[p][i], s, r, slow);
+                uint2 o;
+                o.x = pack4_s8(q[0], q[1], q[2], q[3]);
+                o.y = pack4_s8(q[4], q[5], q[6], q[7]);
+                *reinterpret_cast<uint2*>(ob + col) = o;
+            }
+        }
+    }
+}
+
+template <typename Tag, bool DYNAMIC>
+static int launch_geglu(int8_t* dst, float* scale_out, const void* hidden, const void* bias, const float* pre,
+                        const float* in_scale, size_t rows, size_t dim, hipStream_t st) {
+    LQ_REQUIRE(dim % 8 == 0 && dim <= 8192, LQ_ERR_SHAPE, "geglu_int8: dim=%zu must be a multiple of 8 and <= 8192", dim);
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(hidden) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 8 == 0 &&
+                   (bias == nullptr || reinterpret_cast<uintptr_t>(bias) % 16 == 0) &&
+                   (pre == nullptr || reinterpret_cast<uintptr_t>(pre) % 16 == 0),
+               LQ_ERR_ARG, "geglu_int8: pointers must be 16-byte aligned");
+    const int np = (int)((dim + 511) / 512);
+    size_t blocks = (rows + 3) / 4;
+    dim3 grid((unsigned)(blocks < 65535 ? blocks : 65535)), block(256);
+    int d = (int)dim;
+#define LQ_GG_CASE(NPV) \
+    hipLaunchKernelGGL((geglu_int8_kernel<Tag, NPV, DYNAMIC>), grid, block, 0, st, dst, scale_out, hidden, bias, pre, in_scale, rows, d)
+    if (np <= 2) LQ_GG_CASE(2);
+    else if (np <= 3) LQ_GG_CASE(3);
+    else if (np <= 5) LQ_GG_CASE(5);
+    else if (np <= 10) LQ_GG_CASE(10);
+    else LQ_GG_CASE(16);
+#undef LQ_GG_CASE
+    return check_launch("geglu_int8");
+}
+
+template <bool DYNAMIC>
+static int dispatch_geglu(int8_t* dst, float* scale_out, const void* hidden, const void* bias, lq_dtype_t dt,
+                          const float* pre, const float* in_scale, size_t rows, size_t dim, hipStream_t st) {
+    switch (dt) {
+        case LQ_F16: return launch_geglu<F16Tag, DYNAMIC>(dst, scale_out, hidden, bias, pre, in_scale, rows, dim, st);
+        case LQ_BF16: return launch_geglu<BF16Tag, DYNAMIC>(dst, scale_out, hidden, bias, pre, in_scale, rows, dim, st);
+        case LQ_F32: return launch_geglu<F32Tag, DYNAMIC>(dst, scale_out, hidden, bias, pre, in_scale, rows, dim, st);
+        default: set_error("geglu_int8: unsupported dtype %d", (int)dt); return LQ_ERR_UNSUPPORTED;
+    }
+}
+
+}  // namespace lq
+
+using namespace lq;
+
+extern "C" int lq_sq_input_quant(int8_t* dst, const void* src, lq_dtype_t src_dtype, const float* pre_quant_scale,
+                                 const float* input_quant_scale, int per_token, size_t rows, size_t dim,
+                                 lq_stream_t stream) {
+    LQ_REQUIRE(dst && src && input_quant_scale, LQ_ERR_ARG, "lq_sq_input_quant: null pointer");
+    if (rows == 0 || dim == 0) return LQ_OK;
+    if (per_token)
+        return dispatch_sq_quant<1>(dst, nullptr, src, src_dtype, pre_quant_scale, input_quant_scale, rows, dim,
+                                    as_stream(stream));
+    return dispatch_sq_quant<0>(dst, nullptr, src, src_dtype, pre_quant_scale, input_quant_scale, rows, dim,
+                                as_stream(stream));
+}
+
+extern "C" int lq_sq_dynamic_quant(int8_t* dst, float* scale_out, const void* src, lq_dtype_t src_dtype,
+                                   const float* pre_quant_scale, size_t rows, size_t dim, lq_stream_t stream) {
+    LQ_REQUIRE(dst && src && scale_out, LQ_ERR_ARG, "lq_sq_dynamic_quant: null pointer");
+    if (rows == 0) return LQ_OK;
+    LQ_REQUIRE(dim > 0, LQ_ERR_SHAPE, "lq_sq_dynamic_quant: dim must be positive");
+    return dispatch_sq_quant<2>(dst, scale_out, src, src_dtype, pre_quant_scale, nullptr, rows, dim, as_stream(stream));
+}
+
+extern "C" int lq_sq_output_dequant(void* dst, lq_dtype_t dst_dtype, const int32_t* src, const float* input_quant_scale,
+                                    const float* weight_quant_scale, int per_token, size_t rows, size_t dim,
+                                    lq_stream_t stream) {
+    LQ_REQUIRE(dst && src && input_quant_scale && weight_quant_scale, LQ_ERR_ARG, "lq_sq_output_dequant: null pointer");
+    if (rows == 0 || dim == 0) return LQ_OK;
+    size_t total = rows * dim;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    dim3 grid((unsigned)blocks), block(256);
+    hipStream_t st = as_stream(stream);
+#define LQ_DQ(TAG)                                                                                                    \
+    if (per_token) hipLaunchKernelGGL((sq_dequant_kernel<TAG, true>), grid, block, 0, st, dst, src, input_quant_scale, \
+                                      weight_quant_scale, rows, dim);                                                 \
+    else hipLaunchKernelGGL((sq_dequant_kernel<TAG, false>), grid, block, 0, st, dst, src, input_quant_scale,          \
+                            weight_quant_scale, rows, dim)
+    switch (dst_dtype) {
+        case LQ_F16: LQ_DQ(F16Tag); break;
+        case LQ_BF16: LQ_DQ(BF16Tag); break;
+        case LQ_F32: LQ_DQ(F32Tag); break;
+        default: set_error("lq_sq_output_dequant: unsupported dtype %d", (int)dst_dtype); return LQ_ERR_UNSUPPORTED;
+    }
+#undef LQ_DQ
+    return check_launch("sq_output_dequant");
+}
+
+extern "C" int lq_int8_weight_quant(float* scale_out, int8_t* q_out, const void* weight, lq_dtype_t w_dtype,
+                                    const float* pre_quant_scale, size_t d_out, size_t d_in, lq_stream_t stream) {
+    LQ_REQUIRE(scale_out && q_out && weight, LQ_ERR_ARG, "lq_int8_weight_quant: null pointer");
+    if (d_out == 0 || d_in == 0) return LQ_OK;
+    dim3 grid((unsigned)(d_out < 65535 ? d_out : 65535)), block(256);
+    hipStream_t st = as_stream(stream);
+    switch (w_dtype) {
+        case LQ_F16: hipLaunchKernelGGL((int8_weight_quant_kernel<F16Tag>), grid, block, 0, st, scale_out, q_out, weight, pre_quant_scale, d_out, d_in); break;
+        case LQ_BF16: hipLaunchKernelGGL((int8_weight_quant_kernel<BF16Tag>), grid, block, 0, st, scale_out, q_out, weight, pre_quant_scale, d_out, d_in); break;
+        case LQ_F32: hipLaunchKernelGGL((int8_weight_quant_kernel<F32Tag>), grid, block, 0, st, scale_out, q_out, weight, pre_quant_scale, d_out, d_in); break;
+        default: set_error("lq_int8_weight_quant: unsupported dtype %d", (int)w_dtype); return LQ_ERR_UNSUPPORTED;
+    }
+    return check_launch("int8_weight_quant");
+}
+
+extern "C" int lq_geglu_int8(int8_t* dst, const void* hidden, const void* bias, lq_dtype_t dtype,
+                             const float* pre_quant_scale, const float* input_quant_scale, size_t rows, size_t dim,
+                             lq_stream_t stream) {
+    LQ_REQUIRE(dst && hidden && input_quant_scale, LQ_ERR_ARG, "lq_geglu_int8: null pointer");
+    if (rows == 0) return LQ_OK;
+    return dispatch_geglu<false>(dst, nullptr, hidden, bias, dtype, pre_quant_scale, input_quant_scale, rows, dim,
+                                 as_stream(stream));
+}
+
+extern "C" int lq_geglu_int8_dynamic(int8_t* dst, float* scale_out, const void* hidden, const void* bias,
+                                     lq_dtype_t dtype, const float* pre_quant_scale, size_t rows, size_t dim,
+                                     lq_stream_t stream) {
+    LQ_REQUIRE(dst && hidden && scale_out, LQ_ERR_ARG, "lq_geglu_int8_dynamic: null pointer");
+    if (rows == 0) return LQ_OK;
+    return dispatch_geglu<true>(dst, scale_out, hidden, bias, dtype, pre_quant_scale, nullptr, rows, dim,
+                                as_stream(stream));
+}

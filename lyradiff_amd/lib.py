@@ -1,0 +1,66 @@
+"""ctypes binding of liblyraquant.so (the C ABI declared in include/lyraquant.h).
+
+The library is the product; this module only loads it and declares argument types.  There is
+no CPU fallback: if the shared library is missing, import of the ops fails with a clear error.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.environ.get("LYRA_LIB_PATH_AMD", os.path.join(PKG, "liblyraquant.so"))
+
+LQ_F32, LQ_F16, LQ_BF16, LQ_I32 = 0, 1, 2, 3
+LQ_W_INT8, LQ_W_FP8, LQ_W_INT4 = 0, 1, 2
+
+# every symbol include/lyraquant.h declares: name -> (restype, argtypes)
+_P, _I, _Z, _F = C.c_void_p, C.c_int, C.c_size_t, C.c_float
+SYMBOLS = {
+    "lq_last_error": (C.c_char_p, []),
+    "lq_version": (_I, []),
+    "lq_sq_input_quant": (_I, [_P, _P, _I, _P, _P, _I, _Z, _Z, _P]),
+    "lq_sq_dynamic_quant": (_I, [_P, _P, _P, _I, _P, _Z, _Z, _P]),
+    "lq_sq_output_dequant": (_I, [_P, _I, _P, _P, _P, _I, _Z, _Z, _P]),
+    "lq_int8_weight_quant": (_I, [_P, _P, _P, _I, _P, _Z, _Z, _P]),
+    "lq_geglu_int8": (_I, [_P, _P, _P, _I, _P, _P, _Z, _Z, _P]),
+    "lq_geglu_int8_dynamic": (_I, [_P, _P, _P, _P, _I, _P, _Z, _Z, _P]),
+    "lq_fp8_amax_scale": (_I, [_P, _P, _I, _Z, _P]),
+    "lq_fp8_scale_cast": (_I, [_P, _P, _I, _P, _I, _Z, _P]),
+    "lq_fp8_amax_cast": (_I, [_P, _P, _P, _I, _Z, _P]),
+    "lq_w4a4_quantize": (_I, [_P, _P, _I, _P, _I, _P, _I, _I, _I, _P]),
+    "lq_weight_row_bytes": (_Z, [_I, _Z]),
+    "lq_repack_rows32": (_I, [_P, _P, _Z, _Z, _P]),
+    "lq_unpack_rows32": (_I, [_P, _P, _Z, _Z, _P]),
+    "lq_gemm_int8": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _P]),
+    "lq_gemm_fp8": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _P, _F, _I, _I, _I, _P]),
+    "lq_gemm_w4a4": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P]),
+}
+
+_lib = None
+
+
+class LyraQuantError(RuntimeError):
+    """Raised when an lq_* call returns a negative status (message from lq_last_error())."""
+
+
+def load() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} not found: build it with `python -m lyradiff_amd.build` "
+                "(hipcc, gfx950). There is no CPU fallback for the quantized-linear path.")
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        msg = load().lq_last_error().decode("utf-8", "replace")
+        raise LyraQuantError(f"[lyradiff Error][{what}] status {status}: {msg}")

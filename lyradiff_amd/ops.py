@@ -1,0 +1,268 @@
+"""Tensor-level Python wrapper over the C ABI (PyTorch-ROCm supplies device memory and streams).
+
+Checks follow the reference's torch binding conventions (CHECK_TH_CUDA / CHECK_CONTIGUOUS /
+dtype TORCH_CHECK, src/lyradiff/th_op/th_utils.h:14-33): inputs must be contiguous device
+tensors of the stated dtype; outputs are allocated with torch.empty on the input's device;
+work is enqueued on the current stream.  The same functions are registered as
+torch.ops.lyradiff.* (see _register_torch_ops).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import lib as _l
+
+_DT = {torch.float32: _l.LQ_F32, torch.float16: _l.LQ_F16, torch.bfloat16: _l.LQ_BF16, torch.int32: _l.LQ_I32}
+
+
+def _chk(t: torch.Tensor, name: str, dtypes=None) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a CUDA(HIP) tensor")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if dtypes is not None and t.dtype not in dtypes:
+        raise TypeError(f"{name} has dtype {t.dtype}, expected one of {dtypes}")
+    return t
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+_FLOATS = (torch.float32, torch.float16, torch.bfloat16)
+
+
+# ---- INT8 SmoothQuant ---------------------------------------------------------------------------
+
+def sq_quant(x, pre_quant_scale, input_quant_scale, per_token: bool = False):
+    """invokeSqInputQuant: x [..., K] -> int8 [..., K] with a static (or given per-token) scale."""
+    _chk(x, "x", _FLOATS)
+    _chk(input_quant_scale, "input_quant_scale", (torch.float32,))
+    if pre_quant_scale is not None:
+        _chk(pre_quant_scale, "pre_quant_scale", (torch.float32,))
+        if pre_quant_scale.numel() != x.shape[-1]:
+            raise ValueError("pre_quant_scale must have K elements")
+    k = x.shape[-1]
+    rows = x.numel() // k if k else 0
+    if per_token and input_quant_scale.numel() != rows:
+        raise ValueError("per-token input_quant_scale must have one element per row")
+    q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    _l.check(_l.load().lq_sq_input_quant(_ptr(q), _ptr(x), _DT[x.dtype], _ptr(pre_quant_scale),
+                                         _ptr(input_quant_scale), int(per_token), rows, k, _stream()),
+             "lq_sq_input_quant")
+    return q
+
+
+def sq_quant_dynamic(x, pre_quant_scale=None):
+    """Dynamic per-token SmoothQuant: returns (q int8 [..., K], scale fp32 [rows])."""
+    _chk(x, "x", _FLOATS)
+    if pre_quant_scale is not None:
+        _chk(pre_quant_scale, "pre_quant_scale", (torch.float32,))
+        if pre_quant_scale.numel() != x.shape[-1]:
+            raise ValueError("pre_quant_scale must have K elements")
+    k = x.shape[-1]
+    rows = x.numel() // k if k else 0
+    q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    s = torch.empty(rows, dtype=torch.float32, device=x.device)
+    _l.check(_l.load().lq_sq_dynamic_quant(_ptr(q), _ptr(s), _ptr(x), _DT[x.dtype], _ptr(pre_quant_scale),
+                                           rows, k, _stream()), "lq_sq_dynamic_quant")
+    return q, s
+
+
+def sq_dequant(acc, input_quant_scale, weight_quant_scale, per_token: bool = False, out_dtype=torch.float16):
+    """invokeSqOutputDequant: int32 [M,N] -> T [M,N]."""
+    _chk(acc, "acc", (torch.int32,))
+    _chk(input_quant_scale, "input_quant_scale", (torch.float32,))
+    _chk(weight_quant_scale, "weight_quant_scale", (torch.float32,))
+    n = acc.shape[-1]
+    rows = acc.numel() // n if n else 0
+    y = torch.empty(acc.shape, dtype=out_dtype, device=acc.device)
+    _l.check(_l.load().lq_sq_output_dequant(_ptr(y), _DT[out_dtype], _ptr(acc), _ptr(input_quant_scale),
+                                            _ptr(weight_quant_scale), int(per_token), rows, n, _stream()),
+             "lq_sq_output_dequant")
+    return y
+
+
+def int8_weight_quant(w, pre_quant_scale=None):
+    """invokeGetINT8WeightScale: w [N,K] -> (q int8 [N,K] row-major, scale fp32 [N])."""
+    _chk(w, "w", _FLOATS)
+    if pre_quant_scale is not None:
+        _chk(pre_quant_scale, "pre_quant_scale", (torch.float32,))
+    n, k = w.shape
+    q = torch.empty((n, k), dtype=torch.int8, device=w.device)
+    s = torch.empty(n, dtype=torch.float32, device=w.device)
+    _l.check(_l.load().lq_int8_weight_quant(_ptr(s), _ptr(q), _ptr(w), _DT[w.dtype], _ptr(pre_quant_scale), n, k,
+                                            _stream()), "lq_int8_weight_quant")
+    return q, s
+
+
+def geglu_int8(hidden, bias, pre_quant_scale, input_quant_scale):
+    """invokeFusedAddBiasGegluInt8O: hidden [..., 2D] -> int8 [..., D], static scale."""
+    _chk(hidden, "hidden", _FLOATS)
+    _chk(input_quant_scale, "input_quant_scale", (torch.float32,))
+    if bias is not None:
+        _chk(bias, "bias", (hidden.dtype,))
+    if pre_quant_scale is not None:
+        _chk(pre_quant_scale, "pre_quant_scale", (torch.float32,))
+    d = hidden.shape[-1] // 2
+    rows = hidden.numel() // (2 * d) if d else 0
+    q = torch.empty(hidden.shape[:-1] + (d,), dtype=torch.int8, device=hidden.device)
+    _l.check(_l.load().lq_geglu_int8(_ptr(q), _ptr(hidden), _ptr(bias), _DT[hidden.dtype], _ptr(pre_quant_scale),
+                                     _ptr(input_quant_scale), rows, d, _stream()), "lq_geglu_int8")
+    return q
+
+
+def geglu_int8_dynamic(hidden, bias=None, pre_quant_scale=None):
+    _chk(hidden, "hidden", _FLOATS)
+    if bias is not None:
+        _chk(bias, "bias", (hidden.dtype,))
+    if pre_quant_scale is not None:
+        _chk(pre_quant_scale, "pre_quant_scale", (torch.float32,))
+    d = hidden.shape[-1] // 2
+    rows = hidden.numel() // (2 * d) if d else 0
+    q = torch.empty(hidden.shape[:-1] + (d,), dtype=torch.int8, device=hidden.device)
+    s = torch.empty(rows, dtype=torch.float32, device=hidden.device)
+    _l.check(_l.load().lq_geglu_int8_dynamic(_ptr(q), _ptr(s), _ptr(hidden), _ptr(bias), _DT[hidden.dtype],
+                                             _ptr(pre_quant_scale), rows, d, _stream()), "lq_geglu_int8_dynamic")
+    return q, s
+
+
+# ---- FP8 -------------------------------------------------------------------------------------------
+
+def fp8_amax_scale(x, scale=None):
+    """invokeGetFP8WeightScale: scale = max(scale, max|x|/448); allocates a zeroed scale if None."""
+    _chk(x, "x", _FLOATS)
+    if scale is None:
+        scale = torch.zeros(1, dtype=torch.float32, device=x.device)
+    _chk(scale, "scale", (torch.float32,))
+    _l.check(_l.load().lq_fp8_amax_scale(_ptr(scale), _ptr(x), _DT[x.dtype], x.numel(), _stream()),
+             "lq_fp8_amax_scale")
+    return scale
+
+
+def fp8_scale_cast(x, scale, invert: bool = True):
+    """invokeCudaD2DScaleCpyConvert to e4m3; returns a uint8 tensor of e4m3fn codes."""
+    _chk(x, "x", _FLOATS)
+    _chk(scale, "scale", (torch.float32,))
+    q = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    _l.check(_l.load().lq_fp8_scale_cast(_ptr(q), _ptr(x), _DT[x.dtype], _ptr(scale), int(invert), x.numel(),
+                                         _stream()), "lq_fp8_scale_cast")
+    return q
+
+
+def fp8_quant(x):
+    """Dynamic per-tensor activation quant: returns (e4m3 codes uint8, scale fp32 [1])."""
+    _chk(x, "x", _FLOATS)
+    q = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    s = torch.empty(1, dtype=torch.float32, device=x.device)
+    _l.check(_l.load().lq_fp8_amax_cast(_ptr(q), _ptr(s), _ptr(x), _DT[x.dtype], x.numel(), _stream()),
+             "lq_fp8_amax_cast")
+    return q, s
+
+
+# ---- W4A4 ------------------------------------------------------------------------------------------
+
+def w4a4_quant(x, smooth=None, scale_dtype=torch.float32, group: int = 64):
+    """Group-64 INT4 quantisation: returns (words int32 [M, K/8], scales [M, K/64])."""
+    _chk(x, "x", _FLOATS)
+    if smooth is not None:
+        _chk(smooth, "smooth", (torch.float32,))
+    m, k = x.shape
+    q = torch.empty((m, k // 8), dtype=torch.int32, device=x.device)
+    s = torch.empty((m, k // group), dtype=scale_dtype, device=x.device)
+    _l.check(_l.load().lq_w4a4_quantize(_ptr(q), _ptr(s), _DT[scale_dtype], _ptr(x), _DT[x.dtype], _ptr(smooth),
+                                        m, k, group, _stream()), "lq_w4a4_quantize")
+    return q, s
+
+
+# ---- weight repack ---------------------------------------------------------------------------------
+
+def repack_weight(w_bytes):
+    """[N, row_bytes] byte matrix (int8 / e4m3 codes / packed nibbles) -> rows32 layout, same size."""
+    _chk(w_bytes, "w", (torch.int8, torch.uint8))
+    n, rb = w_bytes.shape
+    out = torch.empty_like(w_bytes)
+    _l.check(_l.load().lq_repack_rows32(_ptr(out), _ptr(w_bytes), n, rb, _stream()), "lq_repack_rows32")
+    return out
+
+
+def unpack_weight(packed):
+    _chk(packed, "packed", (torch.int8, torch.uint8))
+    n, rb = packed.shape
+    out = torch.empty_like(packed)
+    _l.check(_l.load().lq_unpack_rows32(_ptr(out), _ptr(packed), n, rb, _stream()), "lq_unpack_rows32")
+    return out
+
+
+# ---- GEMMs -----------------------------------------------------------------------------------------
+
+def int8_linear(a_q, w_rows32, alpha_col, alpha_row, bias=None, out_dtype=torch.float16):
+    """runGemmInt8 + fused bias: a_q int8 [M,K], w_rows32 int8 [N,K] (rows32), returns [M,N]."""
+    _chk(a_q, "a_q", (torch.int8,))
+    _chk(w_rows32, "w_rows32", (torch.int8,))
+    m, k = a_q.shape
+    n = w_rows32.shape[0]
+    if w_rows32.shape[1] != k:
+        raise ValueError("K mismatch between activation and weight")
+    per_token = 0
+    if out_dtype != torch.int32:
+        _chk(alpha_col, "alpha_col", (torch.float32,))
+        _chk(alpha_row, "alpha_row", (torch.float32,))
+        if alpha_col.numel() != n:
+            raise ValueError("alpha_col must have N elements")
+        if alpha_row.numel() not in (1, m):
+            raise ValueError("alpha_row must have 1 or M elements")
+        per_token = int(alpha_row.numel() == m and m != 1)
+    if bias is not None:
+        _chk(bias, "bias", (out_dtype,))
+    c = torch.empty((m, n), dtype=out_dtype, device=a_q.device)
+    _l.check(_l.load().lq_gemm_int8(_ptr(c), _DT[out_dtype], _ptr(a_q), _ptr(w_rows32), _ptr(alpha_col),
+                                    _ptr(alpha_row), per_token, _ptr(bias), m, n, k, _stream()), "lq_gemm_int8")
+    return c
+
+
+def fp8_linear(a_q, w_rows32, a_scale, b_scale, bias=None, gelu: bool = False, residual=None, beta: float = 0.0,
+               out_dtype=torch.bfloat16):
+    """FP8 GemmWithResidualAndBias: a_q uint8 e4m3 [M,K], w_rows32 uint8 e4m3 [N,K] (rows32)."""
+    _chk(a_q, "a_q", (torch.uint8,))
+    _chk(w_rows32, "w_rows32", (torch.uint8,))
+    _chk(a_scale, "a_scale", (torch.float32,))
+    _chk(b_scale, "b_scale", (torch.float32,))
+    m, k = a_q.shape
+    n = w_rows32.shape[0]
+    if w_rows32.shape[1] != k:
+        raise ValueError("K mismatch between activation and weight")
+    if bias is not None:
+        _chk(bias, "bias", (out_dtype,))
+    if residual is not None:
+        _chk(residual, "residual", (out_dtype,))
+    c = torch.empty((m, n), dtype=out_dtype, device=a_q.device)
+    _l.check(_l.load().lq_gemm_fp8(_ptr(c), _DT[out_dtype], _ptr(a_q), _ptr(w_rows32), _ptr(a_scale), _ptr(b_scale),
+                                   _ptr(bias), int(gelu), _ptr(residual), float(beta), m, n, k, _stream()),
+             "lq_gemm_fp8")
+    return c
+
+
+def w4a4_linear(a_words, w_rows32, sA, sB, bias=None, out_dtype=torch.bfloat16, group: int = 64):
+    """W4A4 GEMM: a_words int32 [M,K/8], w_rows32 uint8 [N,K/2] (rows32), scales [M,G] / [N,G]."""
+    _chk(a_words, "a_words", (torch.int32,))
+    _chk(w_rows32, "w_rows32", (torch.uint8, torch.int8))
+    _chk(sA, "sA", (torch.float32, torch.float16))
+    _chk(sB, "sB", (sA.dtype,))
+    m = a_words.shape[0]
+    k = a_words.shape[1] * 8
+    n = w_rows32.shape[0]
+    if w_rows32.shape[1] * 2 != k:
+        raise ValueError("K mismatch between activation and weight")
+    if bias is not None:
+        _chk(bias, "bias", (out_dtype,))
+    c = torch.empty((m, n), dtype=out_dtype, device=a_words.device)
+    _l.check(_l.load().lq_gemm_w4a4(_ptr(c), _DT[out_dtype], _ptr(a_words), _ptr(w_rows32), _ptr(sA), _ptr(sB),
+                                    _DT[sA.dtype], _ptr(bias), m, n, k, group, _stream()), "lq_gemm_w4a4")
+    return c

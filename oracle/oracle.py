@@ -1,0 +1,463 @@
+"""CPU oracle for the quantized-linear path (TEST INFRASTRUCTURE, NOT PRODUCT CODE).
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import this
+module.  Nothing under lyradiff_amd/ imports it; the product path has no CPU fallback.
+
+Every function restates, in IEEE-754 binary32 numpy arithmetic, the formula of one
+function of the lyraDiff reference (cited file:line, relative to the reference root
+src/lyradiff/ unless a longer path is given).  The reference has no tests and no golden
+vectors for this path, and none of its CUDA compiles here, so every function is pinned by
+closed forms / exhaustive tables / brute force in tests/test_oracle_*.py:
+
+  rne_sat_s8            half-integer table, NaN/inf                  (pinned)
+  sq_* / weight quant   amax element -> +-127, sign symmetry, brute   (pinned)
+  e4m3 codec            all 256 codes and all 2^16 bf16 inputs vs
+                        torch.float8_e4m3fn after clamping             (pinned)
+  gemm_i8_acc           naive triple loop, torch int32 matmul          (pinned)
+  w4a4 pack             hand-computed words, unpack round trip         (pinned)
+  w4a4 gemm             C twin with libm fmaf (oracle_c.c) + fp64      (pinned)
+  gelu_tanh_f32         torch.nn.functional.gelu(approximate="tanh")   (pinned to 2e-7 abs)
+  fp8_gemm              fp64 evaluation (summation order is free in the
+                        reference's closed-source cuBLASLt)            (pinned to tolerance)
+
+The calibration that produces SmoothQuant `pre_quant_scale` in the reference lives in
+nvidia-modelopt (absent): parity unpinned, replaced by the closed form in smooth_vector().
+"""
+from __future__ import annotations
+
+import numpy as np
+
+F32 = np.float32
+
+# ----------------------------------------------------------------------------------------
+# dtype helpers (fp16 via numpy, bf16 via bit tricks; both round-to-nearest-even)
+# ----------------------------------------------------------------------------------------
+
+
+def f32_to_bf16_bits(x) -> np.ndarray:
+    """fp32 -> bf16 bit pattern (uint16), RNE, NaN kept quiet."""
+    x = np.ascontiguousarray(x, dtype=F32)
+    u = x.view(np.uint32).astype(np.uint64)
+    rounded = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
+    out = rounded.astype(np.uint16)
+    nan = np.isnan(x)
+    if nan.any():
+        out = np.where(nan, ((u >> 16) | 0x40).astype(np.uint16), out)
+    return out
+
+
+def bf16_bits_to_f32(b) -> np.ndarray:
+    b = np.ascontiguousarray(b, dtype=np.uint16)
+    return (b.astype(np.uint32) << 16).view(F32)
+
+
+def round_to(x, dtype: str) -> np.ndarray:
+    """Round an fp32 array to `dtype` ('f32' | 'f16' | 'bf16') and return it as fp32."""
+    x = np.asarray(x, dtype=F32)
+    if dtype == "f32":
+        return x
+    if dtype == "f16":
+        with np.errstate(over="ignore"):
+            return x.astype(np.float16).astype(F32)
+    if dtype == "bf16":
+        return bf16_bits_to_f32(f32_to_bf16_bits(x))
+    raise ValueError(dtype)
+
+
+# ----------------------------------------------------------------------------------------
+# a1  float_to_int8_rn  (kernels/quant_kernels/int8_utils.cuh:23-28)
+# ----------------------------------------------------------------------------------------
+
+
+def rne_sat_s8(x) -> np.ndarray:
+    """rint (half-to-even) then saturate to [-128, 127]; NaN -> 0 (cvt.rni.sat semantics)."""
+    x = np.asarray(x, dtype=F32)
+    with np.errstate(invalid="ignore"):
+        r = np.rint(x)
+        r = np.where(np.isnan(r), F32(0), r)
+        r = np.clip(r, F32(-128), F32(127))
+    return r.astype(np.int8)
+
+
+# ----------------------------------------------------------------------------------------
+# a2/a3  SmoothQuant activation quant  (kernels/quant_kernels/quant_kernels.cu:51-115)
+# ----------------------------------------------------------------------------------------
+
+
+def sq_smoothed(x, pre) -> np.ndarray:
+    """t[m,k] = f32(x[m,k]) * pre[k]  -- one fp32 multiply (quant_kernels.cu:86-89)."""
+    x = np.asarray(x, dtype=F32)
+    if pre is None:
+        return x
+    return x * np.asarray(pre, dtype=F32)[None, :]
+
+
+def sq_input_quant(x, pre, scale, per_token: bool) -> np.ndarray:
+    """q = sat_s8(rne((f32(x)*pre[k]) / s)); s = scale[0] or scale[m]
+    (sqInputQuant quant_kernels.cu:51-91, sqPerTokenInputQuant :93-115)."""
+    t = sq_smoothed(x, pre)
+    s = np.asarray(scale, dtype=F32).reshape(-1)
+    s = s[:, None] if per_token else s[:1].reshape(1, 1)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        return rne_sat_s8(t / s)
+
+
+def sq_dynamic_scale(x, pre) -> np.ndarray:
+    """s[m] = max_k |f32(x)*pre[k]| / 127, formula of the reference's weight path
+    (quant_kernels.cu:207 `amax / 127.0`; exporter convert_model_scripts/
+    convert_sd_quant_model.py:135,195-197).  Zero-row rule of the exporter
+    (convert_sd_quant_model.py:137-150): amax <= 2^-24 -> scale 1 (q is 0 either way).
+    `amax / 127.0` is a double division narrowed to float == correctly rounded fp32 division."""
+    t = sq_smoothed(x, pre)
+    amax = np.max(np.abs(t), axis=1).astype(F32)
+    s = amax / F32(127.0)
+    return np.where(amax <= F32(2.0 ** -24), F32(1.0), s).astype(F32)
+
+
+def sq_dynamic_quant(x, pre):
+    s = sq_dynamic_scale(x, pre)
+    return sq_input_quant(x, pre, s, per_token=True), s
+
+
+def smooth_vector(x, w, alpha: float = 0.5) -> np.ndarray:
+    """SmoothQuant per-channel smoothing s[k] = max|X_k|^a / max|W_k|^(1-a); the reference
+    consumes a precomputed pre_quant_scale = 1/s (convert_sd_quant_model.py:199)."""
+    ax = np.max(np.abs(np.asarray(x, dtype=F32)), axis=0)
+    aw = np.max(np.abs(np.asarray(w, dtype=F32)), axis=0)
+    return (np.power(ax, F32(alpha)) / np.power(aw, F32(1.0 - alpha))).astype(F32)
+
+
+# ----------------------------------------------------------------------------------------
+# a5  weight quant: device (quant_kernels.cu:173-223) and exporter
+#     (lyradiff/convert_model_scripts/convert_sd_quant_model.py:108-155)
+# ----------------------------------------------------------------------------------------
+
+
+def int8_weight_quant_device(w, pre):
+    """w' = f32(w)/pre[k]; s[n] = max_k|w'|/127; q = sat_s8(rne(w'/s))  (range -128..127)."""
+    w = np.asarray(w, dtype=F32)
+    wp = w / np.asarray(pre, dtype=F32)[None, :] if pre is not None else w
+    amax = np.max(np.abs(wp), axis=1).astype(F32)
+    s = (amax / F32(127.0)).astype(F32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        q = rne_sat_s8(wp / s[:, None])
+    return q, s
+
+
+def int8_weight_quant_export(w, narrow_range: bool = True):
+    """Exporter flavour: scale = 127/amax, q = clamp(rne(w*scale), -127|-128, 127);
+    amax <= 2^-24 -> q = 0, stored scale 1 (convert_sd_quant_model.py:127-150).
+    Returns (q, stored_scale = amax/127 as 1/(127/amax))."""
+    w = np.asarray(w, dtype=F32)
+    amax = np.max(np.abs(w), axis=1).astype(F32)
+    tiny = amax <= F32(2.0 ** -24)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        mult = F32(127.0) / amax
+        mult = np.where(tiny, F32(1.0), mult).astype(F32)
+        r = np.rint(w * mult[:, None])
+    lo = -127 if narrow_range else -128
+    q = np.clip(r, lo, 127)
+    q = np.where(tiny[:, None], 0, q).astype(np.int8)
+    with np.errstate(divide="ignore"):
+        stored = np.where(tiny, F32(1.0), F32(1.0) / mult).astype(F32)
+    return q, stored
+
+
+# ----------------------------------------------------------------------------------------
+# a6/a7/a8  INT8 GEMM + per-row/per-col epilogue
+#   (kernels/cutlass_kernels/int8_gemm/int8_gemm_template.h:63-158,
+#    kernels/cutlass_extensions/include/cutlass_extensions/epilogue/threadblock/
+#    epilogue_per_row_per_col_scale.h:239-257,278-305)
+# ----------------------------------------------------------------------------------------
+
+
+def gemm_i8_acc(a_q, w_q) -> np.ndarray:
+    """acc[m,n] = sum_k i32(a[m,k]) * i32(w[n,k])  (exact)."""
+    import torch
+
+    a = torch.from_numpy(np.ascontiguousarray(a_q)).to(torch.int32)
+    w = torch.from_numpy(np.ascontiguousarray(w_q)).to(torch.int32)
+    return (a @ w.t()).numpy()
+
+
+def int8_epilogue(acc, alpha_col, alpha_row, bias=None, out_dtype: str = "f16") -> np.ndarray:
+    """y = T( f32(acc) * (alpha_col[n] * alpha_row[m|0]) [+ f32(bias[n])] ), scales multiplied
+    first (epilogue_per_row_per_col_scale.h:286,301).  The bias add is the fused form of the
+    reference's separate bias kernel (layers/basic_transformer/BasicTransformerInt8Block.cc:452,838):
+    one fp32 multiply, one fp32 add, one rounding to T.  Returned as fp32 holding T values."""
+    acc = np.asarray(acc)
+    ac = np.asarray(alpha_col, dtype=F32).reshape(1, -1)
+    ar = np.asarray(alpha_row, dtype=F32).reshape(-1)
+    ar = ar.reshape(-1, 1) if ar.size > 1 else ar.reshape(1, 1)
+    y = acc.astype(F32) * (ac * ar)
+    if bias is not None:
+        y = y + np.asarray(bias, dtype=F32).reshape(1, -1)
+    if out_dtype == "i32":
+        return acc.astype(np.int32)
+    return round_to(y, out_dtype)
+
+
+def sq_output_dequant(acc, in_scale, w_scale, per_token: bool, out_dtype: str) -> np.ndarray:
+    """y = T(f32(acc) * s_in * s_w[n]) -- left-to-right order of the unfused dequant kernel
+    (quant_kernels.cu:117-171)."""
+    s_in = np.asarray(in_scale, dtype=F32).reshape(-1)
+    s_in = s_in[:, None] if per_token else s_in[:1].reshape(1, 1)
+    y = (np.asarray(acc).astype(F32) * s_in) * np.asarray(w_scale, dtype=F32)[None, :]
+    return round_to(y, out_dtype)
+
+
+# ----------------------------------------------------------------------------------------
+# a9  bias + GEGLU -> INT8  (kernels/quant_kernels/ffn_kernels_int8.cu:102-147,
+#     kernels/activation_kernels.h:70-83)
+# ----------------------------------------------------------------------------------------
+
+_EXP2_POLY = [F32(c) for c in (
+    1.0, 0.693147180559945, 0.240226506959101, 0.0555041086648216,
+    0.00961812910762848, 0.00133335581464284, 0.000154035303933816, 1.52527338040598e-05)]
+
+
+def tanh_f32(u) -> np.ndarray:
+    """tanh built from +,*,/ and one exact power-of-two scaling only, so that the HIP kernel
+    (compiled without fp contraction) reproduces it bit for bit:
+        a = min(|u|, 10);  t = a * (2*log2 e);  n = rint(t);  f = t - n
+        e = P7(f) * 2^n  (P7 = Taylor of 2^f, Horner, separate mul and add)
+        tanh = copysign(1 - 2/(e + 1), u)
+    The reference uses the hardware `tanh.approx.f32` (activation_kernels.h:19-24), which is
+    NVIDIA-specific and only ~2^-11 accurate; this form is accurate to ~2e-7."""
+    u = np.asarray(u, dtype=F32)
+    a = np.minimum(np.abs(u), F32(10.0))
+    t = a * F32(2.8853900817779268)
+    n = np.rint(t)
+    f = t - n
+    p = np.full_like(f, _EXP2_POLY[7])
+    for c in _EXP2_POLY[6::-1]:
+        p = p * f + c
+    e = np.ldexp(p, n.astype(np.int32)).astype(F32)
+    r = F32(1.0) - F32(2.0) / (e + F32(1.0))
+    return np.copysign(r, u).astype(F32)
+
+
+def gelu_tanh_f32(x) -> np.ndarray:
+    """x * 0.5*(1+tanh(0.79788456*(x + 0.044715*x^3))) in fp32 (activation_kernels.h:31-40)."""
+    x = np.asarray(x, dtype=F32)
+    inner = F32(0.7978845608028654) * (x + F32(0.044715) * (x * x * x))
+    return x * (F32(0.5) * (F32(1.0) + tanh_f32(inner)))
+
+
+def geglu_product(x, bias, dtype: str) -> np.ndarray:
+    """h*g of the fused GEGLU kernel in T arithmetic (ffn_kernels_int8.cu:127-146 with
+    GeluActivation<half2>, activation_kernels.h:70-83): adds, cube and products are rounded
+    to T after every operation; the tanh argument is evaluated in fp32.
+    x: [M, 2D] holding T values; returns [M, D] fp32 holding T values."""
+    x = np.asarray(x, dtype=F32)
+    d = x.shape[1] // 2
+    h, g = x[:, :d], x[:, d:]
+    if bias is not None:
+        b = np.asarray(bias, dtype=F32)
+        h = round_to(h + b[None, :d], dtype)
+        g = round_to(g + b[None, d:], dtype)
+    cube = round_to(g * round_to(g * g, dtype), dtype)
+    cdf = F32(0.5) * (F32(1.0) + tanh_f32(F32(0.7978845608028654) * (g + F32(0.044715) * cube)))
+    gel = round_to(g * round_to(cdf, dtype), dtype)
+    return round_to(h * gel, dtype)
+
+
+def geglu_int8(x, bias, pre, scale, dtype: str = "f16") -> np.ndarray:
+    """q = sat_s8(rne(f32(h*g) * pre[k] / s)), static per-tensor s (ffn_kernels_int8.cu:143-146)."""
+    return sq_input_quant(geglu_product(x, bias, dtype), pre, scale, per_token=False)
+
+
+def geglu_int8_dynamic(x, bias, pre, dtype: str = "f16"):
+    """Same with the dynamic per-token scale of sq_dynamic_scale()."""
+    return sq_dynamic_quant(geglu_product(x, bias, dtype), pre)
+
+
+# ----------------------------------------------------------------------------------------
+# a10/a11  FP8 e4m3 per-tensor  (kernels/lora/load_lora.cu:16-54, utils/memory_utils.cu:431-446)
+# ----------------------------------------------------------------------------------------
+
+
+def _e4m3_table() -> np.ndarray:
+    codes = np.arange(256, dtype=np.uint32)
+    sign = np.where(codes & 0x80, -1.0, 1.0)
+    e = (codes >> 3) & 0xF
+    m = codes & 7
+    val = np.where(e == 0, m / 8.0 * 2.0 ** -6, (1 + m / 8.0) * np.exp2(e.astype(np.float64) - 7))
+    val = sign * val
+    val[(codes & 0x7F) == 0x7F] = np.nan
+    return val.astype(F32)
+
+
+E4M3_VALUES = _e4m3_table()  # code -> fp32 (OCP e4m3fn: max 448, NaN = 0x7F/0xFF, no inf)
+
+
+def e4m3_decode(codes) -> np.ndarray:
+    return E4M3_VALUES[np.asarray(codes, dtype=np.uint8)]
+
+
+def e4m3_encode(x) -> np.ndarray:
+    """fp32 -> e4m3fn code, round-to-nearest-even, saturate-to-finite (|v|>448 and inf -> 448),
+    NaN -> 0x7F | sign: the `__nv_fp8_e4m3(float)` constructor semantics the reference relies on
+    (utils/cuda_type_utils.cuh:599-613).  Bit-level, no table search."""
+    x = np.ascontiguousarray(x, dtype=F32)
+    u = x.view(np.uint32)
+    sign = ((u >> 24) & 0x80).astype(np.uint8)
+    a = np.abs(x)
+    with np.errstate(invalid="ignore", over="ignore", divide="ignore"):
+        a64 = np.where(np.isfinite(a), a, F32(1e30)).astype(np.float64)
+        # floor(log2 a) from frexp (exact); e4m3 normals span 2^-6..2^8, subnormal step 2^-9
+        ex = np.clip(np.frexp(a64)[1] - 1, -6, 8).astype(np.float64)
+        step = np.exp2(ex - 3)
+        qv = np.rint(a64 / step) * step  # RNE on the e4m3 grid (exact in fp64)
+        qv = np.minimum(qv, 448.0)
+        e2 = np.clip(np.frexp(qv)[1] - 1, -6, 8).astype(np.float64)
+        is_sub = qv < 2.0 ** -6
+        code = np.where(is_sub, np.rint(qv * 512.0), (e2 + 7) * 8 + np.rint((qv / np.exp2(e2) - 1.0) * 8.0))
+        code = np.where(np.isnan(x), 0x7F, code)
+    return (code.astype(np.uint8) | sign).astype(np.uint8)
+
+
+def fp8_scale(x) -> np.float32:
+    """scale = max_i |f32(x_i)| / 448  (load_lora.cu:48-54; the double division narrowed to
+    float there equals the correctly rounded fp32 division)."""
+    amax = F32(np.max(np.abs(np.asarray(x, dtype=F32)))) if np.size(x) else F32(0)
+    return F32(amax / F32(448.0))
+
+
+def fp8_scale_cast(x, scale, invert: bool = True) -> np.ndarray:
+    """q = e4m3(f32(x) * (invert ? 1.0f/scale : scale))  (memory_utils.cu:431-439)."""
+    s = F32(np.asarray(scale, dtype=F32).reshape(-1)[0])
+    with np.errstate(divide="ignore"):
+        r = F32(1.0) / s if invert else s
+    with np.errstate(invalid="ignore", over="ignore"):
+        return e4m3_encode(np.asarray(x, dtype=F32) * r)
+
+
+def fp8_amax_cast(x):
+    """Dynamic per-tensor activation quant = fp8_scale() then fp8_scale_cast(invert=True)."""
+    s = fp8_scale(x)
+    return fp8_scale_cast(x, s, True), s
+
+
+# ----------------------------------------------------------------------------------------
+# a12  FP8 GEMM contract  (utils/cublasMMWrapper.cc:1104-1274): closed-source cuBLASLt;
+#      C = T( (sa*sb) * sum_k A*B + bias [-> gelu] [+ beta*residual] ), fp32 compute.
+# ----------------------------------------------------------------------------------------
+
+
+def fp8_gemm(qa, qb, sa, sb, bias=None, gelu: bool = False, residual=None, beta: float = 0.0,
+             out_dtype: str = "bf16") -> np.ndarray:
+    """fp64 evaluation of the contract (summation order is not pinned by the reference)."""
+    a = e4m3_decode(qa).astype(np.float64)
+    b = e4m3_decode(qb).astype(np.float64)
+    acc = a @ b.T
+    alpha = F32(F32(np.asarray(sa).reshape(-1)[0]) * F32(np.asarray(sb).reshape(-1)[0]))
+    y = acc.astype(F32) * alpha
+    if bias is not None:
+        y = y + np.asarray(bias, dtype=F32)[None, :]
+    if gelu:
+        y = gelu_tanh_f32(y)
+    if residual is not None and beta != 0.0:
+        y = y + F32(beta) * np.asarray(residual, dtype=F32)
+    return round_to(y, out_dtype)
+
+
+# ----------------------------------------------------------------------------------------
+# a13  W4A4 group-64 activation quant + nibble packing  (kernels/w4a4_gemm/w4a4_gemm.cu:206-214,
+#      897-930)
+# ----------------------------------------------------------------------------------------
+
+
+def w4a4_quant_values(x, smooth, group: int = 64, scale_dtype: str = "f32"):
+    """v = f32(x)/smooth[k]; s[m,g] = max_{k in g}|v| / 7; q = clamp(rne(v/s), -8, 7).
+    Zero group: s = 0 and q = 0 (the reference's NaN -> cvt.rni -> 0).  With scale_dtype
+    'f16' the scale is rounded to fp16 first and the rounded value quantises (so quant and
+    dequant use the same number).  Returns (q int8 [M,K], s fp32 [M,K/group])."""
+    x = np.asarray(x, dtype=F32)
+    m, k = x.shape
+    v = x / np.asarray(smooth, dtype=F32)[None, :] if smooth is not None else x
+    vg = v.reshape(m, k // group, group)
+    amax = np.max(np.abs(vg), axis=2).astype(F32)
+    s = (amax / F32(7.0)).astype(F32)
+    s = round_to(s, scale_dtype)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        r = np.rint(vg / s[:, :, None])
+    r = np.where(np.isnan(r), F32(0), r)
+    q = np.clip(r, -8, 7).astype(np.int8).reshape(m, k)
+    return q, s
+
+
+def pack_int4(q) -> np.ndarray:
+    """[M,K] int8 in [-8,7] -> [M,K/8] uint32; element i of a word sits in bits [4i, 4i+3]
+    (w4a4_gemm.cu:914-929: lane pair packs low nibble first, byte j of the word = lanes 4w+j)."""
+    q = np.asarray(q, dtype=np.int8)
+    m, k = q.shape
+    nib = (q.astype(np.uint32) & 0xF).reshape(m, k // 8, 8)
+    shifts = (4 * np.arange(8, dtype=np.uint32))[None, None, :]
+    return np.bitwise_or.reduce(nib << shifts, axis=2).astype(np.uint32)
+
+
+def unpack_int4(words, k: int | None = None) -> np.ndarray:
+    """Inverse of pack_int4 (sign-extending); same low-nibble-first convention as
+    layers/gemm_utils/WeightOnlyQuantOps.cc:275-283."""
+    w = np.asarray(words, dtype=np.uint32)
+    shifts = (4 * np.arange(8, dtype=np.uint32))[None, None, :]
+    nib = ((w[:, :, None] >> shifts) & 0xF).astype(np.int8)
+    q = np.where(nib >= 8, nib - 16, nib).astype(np.int8)
+    return q.reshape(w.shape[0], -1)
+
+
+def w4a4_quant(x, smooth, group: int = 64, scale_dtype: str = "f32"):
+    q, s = w4a4_quant_values(x, smooth, group, scale_dtype)
+    return pack_int4(q), s
+
+
+# ----------------------------------------------------------------------------------------
+# a14  W4A4 GEMM  (kernels/w4a4_gemm/w4a4_gemm.cu:473-506,717)
+# ----------------------------------------------------------------------------------------
+
+
+def w4a4_group_acc(qa, qb, group: int = 64) -> np.ndarray:
+    """p[m,n,g] = sum_{k in g} i32(qa[m,k]) * i32(qb[n,k])  (exact), shape [M,N,G]."""
+    import torch
+
+    a = torch.from_numpy(np.ascontiguousarray(qa)).to(torch.int32)
+    b = torch.from_numpy(np.ascontiguousarray(qb)).to(torch.int32)
+    m, k = a.shape
+    n = b.shape[0]
+    g = k // group
+    a = a.reshape(m, g, group).permute(1, 0, 2)
+    b = b.reshape(n, g, group).permute(1, 2, 0)
+    return torch.bmm(a, b).permute(1, 2, 0).contiguous().numpy()
+
+
+def w4a4_gemm_f64(qa, qb, sA, sB, bias=None, group: int = 64, out_dtype: str = "bf16") -> np.ndarray:
+    """fp64 evaluation of y = sum_g p*sA*sB (+bias); tolerance reference.  The bit-exact fp32
+    fmaf chain in ascending g lives in oracle_c.c (w4a4_gemm_ref), which this is pinned against."""
+    p = w4a4_group_acc(qa, qb, group).astype(np.float64)
+    y = np.einsum("mng,mg,ng->mn", p, np.asarray(sA, np.float64), np.asarray(sB, np.float64))
+    if bias is not None:
+        y = y + np.asarray(bias, dtype=np.float64)[None, :]
+    return round_to(y.astype(F32), out_dtype)
+
+
+# ----------------------------------------------------------------------------------------
+# a16  weight repack contract: a bijection of the [N,K] byte matrix
+#      (reference counterpart: kernels/cutlass_kernels/cutlass_preprocessors.cpp:129-530,
+#       NVIDIA-mma specific; only the "pure permutation, same byte count" contract is kept)
+# ----------------------------------------------------------------------------------------
+
+
+def repack_rows32(w_bytes) -> np.ndarray:
+    """[N, Kb] bytes (Kb % 16 == 0, N % 32 == 0) -> tile-linear order
+    [N/32][Kb/16][32 rows][16 bytes]: every (32-row, 16-byte-column) block is 512 contiguous
+    bytes, so an MFMA operand fragment is one 16-byte load per lane at lane-linear addresses."""
+    w = np.ascontiguousarray(w_bytes).view(np.uint8)
+    n, kb = w.shape
+    assert n % 32 == 0 and kb % 16 == 0
+    return np.ascontiguousarray(w.reshape(n // 32, 32, kb // 16, 16).transpose(0, 2, 1, 3)).reshape(-1)
+
+
+def unpack_rows32(packed, n: int, kb: int) -> np.ndarray:
+    p = np.asarray(packed, dtype=np.uint8).reshape(n // 32, kb // 16, 32, 16)
+    return np.ascontiguousarray(p.transpose(0, 2, 1, 3)).reshape(n, kb)

@@ -1,0 +1,130 @@
+"""GPU parity of the quantized GEMMs against the CPU oracle, through the C ABI.
+
+int32 accumulators bit-exact; fp16/bf16/fp32 outputs of the INT8 and W4A4 paths bit-exact against
+the oracle's fp32 formula (same operation order, no contraction); FP8 outputs within the stated
+tolerance (1e-2 relative or 2 fp16 ULP) of an fp64 evaluation."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from oracle import oracle_c as OC
+from tests.helpers import TORCH_DT, assert_close_tol, rng_t, to_np_f32
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops(dev):
+    from lyradiff_amd import ops as _ops
+
+    return _ops
+
+
+INT8_SHAPES = [(1024, 1280, 1280), (4096, 5120, 640), (4096, 640, 2560), (77, 96, 64), (300, 1280, 192),
+               (1, 32, 64), (513, 3072, 3072)]
+
+
+@pytest.mark.parametrize("m,n,k", INT8_SHAPES)
+def test_int8_gemm_int32_exact(ops, dev, m, n, k):
+    g = rng_t(m * 7 + n + k)
+    a = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int8)
+    w = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8)
+    wp = ops.repack_weight(w.to(dev))
+    acc = ops.int8_linear(a.to(dev), wp, None, None, None, torch.int32)
+    assert np.array_equal(acc.cpu().numpy(), O.gemm_i8_acc(a.numpy(), w.numpy()))
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("per_token", [True, False])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_int8_gemm_epilogue(ops, dev, dt, per_token, with_bias):
+    m, n, k = 1024, 1280, 1280
+    g = rng_t(42)
+    a = torch.randint(-127, 128, (m, k), generator=g, dtype=torch.int8)
+    w = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8)
+    ac = (torch.rand(n, generator=g) * 9e-3 + 1e-3).float()
+    ar = (torch.rand(m if per_token else 1, generator=g) * 0.05 + 0.01).float()
+    bias = (torch.randn(n, generator=g) * 0.02).to(TORCH_DT[dt]) if with_bias else None
+    y = ops.int8_linear(a.to(dev), ops.repack_weight(w.to(dev)), ac.to(dev), ar.to(dev),
+                        bias.to(dev) if with_bias else None, TORCH_DT[dt])
+    acc = O.gemm_i8_acc(a.numpy(), w.numpy())
+    ref = O.int8_epilogue(acc, ac.numpy(), ar.numpy(), to_np_f32(bias) if with_bias else None, dt)
+    got = to_np_f32(y)
+    assert_close_tol(got, ref, "int8 epilogue")
+    assert np.array_equal(got, ref), "fused epilogue should reproduce the oracle's fp32 formula bit for bit"
+
+
+def fp32_sum_floor(qa, qb, sa, sb):
+    """8 fp32 ULPs of alpha * sum_k |a_k*b_k|: the accuracy an fp32 accumulator can deliver
+    when the K products cancel (the reference's cuBLASLt has the same property)."""
+    mag = np.abs(O.e4m3_decode(qa)).astype(np.float64) @ np.abs(O.e4m3_decode(qb)).astype(np.float64).T
+    return 8 * 2.0 ** -24 * mag * float(sa) * float(sb)
+
+
+FP8_SHAPES = [(512, 3072, 3072), (100, 256, 128), (33, 64, 64), (256, 12288, 3072), (640, 3072, 12288)]
+
+
+@pytest.mark.parametrize("m,n,k", FP8_SHAPES)
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+def test_fp8_gemm(ops, dev, m, n, k, dt):
+    g = rng_t(m + n + k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.02).bfloat16()
+    bias = (torch.randn(n, generator=g) * 0.1).to(TORCH_DT[dt])
+    qa, sa = O.fp8_amax_cast(to_np_f32(x))
+    qb, sb = O.fp8_amax_cast(to_np_f32(w))
+    qa_d = torch.from_numpy(qa).to(dev)
+    wp = ops.repack_weight(torch.from_numpy(qb).to(dev))
+    sa_d = torch.tensor([sa], dtype=torch.float32, device=dev)
+    sb_d = torch.tensor([sb], dtype=torch.float32, device=dev)
+    y = ops.fp8_linear(qa_d, wp, sa_d, sb_d, bias.to(dev), False, None, 0.0, TORCH_DT[dt])
+    ref = O.fp8_gemm(qa, qb, sa, sb, to_np_f32(bias), False, None, 0.0, dt)
+    assert_close_tol(to_np_f32(y), ref, "fp8 gemm", abs_floor=fp32_sum_floor(qa, qb, sa, sb))
+
+
+def test_fp8_gemm_gelu_residual(ops, dev):
+    m, n, k = 384, 512, 256
+    g = rng_t(3)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.05).bfloat16()
+    bias = (torch.randn(n, generator=g) * 0.1).bfloat16()
+    res = torch.randn(m, n, generator=g).bfloat16()
+    qa, sa = O.fp8_amax_cast(to_np_f32(x))
+    qb, sb = O.fp8_amax_cast(to_np_f32(w))
+    args = (torch.from_numpy(qa).to(dev), ops.repack_weight(torch.from_numpy(qb).to(dev)),
+            torch.tensor([sa], dtype=torch.float32, device=dev), torch.tensor([sb], dtype=torch.float32, device=dev))
+    y = ops.fp8_linear(*args, bias.to(dev), True, None, 0.0, torch.bfloat16)
+    floor = fp32_sum_floor(qa, qb, sa, sb)
+    assert_close_tol(to_np_f32(y), O.fp8_gemm(qa, qb, sa, sb, to_np_f32(bias), True, None, 0.0, "bf16"), "gelu",
+                     abs_floor=floor + 2e-6)  # + hardware exp2/rcp in the GELU (about 1e-6 absolute)
+    y2 = ops.fp8_linear(*args, bias.to(dev), False, res.to(dev), 0.5, torch.bfloat16)
+    assert_close_tol(to_np_f32(y2), O.fp8_gemm(qa, qb, sa, sb, to_np_f32(bias), False, to_np_f32(res), 0.5, "bf16"),
+                     "residual", abs_floor=floor)
+
+
+W4_SHAPES = [(256, 256, 256), (130, 96, 128), (512, 1024, 3072)]
+
+
+@pytest.mark.parametrize("m,n,k", W4_SHAPES)
+@pytest.mark.parametrize("sdt", ["f32", "f16"])
+def test_w4a4_gemm(ops, dev, m, n, k, sdt):
+    g = rng_t(m + n + k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.02).bfloat16()
+    bias = (torch.randn(n, generator=g) * 0.1).bfloat16()
+    qa, sA = O.w4a4_quant(to_np_f32(x), None, 64, sdt)
+    qb, sB = O.w4a4_quant(to_np_f32(w), None, 64, sdt)
+    wp = ops.repack_weight(torch.from_numpy(qb.view(np.uint8).reshape(n, k // 2)).to(dev))
+    sdt_t = TORCH_DT[sdt]
+    y = ops.w4a4_linear(torch.from_numpy(qa.view(np.int32)).to(dev), wp, torch.from_numpy(sA).to(sdt_t).to(dev),
+                        torch.from_numpy(sB).to(sdt_t).to(dev), bias.to(dev), torch.bfloat16)
+    ref32 = OC.w4a4_gemm(qa, qb, sA, sB, to_np_f32(bias))  # ascending-g fmaf chain, fp32
+    ref = O.round_to(ref32, "bf16")
+    got = to_np_f32(y)
+    assert_close_tol(got, ref, "w4a4 gemm")
+    assert np.array_equal(got, ref), "group accumulation order should match the oracle bit for bit"
+    # fp32 output exposes the accumulation itself
+    y32 = ops.w4a4_linear(torch.from_numpy(qa.view(np.int32)).to(dev), wp, torch.from_numpy(sA).to(sdt_t).to(dev),
+                          torch.from_numpy(sB).to(sdt_t).to(dev), None, torch.float32)
+    assert np.array_equal(y32.cpu().numpy(), OC.w4a4_gemm(qa, qb, sA, sB, None))

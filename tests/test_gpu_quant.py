@@ -1,0 +1,137 @@
+"""GPU parity of the activation-quantisation kernels against the CPU oracle, through the C ABI.
+
+Bit-exact for every integer / byte output and for the fp32 scales."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from tests.helpers import TORCH_DT, make_outlier_acts, rng_t, to_np_f32
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops(dev):
+    from lyradiff_amd import ops as _ops
+
+    return _ops
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("m,k", [(1024, 1280), (37, 640), (5, 8), (3, 2560), (64, 12288), (7, 1283)])
+def test_sq_dynamic_quant(ops, dev, dt, m, k):
+    x = make_outlier_acts(m, k, min(8, k), 20.0, TORCH_DT[dt], 1000 + m + k)
+    pre = (torch.rand(k, generator=rng_t(7)) * 1.5 + 0.25).float()
+    q, s = ops.sq_quant_dynamic(x.to(dev), pre.to(dev))
+    q_ref, s_ref = O.sq_dynamic_quant(to_np_f32(x), pre.numpy())
+    assert np.array_equal(s.cpu().numpy(), s_ref)
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+    # no smoothing vector
+    q2, s2 = ops.sq_quant_dynamic(x.to(dev), None)
+    q2_ref, s2_ref = O.sq_dynamic_quant(to_np_f32(x), None)
+    assert np.array_equal(s2.cpu().numpy(), s2_ref) and np.array_equal(q2.cpu().numpy(), q2_ref)
+
+
+def test_sq_dynamic_zero_rows(ops, dev):
+    x = torch.randn(16, 1280).half()
+    x[3] = 0
+    x[9] = 0
+    q, s = ops.sq_quant_dynamic(x.to(dev), None)
+    assert s[3].item() == 1.0 and s[9].item() == 1.0
+    assert int(q[3].abs().max()) == 0 and int(q[9].abs().max()) == 0
+    q_ref, s_ref = O.sq_dynamic_quant(to_np_f32(x), None)
+    assert np.array_equal(q.cpu().numpy(), q_ref) and np.array_equal(s.cpu().numpy(), s_ref)
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("per_token", [False, True])
+def test_sq_static_quant(ops, dev, dt, per_token):
+    m, k = 300, 1280
+    x = make_outlier_acts(m, k, 8, 20.0, TORCH_DT[dt], 5)
+    pre = (torch.rand(k, generator=rng_t(8)) + 0.5).float()
+    # a static scale small enough that saturation to -128 / 127 happens
+    scale = (torch.rand(m if per_token else 1, generator=rng_t(9)) * 0.02 + 0.01).float()
+    q = ops.sq_quant(x.to(dev), pre.to(dev), scale.to(dev), per_token)
+    q_ref = O.sq_input_quant(to_np_f32(x), pre.numpy(), scale.numpy(), per_token)
+    assert q_ref.min() == -128 and q_ref.max() == 127
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+
+
+def test_sq_quant_ties_and_specials(ops, dev):
+    # exact half-integers, saturation edges, NaN and inf, with s = 1 and a power-of-two s
+    vals = [0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 126.5, 127.5, -127.5, -128.5, 300.0, -300.0,
+            float("nan"), float("inf"), float("-inf"), 0.0]
+    x = torch.tensor(vals * 4, dtype=torch.float32).reshape(1, -1)
+    for s in (1.0, 0.5, 3.0):
+        sc = torch.tensor([s], dtype=torch.float32)
+        q = ops.sq_quant(x.to(dev), None, sc.to(dev), False)
+        assert np.array_equal(q.cpu().numpy(), O.sq_input_quant(x.numpy(), None, sc.numpy(), False))
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_geglu_int8(ops, dev, dt, with_bias):
+    m, d = 200, 2560
+    g = rng_t(11)
+    x = (torch.randn(m, 2 * d, generator=g) * 1.5).to(TORCH_DT[dt])
+    bias = (torch.randn(2 * d, generator=g) * 0.1).to(TORCH_DT[dt]) if with_bias else None
+    pre = (torch.rand(d, generator=g) + 0.5).float()
+    xn, bn = to_np_f32(x), (to_np_f32(bias) if with_bias else None)
+    q, s = ops.geglu_int8_dynamic(x.to(dev), bias.to(dev) if with_bias else None, pre.to(dev))
+    q_ref, s_ref = O.geglu_int8_dynamic(xn, bn, pre.numpy(), dt)
+    assert np.array_equal(s.cpu().numpy(), s_ref)
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+    sc = torch.tensor([0.03], dtype=torch.float32)
+    q2 = ops.geglu_int8(x.to(dev), bias.to(dev) if with_bias else None, pre.to(dev), sc.to(dev))
+    assert np.array_equal(q2.cpu().numpy(), O.geglu_int8(xn, bn, pre.numpy(), sc.numpy(), dt))
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("n", [4608 * 3072, 1000003, 17, 4096])
+def test_fp8_amax_cast(ops, dev, dt, n):
+    x = (torch.randn(n, generator=rng_t(n % 1000)) * 3).to(TORCH_DT[dt])
+    q, s = ops.fp8_quant(x.to(dev))
+    q_ref, s_ref = O.fp8_amax_cast(to_np_f32(x))
+    assert s.item() == float(s_ref)
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+
+
+def test_fp8_static_cast_saturates_and_nan(ops, dev):
+    x = torch.tensor([1.0, -1.0, 447.0, 449.0, 1e6, -1e6, float("nan"), float("inf"), 0.0, 1e-4, -3e-3, 0.0175] * 4,
+                     dtype=torch.float32)
+    for sc, inv in ((1.0, True), (0.5, True), (2.0, False)):
+        s = torch.tensor([sc], dtype=torch.float32)
+        q = ops.fp8_scale_cast(x.to(dev), s.to(dev), inv)
+        assert np.array_equal(q.cpu().numpy(), O.fp8_scale_cast(x.numpy(), s.numpy(), inv))
+
+
+def test_fp8_amax_scale_accumulates(ops, dev):
+    x = torch.randn(100000).bfloat16()
+    s = torch.tensor([10.0], dtype=torch.float32, device=dev)  # larger than any |x|/448
+    ops.fp8_amax_scale(x.to(dev), s)
+    assert s.item() == 10.0
+    s2 = ops.fp8_amax_scale(x.to(dev))
+    assert s2.item() == float(O.fp8_scale(to_np_f32(x)))
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32"])
+@pytest.mark.parametrize("sdt", ["f32", "f16"])
+@pytest.mark.parametrize("m,k", [(4608, 3072), (33, 64), (256, 12288), (5, 640)])
+def test_w4a4_quant(ops, dev, dt, sdt, m, k):
+    g = rng_t(m + k)
+    x = torch.randn(m, k, generator=g).to(TORCH_DT[dt])
+    x[0, :64] = 0  # an all-zero group
+    smooth = (torch.rand(k, generator=g) * 1.5 + 0.5).float()
+    for sm in (smooth, None):
+        q, s = ops.w4a4_quant(x.to(dev), None if sm is None else sm.to(dev), TORCH_DT[sdt])
+        q_ref, s_ref = O.w4a4_quant(to_np_f32(x), None if sm is None else sm.numpy(), 64, sdt)
+        assert np.array_equal(s.cpu().float().numpy(), s_ref)
+        assert np.array_equal(q.cpu().numpy().view(np.uint32), q_ref)
+
+
+def test_repack_roundtrip(ops, dev):
+    w = torch.randint(-128, 128, (1280, 640), dtype=torch.int8)
+    p = ops.repack_weight(w.to(dev))
+    assert np.array_equal(p.cpu().numpy().view(np.uint8).reshape(-1), O.repack_rows32(w.numpy()))
+    assert torch.equal(ops.unpack_weight(p).cpu(), w)
