@@ -182,6 +182,13 @@ int lq_gemm_w4a4(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const u
                  const void* sA, const void* sB, lq_dtype_t scale_dtype, const void* bias,
                  int m, int n, int k, int group, lq_stream_t stream);
 
+/* Forces the tile configuration ("tactic") used by the GEMM of `kind` (process-wide); -1 restores
+ * the built-in static table.  Stands in for the CutlassGemmConfig argument of
+ * CutlassInt8GemmRunner<T>::gemm and the tactic cache of GemmPluginProfiler
+ * (kernels/cutlass_kernels/int8_gemm/int8_gemm.h:24-39, layers/gemm_utils/GemmProfiler.cc:78-143).
+ * Unknown tactic numbers make the next GEMM call fail with LQ_ERR_ARG. */
+int lq_gemm_set_tactic(lq_weight_kind_t kind, int tactic);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,7 +1,7 @@
 // Tiled quantized GEMM core for gfx950 (MI355X): C[M,N] = epilogue( A[M,K] . B[N,K]^T ).
 //
 // Data flow per workgroup (BM x BN output tile, K walked in steps of BKB bytes):
-//   HBM --128-bit loads--> VGPR --ds_write_b128--> LDS (2 stages) --ds_read_b128--> MFMA operands.
+//   HBM --16 B/lane direct-to-LDS transfers--> LDS (NSTAGE stages) --ds_read_b128--> MFMA operands.
 //   * B (weights) arrive in the rows32 layout [N/32][Kb/16][32][16]: the bytes a 32x32 MFMA
 //     needs for one k-step are 1 KiB contiguous in HBM and in LDS, so a lane's operand is a
 //     single 16-byte read at a lane-linear LDS address (conflict free).
@@ -20,6 +20,7 @@
 #pragma once
 
 #include <type_traits>
+#include <utility>
 
 #include "lq_common.h"
 
@@ -120,66 +121,100 @@ __device__ __forceinline__ float gelu_fast(float x) {
     return 0.5f * x * (1.0f + t);
 }
 
-template <int KIND, typename OutTag, int BM, int BN, int BKB, int WM, int WN>
+// One 16-byte-per-lane global -> LDS transfer without passing through registers: lane l of the
+// wavefront fetches 16 bytes at gbase + voff and the hardware writes them to LDS byte address
+// lds_addr + 16*l (lds_addr is wavefront-uniform, carried in M0).  Issued as inline assembly
+// because the compiler would otherwise make every later LDS read wait for all such transfers;
+// completion is awaited explicitly with wait_vmcnt<N>() before the workgroup barrier.
+__device__ __forceinline__ void dma16(const void* gbase, u32 voff, u32 lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(gbase) : "memory");
+}
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// Scheduling hint for a region that holds G MFMAs and NP LDS reads: keep them in the interleaved
+// order "reads for slot I, then MFMA I" instead of letting the scheduler cluster the reads.
+template <int NP, int G, int I> __device__ __forceinline__ void sched_slot() {
+    constexpr int n = (I + 1) * NP / G - I * NP / G;
+    if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x100, n, 0);  // DS read
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                       // MFMA
+}
+template <int NP, int G, int... I> __device__ __forceinline__ void sched_interleave(std::integer_sequence<int, I...>) {
+    (sched_slot<NP, G, I>(), ...);
+}
+
+template <int KIND, typename OutTag, int BM, int BN, int BKB, int WM, int WN, int NSTAGE>
 struct GemmKernel {
-    static constexpr int THREADS = WM * WN * 64;
+    static constexpr int NW = WM * WN;
+    static constexpr int THREADS = NW * 64;
     static constexpr int TM = BM / WM, TN = BN / WN;  // wavefront tile
     static constexpr int MT = TM / 32, NT = TN / 32;  // 32x32 MFMA tiles per wavefront
     static constexpr int CH = BKB / 16;               // 16-byte chunks per tile row
     static constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
-    static constexpr int SCALE_BYTES = (KIND == K_W4A4) ? (BM + BN) * (BKB / 32) * 4 : 0;
+    static constexpr int NGS = BKB / 32;  // W4A4 groups per k-tile (one group of 64 int4 = 32 bytes)
+    static constexpr int NS = NGS * (BM + BN);
+    static constexpr int SCALE_BYTES = (KIND == K_W4A4) ? NS * 4 : 0;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + SCALE_BYTES;
-    static constexpr int SMEM_BYTES = 2 * STAGE_BYTES;
-    static constexpr int ACH = A_BYTES / 16 / THREADS, BCH = B_BYTES / 16 / THREADS;
-    static_assert(A_BYTES % (16 * THREADS) == 0 && B_BYTES % (16 * THREADS) == 0, "tile/threads mismatch");
+    static constexpr int SMEM_BYTES = NSTAGE * STAGE_BYTES;
+    static constexpr int A_DMA = A_BYTES / 1024 / NW, B_DMA = B_BYTES / 1024 / NW;  // transfers per wavefront per tile
+    static constexpr int SCH = (KIND == K_W4A4) ? (NS + THREADS - 1) / THREADS : 1;
+    static_assert(A_BYTES % (1024 * NW) == 0 && B_BYTES % (1024 * NW) == 0, "tile/wavefront mismatch");
     static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of 32");
     static_assert(CH == 4 || CH == 8, "BKB must be 64 or 128");
+    static_assert(KIND != K_W4A4 || NSTAGE == 2, "the W4A4 scale staging assumes two stages");
+    static_assert((A_DMA + B_DMA) * NSTAGE < 64, "vmcnt is a 6-bit counter");
     using AccT = typename std::conditional<KIND == K_FP8, v16f, v16i>::type;
+    using FragT = typename std::conditional<KIND == K_FP8, v8i, v4i>::type;
+    static constexpr int KSTEP = (KIND == K_FP8) ? 64 : 32;  // operand bytes per MFMA k-step
+    static constexpr int KS = BKB / KSTEP;
 
     static __device__ __forceinline__ void run(const GemmParams& p, char* smem) {
-        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+        const int tid = threadIdx.x, lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const int wm = wave / WN, wn = wave % WN;
         int tm, tn;
         tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
         const int m0 = tm * BM, n0 = tn * BN;
         const int kb = p.kb;
         const int ktiles = kb / BKB;
-        const int nb_last = p.n / 32 - 1;
         const size_t b_block_stride = (size_t)(kb / 16) * 512;  // bytes per 32-row block in rows32 layout
+        const u32 smem_base = (u32)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
 
-        // ---- global -> register staging ------------------------------------------------------
-        uint4 ra[ACH], rb[BCH];
-        const uint8_t* a_src[ACH];
-        const uint8_t* b_src[BCH];
-        int a_dst[ACH];
+        // ---- global -> LDS transfer plan (per lane offsets are fixed; the bases advance with k) ----
+        const uint8_t* a_base = p.A + (size_t)m0 * kb;
+        const uint8_t* b_base = p.B + (size_t)(n0 / 32) * b_block_stride;
+        u32 a_voff[A_DMA], b_voff[B_DMA];
+        const int row_last = p.m - 1 - m0, blk_last = p.n / 32 - 1 - n0 / 32;
 #pragma unroll
-        for (int i = 0; i < ACH; ++i) {
-            int q = tid + i * THREADS, row = q / CH, c = q % CH;
-            int grow = min(m0 + row, p.m - 1);
-            a_src[i] = p.A + (size_t)grow * kb + c * 16;
-            a_dst[i] = row * BKB + ((c ^ chunk_swizzle<CH>(row)) << 4);
+        for (int i = 0; i < A_DMA; ++i) {
+            int slot = (wave * A_DMA + i) * 64 + lane;  // 16-byte slot inside the A stage
+            int row = slot / CH, c = (slot % CH) ^ chunk_swizzle<CH>(row);
+            a_voff[i] = (u32)min(row, row_last) * (u32)kb + c * 16;
         }
 #pragma unroll
-        for (int i = 0; i < BCH; ++i) {
-            int q = tid + i * THREADS, rblk = q / (BKB * 2), within = q % (BKB * 2);
-            int nb = min(n0 / 32 + rblk, nb_last);
-            b_src[i] = p.B + (size_t)nb * b_block_stride + within * 16;
+        for (int i = 0; i < B_DMA; ++i) {
+            int byteoff = (wave * B_DMA + i) * 1024;
+            int rblk = byteoff / (BKB * 32), within = byteoff % (BKB * 32);
+            b_voff[i] = (u32)((size_t)min(rblk, blk_last) * b_block_stride) + within + lane * 16;
         }
-        // W4A4 group scales of a k-tile staged as [NGS][BM] then [NGS][BN] floats (int4: one group
-        // of 64 values is 32 bytes); the activation scales absorb the 1/256 of the widened nibbles
-        constexpr int NGS = BKB / 32;
-        constexpr int NS = NGS * (BM + BN);
-        constexpr int SCH = (KIND == K_W4A4) ? (NS + THREADS - 1) / THREADS : 1;
         float rs[SCH];
         auto load_scale = [&](const void* base, size_t idx) -> float {
             if (p.scale_f16) return f16_bits_to_f32(static_cast<const unsigned short*>(base)[idx]);
             return static_cast<const float*>(base)[idx];
         };
-        auto load_tile = [&](int kt) {
+        auto issue_tile = [&](int kt, int stage) {
+            const uint8_t* ga = a_base + (size_t)kt * BKB;
+            const uint8_t* gb = b_base + (size_t)kt * (BKB * 32);
+            const u32 sa = smem_base + stage * STAGE_BYTES + wave * (A_DMA * 1024);
+            const u32 sb = smem_base + stage * STAGE_BYTES + A_BYTES + wave * (B_DMA * 1024);
 #pragma unroll
-            for (int i = 0; i < ACH; ++i) ra[i] = *reinterpret_cast<const uint4*>(a_src[i] + (size_t)kt * BKB);
+            for (int i = 0; i < A_DMA; ++i) dma16(ga, a_voff[i], sa + i * 1024);
 #pragma unroll
-            for (int i = 0; i < BCH; ++i) rb[i] = *reinterpret_cast<const uint4*>(b_src[i] + (size_t)kt * BKB * 32);
+            for (int i = 0; i < B_DMA; ++i) dma16(gb, b_voff[i], sb + i * 1024);
+        };
+        // W4A4 group scales of a k-tile, staged through registers as [NGS][BM] then [NGS][BN] floats
+        auto load_scales = [&](int kt) {
             if constexpr (KIND == K_W4A4) {
                 const int ng = p.k / 64;
 #pragma unroll
@@ -188,28 +223,21 @@ struct GemmKernel {
                     rs[i] = 0.0f;
                     if (s < NGS * BM) {
                         int g = s / BM, r = s % BM;
-                        int row = min(m0 + r, p.m - 1);
-                        rs[i] = load_scale(p.sA, (size_t)row * ng + kt * NGS + g) * 0.00390625f;
+                        rs[i] = load_scale(p.sA, (size_t)(m0 + min(r, row_last)) * ng + kt * NGS + g) * 0.00390625f;
                     } else if (s < NS) {
                         int t2 = s - NGS * BM;
                         int g = t2 / BN, r = t2 % BN;
-                        int row = min(n0 + r, p.n - 1);
-                        rs[i] = load_scale(p.sB, (size_t)row * ng + kt * NGS + g);
+                        rs[i] = load_scale(p.sB, (size_t)min(n0 + r, p.n - 1) * ng + kt * NGS + g);
                     }
                 }
             }
         };
-        auto store_tile = [&](int stage) {
-            char* sa = smem + stage * STAGE_BYTES;
-            char* sb = sa + A_BYTES;
-#pragma unroll
-            for (int i = 0; i < ACH; ++i) *reinterpret_cast<uint4*>(sa + a_dst[i]) = ra[i];
-#pragma unroll
-            for (int i = 0; i < BCH; ++i) *reinterpret_cast<uint4*>(sb + (tid + i * THREADS) * 16) = rb[i];
+        auto store_scales = [&](int stage) {
             if constexpr (KIND == K_W4A4) {
+                float* ss = reinterpret_cast<float*>(smem + stage * STAGE_BYTES + A_BYTES + B_BYTES);
 #pragma unroll
                 for (int i = 0; i < SCH; ++i)
-                    if (tid + i * THREADS < NS) reinterpret_cast<float*>(sb + B_BYTES)[tid + i * THREADS] = rs[i];
+                    if (tid + i * THREADS < NS) ss[tid + i * THREADS] = rs[i];
             }
         };
 
@@ -226,75 +254,70 @@ struct GemmKernel {
                     if constexpr (KIND == K_W4A4) res[i][j][v] = 0.0f;
                 }
 
+        // ---- LDS -> register operand fragments ---------------------------------------------------
         const int lr = lane & 31, lh = lane >> 5;
+        const int xrow = wm * TM + lr;           // activation row of this lane inside the tile (+32 per MFMA tile)
+        const int xsw = chunk_swizzle<CH>(xrow);  // same for xrow + 32*i (only the low five row bits enter)
+        const int w_off = wn * NT * (BKB * 32) + lane * 16;
+        auto ldsv = [&](const char* ptr) -> v4i { return *reinterpret_cast<const v4i*>(ptr); };
+        auto load_frags = [&](const char* sa, const char* sb, int ks, FragT* w, FragT* x) {
+            if constexpr (KIND == K_FP8) {
+#pragma unroll
+                for (int j = 0; j < NT; ++j) {
+                    v4i lo = ldsv(sb + w_off + j * (BKB * 32) + ks * 2048);
+                    v4i hi = ldsv(sb + w_off + j * (BKB * 32) + ks * 2048 + 1024);
+                    w[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                }
+#pragma unroll
+                for (int i = 0; i < MT; ++i) {
+                    const char* rowp = sa + (xrow + i * 32) * BKB;
+                    v4i lo = ldsv(rowp + (((4 * ks + lh) ^ xsw) << 4));
+                    v4i hi = ldsv(rowp + (((4 * ks + 2 + lh) ^ xsw) << 4));
+                    x[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < NT; ++j) w[j] = ldsv(sb + w_off + j * (BKB * 32) + ks * 1024);
+#pragma unroll
+                for (int i = 0; i < MT; ++i) x[i] = ldsv(sa + (xrow + i * 32) * BKB + (((2 * ks + lh) ^ xsw) << 4));
+            }
+        };
+        auto widen = [](const v4i& q, int half) -> v4i {  // int4 -> int8 * 16: even nibbles, odd nibbles
+            int d0 = q[2 * half], d1 = q[2 * half + 1];
+            return v4i{(int)(((u32)d0 << 4) & 0xF0F0F0F0u), (int)((u32)d0 & 0xF0F0F0F0u),
+                       (int)(((u32)d1 << 4) & 0xF0F0F0F0u), (int)((u32)d1 & 0xF0F0F0F0u)};
+        };
+
         auto compute_tile = [&](int stage) {
             const char* sa = smem + stage * STAGE_BYTES;
             const char* sb = sa + A_BYTES;
-            if constexpr (KIND == K_INT8) {
+            if constexpr (KIND != K_W4A4) {
+                FragT w[2][NT], x[2][MT];
+                load_frags(sa, sb, 0, w[0], x[0]);
 #pragma unroll
-                for (int ks = 0; ks < BKB / 32; ++ks) {
-                    v4i w[NT], x[MT];
-#pragma unroll
-                    for (int j = 0; j < NT; ++j)
-                        w[j] = *reinterpret_cast<const v4i*>(sb + (wn * NT + j) * (BKB * 32) + ks * 1024 + lane * 16);
-#pragma unroll
-                    for (int i = 0; i < MT; ++i) {
-                        int row = wm * TM + i * 32 + lr, c = 2 * ks + lh;
-                        x[i] = *reinterpret_cast<const v4i*>(sa + row * BKB + ((c ^ chunk_swizzle<CH>(row)) << 4));
-                    }
+                for (int ks = 0; ks < KS; ++ks) {
+                    if (ks + 1 < KS) load_frags(sa, sb, ks + 1, w[(ks + 1) & 1], x[(ks + 1) & 1]);
 #pragma unroll
                     for (int i = 0; i < MT; ++i)
 #pragma unroll
-                        for (int j = 0; j < NT; ++j)
-                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[j], x[i], acc[i][j], 0, 0, 0);
+                        for (int j = 0; j < NT; ++j) {
+                            if constexpr (KIND == K_FP8)
+                                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w[ks & 1][j], x[ks & 1][i], acc[i][j],
+                                                                                           0, 0, 0, 0, 0, 0);
+                            else
+                                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[ks & 1][j], x[ks & 1][i], acc[i][j], 0, 0, 0);
+                        }
                 }
-            } else if constexpr (KIND == K_FP8) {
-#pragma unroll
-                for (int ks = 0; ks < BKB / 64; ++ks) {
-                    v8i w[NT], x[MT];
-#pragma unroll
-                    for (int j = 0; j < NT; ++j) {
-                        const char* base = sb + (wn * NT + j) * (BKB * 32) + ks * 2048 + lane * 16;
-                        v4i lo = *reinterpret_cast<const v4i*>(base);
-                        v4i hi = *reinterpret_cast<const v4i*>(base + 1024);
-                        w[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    }
-#pragma unroll
-                    for (int i = 0; i < MT; ++i) {
-                        int row = wm * TM + i * 32 + lr, c0 = 4 * ks + lh, sw = chunk_swizzle<CH>(row);
-                        v4i lo = *reinterpret_cast<const v4i*>(sa + row * BKB + ((c0 ^ sw) << 4));
-                        v4i hi = *reinterpret_cast<const v4i*>(sa + row * BKB + (((c0 + 2) ^ sw) << 4));
-                        x[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    }
-#pragma unroll
-                    for (int i = 0; i < MT; ++i)
-#pragma unroll
-                        for (int j = 0; j < NT; ++j)
-                            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w[j], x[i], acc[i][j], 0, 0, 0, 0, 0, 0);
-                }
-            } else {  // W4A4: one 64-value group = 32 bytes = chunks (2g, 2g+1)
+            } else {  // W4A4: one 64-value group = 32 bytes = two 16-byte chunks = two int8 k-steps
                 const float* ssa = reinterpret_cast<const float*>(sb + B_BYTES);  // [NGS][BM]
                 const float* ssb = ssa + NGS * BM;                                 // [NGS][BN]
 #pragma unroll
                 for (int g = 0; g < NGS; ++g) {
                     v4i wq[NT], xq[MT];
-#pragma unroll
-                    for (int j = 0; j < NT; ++j)
-                        wq[j] = *reinterpret_cast<const v4i*>(sb + (wn * NT + j) * (BKB * 32) + g * 1024 + lane * 16);
-#pragma unroll
-                    for (int i = 0; i < MT; ++i) {
-                        int row = wm * TM + i * 32 + lr, c = 2 * g + lh;
-                        xq[i] = *reinterpret_cast<const v4i*>(sa + row * BKB + ((c ^ chunk_swizzle<CH>(row)) << 4));
-                    }
+                    load_frags(sa, sb, g, wq, xq);
                     float sa_l[MT];
 #pragma unroll
-                    for (int i = 0; i < MT; ++i) sa_l[i] = ssa[g * BM + wm * TM + i * 32 + lr];
-                    // widen: even nibbles -> (d << 4) & 0xF0F0F0F0, odd nibbles -> d & 0xF0F0F0F0
-                    auto widen = [](const v4i& q, int half) -> v4i {
-                        int d0 = q[2 * half], d1 = q[2 * half + 1];
-                        return v4i{(int)(((u32)d0 << 4) & 0xF0F0F0F0u), (int)((u32)d0 & 0xF0F0F0F0u),
-                                   (int)(((u32)d1 << 4) & 0xF0F0F0F0u), (int)((u32)d1 & 0xF0F0F0F0u)};
-                    };
+                    for (int i = 0; i < MT; ++i) sa_l[i] = ssa[g * BM + xrow + i * 32];
 #pragma unroll
                     for (int j = 0; j < NT; ++j) {
                         v4i w0 = widen(wq[j], 0), w1 = widen(wq[j], 1);
@@ -319,42 +342,156 @@ struct GemmKernel {
             }
         };
 
-        // ---- main loop: 2 LDS stages, one barrier per k-tile -------------------------------------
-        load_tile(0);
-        store_tile(0);
-        __syncthreads();
-        for (int kt = 0; kt < ktiles; ++kt) {
-            if (kt + 1 < ktiles) load_tile(kt + 1);
-            compute_tile(kt & 1);
-            if (kt + 1 < ktiles) store_tile((kt + 1) & 1);
+        // ---- main loop ---------------------------------------------------------------------------------
+        // Tile t lives in LDS stage t % NSTAGE.  INT8/FP8: operand fragments are double-buffered in
+        // registers ACROSS tile boundaries: at the last k-step of tile kt a wavefront waits for its own
+        // transfers of tile kt+1, passes the workgroup barrier (after which tile kt+1 is complete and
+        // nobody reads stage kt % NSTAGE any more), re-arms that stage with tile kt+NSTAGE, prefetches
+        // the first fragments of tile kt+1 and only then issues the MFMAs of the step -- so the matrix
+        // pipe always has queued work while wavefronts sit in the barrier.  One barrier per tile.
+        // Every iteration issues exactly one tile of transfers (past the end it re-fetches the last
+        // tile into a stage nobody reads again), which makes the vmcnt thresholds compile-time values.
+        constexpr int PER_TILE = A_DMA + B_DMA;
+        if constexpr (KIND != K_W4A4) {
+            // Operand fragments as 16-byte pieces (an fp8 fragment is two pieces), so that the LDS reads
+            // of the next k-step can be interleaved one by one with the MFMAs of the current step.
+            constexpr int PPF = (KIND == K_FP8) ? 2 : 1;
+            constexpr int KCH = KSTEP / 16;  // chunks per k-step
+            constexpr int NPIECE = (NT + MT) * PPF;
+            constexpr int NMFMA = MT * NT;
+            v4i wp[2][NT][PPF], xp[2][MT][PPF];
+            // piece order follows first use: x0, w0..w(NT-1), x1..x(MT-1)
+            auto load_piece = [&](const char* sa, int ks, int buf, int pc) {
+                const int f = pc / PPF, h = pc % PPF;
+                if (f == 0 || f > NT) {
+                    const int i = f == 0 ? 0 : f - NT;
+                    xp[buf][i][h] = ldsv(sa + (xrow + i * 32) * BKB + (((KCH * ks + lh + 2 * h) ^ xsw) << 4));
+                } else {
+                    const int j = f - 1;
+                    wp[buf][j][h] = ldsv(sa + A_BYTES + w_off + j * (BKB * 32) + ks * (KSTEP * 32) + h * 1024);
+                }
+            };
+            auto do_mfma = [&](int buf, int idx) {
+                const int i = idx / NT, j = idx % NT;
+                if constexpr (KIND == K_FP8) {
+                    v8i w = __builtin_shufflevector(wp[buf][j][0], wp[buf][j][PPF - 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                    v8i x = __builtin_shufflevector(xp[buf][i][0], xp[buf][i][PPF - 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w, x, acc[i][j], 0, 0, 0, 0, 0, 0);
+                } else {
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wp[buf][j][0], xp[buf][i][0], acc[i][j], 0, 0, 0);
+                }
+            };
+            auto tile_iter = [&](int kt, auto parity) {
+                constexpr int P = decltype(parity)::value;
+                const char* sa = smem + (kt % NSTAGE) * STAGE_BYTES;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const int cur = (P + ks) & 1, nxt = cur ^ 1;
+                    if (ks + 1 < KS) {
+                        // MFMAs of this step interleaved with the fragment reads of the next step
+#pragma unroll
+                        for (int idx = 0; idx < NMFMA; ++idx) {
+#pragma unroll
+                            for (int pc = idx * NPIECE / NMFMA; pc < (idx + 1) * NPIECE / NMFMA; ++pc)
+                                load_piece(sa, ks + 1, nxt, pc);
+                            do_mfma(cur, idx);
+                        }
+                        sched_interleave<NPIECE, NMFMA>(std::make_integer_sequence<int, NMFMA>{});
+                    } else {
+                        // last step of the tile: half of the MFMAs go ahead of the barrier so that the matrix
+                        // pipe has queued work while the wavefront waits; the other half is interleaved with
+                        // the first fragment reads of the next tile.
+                        constexpr int H = NMFMA / 2, R = NMFMA - H;
+#pragma unroll
+                        for (int idx = 0; idx < H; ++idx) do_mfma(cur, idx);
+                        __builtin_amdgcn_sched_barrier(0);
+                        wait_vmcnt<PER_TILE*(NSTAGE - 2)>();
+                        __syncthreads();
+                        issue_tile(min(kt + NSTAGE, ktiles - 1), kt % NSTAGE);
+                        __builtin_amdgcn_sched_barrier(0);
+                        const char* sn = smem + ((kt + 1) % NSTAGE) * STAGE_BYTES;
+#pragma unroll
+                        for (int idx = 0; idx < R; ++idx) {
+#pragma unroll
+                            for (int pc = idx * NPIECE / R; pc < (idx + 1) * NPIECE / R; ++pc) load_piece(sn, 0, nxt, pc);
+                            do_mfma(cur, H + idx);
+                        }
+                        sched_interleave<NPIECE, R>(std::make_integer_sequence<int, R>{});
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            };
+#pragma unroll
+            for (int s = 0; s < NSTAGE; ++s) issue_tile(min(s, ktiles - 1), s);
+            wait_vmcnt<PER_TILE*(NSTAGE - 1)>();
             __syncthreads();
+#pragma unroll
+            for (int pc = 0; pc < NPIECE; ++pc) load_piece(smem, 0, 0, pc);
+            int kt = 0;
+            if constexpr (KS % 2 == 1) {
+                for (; kt + 1 < ktiles; kt += 2) {
+                    tile_iter(kt, std::integral_constant<int, 0>{});
+                    tile_iter(kt + 1, std::integral_constant<int, 1>{});
+                }
+                if (kt < ktiles) tile_iter(kt, std::integral_constant<int, 0>{});
+            } else {
+                for (; kt < ktiles; ++kt) tile_iter(kt, std::integral_constant<int, 0>{});
+            }
+        } else {
+            load_scales(0);
+            issue_tile(0, 0);
+            store_scales(0);
+            for (int kt = 0; kt < ktiles; ++kt) {
+                wait_vmcnt<0>();
+                __syncthreads();
+                issue_tile(min(kt + 1, ktiles - 1), (kt + 1) % NSTAGE);
+                if (kt + 1 < ktiles) load_scales(kt + 1);
+                compute_tile(kt % NSTAGE);
+                if (kt + 1 < ktiles) store_scales((kt + 1) % NSTAGE);
+            }
         }
+        wait_vmcnt<0>();
+        __syncthreads();  // every transfer has landed and nobody reads operands any more: LDS is reusable
 
-        // ---- epilogue -------------------------------------------------------------------------------
+        // ---- epilogue -------------------------------------------------------------------------------------
+        // Each wavefront turns one 32-row band of its tile at a time into output values (dequant scales,
+        // bias, activation), parks it in a private LDS strip laid out [row][n], and writes it back with
+        // rows contiguous, so that every global store covers whole 128-byte (or longer) row segments.
+        constexpr bool kI32 = std::is_same<OutTag, I32Tag>::value;
+        constexpr int ESZ = (std::is_same<OutTag, F16Tag>::value || std::is_same<OutTag, BF16Tag>::value) ? 2 : 4;
+        constexpr int CB = 4 * ESZ;        // bytes of the four consecutive n one lane produces per register quad
+        constexpr int PITCH = TN * ESZ + CB;  // odd multiple of CB: conflict-free column-wise writes
+        constexpr int LPR = TN / 4;        // lanes per output row on the way out
+        constexpr int RPI = 64 / LPR;      // rows per store instruction
+        static_assert(NW * 32 * PITCH <= SMEM_BYTES, "epilogue strip does not fit in the operand stages");
+        static_assert(64 % LPR == 0 && 32 % RPI == 0, "wave tile width must be 32, 64, 128 or 256");
+        char* strip = smem + wave * (32 * PITCH);
         float alpha = 1.0f;
         if constexpr (KIND == K_FP8) alpha = p.a_scale[0] * p.b_scale[0];
+        const bool direct = (KIND == K_FP8) && p.residual != nullptr;  // residual add needs the fp32 value
+        const int out_row = lane / LPR, out_n = n0 + wn * TN + (lane % LPR) * 4;
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             const int m = m0 + wm * TM + i * 32 + lr;
             float arow = 1.0f;
-            if constexpr (KIND == K_INT8 && !std::is_same<OutTag, I32Tag>::value)
-                arow = p.alpha_row[p.per_token ? min(m, p.m - 1) : 0];
+            if constexpr (KIND == K_INT8 && !kI32) arow = p.alpha_row[p.per_token ? min(m, p.m - 1) : 0];
 #pragma unroll
             for (int j = 0; j < NT; ++j) {
                 const int nbase = n0 + wn * TN + j * 32;
-                if (nbase >= p.n || m >= p.m) continue;
+                const bool ncol_ok = nbase < p.n;
 #pragma unroll
                 for (int q4 = 0; q4 < 4; ++q4) {
                     const int n = nbase + q4 * 8 + lh * 4;
-                    const size_t idx = (size_t)m * p.n + n;
-                    if constexpr (std::is_same<OutTag, I32Tag>::value) {
-                        *reinterpret_cast<int4*>(static_cast<int*>(p.C) + idx) =
+                    char* spot = strip + lr * PITCH + (j * 32 + q4 * 8 + lh * 4) * ESZ;
+                    if constexpr (kI32) {
+                        *reinterpret_cast<int4*>(spot) =
                             make_int4(acc[i][j][q4 * 4], acc[i][j][q4 * 4 + 1], acc[i][j][q4 * 4 + 2], acc[i][j][q4 * 4 + 3]);
                     } else {
                         float y[4], b[4] = {0.f, 0.f, 0.f, 0.f};
-                        if (p.bias != nullptr) OutStore<OutTag>::load4(p.bias, n, b);
+                        if (p.bias != nullptr && ncol_ok) OutStore<OutTag>::load4(p.bias, n, b);
                         if constexpr (KIND == K_INT8) {
-                            float4 ac = *reinterpret_cast<const float4*>(p.alpha_col + n);
+                            float4 ac = make_float4(0.f, 0.f, 0.f, 0.f);
+                            if (ncol_ok) ac = *reinterpret_cast<const float4*>(p.alpha_col + n);
                             const float acv[4] = {ac.x, ac.y, ac.z, ac.w};
 #pragma unroll
                             for (int t = 0; t < 4; ++t) {
@@ -368,11 +505,16 @@ struct GemmKernel {
                                 if (p.bias != nullptr) y[t] = y[t] + b[t];
                                 if (p.gelu) y[t] = gelu_fast(y[t]);
                             }
-                            if (p.residual != nullptr) {
-                                float rr[4];
-                                OutStore<OutTag>::load4(p.residual, idx, rr);
+                            if (direct) {
+                                if (ncol_ok && m < p.m) {
+                                    const size_t idx = (size_t)m * p.n + n;
+                                    float rr[4];
+                                    OutStore<OutTag>::load4(p.residual, idx, rr);
 #pragma unroll
-                                for (int t = 0; t < 4; ++t) y[t] = y[t] + p.beta * rr[t];
+                                    for (int t = 0; t < 4; ++t) y[t] = y[t] + p.beta * rr[t];
+                                    OutStore<OutTag>::store4(p.C, idx, y);
+                                }
+                                continue;
                             }
                         } else {
 #pragma unroll
@@ -381,26 +523,45 @@ struct GemmKernel {
                                 if (p.bias != nullptr) y[t] = y[t] + b[t];
                             }
                         }
-                        OutStore<OutTag>::store4(p.C, idx, y);
+                        OutStore<OutTag>::store4(spot, 0, y);
                     }
+                }
+            }
+            if (direct) continue;
+            // strip -> global, rows contiguous (the wavefront's own LDS accesses complete in order)
+#pragma unroll
+            for (int t = 0; t < 32 / RPI; ++t) {
+                const int row = t * RPI + out_row;
+                const int mo = m0 + wm * TM + i * 32 + row;
+                const char* src = strip + row * PITCH + (lane % LPR) * CB;
+                if constexpr (ESZ == 2) {
+                    uint2 v = *reinterpret_cast<const uint2*>(src);
+                    if (mo < p.m && out_n < p.n)
+                        *reinterpret_cast<uint2*>(static_cast<char*>(p.C) + ((size_t)mo * p.n + out_n) * 2) = v;
+                } else {
+                    uint4 v = *reinterpret_cast<const uint4*>(src);
+                    if (mo < p.m && out_n < p.n)
+                        *reinterpret_cast<uint4*>(static_cast<char*>(p.C) + ((size_t)mo * p.n + out_n) * 4) = v;
                 }
             }
         }
     }
 };
 
-template <int KIND, typename OutTag, int BM, int BN, int BKB, int WM, int WN>
-__global__ __launch_bounds__(WM* WN * 64) void gemm_kernel(GemmParams p) {
+// 256-thread configurations are meant to run two workgroups per CU (two wavefronts per SIMD), so that
+// one workgroup's barrier waits, pipeline fill and epilogue overlap with the other's MFMA work.
+template <int KIND, typename OutTag, int BM, int BN, int BKB, int WM, int WN, int NSTAGE>
+__global__ __launch_bounds__(WM* WN * 64, 2) void gemm_kernel(GemmParams p) {
     extern __shared__ __attribute__((aligned(16))) char lq_smem[];
-    GemmKernel<KIND, OutTag, BM, BN, BKB, WM, WN>::run(p, lq_smem);
+    GemmKernel<KIND, OutTag, BM, BN, BKB, WM, WN, NSTAGE>::run(p, lq_smem);
 }
 
-template <int KIND, typename OutTag, int BM, int BN, int BKB, int WM, int WN>
+template <int KIND, typename OutTag, int BM, int BN, int BKB, int WM, int WN, int NSTAGE>
 static int launch_gemm(GemmParams p, hipStream_t st) {
-    using GK = GemmKernel<KIND, OutTag, BM, BN, BKB, WM, WN>;
+    using GK = GemmKernel<KIND, OutTag, BM, BN, BKB, WM, WN, NSTAGE>;
     p.tiles_m = (p.m + BM - 1) / BM;
     p.tiles_n = (p.n + BN - 1) / BN;
-    auto kern = gemm_kernel<KIND, OutTag, BM, BN, BKB, WM, WN>;
+    auto kern = gemm_kernel<KIND, OutTag, BM, BN, BKB, WM, WN, NSTAGE>;
     static bool attr_done = false;  // raising the dynamic LDS limit is idempotent; races are benign
     if (!attr_done && GK::SMEM_BYTES > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,

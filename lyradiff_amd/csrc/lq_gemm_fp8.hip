@@ -6,12 +6,24 @@
 
 namespace lq {
 
+int g_tactic_fp8 = -1;
+
 template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
-    const long t256 = (long)((p.m + 255) / 256) * ((p.n + 255) / 256);
-    const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
-    if (t256 >= 192) return launch_gemm<K_FP8, OutTag, 256, 256, 64, 2, 4>(p, st);
-    if (t128 >= 192) return launch_gemm<K_FP8, OutTag, 128, 128, 64, 2, 2>(p, st);
-    return launch_gemm<K_FP8, OutTag, 64, 64, 64, 2, 2>(p, st);
+    int t = g_tactic_fp8;
+    if (t < 0) {
+        const long t256 = (long)((p.m + 255) / 256) * ((p.n + 255) / 256);
+        const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
+        t = t256 >= 192 ? 0 : (t128 >= 192 ? 2 : 3);
+    }
+    switch (t) {
+        case 0: return launch_gemm<K_FP8, OutTag, 256, 256, 64, 2, 4, 3>(p, st);
+        case 1: return launch_gemm<K_FP8, OutTag, 256, 256, 128, 2, 4, 2>(p, st);
+        case 2: return launch_gemm<K_FP8, OutTag, 128, 128, 64, 2, 2, 3>(p, st);
+        case 3: return launch_gemm<K_FP8, OutTag, 64, 64, 64, 2, 2, 3>(p, st);
+        case 4: return launch_gemm<K_FP8, OutTag, 128, 256, 64, 2, 2, 3>(p, st);
+        case 5: return launch_gemm<K_FP8, OutTag, 256, 128, 64, 2, 2, 3>(p, st);
+        default: set_error("lq_gemm_fp8: unknown tactic %d", t); return LQ_ERR_ARG;
+    }
 }
 
 }  // namespace lq

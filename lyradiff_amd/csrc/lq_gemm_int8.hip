@@ -6,14 +6,26 @@
 
 namespace lq {
 
+int g_tactic_int8 = -1;  // -1: static table below; otherwise forced (see lq_gemm_set_tactic)
+
 template <typename OutTag> static int run_int8(GemmParams p, hipStream_t st) {
     // static tile table in place of the reference's run-time tactic profiler
     // (layers/gemm_utils/GemmProfiler.cc:78-127): largest tile that still fills the 256 CUs.
-    const long t256 = (long)((p.m + 255) / 256) * ((p.n + 255) / 256);
-    const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
-    if (t256 >= 192) return launch_gemm<K_INT8, OutTag, 256, 256, 64, 2, 4>(p, st);
-    if (t128 >= 192) return launch_gemm<K_INT8, OutTag, 128, 128, 64, 2, 2>(p, st);
-    return launch_gemm<K_INT8, OutTag, 64, 64, 64, 2, 2>(p, st);
+    int t = g_tactic_int8;
+    if (t < 0) {
+        const long t256 = (long)((p.m + 255) / 256) * ((p.n + 255) / 256);
+        const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
+        t = t256 >= 192 ? 0 : (t128 >= 192 ? 2 : 3);
+    }
+    switch (t) {
+        case 0: return launch_gemm<K_INT8, OutTag, 256, 256, 64, 2, 4, 3>(p, st);
+        case 1: return launch_gemm<K_INT8, OutTag, 256, 256, 128, 2, 4, 2>(p, st);
+        case 2: return launch_gemm<K_INT8, OutTag, 128, 128, 64, 2, 2, 3>(p, st);
+        case 3: return launch_gemm<K_INT8, OutTag, 64, 64, 64, 2, 2, 3>(p, st);
+        case 4: return launch_gemm<K_INT8, OutTag, 128, 256, 64, 2, 2, 3>(p, st);
+        case 5: return launch_gemm<K_INT8, OutTag, 256, 128, 64, 2, 2, 3>(p, st);
+        default: set_error("lq_gemm_int8: unknown tactic %d", t); return LQ_ERR_ARG;
+    }
 }
 
 }  // namespace lq

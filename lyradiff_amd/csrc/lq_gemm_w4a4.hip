@@ -6,10 +6,19 @@
 
 namespace lq {
 
+int g_tactic_w4a4 = -1;
+
 template <typename OutTag> static int run_w4a4(GemmParams p, hipStream_t st) {
-    const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
-    if (t128 >= 192) return launch_gemm<K_W4A4, OutTag, 128, 128, 64, 2, 2>(p, st);
-    return launch_gemm<K_W4A4, OutTag, 64, 64, 64, 2, 2>(p, st);
+    int t = g_tactic_w4a4;
+    if (t < 0) {
+        const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
+        t = t128 >= 192 ? 0 : 1;
+    }
+    switch (t) {
+        case 0: return launch_gemm<K_W4A4, OutTag, 128, 128, 64, 2, 2, 2>(p, st);
+        case 1: return launch_gemm<K_W4A4, OutTag, 64, 64, 64, 2, 2, 2>(p, st);
+        default: set_error("lq_gemm_w4a4: unknown tactic %d", t); return LQ_ERR_ARG;
+    }
 }
 
 }  // namespace lq

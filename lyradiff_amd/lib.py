@@ -35,6 +35,7 @@ SYMBOLS = {
     "lq_gemm_int8": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _P]),
     "lq_gemm_fp8": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _P, _F, _I, _I, _I, _P]),
     "lq_gemm_w4a4": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P]),
+    "lq_gemm_set_tactic": (_I, [_I, _I]),
 }
 
 _lib = None
