@@ -45,9 +45,18 @@ struct F32Tag {};
 
 __device__ __forceinline__ float bf16_bits_to_f32(u32 b) { return __uint_as_float(b << 16); }
 __device__ __forceinline__ u32 f32_to_bf16_bits(float f) {
-    u32 u = __float_as_uint(f);
-    u32 r = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
-    return (f != f) ? ((u >> 16) | 0x40u) : r;
+    return (u32)__builtin_bit_cast(unsigned short, (__bf16)f);  // v_cvt_pk_bf16_f32, RNE
+}
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u32 pack2_bf16(float a, float b) {  // one v_cvt_pk_bf16_f32
+    f32x2_t v = {a, b};
+    return __builtin_bit_cast(u32, __builtin_convertvector(v, bf16x2_t));
+}
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u32 pack2_f16(float a, float b) {
+    f32x2_t v = {a, b};
+    return __builtin_bit_cast(u32, __builtin_convertvector(v, f16x2_t));
 }
 __device__ __forceinline__ float f16_bits_to_f32(u32 h) {
     return (float)__builtin_bit_cast(_Float16, (unsigned short)h);

@@ -78,8 +78,8 @@ template <typename OutTag> struct OutStore;
 template <> struct OutStore<F16Tag> {
     static __device__ __forceinline__ void store4(void* C, size_t idx, const float* y) {
         uint2 o;
-        o.x = f32_to_f16_bits(y[0]) | (f32_to_f16_bits(y[1]) << 16);
-        o.y = f32_to_f16_bits(y[2]) | (f32_to_f16_bits(y[3]) << 16);
+        o.x = pack2_f16(y[0], y[1]);
+        o.y = pack2_f16(y[2], y[3]);
         *reinterpret_cast<uint2*>(static_cast<unsigned short*>(C) + idx) = o;
     }
     static __device__ __forceinline__ void load4(const void* P, size_t idx, float* y) {
@@ -91,8 +91,8 @@ template <> struct OutStore<F16Tag> {
 template <> struct OutStore<BF16Tag> {
     static __device__ __forceinline__ void store4(void* C, size_t idx, const float* y) {
         uint2 o;
-        o.x = f32_to_bf16_bits(y[0]) | (f32_to_bf16_bits(y[1]) << 16);
-        o.y = f32_to_bf16_bits(y[2]) | (f32_to_bf16_bits(y[3]) << 16);
+        o.x = pack2_bf16(y[0], y[1]);
+        o.y = pack2_bf16(y[2], y[3]);
         *reinterpret_cast<uint2*>(static_cast<unsigned short*>(C) + idx) = o;
     }
     static __device__ __forceinline__ void load4(const void* P, size_t idx, float* y) {
@@ -454,94 +454,101 @@ struct GemmKernel {
         __syncthreads();  // every transfer has landed and nobody reads operands any more: LDS is reusable
 
         // ---- epilogue -------------------------------------------------------------------------------------
-        // Each wavefront turns one 32-row band of its tile at a time into output values (dequant scales,
-        // bias, activation), parks it in a private LDS strip laid out [row][n], and writes it back with
-        // rows contiguous, so that every global store covers whole 128-byte (or longer) row segments.
+        // Each wavefront parks one 32-row band of raw 32-bit accumulators at a time in a private LDS
+        // strip laid out [row][n] (plus the band's per-token scales in the row padding), reads it back
+        // with rows contiguous -- a lane then owns four consecutive n of one row -- applies the dequant
+        // scales, bias and activation there and stores whole 128-byte (or longer) row segments.  The
+        // per-lane constants (bias, per-channel scales for the lane's four columns) are loaded once,
+        // BEFORE the first store: on this architecture loads and stores share one in-order counter, so a
+        // load issued after a store would have to wait for that store to be acknowledged by memory.
         constexpr bool kI32 = std::is_same<OutTag, I32Tag>::value;
         constexpr int ESZ = (std::is_same<OutTag, F16Tag>::value || std::is_same<OutTag, BF16Tag>::value) ? 2 : 4;
-        constexpr int CB = 4 * ESZ;        // bytes of the four consecutive n one lane produces per register quad
-        constexpr int PITCH = TN * ESZ + CB;  // odd multiple of CB: conflict-free column-wise writes
-        constexpr int LPR = TN / 4;        // lanes per output row on the way out
-        constexpr int RPI = 64 / LPR;      // rows per store instruction
+        constexpr int PITCH = TN * 4 + 16;  // strip row: TN raw values + one 16-byte pad slot
+        constexpr int LPR = TN / 4;         // lanes per output row on the way out
+        constexpr int RPI = 64 / LPR;       // rows per store instruction
         static_assert(NW * 32 * PITCH <= SMEM_BYTES, "epilogue strip does not fit in the operand stages");
         static_assert(64 % LPR == 0 && 32 % RPI == 0, "wave tile width must be 32, 64, 128 or 256");
         char* strip = smem + wave * (32 * PITCH);
-        float alpha = 1.0f;
-        if constexpr (KIND == K_FP8) alpha = p.a_scale[0] * p.b_scale[0];
-        const bool direct = (KIND == K_FP8) && p.residual != nullptr;  // residual add needs the fp32 value
         const int out_row = lane / LPR, out_n = n0 + wn * TN + (lane % LPR) * 4;
+        const bool n_ok = out_n < p.n;
+        float alpha = 1.0f, bias4[4] = {0.f, 0.f, 0.f, 0.f}, acol4[4] = {0.f, 0.f, 0.f, 0.f}, arow_l[MT];
+        if constexpr (KIND == K_FP8) alpha = p.a_scale[0] * p.b_scale[0];
+        if constexpr (!kI32) {
+            if (p.bias != nullptr && n_ok) OutStore<OutTag>::load4(p.bias, out_n, bias4);
+            if constexpr (KIND == K_INT8) {
+                if (n_ok) {
+                    float4 ac = *reinterpret_cast<const float4*>(p.alpha_col + out_n);
+                    acol4[0] = ac.x; acol4[1] = ac.y; acol4[2] = ac.z; acol4[3] = ac.w;
+                }
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+                    arow_l[i] = p.alpha_row[p.per_token ? min(m0 + wm * TM + i * 32 + lr, p.m - 1) : 0];
+            }
+        }
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
-            const int m = m0 + wm * TM + i * 32 + lr;
-            float arow = 1.0f;
-            if constexpr (KIND == K_INT8 && !kI32) arow = p.alpha_row[p.per_token ? min(m, p.m - 1) : 0];
 #pragma unroll
-            for (int j = 0; j < NT; ++j) {
-                const int nbase = n0 + wn * TN + j * 32;
-                const bool ncol_ok = nbase < p.n;
+            for (int j = 0; j < NT; ++j)
 #pragma unroll
                 for (int q4 = 0; q4 < 4; ++q4) {
-                    const int n = nbase + q4 * 8 + lh * 4;
-                    char* spot = strip + lr * PITCH + (j * 32 + q4 * 8 + lh * 4) * ESZ;
-                    if constexpr (kI32) {
-                        *reinterpret_cast<int4*>(spot) =
-                            make_int4(acc[i][j][q4 * 4], acc[i][j][q4 * 4 + 1], acc[i][j][q4 * 4 + 2], acc[i][j][q4 * 4 + 3]);
-                    } else {
-                        float y[4], b[4] = {0.f, 0.f, 0.f, 0.f};
-                        if (p.bias != nullptr && ncol_ok) OutStore<OutTag>::load4(p.bias, n, b);
-                        if constexpr (KIND == K_INT8) {
-                            float4 ac = make_float4(0.f, 0.f, 0.f, 0.f);
-                            if (ncol_ok) ac = *reinterpret_cast<const float4*>(p.alpha_col + n);
-                            const float acv[4] = {ac.x, ac.y, ac.z, ac.w};
-#pragma unroll
-                            for (int t = 0; t < 4; ++t) {
-                                y[t] = (float)acc[i][j][q4 * 4 + t] * (acv[t] * arow);
-                                if (p.bias != nullptr) y[t] = y[t] + b[t];
-                            }
-                        } else if constexpr (KIND == K_FP8) {
-#pragma unroll
-                            for (int t = 0; t < 4; ++t) {
-                                y[t] = acc[i][j][q4 * 4 + t] * alpha;
-                                if (p.bias != nullptr) y[t] = y[t] + b[t];
-                                if (p.gelu) y[t] = gelu_fast(y[t]);
-                            }
-                            if (direct) {
-                                if (ncol_ok && m < p.m) {
-                                    const size_t idx = (size_t)m * p.n + n;
-                                    float rr[4];
-                                    OutStore<OutTag>::load4(p.residual, idx, rr);
-#pragma unroll
-                                    for (int t = 0; t < 4; ++t) y[t] = y[t] + p.beta * rr[t];
-                                    OutStore<OutTag>::store4(p.C, idx, y);
-                                }
-                                continue;
-                            }
-                        } else {
-#pragma unroll
-                            for (int t = 0; t < 4; ++t) {
-                                y[t] = res[i][j][q4 * 4 + t];
-                                if (p.bias != nullptr) y[t] = y[t] + b[t];
-                            }
-                        }
-                        OutStore<OutTag>::store4(spot, 0, y);
-                    }
+                    char* spot = strip + lr * PITCH + (j * 32 + q4 * 8 + lh * 4) * 4;
+                    if constexpr (KIND == K_W4A4)
+                        *reinterpret_cast<float4*>(spot) = make_float4(res[i][j][q4 * 4], res[i][j][q4 * 4 + 1],
+                                                                       res[i][j][q4 * 4 + 2], res[i][j][q4 * 4 + 3]);
+                    else if constexpr (KIND == K_FP8)
+                        *reinterpret_cast<float4*>(spot) = make_float4(acc[i][j][q4 * 4], acc[i][j][q4 * 4 + 1],
+                                                                       acc[i][j][q4 * 4 + 2], acc[i][j][q4 * 4 + 3]);
+                    else
+                        *reinterpret_cast<int4*>(spot) = make_int4(acc[i][j][q4 * 4], acc[i][j][q4 * 4 + 1],
+                                                                   acc[i][j][q4 * 4 + 2], acc[i][j][q4 * 4 + 3]);
                 }
+            if constexpr (KIND == K_INT8 && !kI32) {
+                if (lh == 0) *reinterpret_cast<float*>(strip + lr * PITCH + TN * 4) = arow_l[i];
             }
-            if (direct) continue;
-            // strip -> global, rows contiguous (the wavefront's own LDS accesses complete in order)
+            // strip -> registers with rows contiguous, math, store (the wavefront's own LDS accesses
+            // complete in order, so no barrier is needed inside the wavefront)
 #pragma unroll
             for (int t = 0; t < 32 / RPI; ++t) {
                 const int row = t * RPI + out_row;
                 const int mo = m0 + wm * TM + i * 32 + row;
-                const char* src = strip + row * PITCH + (lane % LPR) * CB;
-                if constexpr (ESZ == 2) {
-                    uint2 v = *reinterpret_cast<const uint2*>(src);
-                    if (mo < p.m && out_n < p.n)
-                        *reinterpret_cast<uint2*>(static_cast<char*>(p.C) + ((size_t)mo * p.n + out_n) * 2) = v;
+                const char* src = strip + row * PITCH + (lane % LPR) * 16;
+                const bool ok = mo < p.m && n_ok;
+                const size_t idx = (size_t)mo * p.n + out_n;
+                if constexpr (kI32) {
+                    int4 v = *reinterpret_cast<const int4*>(src);
+                    if (ok) *reinterpret_cast<int4*>(static_cast<int*>(p.C) + idx) = v;
                 } else {
-                    uint4 v = *reinterpret_cast<const uint4*>(src);
-                    if (mo < p.m && out_n < p.n)
-                        *reinterpret_cast<uint4*>(static_cast<char*>(p.C) + ((size_t)mo * p.n + out_n) * 4) = v;
+                    float y[4];
+                    if constexpr (KIND == K_INT8) {
+                        int4 v = *reinterpret_cast<const int4*>(src);
+                        const float ar = *reinterpret_cast<const float*>(strip + row * PITCH + TN * 4);
+                        const int vi[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            y[e] = (float)vi[e] * (acol4[e] * ar);
+                            if (p.bias != nullptr) y[e] = y[e] + bias4[e];
+                        }
+                    } else {
+                        float4 v = *reinterpret_cast<const float4*>(src);
+                        const float vf[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            y[e] = (KIND == K_FP8) ? vf[e] * alpha : vf[e];
+                            if (p.bias != nullptr) y[e] = y[e] + bias4[e];
+                            if constexpr (KIND == K_FP8) {
+                                if (p.gelu) y[e] = gelu_fast(y[e]);
+                            }
+                        }
+                        if constexpr (KIND == K_FP8) {
+                            if (p.residual != nullptr && ok) {
+                                float rr[4];
+                                OutStore<OutTag>::load4(p.residual, idx, rr);
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) y[e] = y[e] + p.beta * rr[e];
+                            }
+                        }
+                    }
+                    if (ok) OutStore<OutTag>::store4(p.C, idx, y);
                 }
             }
         }

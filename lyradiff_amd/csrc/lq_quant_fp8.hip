@@ -34,18 +34,28 @@ template <typename Tag> __device__ __forceinline__ float load_one(const void* ba
 }
 
 // saturate-to-finite RNE conversion of two floats into the low or high half of a dword
+// (finite inputs and infinities; NaN lanes are patched by the caller)
 __device__ __forceinline__ u32 cvt2_e4m3(float a, float b, u32 old, bool hi) {
     float ca = __builtin_amdgcn_fmed3f(a, 448.0f, -448.0f);
     float cb = __builtin_amdgcn_fmed3f(b, 448.0f, -448.0f);
-    ca = (a != a) ? a : ca;  // keep NaN (-> 0x7F)
-    cb = (b != b) ? b : cb;
     return hi ? (u32)__builtin_amdgcn_cvt_pk_fp8_f32(ca, cb, (int)old, true)
               : (u32)__builtin_amdgcn_cvt_pk_fp8_f32(ca, cb, (int)old, false);
 }
+__device__ __forceinline__ u32 nan_code(float v) { return 0x7Fu | ((__float_as_uint(v) >> 24) & 0x80u); }
+// four floats -> four e4m3 codes; NaN -> 0x7F with the sign of the NaN (rare: one unordered
+// compare per pair decides whether the patch-up path runs at all)
 __device__ __forceinline__ u32 cvt4_e4m3(float a, float b, float c, float d) {
     u32 w = cvt2_e4m3(a, b, 0u, false);
-    return cvt2_e4m3(c, d, w, true);
+    w = cvt2_e4m3(c, d, w, true);
+    if (__builtin_expect(__builtin_isunordered(a, b) || __builtin_isunordered(c, d), 0)) {
+        if (a != a) w = (w & 0xFFFFFF00u) | nan_code(a);
+        if (b != b) w = (w & 0xFFFF00FFu) | (nan_code(b) << 8);
+        if (c != c) w = (w & 0xFF00FFFFu) | (nan_code(c) << 16);
+        if (d != d) w = (w & 0x00FFFFFFu) | (nan_code(d) << 24);
+    }
+    return w;
 }
+__device__ __forceinline__ u32 cvt1_e4m3(float a) { return cvt4_e4m3(a, 0.0f, 0.0f, 0.0f) & 0xFFu; }
 
 // Non-negative floats order like their bit patterns, so an integer atomic max works.  Thousands of
 // same-address atomics serialise in L2, so a workgroup first looks at the current value and only
@@ -101,7 +111,7 @@ __global__ __launch_bounds__(256) void fp8_cast_kernel(uint8_t* __restrict__ dst
     }
     if (blockIdx.x == 0) {
         size_t i = nchunks * E + threadIdx.x;
-        if (i < n) dst[i] = (uint8_t)(cvt2_e4m3(load_one<Tag>(src, i) * r, 0.0f, 0u, false) & 0xFFu);
+        if (i < n) dst[i] = (uint8_t)cvt1_e4m3(load_one<Tag>(src, i) * r);
     }
 }
 
@@ -112,7 +122,7 @@ __global__ __launch_bounds__(256) void fp8_cast_scalar_kernel(uint8_t* __restric
     const float s = scale[0];
     const float r = invert ? 1.0f / s : s;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
-        dst[i] = (uint8_t)(cvt2_e4m3(load_one<Tag>(src, i) * r, 0.0f, 0u, false) & 0xFFu);
+        dst[i] = (uint8_t)cvt1_e4m3(load_one<Tag>(src, i) * r);
 }
 template <typename Tag>
 __global__ __launch_bounds__(256) void fp8_amax_scalar_kernel(float* __restrict__ scale, const void* __restrict__ x, size_t n) {
