@@ -1,0 +1,251 @@
+// lyradiff_compat.h -- header-only C++ layer that re-creates, on top of the C ABI of lyraquant.h,
+// the names and argument meaning of the lyraDiff reference's quantized-linear interfaces, so that
+// reference-style call sites compile against liblyraquant.so with `cudaStream_t` spelled
+// `hipStream_t`.  Each entity cites what it stands in for (paths relative to the reference's
+// src/lyradiff/).  Errors follow the reference's convention: std::runtime_error with a
+// "[lyradiff Error][...]" prefix (kernels/cutlass_kernels/int8_gemm/int8_gemm_template.h:169-188).
+//
+// Differences a maintainer has to know:
+//   * the weight operand "B" of every GEMM is the rows32 layout produced once by
+//     repackWeight() / lq_repack_rows32 (same byte count as the [N,K] matrix);
+//   * workspaces are accepted and ignored; tactic profiling is a no-op (static table);
+//   * the SVDQuant low-rank branch of W4A4 is not built: passing LoRA pointers throws.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <hip/hip_bfloat16.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <memory>
+#include <stdexcept>
+#include <string>
+
+#include "lyraquant.h"
+
+namespace lyradiff {
+
+namespace detail {
+template <typename T> struct DType;
+template <> struct DType<float> { static constexpr lq_dtype_t value = LQ_F32; };
+template <> struct DType<__half> { static constexpr lq_dtype_t value = LQ_F16; };
+template <> struct DType<hip_bfloat16> { static constexpr lq_dtype_t value = LQ_BF16; };
+template <> struct DType<int32_t> { static constexpr lq_dtype_t value = LQ_I32; };
+inline void check(int status, const char* what) {
+    if (status != LQ_OK)
+        throw std::runtime_error(std::string("[lyradiff Error][") + what + "] " + lq_last_error());
+}
+}  // namespace detail
+
+// ---- utils/quantization.h:9-274 (the subset the quantized-linear path reads) -------------------------
+class QuantMode {
+public:
+    using BaseType = std::uint32_t;
+    explicit constexpr QuantMode(BaseType value) noexcept : mValue{value} {}
+    QuantMode() noexcept = default;
+    static constexpr QuantMode none() noexcept { return QuantMode(0); }
+    static constexpr QuantMode int4Weights() noexcept { return QuantMode(1u << 0); }
+    static constexpr QuantMode int8Weights() noexcept { return QuantMode(1u << 1); }
+    static constexpr QuantMode activations() noexcept { return QuantMode(1u << 2); }
+    static constexpr QuantMode perChannelScaling() noexcept { return QuantMode(1u << 3); }
+    static constexpr QuantMode perTokenScaling() noexcept { return QuantMode(1u << 4); }
+    static constexpr QuantMode perGroupScaling() noexcept { return QuantMode(1u << 5); }
+    constexpr BaseType value() const noexcept { return mValue; }
+    constexpr bool isSet(QuantMode const& m) const noexcept { return (mValue & m.mValue) == m.mValue; }
+    constexpr bool hasInt4Weights() const noexcept { return isSet(int4Weights()); }
+    constexpr bool hasInt8Weights() const noexcept { return isSet(int8Weights()); }
+    constexpr bool hasActivations() const noexcept { return isSet(activations()); }
+    constexpr bool hasPerChannelScaling() const noexcept { return isSet(perChannelScaling()); }
+    constexpr bool hasPerTokenScaling() const noexcept { return isSet(perTokenScaling()); }
+    constexpr bool hasPerGroupScaling() const noexcept { return isSet(perGroupScaling()); }
+    constexpr bool hasStaticActivationScaling() const noexcept { return !hasPerTokenScaling(); }
+    static constexpr QuantMode useSmoothQuant(bool perToken = false, bool perChannel = false) {
+        return QuantMode((1u << 1) | (1u << 2) | (perChannel ? 1u << 3 : 0u) | (perToken ? 1u << 4 : 0u));
+    }
+    constexpr bool operator==(QuantMode const& o) const noexcept { return mValue == o.mValue; }
+    constexpr bool operator!=(QuantMode const& o) const noexcept { return mValue != o.mValue; }
+
+private:
+    BaseType mValue{0};
+};
+
+// ---- kernels/quant_kernels/quant_kernels.h:8-37 --------------------------------------------------------
+template <typename T>
+void invokeSqInputQuant(int8_t* dst, const T* src, const float* pre_quant_scale, const float* input_quant_scale,
+                        QuantMode quant_mode, size_t batch_size, size_t seq_len, size_t dim, hipStream_t stream) {
+    detail::check(lq_sq_input_quant(dst, src, detail::DType<T>::value, pre_quant_scale, input_quant_scale,
+                                    quant_mode.hasPerTokenScaling(), batch_size * seq_len, dim, stream),
+                  "invokeSqInputQuant");
+}
+// dynamic per-token flavour (writes the per-token scales it used); no reference counterpart
+template <typename T>
+void invokeSqDynamicPerTokenQuant(int8_t* dst, float* token_scale, const T* src, const float* pre_quant_scale,
+                                  size_t batch_size, size_t seq_len, size_t dim, hipStream_t stream) {
+    detail::check(lq_sq_dynamic_quant(dst, token_scale, src, detail::DType<T>::value, pre_quant_scale,
+                                      batch_size * seq_len, dim, stream),
+                  "invokeSqDynamicPerTokenQuant");
+}
+template <typename T>
+void invokeSqOutputDequant(T* dst, const int32_t* src, const float* input_quant_scale, const float* weight_quant_scale,
+                           QuantMode quant_mode, size_t batch_size, size_t seq_len, size_t dim, hipStream_t stream) {
+    detail::check(lq_sq_output_dequant(dst, detail::DType<T>::value, src, input_quant_scale, weight_quant_scale,
+                                       quant_mode.hasPerTokenScaling(), batch_size * seq_len, dim, stream),
+                  "invokeSqOutputDequant");
+}
+template <typename T>
+void invokeGetINT8WeightScale(float* new_weight_scale, int8_t* quantized_weight, const T* weight,
+                              const float* pre_quant_scale, const size_t d_out, const size_t d_in,
+                              hipStream_t stream = 0) {
+    detail::check(lq_int8_weight_quant(new_weight_scale, quantized_weight, weight, detail::DType<T>::value,
+                                       pre_quant_scale, d_out, d_in, stream),
+                  "invokeGetINT8WeightScale");
+}
+
+// ---- kernels/quant_kernels/ffn_kernels_int8.h:12-21 ----------------------------------------------------
+template <typename T>
+void invokeFusedAddBiasGegluInt8O(int8_t* dst, const T* hidden_states, const T* bias, const float* pre_quant_scale,
+                                  const float* input_quant_scale, const int seq_len, const int dim,
+                                  const int batch_size, hipStream_t stream) {
+    detail::check(lq_geglu_int8(dst, hidden_states, bias, detail::DType<T>::value, pre_quant_scale, input_quant_scale,
+                                (size_t)seq_len * batch_size, dim, stream),
+                  "invokeFusedAddBiasGegluInt8O");
+}
+
+// ---- kernels/lora/load_lora.h:30-31 and utils/memory_utils.cu:441-446 ------------------------------------
+struct fp8_e4m3_t { uint8_t bits; };  // storage type standing in for __nv_fp8_e4m3
+template <typename T>
+void invokeGetFP8WeightScale(float* new_weight_scale, const T* weight, const size_t size, hipStream_t stream = 0) {
+    detail::check(lq_fp8_amax_scale(new_weight_scale, weight, detail::DType<T>::value, size, stream),
+                  "invokeGetFP8WeightScale");
+}
+template <typename T_IN>
+void invokeCudaD2DScaleCpyConvert(fp8_e4m3_t* tgt, const T_IN* src, const float* scale, bool invert_scale,
+                                  const size_t size, hipStream_t stream) {
+    detail::check(lq_fp8_scale_cast(reinterpret_cast<uint8_t*>(tgt), src, detail::DType<T_IN>::value, scale,
+                                    invert_scale, size, stream),
+                  "invokeCudaD2DScaleCpyConvert");
+}
+
+// ---- kernels/w4a4_gemm/w4a4_gemm.h:6-30 ------------------------------------------------------------------
+inline void invokeFusedQuantizeAndLoraDownSimple(float* Cptr, uint32_t* quantized_input, float* quantized_scale,
+                                                 const void* Aptr /* bf16 [m,k] */, const void* Bptr /* lora down */,
+                                                 const float* Smoothptr, int m, int n, int k, int group_dim = 64,
+                                                 hipStream_t stream = 0) {
+    (void)n;
+    if (Cptr != nullptr || Bptr != nullptr)
+        throw std::runtime_error("[lyradiff Error][invokeFusedQuantizeAndLoraDownSimple] the low-rank (LoRA-down) "
+                                 "branch is not built; pass null Cptr/Bptr");
+    detail::check(lq_w4a4_quantize(quantized_input, quantized_scale, LQ_F32, Aptr, LQ_BF16, Smoothptr, m, k, group_dim,
+                                   stream),
+                  "invokeFusedQuantizeAndLoraDownSimple");
+}
+inline void invokeFusedW4A4GemmAndLoraUp(void* Dptr /* bf16 [m,n] */, const void* Aptr, const void* Bptr_rows32,
+                                         const void* LoraAptr, const void* LoraBptr, const float* AweightScale,
+                                         const float* BweightScale, int m, int n, int k, int lora_k, int groups,
+                                         hipStream_t stream, const void* bias = nullptr) {
+    (void)lora_k;
+    if (LoraAptr != nullptr || LoraBptr != nullptr)
+        throw std::runtime_error("[lyradiff Error][invokeFusedW4A4GemmAndLoraUp] the low-rank (LoRA-up) branch is "
+                                 "not built; pass null LoRA pointers");
+    if (groups != k / 64)
+        throw std::runtime_error("[lyradiff Error][invokeFusedW4A4GemmAndLoraUp] groups must equal k / 64");
+    detail::check(lq_gemm_w4a4(Dptr, LQ_BF16, static_cast<const uint32_t*>(Aptr), static_cast<const uint8_t*>(Bptr_rows32),
+                               AweightScale, BweightScale, LQ_F32, bias, m, n, k, 64, stream),
+                  "invokeFusedW4A4GemmAndLoraUp");
+}
+
+// ---- one-time weight repack (role of kernels/cutlass_kernels/cutlass_preprocessors.cpp:484-530) -----------
+inline void repackWeight(void* dst_rows32, const void* src_row_major, lq_weight_kind_t kind, size_t n, size_t k,
+                         hipStream_t stream = 0) {
+    detail::check(lq_repack_rows32(static_cast<uint8_t*>(dst_rows32), static_cast<const uint8_t*>(src_row_major), n,
+                                   lq_weight_row_bytes(kind, k), stream),
+                  "repackWeight");
+}
+
+namespace gemm {
+
+// ---- layers/gemm_utils/SmoothQuantGemm.h:29-103, layers/gemm_utils/GemmProfiler.h:131-251 -----------------
+// The run-time tactic search is replaced by a static table inside the library, so the profiler is an
+// empty shell kept for signature compatibility.
+class SmoothQuantGemmPluginProfiler {
+public:
+    void setQuantMode(QuantMode const& quantMode) { mQuantMode = quantMode; }
+    QuantMode mQuantMode;
+};
+
+template <typename DataType>
+class SmoothQuantGemmPlugin {
+public:
+    using PluginProfilerPtr = std::shared_ptr<SmoothQuantGemmPluginProfiler>;
+    SmoothQuantGemmPlugin() = delete;
+    SmoothQuantGemmPlugin(const QuantMode& quantMode, PluginProfilerPtr const& profiler)
+        : mQuantMode(quantMode), mPluginProfiler(profiler) {}
+    SmoothQuantGemmPlugin<DataType>* clone() { return new SmoothQuantGemmPlugin<DataType>(*this); }
+    void configurePlugin(int maxM, int K, int N) { mMaxM = maxM; mK = K; mN = N; }
+    int initialize() { return 0; }  // nothing to profile
+    void terminate() {}
+    size_t getWorkspaceSize(int, int, int) { return 0; }
+    // C[m,n] = T(float(acc) * (alphaCol[n] * alphaRow[m or 0])); B is the rows32 layout of the [n,k] weight
+    void RunGemm(int8_t const* A, int8_t const* B, float const* alphaCol, float const* alphaRow, void* C, int m, int n,
+                 int k, char* /*workspacePtr*/, hipStream_t stream, const void* bias = nullptr) {
+        detail::check(lq_gemm_int8(C, detail::DType<DataType>::value, A, B, alphaCol, alphaRow,
+                                   mQuantMode.hasPerTokenScaling(), bias, m, n, k, stream),
+                      "SmoothQuantGemmPlugin::RunGemm");
+    }
+    QuantMode mQuantMode;
+
+private:
+    int mMaxM = 0, mK = 0, mN = 0;
+    PluginProfilerPtr mPluginProfiler;
+};
+
+}  // namespace gemm
+
+// stand-in for the cuBLAS transpose enum in the signature below
+enum cublasOperation_t { CUBLAS_OP_N = 0, CUBLAS_OP_T = 1 };
+
+// ---- utils/cublasMMWrapper.h:299-318,354-385 (the two quantized entry points) -----------------------------
+// DataType is the activation/output type the wrapper was configured with (setFP16GemmConfig /
+// setBF16GemmConfig in the reference).
+template <typename DataType>
+class cublasMMWrapper {
+public:
+    explicit cublasMMWrapper(hipStream_t stream, bool per_token_int8 = false)
+        : stream_(stream),
+          int8_runner_(QuantMode::useSmoothQuant(per_token_int8, true),
+                       std::make_shared<gemm::SmoothQuantGemmPluginProfiler>()) {}
+    void setStream(hipStream_t s) { stream_ = s; }
+    void profileGemmInt8(const int maxM, const int n, const int k) {
+        int8_runner_.configurePlugin(maxM, k, n);
+        int8_runner_.initialize();
+    }
+    void runGemmInt8(int8_t const* A, int8_t const* B, float const* alphaCol, float const* alphaRow, void* C, int m,
+                     int n, int k, char* workspacePtr, hipStream_t stream) {
+        int8_runner_.RunGemm(A, B, alphaCol, alphaRow, C, m, n, k, workspacePtr, stream);
+    }
+    // The reference calls this in cuBLAS column-major convention with the WEIGHT as "A":
+    //   GemmWithResidualAndBias(OP_T, OP_N, m=N_out, n=M_tokens, k, W, lda=k, w_scale, X, ldb=k, x_scale, C, ldc=N_out, ...)
+    // (layers/flux_attn_post_processor/FluxAttnPostFP8Processor.cc:146-163), i.e. the row-major product
+    // C[tokens, N_out] = X[tokens,k] . W[N_out,k]^T.  Only that (T, N) form exists in the reference's callers.
+    void GemmWithResidualAndBias(cublasOperation_t transa, cublasOperation_t transb, const int m, const int n,
+                                 const int k, const fp8_e4m3_t* A_weight_rows32, const int lda, const float* a_scale,
+                                 const fp8_e4m3_t* B_act, const int ldb, const float* b_scale, void* C, const int ldc,
+                                 const void* bias = nullptr, const void* Residual = nullptr, float f_alpha = 1.0f,
+                                 float f_beta = 0.0f, const bool is_gelu = false) {
+        if (transa != CUBLAS_OP_T || transb != CUBLAS_OP_N || lda != k || ldb != k || ldc != m || f_alpha != 1.0f)
+            throw std::runtime_error("[lyradiff Error][GemmWithResidualAndBias] only the (OP_T weight, OP_N activation, "
+                                     "lda = ldb = k, ldc = m, alpha = 1) form used by the FP8 blocks is supported");
+        if (Residual == nullptr) f_beta = 0.0f;  // utils/cublasMMWrapper.cc:1123-1125
+        detail::check(lq_gemm_fp8(C, detail::DType<DataType>::value, reinterpret_cast<const uint8_t*>(B_act),
+                                  reinterpret_cast<const uint8_t*>(A_weight_rows32), b_scale, a_scale, bias, is_gelu,
+                                  Residual, f_beta, /*tokens*/ n, /*out features*/ m, k, stream_),
+                      "GemmWithResidualAndBias");
+    }
+
+private:
+    hipStream_t stream_;
+    gemm::SmoothQuantGemmPlugin<DataType> int8_runner_;
+};
+
+}  // namespace lyradiff

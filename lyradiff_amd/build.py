@@ -62,7 +62,25 @@ def build(force: bool = False, jobs: int | None = None) -> str:
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
+    build_compat_check(force)
     return LIB
+
+
+def build_compat_check(force: bool = False) -> str:
+    """Compiles tests/cpp/compat_check.cpp (reference-style C++ call sites) against the library."""
+    src = os.path.join(ROOT, "tests", "cpp", "compat_check.cpp")
+    exe = os.path.join(ROOT, "tests", "cpp", "compat_check")
+    hdr = os.path.join(ROOT, "include", "lyradiff_compat.h")
+    if not os.path.exists(src):
+        return ""
+    if not force and os.path.exists(exe) and os.path.getmtime(exe) >= max(os.path.getmtime(src), os.path.getmtime(hdr), os.path.getmtime(LIB)):
+        return exe
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-Wno-unused-command-line-argument", "-I", os.path.join(ROOT, "include"), src, "-o", exe,
+           "-L", PKG, "-llyraquant", "-Wl,-rpath,$ORIGIN/../../lyradiff_amd"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"compat_check build failed:\n{r.stdout}\n{r.stderr}")
+    return exe
 
 
 if __name__ == "__main__":

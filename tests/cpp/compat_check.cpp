@@ -1,0 +1,131 @@
+// Reference-style C++ call sites (names of lyraDiff's quant-linear API) running on liblyraquant.so.
+// Exit code 0 when the INT8 path is bit-exact against a host triple loop and the FP8 path is within
+// tolerance; prints one line per check.  Built by lyradiff_amd/build.py, run by tests/test_gpu_compat.py.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "lyradiff_compat.h"
+
+#define CK(x)                                                                        \
+    do {                                                                             \
+        hipError_t e = (x);                                                          \
+        if (e != hipSuccess) {                                                       \
+            std::printf("HIP error %s at line %d\n", hipGetErrorString(e), __LINE__); \
+            return 2;                                                                \
+        }                                                                            \
+    } while (0)
+
+using namespace lyradiff;
+
+static float lcg(unsigned& s) { s = s * 1664525u + 1013904223u; return ((s >> 8) & 0xFFFF) / 65536.0f - 0.5f; }
+
+int main() {
+    const int m = 96, n = 64, k = 128;
+    unsigned seed = 7;
+    hipStream_t st;
+    CK(hipStreamCreate(&st));
+    // ---------------- INT8: dynamic per-token quant -> repack -> runGemmInt8 (fp16 out) ----------------
+    std::vector<__half> hx(m * k);
+    std::vector<float> fx(m * k), pre(k), wscale(n);
+    std::vector<int8_t> hw(n * k);
+    for (auto& v : fx) v = 4.0f * lcg(seed);
+    for (int i = 0; i < m * k; ++i) { hx[i] = __float2half(fx[i]); fx[i] = __half2float(hx[i]); }
+    for (auto& v : pre) v = 1.0f + lcg(seed);
+    for (auto& v : wscale) v = 0.005f + 0.004f * lcg(seed);
+    for (auto& v : hw) v = (int8_t)(254.0f * lcg(seed));
+    __half *dx, *dy;
+    int8_t *dq, *dw, *dwp;
+    float *dpre, *dscale, *dws;
+    CK(hipMalloc(&dx, m * k * 2)); CK(hipMalloc(&dy, m * n * 2)); CK(hipMalloc(&dq, m * k)); CK(hipMalloc(&dw, n * k));
+    CK(hipMalloc(&dwp, n * k)); CK(hipMalloc(&dpre, k * 4)); CK(hipMalloc(&dscale, m * 4)); CK(hipMalloc(&dws, n * 4));
+    CK(hipMemcpy(dx, hx.data(), m * k * 2, hipMemcpyHostToDevice));
+    CK(hipMemcpy(dw, hw.data(), n * k, hipMemcpyHostToDevice));
+    CK(hipMemcpy(dpre, pre.data(), k * 4, hipMemcpyHostToDevice));
+    CK(hipMemcpy(dws, wscale.data(), n * 4, hipMemcpyHostToDevice));
+    try {
+        invokeSqDynamicPerTokenQuant<__half>(dq, dscale, dx, dpre, 1, m, k, st);
+        repackWeight(dwp, dw, LQ_W_INT8, n, k, st);
+        cublasMMWrapper<__half> wrapper(st, /*per_token_int8=*/true);
+        wrapper.profileGemmInt8(16384, n, k);
+        wrapper.runGemmInt8(dq, dwp, dws, dscale, dy, m, n, k, nullptr, st);
+    } catch (const std::exception& e) {
+        std::printf("exception: %s\n", e.what());
+        return 3;
+    }
+    CK(hipStreamSynchronize(st));
+    std::vector<__half> hy(m * n);
+    std::vector<int8_t> hq(m * k);
+    std::vector<float> hs(m);
+    CK(hipMemcpy(hy.data(), dy, m * n * 2, hipMemcpyDeviceToHost));
+    CK(hipMemcpy(hq.data(), dq, m * k, hipMemcpyDeviceToHost));
+    CK(hipMemcpy(hs.data(), dscale, m * 4, hipMemcpyDeviceToHost));
+    int bad = 0;
+    for (int i = 0; i < m; ++i) {
+        float amax = 0.f;
+        for (int j = 0; j < k; ++j) amax = std::fmax(amax, std::fabs(fx[i * k + j] * pre[j]));
+        float s = amax / 127.0f;
+        if (s != hs[i]) ++bad;
+        for (int j = 0; j < k; ++j) {
+            float r = std::rint((fx[i * k + j] * pre[j]) / s);
+            r = std::fmin(std::fmax(r, -128.f), 127.f);
+            if ((int8_t)r != hq[i * k + j]) ++bad;
+        }
+        for (int j = 0; j < n; ++j) {
+            int acc = 0;
+            for (int p = 0; p < k; ++p) acc += (int)hq[i * k + p] * (int)hw[j * k + p];
+            float y = (float)acc * (wscale[j] * s);
+            if (__half2float(__float2half(y)) != __half2float(hy[i * n + j])) ++bad;
+        }
+    }
+    std::printf("int8 path (invokeSqDynamicPerTokenQuant + runGemmInt8): %d mismatches\n", bad);
+    // ---------------- FP8: weight scale + cast + GemmWithResidualAndBias (bf16 out) ----------------------
+    std::vector<hip_bfloat16> bx(m * k), bw(n * k);
+    std::vector<float> fbx(m * k), fbw(n * k);
+    for (int i = 0; i < m * k; ++i) { bx[i] = hip_bfloat16(2.0f * lcg(seed)); fbx[i] = (float)bx[i]; }
+    for (int i = 0; i < n * k; ++i) { bw[i] = hip_bfloat16(0.1f * lcg(seed)); fbw[i] = (float)bw[i]; }
+    hip_bfloat16 *dbx, *dbw, *dby;
+    fp8_e4m3_t *qx, *qw, *qwp;
+    float *sx, *sw;
+    CK(hipMalloc(&dbx, m * k * 2)); CK(hipMalloc(&dbw, n * k * 2)); CK(hipMalloc(&dby, m * n * 2));
+    CK(hipMalloc(&qx, m * k)); CK(hipMalloc(&qw, n * k)); CK(hipMalloc(&qwp, n * k));
+    CK(hipMalloc(&sx, 4)); CK(hipMalloc(&sw, 4));
+    CK(hipMemcpy(dbx, bx.data(), m * k * 2, hipMemcpyHostToDevice));
+    CK(hipMemcpy(dbw, bw.data(), n * k * 2, hipMemcpyHostToDevice));
+    CK(hipMemsetAsync(sx, 0, 4, st)); CK(hipMemsetAsync(sw, 0, 4, st));
+    try {
+        invokeGetFP8WeightScale(sw, dbw, (size_t)n * k, st);
+        invokeCudaD2DScaleCpyConvert(qw, dbw, sw, true, (size_t)n * k, st);
+        invokeGetFP8WeightScale(sx, dbx, (size_t)m * k, st);
+        invokeCudaD2DScaleCpyConvert(qx, dbx, sx, true, (size_t)m * k, st);
+        repackWeight(qwp, qw, LQ_W_FP8, n, k, st);
+        cublasMMWrapper<hip_bfloat16> wrapper(st);
+        wrapper.GemmWithResidualAndBias(CUBLAS_OP_T, CUBLAS_OP_N, n, m, k, qwp, k, sw, qx, k, sx, dby, n);
+    } catch (const std::exception& e) {
+        std::printf("exception: %s\n", e.what());
+        return 3;
+    }
+    CK(hipStreamSynchronize(st));
+    std::vector<hip_bfloat16> by(m * n);
+    CK(hipMemcpy(by.data(), dby, m * n * 2, hipMemcpyDeviceToHost));
+    int bad8 = 0;
+    for (int i = 0; i < m; ++i)
+        for (int j = 0; j < n; ++j) {
+            double ref = 0;
+            for (int p = 0; p < k; ++p) ref += (double)fbx[i * k + p] * (double)fbw[j * k + p];
+            double got = (double)(float)by[i * n + j];
+            if (std::fabs(got - ref) > 0.08 * std::fabs(ref) + 0.02) ++bad8;  // e4m3 operands: ~3 mantissa bits
+        }
+    std::printf("fp8 path (GetFP8WeightScale + ScaleCpyConvert + GemmWithResidualAndBias): %d outliers\n", bad8);
+    // error convention: exception with the reference's prefix
+    bool threw = false;
+    try {
+        cublasMMWrapper<__half> wrapper(st);
+        wrapper.runGemmInt8(dq, dwp, dws, dscale, dy, m, 33, k, nullptr, st);
+    } catch (const std::runtime_error& e) {
+        threw = std::string(e.what()).find("[lyradiff Error]") == 0;
+    }
+    std::printf("bad shape raises std::runtime_error with the reference's prefix: %s\n", threw ? "yes" : "no");
+    return (bad == 0 && bad8 == 0 && threw) ? 0 : 1;
+}

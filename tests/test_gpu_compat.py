@@ -1,0 +1,17 @@
+"""Reference-named C++ call sites (include/lyradiff_compat.h) on the GPU through the C ABI."""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_cpp_reference_style_call_sites(dev):
+    exe = os.path.join(ROOT, "tests", "cpp", "compat_check")
+    assert os.path.exists(exe), "build it with `python -m lyradiff_amd.build` (prebuilt binaries travel to the GPU box)"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    print(r.stdout, r.stderr)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "0 mismatches" in r.stdout and "0 outliers" in r.stdout and "prefix: yes" in r.stdout
