@@ -141,6 +141,192 @@ __global__ __launch_bounds__(256) void fp8_amax_scalar_kernel(float* __restrict_
 
 __global__ void fill_f32_kernel(float* p, float v) { p[0] = v; }
 
+// Fused dynamic per-tensor quantisation in ONE launch: every thread keeps up to KEEP 16-element
+// chunks of its slice in registers while the tensor-wide absmax is formed (workgroup partials ->
+// grid-wide barrier -> every workgroup reduces the partials), then casts from registers, so the
+// source is read from HBM once (3 bytes moved per element: the algorithmic minimum).  Chunks
+// beyond KEEP are re-read in the second phase (from L2 / Infinity Cache when they fit).
+//
+// The grid never exceeds what the device holds at once (CUs x resident workgroups), so every
+// workgroup is running when the barrier is reached.  The barrier re-arms itself (safe to replay from
+// a HIP graph); the wait is bounded,
+// so that even a starved grid terminates: on time-out the kernel raises g_amax_timeout and the
+// scale it writes is NaN, which poisons the output visibly instead of hanging the device.
+// Launches that overlap in time must use different slots: the host hands slots out round-robin.
+constexpr int kCoopThreads = 512;
+constexpr int kCoopMaxBlocks = 1024;
+constexpr int kCoopSlots = 16;
+__device__ float g_amax_partials[kCoopSlots][kCoopMaxBlocks];
+__device__ unsigned g_amax_group_count[kCoopSlots][8];
+__device__ unsigned g_amax_top_count[kCoopSlots];
+__device__ unsigned g_amax_flag[kCoopSlots];
+__device__ unsigned g_amax_timeout;
+
+// Two-level arrive counter (workgroup ids congruent modulo 8 share a counter, so at most G/8 atomics
+// hit one address; the last arriver of a group bumps the top counter, the last group flips the flag
+// everybody polls).  Counters are cleared by their last arriver, so the barrier re-arms itself and can
+// be replayed from a HIP graph.  Only relaxed device-scope atomics are used for the hand-over -- no
+// release/acquire fences, which on this multi-die part would write back / invalidate whole L2s -- and
+// the partial maxima travel through the same kind of atomics; a workgroup-scope release fence (a plain
+// wait for outstanding memory operations) orders the partial store before the arrival.
+// Returns false on time-out.
+__device__ __forceinline__ bool grid_barrier(int slot) {
+    __shared__ int ok;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned G = gridDim.x, grp = blockIdx.x & 7;
+        const unsigned in_group = (G - grp + 7) / 8, ngroups = G < 8 ? G : 8;
+        const unsigned f0 = __hip_atomic_load(&g_amax_flag[slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        unsigned x = __hip_atomic_fetch_add(&g_amax_group_count[slot][grp], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (x == in_group - 1) {
+            __hip_atomic_store(&g_amax_group_count[slot][grp], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            unsigned t = __hip_atomic_fetch_add(&g_amax_top_count[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (t == ngroups - 1) {
+                __hip_atomic_store(&g_amax_top_count[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                __hip_atomic_store(&g_amax_flag[slot], f0 + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        int good = 0;
+        for (int spin = 0; spin < (1 << 22); ++spin) {
+            if (__hip_atomic_load(&g_amax_flag[slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != f0) {
+                good = 1;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+        if (!good) __hip_atomic_store(&g_amax_timeout, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ok = good;
+    }
+    __syncthreads();
+    return ok != 0;
+}
+
+template <typename Tag, int KEEP>
+__global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_t* __restrict__ dst,
+                                                                          float* __restrict__ scale_out,
+                                                                          const void* __restrict__ src, size_t n,
+                                                                          int slot) {
+    constexpr int E = Chunk16<Tag>::elems;
+    constexpr int V = Elem<Tag>::bytes == 2 ? 2 : 2;  // uint4 vectors per chunk (32 bytes either way)
+    const size_t nchunks = n / E;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint4 keep[KEEP][V];
+    float amax = 0.0f;
+    auto chunk_amax = [&](const uint4* v) {
+        float f[16];
+        if constexpr (Elem<Tag>::bytes == 2) { unpack8<Tag>(v[0], f); unpack8<Tag>(v[1], f + 8); }
+        else { f[0] = __uint_as_float(v[0].x); f[1] = __uint_as_float(v[0].y); f[2] = __uint_as_float(v[0].z); f[3] = __uint_as_float(v[0].w);
+               f[4] = __uint_as_float(v[1].x); f[5] = __uint_as_float(v[1].y); f[6] = __uint_as_float(v[1].z); f[7] = __uint_as_float(v[1].w); }
+#pragma unroll
+        for (int i = 0; i < E; ++i) amax = fmaxf(amax, fabsf(f[i]));
+    };
+#pragma unroll
+    for (int it = 0; it < KEEP; ++it) {
+        size_t c = first + it * stride;
+        keep[it][0] = make_uint4(0, 0, 0, 0);
+        keep[it][1] = make_uint4(0, 0, 0, 0);
+        if (c < nchunks) {
+            const uint4* p = reinterpret_cast<const uint4*>(static_cast<const char*>(src) + c * 32);
+            keep[it][0] = p[0];
+            keep[it][1] = p[1];
+        }
+    }
+#pragma unroll
+    for (int it = 0; it < KEEP; ++it) chunk_amax(keep[it]);
+    for (size_t c = first + KEEP * stride; c < nchunks; c += stride) {
+        const uint4* p = reinterpret_cast<const uint4*>(static_cast<const char*>(src) + c * 32);
+        uint4 v[2] = {p[0], p[1]};
+        chunk_amax(v);
+    }
+    if (blockIdx.x == 0) {
+        size_t i = nchunks * E + threadIdx.x;
+        if (i < n) amax = fmaxf(amax, fabsf(load_one<Tag>(src, i)));
+    }
+    __shared__ float red[kCoopThreads / 64];
+    amax = wave_max(amax);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float m = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kCoopThreads / 64; ++i) m = fmaxf(m, red[i]);
+        __hip_atomic_store(&g_amax_partials[slot][blockIdx.x], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    const bool arrived = grid_barrier(slot);
+    float m = 0.0f;
+    for (int i = threadIdx.x; i < (int)gridDim.x; i += kCoopThreads)
+        m = fmaxf(m, __hip_atomic_load(&g_amax_partials[slot][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    m = wave_max(m);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    m = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kCoopThreads / 64; ++i) m = fmaxf(m, red[i]);
+    const float s = arrived ? m / 448.0f : __builtin_nanf("");
+    if (blockIdx.x == 0 && threadIdx.x == 0) scale_out[0] = s;
+    const float r = 1.0f / s;
+    auto chunk_cast = [&](const uint4* v, size_t c) {
+        float f[16];
+        if constexpr (Elem<Tag>::bytes == 2) { unpack8<Tag>(v[0], f); unpack8<Tag>(v[1], f + 8); }
+        else { f[0] = __uint_as_float(v[0].x); f[1] = __uint_as_float(v[0].y); f[2] = __uint_as_float(v[0].z); f[3] = __uint_as_float(v[0].w);
+               f[4] = __uint_as_float(v[1].x); f[5] = __uint_as_float(v[1].y); f[6] = __uint_as_float(v[1].z); f[7] = __uint_as_float(v[1].w); }
+        u32 w[4];
+#pragma unroll
+        for (int i = 0; i < E / 4; ++i) w[i] = cvt4_e4m3(f[4 * i] * r, f[4 * i + 1] * r, f[4 * i + 2] * r, f[4 * i + 3] * r);
+        if constexpr (E == 16) *reinterpret_cast<uint4*>(dst + c * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+        else *reinterpret_cast<uint2*>(dst + c * 8) = make_uint2(w[0], w[1]);
+    };
+#pragma unroll
+    for (int it = 0; it < KEEP; ++it) {
+        size_t c = first + it * stride;
+        if (c < nchunks) chunk_cast(keep[it], c);
+    }
+    for (size_t c = first + KEEP * stride; c < nchunks; c += stride) {
+        const uint4* p = reinterpret_cast<const uint4*>(static_cast<const char*>(src) + c * 32);
+        uint4 v[2] = {p[0], p[1]};
+        chunk_cast(v, c);
+    }
+    if (blockIdx.x == 0) {
+        size_t i = nchunks * E + threadIdx.x;
+        if (i < n) dst[i] = (uint8_t)cvt1_e4m3(load_one<Tag>(src, i) * r);
+    }
+}
+
+// Returns LQ_OK when the fused launch was issued, 1 when the caller should fall back to the
+// three-kernel sequence (unaligned buffers, or the occupancy query failed).
+template <typename Tag>
+static int launch_amax_cast_coop(uint8_t* dst, float* scale_out, const void* src, size_t n, hipStream_t st) {
+    static int blocks_per_cu = -1, num_cu = 0;
+    static unsigned next_slot = 0;
+    constexpr int KEEP = 8;
+    auto kern = fp8_amax_cast_coop_kernel<Tag, KEEP>;
+    if (reinterpret_cast<uintptr_t>(src) % 16 != 0 || reinterpret_cast<uintptr_t>(dst) % 16 != 0) return 1;
+    if (blocks_per_cu < 0) {
+        int dev = 0, occ = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess ||
+            hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, kCoopThreads, 0) != hipSuccess || occ < 1) {
+            blocks_per_cu = 0;
+        } else {
+            blocks_per_cu = occ > 2 ? 2 : occ;
+            num_cu = prop.multiProcessorCount;
+        }
+        (void)hipGetLastError();
+    }
+    if (blocks_per_cu == 0) return 1;
+    int grid = blocks_per_cu * num_cu;
+    if (grid > kCoopMaxBlocks) grid = kCoopMaxBlocks;
+    size_t need = (n / Chunk16<Tag>::elems + kCoopThreads - 1) / kCoopThreads;
+    if ((size_t)grid > need) grid = need ? (int)need : 1;
+    int slot = (int)(next_slot++ % kCoopSlots);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kCoopThreads), 0, st, dst, scale_out, src, n, slot);
+    return check_launch("fp8_amax_cast_fused");
+}
+
 static unsigned stream_grid(size_t n, int elems_per_thread) {
     size_t blocks = (n / elems_per_thread + 255) / 256;
     const size_t cap = 256 * 8;  // 8 workgroups of 4 wavefronts per CU keep HBM busy
@@ -151,7 +337,10 @@ static unsigned stream_grid(size_t n, int elems_per_thread) {
 
 template <typename Tag> static int launch_amax(float* scale, const void* x, size_t n, hipStream_t st) {
     if (reinterpret_cast<uintptr_t>(x) % 16 == 0) {
-        hipLaunchKernelGGL((fp8_amax_kernel<Tag>), dim3(stream_grid(n, Chunk16<Tag>::elems)), dim3(256), 0, st, scale, x, n);
+        // 512 workgroups at most: every workgroup ends with one same-address atomic, and those serialise
+        unsigned grid = stream_grid(n, Chunk16<Tag>::elems);
+        if (grid > 512) grid = 512;
+        hipLaunchKernelGGL((fp8_amax_kernel<Tag>), dim3(grid), dim3(256), 0, st, scale, x, n);
     } else {
         hipLaunchKernelGGL((fp8_amax_scalar_kernel<Tag>), dim3(stream_grid(n, 4)), dim3(256), 0, st, scale, x, n);
     }
@@ -197,6 +386,16 @@ extern "C" int lq_fp8_scale_cast(uint8_t* dst, const void* src, lq_dtype_t dtype
 extern "C" int lq_fp8_amax_cast(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t n,
                                 lq_stream_t stream) {
     LQ_REQUIRE(scale_out && ((dst && src) || n == 0), LQ_ERR_ARG, "lq_fp8_amax_cast: null pointer");
+    if (n >= 4096) {
+        int rc = 1;
+        switch (dtype) {
+            case LQ_F16: rc = launch_amax_cast_coop<F16Tag>(dst, scale_out, src, n, as_stream(stream)); break;
+            case LQ_BF16: rc = launch_amax_cast_coop<BF16Tag>(dst, scale_out, src, n, as_stream(stream)); break;
+            case LQ_F32: rc = launch_amax_cast_coop<F32Tag>(dst, scale_out, src, n, as_stream(stream)); break;
+            default: set_error("lq_fp8_amax_cast: unsupported dtype %d", (int)dtype); return LQ_ERR_UNSUPPORTED;
+        }
+        if (rc == LQ_OK) return LQ_OK;
+    }
     hipLaunchKernelGGL(fill_f32_kernel, dim3(1), dim3(1), 0, as_stream(stream), scale_out, 0.0f);
     int rc = check_launch("fp8_amax_cast(fill)");
     if (rc != LQ_OK || n == 0) return rc;

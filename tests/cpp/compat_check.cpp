@@ -115,7 +115,7 @@ int main() {
             double ref = 0;
             for (int p = 0; p < k; ++p) ref += (double)fbx[i * k + p] * (double)fbw[j * k + p];
             double got = (double)(float)by[i * n + j];
-            if (std::fabs(got - ref) > 0.08 * std::fabs(ref) + 0.02) ++bad8;  // e4m3 operands: ~3 mantissa bits
+            if (std::fabs(got - ref) > 0.1 * std::fabs(ref) + 0.05) ++bad8;  // e4m3 operands (3 mantissa bits): noise ~0.01 rms here
         }
     std::printf("fp8 path (GetFP8WeightScale + ScaleCpyConvert + GemmWithResidualAndBias): %d outliers\n", bad8);
     // error convention: exception with the reference's prefix
