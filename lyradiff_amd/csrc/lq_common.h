@@ -81,8 +81,12 @@ template <> struct Elem<F32Tag> {
     static __device__ __forceinline__ float load(u32 bits) { return __uint_as_float(bits); }
     static __device__ __forceinline__ u32 store(float f) { return __float_as_uint(f); }
 };
-// round an fp32 value to T and bring it back (the "T arithmetic" of the reference's half2 code)
+// round an fp32 value to T and bring it back (the "T arithmetic" of the reference's half2 code).
+// The empty asm pins the fp32 value: without it the compiler may merge the producing fma/add with
+// the conversion into a mixed-precision instruction that rounds the exact result once to 16 bits,
+// which differs (rarely) from rounding to fp32 first as the specification of these kernels does.
 template <typename Tag> __device__ __forceinline__ float round_through(float f) {
+    asm volatile("" : "+v"(f));
     return Elem<Tag>::load(Elem<Tag>::store(f));
 }
 
@@ -97,13 +101,32 @@ template <typename Tag> __device__ __forceinline__ void unpack8(const uint4& v, 
 }
 
 // ---- wavefront (64 lanes) reductions ------------------------------------------------------------
+// Cross-lane steps inside a row of 16 lanes use DPP operand swizzles (no LDS traffic):
+// quad_perm [1,0,3,2] and [2,3,0,1] exchange with the lanes at distance 1 and 2, row_half_mirror
+// and row_mirror bring in the other quad / the other half of the row.
+template <int CTRL> __device__ __forceinline__ int dpp_i32(int v) {
+    return __builtin_amdgcn_update_dpp(v, v, CTRL, 0xF, 0xF, false);
+}
+// max over aligned groups of 8 consecutive lanes of a NON-NEGATIVE float (or +NaN pattern), result in
+// every lane of the group.  Non-negative floats order like their bit patterns, so the steps run as
+// integer max (no NaN canonicalisation needed around the DPP moves).
+__device__ __forceinline__ float group8_max(float v) {
+    int x = __builtin_bit_cast(int, v);
+    x = max(x, dpp_i32<0xB1>(x));
+    x = max(x, dpp_i32<0x4E>(x));
+    x = max(x, dpp_i32<0x141>(x));
+    return __builtin_bit_cast(float, x);
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    v = group8_max(v);
+    v = __builtin_bit_cast(float, max(__builtin_bit_cast(int, v), dpp_i32<0x140>(__builtin_bit_cast(int, v))));  // row_mirror
+    v = fmaxf(v, __shfl_xor(v, 16, 64));  // across rows
+    v = fmaxf(v, __shfl_xor(v, 32, 64));
     return v;
 }
 // max over aligned groups of G consecutive lanes (G power of two)
 template <int G> __device__ __forceinline__ float group_max(float v) {
+    if constexpr (G == 8) return group8_max(v);
 #pragma unroll
     for (int off = G / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
     return v;
@@ -122,6 +145,64 @@ __device__ __forceinline__ int rne_sat_s4(float x) {
     r = fminf(fmaxf(r, -8.0f), 7.0f);
     r = (x != x) ? 0.0f : r;
     return (int)r;
+}
+
+// q[i] = clamp(rint(t[i] / s), LO, HI) (NaN -> 0) for eight values, bit-identical to the IEEE
+// division but normally computed from r ~ 1/s (within 1 ulp):  |t*r - t/s| <= 2.5*2^-24*|t/s| and
+// |fl(t/s) - t/s| <= 2^-24*|t/s|, so whenever |t*r| < 512 both lie within 1.1e-4 of the true quotient;
+// if t*r is at least 2e-4 away from every tie (|t*r - rint(t*r)| <= 0.4998) the true quotient, its
+// fp32 rounding and t*r all round to the same integer.  Beyond 512 in magnitude everything saturates.
+// If any of the eight values fails the test (or is NaN/inf, or the caller flags the scale as
+// unsafe for a reciprocal), the whole octet is redone with true divisions: one rarely taken branch.
+template <int LO, int HI>
+__device__ __forceinline__ void quant8(const float* t, float s, float r, bool slow, int* q) {
+    float rq[8], dev = 0.0f, nonfinite = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float qa = t[i] * r;
+        rq[i] = __builtin_rintf(qa);
+        dev = fmaxf(dev, fabsf(qa - rq[i]));                   // largest distance from an integer
+        nonfinite = __builtin_fmaf(t[i], 0.0f, nonfinite);    // stays 0 unless some t is inf or NaN
+    }
+    const bool risky = slow | !(dev <= 0.4998f) | !(nonfinite == 0.0f);
+    if (__builtin_expect(risky, 0)) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float e = t[i] / s;
+            rq[i] = (e != e) ? 0.0f : __builtin_rintf(e);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) q[i] = (int)__builtin_amdgcn_fmed3f(rq[i], (float)LO, (float)HI);
+}
+// true unless |s| lies in [2^-100, 2^100]: zero, subnormal, huge, infinite and NaN scales all take the
+// exact-division path (one integer subtract and compare on the exponent field)
+__device__ __forceinline__ bool scale_out_of_range(float s) {
+    return ((__float_as_uint(s) & 0x7FFFFFFFu) - 0x0D800000u) > (0x71800000u - 0x0D800000u);
+}
+// fl(a / D) for a compile-time divisor D from its correctly rounded reciprocal (three operations
+// instead of the ~12 of an IEEE division): q0 = fl(a*Y), rem = a - q0*D exactly (one fma),
+// result = fl(q0 + rem*Y) is the correctly rounded quotient when Y = fl(1/D) and nothing leaves
+// the normal range (Markstein).  Callers check the result with scale_out_of_range() and redo the
+// division exactly when it fails.
+__device__ __forceinline__ float div_by_const_fast(float a, float D, float Y) {
+    float q0 = a * Y;
+    float rem = __builtin_fmaf(-q0, D, a);
+    return __builtin_fmaf(rem, Y, q0);
+}
+// reciprocal good to 1 ulp (hardware v_rcp_f32): enough for quant8's argument, whose margin of 2e-4
+// covers 2.5*2^-24*512 + 2^-24*512 = 1.1e-4
+__device__ __forceinline__ float fast_recip(float s) { return __builtin_amdgcn_rcpf(s); }
+
+// true when 1/s cannot be trusted as a reciprocal (zero, subnormal, infinite or NaN scale)
+__device__ __forceinline__ bool recip_unsafe(float s, float r) {
+    return !(fabsf(s) >= 1e-30f && fabsf(r) < 1e30f && fabsf(r) >= 1e-30f);
+}
+// four ints in [-128,127] -> packed bytes
+__device__ __forceinline__ u32 pack4_s8(int a, int b, int c, int d) {
+    u32 lo = __builtin_amdgcn_perm((u32)b, (u32)a, 0x0c0c0400u);  // bytes: a.b0, b.b0, 0, 0
+    u32 hi = __builtin_amdgcn_perm((u32)d, (u32)c, 0x04000c0cu);  // bytes: 0, 0, c.b0, d.b0
+    return lo | hi;
 }
 
 // tanh from basic IEEE operations only (no fused multiply-add), so that a CPU restatement can

@@ -13,25 +13,6 @@
 
 namespace lq {
 
-// q = sat_s8(rne(t / s)) with the IEEE quotient, computed from r = 1/s whenever that provably
-// gives the same integer: |t*r - t/s| <= 1.5*2^-23*|t/s| and |fl(t/s) - t/s| <= 2^-24*|t/s|, so for
-// |t*r| < 512 both lie within 1e-4 of the true quotient; unless t*r is that close to a half
-// integer the two round to the same integer.  Beyond 512 both saturate.  Otherwise divide.
-__device__ __forceinline__ int quant_div_s8(float t, float s, float r, bool slow_row) {
-    float qa = t * r;
-    float fr = __builtin_amdgcn_fractf(qa);
-    bool risky = slow_row || (fabsf(fr - 0.5f) < 2e-4f && fabsf(qa) < 512.0f);
-    if (__builtin_expect(risky, 0)) qa = t / s;
-    return rne_sat_s8(qa);
-}
-__device__ __forceinline__ bool recip_unsafe(float s, float r) {
-    return !(fabsf(s) >= 1e-30f && fabsf(r) < 1e30f && fabsf(r) >= 1e-30f);
-}
-
-__device__ __forceinline__ u32 pack4_s8(int a, int b, int c, int d) {
-    return (u32)(a & 0xFF) | ((u32)(b & 0xFF) << 8) | ((u32)(c & 0xFF) << 16) | ((u32)d << 24);
-}
-
 // Load 8 consecutive elements (element offset `col` inside the row) as floats.
 template <typename Tag> __device__ __forceinline__ void load8(const void* row_base, int col, float* o) {
     if constexpr (Elem<Tag>::bytes == 2) {
@@ -46,53 +27,64 @@ template <typename Tag> __device__ __forceinline__ void load8(const void* row_ba
 }
 
 // MODE 0: static per-tensor scale, 1: given per-token scale, 2: dynamic per-token scale.
-template <typename Tag, int NP, int MODE, bool PRE_REGS>
+// The smoothing vector (fp32, twice the bytes of an fp16 row) is staged once per workgroup in LDS
+// and shared by the rows its four wavefronts quantise.
+template <typename Tag, int NP, int MODE, bool HAS_PRE>
 __global__ __launch_bounds__(256) void sq_quant_rows_kernel(int8_t* __restrict__ dst,
                                                             float* __restrict__ scale_out,
                                                             const void* __restrict__ src,
                                                             const float* __restrict__ pre,
                                                             const float* __restrict__ in_scale,
-                                                            size_t rows, int dim) {
-    const int lane = threadIdx.x & 63;
-    const size_t wave = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const size_t nwaves = (size_t)gridDim.x * 4;
+                                                            size_t rows, int dim, int rows_per_wave) {
+    extern __shared__ __attribute__((aligned(16))) float s_pre[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const size_t row_bytes = (size_t)dim * Elem<Tag>::bytes;
-
-    float pr[PRE_REGS ? NP : 1][8];
-    if constexpr (PRE_REGS) {
-#pragma unroll
-        for (int p = 0; p < NP; ++p) {
-            int col = (p * 64 + lane) * 8;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) pr[p][i] = 1.0f;
-            if (pre != nullptr && col < dim) load8<F32Tag>(pre, col, pr[p]);
-        }
+    if constexpr (HAS_PRE) {
+        for (int c = threadIdx.x * 4; c < dim; c += 1024)
+            *reinterpret_cast<float4*>(s_pre + c) = *reinterpret_cast<const float4*>(pre + c);
+        __syncthreads();
     }
-
-    for (size_t row = wave; row < rows; row += nwaves) {
+    // Raw row data is double buffered in registers: the loads of the wavefront's next row are in
+    // flight while the current row is quantised.
+    constexpr int VPP = Elem<Tag>::bytes == 2 ? 1 : 2;  // 16-byte vectors per 8 elements
+    auto load_raw = [&](size_t row, uint4 (*raw)[VPP]) {
         const char* rb = static_cast<const char*>(src) + row * row_bytes;
-        float t[NP][8];
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             int col = (p * 64 + lane) * 8;
-            if (col < dim) {
-                load8<Tag>(rb, col, t[p]);
-            } else {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) t[p][i] = 0.0f;
+            for (int u = 0; u < VPP; ++u) {
+                raw[p][u] = make_uint4(0, 0, 0, 0);
+                if (col < dim) raw[p][u] = *reinterpret_cast<const uint4*>(rb + (size_t)col * Elem<Tag>::bytes + u * 16);
             }
         }
+    };
+    auto unpack_raw = [&](const uint4* r, float* o) {
+        if constexpr (Elem<Tag>::bytes == 2) unpack8<Tag>(r[0], o);
+        else {
+            o[0] = __uint_as_float(r[0].x); o[1] = __uint_as_float(r[0].y); o[2] = __uint_as_float(r[0].z); o[3] = __uint_as_float(r[0].w);
+            o[4] = __uint_as_float(r[VPP - 1].x); o[5] = __uint_as_float(r[VPP - 1].y); o[6] = __uint_as_float(r[VPP - 1].z); o[7] = __uint_as_float(r[VPP - 1].w);
+        }
+    };
+    const size_t row0 = (size_t)blockIdx.x * 4 * rows_per_wave + wave;
+    uint4 cur[NP][VPP], nxt[NP][VPP];
+    if (row0 < rows) load_raw(row0, cur);
+    for (int j = 0; j < rows_per_wave; ++j) {
+        const size_t row = row0 + 4 * (size_t)j;
+        if (row >= rows) break;
+        const bool has_next = j + 1 < rows_per_wave && row + 4 < rows;
+        if (has_next) load_raw(row + 4, nxt);
+        float t[NP][8];
         float amax = 0.0f;
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             int col = (p * 64 + lane) * 8;
-            if constexpr (PRE_REGS) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) t[p][i] = t[p][i] * pr[p][i];
-            } else {
-                if (pre != nullptr && col < dim) {
-                    float pv[8];
-                    load8<F32Tag>(pre, col, pv);
+            unpack_raw(cur[p], t[p]);
+            if constexpr (HAS_PRE) {
+                if (col < dim) {
+                    float4 a = *reinterpret_cast<const float4*>(s_pre + col);
+                    float4 b = *reinterpret_cast<const float4*>(s_pre + col + 4);
+                    const float pv[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
 #pragma unroll
                     for (int i = 0; i < 8; ++i) t[p][i] = t[p][i] * pv[i];
                 }
@@ -105,28 +97,35 @@ __global__ __launch_bounds__(256) void sq_quant_rows_kernel(int8_t* __restrict__
         float s;
         if constexpr (MODE == 2) {
             amax = wave_max(amax);
-            s = (amax <= 5.9604644775390625e-08f) ? 1.0f : amax / 127.0f;
+            s = div_by_const_fast(amax, 127.0f, 0x1.020408p-7f);
+            if (scale_out_of_range(s)) s = amax / 127.0f;
+            if (amax <= 5.9604644775390625e-08f) s = 1.0f;
             if (lane == 0) scale_out[row] = s;
         } else if constexpr (MODE == 1) {
             s = in_scale[row];
         } else {
             s = in_scale[0];
         }
-        const float r = 1.0f / s;
-        const bool slow = recip_unsafe(s, r);
+        const float r = fast_recip(s);
+        const bool slow = scale_out_of_range(s);
         int8_t* ob = dst + row * (size_t)dim;
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             int col = (p * 64 + lane) * 8;
             if (col < dim) {
                 int q[8];
-#pragma unroll
-                for (int i = 0; i < 8; ++i) q[i] = quant_div_s8(t[p][i], s, r, slow);
+                quant8<-128, 127>(t[p], s, r, slow, q);
                 uint2 o;
                 o.x = pack4_s8(q[0], q[1], q[2], q[3]);
                 o.y = pack4_s8(q[4], q[5], q[6], q[7]);
                 *reinterpret_cast<uint2*>(ob + col) = o;
             }
+        }
+        if (has_next) {
+#pragma unroll
+            for (int p = 0; p < NP; ++p)
+#pragma unroll
+                for (int u = 0; u < VPP; ++u) cur[p][u] = nxt[p][u];
         }
     }
 }
@@ -181,25 +180,28 @@ static int launch_sq_quant(int8_t* dst, float* scale_out, const void* src, const
         return check_launch("sq_quant_generic");
     }
     const int np = (int)((dim + 511) / 512);
-    // each wavefront walks several rows so that the smoothing vector is fetched once per wavefront
-    size_t blocks = (rows + 3) / 4;
-    const size_t max_blocks = 256 * 8;
-    if (blocks > max_blocks) blocks = max_blocks;
+    // four rows per workgroup pass; more rows per wavefront only when there are plenty of rows
+    int rpw = (int)(rows / (4 * 768));
+    rpw = rpw < 1 ? 1 : (rpw > 8 ? 8 : rpw);
+    const size_t blocks = (rows + 4 * (size_t)rpw - 1) / (4 * (size_t)rpw);
     dim3 grid((unsigned)blocks), block(256);
     int d = (int)dim;
-#define LQ_SQ_CASE(NPV, PREREG)                                                                                  \
-    hipLaunchKernelGGL((sq_quant_rows_kernel<Tag, NPV, MODE, PREREG>), grid, block, 0, st, dst, scale_out, src, pre, \
-                       in_scale, rows, d)
-    if (np <= 1) LQ_SQ_CASE(1, true);
-    else if (np <= 2) LQ_SQ_CASE(2, true);
-    else if (np <= 3) LQ_SQ_CASE(3, true);
-    else if (np <= 4) LQ_SQ_CASE(4, true);
-    else if (np <= 6) LQ_SQ_CASE(6, true);
-    else if (np <= 8) LQ_SQ_CASE(8, true);
-    else if (np <= 12) LQ_SQ_CASE(12, false);
-    else if (np <= 16) LQ_SQ_CASE(16, false);
-    else if (np <= 24) LQ_SQ_CASE(24, false);
-    else LQ_SQ_CASE(32, false);
+    const size_t lds = pre ? dim * sizeof(float) : 0;
+#define LQ_SQ_CASE(NPV)                                                                                             \
+    do {                                                                                                            \
+        if (pre) hipLaunchKernelGGL((sq_quant_rows_kernel<Tag, NPV, MODE, true>), grid, block, lds, st, dst, scale_out, src, pre, in_scale, rows, d, rpw); \
+        else hipLaunchKernelGGL((sq_quant_rows_kernel<Tag, NPV, MODE, false>), grid, block, 0, st, dst, scale_out, src, pre, in_scale, rows, d, rpw);      \
+    } while (0)
+    if (np <= 1) LQ_SQ_CASE(1);
+    else if (np <= 2) LQ_SQ_CASE(2);
+    else if (np <= 3) LQ_SQ_CASE(3);
+    else if (np <= 4) LQ_SQ_CASE(4);
+    else if (np <= 6) LQ_SQ_CASE(6);
+    else if (np <= 8) LQ_SQ_CASE(8);
+    else if (np <= 12) LQ_SQ_CASE(12);
+    else if (np <= 16) LQ_SQ_CASE(16);
+    else if (np <= 24) LQ_SQ_CASE(24);
+    else LQ_SQ_CASE(32);
 #undef LQ_SQ_CASE
     return check_launch("sq_quant_rows");
 }
@@ -324,8 +326,7 @@ __global__ __launch_bounds__(256) void geglu_int8_kernel(int8_t* __restrict__ ds
             int col = (p * 64 + lane) * 8;
             if (col < dim) {
                 int q[8];
-#pragma unroll
-                for (int i = 0; i < 8; ++i) q[i] = quant_div_s8(t[p][i], s, r, slow);
+                quant8<-128, 127>(t[p], s, r, slow, q);
                 uint2 o;
                 o.x = pack4_s8(q[0], q[1], q[2], q[3]);
                 o.y = pack4_s8(q[4], q[5], q[6], q[7]);

@@ -9,15 +9,6 @@
 
 namespace lq {
 
-// same argument as quant_div_s8 (see lq_quant_int8.hip), bounds [-8, 7]
-__device__ __forceinline__ int quant_div_s4(float t, float s, float r, bool slow) {
-    float qa = t * r;
-    float fr = __builtin_amdgcn_fractf(qa);
-    bool risky = slow || (fabsf(fr - 0.5f) < 2e-4f && fabsf(qa) < 512.0f);
-    if (__builtin_expect(risky, 0)) qa = t / s;
-    return rne_sat_s4(qa);
-}
-
 template <typename Tag> __device__ __forceinline__ void load8w(const void* row_base, int col, float* o) {
     if constexpr (Elem<Tag>::bytes == 2) {
         uint4 v = *reinterpret_cast<const uint4*>(static_cast<const char*>(row_base) + (size_t)col * 2);
@@ -30,69 +21,142 @@ template <typename Tag> __device__ __forceinline__ void load8w(const void* row_b
     }
 }
 
-template <typename Tag, int NP, bool F16_SCALE, bool SMOOTH_REGS>
+// SMOOTH 0: no smoothing vector; 1: divisors d and their correctly rounded reciprocals y = fl(1/d)
+// are computed once per workgroup into LDS and shared by the rows of its four wavefronts;
+// 2: plain IEEE division straight from global memory (rows too long for the LDS staging).
+template <typename Tag, int NP, bool F16_SCALE, int SMOOTH>
 __global__ __launch_bounds__(256) void w4a4_quant_kernel(u32* __restrict__ q_words, void* __restrict__ scales,
                                                          const void* __restrict__ x,
-                                                         const float* __restrict__ smooth, int m, int k) {
-    const int lane = threadIdx.x & 63;
-    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int nwaves = gridDim.x * 4;
+                                                         const float* __restrict__ smooth, int m, int k,
+                                                         int rows_per_wave) {
+    extern __shared__ __attribute__((aligned(16))) float s_dy[];  // [k] divisors, then [k] reciprocals
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int ng = k >> 6;
-    float sm[SMOOTH_REGS ? NP : 1][8];
-    if constexpr (SMOOTH_REGS) {
-#pragma unroll
-        for (int p = 0; p < NP; ++p) {
-            int col = (p * 64 + lane) * 8;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) sm[p][i] = 1.0f;
-            if (smooth != nullptr && col < k) load8w<F32Tag>(smooth, col, sm[p]);
+    if constexpr (SMOOTH == 1) {
+        for (int c = threadIdx.x * 4; c < k; c += 1024) {
+            float4 d = *reinterpret_cast<const float4*>(smooth + c);
+            *reinterpret_cast<float4*>(s_dy + c) = d;
+            *reinterpret_cast<float4*>(s_dy + k + c) = make_float4(1.0f / d.x, 1.0f / d.y, 1.0f / d.z, 1.0f / d.w);
         }
+        __syncthreads();
     }
-    for (int row = wave; row < m; row += nwaves) {
+    // Raw row data is double buffered in registers: the loads of the wavefront's next row are in
+    // flight while the current row is quantised.
+    constexpr int VPP = Elem<Tag>::bytes == 2 ? 1 : 2;  // 16-byte vectors per 8 elements
+    auto load_raw = [&](int row, uint4 (*raw)[VPP]) {
         const char* rb = static_cast<const char*>(x) + (size_t)row * k * Elem<Tag>::bytes;
-        float v[NP][8];
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             int col = (p * 64 + lane) * 8;
-            if (col < k) load8w<Tag>(rb, col, v[p]);
-            else {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) v[p][i] = 0.0f;
+            for (int u = 0; u < VPP; ++u) {
+                raw[p][u] = make_uint4(0, 0, 0, 0);
+                if (col < k) raw[p][u] = *reinterpret_cast<const uint4*>(rb + (size_t)col * Elem<Tag>::bytes + u * 16);
             }
         }
+    };
+    auto unpack_raw = [&](const uint4* r, float* o) {
+        if constexpr (Elem<Tag>::bytes == 2) unpack8<Tag>(r[0], o);
+        else {
+            o[0] = __uint_as_float(r[0].x); o[1] = __uint_as_float(r[0].y); o[2] = __uint_as_float(r[0].z); o[3] = __uint_as_float(r[0].w);
+            o[4] = __uint_as_float(r[VPP - 1].x); o[5] = __uint_as_float(r[VPP - 1].y); o[6] = __uint_as_float(r[VPP - 1].z); o[7] = __uint_as_float(r[VPP - 1].w);
+        }
+    };
+    const int row0 = blockIdx.x * 4 * rows_per_wave + wave;
+    uint4 cur[NP][VPP], nxt[NP][VPP];
+    if (row0 < m) load_raw(row0, cur);
+    for (int j = 0; j < rows_per_wave; ++j) {
+        const int row = row0 + 4 * j;
+        if (row >= m) break;
+        const bool has_next = j + 1 < rows_per_wave && row + 4 < m;
+        if (has_next) load_raw(row + 4, nxt);
+        const char* rb = static_cast<const char*>(x) + (size_t)row * k * Elem<Tag>::bytes;
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             int col = (p * 64 + lane) * 8;
-            if (smooth != nullptr) {
-                if constexpr (SMOOTH_REGS) {
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) v[p][i] = v[p][i] / sm[p][i];
-                } else if (col < k) {
-                    float sv[8];
-                    load8w<F32Tag>(smooth, col, sv);
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) v[p][i] = v[p][i] / sv[i];
-                }
-            }
+            float v[8];
+            unpack_raw(cur[p], v);
             float amax = 0.0f;
+            if constexpr (SMOOTH == 1) {
+                // v = fl(x/d) from the stored reciprocal: q0 = fl(x*y), rem = x - q0*d (exact in one
+                // fma), v = fl(q0 + rem*y) is the correctly rounded quotient when y = fl(1/d) and no
+                // intermediate leaves the normal range (Markstein).  The range condition is checked
+                // on the group's absmax, which is the only magnitude the outputs depend on: elements
+                // far below it quantise to 0 whatever their last bit.  The max runs on the bit
+                // patterns of |v| so that an inf or NaN anywhere in the group also takes the exact path.
+                float dv[8], yv[8];
+                {
+                    const int cc = col < k ? col : 0;
+                    float4 a = *reinterpret_cast<const float4*>(s_dy + cc), b = *reinterpret_cast<const float4*>(s_dy + cc + 4);
+                    float4 c = *reinterpret_cast<const float4*>(s_dy + k + cc), d = *reinterpret_cast<const float4*>(s_dy + k + cc + 4);
+                    dv[0] = a.x; dv[1] = a.y; dv[2] = a.z; dv[3] = a.w; dv[4] = b.x; dv[5] = b.y; dv[6] = b.z; dv[7] = b.w;
+                    yv[0] = c.x; yv[1] = c.y; yv[2] = c.z; yv[3] = c.w; yv[4] = d.x; yv[5] = d.y; yv[6] = d.z; yv[7] = d.w;
+                }
+                float xr[8];
+                u32 mbits = 0;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[p][i]));
-            amax = group_max<8>(amax);
-            float s = amax / 7.0f;
+                for (int i = 0; i < 8; ++i) {
+                    xr[i] = v[i];
+                    float q0 = xr[i] * yv[i];
+                    float rem = __builtin_fmaf(-q0, dv[i], xr[i]);
+                    v[i] = __builtin_fmaf(rem, yv[i], q0);
+                    u32 b = __float_as_uint(v[i]) & 0x7FFFFFFFu;
+                    mbits = b > mbits ? b : mbits;
+                }
+                float mf = group8_max(__uint_as_float(mbits));  // non-negative patterns order like floats
+                mbits = __float_as_uint(mf);
+                const bool odd = mbits != 0 && !(mbits >= 0x219392EFu /*1e-18f*/ && mbits <= 0x5D5E0B6Bu /*1e18f*/);
+                amax = mf;
+                if (__builtin_expect(odd, 0)) {  // uniform over the 8 lanes of the group
+                    amax = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        v[i] = xr[i] / dv[i];
+                        amax = fmaxf(amax, fabsf(v[i]));
+                    }
+                    amax = group8_max(amax);
+                }
+            } else {
+                if constexpr (SMOOTH == 2) {
+                    if (col < k) {
+                        float sv[8];
+                        load8w<F32Tag>(smooth, col, sv);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) v[i] = v[i] / sv[i];
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+                amax = group8_max(amax);
+            }
+            float s = div_by_const_fast(amax, 7.0f, 0x1.24924ap-3f);
             if constexpr (F16_SCALE) s = round_through<F16Tag>(s);
-            const float r = 1.0f / s;
-            const bool slow = !(fabsf(s) >= 1e-30f && fabsf(r) < 1e30f && fabsf(r) >= 1e-30f);
-            u32 word = 0;
+            const bool slow = scale_out_of_range(s);  // also covers an absmax outside the fast division's range
+            if (__builtin_expect(slow, 0)) {
+                s = amax / 7.0f;
+                if constexpr (F16_SCALE) s = round_through<F16Tag>(s);
+            }
+            const float r = fast_recip(s);
+            int q[8];
+            quant8<-8, 7>(v, s, r, slow, q);
+            u32 word = (u32)q[0] & 0xFu;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) word |= ((u32)quant_div_s4(v[p][i], s, r, slow) & 0xFu) << (4 * i);
+            for (int i = 1; i < 8; ++i) word = (word & ~(0xFu << (4 * i))) | (((u32)q[i] << (4 * i)) & (0xFu << (4 * i)));
             if (col < k) {
                 q_words[(size_t)row * (k >> 3) + (col >> 3)] = word;
                 if ((lane & 7) == 0) {
                     size_t si = (size_t)row * ng + (col >> 6);
-                    if constexpr (F16_SCALE) static_cast<unsigned short*>(scales)[si] = (unsigned short)f32_to_f16_bits(s);
+                    if constexpr (F16_SCALE) static_cast<unsigned short*>(scales)[si] = (unsigned short)f32_to_f16_bits(s);  // s is already an fp16 value
                     else static_cast<float*>(scales)[si] = s;
                 }
             }
+        }
+        (void)rb;
+        if (has_next) {
+#pragma unroll
+            for (int p = 0; p < NP; ++p)
+#pragma unroll
+                for (int u = 0; u < VPP; ++u) cur[p][u] = nxt[p][u];
         }
     }
 }
@@ -127,25 +191,39 @@ extern "C" int lq_w4a4_quantize(uint32_t* q_words, void* scales, lq_dtype_t scal
                LQ_ERR_ARG, "lq_w4a4_quantize: x and smooth must be 16-byte aligned");
     if (m == 0) return LQ_OK;
     const int np = (k + 511) / 512;
-    int blocks = (m + 3) / 4;
-    if (blocks > 256 * 8) blocks = 256 * 8;
+    // rows per wavefront: enough wavefronts to fill the chip (about 3 per SIMD), then more rows each so
+    // that the loads of one row overlap the arithmetic of the previous one
+    int rpw = m / (4 * 768);
+    rpw = rpw < 1 ? 1 : (rpw > 8 ? 8 : rpw);
+    const int blocks = (m + 4 * rpw - 1) / (4 * rpw);
     dim3 grid(blocks), block(256);
     hipStream_t st = as_stream(stream);
     const bool f16s = scale_dtype == LQ_F16;
-#define LQ_W4_LAUNCH(TAG, NPV, SR)                                                                                        \
-    do {                                                                                                                  \
-        if (f16s) hipLaunchKernelGGL((w4a4_quant_kernel<TAG, NPV, true, SR>), grid, block, 0, st, q_words, scales, x, smooth, m, k); \
-        else hipLaunchKernelGGL((w4a4_quant_kernel<TAG, NPV, false, SR>), grid, block, 0, st, q_words, scales, x, smooth, m, k);      \
+    const int smode = smooth == nullptr ? 0 : (k <= 8192 ? 1 : 2);
+    const size_t lds = smode == 1 ? 2 * (size_t)k * sizeof(float) : 0;
+#define LQ_W4_LAUNCH2(TAG, NPV, F16S, SM) \
+    hipLaunchKernelGGL((w4a4_quant_kernel<TAG, NPV, F16S, SM>), grid, block, lds, st, q_words, scales, x, smooth, m, k, rpw)
+#define LQ_W4_LAUNCH(TAG, NPV)                                                     \
+    do {                                                                           \
+        if (f16s) {                                                                \
+            if (smode == 0) LQ_W4_LAUNCH2(TAG, NPV, true, 0);                      \
+            else if (smode == 1) LQ_W4_LAUNCH2(TAG, NPV, true, 1);                 \
+            else LQ_W4_LAUNCH2(TAG, NPV, true, 2);                                 \
+        } else {                                                                   \
+            if (smode == 0) LQ_W4_LAUNCH2(TAG, NPV, false, 0);                     \
+            else if (smode == 1) LQ_W4_LAUNCH2(TAG, NPV, false, 1);                \
+            else LQ_W4_LAUNCH2(TAG, NPV, false, 2);                                \
+        }                                                                          \
     } while (0)
-#define LQ_W4_NP(TAG)                          \
-    do {                                       \
-        if (np <= 1) LQ_W4_LAUNCH(TAG, 1, true);       \
-        else if (np <= 2) LQ_W4_LAUNCH(TAG, 2, true);  \
-        else if (np <= 4) LQ_W4_LAUNCH(TAG, 4, true);  \
-        else if (np <= 6) LQ_W4_LAUNCH(TAG, 6, true);  \
-        else if (np <= 8) LQ_W4_LAUNCH(TAG, 8, true);  \
-        else if (np <= 16) LQ_W4_LAUNCH(TAG, 16, false); \
-        else LQ_W4_LAUNCH(TAG, 32, false);             \
+#define LQ_W4_NP(TAG)                            \
+    do {                                         \
+        if (np <= 1) LQ_W4_LAUNCH(TAG, 1);       \
+        else if (np <= 2) LQ_W4_LAUNCH(TAG, 2);  \
+        else if (np <= 4) LQ_W4_LAUNCH(TAG, 4);  \
+        else if (np <= 6) LQ_W4_LAUNCH(TAG, 6);  \
+        else if (np <= 8) LQ_W4_LAUNCH(TAG, 8);  \
+        else if (np <= 16) LQ_W4_LAUNCH(TAG, 16); \
+        else LQ_W4_LAUNCH(TAG, 32);              \
     } while (0)
     switch (x_dtype) {
         case LQ_F16: LQ_W4_NP(F16Tag); break;
@@ -155,6 +233,7 @@ extern "C" int lq_w4a4_quantize(uint32_t* q_words, void* scales, lq_dtype_t scal
     }
 #undef LQ_W4_NP
 #undef LQ_W4_LAUNCH
+#undef LQ_W4_LAUNCH2
     return check_launch("w4a4_quantize");
 }
 

@@ -109,7 +109,7 @@ def sq_dynamic_scale(x, pre) -> np.ndarray:
     (convert_sd_quant_model.py:137-150): amax <= 2^-24 -> scale 1 (q is 0 either way).
     `amax / 127.0` is a double division narrowed to float == correctly rounded fp32 division."""
     t = sq_smoothed(x, pre)
-    amax = np.max(np.abs(t), axis=1).astype(F32)
+    amax = np.fmax.reduce(np.abs(t), axis=1).astype(F32)  # fmax: a NaN operand is dropped, as CUDA's max does
     s = amax / F32(127.0)
     return np.where(amax <= F32(2.0 ** -24), F32(1.0), s).astype(F32)
 
@@ -137,7 +137,7 @@ def int8_weight_quant_device(w, pre):
     """w' = f32(w)/pre[k]; s[n] = max_k|w'|/127; q = sat_s8(rne(w'/s))  (range -128..127)."""
     w = np.asarray(w, dtype=F32)
     wp = w / np.asarray(pre, dtype=F32)[None, :] if pre is not None else w
-    amax = np.max(np.abs(wp), axis=1).astype(F32)
+    amax = np.fmax.reduce(np.abs(wp), axis=1).astype(F32)
     s = (amax / F32(127.0)).astype(F32)
     with np.errstate(divide="ignore", invalid="ignore"):
         q = rne_sat_s8(wp / s[:, None])
@@ -320,7 +320,7 @@ def e4m3_encode(x) -> np.ndarray:
 def fp8_scale(x) -> np.float32:
     """scale = max_i |f32(x_i)| / 448  (load_lora.cu:48-54; the double division narrowed to
     float there equals the correctly rounded fp32 division)."""
-    amax = F32(np.max(np.abs(np.asarray(x, dtype=F32)))) if np.size(x) else F32(0)
+    amax = F32(np.fmax.reduce(np.abs(np.asarray(x, dtype=F32)).reshape(-1))) if np.size(x) else F32(0)
     return F32(amax / F32(448.0))
 
 
@@ -377,7 +377,7 @@ def w4a4_quant_values(x, smooth, group: int = 64, scale_dtype: str = "f32"):
     m, k = x.shape
     v = x / np.asarray(smooth, dtype=F32)[None, :] if smooth is not None else x
     vg = v.reshape(m, k // group, group)
-    amax = np.max(np.abs(vg), axis=2).astype(F32)
+    amax = np.fmax.reduce(np.abs(vg), axis=2).astype(F32)  # fmax semantics (w4a4_gemm.cu:905-907 use max())
     s = (amax / F32(7.0)).astype(F32)
     s = round_to(s, scale_dtype)
     with np.errstate(divide="ignore", invalid="ignore"):
