@@ -60,12 +60,12 @@ template <int CH> __device__ __forceinline__ int chunk_swizzle(int row) {
 
 // Remap the linear workgroup id so that ids congruent modulo 8 (one XCD) get consecutive tile
 // numbers, then walk tiles in bands of GROUP_M tile rows (column-major inside a band).
+template <int GROUP_M>
 __device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
     const int total = tiles_m * tiles_n;
     const int per_xcd = total / 8;
     int pid = bid;
     if (bid < per_xcd * 8) pid = (bid & 7) * per_xcd + (bid >> 3);
-    constexpr int GROUP_M = 4;
     const int band = GROUP_M * tiles_n;
     const int first_m = (pid / band) * GROUP_M;
     const int rows = min(tiles_m - first_m, GROUP_M);
@@ -174,7 +174,8 @@ struct GemmKernel {
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const int wm = wave / WN, wn = wave % WN;
         int tm, tn;
-        tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+        // band height chosen so that the workgroups an XCD runs at once cover a roughly square block of C
+        tile_coords<(BM >= 256 ? 4 : 8)>(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
         const int m0 = tm * BM, n0 = tn * BN;
         const int kb = p.kb;
         const int ktiles = kb / BKB;

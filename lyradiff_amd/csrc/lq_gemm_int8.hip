@@ -15,7 +15,9 @@ template <typename OutTag> static int run_int8(GemmParams p, hipStream_t st) {
     if (t < 0) {
         const long t256 = (long)((p.m + 255) / 256) * ((p.n + 255) / 256);
         const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
-        t = t256 >= 192 ? 0 : (t128 >= 192 ? 2 : 3);
+        // one round of 256x256 tiles when they fit the 256 CUs at once; otherwise 128x256 tiles, two workgroups
+        // per CU (finer tail, one workgroup's epilogue overlaps the other's MFMA work)
+        t = t256 >= 192 ? (t256 <= 256 ? 0 : 4) : (t128 >= 192 ? 2 : 3);
     }
     switch (t) {
         case 0: return launch_gemm<K_INT8, OutTag, 256, 256, 64, 2, 4, 3>(p, st);
