@@ -26,7 +26,9 @@
 
 namespace lq {
 
-enum GemmKind { K_INT8 = 0, K_FP8 = 1, K_W4A4 = 2 };
+// K_W4A4H: W4A4 whose group scales are 16-bit floats; it converts the int32 group sums for free (see
+// compute_tile), which is exact only because three times such a scale is still an fp32 number.
+enum GemmKind { K_INT8 = 0, K_FP8 = 1, K_W4A4 = 2, K_W4A4H = 3 };
 
 struct GemmParams {
     void* C;
@@ -129,6 +131,10 @@ __device__ __forceinline__ float gelu_fast(float x) {
 __device__ __forceinline__ void dma16(const void* gbase, u32 voff, u32 lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(gbase) : "memory");
 }
+// Same with 4 bytes per lane (lane l lands at lds_addr + 4*l); used for the W4A4 group scales.
+__device__ __forceinline__ void dma4(const void* gbase, u32 voff, u32 lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(voff), "s"(gbase) : "memory");
+}
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
@@ -147,6 +153,7 @@ template <int NP, int G, int... I> __device__ __forceinline__ void sched_interle
 template <int KIND, typename OutTag, int BM, int BN, int BKB, int WM, int WN, int NSTAGE>
 struct GemmKernel {
     static constexpr int NW = WM * WN;
+    static constexpr bool W4 = (KIND == K_W4A4 || KIND == K_W4A4H);
     static constexpr int THREADS = NW * 64;
     static constexpr int TM = BM / WM, TN = BN / WN;  // wavefront tile
     static constexpr int MT = TM / 32, NT = TN / 32;  // 32x32 MFMA tiles per wavefront
@@ -154,16 +161,17 @@ struct GemmKernel {
     static constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
     static constexpr int NGS = BKB / 32;  // W4A4 groups per k-tile (one group of 64 int4 = 32 bytes)
     static constexpr int NS = NGS * (BM + BN);
-    static constexpr int SCALE_BYTES = (KIND == K_W4A4) ? NS * 4 : 0;
+    static constexpr int S_DMA = W4 ? (NS + 64 * NW - 1) / (64 * NW) : 0;  // 4-byte scale transfers per wavefront per tile
+    static constexpr int SCALE_BYTES = S_DMA * NW * 256;  // NS floats, padded to whole transfers
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + SCALE_BYTES;
     static constexpr int SMEM_BYTES = NSTAGE * STAGE_BYTES;
     static constexpr int A_DMA = A_BYTES / 1024 / NW, B_DMA = B_BYTES / 1024 / NW;  // transfers per wavefront per tile
-    static constexpr int SCH = (KIND == K_W4A4) ? (NS + THREADS - 1) / THREADS : 1;
+    static constexpr int PER_TILE = A_DMA + B_DMA + S_DMA;
     static_assert(A_BYTES % (1024 * NW) == 0 && B_BYTES % (1024 * NW) == 0, "tile/wavefront mismatch");
     static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of 32");
     static_assert(CH == 4 || CH == 8, "BKB must be 64 or 128");
-    static_assert(KIND != K_W4A4 || NSTAGE == 2, "the W4A4 scale staging assumes two stages");
-    static_assert((A_DMA + B_DMA) * NSTAGE < 64, "vmcnt is a 6-bit counter");
+    static_assert(!W4 || ((NGS * BM) % 64 == 0 && NGS % 2 == 0), "scale transfer plan");
+    static_assert(PER_TILE * NSTAGE < 64, "vmcnt is a 6-bit counter");
     using AccT = typename std::conditional<KIND == K_FP8, v16f, v16i>::type;
     using FragT = typename std::conditional<KIND == K_FP8, v8i, v4i>::type;
     static constexpr int KSTEP = (KIND == K_FP8) ? 64 : 32;  // operand bytes per MFMA k-step
@@ -199,11 +207,54 @@ struct GemmKernel {
             int rblk = byteoff / (BKB * 32), within = byteoff % (BKB * 32);
             b_voff[i] = (u32)((size_t)min(rblk, blk_last) * b_block_stride) + within + lane * 16;
         }
-        float rs[SCH];
-        auto load_scale = [&](const void* base, size_t idx) -> float {
-            if (p.scale_f16) return f16_bits_to_f32(static_cast<const unsigned short*>(base)[idx]);
-            return static_cast<const float*>(base)[idx];
+        // W4A4 group scales of a k-tile: [NGS][BM] activation scales then [NGS][BN] weight scales, one
+        // 4-byte transfer per scale.  16-bit scales are fetched as the aligned word that holds them (the
+        // number of groups per row and per k-tile is even, so the half is fixed per lane); each lane then
+        // rewrites the slots its own transfers filled as fp32 -- activation scales times 2^-8, which
+        // undoes the widening of both nibble operands -- before the barrier that publishes the stage.
+        const int ng = p.k / 64;
+        constexpr bool S16 = (KIND == K_W4A4H);
+        constexpr int sesz = S16 ? 2 : 4;
+        const char* s_base[S_DMA > 0 ? S_DMA : 1];
+        u32 s_voff[S_DMA > 0 ? S_DMA : 1];
+        if constexpr (W4) {
+#pragma unroll
+            for (int i = 0; i < S_DMA; ++i) {
+                const int first = (wave * S_DMA + i) * 64;  // wavefront-uniform: a transfer is all-A or all-B
+                const bool is_a = first < NGS * BM;
+                int s = first + lane - (is_a ? 0 : NGS * BM);
+                if (!is_a && s >= NGS * BN) s = 0;  // padding slots of the last transfer: fetch something valid
+                const int g = is_a ? s / BM : s / BN, r = is_a ? s % BM : s % BN;
+                const int row = is_a ? min(r, row_last) : min(r, p.n - 1 - n0);
+                s_base[i] = static_cast<const char*>(is_a ? p.sA : p.sB) + (size_t)(is_a ? m0 : n0) * ng * sesz;
+                s_voff[i] = ((u32)(row * ng + g) * (u32)sesz) & ~3u;
+            }
+        }
+        auto issue_scales = [&](int kt, int stage) {
+            if constexpr (W4) {
+                const u32 ss = smem_base + stage * STAGE_BYTES + A_BYTES + B_BYTES + wave * (S_DMA * 256);
+#pragma unroll
+                for (int i = 0; i < S_DMA; ++i) dma4(s_base[i] + (size_t)kt * NGS * sesz, s_voff[i], ss + i * 256);
+            }
         };
+        auto convert_scales = [&](int stage) {
+            if constexpr (W4) {
+                u32* ss = reinterpret_cast<u32*>(smem + stage * STAGE_BYTES + A_BYTES + B_BYTES) + wave * (S_DMA * 64) + lane;
+#pragma unroll
+                for (int i = 0; i < S_DMA; ++i) {
+                    const int first = (wave * S_DMA + i) * 64;
+                    const bool is_a = first < NGS * BM;
+                    if (!is_a && !S16) continue;
+                    const u32 raw = ss[i * 64];
+                    const int slot = first + lane - (is_a ? 0 : NGS * BM);
+                    const int g = (is_a ? slot / BM : slot / BN) & 1;  // which half of the fetched word
+                    float f = S16 ? f16_bits_to_f32((raw >> (16 * g)) & 0xFFFFu) : __uint_as_float(raw);
+                    if (is_a) f *= 0.00390625f;
+                    ss[i * 64] = __float_as_uint(f);
+                }
+            }
+        };
+
         auto issue_tile = [&](int kt, int stage) {
             const uint8_t* ga = a_base + (size_t)kt * BKB;
             const uint8_t* gb = b_base + (size_t)kt * (BKB * 32);
@@ -213,38 +264,11 @@ struct GemmKernel {
             for (int i = 0; i < A_DMA; ++i) dma16(ga, a_voff[i], sa + i * 1024);
 #pragma unroll
             for (int i = 0; i < B_DMA; ++i) dma16(gb, b_voff[i], sb + i * 1024);
+            issue_scales(kt, stage);
         };
-        // W4A4 group scales of a k-tile, staged through registers as [NGS][BM] then [NGS][BN] floats
-        auto load_scales = [&](int kt) {
-            if constexpr (KIND == K_W4A4) {
-                const int ng = p.k / 64;
-#pragma unroll
-                for (int i = 0; i < SCH; ++i) {
-                    int s = tid + i * THREADS;
-                    rs[i] = 0.0f;
-                    if (s < NGS * BM) {
-                        int g = s / BM, r = s % BM;
-                        rs[i] = load_scale(p.sA, (size_t)(m0 + min(r, row_last)) * ng + kt * NGS + g) * 0.00390625f;
-                    } else if (s < NS) {
-                        int t2 = s - NGS * BM;
-                        int g = t2 / BN, r = t2 % BN;
-                        rs[i] = load_scale(p.sB, (size_t)min(n0 + r, p.n - 1) * ng + kt * NGS + g);
-                    }
-                }
-            }
-        };
-        auto store_scales = [&](int stage) {
-            if constexpr (KIND == K_W4A4) {
-                float* ss = reinterpret_cast<float*>(smem + stage * STAGE_BYTES + A_BYTES + B_BYTES);
-#pragma unroll
-                for (int i = 0; i < SCH; ++i)
-                    if (tid + i * THREADS < NS) ss[tid + i * THREADS] = rs[i];
-            }
-        };
-
         // ---- accumulators ----------------------------------------------------------------------
         AccT acc[MT][NT];
-        v16f res[KIND == K_W4A4 ? MT : 1][KIND == K_W4A4 ? NT : 1];
+        v16f res[W4 ? MT : 1][W4 ? NT : 1];
 #pragma unroll
         for (int i = 0; i < MT; ++i)
 #pragma unroll
@@ -252,7 +276,7 @@ struct GemmKernel {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     acc[i][j][v] = 0;
-                    if constexpr (KIND == K_W4A4) res[i][j][v] = 0.0f;
+                    if constexpr (W4) res[i][j][v] = 0.0f;
                 }
 
         // ---- LDS -> register operand fragments ---------------------------------------------------
@@ -289,56 +313,67 @@ struct GemmKernel {
                        (int)(((u32)d1 << 4) & 0xF0F0F0F0u), (int)((u32)d1 & 0xF0F0F0F0u)};
         };
 
+        // W4A4: one 64-value group = 32 bytes = two 16-byte chunks = two int8 k-steps.  The work of a
+        // stage is a list of (group, n-tile, m-tile) items; the two MFMAs of item t+1 are issued before
+        // the 48 scale operations of item t, so the matrix pipe works in the shadow of the VALU, which
+        // is the bound of this kernel (cvt + mul + fma per output per group, see the header comment).
         auto compute_tile = [&](int stage) {
-            const char* sa = smem + stage * STAGE_BYTES;
-            const char* sb = sa + A_BYTES;
-            if constexpr (KIND != K_W4A4) {
-                FragT w[2][NT], x[2][MT];
-                load_frags(sa, sb, 0, w[0], x[0]);
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    if (ks + 1 < KS) load_frags(sa, sb, ks + 1, w[(ks + 1) & 1], x[(ks + 1) & 1]);
-#pragma unroll
-                    for (int i = 0; i < MT; ++i)
-#pragma unroll
-                        for (int j = 0; j < NT; ++j) {
-                            if constexpr (KIND == K_FP8)
-                                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w[ks & 1][j], x[ks & 1][i], acc[i][j],
-                                                                                           0, 0, 0, 0, 0, 0);
-                            else
-                                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[ks & 1][j], x[ks & 1][i], acc[i][j], 0, 0, 0);
-                        }
-                }
-            } else {  // W4A4: one 64-value group = 32 bytes = two 16-byte chunks = two int8 k-steps
+            if constexpr (W4) {
+                const char* sa = smem + stage * STAGE_BYTES;
+                const char* sb = sa + A_BYTES;
                 const float* ssa = reinterpret_cast<const float*>(sb + B_BYTES);  // [NGS][BM]
                 const float* ssb = ssa + NGS * BM;                                 // [NGS][BN]
+                constexpr int PER_GROUP = NT * MT;
+                v4i wq[2][NT], xq[2][MT];  // raw nibble fragments of the current and the next group
+                v16i pz[2];
+                // K_W4A4H: the group sum S (|S| <= 2^20 after widening) is accumulated on top of the bit
+                // pattern of 1.5 * 2^23, so the accumulator register READ AS A FLOAT is 12582912 + S and
+                // fma(that, sa, -12582912 * sa) = RN(S * sa): the int->float conversion and the first
+                // multiplication in one operation, with the same single rounding.  12582912 * sa is exact
+                // for a scale of at most 22 significant bits, which every 16-bit float has.
+                constexpr int kMagicBits = 0x4B400000;
+                constexpr float kMagic = 12582912.0f;
+                v16i zinit;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) zinit[v] = (KIND == K_W4A4H) ? kMagicBits : 0;
+                if constexpr (KIND == K_W4A4H) asm volatile("" : "+v"(zinit));  // keep one copy in registers, do not rebuild it per item
+                auto issue_item = [&](int g, int t) {  // t: item inside group g
+                    const int j = t / MT, i = t % MT;
+                    v16i z = zinit;
+                    z = __builtin_amdgcn_mfma_i32_32x32x32_i8(widen(wq[g & 1][j], 0), widen(xq[g & 1][i], 0), z, 0, 0, 0);
+                    pz[(g * PER_GROUP + t) & 1] =
+                        __builtin_amdgcn_mfma_i32_32x32x32_i8(widen(wq[g & 1][j], 1), widen(xq[g & 1][i], 1), z, 0, 0, 0);
+                };
+                load_frags(sa, sb, 0, wq[0], xq[0]);
+                issue_item(0, 0);
 #pragma unroll
                 for (int g = 0; g < NGS; ++g) {
-                    v4i wq[NT], xq[MT];
-                    load_frags(sa, sb, g, wq, xq);
-                    float sa_l[MT];
+                    if (g + 1 < NGS) load_frags(sa, sb, g + 1, wq[(g + 1) & 1], xq[(g + 1) & 1]);
+                    float sbv[16];
 #pragma unroll
-                    for (int i = 0; i < MT; ++i) sa_l[i] = ssa[g * BM + xrow + i * 32];
+                    for (int t = 0; t < PER_GROUP; ++t) {
+                        const int j = t / MT, i = t % MT;
+                        if (t + 1 < PER_GROUP) issue_item(g, t + 1);
+                        else if (g + 1 < NGS) issue_item(g + 1, 0);
+                        if (i == 0) {
 #pragma unroll
-                    for (int j = 0; j < NT; ++j) {
-                        v4i w0 = widen(wq[j], 0), w1 = widen(wq[j], 1);
-                        float sbv[16];
-#pragma unroll
-                        for (int q4 = 0; q4 < 4; ++q4) {
-                            float4 t = *reinterpret_cast<const float4*>(ssb + g * BN + wn * TN + j * 32 + q4 * 8 + lh * 4);
-                            sbv[q4 * 4] = t.x; sbv[q4 * 4 + 1] = t.y; sbv[q4 * 4 + 2] = t.z; sbv[q4 * 4 + 3] = t.w;
+                            for (int q4 = 0; q4 < 4; ++q4) {
+                                float4 f = *reinterpret_cast<const float4*>(ssb + g * BN + wn * TN + j * 32 + q4 * 8 + lh * 4);
+                                sbv[q4 * 4] = f.x; sbv[q4 * 4 + 1] = f.y; sbv[q4 * 4 + 2] = f.z; sbv[q4 * 4 + 3] = f.w;
+                            }
                         }
+                        const float sa_l = ssa[g * BM + xrow + i * 32];
+                        const float nmagic_sa = -(kMagic * sa_l);
+                        const v16i cur = pz[(g * PER_GROUP + t) & 1];
 #pragma unroll
-                        for (int i = 0; i < MT; ++i) {
-                            v4i x0 = widen(xq[i], 0), x1 = widen(xq[i], 1);
-                            v16i pz = {0};
-                            pz = __builtin_amdgcn_mfma_i32_32x32x32_i8(w0, x0, pz, 0, 0, 0);
-                            pz = __builtin_amdgcn_mfma_i32_32x32x32_i8(w1, x1, pz, 0, 0, 0);
-#pragma unroll
-                            for (int v = 0; v < 16; ++v)
-                                res[i][j][v] = __builtin_fmaf((float)pz[v] * sa_l[i], sbv[v], res[i][j][v]);
+                        for (int v = 0; v < 16; ++v) {
+                            float t;
+                            if constexpr (KIND == K_W4A4H) t = __builtin_fmaf(__int_as_float(cur[v]), sa_l, nmagic_sa);
+                            else t = (float)cur[v] * sa_l;
+                            res[i][j][v] = __builtin_fmaf(t, sbv[v], res[i][j][v]);
                         }
                     }
+                    __builtin_amdgcn_sched_barrier(0);  // keep the next group's reads and widening from piling up
                 }
             }
         };
@@ -352,8 +387,7 @@ struct GemmKernel {
         // pipe always has queued work while wavefronts sit in the barrier.  One barrier per tile.
         // Every iteration issues exactly one tile of transfers (past the end it re-fetches the last
         // tile into a stage nobody reads again), which makes the vmcnt thresholds compile-time values.
-        constexpr int PER_TILE = A_DMA + B_DMA;
-        if constexpr (KIND != K_W4A4) {
+        if constexpr (!W4) {
             // Operand fragments as 16-byte pieces (an fp8 fragment is two pieces), so that the LDS reads
             // of the next k-step can be interleaved one by one with the MFMAs of the current step.
             constexpr int PPF = (KIND == K_FP8) ? 2 : 1;
@@ -439,16 +473,19 @@ struct GemmKernel {
                 for (; kt < ktiles; ++kt) tile_iter(kt, std::integral_constant<int, 0>{});
             }
         } else {
-            load_scales(0);
-            issue_tile(0, 0);
-            store_scales(0);
+            // W4A4: tile kt+NSTAGE-1 is requested right after the barrier that retires tile kt-1; at the
+            // end of an iteration a wavefront waits for its own transfers of tile kt+1 and rewrites the
+            // scales among them, which the next barrier publishes.
+#pragma unroll
+            for (int s = 0; s < NSTAGE - 1; ++s) issue_tile(min(s, ktiles - 1), s);
+            wait_vmcnt<PER_TILE*(NSTAGE - 2)>();
+            convert_scales(0);
             for (int kt = 0; kt < ktiles; ++kt) {
-                wait_vmcnt<0>();
                 __syncthreads();
-                issue_tile(min(kt + 1, ktiles - 1), (kt + 1) % NSTAGE);
-                if (kt + 1 < ktiles) load_scales(kt + 1);
+                issue_tile(min(kt + NSTAGE - 1, ktiles - 1), (kt + NSTAGE - 1) % NSTAGE);
                 compute_tile(kt % NSTAGE);
-                if (kt + 1 < ktiles) store_scales((kt + 1) % NSTAGE);
+                wait_vmcnt<PER_TILE*(NSTAGE - 2)>();
+                if (kt + 1 < ktiles) convert_scales((kt + 1) % NSTAGE);
             }
         }
         wait_vmcnt<0>();
@@ -493,7 +530,7 @@ struct GemmKernel {
 #pragma unroll
                 for (int q4 = 0; q4 < 4; ++q4) {
                     char* spot = strip + lr * PITCH + (j * 32 + q4 * 8 + lh * 4) * 4;
-                    if constexpr (KIND == K_W4A4)
+                    if constexpr (W4)
                         *reinterpret_cast<float4*>(spot) = make_float4(res[i][j][q4 * 4], res[i][j][q4 * 4 + 1],
                                                                        res[i][j][q4 * 4 + 2], res[i][j][q4 * 4 + 3]);
                     else if constexpr (KIND == K_FP8)
@@ -558,8 +595,19 @@ struct GemmKernel {
 
 // 256-thread configurations are meant to run two workgroups per CU (two wavefronts per SIMD), so that
 // one workgroup's barrier waits, pipeline fill and epilogue overlap with the other's MFMA work.
+// The W4A4 kernel is bound by the vector ALU (three fp32 operations per output per group), so its
+// small-tile configurations ask for more resident wavefronts instead.
+template <int KIND, int BM, int BN, int BKB, int WM, int WN> constexpr int min_workgroups_per_cu() {
+    if (KIND != K_W4A4 && KIND != K_W4A4H) return 2;
+    if (WM * WN > 4) return 1;
+    const int wave_tile = (BM / WM) * (BN / WN);
+    if (wave_tile <= 32 * 32) return 4;
+    if (wave_tile <= 64 * 32) return 3;
+    return BKB == 128 ? 1 : 2;
+}
+
 template <int KIND, typename OutTag, int BM, int BN, int BKB, int WM, int WN, int NSTAGE>
-__global__ __launch_bounds__(WM* WN * 64, 2) void gemm_kernel(GemmParams p) {
+__global__ __launch_bounds__(WM* WN * 64, (min_workgroups_per_cu<KIND, BM, BN, BKB, WM, WN>())) void gemm_kernel(GemmParams p) {
     extern __shared__ __attribute__((aligned(16))) char lq_smem[];
     GemmKernel<KIND, OutTag, BM, BN, BKB, WM, WN, NSTAGE>::run(p, lq_smem);
 }
@@ -567,6 +615,10 @@ __global__ __launch_bounds__(WM* WN * 64, 2) void gemm_kernel(GemmParams p) {
 template <int KIND, typename OutTag, int BM, int BN, int BKB, int WM, int WN, int NSTAGE>
 static int launch_gemm(GemmParams p, hipStream_t st) {
     using GK = GemmKernel<KIND, OutTag, BM, BN, BKB, WM, WN, NSTAGE>;
+    if (p.kb % BKB != 0) {
+        set_error("gemm: row length %d bytes is not a multiple of the %d-byte k-tile", p.kb, BKB);
+        return LQ_ERR_SHAPE;
+    }
     p.tiles_m = (p.m + BM - 1) / BM;
     p.tiles_n = (p.n + BN - 1) / BN;
     auto kern = gemm_kernel<KIND, OutTag, BM, BN, BKB, WM, WN, NSTAGE>;

@@ -16,7 +16,9 @@ template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
         // one round of 256x256 tiles when they fit the 256 CUs at once; otherwise 128x256 tiles, two workgroups
         // per CU (finer tail, one workgroup's epilogue overlaps the other's MFMA work)
         t = t256 >= 192 ? (t256 <= 256 ? 0 : 4) : (t128 >= 192 ? 2 : 3);
+        if (p.k <= 1024 && t128 >= 192) t = 2;  // short K: prologue and epilogue dominate, smaller tiles overlap them better
     }
+    if (t == 1 && p.kb % 128 != 0) t = 0;  // the 128-byte k-tile needs k % 128 == 0
     switch (t) {
         case 0: return launch_gemm<K_FP8, OutTag, 256, 256, 64, 2, 4, 3>(p, st);
         case 1: return launch_gemm<K_FP8, OutTag, 256, 256, 128, 2, 4, 2>(p, st);

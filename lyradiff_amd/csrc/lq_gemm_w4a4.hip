@@ -8,15 +8,19 @@ namespace lq {
 
 int g_tactic_w4a4 = -1;
 
-template <typename OutTag> static int run_w4a4(GemmParams p, hipStream_t st) {
+// Tile configurations.  The kernel is bound by the vector ALU (two or three fp32 operations per output
+// per group, plus widening the nibbles), so the wavefront tile is kept at 64x32 or 32x32 outputs: small
+// enough for three or four wavefronts per SIMD, which hide each other's LDS and MFMA latencies.
+template <int KIND, typename OutTag> static int run_w4a4(GemmParams p, hipStream_t st) {
     int t = g_tactic_w4a4;
     if (t < 0) {
-        const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
-        t = t128 >= 192 ? 0 : 1;
+        const long tiles = (long)((p.m + 63) / 64) * ((p.n + 127) / 128);
+        t = tiles >= 768 ? 0 : 1;  // three workgroups per CU on 256 CUs
     }
     switch (t) {
-        case 0: return launch_gemm<K_W4A4, OutTag, 128, 128, 64, 2, 2, 2>(p, st);
-        case 1: return launch_gemm<K_W4A4, OutTag, 64, 64, 64, 2, 2, 2>(p, st);
+        case 0: return launch_gemm<KIND, OutTag, 64, 128, 64, 1, 4, 2>(p, st);
+        case 1: return launch_gemm<KIND, OutTag, 64, 64, 64, 2, 2, 2>(p, st);
+        case 2: return launch_gemm<KIND, OutTag, 128, 64, 64, 2, 2, 2>(p, st);
         default: set_error("lq_gemm_w4a4: unknown tactic %d", t); return LQ_ERR_ARG;
     }
 }
@@ -37,6 +41,8 @@ extern "C" int lq_gemm_w4a4(void* C, lq_dtype_t out_dtype, const uint32_t* A_wor
     LQ_REQUIRE(reinterpret_cast<uintptr_t>(A_words) % 16 == 0 && reinterpret_cast<uintptr_t>(B_rows32) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(C) % 16 == 0 && reinterpret_cast<uintptr_t>(bias) % 8 == 0,
                LQ_ERR_ARG, "lq_gemm_w4a4: A, B, C must be 16-byte aligned and bias 8-byte aligned");
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(sA) % 4 == 0 && reinterpret_cast<uintptr_t>(sB) % 4 == 0, LQ_ERR_ARG,
+               "lq_gemm_w4a4: scale arrays must be 4-byte aligned");
     if (m == 0) return LQ_OK;
     GemmParams p = {};
     p.C = C; p.A = reinterpret_cast<const uint8_t*>(A_words); p.B = B_rows32; p.bias = bias;
@@ -44,9 +50,9 @@ extern "C" int lq_gemm_w4a4(void* C, lq_dtype_t out_dtype, const uint32_t* A_wor
     p.m = m; p.n = n; p.k = k; p.kb = k / 2;
     hipStream_t st = as_stream(stream);
     switch (out_dtype) {
-        case LQ_F16: return run_w4a4<F16Tag>(p, st);
-        case LQ_BF16: return run_w4a4<BF16Tag>(p, st);
-        case LQ_F32: return run_w4a4<F32Tag>(p, st);
+        case LQ_F16: return p.scale_f16 ? run_w4a4<K_W4A4H, F16Tag>(p, st) : run_w4a4<K_W4A4, F16Tag>(p, st);
+        case LQ_BF16: return p.scale_f16 ? run_w4a4<K_W4A4H, BF16Tag>(p, st) : run_w4a4<K_W4A4, BF16Tag>(p, st);
+        case LQ_F32: return p.scale_f16 ? run_w4a4<K_W4A4H, F32Tag>(p, st) : run_w4a4<K_W4A4, F32Tag>(p, st);
         default: set_error("lq_gemm_w4a4: unsupported output dtype %d", (int)out_dtype); return LQ_ERR_UNSUPPORTED;
     }
 }

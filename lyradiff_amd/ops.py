@@ -266,3 +266,14 @@ def w4a4_linear(a_words, w_rows32, sA, sB, bias=None, out_dtype=torch.bfloat16, 
     _l.check(_l.load().lq_gemm_w4a4(_ptr(c), _DT[out_dtype], _ptr(a_words), _ptr(w_rows32), _ptr(sA), _ptr(sB),
                                     _DT[sA.dtype], _ptr(bias), m, n, k, group, _stream()), "lq_gemm_w4a4")
     return c
+
+
+_KINDS = {"int8": _l.LQ_W_INT8, "fp8": _l.LQ_W_FP8, "int4": _l.LQ_W_INT4}
+
+
+def gemm_set_tactic(kind: str, tactic: int = -1) -> None:
+    """Forces the tile configuration of the `kind` GEMM ("int8", "fp8", "int4"); -1 restores the
+    built-in table (the role of the tactic argument of CutlassInt8GemmRunner<T>::gemm,
+    src/lyradiff/kernels/cutlass_kernels/int8_gemm/int8_gemm.h:24-39)."""
+    _l.check(_l.load().lq_gemm_set_tactic(_KINDS[kind], int(tactic)), "lq_gemm_set_tactic")
+

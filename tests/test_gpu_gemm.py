@@ -135,3 +135,70 @@ def test_w4a4_gemm(ops, dev, m, n, k, sdt):
     y32 = ops.w4a4_linear(torch.from_numpy(qa.view(np.int32)).to(dev), wp, torch.from_numpy(sA).to(sdt_t).to(dev),
                           torch.from_numpy(sB).to(sdt_t).to(dev), None, torch.float32)
     assert np.array_equal(y32.cpu().numpy(), OC.w4a4_gemm(qa, qb, sA, sB, None))
+
+
+# ---- every tile configuration, forced one by one, against the same oracle -------------------------------------------
+N_TACTICS = {"int8": 6, "fp8": 6, "int4": 3}
+
+
+@pytest.fixture
+def tactic_guard(ops):
+    yield
+    for kind in N_TACTICS:
+        ops.gemm_set_tactic(kind, -1)
+
+
+@pytest.mark.parametrize("tactic", range(N_TACTICS["int8"]))
+@pytest.mark.parametrize("k", [704, 768])  # 704: a multiple of 64 only, the 128-byte k-tile configuration falls back
+def test_int8_gemm_every_tactic(ops, dev, tactic, k, tactic_guard):
+    m, n = 333, 416  # ragged M, N a multiple of 32 only
+    g = rng_t(900 + tactic)
+    a = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int8)
+    w = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8)
+    ac = (torch.rand(n, generator=g) * 9e-3 + 1e-3).float()
+    ar = (torch.rand(m, generator=g) * 0.05 + 0.01).float()
+    bias = (torch.randn(n, generator=g) * 0.02).half()
+    ops.gemm_set_tactic("int8", tactic)
+    wp = ops.repack_weight(w.to(dev))
+    acc = ops.int8_linear(a.to(dev), wp, None, None, None, torch.int32)
+    y = ops.int8_linear(a.to(dev), wp, ac.to(dev), ar.to(dev), bias.to(dev), torch.float16)
+    ref_acc = O.gemm_i8_acc(a.numpy(), w.numpy())
+    assert np.array_equal(acc.cpu().numpy(), ref_acc)
+    assert np.array_equal(to_np_f32(y), O.int8_epilogue(ref_acc, ac.numpy(), ar.numpy(), to_np_f32(bias), "f16"))
+
+
+@pytest.mark.parametrize("tactic", range(N_TACTICS["fp8"]))
+@pytest.mark.parametrize("k", [704, 768])
+def test_fp8_gemm_every_tactic(ops, dev, tactic, k, tactic_guard):
+    m, n = 333, 416
+    g = rng_t(950 + tactic)
+    qa, sa = O.fp8_amax_cast(to_np_f32(torch.randn(m, k, generator=g).bfloat16()))
+    qb, sb = O.fp8_amax_cast(to_np_f32((torch.randn(n, k, generator=g) * 0.02).bfloat16()))
+    bias = (torch.randn(n, generator=g) * 0.1).bfloat16()
+    ops.gemm_set_tactic("fp8", tactic)
+    y = ops.fp8_linear(torch.from_numpy(qa).to(dev), ops.repack_weight(torch.from_numpy(qb).to(dev)),
+                       torch.tensor([sa], dtype=torch.float32, device=dev), torch.tensor([sb], dtype=torch.float32, device=dev),
+                       bias.to(dev), False, None, 0.0, torch.bfloat16)
+    assert_close_tol(to_np_f32(y), O.fp8_gemm(qa, qb, sa, sb, to_np_f32(bias), False, None, 0.0, "bf16"), "fp8 tactic",
+                     abs_floor=fp32_sum_floor(qa, qb, sa, sb))
+
+
+@pytest.mark.parametrize("tactic", range(N_TACTICS["int4"]))
+@pytest.mark.parametrize("sdt", ["f32", "f16"])
+def test_w4a4_gemm_every_tactic(ops, dev, tactic, sdt, tactic_guard):
+    m, n, k = 333, 416, 640
+    g = rng_t(1000 + tactic)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.02).bfloat16()
+    qa, sA = O.w4a4_quant(to_np_f32(x), None, 64, sdt)
+    qb, sB = O.w4a4_quant(to_np_f32(w), None, 64, sdt)
+    sdt_t = TORCH_DT[sdt]
+    ops.gemm_set_tactic("int4", tactic)
+    for kk in (k, 128):  # 128: a single k-tile
+        y32 = ops.w4a4_linear(torch.from_numpy(np.ascontiguousarray(qa[:, :kk // 8]).view(np.int32)).to(dev),
+                              ops.repack_weight(torch.from_numpy(np.ascontiguousarray(qb[:, :kk // 8]).view(np.uint8).reshape(n, kk // 2)).to(dev)),
+                              torch.from_numpy(np.ascontiguousarray(sA[:, :kk // 64])).to(sdt_t).to(dev),
+                              torch.from_numpy(np.ascontiguousarray(sB[:, :kk // 64])).to(sdt_t).to(dev), None, torch.float32)
+        ref = OC.w4a4_gemm(np.ascontiguousarray(qa[:, :kk // 8]), np.ascontiguousarray(qb[:, :kk // 8]),
+                           np.ascontiguousarray(sA[:, :kk // 64]), np.ascontiguousarray(sB[:, :kk // 64]), None)
+        assert np.array_equal(y32.cpu().numpy(), ref), f"k={kk}"
