@@ -8,7 +8,8 @@
 // Differences a maintainer has to know:
 //   * the weight operand "B" of every GEMM is the rows32 layout produced once by
 //     repackWeight() / lq_repack_rows32 (same byte count as the [N,K] matrix);
-//   * workspaces are accepted and ignored; tactic profiling is a no-op (static table);
+//   * workspaces are accepted and ignored; tactics are small integers (tile configurations of the
+//     library) and the profiler caches the fastest one per (m bucket, n, k) inside the library;
 //   * the SVDQuant low-rank branch of W4A4 is not built: passing LoRA pointers throws.
 #pragma once
 
@@ -21,6 +22,7 @@
 #include <memory>
 #include <stdexcept>
 #include <string>
+#include <vector>
 
 #include "lyraquant.h"
 
@@ -163,15 +165,97 @@ inline void repackWeight(void* dst_rows32, const void* src_row_major, lq_weight_
                   "repackWeight");
 }
 
+// ---- kernels/cutlass_extensions/.../gemm_configs.h:101-130 --------------------------------------------------
+// A configuration is one of the library's tile configurations; tile_config = -1 means "choose"
+// (ChooseWithHeuristic).  split_k_factor and stages are carried for source compatibility only: the
+// reference's launcher never applies split-k either (int8_gemm_template.h:146-148).
+namespace cutlass_extensions {
+struct CutlassGemmConfig {
+    int tile_config = -1;
+    int split_k_factor = -1;
+    int stages = -1;
+    CutlassGemmConfig() {}
+    CutlassGemmConfig(int tile_config_, int split_k_factor_, int stages_)
+        : tile_config(tile_config_), split_k_factor(split_k_factor_), stages(stages_) {}
+};
+}  // namespace cutlass_extensions
+
+// ---- kernels/cutlass_kernels/int8_gemm/int8_gemm.h:16-90 ----------------------------------------------------
+namespace cutlass_kernels {
+class CutlassInt8GemmRunnerInterface {
+public:
+    virtual ~CutlassInt8GemmRunnerInterface() {}
+    virtual void gemm(int8_t const* A, int8_t const* B, QuantMode quantOption, float const* alphaCol,
+                      float const* alphaRow, void* C, int m, int n, int k,
+                      cutlass_extensions::CutlassGemmConfig gemmConfig, char* workspacePtr, const size_t workspaceBytes,
+                      hipStream_t stream) = 0;
+    virtual size_t getWorkspaceSize(int const m, int const n, int const k) = 0;
+    virtual std::vector<cutlass_extensions::CutlassGemmConfig> getConfigs() const = 0;
+};
+
+template <typename T>
+class CutlassInt8GemmRunner : public virtual CutlassInt8GemmRunnerInterface {
+public:
+    // B is the rows32 layout of the [n,k] weight; C[m,n] = T(float(acc) * (alphaCol[n] * alphaRow[m or 0]))
+    void gemm(int8_t const* A, int8_t const* B, QuantMode quantOption, float const* alphaCol, float const* alphaRow,
+              void* C, int m, int n, int k, cutlass_extensions::CutlassGemmConfig gemmConfig, char* /*workspacePtr*/,
+              const size_t /*workspaceBytes*/, hipStream_t stream) override {
+        lq_gemm_set_thread_tactic(gemmConfig.tile_config);
+        const int status = lq_gemm_int8(C, detail::DType<T>::value, A, B, alphaCol, alphaRow,
+                                        quantOption.hasPerTokenScaling(), nullptr, m, n, k, stream);
+        lq_gemm_set_thread_tactic(-1);
+        detail::check(status, "CutlassInt8GemmRunner::gemm");
+    }
+    size_t getWorkspaceSize(int const, int const, int const) override { return 0; }
+    std::vector<cutlass_extensions::CutlassGemmConfig> getConfigs() const override {
+        std::vector<cutlass_extensions::CutlassGemmConfig> configs;
+        for (int t = 0; t < lq_gemm_tactic_count(LQ_W_INT8); ++t) configs.emplace_back(t, 1, -1);
+        return configs;
+    }
+};
+}  // namespace cutlass_kernels
+
 namespace gemm {
 
-// ---- layers/gemm_utils/SmoothQuantGemm.h:29-103, layers/gemm_utils/GemmProfiler.h:131-251 -----------------
-// The run-time tactic search is replaced by a static table inside the library, so the profiler is an
-// empty shell kept for signature compatibility.
+// ---- layers/gemm_utils/GemmProfiler.h:36-63,131-251, layers/gemm_utils/SmoothQuantGemm.h:29-48 ---------------
+struct GemmDims {
+    int minM = 1, maxM = 0, n = 0, k = 0;
+    GemmDims() {}
+    GemmDims(int minM_, int maxM_, int n_, int k_) : minM(minM_), maxM(maxM_), n(n_), k(k_) {}
+};
+
+// Times the library's tile configurations for m = minM rounded up to a power of two, doubling up to
+// maxM, plus maxM itself (GemmProfiler.cc:78-127), and leaves the winners in the library's per-shape
+// cache, where every later GEMM call of that (m bucket, n, k) finds them.  Temporary device memory
+// is allocated for the duration of profileTactics, as the reference's allocateTmpData does.
 class SmoothQuantGemmPluginProfiler {
 public:
     void setQuantMode(QuantMode const& quantMode) { mQuantMode = quantMode; }
+    void setSkip(bool skip) { mSkip = skip; }
+    void profileTactics(GemmDims const& dims, hipStream_t stream = 0) {
+        if (mSkip || dims.maxM <= 0) return;
+        const size_t bytes = lq_gemm_profile_workspace(LQ_W_INT8, dims.maxM, dims.n, dims.k);
+        void* tmp = nullptr;
+        if (bytes == 0 || hipMalloc(&tmp, bytes) != hipSuccess)
+            throw std::runtime_error("[lyradiff Error][profileTactics] Can't allocate tmp workspace for GEMM tactics profiling.");
+        int status = LQ_OK;
+        auto one = [&](int m) {
+            if (status == LQ_OK && lq_gemm_get_shape_tactic(LQ_W_INT8, m, dims.n, dims.k) < 0)
+                status = lq_gemm_profile(LQ_W_INT8, m, dims.n, dims.k, tmp, bytes, nullptr, nullptr, stream);
+        };
+        int m = 1;
+        while (m < dims.minM) m *= 2;
+        for (; m < dims.maxM; m *= 2) one(m);
+        one(dims.maxM);
+        (void)hipFree(tmp);
+        detail::check(status, "profileTactics");
+    }
+    // -1: nothing profiled for this shape, the library's built-in table applies
+    int getBestConfig(int m, int n, int k) const { return mSkip ? -1 : lq_gemm_get_shape_tactic(LQ_W_INT8, m, n, k); }
     QuantMode mQuantMode;
+
+private:
+    bool mSkip = false;
 };
 
 template <typename DataType>
@@ -183,7 +267,10 @@ public:
         : mQuantMode(quantMode), mPluginProfiler(profiler) {}
     SmoothQuantGemmPlugin<DataType>* clone() { return new SmoothQuantGemmPlugin<DataType>(*this); }
     void configurePlugin(int maxM, int K, int N) { mMaxM = maxM; mK = K; mN = N; }
-    int initialize() { return 0; }  // nothing to profile
+    int initialize() {  // configGemm(): profile for mDims = {1, maxM, N, K} (layers/gemm_utils/SmoothQuantGemm.cc:86-96,166-170)
+        if (mPluginProfiler && mMaxM > 0) mPluginProfiler->profileTactics(GemmDims(1, mMaxM, mN, mK));
+        return 0;
+    }
     void terminate() {}
     size_t getWorkspaceSize(int, int, int) { return 0; }
     // C[m,n] = T(float(acc) * (alphaCol[n] * alphaRow[m or 0])); B is the rows32 layout of the [n,k] weight

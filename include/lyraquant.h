@@ -189,6 +189,35 @@ int lq_gemm_w4a4(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const u
  * Unknown tactic numbers make the next GEMM call fail with LQ_ERR_ARG. */
 int lq_gemm_set_tactic(lq_weight_kind_t kind, int tactic);
 
+/* Tile configuration for the GEMM calls the CALLING THREAD makes from now on (any kind), ahead of every
+ * other choice; -1 clears it.  This is how a per-call configuration argument is expressed
+ * (the gemmConfig parameter of CutlassInt8GemmRunner<T>::gemm,
+ * kernels/cutlass_kernels/int8_gemm/int8_gemm.h:24-36) without a process-wide side effect. */
+int lq_gemm_set_thread_tactic(int tactic);
+
+/* Number of tile configurations of the `kind` GEMM: valid tactic numbers are 0 .. count-1
+ * (CutlassInt8GemmRunner<T>::getConfigs, kernels/cutlass_kernels/int8_gemm/int8_gemm.h:38-39). */
+int lq_gemm_tactic_count(lq_weight_kind_t kind);
+
+/* Per-shape tactic cache, the role of the reference's MNKProfileMap
+ * (layers/gemm_utils/GemmProfiler.h:131-251).  A GEMM call picks, in this order: the process-wide
+ * tactic of lq_gemm_set_tactic, the cache entry for its exact (m, n, k), the entry for (m rounded up
+ * to a power of two, n, k) -- the bucket GemmPluginProfiler::getBestConfig uses
+ * (layers/gemm_utils/GemmProfiler.cc:131-143) -- and last the built-in table.  tactic = -1 removes
+ * an entry; lq_gemm_get_shape_tactic returns -1 when no entry applies.  Thread safe. */
+int lq_gemm_set_shape_tactic(lq_weight_kind_t kind, int m, int n, int k, int tactic);
+int lq_gemm_get_shape_tactic(lq_weight_kind_t kind, int m, int n, int k);
+
+/* Set-up-time profiler, the role of GemmPluginProfiler::profileTactics
+ * (layers/gemm_utils/GemmProfiler.cc:78-127,161-265): runs every tile configuration of the `kind`
+ * GEMM on shape (m, n, k) with synthetic operands placed in `workspace` (caller-owned device memory
+ * of at least lq_gemm_profile_workspace(kind, m, n, k) bytes, 256-byte aligned), times each between
+ * two events on `stream`, stores the fastest in the per-shape cache and reports it.  Blocks the host
+ * until the timed runs have finished; not for use under stream capture. */
+size_t lq_gemm_profile_workspace(lq_weight_kind_t kind, int m, int n, int k);
+int lq_gemm_profile(lq_weight_kind_t kind, int m, int n, int k, void* workspace, size_t workspace_bytes,
+                    int* best_tactic, float* best_us, lq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -45,7 +45,7 @@ def _compile(src: str, force: bool) -> str:
         return obj
     cmd = [HIPCC, *FLAGS, "-c", path, "-o", obj]
     if src.endswith(".cpp"):
-        cmd = [HIPCC, "-O2", "-fPIC", "-std=c++17", "-I", os.path.join(ROOT, "include"), "-c", path, "-o", obj]
+        cmd = [HIPCC, "-x", "c++", "-O2", "-fPIC", "-std=c++17", "-I", os.path.join(ROOT, "include"), "-c", path, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")
@@ -66,21 +66,25 @@ def build(force: bool = False, jobs: int | None = None) -> str:
     return LIB
 
 
-def build_compat_check(force: bool = False) -> str:
-    """Compiles tests/cpp/compat_check.cpp (reference-style C++ call sites) against the library."""
-    src = os.path.join(ROOT, "tests", "cpp", "compat_check.cpp")
-    exe = os.path.join(ROOT, "tests", "cpp", "compat_check")
-    hdr = os.path.join(ROOT, "include", "lyradiff_compat.h")
-    if not os.path.exists(src):
-        return ""
-    if not force and os.path.exists(exe) and os.path.getmtime(exe) >= max(os.path.getmtime(src), os.path.getmtime(hdr), os.path.getmtime(LIB)):
-        return exe
-    cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-Wno-unused-command-line-argument", "-I", os.path.join(ROOT, "include"), src, "-o", exe,
-           "-L", PKG, "-llyraquant", "-Wl,-rpath,$ORIGIN/../../lyradiff_amd"]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError(f"compat_check build failed:\n{r.stdout}\n{r.stderr}")
-    return exe
+def build_compat_check(force: bool = False) -> list:
+    """Compiles the reference-style C++ call-site programs under tests/cpp against the library."""
+    exes = []
+    hdrs = [os.path.join(ROOT, "include", h) for h in ("lyradiff_compat.h", "lyradiff_layers.h", "lyraquant.h")]
+    for name in ("compat_check", "layers_check"):
+        src = os.path.join(ROOT, "tests", "cpp", name + ".cpp")
+        exe = os.path.join(ROOT, "tests", "cpp", name)
+        if not os.path.exists(src):
+            continue
+        newest = max(os.path.getmtime(f) for f in [src, LIB, *hdrs])
+        if force or not os.path.exists(exe) or os.path.getmtime(exe) < newest:
+            cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-ffp-contract=off", "-Wno-unused-command-line-argument",
+                   "-I", os.path.join(ROOT, "include"), src, "-o", exe, "-L", PKG, "-llyraquant",
+                   "-Wl,-rpath,$ORIGIN/../../lyradiff_amd"]
+            r = subprocess.run(cmd, capture_output=True, text=True)
+            if r.returncode != 0:
+                raise RuntimeError(f"{name} build failed:\n{r.stdout}\n{r.stderr}")
+        exes.append(exe)
+    return exes
 
 
 if __name__ == "__main__":

@@ -12,6 +12,15 @@ namespace lq {
 
 // ---- error plumbing ---------------------------------------------------------------------------
 void set_error(const char* fmt, ...);  // stores the message for lq_last_error() (thread local)
+extern int g_tactic_int8, g_tactic_fp8, g_tactic_w4a4;  // process-wide forced tile configuration, -1 = none
+extern thread_local int tl_forced_tactic;                // per-thread override used while profiling
+int shape_tactic_lookup(int kind, int m, int n, int k);   // per-shape cache, -1 = no entry
+// Order of precedence for the tile configuration of one GEMM call; -1 means "use the built-in table".
+static inline int requested_tactic(int process_wide, int kind, int m, int n, int k) {
+    if (tl_forced_tactic >= 0) return tl_forced_tactic;
+    if (process_wide >= 0) return process_wide;
+    return shape_tactic_lookup(kind, m, n, k);
+}
 
 #define LQ_REQUIRE(cond, code, ...)     \
     do {                                \

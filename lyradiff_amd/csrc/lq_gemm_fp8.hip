@@ -6,10 +6,9 @@
 
 namespace lq {
 
-int g_tactic_fp8 = -1;
 
 template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
-    int t = g_tactic_fp8;
+    int t = requested_tactic(g_tactic_fp8, LQ_W_FP8, p.m, p.n, p.k);
     if (t < 0) {
         const long t256 = (long)((p.m + 255) / 256) * ((p.n + 255) / 256);
         const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);

@@ -6,12 +6,11 @@
 
 namespace lq {
 
-int g_tactic_int8 = -1;  // -1: static table below; otherwise forced (see lq_gemm_set_tactic)
 
 template <typename OutTag> static int run_int8(GemmParams p, hipStream_t st) {
     // static tile table in place of the reference's run-time tactic profiler
     // (layers/gemm_utils/GemmProfiler.cc:78-127): largest tile that still fills the 256 CUs.
-    int t = g_tactic_int8;
+    int t = requested_tactic(g_tactic_int8, LQ_W_INT8, p.m, p.n, p.k);
     if (t < 0) {
         const long t256 = (long)((p.m + 255) / 256) * ((p.n + 255) / 256);
         const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);

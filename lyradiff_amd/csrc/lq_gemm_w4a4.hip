@@ -6,13 +6,12 @@
 
 namespace lq {
 
-int g_tactic_w4a4 = -1;
 
 // Tile configurations.  The kernel is bound by the vector ALU (two or three fp32 operations per output
 // per group, plus widening the nibbles), so the wavefront tile is kept at 64x32 or 32x32 outputs: small
 // enough for three or four wavefronts per SIMD, which hide each other's LDS and MFMA latencies.
 template <int KIND, typename OutTag> static int run_w4a4(GemmParams p, hipStream_t st) {
-    int t = g_tactic_w4a4;
+    int t = requested_tactic(g_tactic_w4a4, LQ_W_INT4, p.m, p.n, p.k);
     if (t < 0) {
         const long tiles = (long)((p.m + 63) / 64) * ((p.n + 127) / 128);
         t = tiles >= 768 ? 0 : 1;  // three workgroups per CU on 256 CUs

@@ -1,0 +1,135 @@
+// Set-up-time tactic profiler: times every tile configuration of a GEMM on one shape with synthetic
+// operands and records the fastest in the per-shape cache.  Stands in for
+// GemmPluginProfiler::profileTactics / profileTacticForProblem of lyraDiff
+// (layers/gemm_utils/GemmProfiler.cc:78-127,161-265): same idea (warm-up runs, timed runs between two
+// events, keep the minimum), but the caller owns the temporary memory and nothing is allocated here.
+#include "lq_common.h"
+
+namespace lq {
+
+// Pseudo-random operand bytes (fp8: never a NaN code, so the timing is not distorted by NaN handling).
+__global__ void profile_fill_bytes_kernel(uint8_t* dst, size_t n, int avoid_fp8_nan) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        u32 h = (u32)i * 2654435761u;
+        h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+        uint8_t b = (uint8_t)(h >> 8);
+        if (avoid_fp8_nan && (b & 0x7F) == 0x7F) b ^= 1;
+        dst[i] = b;
+    }
+}
+__global__ void profile_fill_f32_kernel(float* dst, size_t n, float v) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = v;
+}
+__global__ void profile_fill_u16_kernel(unsigned short* dst, size_t n, unsigned short v) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = v;
+}
+
+static size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct ProfileLayout {
+    size_t a, b, c, s0, s1, total;  // byte offsets of A, B, C and the two scale arrays
+    size_t a_bytes, b_bytes, s0_elems, s1_elems;
+};
+
+static ProfileLayout profile_layout(lq_weight_kind_t kind, int m, int n, int k) {
+    ProfileLayout L = {};
+    const size_t kb = lq_weight_row_bytes(kind, k);
+    L.a_bytes = (size_t)m * kb;
+    L.b_bytes = (size_t)n * kb;
+    if (kind == LQ_W_INT8) { L.s0_elems = n; L.s1_elems = m; }                      // alpha_col, alpha_row (fp32)
+    else if (kind == LQ_W_FP8) { L.s0_elems = 1; L.s1_elems = 1; }                  // a_scale, b_scale (fp32)
+    else { L.s0_elems = (size_t)m * (k / 64); L.s1_elems = (size_t)n * (k / 64); }  // group scales (fp16)
+    const size_t esz = kind == LQ_W_INT4 ? 2 : 4;
+    L.a = 0;
+    L.b = L.a + up256(L.a_bytes);
+    L.c = L.b + up256(L.b_bytes);
+    L.s0 = L.c + up256((size_t)m * n * 2);
+    L.s1 = L.s0 + up256(L.s0_elems * esz);
+    L.total = L.s1 + up256(L.s1_elems * esz);
+    return L;
+}
+
+}  // namespace lq
+
+using namespace lq;
+
+extern "C" size_t lq_gemm_profile_workspace(lq_weight_kind_t kind, int m, int n, int k) {
+    if (m <= 0 || n <= 0 || k <= 0 || lq_gemm_tactic_count(kind) < 0) return 0;
+    return profile_layout(kind, m, n, k).total;
+}
+
+extern "C" int lq_gemm_profile(lq_weight_kind_t kind, int m, int n, int k, void* workspace, size_t workspace_bytes,
+                               int* best_tactic, float* best_us, lq_stream_t stream) {
+    const int count = lq_gemm_tactic_count(kind);
+    if (count < 0) return count;
+    LQ_REQUIRE(m > 0 && n > 0 && k > 0, LQ_ERR_SHAPE, "lq_gemm_profile: bad shape m=%d n=%d k=%d", m, n, k);
+    const ProfileLayout L = profile_layout(kind, m, n, k);
+    LQ_REQUIRE(workspace != nullptr && workspace_bytes >= L.total && reinterpret_cast<uintptr_t>(workspace) % 256 == 0,
+               LQ_ERR_ARG, "lq_gemm_profile: workspace must be 256-byte aligned and hold %zu bytes (got %zu)", L.total,
+               workspace_bytes);
+    hipStream_t st = as_stream(stream);
+    char* base = static_cast<char*>(workspace);
+    hipLaunchKernelGGL(profile_fill_bytes_kernel, dim3(1024), dim3(256), 0, st, reinterpret_cast<uint8_t*>(base + L.a),
+                       L.a_bytes, kind == LQ_W_FP8);
+    hipLaunchKernelGGL(profile_fill_bytes_kernel, dim3(1024), dim3(256), 0, st, reinterpret_cast<uint8_t*>(base + L.b),
+                       L.b_bytes, kind == LQ_W_FP8);
+    if (kind == LQ_W_INT4) {
+        hipLaunchKernelGGL(profile_fill_u16_kernel, dim3(256), dim3(256), 0, st, reinterpret_cast<unsigned short*>(base + L.s0),
+                           L.s0_elems, (unsigned short)0x2C00);  // 1/16 as fp16
+        hipLaunchKernelGGL(profile_fill_u16_kernel, dim3(256), dim3(256), 0, st, reinterpret_cast<unsigned short*>(base + L.s1),
+                           L.s1_elems, (unsigned short)0x2C00);
+    } else {
+        hipLaunchKernelGGL(profile_fill_f32_kernel, dim3(256), dim3(256), 0, st, reinterpret_cast<float*>(base + L.s0),
+                           L.s0_elems, 0.01f);
+        hipLaunchKernelGGL(profile_fill_f32_kernel, dim3(256), dim3(256), 0, st, reinterpret_cast<float*>(base + L.s1),
+                           L.s1_elems, 0.01f);
+    }
+    int rc = check_launch("lq_gemm_profile fill");
+    if (rc != LQ_OK) return rc;
+
+    auto run_once = [&]() -> int {
+        void* C = base + L.c;
+        switch (kind) {
+            case LQ_W_INT8:
+                return lq_gemm_int8(C, LQ_BF16, reinterpret_cast<const int8_t*>(base + L.a), reinterpret_cast<const int8_t*>(base + L.b),
+                                    reinterpret_cast<const float*>(base + L.s0), reinterpret_cast<const float*>(base + L.s1), 1,
+                                    nullptr, m, n, k, stream);
+            case LQ_W_FP8:
+                return lq_gemm_fp8(C, LQ_BF16, reinterpret_cast<const uint8_t*>(base + L.a), reinterpret_cast<const uint8_t*>(base + L.b),
+                                   reinterpret_cast<const float*>(base + L.s0), reinterpret_cast<const float*>(base + L.s1), nullptr, 0,
+                                   nullptr, 0.0f, m, n, k, stream);
+            default:
+                return lq_gemm_w4a4(C, LQ_BF16, reinterpret_cast<const uint32_t*>(base + L.a), reinterpret_cast<const uint8_t*>(base + L.b),
+                                    base + L.s0, base + L.s1, LQ_F16, nullptr, m, n, k, 64, stream);
+        }
+    };
+
+    hipEvent_t ev0, ev1;
+    LQ_REQUIRE(hipEventCreate(&ev0) == hipSuccess && hipEventCreate(&ev1) == hipSuccess, LQ_ERR_HIP,
+               "lq_gemm_profile: cannot create events");
+    constexpr int kWarmup = 2, kRuns = 5;
+    int best = -1;
+    float best_ms = 0.0f;
+    for (int t = 0; t < count; ++t) {
+        tl_forced_tactic = t;
+        bool ok = true;
+        for (int i = 0; i < kWarmup && ok; ++i) ok = run_once() == LQ_OK;
+        if (ok) ok = hipEventRecord(ev0, st) == hipSuccess;
+        for (int i = 0; i < kRuns && ok; ++i) ok = run_once() == LQ_OK;
+        if (ok) ok = hipEventRecord(ev1, st) == hipSuccess && hipEventSynchronize(ev1) == hipSuccess;
+        float ms = 0.0f;
+        if (ok) ok = hipEventElapsedTime(&ms, ev0, ev1) == hipSuccess;
+        if (!ok) {
+            (void)hipGetLastError();  // a configuration that cannot run this shape is skipped, as in the reference
+            continue;
+        }
+        if (best < 0 || ms < best_ms) { best = t; best_ms = ms; }
+    }
+    tl_forced_tactic = -1;
+    (void)hipEventDestroy(ev0);
+    (void)hipEventDestroy(ev1);
+    LQ_REQUIRE(best >= 0, LQ_ERR_UNSUPPORTED, "lq_gemm_profile: no configuration ran for m=%d n=%d k=%d", m, n, k);
+    if (best_tactic) *best_tactic = best;
+    if (best_us) *best_us = best_ms * 1000.0f / kRuns;
+    return lq_gemm_set_shape_tactic(kind, m, n, k, best);
+}

@@ -36,6 +36,12 @@ SYMBOLS = {
     "lq_gemm_fp8": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _P, _F, _I, _I, _I, _P]),
     "lq_gemm_w4a4": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P]),
     "lq_gemm_set_tactic": (_I, [_I, _I]),
+    "lq_gemm_set_thread_tactic": (_I, [_I]),
+    "lq_gemm_tactic_count": (_I, [_I]),
+    "lq_gemm_set_shape_tactic": (_I, [_I, _I, _I, _I, _I]),
+    "lq_gemm_get_shape_tactic": (_I, [_I, _I, _I, _I]),
+    "lq_gemm_profile_workspace": (_Z, [_I, _I, _I, _I]),
+    "lq_gemm_profile": (_I, [_I, _I, _I, _I, _P, _Z, C.POINTER(_I), C.POINTER(_F), _P]),
 }
 
 _lib = None

@@ -3,8 +3,8 @@
 Checks follow the reference's torch binding conventions (CHECK_TH_CUDA / CHECK_CONTIGUOUS /
 dtype TORCH_CHECK, src/lyradiff/th_op/th_utils.h:14-33): inputs must be contiguous device
 tensors of the stated dtype; outputs are allocated with torch.empty on the input's device;
-work is enqueued on the current stream.  The same functions are registered as
-torch.ops.lyradiff.* (see _register_torch_ops).
+work is enqueued on the current stream.  lyradiff_amd/torch_ops.py registers the same functions as
+torch.ops.lyradiff.* custom operators.
 """
 from __future__ import annotations
 
@@ -276,4 +276,34 @@ def gemm_set_tactic(kind: str, tactic: int = -1) -> None:
     built-in table (the role of the tactic argument of CutlassInt8GemmRunner<T>::gemm,
     src/lyradiff/kernels/cutlass_kernels/int8_gemm/int8_gemm.h:24-39)."""
     _l.check(_l.load().lq_gemm_set_tactic(_KINDS[kind], int(tactic)), "lq_gemm_set_tactic")
+
+
+def gemm_tactic_count(kind: str) -> int:
+    return int(_l.load().lq_gemm_tactic_count(_KINDS[kind]))
+
+
+def gemm_profile(kind: str, m: int, n: int, k: int, device=None):
+    """Times every tile configuration of the `kind` GEMM on (m, n, k) and caches the fastest for later
+    calls of that shape (GemmPluginProfiler::profileTactics, src/lyradiff/layers/gemm_utils/
+    GemmProfiler.cc:78-127).  Set-up-time only: allocates a temporary buffer and blocks until timed.
+    Returns (tactic, microseconds per call)."""
+    import ctypes as C
+
+    lib = _l.load()
+    nbytes = int(lib.lq_gemm_profile_workspace(_KINDS[kind], m, n, k))
+    if nbytes == 0:
+        raise ValueError(f"bad profile request kind={kind} m={m} n={n} k={k}")
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device or "cuda")
+    best, us = C.c_int(-1), C.c_float(0.0)
+    _l.check(lib.lq_gemm_profile(_KINDS[kind], m, n, k, ws.data_ptr(), nbytes, C.byref(best), C.byref(us), _stream()),
+             "lq_gemm_profile")
+    return best.value, us.value
+
+
+def gemm_shape_tactic(kind: str, m: int, n: int, k: int, tactic=None) -> int:
+    """Reads (tactic=None) or writes the per-shape tactic cache; -1 removes an entry / means no entry."""
+    lib = _l.load()
+    if tactic is not None:
+        _l.check(lib.lq_gemm_set_shape_tactic(_KINDS[kind], m, n, k, int(tactic)), "lq_gemm_set_shape_tactic")
+    return int(lib.lq_gemm_get_shape_tactic(_KINDS[kind], m, n, k))
 

@@ -1,0 +1,131 @@
+"""torch.ops.lyradiff.* : the tensor-level functions of ops.py registered as PyTorch custom operators.
+
+The reference exposes its kernels to Python through a TORCH_LIBRARY named `lyradiff`
+(src/lyradiff/th_op/pybind.cc:9-97) and functional operators through torch::RegisterOperators
+(src/lyradiff/layers/gemm_utils/WeightOnlyQuantOps.cc:326-351).  Here the same namespace carries
+the quantized-linear operators; each one has a shape-only ("fake") implementation so that the
+operators can be traced and shape-checked without a GPU, and a device implementation that calls the
+C ABI on the current HIP stream.  Importing this module registers the operators once per process.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from . import ops as _ops
+
+_lib_op = torch.library.custom_op
+NAMES = ("sq_quant", "sq_quant_dynamic", "geglu_int8_dynamic", "int8_linear", "fp8_quant", "fp8_scale_cast", "fp8_linear",
+         "w4a4_quant", "w4a4_linear", "repack_weight")
+
+
+@_lib_op("lyradiff::sq_quant", mutates_args=())
+def sq_quant(x: Tensor, pre_quant_scale: Optional[Tensor], input_quant_scale: Tensor, per_token: bool = False) -> Tensor:
+    return _ops.sq_quant(x, pre_quant_scale, input_quant_scale, per_token)
+
+
+@sq_quant.register_fake
+def _(x, pre_quant_scale, input_quant_scale, per_token=False):
+    return x.new_empty(x.shape, dtype=torch.int8)
+
+
+@_lib_op("lyradiff::sq_quant_dynamic", mutates_args=())
+def sq_quant_dynamic(x: Tensor, pre_quant_scale: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
+    return _ops.sq_quant_dynamic(x, pre_quant_scale)
+
+
+@sq_quant_dynamic.register_fake
+def _(x, pre_quant_scale=None):
+    rows = x.numel() // x.shape[-1] if x.shape[-1] else 0
+    return x.new_empty(x.shape, dtype=torch.int8), x.new_empty((rows,), dtype=torch.float32)
+
+
+@_lib_op("lyradiff::geglu_int8_dynamic", mutates_args=())
+def geglu_int8_dynamic(hidden: Tensor, bias: Optional[Tensor] = None,
+                       pre_quant_scale: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
+    return _ops.geglu_int8_dynamic(hidden, bias, pre_quant_scale)
+
+
+@geglu_int8_dynamic.register_fake
+def _(hidden, bias=None, pre_quant_scale=None):
+    d = hidden.shape[-1] // 2
+    rows = hidden.numel() // (2 * d) if d else 0
+    return hidden.new_empty(tuple(hidden.shape[:-1]) + (d,), dtype=torch.int8), hidden.new_empty((rows,), dtype=torch.float32)
+
+
+@_lib_op("lyradiff::int8_linear", mutates_args=())
+def int8_linear(a_q: Tensor, w_rows32: Tensor, alpha_col: Optional[Tensor], alpha_row: Optional[Tensor],
+                bias: Optional[Tensor] = None, out_dtype: torch.dtype = torch.float16) -> Tensor:
+    return _ops.int8_linear(a_q, w_rows32, alpha_col, alpha_row, bias, out_dtype)
+
+
+@int8_linear.register_fake
+def _(a_q, w_rows32, alpha_col, alpha_row, bias=None, out_dtype=torch.float16):
+    return a_q.new_empty((a_q.shape[0], w_rows32.shape[0]), dtype=out_dtype)
+
+
+@_lib_op("lyradiff::fp8_quant", mutates_args=())
+def fp8_quant(x: Tensor) -> Tuple[Tensor, Tensor]:
+    return _ops.fp8_quant(x)
+
+
+@fp8_quant.register_fake
+def _(x):
+    return x.new_empty(x.shape, dtype=torch.uint8), x.new_empty((1,), dtype=torch.float32)
+
+
+@_lib_op("lyradiff::fp8_scale_cast", mutates_args=())
+def fp8_scale_cast(x: Tensor, scale: Tensor, invert: bool = True) -> Tensor:
+    return _ops.fp8_scale_cast(x, scale, invert)
+
+
+@fp8_scale_cast.register_fake
+def _(x, scale, invert=True):
+    return x.new_empty(x.shape, dtype=torch.uint8)
+
+
+@_lib_op("lyradiff::fp8_linear", mutates_args=())
+def fp8_linear(a_q: Tensor, w_rows32: Tensor, a_scale: Tensor, b_scale: Tensor, bias: Optional[Tensor] = None,
+               gelu: bool = False, residual: Optional[Tensor] = None, beta: float = 0.0,
+               out_dtype: torch.dtype = torch.bfloat16) -> Tensor:
+    return _ops.fp8_linear(a_q, w_rows32, a_scale, b_scale, bias, gelu, residual, beta, out_dtype)
+
+
+@fp8_linear.register_fake
+def _(a_q, w_rows32, a_scale, b_scale, bias=None, gelu=False, residual=None, beta=0.0, out_dtype=torch.bfloat16):
+    return a_q.new_empty((a_q.shape[0], w_rows32.shape[0]), dtype=out_dtype)
+
+
+@_lib_op("lyradiff::w4a4_quant", mutates_args=())
+def w4a4_quant(x: Tensor, smooth: Optional[Tensor] = None, scale_dtype: torch.dtype = torch.float32,
+               group: int = 64) -> Tuple[Tensor, Tensor]:
+    return _ops.w4a4_quant(x, smooth, scale_dtype, group)
+
+
+@w4a4_quant.register_fake
+def _(x, smooth=None, scale_dtype=torch.float32, group=64):
+    m, k = x.shape
+    return x.new_empty((m, k // 8), dtype=torch.int32), x.new_empty((m, k // group), dtype=scale_dtype)
+
+
+@_lib_op("lyradiff::w4a4_linear", mutates_args=())
+def w4a4_linear(a_words: Tensor, w_rows32: Tensor, sA: Tensor, sB: Tensor, bias: Optional[Tensor] = None,
+                out_dtype: torch.dtype = torch.bfloat16, group: int = 64) -> Tensor:
+    return _ops.w4a4_linear(a_words, w_rows32, sA, sB, bias, out_dtype, group)
+
+
+@w4a4_linear.register_fake
+def _(a_words, w_rows32, sA, sB, bias=None, out_dtype=torch.bfloat16, group=64):
+    return a_words.new_empty((a_words.shape[0], w_rows32.shape[0]), dtype=out_dtype)
+
+
+@_lib_op("lyradiff::repack_weight", mutates_args=())
+def repack_weight(w_bytes: Tensor) -> Tensor:
+    return _ops.repack_weight(w_bytes)
+
+
+@repack_weight.register_fake
+def _(w_bytes):
+    return torch.empty_like(w_bytes)

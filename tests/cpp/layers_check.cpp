@@ -1,0 +1,186 @@
+// Reference-style use of the layer types (Tensor, TensorMap, Allocator, W4A4GemmWeight, W4A4Gemm,
+// CutlassInt8GemmRunner + profiler) on liblyraquant.so, checked bit for bit against host loops.
+// Exit code 0 when every check passes; one line per check.  Built by lyradiff_amd/build.py, run by
+// tests/test_gpu_compat.py.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "lyradiff_layers.h"
+
+#define CK(x)                                                                        \
+    do {                                                                             \
+        hipError_t e = (x);                                                          \
+        if (e != hipSuccess) {                                                       \
+            std::printf("HIP error %s at line %d\n", hipGetErrorString(e), __LINE__); \
+            return 2;                                                                \
+        }                                                                            \
+    } while (0)
+
+using namespace lyradiff;
+
+static float lcg(unsigned& s) { s = s * 1664525u + 1013904223u; return ((s >> 8) & 0xFFFF) / 65536.0f - 0.5f; }
+static float bf16_round(float f) { return (float)hip_bfloat16(f); }
+
+// group-64 int4 quantisation of one row on the host: q in [-8,7], scale = amax/7 (0 for an all-zero group)
+static void quant_row(const float* v, int k, std::vector<int>& q, std::vector<float>& s) {
+    for (int g = 0; g < k / 64; ++g) {
+        float amax = 0.f;
+        for (int j = 0; j < 64; ++j) amax = std::fmax(amax, std::fabs(v[g * 64 + j]));
+        const float sc = amax / 7.0f;
+        s[g] = sc;
+        for (int j = 0; j < 64; ++j) {
+            float r = sc == 0.f ? 0.f : std::rint(v[g * 64 + j] / sc);
+            q[g * 64 + j] = (int)std::fmin(std::fmax(r, -8.f), 7.f);
+        }
+    }
+}
+
+int main() {
+    hipStream_t st;
+    CK(hipStreamCreate(&st));
+    int failures = 0;
+    unsigned seed = 11;
+
+    // ---------------- W4A4Gemm<bf16> layer: weights from a host cache, forward through TensorMaps -------------
+    {
+        const int m = 100, n = 96, k = 256, G = k / 64;
+        std::vector<float> w(n * k), x(m * k), smooth(k), biasf(n);
+        for (auto& v : w) v = bf16_round(0.1f * lcg(seed));
+        for (auto& v : x) v = bf16_round(3.0f * lcg(seed));
+        for (auto& v : smooth) v = 1.0f + lcg(seed);
+        for (auto& v : biasf) v = bf16_round(lcg(seed));
+        // offline weight quantisation on the host: nibble pairs, low nibble first, row-major [n, k/2]
+        std::vector<int> wq(n * k);
+        std::vector<float> ws(n * G);
+        std::vector<int8_t> wpacked(n * k / 2);
+        for (int r = 0; r < n; ++r) {
+            std::vector<int> q(k);
+            std::vector<float> s(G);
+            quant_row(&w[r * k], k, q, s);
+            for (int j = 0; j < k; ++j) wq[r * k + j] = q[j];
+            for (int g = 0; g < G; ++g) ws[r * G + g] = s[g];
+            for (int j = 0; j < k / 2; ++j) wpacked[r * k / 2 + j] = (int8_t)((q[2 * j] & 0xF) | ((q[2 * j + 1] & 0xF) << 4));
+        }
+        std::vector<hip_bfloat16> bias(n), xb(m * k);
+        for (int i = 0; i < n; ++i) bias[i] = hip_bfloat16(biasf[i]);
+        for (int i = 0; i < m * k; ++i) xb[i] = hip_bfloat16(x[i]);
+
+        Allocator allocator;
+        allocator.setStream(st);
+        W4A4GemmWeight<hip_bfloat16> weights(n, k, 32, /*has_bias=*/true, 64, LyraQuantType::INT4_W4A4, &allocator);
+        std::unordered_map<std::string, void*> cache = {{"blk.packed_weight", wpacked.data()}, {"blk.weight_scale", ws.data()},
+                                                        {"blk.smooth", smooth.data()}, {"blk.bias", bias.data()}};
+        hip_bfloat16 *dx, *dy;
+        CK(hipMalloc(&dx, m * k * 2));
+        CK(hipMalloc(&dy, m * n * 2));
+        CK(hipMemcpy(dx, xb.data(), m * k * 2, hipMemcpyHostToDevice));
+        try {
+            weights.loadWeightsFromCache("blk.", cache, hipMemcpyHostToDevice, st);
+            W4A4Gemm<hip_bfloat16> layer(n, k, 32, true, 64, st, nullptr, &allocator, false);
+            TensorMap in({{"input", Tensor(MEMORY_GPU, TYPE_BF16, {(size_t)m, (size_t)k}, dx)}});
+            TensorMap out({{"output", Tensor(MEMORY_GPU, TYPE_BF16, {(size_t)m, (size_t)n}, dy)}});
+            layer.forward(&out, &in, &weights);
+            layer.forward(&out, &in, &weights);  // second call reuses the named pool buffers
+        } catch (const std::exception& e) {
+            std::printf("exception: %s\n", e.what());
+            return 3;
+        }
+        CK(hipStreamSynchronize(st));
+        std::vector<hip_bfloat16> y(m * n);
+        CK(hipMemcpy(y.data(), dy, m * n * 2, hipMemcpyDeviceToHost));
+        int bad = 0;
+        for (int i = 0; i < m; ++i) {
+            std::vector<float> v(k), s(G);
+            std::vector<int> q(k);
+            for (int j = 0; j < k; ++j) v[j] = x[i * k + j] / smooth[j];
+            quant_row(v.data(), k, q, s);
+            for (int j = 0; j < n; ++j) {
+                float r = 0.f;
+                for (int g = 0; g < G; ++g) {
+                    int p = 0;
+                    for (int t = 0; t < 64; ++t) p += q[g * 64 + t] * wq[j * k + g * 64 + t];
+                    const float t1 = (float)p * s[g];
+                    r = std::fmaf(t1, ws[j * G + g], r);
+                }
+                const float t2 = r + biasf[j];
+                if (bf16_round(t2) != (float)y[i * n + j]) ++bad;
+            }
+        }
+        std::printf("W4A4Gemm<bf16>::forward (quantize + gemm + bias through TensorMap/Allocator): %d mismatches\n", bad);
+        failures += bad != 0;
+        const bool pooled = allocator.getAllSize() == (size_t)((4 * m * G + 31) / 32 * 32 + (4 * m * k / 8 + 31) / 32 * 32);
+        std::printf("named pool holds exactly the two scratch buffers after two forwards: %s\n", pooled ? "yes" : "no");
+        failures += !pooled;
+        bool threw = false;
+        try {
+            TensorMap in({{"inputs", Tensor(MEMORY_GPU, TYPE_BF16, {(size_t)m, (size_t)k}, dx)}});
+            in.at("input");
+        } catch (const LyraException& e) {
+            threw = std::string(e.what()).find("Cannot find a tensor of name input") != std::string::npos;
+        }
+        std::printf("TensorMap::at on a missing key raises LyraException naming the key: %s\n", threw ? "yes" : "no");
+        failures += !threw;
+    }
+
+    // ---------------- CutlassInt8GemmRunner<half>: every configuration gives the same exact result -----------------
+    {
+        const int m = 200, n = 160, k = 192;
+        std::vector<int8_t> a(m * k), w(n * k);
+        std::vector<float> ac(n), ar(m);
+        for (auto& v : a) v = (int8_t)(254.0f * lcg(seed));
+        for (auto& v : w) v = (int8_t)(254.0f * lcg(seed));
+        for (auto& v : ac) v = 0.005f + 0.004f * lcg(seed);
+        for (auto& v : ar) v = 0.05f + 0.04f * lcg(seed);
+        int8_t *da, *dw, *dwp;
+        float *dac, *dar;
+        __half* dc;
+        CK(hipMalloc(&da, m * k)); CK(hipMalloc(&dw, n * k)); CK(hipMalloc(&dwp, n * k));
+        CK(hipMalloc(&dac, n * 4)); CK(hipMalloc(&dar, m * 4)); CK(hipMalloc(&dc, m * n * 2));
+        CK(hipMemcpy(da, a.data(), m * k, hipMemcpyHostToDevice));
+        CK(hipMemcpy(dw, w.data(), n * k, hipMemcpyHostToDevice));
+        CK(hipMemcpy(dac, ac.data(), n * 4, hipMemcpyHostToDevice));
+        CK(hipMemcpy(dar, ar.data(), m * 4, hipMemcpyHostToDevice));
+        std::vector<float> ref(m * n);
+        for (int i = 0; i < m; ++i)
+            for (int j = 0; j < n; ++j) {
+                int acc = 0;
+                for (int p = 0; p < k; ++p) acc += (int)a[i * k + p] * (int)w[j * k + p];
+                ref[i * n + j] = __half2float(__float2half((float)acc * (ac[j] * ar[i])));
+            }
+        int bad = 0, nconf = 0;
+        try {
+            repackWeight(dwp, dw, LQ_W_INT8, n, k, st);
+            cutlass_kernels::CutlassInt8GemmRunner<__half> runner;
+            std::vector<__half> c(m * n);
+            for (auto cfg : runner.getConfigs()) {
+                CK(hipMemsetAsync(dc, 0, m * n * 2, st));
+                runner.gemm(da, dwp, QuantMode::useSmoothQuant(true, true), dac, dar, dc, m, n, k, cfg, nullptr, 0, st);
+                CK(hipStreamSynchronize(st));
+                CK(hipMemcpy(c.data(), dc, m * n * 2, hipMemcpyDeviceToHost));
+                for (int i = 0; i < m * n; ++i) bad += __half2float(c[i]) != ref[i];
+                ++nconf;
+            }
+            // profiler: fills the library's per-shape cache, the plugin then runs the cached configuration
+            auto profiler = std::make_shared<gemm::SmoothQuantGemmPluginProfiler>();
+            gemm::SmoothQuantGemmPlugin<__half> plugin(QuantMode::useSmoothQuant(true, true), profiler);
+            plugin.configurePlugin(/*maxM=*/m, k, n);
+            plugin.initialize();
+            const int best = profiler->getBestConfig(m, n, k);
+            std::printf("profiler picked configuration %d for m=%d n=%d k=%d\n", best, m, n, k);
+            failures += best < 0 || best >= nconf;
+            CK(hipMemsetAsync(dc, 0, m * n * 2, st));
+            plugin.RunGemm(da, dwp, dac, dar, dc, m, n, k, nullptr, st);
+            CK(hipStreamSynchronize(st));
+            CK(hipMemcpy(c.data(), dc, m * n * 2, hipMemcpyDeviceToHost));
+            for (int i = 0; i < m * n; ++i) bad += __half2float(c[i]) != ref[i];
+        } catch (const std::exception& e) {
+            std::printf("exception: %s\n", e.what());
+            return 3;
+        }
+        std::printf("CutlassInt8GemmRunner<half>: %d configurations + profiled plugin run, %d mismatches\n", nconf, bad);
+        failures += bad != 0 || nconf != 6;
+    }
+    return failures == 0 ? 0 : 1;
+}

@@ -69,3 +69,28 @@ def test_wrapper_rejects_host_tensors():
         ops.sq_quant_dynamic(torch.zeros(4, 8, dtype=torch.float16), None)
     with pytest.raises(TypeError):
         ops.sq_quant_dynamic("x", None)
+
+
+def test_shape_tactic_cache(lib):
+    """The per-shape tactic cache is host logic: exact shape first, then m rounded up to a power of two."""
+    from lyradiff_amd import lib as L
+
+    k8, k4 = L.LQ_W_INT8, L.LQ_W_INT4
+    assert lib.lq_gemm_tactic_count(k8) == 6 and lib.lq_gemm_tactic_count(L.LQ_W_FP8) == 6 and lib.lq_gemm_tactic_count(k4) == 3
+    assert lib.lq_gemm_tactic_count(7) < 0
+    assert lib.lq_gemm_get_shape_tactic(k8, 4096, 640, 2560) == -1
+    assert lib.lq_gemm_set_shape_tactic(k8, 4096, 640, 2560, 2) == 0
+    assert lib.lq_gemm_get_shape_tactic(k8, 4096, 640, 2560) == 2
+    assert lib.lq_gemm_get_shape_tactic(k8, 3000, 640, 2560) == 2      # 3000 -> bucket 4096
+    assert lib.lq_gemm_get_shape_tactic(k8, 2048, 640, 2560) == -1     # another bucket
+    assert lib.lq_gemm_get_shape_tactic(k4, 4096, 640, 2560) == -1     # another GEMM
+    assert lib.lq_gemm_set_shape_tactic(k8, 3000, 640, 2560, 4) == 0   # an exact entry wins over the bucket
+    assert lib.lq_gemm_get_shape_tactic(k8, 3000, 640, 2560) == 4
+    assert lib.lq_gemm_set_shape_tactic(k8, 4096, 640, 2560, 6) == -1  # tactic out of range
+    assert b"tactic" in lib.lq_last_error()
+    assert lib.lq_gemm_set_shape_tactic(k8, 3000, 640, 2560, -1) == 0 and lib.lq_gemm_set_shape_tactic(k8, 4096, 640, 2560, -1) == 0
+    assert lib.lq_gemm_get_shape_tactic(k8, 3000, 640, 2560) == -1
+    # profiler argument checks (no GPU work is started)
+    assert lib.lq_gemm_profile_workspace(k8, 1024, 1280, 1280) >= 1024 * 1280 * 2 + 1024 * 1280 * 2
+    assert lib.lq_gemm_profile(k8, 1024, 1280, 1280, None, 0, None, None, None) == -1
+    assert b"workspace" in lib.lq_last_error()

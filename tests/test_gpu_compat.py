@@ -15,3 +15,13 @@ def test_cpp_reference_style_call_sites(dev):
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
     assert "0 mismatches" in r.stdout and "0 outliers" in r.stdout and "prefix: yes" in r.stdout
+
+
+def test_cpp_layer_types(dev):
+    """Tensor/TensorMap/Allocator/W4A4Gemm/CutlassInt8GemmRunner/profiler (include/lyradiff_layers.h)."""
+    exe = os.path.join(ROOT, "tests", "cpp", "layers_check")
+    assert os.path.exists(exe), "build it with `python -m lyradiff_amd.build` (prebuilt binaries travel to the GPU box)"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    print(r.stdout, r.stderr)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.count("0 mismatches") == 2 and r.stdout.count(": yes") == 2

@@ -202,3 +202,22 @@ def test_w4a4_gemm_every_tactic(ops, dev, tactic, sdt, tactic_guard):
         ref = OC.w4a4_gemm(np.ascontiguousarray(qa[:, :kk // 8]), np.ascontiguousarray(qb[:, :kk // 8]),
                            np.ascontiguousarray(sA[:, :kk // 64]), np.ascontiguousarray(sB[:, :kk // 64]), None)
         assert np.array_equal(y32.cpu().numpy(), ref), f"k={kk}"
+
+
+def test_profiler_fills_the_shape_cache(ops, dev, tactic_guard):
+    """lq_gemm_profile picks a valid configuration, later calls of that shape use it, results stay exact."""
+    m, n, k = 1000, 1280, 1280
+    try:
+        for kind in ("int8", "fp8", "int4"):
+            assert ops.gemm_shape_tactic(kind, m, n, k) == -1
+            best, us = ops.gemm_profile(kind, m, n, k, dev)
+            assert 0 <= best < ops.gemm_tactic_count(kind) and 0.5 < us < 5000.0, (kind, best, us)
+            assert ops.gemm_shape_tactic(kind, m, n, k) == best
+        g = rng_t(77)
+        a = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int8)
+        w = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8)
+        acc = ops.int8_linear(a.to(dev), ops.repack_weight(w.to(dev)), None, None, None, torch.int32)
+        assert np.array_equal(acc.cpu().numpy(), O.gemm_i8_acc(a.numpy(), w.numpy()))
+    finally:
+        for kind in ("int8", "fp8", "int4"):
+            ops.gemm_shape_tactic(kind, m, n, k, -1)
