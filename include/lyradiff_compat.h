@@ -10,7 +10,7 @@
 //     repackWeight() / lq_repack_rows32 (same byte count as the [N,K] matrix);
 //   * workspaces are accepted and ignored; tactics are small integers (tile configurations of the
 //     library) and the profiler caches the fastest one per (m bucket, n, k) inside the library;
-//   * the SVDQuant low-rank branch of W4A4 is not built: passing LoRA pointers throws.
+//   * the W4A4 low-rank down projection overwrites its fp32 output instead of adding into it.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -130,30 +130,39 @@ void invokeCudaD2DScaleCpyConvert(fp8_e4m3_t* tgt, const T_IN* src, const float*
 }
 
 // ---- kernels/w4a4_gemm/w4a4_gemm.h:6-30 ------------------------------------------------------------------
+// Quantises A [m,k] (bf16) to group-64 int4 words + fp32 group scales and, when Bptr (lora down, bf16
+// [n = rank, k]) is given, writes the fp32 down projection A . B^T to Cptr [m, n].  The reference ADDS its
+// k-tiles into a Cptr that the caller zeroed (float atomics); here Cptr is simply overwritten with the full sum.
+// group_dim: the reference's own call site passes the number of groups in this slot
+// (layers/w4a4_gemm_block/W4A4Gemm.cc:127-137); both that and the group size 64 are accepted.
 inline void invokeFusedQuantizeAndLoraDownSimple(float* Cptr, uint32_t* quantized_input, float* quantized_scale,
                                                  const void* Aptr /* bf16 [m,k] */, const void* Bptr /* lora down */,
                                                  const float* Smoothptr, int m, int n, int k, int group_dim = 64,
                                                  hipStream_t stream = 0) {
-    (void)n;
-    if (Cptr != nullptr || Bptr != nullptr)
-        throw std::runtime_error("[lyradiff Error][invokeFusedQuantizeAndLoraDownSimple] the low-rank (LoRA-down) "
-                                 "branch is not built; pass null Cptr/Bptr");
-    detail::check(lq_w4a4_quantize(quantized_input, quantized_scale, LQ_F32, Aptr, LQ_BF16, Smoothptr, m, k, group_dim,
-                                   stream),
+    if (group_dim != 64 && group_dim != k / 64)
+        throw std::runtime_error("[lyradiff Error][invokeFusedQuantizeAndLoraDownSimple] only group size 64 is supported");
+    if ((Cptr == nullptr) != (Bptr == nullptr))
+        throw std::runtime_error("[lyradiff Error][invokeFusedQuantizeAndLoraDownSimple] Cptr and Bptr go together");
+    detail::check(lq_w4a4_quantize(quantized_input, quantized_scale, LQ_F32, Aptr, LQ_BF16, Smoothptr, m, k, 64, stream),
                   "invokeFusedQuantizeAndLoraDownSimple");
+    if (Bptr != nullptr)
+        detail::check(lq_lora_down(Cptr, LQ_F32, Aptr, Bptr, LQ_BF16, m, k, n, stream), "invokeFusedQuantizeAndLoraDownSimple");
 }
+// utils/memory_utils.cu:398-402, the float -> T instantiations
+template <typename T_OUT>
+void invokeCudaD2DcpyConvert(T_OUT* tgt, const float* src, const size_t size, hipStream_t stream = 0) {
+    detail::check(lq_cast_f32(tgt, detail::DType<T_OUT>::value, src, size, stream), "invokeCudaD2DcpyConvert");
+}
+// D [m,n] bf16 = W4A4(A, B) + LoraA [m, lora_k] . LoraB [n, lora_k]^T (bf16 operands; both null: no low-rank branch)
 inline void invokeFusedW4A4GemmAndLoraUp(void* Dptr /* bf16 [m,n] */, const void* Aptr, const void* Bptr_rows32,
                                          const void* LoraAptr, const void* LoraBptr, const float* AweightScale,
                                          const float* BweightScale, int m, int n, int k, int lora_k, int groups,
                                          hipStream_t stream, const void* bias = nullptr) {
-    (void)lora_k;
-    if (LoraAptr != nullptr || LoraBptr != nullptr)
-        throw std::runtime_error("[lyradiff Error][invokeFusedW4A4GemmAndLoraUp] the low-rank (LoRA-up) branch is "
-                                 "not built; pass null LoRA pointers");
     if (groups != k / 64)
         throw std::runtime_error("[lyradiff Error][invokeFusedW4A4GemmAndLoraUp] groups must equal k / 64");
-    detail::check(lq_gemm_w4a4(Dptr, LQ_BF16, static_cast<const uint32_t*>(Aptr), static_cast<const uint8_t*>(Bptr_rows32),
-                               AweightScale, BweightScale, LQ_F32, bias, m, n, k, 64, stream),
+    detail::check(lq_gemm_w4a4_lora(Dptr, LQ_BF16, static_cast<const uint32_t*>(Aptr), static_cast<const uint8_t*>(Bptr_rows32),
+                                    AweightScale, BweightScale, LQ_F32, bias, LoraAptr, LoraBptr, LQ_BF16, lora_k, m, n, k, 64,
+                                    stream),
                   "invokeFusedW4A4GemmAndLoraUp");
 }
 

@@ -4,8 +4,7 @@
 // with the reference's names, members and call shapes (paths relative to the reference's
 // src/lyradiff/), so that reference-style layer code compiles against liblyraquant.so.
 //
-// Not built: file loading (loadWeights from .bin files), the npy/torch tensor readers of Tensor, and
-// the SVDQuant low-rank members of the W4A4 layer (kept as null pointers; the layer refuses non-null ones).
+// Not built: file loading (loadWeights from .bin files) and the npy/torch tensor readers of Tensor.
 #pragma once
 
 #include <cstring>
@@ -226,7 +225,7 @@ enum LyraQuantType {
 // ---- layers/w4a4_gemm_block/W4A4GemmWeight.h:7-45, W4A4GemmWeight.cc:31-83 -----------------------------------------
 // Device-resident weights of one W4A4 linear.  `packed_weight` holds the [d_out, d_in/2] nibble matrix in
 // the rows32 layout the GEMM reads; loadWeightsFromCache takes the reference's row-major bytes and
-// repacks them once.  The low-rank members stay null (that branch is not built).
+// repacks them once.  lora_rank = 0 leaves the low-rank members null and the layer skips that branch.
 template <typename T>
 class W4A4GemmWeight {
 public:
@@ -246,6 +245,7 @@ public:
         (void)allocator;
         LYRA_CHECK_WITH_INFO(group_size == 64 && d_in % 128 == 0 && d_out % 32 == 0,
                              "W4A4GemmWeight: needs group_size 64, d_in % 128 == 0, d_out % 32 == 0");
+        LYRA_CHECK_WITH_INFO(lora_rank == 0 || lora_rank == 32 || lora_rank == 64, "W4A4GemmWeight: lora_rank must be 0, 32 or 64");
     }
     W4A4GemmWeight(const W4A4GemmWeight&) = delete;
     W4A4GemmWeight& operator=(const W4A4GemmWeight&) = delete;
@@ -254,6 +254,8 @@ public:
             (void)hipFree(packed_weight);
             (void)hipFree(weight_scale);
             (void)hipFree(smooth);
+            (void)hipFree(lora_up);
+            (void)hipFree(lora_down);
             if (has_bias_) (void)hipFree(bias);
         }
     }
@@ -262,12 +264,17 @@ public:
             dmalloc(&packed_weight, d_out_ * d_in_ / 2);
             dmalloc(&weight_scale, d_out_ * group_num_);
             dmalloc(&smooth, d_in_);
+            if (lora_rank_ > 0) {
+                dmalloc(&lora_up, d_out_ * lora_rank_);
+                dmalloc(&lora_down, d_in_ * lora_rank_);
+            }
             if (has_bias_) dmalloc(&bias, d_out_);
         }
         is_maintain_buffer = true;
     }
     // Keys: prefix + "packed_weight" (row-major [d_out, d_in/2] bytes, two int4 per byte, low nibble first),
-    // "weight_scale", "smooth", "bias" -- the names of the reference's .bin files (W4A4GemmWeight.cc:65-83).
+    // "weight_scale", "smooth", "lora_up" ([d_out, rank]), "lora_down" ([rank, d_in]), "bias" -- the names of
+    // the reference's .bin files (W4A4GemmWeight.cc:65-83).
     virtual void loadWeightsFromCache(std::string prefix, std::unordered_map<std::string, void*>& weights,
                                       hipMemcpyKind memcpyKind, hipStream_t stream = 0) {
         if (!is_maintain_buffer) mallocWeights();
@@ -284,11 +291,16 @@ public:
                                     d_out_, d_in_ / 2, stream) == LQ_OK;
         ok = ok && hipMemcpyAsync(weight_scale, get("weight_scale"), sizeof(float) * d_out_ * group_num_, memcpyKind, stream) == hipSuccess;
         ok = ok && hipMemcpyAsync(smooth, get("smooth"), sizeof(float) * d_in_, memcpyKind, stream) == hipSuccess;
+        if (lora_rank_ > 0) {
+            ok = ok && hipMemcpyAsync(lora_up, get("lora_up"), sizeof(T) * d_out_ * lora_rank_, memcpyKind, stream) == hipSuccess;
+            ok = ok && hipMemcpyAsync(lora_down, get("lora_down"), sizeof(T) * d_in_ * lora_rank_, memcpyKind, stream) == hipSuccess;
+        }
         if (has_bias_) ok = ok && hipMemcpyAsync(bias, get("bias"), sizeof(T) * d_out_, memcpyKind, stream) == hipSuccess;
         ok = ok && hipStreamSynchronize(stream) == hipSuccess;
         (void)hipFree(staging);
         LYRA_CHECK_WITH_INFO(ok, std::string("W4A4GemmWeight::loadWeightsFromCache failed: ") + lq_last_error());
     }
+    size_t lora_rank() const { return lora_rank_; }
     size_t d_out() const { return d_out_; }
     size_t d_in() const { return d_in_; }
     bool has_bias() const { return has_bias_; }
@@ -327,23 +339,31 @@ public:
         LYRA_CHECK_WITH_INFO(input_tensor.shape.size() == 2 && output_tensor.shape.size() == 2, "W4A4Gemm: tensors must be 2-D");
         const size_t m = input_tensor.shape[0], k = input_tensor.shape[1], n = output_tensor.shape[1];
         LYRA_CHECK_WITH_INFO(k == d_in_ && n == d_out_ && output_tensor.shape[0] == m, "W4A4Gemm: shape mismatch");
-        LYRA_CHECK_WITH_INFO(weights->lora_up == nullptr && weights->lora_down == nullptr,
-                             "W4A4Gemm: the low-rank (LoRA) branch is not built");
+        const bool low_rank = weights->lora_up != nullptr && weights->lora_down != nullptr;
+        LYRA_CHECK_WITH_INFO(!low_rank || weights->lora_rank() == lora_rank_, "W4A4Gemm: lora rank of layer and weights differ");
         allocateBuffer(m);
         detail::check(lq_w4a4_quantize(quantized_input_buffer, input_scale_buffer, LQ_F32, input_tensor.getPtr<T>(),
                                        detail::DType<T>::value, weights->smooth, (int)m, (int)k, (int)group_size_, stream_),
                       "W4A4Gemm::forward quantize");
-        detail::check(lq_gemm_w4a4(output_tensor.getPtr<T>(), detail::DType<T>::value, quantized_input_buffer,
-                                   reinterpret_cast<const uint8_t*>(weights->packed_weight), input_scale_buffer,
-                                   weights->weight_scale, LQ_F32, has_bias_ ? weights->bias : nullptr, (int)m, (int)n,
-                                   (int)k, (int)group_size_, stream_),
+        if (low_rank)  // down projection of the unsmoothed input, written as T directly (no fp32 detour)
+            detail::check(lq_lora_down(lora_down_res_buffer2, detail::DType<T>::value, input_tensor.getPtr<T>(), weights->lora_down,
+                                       detail::DType<T>::value, (int)m, (int)k, (int)lora_rank_, stream_),
+                          "W4A4Gemm::forward lora down");
+        detail::check(lq_gemm_w4a4_lora(output_tensor.getPtr<T>(), detail::DType<T>::value, quantized_input_buffer,
+                                        reinterpret_cast<const uint8_t*>(weights->packed_weight), input_scale_buffer,
+                                        weights->weight_scale, LQ_F32, has_bias_ ? weights->bias : nullptr,
+                                        low_rank ? lora_down_res_buffer2 : nullptr, low_rank ? weights->lora_up : nullptr,
+                                        detail::DType<T>::value, (int)lora_rank_, (int)m, (int)n, (int)k, (int)group_size_, stream_),
                       "W4A4Gemm::forward gemm");
         if (is_free_buffer_after_forward_) freeBuffer();
     }
 
 protected:
-    // sizes follow W4A4Gemm.cc:89-92: 4 bytes per 8 inputs, one fp32 scale per group
+    // sizes follow W4A4Gemm.cc:89-92: 4 bytes per 8 inputs, one fp32 scale per group, m x rank low-rank activations
     void allocateBuffer(size_t m) {
+        if (lora_rank_ > 0)
+            lora_down_res_buffer2 = static_cast<T*>(
+                allocator_->reMallocWithName("W4A4Gemm_lora_down_res_buffer2", sizeof(T) * m * lora_rank_, false));
         input_scale_buffer = static_cast<float*>(
             allocator_->reMallocWithName("W4A4Gemm_context_input_scale_buffer", sizeof(float) * m * group_num_, false));
         quantized_input_buffer = static_cast<uint32_t*>(
@@ -358,6 +378,7 @@ protected:
     bool is_free_buffer_after_forward_;
     float* input_scale_buffer = nullptr;
     uint32_t* quantized_input_buffer = nullptr;
+    T* lora_down_res_buffer2 = nullptr;
 };
 
 }  // namespace lyradiff

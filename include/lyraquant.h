@@ -182,6 +182,31 @@ int lq_gemm_w4a4(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const u
                  const void* sA, const void* sB, lq_dtype_t scale_dtype, const void* bias,
                  int m, int n, int k, int group, lq_stream_t stream);
 
+/* W4A4 GEMM with the SVDQuant low-rank branch of invokeFusedW4A4GemmAndLoraUp
+ * (kernels/w4a4_gemm/w4a4_gemm.h:18-30; lora_up_gemm, kernels/w4a4_gemm/w4a4_gemm.cu:514-663):
+ *   C = T( sum_g f32(p_g) * sA * sB  +  sum_r lora_act[m, r] * lora_up[n, r]  [+ bias[n]] ),
+ * the second sum on the 16-bit float matrix instruction with fp32 accumulation, added to the same fp32
+ * accumulator before the single rounding to T.  lora_act [m, lora_rank] and lora_up [n, lora_rank] are
+ * row-major F16 or BF16 (lora_dtype), lora_rank a multiple of 16; both NULL disables the branch and the call
+ * is then exactly lq_gemm_w4a4. */
+int lq_gemm_w4a4_lora(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const uint8_t* B_rows32,
+                      const void* sA, const void* sB, lq_dtype_t scale_dtype, const void* bias,
+                      const void* lora_act, const void* lora_up, lq_dtype_t lora_dtype, int lora_rank,
+                      int m, int n, int k, int group, lq_stream_t stream);
+
+/* Down projection of the low-rank branch, the second half of invokeFusedQuantizeAndLoraDownSimple
+ * (kernels/w4a4_gemm/w4a4_gemm.h:6-16; kernels/w4a4_gemm/w4a4_gemm.cu:931-953):
+ *   out[m, r] = T_out( sum_k x[m, k] * lora_down[r, k] ),  x the UNsmoothed activations,
+ * fp32 accumulation in a fixed order (the reference adds k-tiles with float atomics into a zeroed buffer).
+ * x [m, k] and lora_down [rank, k] row-major F16 or BF16 (dtype), rank 32 or 64, k % 64 == 0;
+ * out_dtype F32 (the reference's intermediate), F16 or BF16. */
+int lq_lora_down(void* out, lq_dtype_t out_dtype, const void* x, const void* lora_down, lq_dtype_t dtype,
+                 int m, int k, int rank, lq_stream_t stream);
+
+/* dst[i] = T(src[i]), the float -> T copy between the reference's two W4A4 kernels
+ * (invokeCudaD2DcpyConvert<T, float>, utils/memory_utils.cu:398-402). */
+int lq_cast_f32(void* dst, lq_dtype_t dst_dtype, const float* src, size_t n, lq_stream_t stream);
+
 /* Forces the tile configuration ("tactic") used by the GEMM of `kind` (process-wide); -1 restores
  * the built-in static table.  Stands in for the CutlassGemmConfig argument of
  * CutlassInt8GemmRunner<T>::gemm and the tactic cache of GemmPluginProfiler

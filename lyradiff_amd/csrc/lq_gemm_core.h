@@ -49,6 +49,11 @@ struct GemmParams {
     const void* sA;
     const void* sB;
     int scale_f16;
+    // w4a4 low-rank branch: C += lora_act[m, rank] . lora_up[n, rank]^T (both 16-bit floats, row-major)
+    const void* lora_act;
+    const void* lora_up;
+    int lora_rank;  // multiple of 16
+    int lora_f16;   // element type: 1 = fp16, 0 = bf16
     int m, n, k;
     int kb;  // bytes per operand row: k (int8/fp8) or k/2 (int4)
     int tiles_m, tiles_n;
@@ -490,6 +495,39 @@ struct GemmKernel {
         }
         wait_vmcnt<0>();
         __syncthreads();  // every transfer has landed and nobody reads operands any more: LDS is reusable
+
+        // ---- W4A4 low-rank branch ---------------------------------------------------------------------------
+        // res += act[m, 0:rank] . up[n, 0:rank]^T on the 16-bit float matrix instruction, straight onto the fp32
+        // accumulators (every 32x32 MFMA has the same result layout).  An operand fragment is the 16 bytes a
+        // lane reads from its own row: eight consecutive rank indices, lanes 32..63 the next eight; rows are
+        // rank*2 bytes apart, so a wavefront reads one contiguous block per fragment.
+        if constexpr (W4) {
+            if (p.lora_act != nullptr) {
+                typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+                typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+                const int rbytes = p.lora_rank * 2;
+                const char* up = static_cast<const char*>(p.lora_up) + (lane >> 5) * 16;
+                const char* act = static_cast<const char*>(p.lora_act) + (lane >> 5) * 16;
+                for (int ks = 0; ks < p.lora_rank / 16; ++ks) {
+                    v4i wf[NT], xf[MT];
+#pragma unroll
+                    for (int j = 0; j < NT; ++j)
+                        wf[j] = *reinterpret_cast<const v4i*>(up + (size_t)min(n0 + wn * TN + j * 32 + (lane & 31), p.n - 1) * rbytes + ks * 32);
+#pragma unroll
+                    for (int i = 0; i < MT; ++i)
+                        xf[i] = *reinterpret_cast<const v4i*>(act + (size_t)min(m0 + wm * TM + i * 32 + (lane & 31), p.m - 1) * rbytes + ks * 32);
+#pragma unroll
+                    for (int i = 0; i < MT; ++i)
+#pragma unroll
+                        for (int j = 0; j < NT; ++j) {
+                            if (p.lora_f16)
+                                res[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, wf[j]), __builtin_bit_cast(v8h, xf[i]), res[i][j], 0, 0, 0);
+                            else
+                                res[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, wf[j]), __builtin_bit_cast(v8bf, xf[i]), res[i][j], 0, 0, 0);
+                        }
+                }
+            }
+        }
 
         // ---- epilogue -------------------------------------------------------------------------------------
         // Each wavefront parks one 32-row band of raw 32-bit accumulators at a time in a private LDS

@@ -28,9 +28,10 @@ template <int KIND, typename OutTag> static int run_w4a4(GemmParams p, hipStream
 
 using namespace lq;
 
-extern "C" int lq_gemm_w4a4(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const uint8_t* B_rows32,
-                            const void* sA, const void* sB, lq_dtype_t scale_dtype, const void* bias, int m, int n,
-                            int k, int group, lq_stream_t stream) {
+extern "C" int lq_gemm_w4a4_lora(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const uint8_t* B_rows32,
+                                 const void* sA, const void* sB, lq_dtype_t scale_dtype, const void* bias,
+                                 const void* lora_act, const void* lora_up, lq_dtype_t lora_dtype, int lora_rank, int m,
+                                 int n, int k, int group, lq_stream_t stream) {
     LQ_REQUIRE(C && A_words && B_rows32 && sA && sB, LQ_ERR_ARG, "lq_gemm_w4a4: null pointer");
     LQ_REQUIRE(group == 64, LQ_ERR_SHAPE, "lq_gemm_w4a4: group=%d, only 64 is supported", group);
     LQ_REQUIRE(scale_dtype == LQ_F32 || scale_dtype == LQ_F16, LQ_ERR_UNSUPPORTED,
@@ -42,10 +43,20 @@ extern "C" int lq_gemm_w4a4(void* C, lq_dtype_t out_dtype, const uint32_t* A_wor
                LQ_ERR_ARG, "lq_gemm_w4a4: A, B, C must be 16-byte aligned and bias 8-byte aligned");
     LQ_REQUIRE(reinterpret_cast<uintptr_t>(sA) % 4 == 0 && reinterpret_cast<uintptr_t>(sB) % 4 == 0, LQ_ERR_ARG,
                "lq_gemm_w4a4: scale arrays must be 4-byte aligned");
+    LQ_REQUIRE((lora_act == nullptr) == (lora_up == nullptr), LQ_ERR_ARG,
+               "lq_gemm_w4a4: the low-rank branch needs both lora_act and lora_up");
+    if (lora_act != nullptr) {
+        LQ_REQUIRE(lora_dtype == LQ_F16 || lora_dtype == LQ_BF16, LQ_ERR_UNSUPPORTED,
+                   "lq_gemm_w4a4: low-rank operands must be F16 or BF16");
+        LQ_REQUIRE(lora_rank > 0 && lora_rank % 16 == 0, LQ_ERR_SHAPE, "lq_gemm_w4a4: lora_rank=%d must be a multiple of 16", lora_rank);
+        LQ_REQUIRE(reinterpret_cast<uintptr_t>(lora_act) % 16 == 0 && reinterpret_cast<uintptr_t>(lora_up) % 16 == 0, LQ_ERR_ARG,
+                   "lq_gemm_w4a4: low-rank operands must be 16-byte aligned");
+    }
     if (m == 0) return LQ_OK;
     GemmParams p = {};
     p.C = C; p.A = reinterpret_cast<const uint8_t*>(A_words); p.B = B_rows32; p.bias = bias;
     p.sA = sA; p.sB = sB; p.scale_f16 = scale_dtype == LQ_F16;
+    p.lora_act = lora_act; p.lora_up = lora_up; p.lora_rank = lora_rank; p.lora_f16 = lora_dtype == LQ_F16;
     p.m = m; p.n = n; p.k = k; p.kb = k / 2;
     hipStream_t st = as_stream(stream);
     switch (out_dtype) {
@@ -54,4 +65,11 @@ extern "C" int lq_gemm_w4a4(void* C, lq_dtype_t out_dtype, const uint32_t* A_wor
         case LQ_F32: return p.scale_f16 ? run_w4a4<K_W4A4H, F32Tag>(p, st) : run_w4a4<K_W4A4, F32Tag>(p, st);
         default: set_error("lq_gemm_w4a4: unsupported output dtype %d", (int)out_dtype); return LQ_ERR_UNSUPPORTED;
     }
+}
+
+extern "C" int lq_gemm_w4a4(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const uint8_t* B_rows32,
+                            const void* sA, const void* sB, lq_dtype_t scale_dtype, const void* bias, int m, int n,
+                            int k, int group, lq_stream_t stream) {
+    return lq_gemm_w4a4_lora(C, out_dtype, A_words, B_rows32, sA, sB, scale_dtype, bias, nullptr, nullptr, LQ_BF16, 0, m, n, k,
+                             group, stream);
 }

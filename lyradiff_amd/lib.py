@@ -35,6 +35,9 @@ SYMBOLS = {
     "lq_gemm_int8": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _P]),
     "lq_gemm_fp8": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _P, _F, _I, _I, _I, _P]),
     "lq_gemm_w4a4": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P]),
+    "lq_gemm_w4a4_lora": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
+    "lq_lora_down": (_I, [_P, _I, _P, _P, _I, _I, _I, _I, _P]),
+    "lq_cast_f32": (_I, [_P, _I, _P, _Z, _P]),
     "lq_gemm_set_tactic": (_I, [_I, _I]),
     "lq_gemm_set_thread_tactic": (_I, [_I]),
     "lq_gemm_tactic_count": (_I, [_I]),

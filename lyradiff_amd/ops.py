@@ -249,8 +249,9 @@ def fp8_linear(a_q, w_rows32, a_scale, b_scale, bias=None, gelu: bool = False, r
     return c
 
 
-def w4a4_linear(a_words, w_rows32, sA, sB, bias=None, out_dtype=torch.bfloat16, group: int = 64):
-    """W4A4 GEMM: a_words int32 [M,K/8], w_rows32 uint8 [N,K/2] (rows32), scales [M,G] / [N,G]."""
+def w4a4_linear(a_words, w_rows32, sA, sB, bias=None, out_dtype=torch.bfloat16, group: int = 64, lora_act=None, lora_up=None):
+    """W4A4 GEMM: a_words int32 [M,K/8], w_rows32 uint8 [N,K/2] (rows32), scales [M,G] / [N,G].
+    lora_act [M,R] and lora_up [N,R] (fp16 or bf16, R a multiple of 16) add the low-rank branch."""
     _chk(a_words, "a_words", (torch.int32,))
     _chk(w_rows32, "w_rows32", (torch.uint8, torch.int8))
     _chk(sA, "sA", (torch.float32, torch.float16))
@@ -262,10 +263,36 @@ def w4a4_linear(a_words, w_rows32, sA, sB, bias=None, out_dtype=torch.bfloat16, 
         raise ValueError("K mismatch between activation and weight")
     if bias is not None:
         _chk(bias, "bias", (out_dtype,))
+    rank, lora_dt = 0, _l.LQ_BF16
+    if (lora_act is None) != (lora_up is None):
+        raise ValueError("the low-rank branch needs both lora_act and lora_up")
+    if lora_act is not None:
+        _chk(lora_act, "lora_act", (torch.float16, torch.bfloat16))
+        _chk(lora_up, "lora_up", (lora_act.dtype,))
+        rank = lora_act.shape[1]
+        if lora_act.shape[0] != m or tuple(lora_up.shape) != (n, rank):
+            raise ValueError("lora_act must be [M,R] and lora_up [N,R]")
+        lora_dt = _DT[lora_act.dtype]
     c = torch.empty((m, n), dtype=out_dtype, device=a_words.device)
-    _l.check(_l.load().lq_gemm_w4a4(_ptr(c), _DT[out_dtype], _ptr(a_words), _ptr(w_rows32), _ptr(sA), _ptr(sB),
-                                    _DT[sA.dtype], _ptr(bias), m, n, k, group, _stream()), "lq_gemm_w4a4")
+    _l.check(_l.load().lq_gemm_w4a4_lora(_ptr(c), _DT[out_dtype], _ptr(a_words), _ptr(w_rows32), _ptr(sA), _ptr(sB),
+                                         _DT[sA.dtype], _ptr(bias), _ptr(lora_act), _ptr(lora_up), lora_dt, rank, m, n, k,
+                                         group, _stream()), "lq_gemm_w4a4_lora")
     return c
+
+
+def lora_down(x, lora_down_w, out_dtype=None):
+    """Low-rank down projection out[M,R] = x[M,K] . lora_down_w[R,K]^T (fp32 accumulation), R = 32 or 64."""
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    _chk(lora_down_w, "lora_down_w", (x.dtype,))
+    m, k = x.shape
+    rank = lora_down_w.shape[0]
+    if lora_down_w.shape[1] != k:
+        raise ValueError("K mismatch between x and lora_down_w")
+    out_dtype = out_dtype or x.dtype
+    out = torch.empty((m, rank), dtype=out_dtype, device=x.device)
+    _l.check(_l.load().lq_lora_down(_ptr(out), _DT[out_dtype], _ptr(x), _ptr(lora_down_w), _DT[x.dtype], m, k, rank, _stream()),
+             "lq_lora_down")
+    return out
 
 
 _KINDS = {"int8": _l.LQ_W_INT8, "fp8": _l.LQ_W_FP8, "int4": _l.LQ_W_INT4}

@@ -441,6 +441,22 @@ def w4a4_gemm_f64(qa, qb, sA, sB, bias=None, group: int = 64, out_dtype: str = "
     return round_to(y.astype(F32), out_dtype)
 
 
+def lora_down_f64(x, down) -> np.ndarray:
+    """Low-rank down projection out[m,r] = sum_k x[m,k]*down[r,k] in fp64 (w4a4_gemm.cu:931-953 accumulates the
+    k-tiles with float atomics, so the reference's own summation order is not defined): tolerance reference."""
+    return np.asarray(x, dtype=np.float64) @ np.asarray(down, dtype=np.float64).T
+
+
+def w4a4_gemm_lora_f64(y32, lora_act, lora_up, bias=None, out_dtype: str = "bf16") -> np.ndarray:
+    """T( y32 + lora_act . lora_up^T [+ bias] ): y32 is the fp32 group-scale sum of the W4A4 GEMM (bit-exact part,
+    see w4a4_gemm in the C twin), the low-rank product is evaluated in fp64 (lora_up_gemm, w4a4_gemm.cu:514-663,
+    runs on tensor cores with an unpinned order): tolerance reference."""
+    y = np.asarray(y32, dtype=np.float64) + np.asarray(lora_act, dtype=np.float64) @ np.asarray(lora_up, dtype=np.float64).T
+    if bias is not None:
+        y = y + np.asarray(bias, dtype=np.float64)[None, :]
+    return round_to(y.astype(F32), out_dtype)
+
+
 # ----------------------------------------------------------------------------------------
 # a16  weight repack contract: a bijection of the [N,K] byte matrix
 #      (reference counterpart: kernels/cutlass_kernels/cutlass_preprocessors.cpp:129-530,

@@ -69,7 +69,7 @@ int main() {
 
         Allocator allocator;
         allocator.setStream(st);
-        W4A4GemmWeight<hip_bfloat16> weights(n, k, 32, /*has_bias=*/true, 64, LyraQuantType::INT4_W4A4, &allocator);
+        W4A4GemmWeight<hip_bfloat16> weights(n, k, /*lora_rank=*/0, /*has_bias=*/true, 64, LyraQuantType::INT4_W4A4, &allocator);
         std::unordered_map<std::string, void*> cache = {{"blk.packed_weight", wpacked.data()}, {"blk.weight_scale", ws.data()},
                                                         {"blk.smooth", smooth.data()}, {"blk.bias", bias.data()}};
         hip_bfloat16 *dx, *dy;
@@ -78,7 +78,7 @@ int main() {
         CK(hipMemcpy(dx, xb.data(), m * k * 2, hipMemcpyHostToDevice));
         try {
             weights.loadWeightsFromCache("blk.", cache, hipMemcpyHostToDevice, st);
-            W4A4Gemm<hip_bfloat16> layer(n, k, 32, true, 64, st, nullptr, &allocator, false);
+            W4A4Gemm<hip_bfloat16> layer(n, k, 0, true, 64, st, nullptr, &allocator, false);
             TensorMap in({{"input", Tensor(MEMORY_GPU, TYPE_BF16, {(size_t)m, (size_t)k}, dx)}});
             TensorMap out({{"output", Tensor(MEMORY_GPU, TYPE_BF16, {(size_t)m, (size_t)n}, dy)}});
             layer.forward(&out, &in, &weights);
@@ -113,6 +113,59 @@ int main() {
         const bool pooled = allocator.getAllSize() == (size_t)((4 * m * G + 31) / 32 * 32 + (4 * m * k / 8 + 31) / 32 * 32);
         std::printf("named pool holds exactly the two scratch buffers after two forwards: %s\n", pooled ? "yes" : "no");
         failures += !pooled;
+        // ---- the same layer with the rank-32 low-rank branch (SVDQuant): y += bf16(x . down^T) . up^T ----
+        {
+            const int R = 32;
+            std::vector<float> down(R * k), up(n * R);
+            for (auto& v : down) v = bf16_round(0.2f * lcg(seed));
+            for (auto& v : up) v = bf16_round(0.5f * lcg(seed));
+            std::vector<hip_bfloat16> downb(R * k), upb(n * R);
+            for (int i = 0; i < R * k; ++i) downb[i] = hip_bfloat16(down[i]);
+            for (int i = 0; i < n * R; ++i) upb[i] = hip_bfloat16(up[i]);
+            W4A4GemmWeight<hip_bfloat16> wl(n, k, R, true, 64, LyraQuantType::INT4_W4A4, &allocator);
+            cache["blk.lora_down"] = downb.data();
+            cache["blk.lora_up"] = upb.data();
+            try {
+                wl.loadWeightsFromCache("blk.", cache, hipMemcpyHostToDevice, st);
+                W4A4Gemm<hip_bfloat16> layer(n, k, R, true, 64, st, nullptr, &allocator, false);
+                TensorMap in({{"input", Tensor(MEMORY_GPU, TYPE_BF16, {(size_t)m, (size_t)k}, dx)}});
+                TensorMap out({{"output", Tensor(MEMORY_GPU, TYPE_BF16, {(size_t)m, (size_t)n}, dy)}});
+                layer.forward(&out, &in, &wl);
+            } catch (const std::exception& e) {
+                std::printf("exception: %s\n", e.what());
+                return 3;
+            }
+            CK(hipStreamSynchronize(st));
+            CK(hipMemcpy(y.data(), dy, m * n * 2, hipMemcpyDeviceToHost));
+            int outliers = 0;
+            for (int i = 0; i < m; ++i) {
+                std::vector<float> v(k), s(G);
+                std::vector<int> q(k);
+                for (int j = 0; j < k; ++j) v[j] = x[i * k + j] / smooth[j];
+                quant_row(v.data(), k, q, s);
+                std::vector<double> ld(R);
+                for (int r = 0; r < R; ++r) {
+                    double acc = 0;
+                    for (int j = 0; j < k; ++j) acc += (double)x[i * k + j] * (double)down[r * k + j];
+                    ld[r] = (double)bf16_round((float)acc);
+                }
+                for (int j = 0; j < n; ++j) {
+                    float r32 = 0.f;
+                    for (int g = 0; g < G; ++g) {
+                        int p = 0;
+                        for (int t = 0; t < 64; ++t) p += q[g * 64 + t] * wq[j * k + g * 64 + t];
+                        r32 = std::fmaf((float)p * s[g], ws[j * G + g], r32);
+                    }
+                    double ref = (double)r32 + (double)biasf[j], mag = std::fabs(ref);
+                    for (int r = 0; r < R; ++r) { ref += ld[r] * (double)up[j * R + r]; mag += std::fabs(ld[r] * (double)up[j * R + r]); }
+                    // bf16 output (8 bits) plus one bf16 ULP of each low-rank activation, whose fp32 sum order is free
+                    if (std::fabs((double)(float)y[i * n + j] - ref) > 0.01 * std::fabs(ref) + 0.01 * mag * 0.5 + 1e-3) ++outliers;
+                }
+            }
+            std::printf("W4A4Gemm<bf16>::forward with the low-rank branch: %d outliers\n", outliers);
+            failures += outliers != 0;
+            allocator.freeWithName("W4A4Gemm_lora_down_res_buffer2");
+        }
         bool threw = false;
         try {
             TensorMap in({{"inputs", Tensor(MEMORY_GPU, TYPE_BF16, {(size_t)m, (size_t)k}, dx)}});

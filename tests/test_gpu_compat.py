@@ -24,4 +24,4 @@ def test_cpp_layer_types(dev):
     r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count("0 mismatches") == 2 and r.stdout.count(": yes") == 2
+    assert r.stdout.count("0 mismatches") == 2 and r.stdout.count(": yes") == 2 and "0 outliers" in r.stdout

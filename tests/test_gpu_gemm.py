@@ -221,3 +221,48 @@ def test_profiler_fills_the_shape_cache(ops, dev, tactic_guard):
     finally:
         for kind in ("int8", "fp8", "int4"):
             ops.gemm_shape_tactic(kind, m, n, k, -1)
+
+
+# ---- W4A4 low-rank branch ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("m,k,rank", [(300, 3072, 32), (4608, 3072, 32), (70, 256, 64)])
+def test_lora_down(ops, dev, dt, m, k, rank):
+    g = rng_t(m + k + rank)
+    x = torch.randn(m, k, generator=g).to(TORCH_DT[dt])
+    down = (torch.randn(rank, k, generator=g) * 0.05).to(TORCH_DT[dt])
+    ref = O.lora_down_f64(to_np_f32(x), to_np_f32(down))
+    mag = np.abs(to_np_f32(x)).astype(np.float64) @ np.abs(to_np_f32(down)).astype(np.float64).T
+    y32 = ops.lora_down(x.to(dev), down.to(dev), torch.float32).cpu().numpy()
+    assert np.all(np.abs(y32 - ref) <= 2.0 ** -20 * mag + 1e-30), "fp32 accumulation error beyond a few ULP of the term magnitudes"
+    y = ops.lora_down(x.to(dev), down.to(dev))
+    assert_close_tol(to_np_f32(y), O.round_to(ref.astype(np.float32), dt), "lora down", abs_floor=2.0 ** -20 * mag)
+    assert torch.equal(ops.lora_down(x.to(dev), down.to(dev)), y), "no atomics: repeated calls agree bit for bit"
+
+
+@pytest.mark.parametrize("sdt", ["f32", "f16"])
+@pytest.mark.parametrize("m,n,k,rank,tactic", [(333, 416, 640, 32, 0), (333, 416, 640, 32, 1), (333, 416, 640, 16, 2), (512, 3072, 3072, 32, -1)])
+def test_w4a4_gemm_with_low_rank_branch(ops, dev, sdt, m, n, k, rank, tactic, tactic_guard):
+    g = rng_t(m + n + k + rank)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.02).bfloat16()
+    bias = (torch.randn(n, generator=g) * 0.1).bfloat16()
+    act = (torch.randn(m, rank, generator=g) * 0.3).bfloat16()
+    up = (torch.randn(n, rank, generator=g) * 0.3).bfloat16()
+    qa, sA = O.w4a4_quant(to_np_f32(x), None, 64, sdt)
+    qb, sB = O.w4a4_quant(to_np_f32(w), None, 64, sdt)
+    sdt_t = TORCH_DT[sdt]
+    ops.gemm_set_tactic("int4", tactic)
+    args = (torch.from_numpy(qa.view(np.int32)).to(dev), ops.repack_weight(torch.from_numpy(qb.view(np.uint8).reshape(n, k // 2)).to(dev)),
+            torch.from_numpy(sA).to(sdt_t).to(dev), torch.from_numpy(sB).to(sdt_t).to(dev))
+    y = ops.w4a4_linear(*args, bias.to(dev), torch.bfloat16, 64, act.to(dev), up.to(dev))
+    y32 = OC.w4a4_gemm(qa, qb, sA, sB, None)
+    ref = O.w4a4_gemm_lora_f64(y32, to_np_f32(act), to_np_f32(up), to_np_f32(bias), "bf16")
+    mag = np.abs(y32).astype(np.float64) + np.abs(to_np_f32(act)).astype(np.float64) @ np.abs(to_np_f32(up)).astype(np.float64).T
+    assert_close_tol(to_np_f32(y), ref, "w4a4 + low rank", abs_floor=2.0 ** -20 * mag)
+    # without the branch the result is still the bit-exact one
+    y0 = ops.w4a4_linear(*args, None, torch.float32)
+    assert np.array_equal(y0.cpu().numpy(), y32)
+    # fp16 operands take the fp16 matrix instruction
+    yh = ops.w4a4_linear(*args, None, torch.float32, 64, act.half().to(dev), up.half().to(dev))
+    refh = y32.astype(np.float64) + to_np_f32(act.half()).astype(np.float64) @ to_np_f32(up.half()).astype(np.float64).T
+    assert np.all(np.abs(yh.cpu().numpy() - refh) <= 2.0 ** -20 * mag + 1e-6 * np.abs(refh))
