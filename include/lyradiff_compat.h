@@ -129,6 +129,38 @@ void invokeCudaD2DScaleCpyConvert(fp8_e4m3_t* tgt, const T_IN* src, const float*
                   "invokeCudaD2DScaleCpyConvert");
 }
 
+// ---- kernels/quant_kernels/layer_norm_int8.h:8-38 ------------------------------------------------------------
+// Static per-tensor scale, as in the reference.  (The C ABI can also produce a dynamic per-token scale.)
+template <typename T>
+void invokeLayerNormInt8O(int8_t* dst, const T* src, const T* gamma, const T* beta, const float* pre_quant_scale,
+                          const float* input_quant_scale, QuantMode /*quant_mode*/, size_t batch_size, size_t channels,
+                          size_t nhiddens, hipStream_t stream, const double eps = 1e-6) {
+    detail::check(lq_layernorm_int8(dst, nullptr, nullptr, src, nullptr, nullptr, gamma, beta, detail::DType<T>::value,
+                                    pre_quant_scale, input_quant_scale, batch_size * channels, nhiddens, (float)eps, stream),
+                  "invokeLayerNormInt8O");
+}
+// dst2 = src + residual + bias (T), dst = int8 of its LayerNorm
+template <typename T>
+void invokeFusedResidualBiasLayerNormInt8O(int8_t* dst, T* dst2, const T* src, const T* residual, const T* bias, const T* gamma,
+                                           const T* beta, const float* pre_quant_scale, const float* input_quant_scale,
+                                           QuantMode /*quant_mode*/, size_t batch_size, size_t channels, size_t nhiddens,
+                                           hipStream_t stream, const double eps = 1e-6) {
+    detail::check(lq_layernorm_int8(dst, nullptr, dst2, src, residual, bias, gamma, beta, detail::DType<T>::value,
+                                    pre_quant_scale, input_quant_scale, batch_size * channels, nhiddens, (float)eps, stream),
+                  "invokeFusedResidualBiasLayerNormInt8O");
+}
+// ---- kernels/norms/layer_norm.h:18-27 followed by utils/memory_utils.cu:441-446 in one launch -------------------
+// (the two calls of layers/flux_attn_post_processor/FluxAttnPostFP8Processor.cc:125-140: adaLN modulation, then the
+// cast to e4m3 with the calibrated static input scale)
+template <typename T>
+void invokeLayerNormWithShiftAndScaleFP8(fp8_e4m3_t* dst, const T* src, const T* scale, const T* shift, const float* input_scale,
+                                         size_t batch_size, size_t channels, size_t nhiddens, hipStream_t stream,
+                                         const double eps = 1e-6) {
+    detail::check(lq_layernorm_mod_fp8(reinterpret_cast<uint8_t*>(dst), src, scale, shift, detail::DType<T>::value, input_scale,
+                                       batch_size, channels, nhiddens, (float)eps, stream),
+                  "invokeLayerNormWithShiftAndScaleFP8");
+}
+
 // ---- kernels/w4a4_gemm/w4a4_gemm.h:6-30 ------------------------------------------------------------------
 // Quantises A [m,k] (bf16) to group-64 int4 words + fp32 group scales and, when Bptr (lora down, bf16
 // [n = rank, k]) is given, writes the fp32 down projection A . B^T to Cptr [m, n].  The reference ADDS its

@@ -182,6 +182,31 @@ int lq_gemm_w4a4(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const u
                  const void* sA, const void* sB, lq_dtype_t scale_dtype, const void* bias,
                  int m, int n, int k, int group, lq_stream_t stream);
 
+/* LayerNorm fused with the INT8 SmoothQuant quantisation that follows it: invokeLayerNormInt8O and, with a
+ * residual, invokeFusedResidualBiasLayerNormInt8O (kernels/quant_kernels/layer_norm_int8.h:8-38):
+ *   h = src [+ residual [+ bias]]   (T arithmetic; h is written to dst2 when a residual is given)
+ *   y = T( gamma[k] * ((h - mean) * rstd) + beta[k] ),  mean/var over the row in fp32, rstd = 1/sqrt(var + eps)
+ *   q = sat_s8(rne( f32(y) * pre[k] / s ))
+ * s = input_quant_scale[0] (static, the reference's mode) or, when scale_out is given instead, the dynamic
+ * per-token scale max_k|f32(y)*pre[k]| / 127 written to scale_out[rows] (amax <= 2^-24: s = 1).
+ * src, residual, dst2 [rows, dim], bias, gamma, beta [dim] of `dtype` (F16 or BF16); pre_quant_scale fp32 [dim]
+ * or NULL; dim % 8 == 0, dim <= 6144.  The statistics are fp32 sums in this library's own fixed order (the
+ * reference runs Welford updates in T), so q agrees with the reference to within one step, not bit for bit. */
+int lq_layernorm_int8(int8_t* dst, float* scale_out, void* dst2, const void* src, const void* residual,
+                      const void* bias, const void* gamma, const void* beta, lq_dtype_t dtype,
+                      const float* pre_quant_scale, const float* input_quant_scale, size_t rows, size_t dim,
+                      float eps, lq_stream_t stream);
+
+/* FLUX adaLN modulation fused with the FP8 cast that follows it: invokeLayerNormWithShiftAndScale
+ * (kernels/norms/layer_norm.h:18-27, kernels/norms/layer_norm.cu:406-475) + invokeCudaD2DScaleCpyConvert
+ * (layers/flux_attn_post_processor/FluxAttnPostFP8Processor.cc:125-140):
+ *   y = T( T( T(scale[b,k] + 1) * T((x - mean) * rstd) ) + shift[b,k] ),  q = e4m3_rne_satfinite( f32(y) * (1/s) )
+ * src [batch * rows_per_batch, dim], scale and shift [batch, dim] of `dtype` (F16 or BF16), s = input_scale[0]
+ * (the reference's calibrated static scale).  Same remark on the statistics as above. */
+int lq_layernorm_mod_fp8(uint8_t* dst, const void* src, const void* scale, const void* shift, lq_dtype_t dtype,
+                         const float* input_scale, size_t batch, size_t rows_per_batch, size_t dim, float eps,
+                         lq_stream_t stream);
+
 /* W4A4 GEMM with the SVDQuant low-rank branch of invokeFusedW4A4GemmAndLoraUp
  * (kernels/w4a4_gemm/w4a4_gemm.h:18-30; lora_up_gemm, kernels/w4a4_gemm/w4a4_gemm.cu:514-663):
  *   C = T( sum_g f32(p_g) * sA * sB  +  sum_r lora_act[m, r] * lora_up[n, r]  [+ bias[n]] ),

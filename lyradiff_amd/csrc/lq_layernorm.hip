@@ -1,0 +1,261 @@
+// LayerNorm fused with the activation quantisation that follows it, the step in front of every
+// quantized linear of the reference's blocks:
+//   * INT8 (SDXL): invokeLayerNormInt8O / invokeFusedResidualBiasLayerNormInt8O
+//     (kernels/quant_kernels/layer_norm_int8.cu:102-556,558-679 of lyraDiff):
+//       h = src [+ residual + bias]  (kept in T, written to dst2 when the residual is fused)
+//       y = T( gamma * ((h - mean) * rstd) + beta ),   q = sat_s8(rne( f32(y) * pre[k] / s ))
+//   * FP8 (FLUX): invokeLayerNormWithShiftAndScale followed by invokeCudaD2DScaleCpyConvert
+//     (kernels/norms/layer_norm.cu:406-475, layers/flux_attn_post_processor/FluxAttnPostFP8Processor.cc:125-140):
+//       y = T( T( T(scale[b,k] + 1) * T((x - mean) * rstd) ) + shift[b,k] ),   q = e4m3( f32(y) * (1/s) )
+// One wavefront owns a row: the row stays in registers between the statistics and the quantisation, so the
+// activation is read once and only the 1-byte codes (and dst2) are written.  Mean and variance are two-pass
+// fp32 sums over the registers (the reference runs Welford updates, in T for the INT8 kernels), reduced across
+// the 64 lanes in a fixed order; rstd = 1 / sqrt(var + eps) with IEEE sqrt and division.
+#include "lq_common.h"
+
+namespace lq {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__device__ __forceinline__ u32 ln_cvt4_e4m3(float a, float b, float c, float d) {  // finite inputs: saturating RNE
+    a = __builtin_amdgcn_fmed3f(a, 448.0f, -448.0f); b = __builtin_amdgcn_fmed3f(b, 448.0f, -448.0f);
+    c = __builtin_amdgcn_fmed3f(c, 448.0f, -448.0f); d = __builtin_amdgcn_fmed3f(d, 448.0f, -448.0f);
+    u32 w = (u32)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    return (u32)__builtin_amdgcn_cvt_pk_fp8_f32(c, d, (int)w, true);
+}
+__device__ __forceinline__ u32 ln_nan_fix(u32 w, const float* y) {  // NaN -> 0x7F | sign, as the cast kernel does
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (y[i] != y[i]) w = (w & ~(0xFFu << (8 * i))) | ((0x7Fu | ((__float_as_uint(y[i]) >> 24) & 0x80u)) << (8 * i));
+    return w;
+}
+
+// QMODE 0: int8, static per-tensor scale; 1: int8, dynamic per-token scale (written to scale_out); 2: fp8, static scale.
+// MOD false: y = gamma*n + beta (vectors of length dim).  MOD true: y = (1 + scale[b])*n + shift[b], b = row / rows_per_batch.
+template <typename Tag, int NP, int QMODE, bool RESID, bool MOD>
+__global__ __launch_bounds__(256) void ln_quant_rows_kernel(uint8_t* __restrict__ dst, void* __restrict__ dst2,
+                                                            float* __restrict__ scale_out, const void* __restrict__ src,
+                                                            const void* __restrict__ residual, const void* __restrict__ bias,
+                                                            const void* __restrict__ gamma, const void* __restrict__ beta,
+                                                            const float* __restrict__ pre, const float* __restrict__ in_scale,
+                                                            size_t rows, int dim, size_t rows_per_batch, float eps) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const size_t row = (size_t)blockIdx.x * 4 + wave;
+    if (row >= rows) return;
+    const size_t row_off = row * (size_t)dim;
+    const unsigned short* xs = static_cast<const unsigned short*>(src) + row_off;
+    const size_t mod_off = MOD ? (row / rows_per_batch) * (size_t)dim : 0;
+    const unsigned short* gs = static_cast<const unsigned short*>(gamma) + mod_off;
+    const unsigned short* bs = static_cast<const unsigned short*>(beta) + mod_off;
+    float h[NP][8];
+    float sum = 0.0f;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        const int col = (p * 64 + lane) * 8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) h[p][i] = 0.0f;
+        if (col < dim) {
+            unpack8<Tag>(*reinterpret_cast<const uint4*>(xs + col), h[p]);
+            if constexpr (RESID) {
+                float r[8], b[8];
+                unpack8<Tag>(*reinterpret_cast<const uint4*>(static_cast<const unsigned short*>(residual) + row_off + col), r);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) h[p][i] = round_through<Tag>(h[p][i] + r[i]);
+                if (bias != nullptr) {
+                    unpack8<Tag>(*reinterpret_cast<const uint4*>(static_cast<const unsigned short*>(bias) + col), b);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) h[p][i] = round_through<Tag>(h[p][i] + b[i]);
+                }
+                uint4 o;
+                u32* ow = reinterpret_cast<u32*>(&o);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) ow[i] = Elem<Tag>::store(h[p][2 * i]) | (Elem<Tag>::store(h[p][2 * i + 1]) << 16);
+                *reinterpret_cast<uint4*>(static_cast<unsigned short*>(dst2) + row_off + col) = o;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sum += h[p][i];
+        }
+    }
+    const float mean = wave_sum(sum) / (float)dim;
+    float sq = 0.0f;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        const int col = (p * 64 + lane) * 8;
+        if (col < dim) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float d = h[p][i] - mean;
+                sq += d * d;
+            }
+        }
+    }
+    const float var = wave_sum(sq) / (float)dim;
+    const float rstd = 1.0f / __builtin_sqrtf(var + eps);
+    // normalise, modulate, round to T; for the int8 modes apply the smoothing vector and collect the row amax
+    float amax = 0.0f;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        const int col = (p * 64 + lane) * 8;
+        if (col < dim) {
+            float g[8], b[8];
+            unpack8<Tag>(*reinterpret_cast<const uint4*>(gs + col), g);
+            unpack8<Tag>(*reinterpret_cast<const uint4*>(bs + col), b);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float n = (h[p][i] - mean) * rstd;
+                float y;
+                if constexpr (MOD) {
+                    const float a = round_through<Tag>(g[i] + 1.0f);
+                    y = round_through<Tag>(round_through<Tag>(a * round_through<Tag>(n)) + b[i]);
+                } else {
+                    y = round_through<Tag>(g[i] * n + b[i]);
+                }
+                h[p][i] = y;
+            }
+            if constexpr (QMODE != 2) {
+                if (pre != nullptr) {
+                    float4 a = *reinterpret_cast<const float4*>(pre + col);
+                    float4 c = *reinterpret_cast<const float4*>(pre + col + 4);
+                    const float pv[8] = {a.x, a.y, a.z, a.w, c.x, c.y, c.z, c.w};
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) h[p][i] = h[p][i] * pv[i];
+                }
+                if constexpr (QMODE == 1) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(h[p][i]));
+                }
+            }
+        }
+    }
+    float s = 1.0f;
+    if constexpr (QMODE == 1) {
+        amax = wave_max(amax);
+        s = amax / 127.0f;
+        if (amax <= 5.9604644775390625e-08f) s = 1.0f;
+        if (lane == 0) scale_out[row] = s;
+    } else {
+        s = in_scale[0];
+    }
+    if constexpr (QMODE == 2) {
+        const float inv = 1.0f / s;
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int col = (p * 64 + lane) * 8;
+            if (col < dim) {
+                float v[8];
+                float nanp = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    v[i] = h[p][i] * inv;
+                    nanp = __builtin_fmaf(v[i], 0.0f, nanp);
+                }
+                uint2 o;
+                o.x = ln_cvt4_e4m3(v[0], v[1], v[2], v[3]);
+                o.y = ln_cvt4_e4m3(v[4], v[5], v[6], v[7]);
+                if (__builtin_expect(!(nanp == 0.0f), 0)) {  // some value is NaN or infinite
+                    o.x = ln_nan_fix(o.x, v);
+                    o.y = ln_nan_fix(o.y, v + 4);
+                }
+                *reinterpret_cast<uint2*>(dst + row_off + col) = o;
+            }
+        }
+    } else {
+        const float r = fast_recip(s);
+        const bool slow = scale_out_of_range(s);
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int col = (p * 64 + lane) * 8;
+            if (col < dim) {
+                int q[8];
+                quant8<-128, 127>(h[p], s, r, slow, q);
+                uint2 o;
+                o.x = pack4_s8(q[0], q[1], q[2], q[3]);
+                o.y = pack4_s8(q[4], q[5], q[6], q[7]);
+                *reinterpret_cast<uint2*>(dst + row_off + col) = o;
+            }
+        }
+    }
+}
+
+struct LnArgs {
+    uint8_t* dst; void* dst2; float* scale_out; const void* src; const void* residual; const void* bias;
+    const void* gamma; const void* beta; const float* pre; const float* in_scale;
+    size_t rows; int dim; size_t rows_per_batch; float eps;
+};
+
+template <typename Tag, int QMODE, bool RESID, bool MOD> static int launch_ln(const LnArgs& a, hipStream_t st) {
+    const int np = (a.dim + 511) / 512;
+    dim3 grid((unsigned)((a.rows + 3) / 4)), block(256);
+#define LQ_LN_CASE(NPV)                                                                                              \
+    hipLaunchKernelGGL((ln_quant_rows_kernel<Tag, NPV, QMODE, RESID, MOD>), grid, block, 0, st, a.dst, a.dst2, a.scale_out, \
+                       a.src, a.residual, a.bias, a.gamma, a.beta, a.pre, a.in_scale, a.rows, a.dim, a.rows_per_batch, a.eps)
+    if (np <= 1) LQ_LN_CASE(1);
+    else if (np <= 2) LQ_LN_CASE(2);
+    else if (np <= 3) LQ_LN_CASE(3);
+    else if (np <= 4) LQ_LN_CASE(4);
+    else if (np <= 6) LQ_LN_CASE(6);
+    else if (np <= 8) LQ_LN_CASE(8);
+    else LQ_LN_CASE(12);
+#undef LQ_LN_CASE
+    return check_launch("layernorm_quant");
+}
+
+static int check_ln_common(const char* what, const void* dst, const void* src, lq_dtype_t dtype, size_t rows, size_t dim) {
+    LQ_REQUIRE(dst && src, LQ_ERR_ARG, "%s: null pointer", what);
+    LQ_REQUIRE(dtype == LQ_F16 || dtype == LQ_BF16, LQ_ERR_UNSUPPORTED, "%s: activations must be F16 or BF16", what);
+    LQ_REQUIRE(dim > 0 && dim % 8 == 0 && dim <= 6144, LQ_ERR_SHAPE, "%s: need dim %% 8 == 0 and dim <= 6144 (dim=%zu)", what, dim);
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(dst) % 8 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0, LQ_ERR_ARG,
+               "%s: src must be 16-byte and dst 8-byte aligned", what);
+    (void)rows;
+    return LQ_OK;
+}
+
+}  // namespace lq
+
+using namespace lq;
+
+extern "C" int lq_layernorm_int8(int8_t* dst, float* scale_out, void* dst2, const void* src, const void* residual,
+                                 const void* bias, const void* gamma, const void* beta, lq_dtype_t dtype,
+                                 const float* pre_quant_scale, const float* input_quant_scale, size_t rows, size_t dim,
+                                 float eps, lq_stream_t stream) {
+    int rc = check_ln_common("lq_layernorm_int8", dst, src, dtype, rows, dim);
+    if (rc != LQ_OK) return rc;
+    LQ_REQUIRE(gamma && beta, LQ_ERR_ARG, "lq_layernorm_int8: gamma and beta are required");
+    LQ_REQUIRE((scale_out != nullptr) != (input_quant_scale != nullptr), LQ_ERR_ARG,
+               "lq_layernorm_int8: pass input_quant_scale (static) or scale_out (dynamic per token), not both");
+    LQ_REQUIRE(residual != nullptr || bias == nullptr, LQ_ERR_ARG, "lq_layernorm_int8: bias is only added together with a residual");
+    LQ_REQUIRE(residual == nullptr || dst2 != nullptr, LQ_ERR_ARG, "lq_layernorm_int8: dst2 is required with a residual");
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(residual) % 16 == 0 && reinterpret_cast<uintptr_t>(dst2) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(bias) % 16 == 0 && reinterpret_cast<uintptr_t>(gamma) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(beta) % 16 == 0 && reinterpret_cast<uintptr_t>(pre_quant_scale) % 16 == 0,
+               LQ_ERR_ARG, "lq_layernorm_int8: vectors must be 16-byte aligned");
+    if (rows == 0) return LQ_OK;
+    LnArgs a = {reinterpret_cast<uint8_t*>(dst), dst2, scale_out, src, residual, bias, gamma, beta, pre_quant_scale,
+                input_quant_scale, rows, (int)dim, 1, eps};
+    hipStream_t st = as_stream(stream);
+    const bool dyn = scale_out != nullptr, res = residual != nullptr, f16 = dtype == LQ_F16;
+#define LQ_LN_GO(Tag)                                                                                   \
+    (dyn ? (res ? launch_ln<Tag, 1, true, false>(a, st) : launch_ln<Tag, 1, false, false>(a, st))       \
+         : (res ? launch_ln<Tag, 0, true, false>(a, st) : launch_ln<Tag, 0, false, false>(a, st)))
+    return f16 ? LQ_LN_GO(F16Tag) : LQ_LN_GO(BF16Tag);
+#undef LQ_LN_GO
+}
+
+extern "C" int lq_layernorm_mod_fp8(uint8_t* dst, const void* src, const void* scale, const void* shift, lq_dtype_t dtype,
+                                    const float* input_scale, size_t batch, size_t rows_per_batch, size_t dim, float eps,
+                                    lq_stream_t stream) {
+    int rc = check_ln_common("lq_layernorm_mod_fp8", dst, src, dtype, batch * rows_per_batch, dim);
+    if (rc != LQ_OK) return rc;
+    LQ_REQUIRE(scale && shift && input_scale, LQ_ERR_ARG, "lq_layernorm_mod_fp8: scale, shift and input_scale are required");
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(scale) % 16 == 0 && reinterpret_cast<uintptr_t>(shift) % 16 == 0, LQ_ERR_ARG,
+               "lq_layernorm_mod_fp8: scale and shift must be 16-byte aligned");
+    if (batch * rows_per_batch == 0) return LQ_OK;
+    LnArgs a = {dst, nullptr, nullptr, src, nullptr, nullptr, scale, shift, nullptr, input_scale, batch * rows_per_batch,
+                (int)dim, rows_per_batch, eps};
+    hipStream_t st = as_stream(stream);
+    return dtype == LQ_F16 ? launch_ln<F16Tag, 2, false, true>(a, st) : launch_ln<BF16Tag, 2, false, true>(a, st);
+}

@@ -133,6 +133,46 @@ def geglu_int8_dynamic(hidden, bias=None, pre_quant_scale=None):
     return q, s
 
 
+def layernorm_int8(x, gamma, beta, pre_quant_scale=None, input_quant_scale=None, residual=None, bias=None, eps: float = 1e-6):
+    """invokeLayerNormInt8O / invokeFusedResidualBiasLayerNormInt8O: LayerNorm over the last dim fused with the
+    INT8 quantisation.  input_quant_scale given: static scale, returns (q, None, h); None: dynamic per-token
+    scale, returns (q, scale[rows], h).  h = x + residual (+ bias) in x's dtype, or None without a residual."""
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    _chk(gamma, "gamma", (x.dtype,))
+    _chk(beta, "beta", (x.dtype,))
+    for name, t in (("residual", residual), ("bias", bias)):
+        if t is not None:
+            _chk(t, name, (x.dtype,))
+    if pre_quant_scale is not None:
+        _chk(pre_quant_scale, "pre_quant_scale", (torch.float32,))
+    if input_quant_scale is not None:
+        _chk(input_quant_scale, "input_quant_scale", (torch.float32,))
+    dim = x.shape[-1]
+    rows = x.numel() // dim if dim else 0
+    q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    s = torch.empty(rows, dtype=torch.float32, device=x.device) if input_quant_scale is None else None
+    h = torch.empty_like(x) if residual is not None else None
+    _l.check(_l.load().lq_layernorm_int8(_ptr(q), _ptr(s), _ptr(h), _ptr(x), _ptr(residual), _ptr(bias), _ptr(gamma), _ptr(beta),
+                                         _DT[x.dtype], _ptr(pre_quant_scale), _ptr(input_quant_scale), rows, dim, float(eps),
+                                         _stream()), "lq_layernorm_int8")
+    return q, s, h
+
+
+def layernorm_mod_fp8(x, scale, shift, input_scale, eps: float = 1e-6):
+    """invokeLayerNormWithShiftAndScale + FP8 cast: x [B, S, D], scale/shift [B, D], static input_scale [1];
+    returns e4m3 codes (uint8) of shape x."""
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    _chk(scale, "scale", (x.dtype,))
+    _chk(shift, "shift", (x.dtype,))
+    _chk(input_scale, "input_scale", (torch.float32,))
+    if x.dim() != 3 or tuple(scale.shape) != (x.shape[0], x.shape[2]) or scale.shape != shift.shape:
+        raise ValueError("x must be [B,S,D] and scale, shift [B,D]")
+    q = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    _l.check(_l.load().lq_layernorm_mod_fp8(_ptr(q), _ptr(x), _ptr(scale), _ptr(shift), _DT[x.dtype], _ptr(input_scale),
+                                            x.shape[0], x.shape[1], x.shape[2], float(eps), _stream()), "lq_layernorm_mod_fp8")
+    return q
+
+
 # ---- FP8 -------------------------------------------------------------------------------------------
 
 def fp8_amax_scale(x, scale=None):

@@ -441,6 +441,50 @@ def w4a4_gemm_f64(qa, qb, sA, sB, bias=None, group: int = 64, out_dtype: str = "
     return round_to(y.astype(F32), out_dtype)
 
 
+# ----------------------------------------------------------------------------------------
+# LayerNorm fused with quantisation (kernels/quant_kernels/layer_norm_int8.cu:102-556,
+# kernels/norms/layer_norm.cu:406-475 + utils/memory_utils.cu:431-439).  The reference's
+# statistics are Welford updates whose order follows its thread layout (in T for the INT8
+# kernels); this restatement takes mean and variance from fp64 sums narrowed to fp32, so
+# a HIP kernel with its own fp32 summation order agrees to within one quantisation step.
+# ----------------------------------------------------------------------------------------
+
+
+def _ln_normalised(h32, eps):
+    dim = h32.shape[1]
+    mean = (h32.astype(np.float64).sum(axis=1) / dim).astype(F32)
+    d = (h32 - mean[:, None]).astype(F32)
+    var = ((d.astype(np.float64) ** 2).sum(axis=1) / dim).astype(F32)
+    rstd = (F32(1.0) / np.sqrt((var + F32(eps)).astype(F32))).astype(F32)
+    return (d * rstd[:, None]).astype(F32)
+
+
+def layernorm_int8(src, residual, bias, gamma, beta, pre, in_scale, dtype: str, eps: float = 1e-6):
+    """h = src [+ residual [+ bias]] in T; y = T(gamma*n + beta); q = sat_s8(rne(f32(y)*pre/s)); s static
+    (in_scale) or, when in_scale is None, dynamic per token.  Returns (q, s or None, h)."""
+    h = np.asarray(src, dtype=F32)
+    if residual is not None:
+        h = round_to(h + np.asarray(residual, dtype=F32), dtype)
+        if bias is not None:
+            h = round_to(h + np.asarray(bias, dtype=F32)[None, :], dtype)
+    n = _ln_normalised(h, eps)
+    y = round_to((np.asarray(gamma, dtype=F32)[None, :] * n).astype(F32) + np.asarray(beta, dtype=F32)[None, :], dtype)
+    if in_scale is None:
+        q, s = sq_dynamic_quant(y, pre)
+        return q, s, h
+    return sq_input_quant(y, pre, np.asarray(in_scale, dtype=F32).reshape(-1), per_token=False), None, h
+
+
+def layernorm_mod_fp8(src, scale, shift, in_scale, rows_per_batch: int, dtype: str, eps: float = 1e-6):
+    """y = T(T(T(scale+1) * T(n)) + shift), q = e4m3(f32(y) * (1/s)); scale/shift are [B, dim]."""
+    x = np.asarray(src, dtype=F32)
+    n = round_to(_ln_normalised(x, eps), dtype)
+    b = np.arange(x.shape[0]) // rows_per_batch
+    a = round_to(np.asarray(scale, dtype=F32)[b] + F32(1.0), dtype)
+    y = round_to(round_to(a * n, dtype) + np.asarray(shift, dtype=F32)[b], dtype)
+    return fp8_scale_cast(y, np.asarray(in_scale, dtype=F32).reshape(-1)[0], True)
+
+
 def lora_down_f64(x, down) -> np.ndarray:
     """Low-rank down projection out[m,r] = sum_k x[m,k]*down[r,k] in fp64 (w4a4_gemm.cu:931-953 accumulates the
     k-tiles with float atomics, so the reference's own summation order is not defined): tolerance reference."""
