@@ -3,7 +3,7 @@
 // that the reference computes inside its quantisation kernel with float atomics
 // (kernels/w4a4_gemm/w4a4_gemm.cu:769-953 of lyraDiff, `reduce_add` into a zeroed fp32 buffer, followed by a
 // separate float -> T conversion, layers/w4a4_gemm_block/W4A4Gemm.cc:138-150).  Here it is a skinny GEMM of its
-// own: a workgroup owns 32 rows and all of K, its four wavefronts take interleaved 64-wide slices of K, the
+// own: a workgroup owns 32 rows and all of K, its eight wavefronts take interleaved 64-wide slices of K, the
 // partial 32 x rank blocks meet in LDS and are added in wavefront order -- no atomics, so the result does not
 // depend on scheduling -- and the output is written once, already in the requested type.  It reads x from HBM
 // only if the quantisation kernel that ran just before did not leave it in the caches.
@@ -22,9 +22,10 @@ template <bool F16> __device__ __forceinline__ v16f_t mfma16(const v4i& a, const
 
 // NR: rank / 32.  OUT: 0 fp32, 1 fp16, 2 bf16.
 template <bool F16, int NR, int OUT>
-__global__ __launch_bounds__(256) void lora_down_kernel(void* __restrict__ out, const unsigned short* __restrict__ x,
+__global__ __launch_bounds__(512) void lora_down_kernel(void* __restrict__ out, const unsigned short* __restrict__ x,
                                                         const unsigned short* __restrict__ down, int m, int k) {
-    __shared__ float part[3][NR][16][64];  // partial blocks of wavefronts 1..3
+    constexpr int W = 8;                    // wavefronts per workgroup, each takes every eighth 64-wide slice of K
+    __shared__ float part[W - 1][NR][16][64];  // partial blocks of wavefronts 1..7
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row0 = blockIdx.x * 32;
     const int lr = lane & 31, lh = lane >> 5;
@@ -35,19 +36,32 @@ __global__ __launch_bounds__(256) void lora_down_kernel(void* __restrict__ out, 
     for (int r = 0; r < NR; ++r)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[r][v] = 0.0f;
-    // a wavefront's slice: 64 consecutive k (four MFMA steps, one 128-byte line per row), every fourth slice
-    for (int k0 = wave * 64; k0 < k; k0 += 256) {
-        v4i xf[4], df[NR][4];
+    // a wavefront's slice: 64 consecutive k (four MFMA steps, one 128-byte line per row), every eighth slice.
+    // The operands of the next slice are requested before the matrix instructions of the current one, so the
+    // memory latency of a slice is hidden behind the previous slice's arithmetic and the other wavefronts.
+    v4i xf[2][4], df[2][NR][4];
+    auto load_slice = [&](int k0, int buf) {
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            xf[s] = *reinterpret_cast<const v4i*>(xrow + k0 + s * 16);
+            xf[buf][s] = *reinterpret_cast<const v4i*>(xrow + k0 + s * 16);
 #pragma unroll
-            for (int r = 0; r < NR; ++r) df[r][s] = *reinterpret_cast<const v4i*>(drow + (size_t)r * 32 * k + k0 + s * 16);
+            for (int r = 0; r < NR; ++r) df[buf][r][s] = *reinterpret_cast<const v4i*>(drow + (size_t)r * 32 * k + k0 + s * 16);
         }
+    };
+    auto compute_slice = [&](int buf) {
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
-            for (int r = 0; r < NR; ++r) acc[r] = mfma16<F16>(df[r][s], xf[s], acc[r]);
+            for (int r = 0; r < NR; ++r) acc[r] = mfma16<F16>(df[buf][r][s], xf[buf][s], acc[r]);
+    };
+    int k0 = wave * 64;
+    if (k0 < k) load_slice(k0, 0);
+    for (; k0 < k; k0 += 2 * 64 * W) {
+        if (k0 + 64 * W < k) load_slice(k0 + 64 * W, 1);
+        compute_slice(0);
+        if (k0 + 64 * W >= k) break;
+        if (k0 + 2 * 64 * W < k) load_slice(k0 + 2 * 64 * W, 0);
+        compute_slice(1);
     }
     if (wave != 0) {
 #pragma unroll
@@ -61,7 +75,9 @@ __global__ __launch_bounds__(256) void lora_down_kernel(void* __restrict__ out, 
 #pragma unroll
     for (int r = 0; r < NR; ++r) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[r][v] = ((acc[r][v] + part[0][r][v][lane]) + part[1][r][v][lane]) + part[2][r][v][lane];
+        for (int v = 0; v < 16; ++v)
+#pragma unroll
+            for (int w = 0; w < W - 1; ++w) acc[r][v] += part[w][r][v][lane];  // wavefront order: 0, 1, ..., 7
         if (row < m) {
             // result layout of the 32x32 MFMA: this lane holds row (= x row) lr and rank indices 8*(v/4) + 4*lh + v%4
 #pragma unroll
@@ -82,7 +98,7 @@ __global__ __launch_bounds__(256) void lora_down_kernel(void* __restrict__ out, 
 }
 
 template <bool F16, int NR> static int launch_lora_down(void* out, lq_dtype_t out_dtype, const void* x, const void* down, int m, int k, hipStream_t st) {
-    dim3 grid((unsigned)((m + 31) / 32)), block(256);
+    dim3 grid((unsigned)((m + 31) / 32)), block(512);
     const unsigned short* xs = static_cast<const unsigned short*>(x);
     const unsigned short* ds = static_cast<const unsigned short*>(down);
     switch (out_dtype) {

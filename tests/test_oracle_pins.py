@@ -287,3 +287,70 @@ def test_property_e4m3_monotone_and_idempotent(seed):
     v = O.e4m3_decode(O.e4m3_encode(x))
     assert (np.diff(v) >= 0).all()  # rounding is monotone
     assert np.array_equal(O.e4m3_decode(O.e4m3_encode(v)), v)  # representable values are fixed points
+
+
+# ---- LayerNorm + quant fusions, low-rank branch -------------------------------------------------------
+def test_layernorm_oracle_against_torch_and_closed_forms():
+    import torch
+
+    rng = np.random.default_rng(21)
+    x = (rng.standard_normal((9, 320)) * 3 + 1.5).astype(np.float32)
+    n = O._ln_normalised(x, 1e-5)
+    ref = torch.nn.functional.layer_norm(torch.from_numpy(x).double(), (320,), eps=1e-5).numpy()
+    assert np.abs(n - ref).max() < 2e-6
+    # shift invariance and scale invariance (eps -> 0) of the normalised value; unit variance, zero mean
+    assert np.abs(O._ln_normalised(x + 7.0, 1e-5) - n).max() < 2e-5
+    assert np.abs(O._ln_normalised(x * 4.0, 0.0) - O._ln_normalised(x, 0.0)).max() < 2e-6
+    assert np.abs(n.mean(axis=1)).max() < 1e-6 and np.abs(n.var(axis=1) - 1).max() < 1e-4
+    # a constant row normalises to 0, so y = beta and q = rne(beta*pre/s) regardless of gamma
+    gamma, beta = rng.standard_normal(320).astype(np.float32), np.full(320, 0.5, np.float32)
+    q, s, h = O.layernorm_int8(np.full((2, 320), 3.25, np.float32), None, None, gamma, beta, None, [0.25], "f16")
+    assert (q == 2).all() and s is None and np.array_equal(h, np.full((2, 320), 3.25, np.float32))
+    # composition: LayerNorm (torch, fp64) -> round to T -> the already pinned SmoothQuant quantiser
+    xh = O.round_to(x, "f16")
+    g16, b16 = O.round_to(gamma, "f16"), O.round_to(beta, "f16")
+    pre = (0.5 + rng.random(320)).astype(np.float32)
+    y = torch.nn.functional.layer_norm(torch.from_numpy(xh).double(), (320,), torch.from_numpy(g16).double(),
+                                       torch.from_numpy(b16).double(), eps=1e-6).numpy()
+    q_ref = O.sq_input_quant(O.round_to(y.astype(np.float32), "f16"), pre, np.float32([0.02]), False)
+    q, _, _ = O.layernorm_int8(xh, None, None, g16, b16, pre, [0.02], "f16")
+    d = np.abs(q.astype(int) - q_ref.astype(int))
+    assert d.max() <= 1 and (d != 0).mean() < 0.01  # one extra fp32 rounding inside gamma*n + beta
+    # residual + bias are added left to right in T; dynamic scale maps the row maximum to +-127
+    r = O.round_to(rng.standard_normal((9, 320)).astype(np.float32), "f16")
+    q, s, h = O.layernorm_int8(xh, r, b16, g16, b16, None, None, "f16")
+    assert np.array_equal(h, O.round_to(O.round_to(xh + r, "f16") + b16[None, :], "f16"))
+    assert (np.abs(q).max(axis=1) == 127).all() and s.shape == (9,)
+
+
+def test_layernorm_mod_fp8_oracle():
+    import torch
+
+    rng = np.random.default_rng(22)
+    x = O.round_to((rng.standard_normal((6, 256)) * 2).astype(np.float32), "bf16")
+    scale = O.round_to((rng.standard_normal((2, 256)) * 0.3).astype(np.float32), "bf16")
+    shift = O.round_to((rng.standard_normal((2, 256)) * 0.3).astype(np.float32), "bf16")
+    q = O.layernorm_mod_fp8(x, scale, shift, [0.02], 3, "bf16")
+    # fp64 evaluation of (1+scale)*LN(x)+shift with the batch index row // rows_per_batch, then the pinned e4m3 cast
+    n = torch.nn.functional.layer_norm(torch.from_numpy(x).double(), (256,), eps=1e-6).numpy()
+    b = np.arange(6) // 3
+    y = (1.0 + scale[b].astype(np.float64)) * n + shift[b].astype(np.float64)
+    v, ref = O.e4m3_decode(q).astype(np.float64), y / 0.02
+    # three bf16 roundings (2^-8 each) and one e4m3 rounding (2^-4) around the exact value
+    assert np.all(np.abs(v - np.clip(ref, -448, 448)) <= 2.0 ** -4 * np.abs(ref) + 3 * 2.0 ** -8 * (np.abs(n) * 1.9 + 1.0) / 0.02 + 2.0 ** -9)
+    # swapping scale and shift, or using the wrong batch row, must be visible
+    assert not np.array_equal(q, O.layernorm_mod_fp8(x, shift, scale, [0.02], 3, "bf16"))
+    assert not np.array_equal(q, O.layernorm_mod_fp8(x, scale[::-1], shift[::-1], [0.02], 3, "bf16"))
+
+
+def test_low_rank_oracle():
+    rng = np.random.default_rng(23)
+    x, down = rng.standard_normal((5, 64)), rng.standard_normal((32, 64))
+    ld = O.lora_down_f64(x, down)
+    assert ld.shape == (5, 32)
+    assert all(abs(ld[i, r] - sum(x[i, k] * down[r, k] for k in range(64))) < 1e-12 for i in (0, 4) for r in (0, 17, 31))
+    y32 = rng.standard_normal((5, 8)).astype(np.float32)
+    act, up, bias = rng.standard_normal((5, 32)), rng.standard_normal((8, 32)), rng.standard_normal(8)
+    y = O.w4a4_gemm_lora_f64(y32, act, up, bias, "f32")
+    assert np.allclose(y, y32 + np.einsum("mr,nr->mn", act, up) + bias[None, :], rtol=1e-6, atol=1e-6)
+    assert np.array_equal(O.w4a4_gemm_lora_f64(y32, act * 0, up, None, "f32"), y32)
