@@ -266,3 +266,36 @@ def test_w4a4_gemm_with_low_rank_branch(ops, dev, sdt, m, n, k, rank, tactic, ta
     yh = ops.w4a4_linear(*args, None, torch.float32, 64, act.half().to(dev), up.half().to(dev))
     refh = y32.astype(np.float64) + to_np_f32(act.half()).astype(np.float64) @ to_np_f32(up.half()).astype(np.float64).T
     assert np.all(np.abs(yh.cpu().numpy() - refh) <= 2.0 ** -20 * mag + 1e-6 * np.abs(refh))
+
+
+# ---- random shapes ---------------------------------------------------------------------------------------------------
+def test_random_shapes_all_gemms(ops, dev):
+    """Forty random (M, N, K) with every alignment the API allows (M free, N % 32, K % 64 or % 128): the default tile
+    choice must be exact on all of them."""
+    rs = np.random.default_rng(2024)
+    for it in range(40):
+        m = int(rs.integers(1, 700))
+        n = 32 * int(rs.integers(1, 24))
+        k = 64 * int(rs.integers(1, 20))
+        g = rng_t(it)
+        a = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int8)
+        w = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8)
+        acc = ops.int8_linear(a.to(dev), ops.repack_weight(w.to(dev)), None, None, None, torch.int32)
+        assert np.array_equal(acc.cpu().numpy(), O.gemm_i8_acc(a.numpy(), w.numpy())), ("int8", m, n, k)
+        k4 = 128 * int(rs.integers(1, 8))
+        x = torch.randn(m, k4, generator=g).bfloat16()
+        wt = (torch.randn(n, k4, generator=g) * 0.05).bfloat16()
+        sdt = "f16" if it % 2 else "f32"
+        qa, sA = O.w4a4_quant(to_np_f32(x), None, 64, sdt)
+        qb, sB = O.w4a4_quant(to_np_f32(wt), None, 64, sdt)
+        y = ops.w4a4_linear(torch.from_numpy(qa.view(np.int32)).to(dev),
+                            ops.repack_weight(torch.from_numpy(qb.view(np.uint8).reshape(n, k4 // 2)).to(dev)),
+                            torch.from_numpy(sA).to(TORCH_DT[sdt]).to(dev), torch.from_numpy(sB).to(TORCH_DT[sdt]).to(dev), None, torch.float32)
+        assert np.array_equal(y.cpu().numpy(), OC.w4a4_gemm(qa, qb, sA, sB, None)), ("w4a4", m, n, k4, sdt)
+        qf, sf = O.fp8_amax_cast(to_np_f32(x))
+        qw, sw = O.fp8_amax_cast(to_np_f32(wt))
+        yf = ops.fp8_linear(torch.from_numpy(qf).to(dev), ops.repack_weight(torch.from_numpy(qw).to(dev)),
+                            torch.tensor([sf], dtype=torch.float32, device=dev), torch.tensor([sw], dtype=torch.float32, device=dev),
+                            None, False, None, 0.0, torch.float32)
+        assert_close_tol(yf.cpu().numpy(), O.fp8_gemm(qf, qw, sf, sw, None, False, None, 0.0, "f32"), f"fp8 {m}x{n}x{k4}",
+                         abs_floor=fp32_sum_floor(qf, qw, sf, sw))
