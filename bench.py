@@ -8,7 +8,8 @@ One "step" is one pass of the FLUX DiT MLP FP8 chain over one batch of synthetic
 
     x bf16 [4608,3072]  --fp8 amax+cast-->  e4m3
         --FP8 GEMM 3072->12288, bias + tanh-GELU fused, bf16 out-->  h [4608,12288]
-    h --fp8 amax+cast--> e4m3  --FP8 GEMM 12288->3072, bias, bf16 out-->  y [4608,3072]
+    h --fp8 cast with the dynamic scale max|h|/448 that the first GEMM's epilogue accumulated--> e4m3
+      --FP8 GEMM 12288->3072, bias, bf16 out-->  y [4608,3072]
 
 Inputs and (pre-quantised, rows32-repacked) weights are resident in HBM before the timed region.
 `value` is the GEMM work of the step (2*M*N*K summed over both GEMMs) divided by the wall time of
@@ -116,6 +117,7 @@ def main():
     # initialisation (outside the timed region; the winners are cached inside the library by shape)
     tactics = {f"{n}x{k}": ops.gemm_profile("fp8", M, n, k, dev)[0] for (n, k) in ((H, D), (D, H))}
 
+    s_h = [torch.zeros(1, dtype=torch.float32, device=dev) for _ in range(2)]
     ev = lambda: torch.cuda.Event(enable_timing=True)
     names = ["quant_x", "gemm_up", "quant_h", "gemm_down"]
     marks = []
@@ -128,10 +130,14 @@ def main():
         qx, sx = ops.fp8_quant(xi)
         if record:
             e[1].record()
-        h = ops.fp8_linear(qx, wp_up, sx, s_up, bu, True, None, 0.0, torch.bfloat16)
+        # the up projection's epilogue also accumulates max|h|/448, the dynamic scale of h, so the quantisation
+        # of h is a single cast pass (the same numbers as an amax pass over h followed by the cast)
+        sh = s_h[i % 2]
+        sh.zero_()
+        h = ops.fp8_linear(qx, wp_up, sx, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh)
         if record:
             e[2].record()
-        qh, sh = ops.fp8_quant(h)
+        qh = ops.fp8_scale_cast(h, sh)
         if record:
             e[3].record()
         y = ops.fp8_linear(qh, wp_dn, sh, s_dn, bd, False, None, 0.0, torch.bfloat16)
@@ -158,7 +164,7 @@ def main():
         "gemm_up_fp8_4608x12288x3072": {"us": round(per["gemm_up"], 2), "TFLOP/s": round(gemm_flops / per["gemm_up"] / 1e6, 1)},
         "gemm_down_fp8_4608x3072x12288": {"us": round(per["gemm_down"], 2), "TFLOP/s": round(gemm_flops / per["gemm_down"] / 1e6, 1)},
         "fp8_amax_cast_4608x3072": {"us": round(per["quant_x"], 2), "GB/s": round(3.0 * M * D / per["quant_x"] / 1e3, 1)},
-        "fp8_amax_cast_4608x12288": {"us": round(per["quant_h"], 2), "GB/s": round(3.0 * M * H / per["quant_h"] / 1e3, 1)},
+        "fp8_cast_with_gemm_scale_4608x12288": {"us": round(per["quant_h"], 2), "GB/s": round(3.0 * M * H / per["quant_h"] / 1e3, 1)},
     }
     achieved = gemm_flops / per["gemm_up"] / 1e6
     roofline = {"bound": "mfma", "kernel": "lq::gemm_kernel<fp8> 4608x12288x3072 (bias+GELU, bf16 out)",
@@ -186,7 +192,7 @@ def main():
         xr = xd[: args.cpu_rows].contiguous()
         qx, sx = ops.fp8_quant(xr)
         hg = ops.fp8_linear(qx, wp_up, sx, s_up, bu, True, None, 0.0, torch.bfloat16)
-        qh, sh = ops.fp8_quant(hg)
+        qh, sh = ops.fp8_quant(hg)  # the two-pass form; the timed chain's fused scale is checked equal in tests/
         y_gpu = ops.fp8_linear(qh, wp_dn, sh, s_dn, bd, False, None, 0.0, torch.bfloat16).float().cpu()
         out["cpu_gpu_max_abs_diff"] = round((y_gpu - y_cpu.float()).abs().max().item(), 4)
     if args.extra:

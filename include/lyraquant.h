@@ -182,6 +182,21 @@ int lq_gemm_w4a4(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const u
                  const void* sA, const void* sB, lq_dtype_t scale_dtype, const void* bias,
                  int m, int n, int k, int group, lq_stream_t stream);
 
+/* lq_gemm_fp8 with the output's re-quantisation for the next FP8 linear prepared in the epilogue (no counterpart as
+ * one call in the reference: its blocks run GemmWithResidualAndBias, then getFP8WeightScale-style amax or a calibrated
+ * static scale, then invokeCudaD2DScaleCpyConvert as separate kernels, e.g.
+ * layers/flux_single_transformer_block/FluxSingleTransformerFP8Block.cc:216-281):
+ *   out_scale (optional): out_scale[0] = max(out_scale[0], max|C| / 448) over the T-rounded outputs -- exactly what
+ *     lq_fp8_amax_scale(out_scale, C, ...) would add, without the pass over C; zero it before the call, then cast with
+ *     lq_fp8_scale_cast(dst, C, dtype, out_scale, 1, m*n, stream).
+ *   C_fp8 + C_fp8_scale (optional, static scale): C_fp8[m,n] = e4m3( f32(T(y)) * (1 / C_fp8_scale[0]) ), the codes
+ *     lq_fp8_scale_cast would produce from C; C may then be NULL and the 16-bit output is never written.
+ * Everything else as lq_gemm_fp8 (which is this call with the three extra pointers NULL). */
+int lq_gemm_fp8_ex(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32,
+                   const float* a_scale, const float* b_scale, const void* bias, int gelu,
+                   const void* residual, float beta, int m, int n, int k,
+                   float* out_scale, uint8_t* C_fp8, const float* C_fp8_scale, lq_stream_t stream);
+
 /* LayerNorm fused with the INT8 SmoothQuant quantisation that follows it: invokeLayerNormInt8O and, with a
  * residual, invokeFusedResidualBiasLayerNormInt8O (kernels/quant_kernels/layer_norm_int8.h:8-38):
  *   h = src [+ residual [+ bias]]   (T arithmetic; h is written to dst2 when a residual is given)

@@ -45,6 +45,9 @@ struct GemmParams {
     int gelu;
     const void* residual;
     float beta;
+    float* out_scale;       // optional: max(out_scale, max|C| / 448), the e4m3 scale of the output for a following cast
+    uint8_t* C8;            // optional: e4m3 codes of C with a given (static) scale, written next to or instead of C
+    const float* c8_scale;  // scale of C8: C8 = e4m3(f32(T(y)) * (1 / c8_scale[0]))
     // w4a4
     const void* sA;
     const void* sB;
@@ -126,6 +129,17 @@ __device__ __forceinline__ float gelu_fast(float x) {
     float e = __builtin_amdgcn_exp2f(inner * 2.8853900817779268f);  // exp(2*inner)
     float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);        // tanh(inner); e=inf -> 1
     return 0.5f * x * (1.0f + t);
+}
+
+// Four floats -> four e4m3 codes, round-to-nearest-even, saturating to +-448, NaN -> 0x7F | sign (the cast kernel's rule).
+__device__ __forceinline__ u32 e4m3x4(float a, float b, float c, float d) {
+    const float v[4] = {a, b, c, d};
+    u32 w = (u32)__builtin_amdgcn_cvt_pk_fp8_f32(__builtin_amdgcn_fmed3f(a, 448.0f, -448.0f), __builtin_amdgcn_fmed3f(b, 448.0f, -448.0f), 0, false);
+    w = (u32)__builtin_amdgcn_cvt_pk_fp8_f32(__builtin_amdgcn_fmed3f(c, 448.0f, -448.0f), __builtin_amdgcn_fmed3f(d, 448.0f, -448.0f), (int)w, true);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (v[i] != v[i]) w = (w & ~(0xFFu << (8 * i))) | ((0x7Fu | ((__float_as_uint(v[i]) >> 24) & 0x80u)) << (8 * i));
+    return w;
 }
 
 // One 16-byte-per-lane global -> LDS transfer without passing through registers: lane l of the
@@ -548,7 +562,11 @@ struct GemmKernel {
         const int out_row = lane / LPR, out_n = n0 + wn * TN + (lane % LPR) * 4;
         const bool n_ok = out_n < p.n;
         float alpha = 1.0f, bias4[4] = {0.f, 0.f, 0.f, 0.f}, acol4[4] = {0.f, 0.f, 0.f, 0.f}, arow_l[MT];
-        if constexpr (KIND == K_FP8) alpha = p.a_scale[0] * p.b_scale[0];
+        float out_amax = 0.0f, c8_inv = 0.0f;
+        if constexpr (KIND == K_FP8) {
+            alpha = p.a_scale[0] * p.b_scale[0];
+            if (p.C8 != nullptr) c8_inv = 1.0f / p.c8_scale[0];
+        }
         if constexpr (!kI32) {
             if (p.bias != nullptr && n_ok) OutStore<OutTag>::load4(p.bias, out_n, bias4);
             if constexpr (KIND == K_INT8) {
@@ -624,7 +642,31 @@ struct GemmKernel {
                             }
                         }
                     }
-                    if (ok) OutStore<OutTag>::store4(p.C, idx, y);
+                    if constexpr (KIND == K_FP8) {
+                        if (ok) {
+                            if (p.out_scale != nullptr)
+                                out_amax = fmaxf(fmaxf(out_amax, fmaxf(fabsf(y[0]), fabsf(y[1]))), fmaxf(fabsf(y[2]), fabsf(y[3])));
+                            if (p.C8 != nullptr) {  // the codes the separate cast kernel would produce from the T-rounded output
+                                float t[4];
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) t[e] = round_through<OutTag>(y[e]) * c8_inv;
+                                *reinterpret_cast<u32*>(p.C8 + idx) = e4m3x4(t[0], t[1], t[2], t[3]);
+                            }
+                        }
+                    }
+                    if (ok && p.C != nullptr) OutStore<OutTag>::store4(p.C, idx, y);
+                }
+            }
+        }
+        if constexpr (KIND == K_FP8 && !kI32) {
+            // Rounding to T is monotone, so the maximum of the rounded outputs is the rounded maximum; so is the
+            // division by 448: the scale published here is exactly what an amax pass over C would produce.
+            if (p.out_scale != nullptr) {
+                out_amax = round_through<OutTag>(wave_max(out_amax));
+                if (lane == 0) {
+                    const float sc = out_amax / 448.0f;
+                    int cur = __hip_atomic_load(reinterpret_cast<int*>(p.out_scale), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (__float_as_int(sc) > cur) atomicMax(reinterpret_cast<int*>(p.out_scale), __float_as_int(sc));
                 }
             }
         }

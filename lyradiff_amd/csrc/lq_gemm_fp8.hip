@@ -33,20 +33,23 @@ template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
 
 using namespace lq;
 
-extern "C" int lq_gemm_fp8(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32,
-                           const float* a_scale, const float* b_scale, const void* bias, int gelu,
-                           const void* residual, float beta, int m, int n, int k, lq_stream_t stream) {
-    LQ_REQUIRE(C && A && B_rows32 && a_scale && b_scale, LQ_ERR_ARG, "lq_gemm_fp8: null pointer");
+extern "C" int lq_gemm_fp8_ex(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32,
+                              const float* a_scale, const float* b_scale, const void* bias, int gelu,
+                              const void* residual, float beta, int m, int n, int k, float* out_scale, uint8_t* C_fp8,
+                              const float* C_fp8_scale, lq_stream_t stream) {
+    LQ_REQUIRE((C || C_fp8) && A && B_rows32 && a_scale && b_scale, LQ_ERR_ARG, "lq_gemm_fp8: null pointer");
+    LQ_REQUIRE((C_fp8 == nullptr) == (C_fp8_scale == nullptr), LQ_ERR_ARG, "lq_gemm_fp8: C_fp8 and C_fp8_scale go together");
     LQ_REQUIRE(m >= 0 && n > 0 && k > 0 && n % 32 == 0 && k % 64 == 0, LQ_ERR_SHAPE,
                "lq_gemm_fp8: need n %% 32 == 0 and k %% 64 == 0 (m=%d n=%d k=%d)", m, n, k);
     LQ_REQUIRE(reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B_rows32) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(C) % 16 == 0 && reinterpret_cast<uintptr_t>(bias) % 8 == 0 &&
-                   reinterpret_cast<uintptr_t>(residual) % 16 == 0,
-               LQ_ERR_ARG, "lq_gemm_fp8: A, B, C, residual must be 16-byte aligned and bias 8-byte aligned");
+                   reinterpret_cast<uintptr_t>(residual) % 16 == 0 && reinterpret_cast<uintptr_t>(C_fp8) % 4 == 0,
+               LQ_ERR_ARG, "lq_gemm_fp8: A, B, C, residual must be 16-byte aligned, bias 8-byte, C_fp8 4-byte aligned");
     if (m == 0) return LQ_OK;
     GemmParams p = {};
     p.C = C; p.A = A; p.B = B_rows32; p.bias = bias; p.a_scale = a_scale; p.b_scale = b_scale;
     p.gelu = gelu; p.residual = (beta != 0.0f) ? residual : nullptr; p.beta = beta;
+    p.out_scale = out_scale; p.C8 = C_fp8; p.c8_scale = C_fp8_scale;
     p.m = m; p.n = n; p.k = k; p.kb = k;
     hipStream_t st = as_stream(stream);
     switch (out_dtype) {
@@ -55,4 +58,12 @@ extern "C" int lq_gemm_fp8(void* C, lq_dtype_t out_dtype, const uint8_t* A, cons
         case LQ_F32: return run_fp8<F32Tag>(p, st);
         default: set_error("lq_gemm_fp8: unsupported output dtype %d", (int)out_dtype); return LQ_ERR_UNSUPPORTED;
     }
+}
+
+extern "C" int lq_gemm_fp8(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32,
+                           const float* a_scale, const float* b_scale, const void* bias, int gelu,
+                           const void* residual, float beta, int m, int n, int k, lq_stream_t stream) {
+    LQ_REQUIRE(C != nullptr, LQ_ERR_ARG, "lq_gemm_fp8: null pointer");
+    return lq_gemm_fp8_ex(C, out_dtype, A, B_rows32, a_scale, b_scale, bias, gelu, residual, beta, m, n, k, nullptr, nullptr,
+                          nullptr, stream);
 }

@@ -268,8 +268,11 @@ def int8_linear(a_q, w_rows32, alpha_col, alpha_row, bias=None, out_dtype=torch.
 
 
 def fp8_linear(a_q, w_rows32, a_scale, b_scale, bias=None, gelu: bool = False, residual=None, beta: float = 0.0,
-               out_dtype=torch.bfloat16):
-    """FP8 GemmWithResidualAndBias: a_q uint8 e4m3 [M,K], w_rows32 uint8 e4m3 [N,K] (rows32)."""
+               out_dtype=torch.bfloat16, out_scale=None, out_fp8_scale=None, want_output: bool = True):
+    """FP8 GemmWithResidualAndBias: a_q uint8 e4m3 [M,K], w_rows32 uint8 e4m3 [N,K] (rows32).
+    out_scale (fp32 [1], zeroed by the caller): also accumulates max|C|/448, the dynamic e4m3 scale of the output.
+    out_fp8_scale (fp32 [1], static): also returns the e4m3 codes of C with that scale -> (C, codes); with
+    want_output=False the 16-bit C is not written at all and only the codes are returned."""
     _chk(a_q, "a_q", (torch.uint8,))
     _chk(w_rows32, "w_rows32", (torch.uint8,))
     _chk(a_scale, "a_scale", (torch.float32,))
@@ -282,11 +285,19 @@ def fp8_linear(a_q, w_rows32, a_scale, b_scale, bias=None, gelu: bool = False, r
         _chk(bias, "bias", (out_dtype,))
     if residual is not None:
         _chk(residual, "residual", (out_dtype,))
-    c = torch.empty((m, n), dtype=out_dtype, device=a_q.device)
-    _l.check(_l.load().lq_gemm_fp8(_ptr(c), _DT[out_dtype], _ptr(a_q), _ptr(w_rows32), _ptr(a_scale), _ptr(b_scale),
-                                   _ptr(bias), int(gelu), _ptr(residual), float(beta), m, n, k, _stream()),
-             "lq_gemm_fp8")
-    return c
+    for name, t in (("out_scale", out_scale), ("out_fp8_scale", out_fp8_scale)):
+        if t is not None:
+            _chk(t, name, (torch.float32,))
+    if not want_output and out_fp8_scale is None:
+        raise ValueError("want_output=False needs out_fp8_scale")
+    c = torch.empty((m, n), dtype=out_dtype, device=a_q.device) if want_output else None
+    c8 = torch.empty((m, n), dtype=torch.uint8, device=a_q.device) if out_fp8_scale is not None else None
+    _l.check(_l.load().lq_gemm_fp8_ex(_ptr(c), _DT[out_dtype], _ptr(a_q), _ptr(w_rows32), _ptr(a_scale), _ptr(b_scale),
+                                      _ptr(bias), int(gelu), _ptr(residual), float(beta), m, n, k, _ptr(out_scale), _ptr(c8),
+                                      _ptr(out_fp8_scale), _stream()), "lq_gemm_fp8")
+    if out_fp8_scale is None:
+        return c
+    return (c, c8) if want_output else c8
 
 
 def w4a4_linear(a_words, w_rows32, sA, sB, bias=None, out_dtype=torch.bfloat16, group: int = 64, lora_act=None, lora_up=None):

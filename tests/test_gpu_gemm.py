@@ -299,3 +299,36 @@ def test_random_shapes_all_gemms(ops, dev):
                             None, False, None, 0.0, torch.float32)
         assert_close_tol(yf.cpu().numpy(), O.fp8_gemm(qf, qw, sf, sw, None, False, None, 0.0, "f32"), f"fp8 {m}x{n}x{k4}",
                          abs_floor=fp32_sum_floor(qf, qw, sf, sw))
+
+
+# ---- FP8 GEMM epilogue outputs for the next FP8 linear -----------------------------------------------------------------
+@pytest.mark.parametrize("m,n,k,gelu", [(333, 416, 704, True), (1024, 3072, 3072, False), (4608, 12288, 3072, True)])
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+def test_fp8_gemm_epilogue_scale_and_codes(ops, dev, m, n, k, gelu, dt):
+    """The scale the epilogue accumulates and the codes it writes are exactly those of the separate amax / cast kernels
+    applied to the GEMM's own 16-bit output (those kernels are checked against the oracle in test_gpu_quant.py)."""
+    g = rng_t(m + n + k)
+    t = TORCH_DT[dt]
+    qa, sa = ops.fp8_quant(torch.randn(m, k, generator=g).to(t).to(dev))
+    qw, sw = ops.fp8_quant((torch.randn(n, k, generator=g) * 0.02).to(t).to(dev))
+    wp = ops.repack_weight(qw)
+    bias = (torch.randn(n, generator=g) * 0.1).to(t).to(dev)
+    plain = ops.fp8_linear(qa, wp, sa, sw, bias, gelu, None, 0.0, t)
+    # dynamic: scale of the output
+    s_out = torch.zeros(1, dtype=torch.float32, device=dev)
+    c = ops.fp8_linear(qa, wp, sa, sw, bias, gelu, None, 0.0, t, out_scale=s_out)
+    assert torch.equal(c, plain)
+    q_ref, s_ref = ops.fp8_quant(plain)
+    assert torch.equal(s_out, s_ref), (s_out.item(), s_ref.item())
+    assert torch.equal(ops.fp8_scale_cast(c, s_out), q_ref)
+    # accumulation semantics: a larger value already in the slot wins
+    big = torch.full((1,), 1e6, dtype=torch.float32, device=dev)
+    ops.fp8_linear(qa, wp, sa, sw, bias, gelu, None, 0.0, t, out_scale=big)
+    assert big.item() == 1e6
+    # static: codes with a given scale, with and without the 16-bit output
+    s_static = torch.tensor([0.037], dtype=torch.float32, device=dev)
+    c2, codes = ops.fp8_linear(qa, wp, sa, sw, bias, gelu, None, 0.0, t, out_fp8_scale=s_static)
+    assert torch.equal(c2, plain)
+    assert torch.equal(codes, ops.fp8_scale_cast(plain, s_static))
+    only = ops.fp8_linear(qa, wp, sa, sw, bias, gelu, None, 0.0, t, out_fp8_scale=s_static, want_output=False)
+    assert torch.equal(only, codes)
