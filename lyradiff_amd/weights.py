@@ -1,0 +1,160 @@
+"""Loaders for the reference's on-disk / in-memory weight formats of the three quantized linears, and the
+linear modules that run them.
+
+The reference keeps each tensor of a linear either as a raw little-endian `.bin` file (`loadWeightFromBin`,
+src/lyradiff/utils/memory_utils.cu:251-314: no header, the element type is implied by the caller) or as an entry of
+a `{name: pointer}` cache filled from a state dict (`loadWeightsFromCache`).  The names:
+
+  INT8 SmoothQuant  prefix + name + {".weight_int8", ".weight_quant_scale", ".input_quant_scale",
+                    ".pre_quant_scale"}                       MACROLoadLinearInt8WeightFromBin,
+                                                              src/lyradiff/utils/common_macro_def.h:51-59
+  FP8               prefix + name + {".weight", ".bias", "_input_scale"}; the 16-bit weight is quantised to e4m3
+                    with a per-tensor scale WHEN IT IS LOADED   MACROLoadFP8WeightFromBin / ...FromCache,
+                                                              common_macro_def.h:66-92
+  W4A4              prefix + {"packed_weight", "weight_scale", "lora_up", "lora_down", "smooth", "bias"}
+                                                              src/lyradiff/layers/w4a4_gemm_block/W4A4GemmWeight.cc:65-83
+
+Every loader ends with the one-time repack of the weight into the rows32 layout the GEMMs read.  The modules hold
+device tensors only and call lyradiff_amd.ops (the C ABI); there is no CPU path.
+"""
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass
+from typing import Callable, Mapping, Optional
+
+import numpy as np
+import torch
+
+from . import ops
+
+_NP = {torch.float32: np.float32, torch.float16: np.float16, torch.int8: np.int8, torch.uint8: np.uint8}
+
+
+def read_bin(path: str, shape, dtype: torch.dtype) -> torch.Tensor:
+    """One raw `.bin` tensor (host).  bf16 files are read as 16-bit words and reinterpreted."""
+    count = int(np.prod(shape))
+    if dtype == torch.bfloat16:
+        raw = np.fromfile(path, dtype=np.uint16)
+    else:
+        raw = np.fromfile(path, dtype=_NP[dtype])
+    if raw.size != count:
+        raise ValueError(f"{path}: holds {raw.size} elements, expected {count} for shape {tuple(shape)}")
+    t = torch.from_numpy(raw.reshape(shape))
+    return t.view(torch.bfloat16) if dtype == torch.bfloat16 else t
+
+
+def _source(src) -> Callable[[str, tuple, torch.dtype], torch.Tensor]:
+    """`src` is a directory of .bin files or a mapping name -> tensor (a state dict)."""
+    if isinstance(src, Mapping):
+        def get(name, shape, dtype):
+            if name not in src:
+                raise KeyError(f"Cannot find a tensor of name {name}")
+            t = src[name]
+            if tuple(t.shape) != tuple(shape) and t.numel() == int(np.prod(shape)):
+                t = t.reshape(shape)
+            if tuple(t.shape) != tuple(shape) or t.dtype != dtype:
+                raise ValueError(f"{name}: got {tuple(t.shape)} {t.dtype}, expected {tuple(shape)} {dtype}")
+            return t
+        return get
+    return lambda name, shape, dtype: read_bin(os.path.join(src, name + ".bin"), shape, dtype)
+
+
+@dataclass
+class Int8Linear:
+    """SmoothQuant W8A8 linear with the reference's calibrated static activation scale
+    (BasicTransformerInt8Block.cc:427-452: invokeSqInputQuant -> runGemmInt8 -> bias)."""
+    weight_rows32: torch.Tensor      # int8 [N, K], rows32
+    weight_scale: torch.Tensor       # fp32 [N]
+    input_quant_scale: torch.Tensor  # fp32 [1]
+    pre_quant_scale: torch.Tensor    # fp32 [K]
+    bias: Optional[torch.Tensor] = None
+
+    def forward(self, x: torch.Tensor, dynamic: bool = False) -> torch.Tensor:
+        k = x.shape[-1]
+        x2 = x.reshape(-1, k)
+        if dynamic:  # per-token scales computed on the fly instead of the calibrated one
+            q, s = ops.sq_quant_dynamic(x2, self.pre_quant_scale)
+        else:
+            q, s = ops.sq_quant(x2, self.pre_quant_scale, self.input_quant_scale), self.input_quant_scale
+        y = ops.int8_linear(q, self.weight_rows32, self.weight_scale, s, self.bias, x.dtype)
+        return y.reshape(*x.shape[:-1], y.shape[-1])
+
+
+@dataclass
+class FP8Linear:
+    """FP8 e4m3 per-tensor linear (FluxAttnPostFP8Processor.cc:135-163: scale-cast with `_input_scale`, then
+    GemmWithResidualAndBias)."""
+    weight_rows32: torch.Tensor  # uint8 e4m3 [N, K], rows32
+    weight_scale: torch.Tensor   # fp32 [1]
+    input_scale: torch.Tensor    # fp32 [1]
+    bias: Optional[torch.Tensor] = None
+
+    def forward(self, x: torch.Tensor, gelu: bool = False, residual=None, beta: float = 0.0, dynamic: bool = False) -> torch.Tensor:
+        k = x.shape[-1]
+        x2 = x.reshape(-1, k)
+        if dynamic:
+            q, s = ops.fp8_quant(x2)
+        else:
+            q, s = ops.fp8_scale_cast(x2, self.input_scale), self.input_scale
+        y = ops.fp8_linear(q, self.weight_rows32, s, self.weight_scale, self.bias, gelu, residual, beta, x.dtype)
+        return y.reshape(*x.shape[:-1], y.shape[-1])
+
+
+@dataclass
+class W4A4Linear:
+    """W4A4 group-64 linear with the SVDQuant low-rank branch (W4A4Gemm.cc:113-169)."""
+    weight_rows32: torch.Tensor  # uint8 [N, K/2], rows32
+    weight_scale: torch.Tensor   # fp32 [N, K/64]
+    smooth: torch.Tensor         # fp32 [K]
+    lora_up: Optional[torch.Tensor] = None    # T [N, R]
+    lora_down: Optional[torch.Tensor] = None  # T [R, K]
+    bias: Optional[torch.Tensor] = None
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        k = x.shape[-1]
+        x2 = x.reshape(-1, k)
+        q, s = ops.w4a4_quant(x2, self.smooth, torch.float32)
+        act = ops.lora_down(x2, self.lora_down) if self.lora_down is not None else None
+        y = ops.w4a4_linear(q, self.weight_rows32, s, self.weight_scale, self.bias, x.dtype, 64, act,
+                            self.lora_up if act is not None else None)
+        return y.reshape(*x.shape[:-1], y.shape[-1])
+
+
+def load_int8_linear(src, prefix: str, name: str, d_out: int, d_in: int, device="cuda", bias_dtype=None) -> Int8Linear:
+    get = _source(src)
+    w = get(prefix + name + ".weight_int8", (d_out, d_in), torch.int8).to(device)
+    bias = None
+    if bias_dtype is not None:
+        bias = get(prefix + name + ".bias", (d_out,), bias_dtype).to(device)
+    return Int8Linear(ops.repack_weight(w),
+                      get(prefix + name + ".weight_quant_scale", (d_out,), torch.float32).to(device),
+                      get(prefix + name + ".input_quant_scale", (1,), torch.float32).to(device),
+                      get(prefix + name + ".pre_quant_scale", (d_in,), torch.float32).to(device), bias)
+
+
+def load_fp8_linear(src, prefix: str, name: str, d_out: int, d_in: int, dtype=torch.bfloat16, device="cuda") -> FP8Linear:
+    """The 16-bit weight is quantised on the device as the reference does at load time: scale = max|w|/448
+    (invokeGetFP8WeightScale), codes = e4m3(w * (1/scale)) (invokeCudaD2DScaleCpyConvert)."""
+    get = _source(src)
+    w = get(prefix + name + ".weight", (d_out, d_in), dtype).to(device)
+    scale = ops.fp8_amax_scale(w)
+    codes = ops.fp8_scale_cast(w, scale)
+    return FP8Linear(ops.repack_weight(codes), scale,
+                     get(prefix + name + "_input_scale", (1,), torch.float32).to(device),
+                     get(prefix + name + ".bias", (d_out,), dtype).to(device))
+
+
+def load_w4a4_linear(src, prefix: str, d_out: int, d_in: int, lora_rank: int = 32, has_bias: bool = False,
+                     dtype=torch.bfloat16, device="cuda") -> W4A4Linear:
+    get = _source(src)
+    packed = get(prefix + "packed_weight", (d_out, d_in // 2), torch.int8).to(device)
+    lin = W4A4Linear(ops.repack_weight(packed.view(torch.uint8)),
+                     get(prefix + "weight_scale", (d_out, d_in // 64), torch.float32).to(device),
+                     get(prefix + "smooth", (d_in,), torch.float32).to(device))
+    if lora_rank:
+        lin.lora_up = get(prefix + "lora_up", (d_out, lora_rank), dtype).to(device)
+        lin.lora_down = get(prefix + "lora_down", (lora_rank, d_in), dtype).to(device)
+    if has_bias:
+        lin.bias = get(prefix + "bias", (d_out,), dtype).to(device)
+    return lin
