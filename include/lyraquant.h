@@ -197,6 +197,18 @@ int lq_gemm_fp8_ex(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_
                    const void* residual, float beta, int m, int n, int k,
                    float* out_scale, uint8_t* C_fp8, const float* C_fp8_scale, lq_stream_t stream);
 
+/* SmoothQuant smoothing vector, device side (calibration time).  The reference consumes a precomputed
+ * pre_quant_scale from nvidia-modelopt (lyradiff/convert_model_scripts/convert_sd_quant_model.py:199,340); these two
+ * calls produce it in the closed form its benchmark configuration states:
+ *   lq_col_absmax:    out[k] = max(out[k], max_m |x[m,k]|)   -- zero `out` once, then call per calibration batch / weight
+ *   lq_smooth_vector: s[k] = act_absmax[k]^alpha / weight_absmax[k]^(1-alpha);  pre_quant_scale[k] = 1/s[k];
+ *                     smooth_out (optional) receives s, the factor the weight columns are multiplied by offline
+ *                     (equivalently lq_int8_weight_quant divides by pre_quant_scale, quant_kernels.cu:197-199).
+ * x [rows, dim] F16/BF16/F32, dim % 8 == 0. */
+int lq_col_absmax(float* out, const void* x, lq_dtype_t dtype, size_t rows, size_t dim, lq_stream_t stream);
+int lq_smooth_vector(float* pre_quant_scale, float* smooth_out, const float* act_absmax, const float* weight_absmax,
+                     float alpha, size_t dim, lq_stream_t stream);
+
 /* LayerNorm fused with the INT8 SmoothQuant quantisation that follows it: invokeLayerNormInt8O and, with a
  * residual, invokeFusedResidualBiasLayerNormInt8O (kernels/quant_kernels/layer_norm_int8.h:8-38):
  *   h = src [+ residual [+ bias]]   (T arithmetic; h is written to dst2 when a residual is given)

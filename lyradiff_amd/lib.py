@@ -36,6 +36,8 @@ SYMBOLS = {
     "lq_gemm_fp8": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _P, _F, _I, _I, _I, _P]),
     "lq_gemm_fp8_ex": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _P, _F, _I, _I, _I, _P, _P, _P, _P]),
     "lq_gemm_w4a4": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P]),
+    "lq_col_absmax": (_I, [_P, _P, _I, _Z, _Z, _P]),
+    "lq_smooth_vector": (_I, [_P, _P, _P, _P, _F, _Z, _P]),
     "lq_layernorm_int8": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _Z, _Z, _F, _P]),
     "lq_layernorm_mod_fp8": (_I, [_P, _P, _P, _P, _I, _P, _Z, _Z, _Z, _F, _P]),
     "lq_gemm_w4a4_lora": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),

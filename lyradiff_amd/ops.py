@@ -40,6 +40,30 @@ _FLOATS = (torch.float32, torch.float16, torch.bfloat16)
 
 # ---- INT8 SmoothQuant ---------------------------------------------------------------------------
 
+def col_absmax(x, out=None):
+    """Per-column max |x| over all rows, accumulated into `out` (fp32 [K]; allocated and zeroed when None)."""
+    _chk(x, "x", _FLOATS)
+    k = x.shape[-1]
+    if out is None:
+        out = torch.zeros(k, dtype=torch.float32, device=x.device)
+    _chk(out, "out", (torch.float32,))
+    _l.check(_l.load().lq_col_absmax(_ptr(out), _ptr(x), _DT[x.dtype], x.numel() // k if k else 0, k, _stream()), "lq_col_absmax")
+    return out
+
+
+def smooth_vector(act_absmax, weight_absmax, alpha: float = 0.5):
+    """SmoothQuant s[k] = act^alpha / weight^(1-alpha); returns (pre_quant_scale = 1/s, s)."""
+    _chk(act_absmax, "act_absmax", (torch.float32,))
+    _chk(weight_absmax, "weight_absmax", (torch.float32,))
+    k = act_absmax.numel()
+    if weight_absmax.numel() != k:
+        raise ValueError("act_absmax and weight_absmax must have the same length")
+    pre, s = torch.empty_like(act_absmax), torch.empty_like(act_absmax)
+    _l.check(_l.load().lq_smooth_vector(_ptr(pre), _ptr(s), _ptr(act_absmax), _ptr(weight_absmax), float(alpha), k, _stream()),
+             "lq_smooth_vector")
+    return pre, s
+
+
 def sq_quant(x, pre_quant_scale, input_quant_scale, per_token: bool = False):
     """invokeSqInputQuant: x [..., K] -> int8 [..., K] with a static (or given per-token) scale."""
     _chk(x, "x", _FLOATS)

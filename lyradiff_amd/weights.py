@@ -158,3 +158,27 @@ def load_w4a4_linear(src, prefix: str, d_out: int, d_in: int, lora_rank: int = 3
     if has_bias:
         lin.bias = get(prefix + "bias", (d_out,), dtype).to(device)
     return lin
+
+
+# ---- int4 <-> int8 host helpers of the weight tooling (offline, CPU tensors, as in the reference) ------------------
+def pack_int8_tensor_to_packed_int4(weight: torch.Tensor) -> torch.Tensor:
+    """int8 values in [-8, 7] -> two per byte along the last dim, element 2j in the low nibble
+    (pack_int8_tensor_to_packed_int4, src/lyradiff/layers/gemm_utils/WeightOnlyQuantOps.cc:286-321)."""
+    if weight.is_cuda or weight.dtype != torch.int8 or not weight.is_contiguous() or weight.numel() == 0:
+        raise ValueError("weight must be a non-empty contiguous CPU int8 tensor")
+    if weight.shape[-1] % 2:
+        raise ValueError("the last dimension must be even")
+    if int(weight.min()) < -8 or int(weight.max()) > 7:
+        raise ValueError("Value in unpacked tensor not in int4 range")
+    w = weight.to(torch.int16)
+    return ((w[..., 0::2] & 0xF) | ((w[..., 1::2] & 0xF) << 4)).to(torch.uint8).view(torch.int8).contiguous()
+
+
+def unpack_int4_packed_tensor_to_int8(weight: torch.Tensor) -> torch.Tensor:
+    """Inverse, sign-extending (unpack_int4_packed_tensor_to_int8, WeightOnlyQuantOps.cc:256-284)."""
+    if weight.is_cuda or weight.dtype != torch.int8 or not weight.is_contiguous() or weight.numel() == 0:
+        raise ValueError("weight must be a non-empty contiguous CPU int8 packed tensor")
+    b = weight.view(torch.uint8).to(torch.int16)
+    lo, hi = b & 0xF, b >> 4
+    lo, hi = torch.where(lo > 7, lo - 16, lo), torch.where(hi > 7, hi - 16, hi)
+    return torch.stack((lo, hi), dim=-1).reshape(*weight.shape[:-1], weight.shape[-1] * 2).to(torch.int8)

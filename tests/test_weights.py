@@ -103,3 +103,37 @@ def test_w4a4_linear_from_bin_files(dev, tmp_path):
     mag = np.abs(y32).astype(np.float64) + np.abs(act).astype(np.float64) @ np.abs(to_np_f32(up)).astype(np.float64).T
     # the low-rank activation is rounded to bf16 from an fp32 sum whose order is free: one bf16 ULP of it is allowed
     assert_close_tol(to_np_f32(y), ref, "w4a4 linear from .bin files", abs_floor=2.0 ** -8 * mag)
+
+
+def test_int4_pack_helpers_match_the_oracle_packing():
+    from lyradiff_amd import weights as W
+
+    q = torch.randint(-8, 8, (6, 32), generator=rng_t(1), dtype=torch.int8)
+    packed = W.pack_int8_tensor_to_packed_int4(q)
+    assert packed.shape == (6, 16) and packed.dtype == torch.int8
+    assert np.array_equal(packed.numpy().view(np.uint32), O.pack_int4(q.numpy()))  # same low-nibble-first convention
+    assert torch.equal(W.unpack_int4_packed_tensor_to_int8(packed), q)
+    assert W.pack_int8_tensor_to_packed_int4(torch.tensor([[-8, 7]], dtype=torch.int8)).view(torch.uint8).item() == 0x78
+    with pytest.raises(ValueError, match="int4 range"):
+        W.pack_int8_tensor_to_packed_int4(torch.tensor([[8, 0]], dtype=torch.int8))
+
+
+@pytest.mark.gpu
+def test_smooth_vector_on_device(dev):
+    from lyradiff_amd import ops
+
+    g = rng_t(44)
+    x = torch.randn(1000, 1280, generator=g).half()
+    x[:, torch.randperm(1280, generator=g)[:8]] *= 20.0
+    w = torch.randint(-127, 128, (640, 1280), generator=g, dtype=torch.int8).float()
+    ax = ops.col_absmax(x[:600].contiguous().to(dev))
+    ax = ops.col_absmax(x[600:].contiguous().to(dev), ax)  # accumulated over two calibration batches
+    aw = ops.col_absmax(w.to(dev))
+    assert np.array_equal(ax.cpu().numpy(), np.abs(to_np_f32(x)).max(axis=0))
+    assert np.array_equal(aw.cpu().numpy(), np.abs(w.numpy()).max(axis=0))
+    pre, s = ops.smooth_vector(ax, aw, 0.5)
+    s_ref = O.smooth_vector(to_np_f32(x), w.numpy(), 0.5)
+    assert np.allclose(s.cpu().numpy(), s_ref, rtol=2e-6) and np.allclose(pre.cpu().numpy(), 1.0 / s_ref, rtol=3e-6)
+    # the vector does its job: the smoothed activation has a flatter column profile
+    t = to_np_f32(x) * pre.cpu().numpy()[None, :]
+    assert np.abs(t).max(axis=0).max() / np.median(np.abs(t).max(axis=0)) < 0.3 * np.abs(to_np_f32(x)).max(axis=0).max() / np.median(np.abs(to_np_f32(x)).max(axis=0))
