@@ -198,3 +198,24 @@ def test_config5_flux_double_block_fp8_chain(ops, dev):
     o = linear("out", attn, False, 53)
     hid = linear("up", o, True, 55)
     linear("down", hid, False, 57)
+
+
+# ---- sizes beyond 2^31 bytes: every row offset must be computed in 64 bits -----------------------------------------------
+def test_more_than_two_gib_of_activations(ops, dev):
+    m, k, n = 720_000, 3072, 64  # fp16 activations 4.4 GB, int8 2.2 GB
+    g = torch.Generator(device=dev).manual_seed(9)
+    x = torch.randn(m, k, generator=g, device=dev, dtype=torch.float16)
+    w = torch.randint(-127, 128, (n, k), generator=rng_t(9), dtype=torch.int8)
+    q, s = ops.sq_quant_dynamic(x, None)
+    acc = ops.int8_linear(q, ops.repack_weight(w.to(dev)), None, None, None, torch.int32)
+    rows = np.concatenate([np.arange(0, 4), np.arange(349_520, 349_530), np.arange(699_046, 699_056), np.arange(m - 4, m)])
+    idx = torch.from_numpy(rows).to(dev)
+    q_ref, s_ref = O.sq_dynamic_quant(to_np_f32(x[idx]), None)
+    assert np.array_equal(q[idx].cpu().numpy(), q_ref) and np.array_equal(s[idx].cpu().numpy(), s_ref)
+    assert np.array_equal(acc[idx].cpu().numpy(), O.gemm_i8_acc(q_ref, w.numpy()))
+    del x
+    xb = torch.randn(m, 1024, generator=g, device=dev, dtype=torch.bfloat16)  # 1.5 GB in, 0.7 GB out
+    qb, sb = ops.fp8_quant(xb)
+    assert np.float32(sb.cpu().numpy()[0]) == np.float32(xb.abs().max().float().cpu().numpy()) / np.float32(448.0)
+    ref = O.fp8_scale_cast(to_np_f32(xb[idx]), np.float32(sb.cpu().numpy()[0]), True)
+    assert np.array_equal(qb[idx].cpu().numpy(), ref)
