@@ -1,12 +1,14 @@
 // lyradiff_layers.h -- header-only host-side layer types of the quantized-linear path, over the C ABI
 // of lyraquant.h and the launchers of lyradiff_compat.h: the tensor plumbing (Tensor, TensorMap), the
-// named scratch pool (IAllocator / Allocator) and the W4A4 linear layer with its weight container,
+// named scratch pool (IAllocator / Allocator), the W4A4 linear layer with its weight container, the FP8 weight
+// that takes LoRA deltas (FP8LoraWeight) and the FP8 feed-forward halves of the FLUX blocks,
 // with the reference's names, members and call shapes (paths relative to the reference's
 // src/lyradiff/), so that reference-style layer code compiles against liblyraquant.so.
 //
 // Not built: file loading (loadWeights from .bin files) and the npy/torch tensor readers of Tensor.
 #pragma once
 
+#include <cstdlib>
 #include <cstring>
 #include <initializer_list>
 #include <sstream>
@@ -379,6 +381,342 @@ protected:
     float* input_scale_buffer = nullptr;
     uint32_t* quantized_input_buffer = nullptr;
     T* lora_down_res_buffer2 = nullptr;
+};
+
+// ---- interface/IFLoraWeight.h:79-128 ------------------------------------------------------------------------------
+// One FP8 weight that can take a full-rank LoRA delta: the 16-bit master copy stays on the host, a merge
+// re-quantises it with a fresh per-tensor scale.  weight_shape is {d_out, d_in} (the rows32 repack needs both;
+// the reference passes the flat element count); `weight` holds rows32 e4m3 codes.
+template <typename T>
+class FP8LoraWeight {
+public:
+    FP8LoraWeight() {}
+    FP8LoraWeight(const std::vector<size_t> weight_shape, fp8_e4m3_t* weight, float* weight_scale, T* weight_h)
+        : weight_shape_(weight_shape), weight_(weight), weight_scale_(weight_scale), weight_h_(weight_h) {
+        LYRA_CHECK_WITH_INFO(weight_shape_.size() == 2, "FP8LoraWeight: weight_shape must be {d_out, d_in}");
+    }
+    virtual ~FP8LoraWeight() {}
+    // lora_weight: device pointer to d_out * d_in elements of T
+    virtual void load_lora(const T* lora_weight, const float lora_scale, IAllocator* allocator) {
+        requantise(lora_weight, lora_scale, allocator);
+        loaded_lora = true;
+    }
+    virtual void clear_lora(IAllocator* allocator) {
+        if (!loaded_lora) return;
+        requantise(nullptr, 0.0f, allocator);
+        loaded_lora = false;
+    }
+    // quantises the master copy as it is (what the reference's load macros do once at load time)
+    void quantise(IAllocator* allocator) { requantise(nullptr, 0.0f, allocator); }
+
+private:
+    void requantise(const T* lora_weight, float lora_scale, IAllocator* allocator) {
+        const size_t n = weight_shape_[0] * weight_shape_[1];
+        hipStream_t st = allocator->returnStream();
+        T* tmp = static_cast<T*>(allocator->reMallocWithName("global_shared_weight_buffer_", sizeof(T) * n, false));
+        uint8_t* codes = static_cast<uint8_t*>(allocator->reMallocWithName("global_shared_weight_codes_buffer_", n, false));
+        LYRA_CHECK_WITH_INFO(hipMemcpyAsync(tmp, weight_h_, sizeof(T) * n, hipMemcpyHostToDevice, st) == hipSuccess,
+                             "FP8LoraWeight: upload of the master copy failed");
+        if (lora_weight != nullptr)
+            detail::check(lq_load_lora(tmp, lora_weight, detail::DType<T>::value, n, lora_scale, st), "FP8LoraWeight load_lora");
+        allocator->memSet(weight_scale_, 0, sizeof(float));
+        detail::check(lq_fp8_amax_scale(weight_scale_, tmp, detail::DType<T>::value, n, st), "FP8LoraWeight scale");
+        detail::check(lq_fp8_scale_cast(codes, tmp, detail::DType<T>::value, weight_scale_, 1, n, st), "FP8LoraWeight cast");
+        detail::check(lq_repack_rows32(reinterpret_cast<uint8_t*>(weight_), codes, weight_shape_[0], weight_shape_[1], st),
+                      "FP8LoraWeight repack");
+    }
+    std::vector<size_t> weight_shape_;
+    fp8_e4m3_t* weight_ = nullptr;
+    float* weight_scale_ = nullptr;
+    T* weight_h_ = nullptr;
+    bool loaded_lora = false;
+};
+
+namespace detail {
+// members of one FP8 linear as the reference's weight classes declare them (X_weight, X_bias, X_weight_scale,
+// X_input_scale, X_weight_h; layers/flux_attention_processor/FluxAttentionFP8ProcessorWeight.h:19-44)
+template <typename T> struct FP8LinearStore {
+    fp8_e4m3_t* weight = nullptr;
+    T* bias = nullptr;
+    float* weight_scale = nullptr;
+    float* input_scale = nullptr;
+    T* weight_h = nullptr;
+    size_t d_out = 0, d_in = 0;
+    void alloc(size_t n, size_t k) {
+        d_out = n; d_in = k;
+        bool ok = hipMalloc(reinterpret_cast<void**>(&weight), n * k) == hipSuccess &&
+                  hipMalloc(reinterpret_cast<void**>(&bias), sizeof(T) * n) == hipSuccess &&
+                  hipMalloc(reinterpret_cast<void**>(&weight_scale), sizeof(float)) == hipSuccess &&
+                  hipMalloc(reinterpret_cast<void**>(&input_scale), sizeof(float)) == hipSuccess;
+        weight_h = static_cast<T*>(std::malloc(sizeof(T) * n * k));
+        LYRA_CHECK_WITH_INFO(ok && weight_h != nullptr, "FP8 weight allocation failed");
+    }
+    void release() {
+        (void)hipFree(weight); (void)hipFree(bias); (void)hipFree(weight_scale); (void)hipFree(input_scale);
+        std::free(weight_h);
+        weight = nullptr; bias = nullptr; weight_scale = nullptr; input_scale = nullptr; weight_h = nullptr;
+    }
+    // MACROLoadFP8WeightFromCache (utils/common_macro_def.h:77-92): keys prefix + name + {".weight", ".bias", "_input_scale"}
+    void load(const std::string& prefix, const std::string& name, std::unordered_map<std::string, void*>& weights,
+              hipMemcpyKind kind, IAllocator* allocator) {
+        auto get = [&](const std::string& key) -> void* {
+            auto it = weights.find(key);
+            LYRA_CHECK_WITH_INFO(it != weights.end() && it->second != nullptr, "missing weight " + key);
+            return it->second;
+        };
+        hipStream_t st = allocator->returnStream();
+        const hipMemcpyKind to_host = kind == hipMemcpyHostToDevice ? hipMemcpyHostToHost : hipMemcpyDeviceToHost;
+        bool ok = hipMemcpyAsync(weight_h, get(prefix + name + ".weight"), sizeof(T) * d_out * d_in, to_host, st) == hipSuccess &&
+                  hipMemcpyAsync(bias, get(prefix + name + ".bias"), sizeof(T) * d_out, kind, st) == hipSuccess &&
+                  hipMemcpyAsync(input_scale, get(prefix + name + "_input_scale"), sizeof(float), kind, st) == hipSuccess &&
+                  hipStreamSynchronize(st) == hipSuccess;
+        LYRA_CHECK_WITH_INFO(ok, "FP8 weight copy failed for " + prefix + name);
+        FP8LoraWeight<T>({d_out, d_in}, weight, weight_scale, weight_h).quantise(allocator);
+    }
+};
+}  // namespace detail
+
+// ---- layers/flux_attn_post_processor/FluxAttnPostFP8ProcessorWeight.h, .cc:20-116 ------------------------------------
+template <typename T>
+class FluxAttnPostFP8ProcessorWeight {
+public:
+    fp8_e4m3_t* gelu_proj_weight = nullptr;  // [4D, D] rows32 e4m3
+    T* gelu_proj_bias = nullptr;
+    float* gelu_proj_weight_scale = nullptr;
+    float* gelu_proj_input_scale = nullptr;
+    T* gelu_proj_weight_h = nullptr;
+    fp8_e4m3_t* ff_linear_weight = nullptr;  // [D, 4D] rows32 e4m3
+    T* ff_linear_bias = nullptr;
+    float* ff_linear_weight_scale = nullptr;
+    float* ff_linear_input_scale = nullptr;
+    T* ff_linear_weight_h = nullptr;
+    std::unordered_map<std::string, FP8LoraWeight<T>*> lora_weight_map;
+
+    FluxAttnPostFP8ProcessorWeight(size_t embedding_dim, LyraQuantType quant_level, IAllocator* allocator)
+        : embedding_dim_(embedding_dim), allocator_(allocator) {
+        (void)quant_level;
+        LYRA_CHECK_WITH_INFO(allocator_ != nullptr && embedding_dim % 64 == 0, "FluxAttnPostFP8ProcessorWeight: bad arguments");
+    }
+    FluxAttnPostFP8ProcessorWeight(const FluxAttnPostFP8ProcessorWeight&) = delete;
+    FluxAttnPostFP8ProcessorWeight& operator=(const FluxAttnPostFP8ProcessorWeight&) = delete;
+    virtual ~FluxAttnPostFP8ProcessorWeight() {
+        if (is_maintain_buffer) {
+            gelu_.release();
+            ff_.release();
+            for (auto& kv : lora_weight_map) delete kv.second;
+        }
+    }
+    virtual void mallocWeights() {
+        if (is_maintain_buffer) return;
+        gelu_.alloc(embedding_dim_ * 4, embedding_dim_);
+        ff_.alloc(embedding_dim_, embedding_dim_ * 4);
+        publish();
+        lora_weight_map = {{"net.0.proj", new FP8LoraWeight<T>({gelu_.d_out, gelu_.d_in}, gelu_proj_weight, gelu_proj_weight_scale, gelu_proj_weight_h)},
+                           {"net.2", new FP8LoraWeight<T>({ff_.d_out, ff_.d_in}, ff_linear_weight, ff_linear_weight_scale, ff_linear_weight_h)}};
+        is_maintain_buffer = true;
+    }
+    virtual void loadWeightsFromCache(std::string prefix, std::unordered_map<std::string, void*>& weights, hipMemcpyKind memcpyKind) {
+        if (!is_maintain_buffer) mallocWeights();
+        gelu_.load(prefix, "net.0.proj", weights, memcpyKind, allocator_);
+        ff_.load(prefix, "net.2", weights, memcpyKind, allocator_);
+    }
+    size_t embedding_dim() const { return embedding_dim_; }
+
+protected:
+    bool is_maintain_buffer = false;
+
+private:
+    void publish() {
+        gelu_proj_weight = gelu_.weight; gelu_proj_bias = gelu_.bias; gelu_proj_weight_scale = gelu_.weight_scale;
+        gelu_proj_input_scale = gelu_.input_scale; gelu_proj_weight_h = gelu_.weight_h;
+        ff_linear_weight = ff_.weight; ff_linear_bias = ff_.bias; ff_linear_weight_scale = ff_.weight_scale;
+        ff_linear_input_scale = ff_.input_scale; ff_linear_weight_h = ff_.weight_h;
+    }
+    size_t embedding_dim_;
+    IAllocator* allocator_;
+    detail::FP8LinearStore<T> gelu_, ff_;
+};
+
+// ---- layers/flux_attn_post_processor/FluxAttnPostFP8Processor.cc:66-240 ---------------------------------------------
+// forward(): inputs "input", "attn_output" [B, S, D] and "msa_input" [6, B, D]; output "output" [B, S, D].
+// The reference's seven launches become three: gate+residual+adaLN+cast, the up GEMM whose epilogue writes the
+// e4m3 codes of gelu(.) for the down GEMM, and the down GEMM whose epilogue applies gate_mlp and the residual.
+template <typename T>
+class FluxAttnPostFP8Processor {
+public:
+    FluxAttnPostFP8Processor(size_t embedding_dim, hipStream_t stream, void* /*cublas_wrapper*/, IAllocator* allocator,
+                             const bool is_free_buffer_after_forward, const bool /*sparse*/ = false)
+        : embedding_dim_(embedding_dim), stream_(stream), allocator_(allocator),
+          is_free_buffer_after_forward_(is_free_buffer_after_forward) {
+        LYRA_CHECK_WITH_INFO(allocator_ != nullptr, "FluxAttnPostFP8Processor needs an allocator");
+    }
+    virtual ~FluxAttnPostFP8Processor() {}
+
+    virtual void forward(const TensorMap* output_tensors, const TensorMap* input_tensors,
+                         const FluxAttnPostFP8ProcessorWeight<T>* weights) {
+        Tensor input_tensor = input_tensors->at("input");
+        Tensor attn_tensor = input_tensors->at("attn_output");
+        Tensor msa_tensor = input_tensors->at("msa_input");
+        Tensor output_tensor = output_tensors->at("output");
+        LYRA_CHECK_WITH_INFO(input_tensor.shape.size() == 3 && input_tensor.shape[2] == embedding_dim_ &&
+                                 msa_tensor.shape.size() == 3 && msa_tensor.shape[0] == 6,
+                             "FluxAttnPostFP8Processor: input must be [B, S, D] and msa_input [6, B, D]");
+        const size_t batch_size = input_tensor.shape[0], seq_len = input_tensor.shape[1], d = embedding_dim_;
+        const size_t m = batch_size * seq_len;
+        allocateBuffer(batch_size, seq_len);
+        T* msa = msa_tensor.getPtr<T>();
+        const T* gate_msa = msa + 2 * batch_size * d;
+        const T* shift_mlp = msa + 3 * batch_size * d;
+        const T* scale_mlp = msa + 4 * batch_size * d;
+        const T* gate_mlp = msa + 5 * batch_size * d;
+        const lq_dtype_t dt = detail::DType<T>::value;
+        detail::check(lq_gate_residual_layernorm_mod_fp8(reinterpret_cast<uint8_t*>(fp8_buffer), hidden_buffer, attn_tensor.getPtr<T>(),
+                                                         gate_msa, input_tensor.getPtr<T>(), scale_mlp, shift_mlp, dt,
+                                                         weights->gelu_proj_input_scale, batch_size, seq_len, d, 1e-6f, stream_),
+                      "FluxAttnPostFP8Processor norm");
+        detail::check(lq_gemm_fp8_codes(reinterpret_cast<uint8_t*>(fp8_buffer2), 4 * d, weights->ff_linear_input_scale, dt,
+                                        reinterpret_cast<const uint8_t*>(fp8_buffer), reinterpret_cast<const uint8_t*>(weights->gelu_proj_weight),
+                                        weights->gelu_proj_input_scale, weights->gelu_proj_weight_scale, weights->gelu_proj_bias,
+                                        /*gelu=*/1, (int)m, (int)(4 * d), (int)d, stream_),
+                      "FluxAttnPostFP8Processor gelu_proj");
+        detail::check(lq_gemm_fp8_gated(output_tensor.getPtr<T>(), dt, reinterpret_cast<const uint8_t*>(fp8_buffer2),
+                                        reinterpret_cast<const uint8_t*>(weights->ff_linear_weight), weights->ff_linear_input_scale,
+                                        weights->ff_linear_weight_scale, weights->ff_linear_bias, gate_mlp, seq_len, hidden_buffer,
+                                        (int)m, (int)d, (int)(4 * d), stream_),
+                      "FluxAttnPostFP8Processor ff_linear");
+        if (is_free_buffer_after_forward_) freeBuffer();
+    }
+
+protected:
+    void allocateBuffer(size_t batch_size, size_t seq_len) {
+        const size_t elems = batch_size * seq_len * embedding_dim_;
+        hidden_buffer = static_cast<T*>(allocator_->reMallocWithName("FluxAttnPostProcessor_hidden_buffer", sizeof(T) * elems, false));
+        fp8_buffer = static_cast<fp8_e4m3_t*>(allocator_->reMallocWithName("fp8_input_buffer", elems * 4, false));
+        fp8_buffer2 = static_cast<fp8_e4m3_t*>(allocator_->reMallocWithName("fp8_input_buffer2", elems * 4, false));
+    }
+    void freeBuffer() {}
+
+    size_t embedding_dim_;
+    hipStream_t stream_;
+    IAllocator* allocator_;
+    bool is_free_buffer_after_forward_;
+    T* hidden_buffer = nullptr;
+    fp8_e4m3_t* fp8_buffer = nullptr;
+    fp8_e4m3_t* fp8_buffer2 = nullptr;
+};
+
+// ---- layers/flux_single_transformer_block/FluxSingleTransformerFP8BlockWeight.cc:60-121 (proj_mlp, proj_out) ---------
+template <typename T>
+class FluxSingleTransformerFP8MlpWeight {
+public:
+    fp8_e4m3_t* proj_mlp_weight = nullptr;  // [mlp_scale*D, D]
+    T* proj_mlp_bias = nullptr;
+    float* proj_mlp_weight_scale = nullptr;
+    float* proj_mlp_input_scale = nullptr;
+    T* proj_mlp_weight_h = nullptr;
+    fp8_e4m3_t* proj_out_weight = nullptr;  // [D, (mlp_scale+1)*D]
+    T* proj_out_bias = nullptr;
+    float* proj_out_weight_scale = nullptr;
+    float* proj_out_input_scale = nullptr;
+    T* proj_out_weight_h = nullptr;
+    std::unordered_map<std::string, FP8LoraWeight<T>*> lora_weight_map;
+
+    FluxSingleTransformerFP8MlpWeight(size_t embedding_dim, size_t mlp_scale, LyraQuantType quant_level, IAllocator* allocator)
+        : embedding_dim_(embedding_dim), mlp_scale_(mlp_scale), allocator_(allocator) {
+        (void)quant_level;
+        LYRA_CHECK_WITH_INFO(allocator_ != nullptr && embedding_dim % 64 == 0 && mlp_scale > 0, "FluxSingleTransformerFP8MlpWeight: bad arguments");
+    }
+    FluxSingleTransformerFP8MlpWeight(const FluxSingleTransformerFP8MlpWeight&) = delete;
+    FluxSingleTransformerFP8MlpWeight& operator=(const FluxSingleTransformerFP8MlpWeight&) = delete;
+    virtual ~FluxSingleTransformerFP8MlpWeight() {
+        if (is_maintain_buffer) {
+            mlp_.release();
+            out_.release();
+            for (auto& kv : lora_weight_map) delete kv.second;
+        }
+    }
+    virtual void mallocWeights() {
+        if (is_maintain_buffer) return;
+        mlp_.alloc(mlp_scale_ * embedding_dim_, embedding_dim_);
+        out_.alloc(embedding_dim_, (mlp_scale_ + 1) * embedding_dim_);
+        proj_mlp_weight = mlp_.weight; proj_mlp_bias = mlp_.bias; proj_mlp_weight_scale = mlp_.weight_scale;
+        proj_mlp_input_scale = mlp_.input_scale; proj_mlp_weight_h = mlp_.weight_h;
+        proj_out_weight = out_.weight; proj_out_bias = out_.bias; proj_out_weight_scale = out_.weight_scale;
+        proj_out_input_scale = out_.input_scale; proj_out_weight_h = out_.weight_h;
+        lora_weight_map = {{"proj_mlp", new FP8LoraWeight<T>({mlp_.d_out, mlp_.d_in}, proj_mlp_weight, proj_mlp_weight_scale, proj_mlp_weight_h)},
+                           {"proj_out", new FP8LoraWeight<T>({out_.d_out, out_.d_in}, proj_out_weight, proj_out_weight_scale, proj_out_weight_h)}};
+        is_maintain_buffer = true;
+    }
+    virtual void loadWeightsFromCache(std::string prefix, std::unordered_map<std::string, void*>& weights, hipMemcpyKind memcpyKind) {
+        if (!is_maintain_buffer) mallocWeights();
+        mlp_.load(prefix, "proj_mlp", weights, memcpyKind, allocator_);
+        out_.load(prefix, "proj_out", weights, memcpyKind, allocator_);
+    }
+    size_t embedding_dim() const { return embedding_dim_; }
+    size_t mlp_scale() const { return mlp_scale_; }
+
+protected:
+    bool is_maintain_buffer = false;
+
+private:
+    size_t embedding_dim_, mlp_scale_;
+    IAllocator* allocator_;
+    detail::FP8LinearStore<T> mlp_, out_;
+};
+
+// ---- layers/flux_single_transformer_block/FluxSingleTransformerFP8Block.cc:209-290 -----------------------------------
+// The part of the single block's forward after the attention: inputs "input", "norm_hidden", "attn_output"
+// [B, S, D] and "gate" [B, D] (chunk 2 of the block's msa buffer); output "output" [B, S, D].  The proj_mlp GEMM
+// writes the e4m3 codes of gelu(mlp) into the right-hand columns of the concatenated projection input, a strided
+// cast fills the attention columns, and the proj_out GEMM applies the gate and the residual in its epilogue.
+template <typename T>
+class FluxSingleTransformerFP8Mlp {
+public:
+    FluxSingleTransformerFP8Mlp(size_t embedding_dim, size_t mlp_scale, hipStream_t stream, void* /*cublas_wrapper*/,
+                                IAllocator* allocator, const bool is_free_buffer_after_forward)
+        : embedding_dim_(embedding_dim), mlp_scale_(mlp_scale), stream_(stream), allocator_(allocator),
+          is_free_buffer_after_forward_(is_free_buffer_after_forward) {
+        LYRA_CHECK_WITH_INFO(allocator_ != nullptr, "FluxSingleTransformerFP8Mlp needs an allocator");
+    }
+    virtual ~FluxSingleTransformerFP8Mlp() {}
+
+    virtual void forward(const TensorMap* output_tensors, const TensorMap* input_tensors,
+                         const FluxSingleTransformerFP8MlpWeight<T>* weights) {
+        Tensor input_tensor = input_tensors->at("input");
+        Tensor norm_tensor = input_tensors->at("norm_hidden");
+        Tensor attn_tensor = input_tensors->at("attn_output");
+        Tensor gate_tensor = input_tensors->at("gate");
+        Tensor output_tensor = output_tensors->at("output");
+        LYRA_CHECK_WITH_INFO(input_tensor.shape.size() == 3 && input_tensor.shape[2] == embedding_dim_,
+                             "FluxSingleTransformerFP8Mlp: input must be [B, S, D]");
+        const size_t batch_size = input_tensor.shape[0], seq_len = input_tensor.shape[1], d = embedding_dim_;
+        const size_t m = batch_size * seq_len, f = mlp_scale_ * d;
+        fp8_buffer1 = static_cast<fp8_e4m3_t*>(allocator_->reMallocWithName("fp8_input_buffer", m * (d + f), false));
+        fp8_buffer2 = static_cast<fp8_e4m3_t*>(allocator_->reMallocWithName("fp8_input_buffer2", m * d, false));
+        const lq_dtype_t dt = detail::DType<T>::value;
+        uint8_t* cat = reinterpret_cast<uint8_t*>(fp8_buffer1);
+        detail::check(lq_fp8_scale_cast(reinterpret_cast<uint8_t*>(fp8_buffer2), norm_tensor.getPtr<T>(), dt, weights->proj_mlp_input_scale, 1,
+                                        m * d, stream_), "FluxSingleTransformerFP8Mlp cast");
+        detail::check(lq_fp8_scale_cast_2d(cat, d + f, attn_tensor.getPtr<T>(), d, dt, weights->proj_out_input_scale, 1, m, d, stream_),
+                      "FluxSingleTransformerFP8Mlp attn cast");
+        detail::check(lq_gemm_fp8_codes(cat + d, d + f, weights->proj_out_input_scale, dt, reinterpret_cast<const uint8_t*>(fp8_buffer2),
+                                        reinterpret_cast<const uint8_t*>(weights->proj_mlp_weight), weights->proj_mlp_input_scale,
+                                        weights->proj_mlp_weight_scale, weights->proj_mlp_bias, /*gelu=*/2, (int)m, (int)f, (int)d, stream_),
+                      "FluxSingleTransformerFP8Mlp proj_mlp");
+        detail::check(lq_gemm_fp8_gated(output_tensor.getPtr<T>(), dt, cat, reinterpret_cast<const uint8_t*>(weights->proj_out_weight),
+                                        weights->proj_out_input_scale, weights->proj_out_weight_scale, weights->proj_out_bias,
+                                        gate_tensor.getPtr<T>(), seq_len, input_tensor.getPtr<T>(), (int)m, (int)d, (int)(d + f), stream_),
+                      "FluxSingleTransformerFP8Mlp proj_out");
+        (void)is_free_buffer_after_forward_;
+    }
+
+protected:
+    size_t embedding_dim_, mlp_scale_;
+    hipStream_t stream_;
+    IAllocator* allocator_;
+    bool is_free_buffer_after_forward_;
+    fp8_e4m3_t* fp8_buffer1 = nullptr;
+    fp8_e4m3_t* fp8_buffer2 = nullptr;
 };
 
 }  // namespace lyradiff

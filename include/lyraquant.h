@@ -197,6 +197,36 @@ int lq_gemm_fp8_ex(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_
                    const void* residual, float beta, int m, int n, int k,
                    float* out_scale, uint8_t* C_fp8, const float* C_fp8_scale, lq_stream_t stream);
 
+/* lq_gemm_fp8 (no activation) whose epilogue applies FLUX's gate and second residual:
+ *   C[m,n] = T( T( T(y[m,n]) * gate[m / rows_per_gate, n] ) + residual[m,n] ),  y = (sa*sb)*acc + bias[n]
+ * with every rounding of the reference's sequence "GEMM stores T, then multiply and add in T": it replaces
+ * GemmWithResidualAndBias followed by invokeFusedGateAndResidual
+ * (layers/flux_attn_post_processor/FluxAttnPostFP8Processor.cc:203-236,
+ * layers/flux_single_transformer_block/FluxSingleTransformerFP8Block.cc:255-290,
+ * kernels/flux_single_transformer_block/flux_single_transformer_kernels.cu:42-65,162-170).
+ * gate [ceil(m / rows_per_gate), n] and residual [m, n] have the output dtype; C may alias residual. */
+int lq_gemm_fp8_gated(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32,
+                      const float* a_scale, const float* b_scale, const void* bias, const void* gate,
+                      size_t rows_per_gate, const void* residual, int m, int n, int k, lq_stream_t stream);
+
+/* lq_gemm_fp8 that writes only e4m3 codes of its output, into a destination whose rows are `ldc` bytes apart:
+ *   C_fp8[m*ldc + n] = e4m3( f32(T(act(y))) * (1 / C_fp8_scale[0]) ),  T = round_dtype (F16/BF16/F32)
+ * gelu: 0 none; 1 tanh-GELU of the fp32 value (the GELU_BIAS epilogue, cublasMMWrapper.cc:1195-1199);
+ * 2 tanh-GELU of T(y), the activation the reference applies to the stored GEMM output in invokeFusedCatAndGelu
+ * (flux_single_transformer_kernels.cu:9-40).  With ldc = attn_dim + mlp_dim and C_fp8 offset by attn_dim this
+ * fills the right-hand block of the single block's concatenated projection input directly
+ * (FluxSingleTransformerFP8Block.cc:216-253) and the 16-bit intermediates are never written.
+ * ldc >= n, ldc % 4 == 0, C_fp8 4-byte aligned. */
+int lq_gemm_fp8_codes(uint8_t* C_fp8, size_t ldc, const float* C_fp8_scale, lq_dtype_t round_dtype,
+                      const uint8_t* A, const uint8_t* B_rows32, const float* a_scale, const float* b_scale,
+                      const void* bias, int gelu, int m, int n, int k, lq_stream_t stream);
+
+/* lq_fp8_scale_cast on a matrix view: rows `src_ld` elements apart are cast into rows `dst_ld` bytes apart
+ * (the left-hand, attention block of the concatenated tensor above).  cols % 16 == 0; every row of both views
+ * 16-byte aligned. */
+int lq_fp8_scale_cast_2d(uint8_t* dst, size_t dst_ld, const void* src, size_t src_ld, lq_dtype_t dtype,
+                         const float* scale, int invert, size_t rows, size_t cols, lq_stream_t stream);
+
 /* SmoothQuant smoothing vector, device side (calibration time).  The reference consumes a precomputed
  * pre_quant_scale from nvidia-modelopt (lyradiff/convert_model_scripts/convert_sd_quant_model.py:199,340); these two
  * calls produce it in the closed form its benchmark configuration states:
@@ -234,6 +264,22 @@ int lq_layernorm_mod_fp8(uint8_t* dst, const void* src, const void* scale, const
                          const float* input_scale, size_t batch, size_t rows_per_batch, size_t dim, float eps,
                          lq_stream_t stream);
 
+/* lq_layernorm_mod_fp8 for a normalised tensor with two consumers, each with its own calibrated input scale (FLUX's
+ * single block feeds norm_hidden to both to_qkv and proj_mlp: FluxSingleAttentionFP8Processor.cc:155-172,
+ * FluxSingleTransformerFP8Block.cc:209-214): one read of src, two code tensors, no 16-bit tensor written. */
+int lq_layernorm_mod_fp8_dual(uint8_t* dst_a, const float* input_scale_a, uint8_t* dst_b, const float* input_scale_b,
+                              const void* src, const void* scale, const void* shift, lq_dtype_t dtype, size_t batch,
+                              size_t rows_per_batch, size_t dim, float eps, lq_stream_t stream);
+
+/* invokeFusedGateAndResidual + invokeLayerNormWithShiftAndScale + invokeCudaD2DScaleCpyConvert in one pass
+ * (layers/flux_attn_post_processor/FluxAttnPostFP8Processor.cc:112-140):
+ *   hidden_out = T( T(attn * gate[b,k]) + input ),  dst = lq_layernorm_mod_fp8(hidden_out, scale, shift, input_scale)
+ * attn, input, hidden_out [batch * rows_per_batch, dim]; gate, scale, shift [batch, dim]; hidden_out may alias input. */
+int lq_gate_residual_layernorm_mod_fp8(uint8_t* dst, void* hidden_out, const void* attn, const void* gate,
+                                       const void* input, const void* scale, const void* shift, lq_dtype_t dtype,
+                                       const float* input_scale, size_t batch, size_t rows_per_batch, size_t dim,
+                                       float eps, lq_stream_t stream);
+
 /* W4A4 GEMM with the SVDQuant low-rank branch of invokeFusedW4A4GemmAndLoraUp
  * (kernels/w4a4_gemm/w4a4_gemm.h:18-30; lora_up_gemm, kernels/w4a4_gemm/w4a4_gemm.cu:514-663):
  *   C = T( sum_g f32(p_g) * sA * sB  +  sum_r lora_act[m, r] * lora_up[n, r]  [+ bias[n]] ),
@@ -258,6 +304,12 @@ int lq_lora_down(void* out, lq_dtype_t out_dtype, const void* x, const void* lor
 /* dst[i] = T(src[i]), the float -> T copy between the reference's two W4A4 kernels
  * (invokeCudaD2DcpyConvert<T, float>, utils/memory_utils.cu:398-402). */
 int lq_cast_f32(void* dst, lq_dtype_t dst_dtype, const float* src, size_t n, lq_stream_t stream);
+
+/* dst[i] = T( dst[i] + T( src[i] * T(alpha) ) ): merges a full-rank LoRA delta into a 16-bit (or fp32) weight
+ * (invokeLoadLora, kernels/lora/load_lora.h + load_lora.cu:6-14,92-96).  An FP8 weight is re-quantised after the
+ * merge the way FP8LoraWeight::load_lora / clear_lora do (interface/IFLoraWeight.h:79-128): restore the 16-bit
+ * master copy, lq_load_lora, zero the scale, lq_fp8_amax_scale, lq_fp8_scale_cast, lq_repack_rows32. */
+int lq_load_lora(void* dst, const void* src, lq_dtype_t dtype, size_t n, float alpha, lq_stream_t stream);
 
 /* Forces the tile configuration ("tactic") used by the GEMM of `kind` (process-wide); -1 restores
  * the built-in static table.  Stands in for the CutlassGemmConfig argument of

@@ -70,7 +70,7 @@ def build_compat_check(force: bool = False) -> list:
     """Compiles the reference-style C++ call-site programs under tests/cpp against the library."""
     exes = []
     hdrs = [os.path.join(ROOT, "include", h) for h in ("lyradiff_compat.h", "lyradiff_layers.h", "lyraquant.h")]
-    for name in ("compat_check", "layers_check"):
+    for name in ("compat_check", "layers_check", "flux_fp8_check"):
         src = os.path.join(ROOT, "tests", "cpp", name + ".cpp")
         exe = os.path.join(ROOT, "tests", "cpp", name)
         if not os.path.exists(src):

@@ -48,6 +48,13 @@ struct GemmParams {
     float* out_scale;       // optional: max(out_scale, max|C| / 448), the e4m3 scale of the output for a following cast
     uint8_t* C8;            // optional: e4m3 codes of C with a given (static) scale, written next to or instead of C
     const float* c8_scale;  // scale of C8: C8 = e4m3(f32(T(y)) * (1 / c8_scale[0]))
+    size_t ldc8;            // row pitch of C8 in bytes (n when the codes are dense)
+    // gelu: 0 none, 1 on the fp32 value, 2 on the value rounded to T first (the activation applied by a separate
+    // kernel to a stored T tensor)
+    // gate: C = T( T( T(y) * gate[m / gate_rows, n] ) + residual[m, n] ), the roundings of a GEMM that stores T
+    // followed by an elementwise multiply and add in T; requires residual, ignores beta
+    const void* gate;
+    size_t gate_rows;
     // w4a4
     const void* sA;
     const void* sB;
@@ -562,10 +569,19 @@ struct GemmKernel {
         const int out_row = lane / LPR, out_n = n0 + wn * TN + (lane % LPR) * 4;
         const bool n_ok = out_n < p.n;
         float alpha = 1.0f, bias4[4] = {0.f, 0.f, 0.f, 0.f}, acol4[4] = {0.f, 0.f, 0.f, 0.f}, arow_l[MT];
-        float out_amax = 0.0f, c8_inv = 0.0f;
+        float out_amax = 0.0f, c8_inv = 0.0f, gate4[4] = {0.f, 0.f, 0.f, 0.f};
+        bool gate_uniform = true;  // every row of the wavefront's tile uses the same gate vector
         if constexpr (KIND == K_FP8) {
             alpha = p.a_scale[0] * p.b_scale[0];
             if (p.C8 != nullptr) c8_inv = 1.0f / p.c8_scale[0];
+            if constexpr (!kI32) {
+                if (p.gate != nullptr) {
+                    const size_t r_first = (size_t)(m0 + wm * TM), r_last = (size_t)min(m0 + wm * TM + TM - 1, p.m - 1);
+                    const size_t b_first = r_first / p.gate_rows;
+                    gate_uniform = b_first == r_last / p.gate_rows;
+                    if (gate_uniform && n_ok && r_first < (size_t)p.m) OutStore<OutTag>::load4(p.gate, b_first * (size_t)p.n + out_n, gate4);
+                }
+            }
         }
         if constexpr (!kI32) {
             if (p.bias != nullptr && n_ok) OutStore<OutTag>::load4(p.bias, out_n, bias4);
@@ -630,15 +646,25 @@ struct GemmKernel {
                             y[e] = (KIND == K_FP8) ? vf[e] * alpha : vf[e];
                             if (p.bias != nullptr) y[e] = y[e] + bias4[e];
                             if constexpr (KIND == K_FP8) {
-                                if (p.gelu) y[e] = gelu_fast(y[e]);
+                                if (p.gelu) {
+                                    if (p.gelu == 2) y[e] = round_through<OutTag>(y[e]);
+                                    y[e] = gelu_fast(y[e]);
+                                }
                             }
                         }
                         if constexpr (KIND == K_FP8) {
                             if (p.residual != nullptr && ok) {
                                 float rr[4];
                                 OutStore<OutTag>::load4(p.residual, idx, rr);
+                                if (p.gate != nullptr) {
+                                    if (!gate_uniform) OutStore<OutTag>::load4(p.gate, ((size_t)mo / p.gate_rows) * (size_t)p.n + out_n, gate4);
 #pragma unroll
-                                for (int e = 0; e < 4; ++e) y[e] = y[e] + p.beta * rr[e];
+                                    for (int e = 0; e < 4; ++e)
+                                        y[e] = round_through<OutTag>(round_through<OutTag>(y[e]) * gate4[e]) + rr[e];
+                                } else {
+#pragma unroll
+                                    for (int e = 0; e < 4; ++e) y[e] = y[e] + p.beta * rr[e];
+                                }
                             }
                         }
                     }
@@ -650,7 +676,7 @@ struct GemmKernel {
                                 float t[4];
 #pragma unroll
                                 for (int e = 0; e < 4; ++e) t[e] = round_through<OutTag>(y[e]) * c8_inv;
-                                *reinterpret_cast<u32*>(p.C8 + idx) = e4m3x4(t[0], t[1], t[2], t[3]);
+                                *reinterpret_cast<u32*>(p.C8 + (size_t)mo * p.ldc8 + out_n) = e4m3x4(t[0], t[1], t[2], t[3]);
                             }
                         }
                     }

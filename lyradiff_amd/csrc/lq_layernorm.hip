@@ -7,6 +7,9 @@
 //   * FP8 (FLUX): invokeLayerNormWithShiftAndScale followed by invokeCudaD2DScaleCpyConvert
 //     (kernels/norms/layer_norm.cu:406-475, layers/flux_attn_post_processor/FluxAttnPostFP8Processor.cc:125-140):
 //       y = T( T( T(scale[b,k] + 1) * T((x - mean) * rstd) ) + shift[b,k] ),   q = e4m3( f32(y) * (1/s) )
+//     optionally preceded by invokeFusedGateAndResidual (kernels/flux_single_transformer_block/
+//     flux_single_transformer_kernels.cu:42-65, FluxAttnPostFP8Processor.cc:112-119):
+//       x = T( T(attn * gate[b,k]) + input ), also written out (the block's second residual uses it)
 // One wavefront owns a row: the row stays in registers between the statistics and the quantisation, so the
 // activation is read once and only the 1-byte codes (and dst2) are written.  Mean and variance are two-pass
 // fp32 sums over the registers (the reference runs Welford updates, in T for the INT8 kernels), reduced across
@@ -36,19 +39,21 @@ __device__ __forceinline__ u32 ln_nan_fix(u32 w, const float* y) {  // NaN -> 0x
 
 // QMODE 0: int8, static per-tensor scale; 1: int8, dynamic per-token scale (written to scale_out); 2: fp8, static scale.
 // MOD false: y = gamma*n + beta (vectors of length dim).  MOD true: y = (1 + scale[b])*n + shift[b], b = row / rows_per_batch.
-template <typename Tag, int NP, int QMODE, bool RESID, bool MOD>
+// RESID 0: h = src.  1: h = T(T(src + residual) + bias).  2: h = T(T(src * gate[b]) + residual), gate passed as `bias`.
+template <typename Tag, int NP, int QMODE, int RESID, bool MOD>
 __global__ __launch_bounds__(256) void ln_quant_rows_kernel(uint8_t* __restrict__ dst, void* __restrict__ dst2,
                                                             float* __restrict__ scale_out, const void* __restrict__ src,
                                                             const void* __restrict__ residual, const void* __restrict__ bias,
                                                             const void* __restrict__ gamma, const void* __restrict__ beta,
                                                             const float* __restrict__ pre, const float* __restrict__ in_scale,
+                                                            uint8_t* __restrict__ dst_b, const float* __restrict__ in_scale_b,
                                                             size_t rows, int dim, size_t rows_per_batch, float eps) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const size_t row = (size_t)blockIdx.x * 4 + wave;
     if (row >= rows) return;
     const size_t row_off = row * (size_t)dim;
     const unsigned short* xs = static_cast<const unsigned short*>(src) + row_off;
-    const size_t mod_off = MOD ? (row / rows_per_batch) * (size_t)dim : 0;
+    const size_t mod_off = (MOD || RESID == 2) ? (row / rows_per_batch) * (size_t)dim : 0;
     const unsigned short* gs = static_cast<const unsigned short*>(gamma) + mod_off;
     const unsigned short* bs = static_cast<const unsigned short*>(beta) + mod_off;
     float h[NP][8];
@@ -60,15 +65,21 @@ __global__ __launch_bounds__(256) void ln_quant_rows_kernel(uint8_t* __restrict_
         for (int i = 0; i < 8; ++i) h[p][i] = 0.0f;
         if (col < dim) {
             unpack8<Tag>(*reinterpret_cast<const uint4*>(xs + col), h[p]);
-            if constexpr (RESID) {
+            if constexpr (RESID != 0) {
                 float r[8], b[8];
                 unpack8<Tag>(*reinterpret_cast<const uint4*>(static_cast<const unsigned short*>(residual) + row_off + col), r);
+                if constexpr (RESID == 2) {
+                    unpack8<Tag>(*reinterpret_cast<const uint4*>(static_cast<const unsigned short*>(bias) + mod_off + col), b);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) h[p][i] = round_through<Tag>(h[p][i] + r[i]);
-                if (bias != nullptr) {
-                    unpack8<Tag>(*reinterpret_cast<const uint4*>(static_cast<const unsigned short*>(bias) + col), b);
+                    for (int i = 0; i < 8; ++i) h[p][i] = round_through<Tag>(round_through<Tag>(h[p][i] * b[i]) + r[i]);
+                } else {
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) h[p][i] = round_through<Tag>(h[p][i] + b[i]);
+                    for (int i = 0; i < 8; ++i) h[p][i] = round_through<Tag>(h[p][i] + r[i]);
+                    if (bias != nullptr) {
+                        unpack8<Tag>(*reinterpret_cast<const uint4*>(static_cast<const unsigned short*>(bias) + col), b);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) h[p][i] = round_through<Tag>(h[p][i] + b[i]);
+                    }
                 }
                 uint4 o;
                 u32* ow = reinterpret_cast<u32*>(&o);
@@ -141,7 +152,11 @@ __global__ __launch_bounds__(256) void ln_quant_rows_kernel(uint8_t* __restrict_
         s = in_scale[0];
     }
     if constexpr (QMODE == 2) {
-        const float inv = 1.0f / s;
+        // one set of codes per consumer of the normalised tensor (each linear has its own calibrated input scale)
+        const int nout = dst_b != nullptr ? 2 : 1;
+        for (int o2 = 0; o2 < nout; ++o2) {
+        uint8_t* const out = o2 ? dst_b : dst;
+        const float inv = 1.0f / (o2 ? in_scale_b[0] : s);
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             const int col = (p * 64 + lane) * 8;
@@ -160,8 +175,9 @@ __global__ __launch_bounds__(256) void ln_quant_rows_kernel(uint8_t* __restrict_
                     o.x = ln_nan_fix(o.x, v);
                     o.y = ln_nan_fix(o.y, v + 4);
                 }
-                *reinterpret_cast<uint2*>(dst + row_off + col) = o;
+                *reinterpret_cast<uint2*>(out + row_off + col) = o;
             }
+        }
         }
     } else {
         const float r = fast_recip(s);
@@ -183,16 +199,16 @@ __global__ __launch_bounds__(256) void ln_quant_rows_kernel(uint8_t* __restrict_
 
 struct LnArgs {
     uint8_t* dst; void* dst2; float* scale_out; const void* src; const void* residual; const void* bias;
-    const void* gamma; const void* beta; const float* pre; const float* in_scale;
+    const void* gamma; const void* beta; const float* pre; const float* in_scale; uint8_t* dst_b; const float* in_scale_b;
     size_t rows; int dim; size_t rows_per_batch; float eps;
 };
 
-template <typename Tag, int QMODE, bool RESID, bool MOD> static int launch_ln(const LnArgs& a, hipStream_t st) {
+template <typename Tag, int QMODE, int RESID, bool MOD> static int launch_ln(const LnArgs& a, hipStream_t st) {
     const int np = (a.dim + 511) / 512;
     dim3 grid((unsigned)((a.rows + 3) / 4)), block(256);
 #define LQ_LN_CASE(NPV)                                                                                              \
     hipLaunchKernelGGL((ln_quant_rows_kernel<Tag, NPV, QMODE, RESID, MOD>), grid, block, 0, st, a.dst, a.dst2, a.scale_out, \
-                       a.src, a.residual, a.bias, a.gamma, a.beta, a.pre, a.in_scale, a.rows, a.dim, a.rows_per_batch, a.eps)
+                       a.src, a.residual, a.bias, a.gamma, a.beta, a.pre, a.in_scale, a.dst_b, a.in_scale_b, a.rows, a.dim, a.rows_per_batch, a.eps)
     if (np <= 1) LQ_LN_CASE(1);
     else if (np <= 2) LQ_LN_CASE(2);
     else if (np <= 3) LQ_LN_CASE(3);
@@ -235,12 +251,12 @@ extern "C" int lq_layernorm_int8(int8_t* dst, float* scale_out, void* dst2, cons
                LQ_ERR_ARG, "lq_layernorm_int8: vectors must be 16-byte aligned");
     if (rows == 0) return LQ_OK;
     LnArgs a = {reinterpret_cast<uint8_t*>(dst), dst2, scale_out, src, residual, bias, gamma, beta, pre_quant_scale,
-                input_quant_scale, rows, (int)dim, 1, eps};
+                input_quant_scale, nullptr, nullptr, rows, (int)dim, 1, eps};
     hipStream_t st = as_stream(stream);
     const bool dyn = scale_out != nullptr, res = residual != nullptr, f16 = dtype == LQ_F16;
 #define LQ_LN_GO(Tag)                                                                                   \
-    (dyn ? (res ? launch_ln<Tag, 1, true, false>(a, st) : launch_ln<Tag, 1, false, false>(a, st))       \
-         : (res ? launch_ln<Tag, 0, true, false>(a, st) : launch_ln<Tag, 0, false, false>(a, st)))
+    (dyn ? (res ? launch_ln<Tag, 1, 1, false>(a, st) : launch_ln<Tag, 1, 0, false>(a, st))       \
+         : (res ? launch_ln<Tag, 0, 1, false>(a, st) : launch_ln<Tag, 0, 0, false>(a, st)))
     return f16 ? LQ_LN_GO(F16Tag) : LQ_LN_GO(BF16Tag);
 #undef LQ_LN_GO
 }
@@ -254,8 +270,43 @@ extern "C" int lq_layernorm_mod_fp8(uint8_t* dst, const void* src, const void* s
     LQ_REQUIRE(reinterpret_cast<uintptr_t>(scale) % 16 == 0 && reinterpret_cast<uintptr_t>(shift) % 16 == 0, LQ_ERR_ARG,
                "lq_layernorm_mod_fp8: scale and shift must be 16-byte aligned");
     if (batch * rows_per_batch == 0) return LQ_OK;
-    LnArgs a = {dst, nullptr, nullptr, src, nullptr, nullptr, scale, shift, nullptr, input_scale, batch * rows_per_batch,
-                (int)dim, rows_per_batch, eps};
+    LnArgs a = {dst, nullptr, nullptr, src, nullptr, nullptr, scale, shift, nullptr, input_scale, nullptr, nullptr,
+                batch * rows_per_batch, (int)dim, rows_per_batch, eps};
     hipStream_t st = as_stream(stream);
-    return dtype == LQ_F16 ? launch_ln<F16Tag, 2, false, true>(a, st) : launch_ln<BF16Tag, 2, false, true>(a, st);
+    return dtype == LQ_F16 ? launch_ln<F16Tag, 2, 0, true>(a, st) : launch_ln<BF16Tag, 2, 0, true>(a, st);
+}
+
+extern "C" int lq_layernorm_mod_fp8_dual(uint8_t* dst_a, const float* input_scale_a, uint8_t* dst_b, const float* input_scale_b,
+                                         const void* src, const void* scale, const void* shift, lq_dtype_t dtype, size_t batch,
+                                         size_t rows_per_batch, size_t dim, float eps, lq_stream_t stream) {
+    int rc = check_ln_common("lq_layernorm_mod_fp8_dual", dst_a, src, dtype, batch * rows_per_batch, dim);
+    if (rc != LQ_OK) return rc;
+    LQ_REQUIRE(dst_b && scale && shift && input_scale_a && input_scale_b, LQ_ERR_ARG, "lq_layernorm_mod_fp8_dual: null pointer");
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(scale) % 16 == 0 && reinterpret_cast<uintptr_t>(shift) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(dst_b) % 8 == 0,
+               LQ_ERR_ARG, "lq_layernorm_mod_fp8_dual: scale and shift must be 16-byte, dst_b 8-byte aligned");
+    if (batch * rows_per_batch == 0) return LQ_OK;
+    LnArgs a = {dst_a, nullptr, nullptr, src, nullptr, nullptr, scale, shift, nullptr, input_scale_a, dst_b, input_scale_b,
+                batch * rows_per_batch, (int)dim, rows_per_batch, eps};
+    hipStream_t st = as_stream(stream);
+    return dtype == LQ_F16 ? launch_ln<F16Tag, 2, 0, true>(a, st) : launch_ln<BF16Tag, 2, 0, true>(a, st);
+}
+
+extern "C" int lq_gate_residual_layernorm_mod_fp8(uint8_t* dst, void* hidden_out, const void* attn, const void* gate,
+                                                  const void* input, const void* scale, const void* shift, lq_dtype_t dtype,
+                                                  const float* input_scale, size_t batch, size_t rows_per_batch, size_t dim,
+                                                  float eps, lq_stream_t stream) {
+    int rc = check_ln_common("lq_gate_residual_layernorm_mod_fp8", dst, attn, dtype, batch * rows_per_batch, dim);
+    if (rc != LQ_OK) return rc;
+    LQ_REQUIRE(hidden_out && gate && input && scale && shift && input_scale, LQ_ERR_ARG,
+               "lq_gate_residual_layernorm_mod_fp8: null pointer");
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(scale) % 16 == 0 && reinterpret_cast<uintptr_t>(shift) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(gate) % 16 == 0 && reinterpret_cast<uintptr_t>(input) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(hidden_out) % 16 == 0,
+               LQ_ERR_ARG, "lq_gate_residual_layernorm_mod_fp8: all tensors must be 16-byte aligned");
+    if (batch * rows_per_batch == 0) return LQ_OK;
+    LnArgs a = {dst, hidden_out, nullptr, attn, input, gate, scale, shift, nullptr, input_scale, nullptr, nullptr,
+                batch * rows_per_batch, (int)dim, rows_per_batch, eps};
+    hipStream_t st = as_stream(stream);
+    return dtype == LQ_F16 ? launch_ln<F16Tag, 2, 2, true>(a, st) : launch_ln<BF16Tag, 2, 2, true>(a, st);
 }

@@ -120,9 +120,40 @@ template <int OUT> __global__ void cast_f32_kernel(void* __restrict__ dst, const
     }
 }
 
+// Merge of a full-rank LoRA delta into a 16/32-bit weight, the first step of re-quantising an FP8 weight
+// (loadLora, kernels/lora/load_lora.cu:6-14; FP8LoraWeight::load_lora, interface/IFLoraWeight.h:100-112):
+//   dst[i] = T( dst[i] + T( src[i] * T(alpha) ) )
+template <typename Tag> __global__ void load_lora_kernel(void* __restrict__ dst, const void* __restrict__ src, size_t n, float alpha) {
+    const float a = round_through<Tag>(alpha);
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        if constexpr (Elem<Tag>::bytes == 2) {
+            unsigned short* d = static_cast<unsigned short*>(dst);
+            const float w = Elem<Tag>::load(d[i]), l = Elem<Tag>::load(static_cast<const unsigned short*>(src)[i]);
+            d[i] = (unsigned short)Elem<Tag>::store(round_through<Tag>(l * a) + w);
+        } else {
+            float* d = static_cast<float*>(dst);
+            d[i] = d[i] + static_cast<const float*>(src)[i] * a;
+        }
+    }
+}
+
 }  // namespace lq
 
 using namespace lq;
+
+extern "C" int lq_load_lora(void* dst, const void* src, lq_dtype_t dtype, size_t n, float alpha, lq_stream_t stream) {
+    LQ_REQUIRE((dst && src) || n == 0, LQ_ERR_ARG, "lq_load_lora: null pointer");
+    if (n == 0) return LQ_OK;
+    hipStream_t st = as_stream(stream);
+    const unsigned blocks = (unsigned)std::min<size_t>((n + 255) / 256, 4096);
+    switch (dtype) {
+        case LQ_F32: hipLaunchKernelGGL((load_lora_kernel<F32Tag>), dim3(blocks), dim3(256), 0, st, dst, src, n, alpha); break;
+        case LQ_F16: hipLaunchKernelGGL((load_lora_kernel<F16Tag>), dim3(blocks), dim3(256), 0, st, dst, src, n, alpha); break;
+        case LQ_BF16: hipLaunchKernelGGL((load_lora_kernel<BF16Tag>), dim3(blocks), dim3(256), 0, st, dst, src, n, alpha); break;
+        default: set_error("lq_load_lora: unsupported dtype %d", (int)dtype); return LQ_ERR_UNSUPPORTED;
+    }
+    return check_launch("lq_load_lora");
+}
 
 extern "C" int lq_lora_down(void* out, lq_dtype_t out_dtype, const void* x, const void* lora_down, lq_dtype_t dtype,
                             int m, int k, int rank, lq_stream_t stream) {

@@ -115,6 +115,30 @@ __global__ __launch_bounds__(256) void fp8_cast_kernel(uint8_t* __restrict__ dst
     }
 }
 
+// The same cast for a matrix whose rows are `src_ld` elements apart, written with rows `dst_ld` bytes apart: a block of
+// columns of a wider destination (the concatenated input of FLUX's single-block output projection).  cols % E == 0.
+template <typename Tag>
+__global__ __launch_bounds__(256) void fp8_cast_2d_kernel(uint8_t* __restrict__ dst, size_t dst_ld, const void* __restrict__ src,
+                                                          size_t src_ld, const float* __restrict__ scale, int invert,
+                                                          size_t rows, size_t cols) {
+    constexpr int E = Chunk16<Tag>::elems;
+    const float s = scale[0];
+    const float r = invert ? 1.0f / s : s;
+    const size_t cpr = cols / E, nchunks = rows * cpr;
+    for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < nchunks; c += (size_t)gridDim.x * blockDim.x) {
+        const size_t row = c / cpr, cc = c - row * cpr;
+        float v[16];
+        load_elems<Tag>(src, row * src_ld + cc * E, v);
+        u32 w[4];
+#pragma unroll
+        for (int i = 0; i < E / 4; ++i)
+            w[i] = cvt4_e4m3(v[4 * i] * r, v[4 * i + 1] * r, v[4 * i + 2] * r, v[4 * i + 3] * r);
+        uint8_t* o = dst + row * dst_ld + cc * E;
+        if constexpr (E == 16) *reinterpret_cast<uint4*>(o) = make_uint4(w[0], w[1], w[2], w[3]);
+        else *reinterpret_cast<uint2*>(o) = make_uint2(w[0], w[1]);
+    }
+}
+
 // scalar fallback for unaligned buffers
 template <typename Tag>
 __global__ __launch_bounds__(256) void fp8_cast_scalar_kernel(uint8_t* __restrict__ dst, const void* __restrict__ src,
@@ -381,6 +405,24 @@ extern "C" int lq_fp8_scale_cast(uint8_t* dst, const void* src, lq_dtype_t dtype
         case LQ_F32: return launch_cast<F32Tag>(dst, src, scale, invert, n, as_stream(stream));
         default: set_error("lq_fp8_scale_cast: unsupported dtype %d", (int)dtype); return LQ_ERR_UNSUPPORTED;
     }
+}
+
+extern "C" int lq_fp8_scale_cast_2d(uint8_t* dst, size_t dst_ld, const void* src, size_t src_ld, lq_dtype_t dtype,
+                                    const float* scale, int invert, size_t rows, size_t cols, lq_stream_t stream) {
+    LQ_REQUIRE(scale && ((dst && src) || rows * cols == 0), LQ_ERR_ARG, "lq_fp8_scale_cast_2d: null pointer");
+    LQ_REQUIRE(dtype == LQ_F16 || dtype == LQ_BF16 || dtype == LQ_F32, LQ_ERR_UNSUPPORTED, "lq_fp8_scale_cast_2d: unsupported dtype %d", (int)dtype);
+    const size_t esz = dtype == LQ_F32 ? 4 : 2, e = dtype == LQ_F32 ? 8 : 16;
+    LQ_REQUIRE(cols % 16 == 0 && dst_ld >= cols && src_ld >= cols && dst_ld % 16 == 0 && (src_ld * esz) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(dst) % 16 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0,
+               LQ_ERR_SHAPE, "lq_fp8_scale_cast_2d: cols and both row pitches must keep every row 16-byte aligned (cols=%zu dst_ld=%zu src_ld=%zu)",
+               cols, dst_ld, src_ld);
+    if (rows * cols == 0) return LQ_OK;
+    const unsigned grid = stream_grid(rows * cols, (int)e);
+    hipStream_t st = as_stream(stream);
+    if (dtype == LQ_F16) hipLaunchKernelGGL((fp8_cast_2d_kernel<F16Tag>), dim3(grid), dim3(256), 0, st, dst, dst_ld, src, src_ld, scale, invert, rows, cols);
+    else if (dtype == LQ_BF16) hipLaunchKernelGGL((fp8_cast_2d_kernel<BF16Tag>), dim3(grid), dim3(256), 0, st, dst, dst_ld, src, src_ld, scale, invert, rows, cols);
+    else hipLaunchKernelGGL((fp8_cast_2d_kernel<F32Tag>), dim3(grid), dim3(256), 0, st, dst, dst_ld, src, src_ld, scale, invert, rows, cols);
+    return check_launch("fp8_cast_2d");
 }
 
 extern "C" int lq_fp8_amax_cast(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t n,

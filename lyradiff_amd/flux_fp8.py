@@ -1,0 +1,100 @@
+"""The FP8 feed-forward halves of the reference's FLUX blocks, built from the quantized-linear kernels.
+
+Two reference call sequences are covered; attention itself (QKV/rotary/flash attention) is not part of the
+quantized-linear path and stays with the caller, who passes its output in.
+
+  FluxAttnPostFP8Processor<T>::forward   (layers/flux_attn_post_processor/FluxAttnPostFP8Processor.cc:93-240)
+      hidden = input + gate_msa * attn          invokeFusedGateAndResidual
+      norm   = adaLN(hidden, scale_mlp, shift_mlp)   invokeLayerNormWithShiftAndScale
+      q1     = e4m3(norm / s_in1)               invokeCudaD2DScaleCpyConvert
+      inner  = gelu(q1 . W1^T + b1)             GemmWithResidualAndBias (GELU_BIAS epilogue)
+      q2     = e4m3(inner / s_in2)              invokeCudaD2DScaleCpyConvert
+      ff     = q2 . W2^T + b2                   GemmWithResidualAndBias
+      out    = hidden + gate_mlp * ff           invokeFusedGateAndResidual
+    Seven launches and five 16-bit intermediate tensors there; three launches here, and only `hidden` is written
+    in 16 bits: (1) gate+residual+adaLN+cast, (2) GEMM whose epilogue emits q2 directly, (3) GEMM whose epilogue
+    applies the gate and the residual.
+
+  FluxSingleTransformerFP8Block<T>::forward, after the attention (layers/flux_single_transformer_block/
+  FluxSingleTransformerFP8Block.cc:209-290)
+      q1   = e4m3(norm_hidden / s_mlp)          invokeCudaD2DScaleCpyConvert
+      mlp  = q1 . Wm^T + bm                     GemmWithResidualAndBias
+      cat  = [attn, gelu(mlp)]                  invokeFusedCatAndGelu
+      q2   = e4m3(cat / s_out)                  invokeCudaD2DScaleCpyConvert
+      o    = q2 . Wo^T + bo                     GemmWithResidualAndBias
+      out  = input + gate * o                   invokeFusedGateAndResidual
+    Here: the mlp GEMM writes the codes of gelu(mlp) straight into the right-hand columns of q2, a strided cast
+    fills the left-hand (attention) columns, and the output GEMM applies gate and residual in its epilogue.
+
+`msa` tensors follow the reference's layout [n_chunks, B, D] (AdaFP8LayerNorm.cc:100-175): for the double block
+chunks 2..5 are gate_msa, shift_mlp, scale_mlp, gate_mlp; for the single block chunk 2 is the gate.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from . import ops
+from .weights import FP8Linear, load_fp8_linear
+
+
+@dataclass
+class FluxAttnPostFP8Weights:
+    gelu_proj: FP8Linear  # "net.0.proj": [4D, D]
+    ff_linear: FP8Linear  # "net.2":      [D, 4D]
+
+
+@dataclass
+class FluxSingleMlpFP8Weights:
+    proj_mlp: FP8Linear  # "proj_mlp": [mlp_scale*D, D]
+    proj_out: FP8Linear  # "proj_out": [D, (mlp_scale+1)*D]
+
+
+def load_flux_attn_post_fp8(src, prefix: str, dim: int, dtype=torch.bfloat16, device="cuda", keep_master: bool = False):
+    """Keys prefix + {"net.0.proj", "net.2"} + {".weight", ".bias", "_input_scale"}
+    (FluxAttnPostFP8ProcessorWeight.cc:70-89; the block passes prefix + "ff." / "ff_context.")."""
+    return FluxAttnPostFP8Weights(load_fp8_linear(src, prefix, "net.0.proj", 4 * dim, dim, dtype, device, keep_master),
+                                  load_fp8_linear(src, prefix, "net.2", dim, 4 * dim, dtype, device, keep_master))
+
+
+def load_flux_single_mlp_fp8(src, prefix: str, dim: int, mlp_scale: int = 4, dtype=torch.bfloat16, device="cuda",
+                             keep_master: bool = False):
+    """Keys prefix + {"proj_mlp", "proj_out"} + {".weight", ".bias", "_input_scale"}
+    (FluxSingleTransformerFP8BlockWeight.cc:94-121)."""
+    return FluxSingleMlpFP8Weights(
+        load_fp8_linear(src, prefix, "proj_mlp", mlp_scale * dim, dim, dtype, device, keep_master),
+        load_fp8_linear(src, prefix, "proj_out", dim, (mlp_scale + 1) * dim, dtype, device, keep_master))
+
+
+def flux_attn_post_fp8(x: torch.Tensor, attn_output: torch.Tensor, msa: torch.Tensor, w: FluxAttnPostFP8Weights,
+                       eps: float = 1e-6) -> torch.Tensor:
+    """x, attn_output [B, S, D]; msa [6, B, D] -> output [B, S, D] in three launches."""
+    b, s, d = x.shape
+    if tuple(msa.shape) != (6, b, d):
+        raise ValueError("msa must be [6, B, D]")
+    gate_msa, shift_mlp, scale_mlp, gate_mlp = msa[2], msa[3], msa[4], msa[5]
+    q1, hidden = ops.gate_residual_layernorm_mod_fp8(attn_output, gate_msa, x, scale_mlp, shift_mlp, w.gelu_proj.input_scale, eps)
+    q2 = ops.fp8_linear_codes(q1.view(b * s, d), w.gelu_proj.weight_rows32, w.gelu_proj.input_scale, w.gelu_proj.weight_scale,
+                              w.gelu_proj.bias, w.ff_linear.input_scale, gelu=1, round_dtype=x.dtype)
+    out = ops.fp8_linear_gated(q2, w.ff_linear.weight_rows32, w.ff_linear.input_scale, w.ff_linear.weight_scale,
+                               w.ff_linear.bias, gate_mlp, hidden.view(b * s, d), rows_per_gate=s)
+    return out.view(b, s, d)
+
+
+def flux_single_mlp_fp8(x: torch.Tensor, norm_hidden, attn_output: torch.Tensor, gate: torch.Tensor,
+                        w: FluxSingleMlpFP8Weights) -> torch.Tensor:
+    """x, attn_output [B, S, D]; gate [B, D] (chunk 2 of the single block's msa) -> output [B, S, D].
+    norm_hidden is either the 16-bit adaLN output [B, S, D] (cast here with proj_mlp's input scale) or its e4m3
+    codes for proj_mlp (uint8 [B, S, D], e.g. the second output of ops.layernorm_mod_fp8_dual)."""
+    b, s, d = x.shape
+    m = b * s
+    f = w.proj_mlp.weight_rows32.shape[0]
+    q1 = norm_hidden if norm_hidden.dtype == torch.uint8 else ops.fp8_scale_cast(norm_hidden, w.proj_mlp.input_scale)
+    q2 = torch.empty((m, d + f), dtype=torch.uint8, device=x.device)
+    ops.fp8_scale_cast_into(attn_output.view(m, d), w.proj_out.input_scale, q2, 0)
+    ops.fp8_linear_codes(q1.view(m, d), w.proj_mlp.weight_rows32, w.proj_mlp.input_scale, w.proj_mlp.weight_scale,
+                         w.proj_mlp.bias, w.proj_out.input_scale, gelu=2, round_dtype=x.dtype, out=q2, col_offset=d)
+    out = ops.fp8_linear_gated(q2, w.proj_out.weight_rows32, w.proj_out.input_scale, w.proj_out.weight_scale,
+                               w.proj_out.bias, gate, x.view(m, d), rows_per_gate=s)
+    return out.view(b, s, d)

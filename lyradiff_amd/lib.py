@@ -35,14 +35,20 @@ SYMBOLS = {
     "lq_gemm_int8": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _P]),
     "lq_gemm_fp8": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _P, _F, _I, _I, _I, _P]),
     "lq_gemm_fp8_ex": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _P, _F, _I, _I, _I, _P, _P, _P, _P]),
+    "lq_gemm_fp8_gated": (_I, [_P, _I, _P, _P, _P, _P, _P, _P, _Z, _P, _I, _I, _I, _P]),
+    "lq_gemm_fp8_codes": (_I, [_P, _Z, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "lq_fp8_scale_cast_2d": (_I, [_P, _Z, _P, _Z, _I, _P, _I, _Z, _Z, _P]),
     "lq_gemm_w4a4": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P]),
     "lq_col_absmax": (_I, [_P, _P, _I, _Z, _Z, _P]),
     "lq_smooth_vector": (_I, [_P, _P, _P, _P, _F, _Z, _P]),
     "lq_layernorm_int8": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _Z, _Z, _F, _P]),
     "lq_layernorm_mod_fp8": (_I, [_P, _P, _P, _P, _I, _P, _Z, _Z, _Z, _F, _P]),
+    "lq_layernorm_mod_fp8_dual": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _Z, _Z, _Z, _F, _P]),
+    "lq_gate_residual_layernorm_mod_fp8": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _P, _Z, _Z, _Z, _F, _P]),
     "lq_gemm_w4a4_lora": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
     "lq_lora_down": (_I, [_P, _I, _P, _P, _I, _I, _I, _I, _P]),
     "lq_cast_f32": (_I, [_P, _I, _P, _Z, _P]),
+    "lq_load_lora": (_I, [_P, _P, _I, _Z, _F, _P]),
     "lq_gemm_set_tactic": (_I, [_I, _I]),
     "lq_gemm_set_thread_tactic": (_I, [_I]),
     "lq_gemm_tactic_count": (_I, [_I]),

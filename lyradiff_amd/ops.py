@@ -197,6 +197,44 @@ def layernorm_mod_fp8(x, scale, shift, input_scale, eps: float = 1e-6):
     return q
 
 
+def layernorm_mod_fp8_dual(x, scale, shift, input_scale_a, input_scale_b, eps: float = 1e-6):
+    """layernorm_mod_fp8 for two consumers of the normalised tensor: returns (codes_a, codes_b)."""
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    _chk(scale, "scale", (x.dtype,))
+    _chk(shift, "shift", (x.dtype,))
+    _chk(input_scale_a, "input_scale_a", (torch.float32,))
+    _chk(input_scale_b, "input_scale_b", (torch.float32,))
+    if x.dim() != 3 or tuple(scale.shape) != (x.shape[0], x.shape[2]) or scale.shape != shift.shape:
+        raise ValueError("x must be [B,S,D] and scale, shift [B,D]")
+    qa = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    qb = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    _l.check(_l.load().lq_layernorm_mod_fp8_dual(_ptr(qa), _ptr(input_scale_a), _ptr(qb), _ptr(input_scale_b), _ptr(x),
+                                                 _ptr(scale), _ptr(shift), _DT[x.dtype], x.shape[0], x.shape[1], x.shape[2],
+                                                 float(eps), _stream()), "lq_layernorm_mod_fp8_dual")
+    return qa, qb
+
+
+def gate_residual_layernorm_mod_fp8(attn, gate, x, scale, shift, input_scale, eps: float = 1e-6, hidden_out=None):
+    """invokeFusedGateAndResidual + invokeLayerNormWithShiftAndScale + FP8 cast in one pass:
+    hidden = x + gate*attn (each op rounded to the tensor dtype), codes = e4m3(adaLN(hidden) / input_scale).
+    attn, x [B,S,D]; gate, scale, shift [B,D].  Returns (codes, hidden); hidden_out may be x itself."""
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    for name, t in (("attn", attn), ("gate", gate), ("scale", scale), ("shift", shift)):
+        _chk(t, name, (x.dtype,))
+    _chk(input_scale, "input_scale", (torch.float32,))
+    if x.dim() != 3 or attn.shape != x.shape or any(tuple(t.shape) != (x.shape[0], x.shape[2]) for t in (gate, scale, shift)):
+        raise ValueError("attn, x must be [B,S,D] and gate, scale, shift [B,D]")
+    if hidden_out is None:
+        hidden_out = torch.empty_like(x)
+    _chk(hidden_out, "hidden_out", (x.dtype,))
+    q = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    _l.check(_l.load().lq_gate_residual_layernorm_mod_fp8(_ptr(q), _ptr(hidden_out), _ptr(attn), _ptr(gate), _ptr(x), _ptr(scale),
+                                                          _ptr(shift), _DT[x.dtype], _ptr(input_scale), x.shape[0], x.shape[1],
+                                                          x.shape[2], float(eps), _stream()),
+             "lq_gate_residual_layernorm_mod_fp8")
+    return q, hidden_out
+
+
 # ---- FP8 -------------------------------------------------------------------------------------------
 
 def fp8_amax_scale(x, scale=None):
@@ -247,11 +285,16 @@ def w4a4_quant(x, smooth=None, scale_dtype=torch.float32, group: int = 64):
 
 # ---- weight repack ---------------------------------------------------------------------------------
 
-def repack_weight(w_bytes):
-    """[N, row_bytes] byte matrix (int8 / e4m3 codes / packed nibbles) -> rows32 layout, same size."""
+def repack_weight(w_bytes, out=None):
+    """[N, row_bytes] byte matrix (int8 / e4m3 codes / packed nibbles) -> rows32 layout, same size.
+    `out` (same shape and dtype, not w_bytes itself) receives the result when given."""
     _chk(w_bytes, "w", (torch.int8, torch.uint8))
     n, rb = w_bytes.shape
-    out = torch.empty_like(w_bytes)
+    if out is None:
+        out = torch.empty_like(w_bytes)
+    _chk(out, "out", (w_bytes.dtype,))
+    if out.shape != w_bytes.shape:
+        raise ValueError("out must have the shape of w")
     _l.check(_l.load().lq_repack_rows32(_ptr(out), _ptr(w_bytes), n, rb, _stream()), "lq_repack_rows32")
     return out
 
@@ -322,6 +365,82 @@ def fp8_linear(a_q, w_rows32, a_scale, b_scale, bias=None, gelu: bool = False, r
     if out_fp8_scale is None:
         return c
     return (c, c8) if want_output else c8
+
+
+def fp8_linear_gated(a_q, w_rows32, a_scale, b_scale, bias, gate, residual, rows_per_gate: int, out=None):
+    """FP8 GEMM + invokeFusedGateAndResidual: out = residual + gate[row // rows_per_gate] * (A.W^T*sa*sb + bias), with
+    the roundings of the unfused sequence.  gate [ceil(M/rows_per_gate), N], residual [M, N]; out may be residual."""
+    _chk(a_q, "a_q", (torch.uint8,))
+    _chk(w_rows32, "w_rows32", (torch.uint8,))
+    _chk(a_scale, "a_scale", (torch.float32,))
+    _chk(b_scale, "b_scale", (torch.float32,))
+    _chk(residual, "residual", _FLOATS)
+    _chk(gate, "gate", (residual.dtype,))
+    if bias is not None:
+        _chk(bias, "bias", (residual.dtype,))
+    m, k = a_q.shape
+    n = w_rows32.shape[0]
+    if w_rows32.shape[1] != k:
+        raise ValueError("K mismatch between activation and weight")
+    if residual.numel() != m * n or rows_per_gate <= 0 or gate.numel() != ((m + rows_per_gate - 1) // rows_per_gate) * n:
+        raise ValueError("residual must be [M,N] and gate [ceil(M/rows_per_gate), N]")
+    if out is None:
+        out = torch.empty((m, n), dtype=residual.dtype, device=a_q.device)
+    _chk(out, "out", (residual.dtype,))
+    _l.check(_l.load().lq_gemm_fp8_gated(_ptr(out), _DT[residual.dtype], _ptr(a_q), _ptr(w_rows32), _ptr(a_scale), _ptr(b_scale),
+                                         _ptr(bias), _ptr(gate), int(rows_per_gate), _ptr(residual), m, n, k, _stream()),
+             "lq_gemm_fp8_gated")
+    return out
+
+
+def fp8_linear_codes(a_q, w_rows32, a_scale, b_scale, bias, out_fp8_scale, gelu: int = 0, round_dtype=torch.bfloat16,
+                     out=None, col_offset: int = 0):
+    """FP8 GEMM that writes only e4m3 codes (static scale out_fp8_scale) of its optionally GELU'd output, into columns
+    [col_offset, col_offset+N) of `out` (uint8 [M, W], allocated [M, N] when None).  gelu: 0 none, 1 on the fp32 value,
+    2 on the value rounded to round_dtype first."""
+    _chk(a_q, "a_q", (torch.uint8,))
+    _chk(w_rows32, "w_rows32", (torch.uint8,))
+    _chk(a_scale, "a_scale", (torch.float32,))
+    _chk(b_scale, "b_scale", (torch.float32,))
+    _chk(out_fp8_scale, "out_fp8_scale", (torch.float32,))
+    if bias is not None:
+        _chk(bias, "bias", (round_dtype,))
+    m, k = a_q.shape
+    n = w_rows32.shape[0]
+    if w_rows32.shape[1] != k:
+        raise ValueError("K mismatch between activation and weight")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.uint8, device=a_q.device)
+    _chk(out, "out", (torch.uint8,))
+    if out.dim() != 2 or out.shape[0] != m or col_offset < 0 or col_offset + n > out.shape[1]:
+        raise ValueError("out must be [M, W] with col_offset + N <= W")
+    _l.check(_l.load().lq_gemm_fp8_codes(out.data_ptr() + col_offset, out.shape[1], _ptr(out_fp8_scale), _DT[round_dtype],
+                                         _ptr(a_q), _ptr(w_rows32), _ptr(a_scale), _ptr(b_scale), _ptr(bias), int(gelu), m, n, k,
+                                         _stream()), "lq_gemm_fp8_codes")
+    return out
+
+
+def fp8_scale_cast_into(x, scale, out, col_offset: int = 0, invert: bool = True):
+    """invokeCudaD2DScaleCpyConvert of x [M, C] into columns [col_offset, col_offset+C) of out (uint8 [M, W])."""
+    _chk(x, "x", _FLOATS)
+    _chk(scale, "scale", (torch.float32,))
+    _chk(out, "out", (torch.uint8,))
+    if x.dim() != 2 or out.dim() != 2 or out.shape[0] != x.shape[0] or col_offset < 0 or col_offset + x.shape[1] > out.shape[1]:
+        raise ValueError("x must be [M, C] and out [M, W] with col_offset + C <= W")
+    _l.check(_l.load().lq_fp8_scale_cast_2d(out.data_ptr() + col_offset, out.shape[1], _ptr(x), x.shape[1], _DT[x.dtype],
+                                            _ptr(scale), int(invert), x.shape[0], x.shape[1], _stream()), "lq_fp8_scale_cast_2d")
+    return out
+
+
+def load_lora(weight, lora, alpha: float):
+    """invokeLoadLora: weight += lora * alpha in the tensors' dtype, in place; returns weight."""
+    _chk(weight, "weight", _FLOATS)
+    _chk(lora, "lora", (weight.dtype,))
+    if lora.numel() != weight.numel():
+        raise ValueError("lora and weight must have the same number of elements")
+    _l.check(_l.load().lq_load_lora(_ptr(weight), _ptr(lora), _DT[weight.dtype], weight.numel(), float(alpha), _stream()),
+             "lq_load_lora")
+    return weight
 
 
 def w4a4_linear(a_words, w_rows32, sA, sB, bias=None, out_dtype=torch.bfloat16, group: int = 64, lora_act=None, lora_up=None):

@@ -89,6 +89,27 @@ class FP8Linear:
     weight_scale: torch.Tensor   # fp32 [1]
     input_scale: torch.Tensor    # fp32 [1]
     bias: Optional[torch.Tensor] = None
+    weight_h: Optional[torch.Tensor] = None  # host master copy of the 16-bit weight [N, K], kept for LoRA merges
+
+    def _requantise(self, w16: torch.Tensor) -> None:
+        self.weight_scale.zero_()
+        ops.fp8_amax_scale(w16, self.weight_scale)
+        ops.repack_weight(ops.fp8_scale_cast(w16, self.weight_scale), out=self.weight_rows32)
+
+    def load_lora(self, lora_weight: torch.Tensor, lora_scale: float) -> None:
+        """FP8LoraWeight::load_lora (interface/IFLoraWeight.h:100-112): master copy + lora_scale * delta in the
+        weight's dtype, new per-tensor scale, new codes; the codes tensor and the scale are updated in place."""
+        if self.weight_h is None:
+            raise RuntimeError("this linear was loaded without its 16-bit master copy (keep_master=False)")
+        w16 = self.weight_h.to(self.weight_rows32.device)
+        ops.load_lora(w16, lora_weight.to(device=w16.device, dtype=w16.dtype).reshape(w16.shape).contiguous(), lora_scale)
+        self._requantise(w16)
+
+    def clear_lora(self) -> None:
+        """FP8LoraWeight::clear_lora (IFLoraWeight.h:114-127): re-quantise the untouched master copy."""
+        if self.weight_h is None:
+            raise RuntimeError("this linear was loaded without its 16-bit master copy (keep_master=False)")
+        self._requantise(self.weight_h.to(self.weight_rows32.device))
 
     def forward(self, x: torch.Tensor, gelu: bool = False, residual=None, beta: float = 0.0, dynamic: bool = False) -> torch.Tensor:
         k = x.shape[-1]
@@ -133,16 +154,20 @@ def load_int8_linear(src, prefix: str, name: str, d_out: int, d_in: int, device=
                       get(prefix + name + ".pre_quant_scale", (d_in,), torch.float32).to(device), bias)
 
 
-def load_fp8_linear(src, prefix: str, name: str, d_out: int, d_in: int, dtype=torch.bfloat16, device="cuda") -> FP8Linear:
+def load_fp8_linear(src, prefix: str, name: str, d_out: int, d_in: int, dtype=torch.bfloat16, device="cuda",
+                    keep_master: bool = False) -> FP8Linear:
     """The 16-bit weight is quantised on the device as the reference does at load time: scale = max|w|/448
-    (invokeGetFP8WeightScale), codes = e4m3(w * (1/scale)) (invokeCudaD2DScaleCpyConvert)."""
+    (invokeGetFP8WeightScale), codes = e4m3(w * (1/scale)) (invokeCudaD2DScaleCpyConvert).  keep_master keeps the
+    16-bit weight on the host (the reference's `*_weight_h`) so that LoRA deltas can be merged and removed later."""
     get = _source(src)
-    w = get(prefix + name + ".weight", (d_out, d_in), dtype).to(device)
+    w_host = get(prefix + name + ".weight", (d_out, d_in), dtype)
+    w = w_host.to(device)
     scale = ops.fp8_amax_scale(w)
     codes = ops.fp8_scale_cast(w, scale)
     return FP8Linear(ops.repack_weight(codes), scale,
                      get(prefix + name + "_input_scale", (1,), torch.float32).to(device),
-                     get(prefix + name + ".bias", (d_out,), dtype).to(device))
+                     get(prefix + name + ".bias", (d_out,), dtype).to(device),
+                     w_host.detach().cpu().clone() if keep_master else None)
 
 
 def load_w4a4_linear(src, prefix: str, d_out: int, d_in: int, lora_rank: int = 32, has_bias: bool = False,

@@ -19,6 +19,8 @@ closed forms / exhaustive tables / brute force in tests/test_oracle_*.py:
   gelu_tanh_f32         torch.nn.functional.gelu(approximate="tanh")   (pinned to 2e-7 abs)
   fp8_gemm              fp64 evaluation (summation order is free in the
                         reference's closed-source cuBLASLt)            (pinned to tolerance)
+  gate_residual         exact rational arithmetic rounded once per op  (pinned)
+  cat_gelu              concatenation + the pinned gelu_tanh_f32        (pinned)
 
 The calibration that produces SmoothQuant `pre_quant_scale` in the reference lives in
 nvidia-modelopt (absent): parity unpinned, replaced by the closed form in smooth_vector().
@@ -483,6 +485,48 @@ def layernorm_mod_fp8(src, scale, shift, in_scale, rows_per_batch: int, dtype: s
     a = round_to(np.asarray(scale, dtype=F32)[b] + F32(1.0), dtype)
     y = round_to(round_to(a * n, dtype) + np.asarray(shift, dtype=F32)[b], dtype)
     return fp8_scale_cast(y, np.asarray(in_scale, dtype=F32).reshape(-1)[0], True)
+
+
+def gate_residual(x, gate, residual, rows_per_gate: int, dtype: str) -> np.ndarray:
+    """out = T( T(x * gate[b]) + residual ), b = row // rows_per_gate: the multiply and the add each round to T
+    (fuseGateAndResidual, kernels/flux_single_transformer_block/flux_single_transformer_kernels.cu:42-65, `mul` then
+    `add` on T2 pairs).  The product of two fp16/bf16 numbers is exact in fp32, and the fp32 sum of two such numbers
+    cannot land on a rounding tie of T unless it is exact, so fp32 arithmetic followed by one rounding to T equals
+    the exactly rounded T operations (checked against rational arithmetic in the tests)."""
+    x = np.asarray(x, dtype=F32)
+    b = np.arange(x.shape[0]) // rows_per_gate
+    g = np.asarray(gate, dtype=F32).reshape(-1, x.shape[1])[b]
+    return round_to(round_to(x * g, dtype) + np.asarray(residual, dtype=F32), dtype)
+
+
+def gate_residual_layernorm_mod_fp8(attn, gate, inp, scale, shift, in_scale, rows_per_batch: int, dtype: str,
+                                    eps: float = 1e-6):
+    """hidden = gate_residual(attn, gate, inp); codes = layernorm_mod_fp8(hidden, ...)
+    (FluxAttnPostFP8Processor.cc:112-140).  Returns (codes, hidden)."""
+    hidden = gate_residual(attn, gate, inp, rows_per_batch, dtype)
+    return layernorm_mod_fp8(hidden, scale, shift, in_scale, rows_per_batch, dtype, eps), hidden
+
+
+def cat_gelu(attn, mlp, dtype: str) -> np.ndarray:
+    """out[:, :Da] = attn, out[:, Da:] = T( gelu_tanh( f32(mlp) ) ) (fuseCatAndGelu,
+    flux_single_transformer_kernels.cu:9-40: GeluActivation<float2> on the T values widened to fp32)."""
+    attn = np.asarray(attn, dtype=F32)
+    return np.concatenate([attn, round_to(gelu_tanh_f32(np.asarray(mlp, dtype=F32)), dtype)], axis=1)
+
+
+def load_lora(weight, lora, alpha: float, dtype: str) -> np.ndarray:
+    """weight + lora * T(alpha) with the product and the sum each rounded to T (loadLora,
+    kernels/lora/load_lora.cu:6-14: `dst[tid] += src[tid] * tmp_lora` on T operands); fp32 is plain fp32 arithmetic."""
+    w, l = np.asarray(weight, dtype=F32), np.asarray(lora, dtype=F32)
+    a = round_to(F32(alpha), dtype)
+    return round_to(w + round_to(l * a, dtype), dtype)
+
+
+def fp8_requantise(weight16):
+    """Per-tensor re-quantisation of a merged weight (FP8LoraWeight::load_lora, interface/IFLoraWeight.h:100-112):
+    scale = max|w|/448, codes = e4m3(w * (1/scale)).  Returns (codes, scale)."""
+    s = fp8_scale(weight16)
+    return fp8_scale_cast(weight16, s, True), s
 
 
 def lora_down_f64(x, down) -> np.ndarray:

@@ -25,3 +25,14 @@ def test_cpp_layer_types(dev):
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
     assert r.stdout.count("0 mismatches") == 2 and r.stdout.count(": yes") == 2 and "0 outliers" in r.stdout
+
+
+def test_cpp_flux_fp8_types(dev):
+    """FluxAttnPostFP8Processor / FluxSingleTransformerFP8Mlp / FP8LoraWeight (include/lyradiff_layers.h): each fused
+    forward equals the reference's launch sequence run step by step, bit for bit."""
+    exe = os.path.join(ROOT, "tests", "cpp", "flux_fp8_check")
+    assert os.path.exists(exe), "build it with `python -m lyradiff_amd.build` (prebuilt binaries travel to the GPU box)"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    print(r.stdout, r.stderr)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.count(" 0 mismatches") == 3

@@ -354,3 +354,65 @@ def test_low_rank_oracle():
     y = O.w4a4_gemm_lora_f64(y32, act, up, bias, "f32")
     assert np.allclose(y, y32 + np.einsum("mr,nr->mn", act, up) + bias[None, :], rtol=1e-6, atol=1e-6)
     assert np.array_equal(O.w4a4_gemm_lora_f64(y32, act * 0, up, None, "f32"), y32)
+
+
+def _round_fraction_to(v, dtype):
+    """Exactly rounded (RNE) conversion of a rational number to bf16 / fp16, by search over the two neighbours."""
+    from fractions import Fraction
+
+    if v == 0:
+        return 0.0
+    f = np.float32(float(v))  # within one fp32 ulp of v; the T neighbours of v are among the T values around f
+    base = O.round_to(np.float32(f), dtype)
+    bits = 16 if dtype == "bf16" else 13  # fp32 mantissa bits below T's last place
+    cands = set()
+    u0 = int(np.asarray(base, np.float32).reshape(1).view(np.uint32)[0])
+    for d in (-1, 0, 1):
+        cands.add(float(np.array([u0 + d * (1 << bits)], np.uint32).view(np.float32)[0]))
+    best = min(cands, key=lambda c: (abs(Fraction(c) - v), int(np.array([c], np.float32).view(np.uint32)[0] >> bits) & 1))
+    return best
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_gate_residual_oracle_vs_rational_arithmetic(dtype):
+    from fractions import Fraction
+
+    rng = np.random.default_rng(31)
+    m, n, rpg = 6, 24, 3
+    x = O.round_to((rng.standard_normal((m, n)) * 3).astype(np.float32), dtype)
+    g = O.round_to(rng.standard_normal((2, n)).astype(np.float32), dtype)
+    r = O.round_to((rng.standard_normal((m, n)) * 3).astype(np.float32), dtype)
+    # widely separated magnitudes (inexact fp32 sums) and exact ties of the product
+    x[0, :4] = O.round_to(np.array([1.0 + 2.0 ** -7, 3.0, 2.0 ** -12, -(1.0 + 2.0 ** -7)], np.float32), dtype)
+    g[0, :4] = O.round_to(np.array([1.0 + 2.0 ** -7, 2.0 ** -9, 1.0, 1.0 + 2.0 ** -6], np.float32), dtype)
+    r[0, :4] = O.round_to(np.array([256.0, 1.0, 1024.0, 2.0 ** -10], np.float32), dtype)
+    out = O.gate_residual(x, g, r, rpg, dtype)
+    for i in range(m):
+        for j in range(n):
+            prod = _round_fraction_to(Fraction(float(x[i, j])) * Fraction(float(g[i // rpg, j])), dtype)
+            want = _round_fraction_to(Fraction(prod) + Fraction(float(r[i, j])), dtype)
+            assert float(out[i, j]) == want, (i, j)
+    # closed forms: a unit gate is a plain rounded sum, a zero gate returns the residual, rows pick their own gate
+    one = np.ones((2, n), np.float32)
+    assert np.array_equal(O.gate_residual(x, one, r, rpg, dtype), O.round_to(x + r, dtype))
+    assert np.array_equal(O.gate_residual(x, one * 0, r, rpg, dtype), r)
+    assert not np.array_equal(out, O.gate_residual(x, g[::-1], r, rpg, dtype))
+    assert np.array_equal(O.gate_residual(-x, g, -r, rpg, dtype), -out)
+
+
+def test_cat_gelu_and_fused_gate_layernorm_oracle():
+    rng = np.random.default_rng(32)
+    attn = O.round_to(rng.standard_normal((5, 16)).astype(np.float32), "bf16")
+    mlp = O.round_to((rng.standard_normal((5, 64)) * 2).astype(np.float32), "bf16")
+    c = O.cat_gelu(attn, mlp, "bf16")
+    assert c.shape == (5, 80) and np.array_equal(c[:, :16], attn)
+    ref = torch.nn.functional.gelu(torch.from_numpy(mlp).double(), approximate="tanh").numpy()
+    assert np.all(np.abs(c[:, 16:] - ref) <= 2.0 ** -8 * np.abs(ref) + 1e-6)
+    assert np.array_equal(O.cat_gelu(attn, mlp * 0, "bf16")[:, 16:], np.zeros((5, 64), np.float32))
+    # the fused form is the composition of its two pinned parts, and the hidden state it returns is the gate/residual sum
+    x = O.round_to(rng.standard_normal((6, 64)).astype(np.float32), "bf16")
+    a = O.round_to(rng.standard_normal((6, 64)).astype(np.float32), "bf16")
+    g, sc, sh = (O.round_to((rng.standard_normal((2, 64)) * 0.5).astype(np.float32), "bf16") for _ in range(3))
+    q, h = O.gate_residual_layernorm_mod_fp8(a, g, x, sc, sh, [0.03], 3, "bf16")
+    assert np.array_equal(h, O.gate_residual(a, g, x, 3, "bf16"))
+    assert np.array_equal(q, O.layernorm_mod_fp8(h, sc, sh, [0.03], 3, "bf16"))
