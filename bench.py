@@ -266,7 +266,63 @@ def extra_kernels(torch, ops, dev):
     pre = (torch.rand(d, generator=g) + 0.5).to(dev)
     us = timeit(lambda: ops.geglu_int8_dynamic(x, b, pre))
     res[f"geglu_int8_{m}x{d}"] = {"us": round(us, 2), "GB/s": round(5.0 * m * d / us / 1e3, 1)}
+    res.update(flux_block_times(torch, ops, dev, timeit))
     return res
+
+
+def flux_block_times(torch, ops, dev, timeit):
+    """FP8 feed-forward halves of the FLUX blocks at 1024x1024 (4608 tokens, d=3072): the fused three-launch forms
+    against the reference's launch sequence run step by step with this library's unfused kernels (torch for the two
+    elementwise gate/residual steps), same operands, bit-identical outputs."""
+    from lyradiff_amd import flux_fp8 as F
+
+    g = torch.Generator().manual_seed(77)
+    b, s, d = 1, 4608, 3072
+    bf = lambda *shape, sc=1.0: (sc * torch.randn(*shape, generator=g)).bfloat16()
+    sd = {"p.net.0.proj.weight": bf(4 * d, d, sc=0.02), "p.net.0.proj.bias": bf(4 * d, sc=0.1),
+          "p.net.2.weight": bf(d, 4 * d, sc=0.02), "p.net.2.bias": bf(d, sc=0.1),
+          "p.net.0.proj_input_scale": torch.tensor([5.0 / 448]), "p.net.2_input_scale": torch.tensor([2.0 / 448]),
+          "p.proj_mlp.weight": bf(4 * d, d, sc=0.02), "p.proj_mlp.bias": bf(4 * d, sc=0.1),
+          "p.proj_out.weight": bf(d, 5 * d, sc=0.02), "p.proj_out.bias": bf(d, sc=0.1),
+          "p.proj_mlp_input_scale": torch.tensor([5.0 / 448]), "p.proj_out_input_scale": torch.tensor([4.0 / 448])}
+    wp = F.load_flux_attn_post_fp8(sd, "p.", d, torch.bfloat16, dev)
+    ws = F.load_flux_single_mlp_fp8(sd, "p.", d, 4, torch.bfloat16, dev)
+    x, attn, norm = bf(b, s, d).to(dev), bf(b, s, d).to(dev), bf(b, s, d).to(dev)
+    msa = bf(6, b, d, sc=0.5).to(dev)
+    for kind, (n, k) in (("fp8", (4 * d, d)), ("fp8", (d, 4 * d)), ("fp8", (d, 5 * d))):
+        ops.gemm_profile(kind, b * s, n, k, dev)
+
+    def post_unfused():
+        hidden = x + msa[2][:, None, :] * attn
+        q1 = ops.layernorm_mod_fp8(hidden, msa[4], msa[3], wp.gelu_proj.input_scale)
+        inner = ops.fp8_linear(q1.view(b * s, d), wp.gelu_proj.weight_rows32, wp.gelu_proj.input_scale, wp.gelu_proj.weight_scale,
+                               wp.gelu_proj.bias, True, None, 0.0, torch.bfloat16)
+        q2 = ops.fp8_scale_cast(inner, wp.ff_linear.input_scale)
+        ff = ops.fp8_linear(q2, wp.ff_linear.weight_rows32, wp.ff_linear.input_scale, wp.ff_linear.weight_scale, wp.ff_linear.bias,
+                            False, None, 0.0, torch.bfloat16)
+        return hidden + msa[5][:, None, :] * ff.view(b, s, d)
+
+    def single_unfused():
+        q1 = ops.fp8_scale_cast(norm, ws.proj_mlp.input_scale)
+        mlp = ops.fp8_linear(q1.view(b * s, d), ws.proj_mlp.weight_rows32, ws.proj_mlp.input_scale, ws.proj_mlp.weight_scale,
+                             ws.proj_mlp.bias, False, None, 0.0, torch.bfloat16)
+        cat = torch.cat([attn.view(b * s, d), torch.nn.functional.gelu(mlp.float(), approximate="tanh").bfloat16()], dim=1)
+        q2 = ops.fp8_scale_cast(cat, ws.proj_out.input_scale)
+        o = ops.fp8_linear(q2, ws.proj_out.weight_rows32, ws.proj_out.input_scale, ws.proj_out.weight_scale, ws.proj_out.bias,
+                           False, None, 0.0, torch.bfloat16)
+        return x + msa[2][:, None, :] * o.view(b, s, d)
+
+    same = bool(torch.equal(F.flux_attn_post_fp8(x, attn, msa, wp), post_unfused()))
+    flops_post, flops_single = 2.0 * b * s * 8 * d * d, 2.0 * b * s * 9 * d * d
+    out = {}
+    for name, fn, fl in (("flux_attn_post_fp8_fused_3_launches", lambda: F.flux_attn_post_fp8(x, attn, msa, wp), flops_post),
+                         ("flux_attn_post_fp8_reference_sequence_7_launches", post_unfused, flops_post),
+                         ("flux_single_mlp_fp8_fused_3_launches", lambda: F.flux_single_mlp_fp8(x, norm, attn, msa[2], ws), flops_single),
+                         ("flux_single_mlp_fp8_reference_sequence_7_launches", single_unfused, flops_single)):
+        us = timeit(fn, iters=20, warm=3)
+        out[name] = {"us": round(us, 2), "TFLOP/s": round(fl / us / 1e6, 1)}
+    out["flux_attn_post_fp8_fused_equals_sequence"] = same
+    return out
 
 
 if __name__ == "__main__":
