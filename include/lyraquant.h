@@ -280,6 +280,14 @@ int lq_gate_residual_layernorm_mod_fp8(uint8_t* dst, void* hidden_out, const voi
                                        const float* input_scale, size_t batch, size_t rows_per_batch, size_t dim,
                                        float eps, lq_stream_t stream);
 
+/* The same without a quantisation: dst = T( adaLN(hidden) ), for the W4A4 linears, which quantise per group of 64 and
+ * also feed the 16-bit tensor to their low-rank branch (layers/flux_attn_post_processor/
+ * FluxAttnPostInt4Processor.cc:118-150).  attn, gate and hidden_out are all NULL for a plain
+ * invokeLayerNormWithShiftAndScale of `input` (kernels/norms/layer_norm.h:18-27). */
+int lq_gate_residual_layernorm_mod(void* dst, void* hidden_out, const void* attn, const void* gate, const void* input,
+                                   const void* scale, const void* shift, lq_dtype_t dtype, size_t batch,
+                                   size_t rows_per_batch, size_t dim, float eps, lq_stream_t stream);
+
 /* W4A4 GEMM with the SVDQuant low-rank branch of invokeFusedW4A4GemmAndLoraUp
  * (kernels/w4a4_gemm/w4a4_gemm.h:18-30; lora_up_gemm, kernels/w4a4_gemm/w4a4_gemm.cu:514-663):
  *   C = T( sum_g f32(p_g) * sA * sB  +  sum_r lora_act[m, r] * lora_up[n, r]  [+ bias[n]] ),
@@ -291,6 +299,35 @@ int lq_gemm_w4a4_lora(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, co
                       const void* sA, const void* sB, lq_dtype_t scale_dtype, const void* bias,
                       const void* lora_act, const void* lora_up, lq_dtype_t lora_dtype, int lora_rank,
                       int m, int n, int k, int group, lq_stream_t stream);
+
+/* Epilogue options of lq_gemm_w4a4_ex, applied in this order to y = acc [+ low-rank] [+ bias] (fp32):
+ *   gelu     0 none; 1 tanh-GELU of y; 2 tanh-GELU of T(y) (invokeFusedBiasAndGelu on a stored GEMM output,
+ *            kernels/flux_single_transformer_block/flux_single_transformer_kernels.cu:122-141,194-201)
+ *   addend   y = T( T(y) + addend[m,n] ): joins another linear's stored output (invokeFusedBiasAndResidual,
+ *            flux_single_transformer_kernels.cu:67-93; FluxSingleTransformerInt4Block.cc:297-305)
+ *   gate + residual   y = T( T( T(y) * gate[m / rows_per_gate, n] ) + residual[m,n] ) (invokeFusedGateAndResidual)
+ *   C_fp8    e4m3( f32(T(y)) / C_fp8_scale[0] ) into rows ldc_fp8 bytes apart, next to or instead of C
+ *            (invokeCudaD2DScaleCpyConvert in front of the FP8 ff_linear, FluxAttnPostInt4Processor.cc:167-173)
+ * All pointers optional (NULL = step skipped); tensors have the output dtype. */
+typedef struct lq_epilogue {
+    int gelu;
+    const void* addend;
+    const void* gate;
+    size_t rows_per_gate;
+    const void* residual;
+    uint8_t* C_fp8;
+    size_t ldc_fp8;
+    const float* C_fp8_scale;
+} lq_epilogue_t;
+
+/* lq_gemm_w4a4_lora with the epilogue options above (epi may be NULL; C may be NULL when epi->C_fp8 is given):
+ * the W4A4 linears of the FLUX INT4 blocks followed by their bias/GELU, residual, gate and FP8 re-quantisation
+ * kernels (layers/flux_attn_post_processor/FluxAttnPostInt4Processor.cc:155-205,
+ * layers/flux_single_transformer_block/FluxSingleTransformerInt4Block.cc:260-316). */
+int lq_gemm_w4a4_ex(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const uint8_t* B_rows32,
+                    const void* sA, const void* sB, lq_dtype_t scale_dtype, const void* bias,
+                    const void* lora_act, const void* lora_up, lq_dtype_t lora_dtype, int lora_rank,
+                    int m, int n, int k, int group, const lq_epilogue_t* epi, lq_stream_t stream);
 
 /* Down projection of the low-rank branch, the second half of invokeFusedQuantizeAndLoraDownSimple
  * (kernels/w4a4_gemm/w4a4_gemm.h:6-16; kernels/w4a4_gemm/w4a4_gemm.cu:931-953):

@@ -42,6 +42,7 @@ struct GemmParams {
     // fp8
     const float* a_scale;
     const float* b_scale;
+    // fp8 and w4a4: activation, residual, re-quantisation and gate epilogues
     int gelu;
     const void* residual;
     float beta;
@@ -55,6 +56,9 @@ struct GemmParams {
     // followed by an elementwise multiply and add in T; requires residual, ignores beta
     const void* gate;
     size_t gate_rows;
+    // addend (optional, [m, n] of T): y = T( T(y) + addend ) before the gate/residual step -- the sum of two linears'
+    // outputs as the reference forms it with invokeFusedBiasAndResidual
+    const void* addend;
     // w4a4
     const void* sA;
     const void* sB;
@@ -571,10 +575,12 @@ struct GemmKernel {
         float alpha = 1.0f, bias4[4] = {0.f, 0.f, 0.f, 0.f}, acol4[4] = {0.f, 0.f, 0.f, 0.f}, arow_l[MT];
         float out_amax = 0.0f, c8_inv = 0.0f, gate4[4] = {0.f, 0.f, 0.f, 0.f};
         bool gate_uniform = true;  // every row of the wavefront's tile uses the same gate vector
-        if constexpr (KIND == K_FP8) {
-            alpha = p.a_scale[0] * p.b_scale[0];
+        // the FP8 and W4A4 linears of the FLUX blocks share the activation / re-quantisation / gate epilogues
+        constexpr bool kExtras = (KIND == K_FP8 || W4) && !kI32;
+        if constexpr (KIND == K_FP8) alpha = p.a_scale[0] * p.b_scale[0];
+        if constexpr (kExtras) {
             if (p.C8 != nullptr) c8_inv = 1.0f / p.c8_scale[0];
-            if constexpr (!kI32) {
+            {
                 if (p.gate != nullptr) {
                     const size_t r_first = (size_t)(m0 + wm * TM), r_last = (size_t)min(m0 + wm * TM + TM - 1, p.m - 1);
                     const size_t b_first = r_first / p.gate_rows;
@@ -645,14 +651,20 @@ struct GemmKernel {
                         for (int e = 0; e < 4; ++e) {
                             y[e] = (KIND == K_FP8) ? vf[e] * alpha : vf[e];
                             if (p.bias != nullptr) y[e] = y[e] + bias4[e];
-                            if constexpr (KIND == K_FP8) {
+                            if constexpr (kExtras) {
                                 if (p.gelu) {
                                     if (p.gelu == 2) y[e] = round_through<OutTag>(y[e]);
                                     y[e] = gelu_fast(y[e]);
                                 }
                             }
                         }
-                        if constexpr (KIND == K_FP8) {
+                        if constexpr (kExtras) {
+                            if (p.addend != nullptr && ok) {  // T( T(y) + addend ): a second linear's output joined in T
+                                float aa[4];
+                                OutStore<OutTag>::load4(p.addend, idx, aa);
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) y[e] = round_through<OutTag>(round_through<OutTag>(y[e]) + aa[e]);
+                            }
                             if (p.residual != nullptr && ok) {
                                 float rr[4];
                                 OutStore<OutTag>::load4(p.residual, idx, rr);
@@ -668,7 +680,7 @@ struct GemmKernel {
                             }
                         }
                     }
-                    if constexpr (KIND == K_FP8) {
+                    if constexpr (kExtras) {
                         if (ok) {
                             if (p.out_scale != nullptr)
                                 out_amax = fmaxf(fmaxf(out_amax, fmaxf(fabsf(y[0]), fabsf(y[1]))), fmaxf(fabsf(y[2]), fabsf(y[3])));
@@ -684,7 +696,7 @@ struct GemmKernel {
                 }
             }
         }
-        if constexpr (KIND == K_FP8 && !kI32) {
+        if constexpr (kExtras) {
             // Rounding to T is monotone, so the maximum of the rounded outputs is the rounded maximum; so is the
             // division by 448: the scale published here is exactly what an amax pass over C would produce.
             if (p.out_scale != nullptr) {

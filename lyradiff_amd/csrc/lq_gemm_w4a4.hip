@@ -28,11 +28,23 @@ template <int KIND, typename OutTag> static int run_w4a4(GemmParams p, hipStream
 
 using namespace lq;
 
-extern "C" int lq_gemm_w4a4_lora(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const uint8_t* B_rows32,
-                                 const void* sA, const void* sB, lq_dtype_t scale_dtype, const void* bias,
-                                 const void* lora_act, const void* lora_up, lq_dtype_t lora_dtype, int lora_rank, int m,
-                                 int n, int k, int group, lq_stream_t stream) {
-    LQ_REQUIRE(C && A_words && B_rows32 && sA && sB, LQ_ERR_ARG, "lq_gemm_w4a4: null pointer");
+extern "C" int lq_gemm_w4a4_ex(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const uint8_t* B_rows32,
+                               const void* sA, const void* sB, lq_dtype_t scale_dtype, const void* bias,
+                               const void* lora_act, const void* lora_up, lq_dtype_t lora_dtype, int lora_rank, int m,
+                               int n, int k, int group, const lq_epilogue_t* epi, lq_stream_t stream) {
+    LQ_REQUIRE((C || (epi && epi->C_fp8)) && A_words && B_rows32 && sA && sB, LQ_ERR_ARG, "lq_gemm_w4a4: null pointer");
+    if (epi != nullptr) {
+        LQ_REQUIRE(epi->gelu >= 0 && epi->gelu <= 2, LQ_ERR_ARG, "lq_gemm_w4a4: gelu must be 0, 1 or 2");
+        LQ_REQUIRE((epi->gate == nullptr) == (epi->residual == nullptr), LQ_ERR_ARG, "lq_gemm_w4a4: gate and residual go together");
+        LQ_REQUIRE(epi->gate == nullptr || epi->rows_per_gate > 0, LQ_ERR_SHAPE, "lq_gemm_w4a4: rows_per_gate must be positive");
+        LQ_REQUIRE((epi->C_fp8 == nullptr) == (epi->C_fp8_scale == nullptr), LQ_ERR_ARG, "lq_gemm_w4a4: C_fp8 and C_fp8_scale go together");
+        LQ_REQUIRE(epi->C_fp8 == nullptr || (epi->ldc_fp8 >= (size_t)(n > 0 ? n : 0) && epi->ldc_fp8 % 4 == 0 &&
+                                             reinterpret_cast<uintptr_t>(epi->C_fp8) % 4 == 0),
+                   LQ_ERR_SHAPE, "lq_gemm_w4a4: need ldc_fp8 >= n, ldc_fp8 %% 4 == 0 and a 4-byte aligned C_fp8");
+        LQ_REQUIRE(reinterpret_cast<uintptr_t>(epi->gate) % 16 == 0 && reinterpret_cast<uintptr_t>(epi->residual) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(epi->addend) % 16 == 0,
+                   LQ_ERR_ARG, "lq_gemm_w4a4: gate, residual and addend must be 16-byte aligned");
+    }
     LQ_REQUIRE(group == 64, LQ_ERR_SHAPE, "lq_gemm_w4a4: group=%d, only 64 is supported", group);
     LQ_REQUIRE(scale_dtype == LQ_F32 || scale_dtype == LQ_F16, LQ_ERR_UNSUPPORTED,
                "lq_gemm_w4a4: scale dtype must be F32 or F16");
@@ -57,6 +69,13 @@ extern "C" int lq_gemm_w4a4_lora(void* C, lq_dtype_t out_dtype, const uint32_t* 
     p.C = C; p.A = reinterpret_cast<const uint8_t*>(A_words); p.B = B_rows32; p.bias = bias;
     p.sA = sA; p.sB = sB; p.scale_f16 = scale_dtype == LQ_F16;
     p.lora_act = lora_act; p.lora_up = lora_up; p.lora_rank = lora_rank; p.lora_f16 = lora_dtype == LQ_F16;
+    p.ldc8 = (size_t)n;
+    if (epi != nullptr) {
+        p.gelu = epi->gelu; p.addend = epi->addend; p.gate = epi->gate; p.gate_rows = epi->rows_per_gate;
+        p.residual = epi->residual; p.beta = 1.0f;
+        p.C8 = epi->C_fp8; p.c8_scale = epi->C_fp8_scale;
+        if (epi->C_fp8 != nullptr) p.ldc8 = epi->ldc_fp8;
+    }
     p.m = m; p.n = n; p.k = k; p.kb = k / 2;
     hipStream_t st = as_stream(stream);
     switch (out_dtype) {
@@ -65,6 +84,15 @@ extern "C" int lq_gemm_w4a4_lora(void* C, lq_dtype_t out_dtype, const uint32_t* 
         case LQ_F32: return p.scale_f16 ? run_w4a4<K_W4A4H, F32Tag>(p, st) : run_w4a4<K_W4A4, F32Tag>(p, st);
         default: set_error("lq_gemm_w4a4: unsupported output dtype %d", (int)out_dtype); return LQ_ERR_UNSUPPORTED;
     }
+}
+
+extern "C" int lq_gemm_w4a4_lora(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const uint8_t* B_rows32,
+                                 const void* sA, const void* sB, lq_dtype_t scale_dtype, const void* bias,
+                                 const void* lora_act, const void* lora_up, lq_dtype_t lora_dtype, int lora_rank, int m,
+                                 int n, int k, int group, lq_stream_t stream) {
+    LQ_REQUIRE(C != nullptr, LQ_ERR_ARG, "lq_gemm_w4a4: null pointer");
+    return lq_gemm_w4a4_ex(C, out_dtype, A_words, B_rows32, sA, sB, scale_dtype, bias, lora_act, lora_up, lora_dtype, lora_rank, m, n,
+                           k, group, nullptr, stream);
 }
 
 extern "C" int lq_gemm_w4a4(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, const uint8_t* B_rows32,

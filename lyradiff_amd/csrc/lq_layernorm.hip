@@ -37,7 +37,8 @@ __device__ __forceinline__ u32 ln_nan_fix(u32 w, const float* y) {  // NaN -> 0x
     return w;
 }
 
-// QMODE 0: int8, static per-tensor scale; 1: int8, dynamic per-token scale (written to scale_out); 2: fp8, static scale.
+// QMODE 0: int8, static per-tensor scale; 1: int8, dynamic per-token scale (written to scale_out); 2: fp8, static scale;
+// 3: no quantisation, y stored as T (the input of a W4A4 linear, which quantises per group and also feeds its low-rank branch).
 // MOD false: y = gamma*n + beta (vectors of length dim).  MOD true: y = (1 + scale[b])*n + shift[b], b = row / rows_per_batch.
 // RESID 0: h = src.  1: h = T(T(src + residual) + bias).  2: h = T(T(src * gate[b]) + residual), gate passed as `bias`.
 template <typename Tag, int NP, int QMODE, int RESID, bool MOD>
@@ -127,7 +128,7 @@ __global__ __launch_bounds__(256) void ln_quant_rows_kernel(uint8_t* __restrict_
                 }
                 h[p][i] = y;
             }
-            if constexpr (QMODE != 2) {
+            if constexpr (QMODE < 2) {
                 if (pre != nullptr) {
                     float4 a = *reinterpret_cast<const float4*>(pre + col);
                     float4 c = *reinterpret_cast<const float4*>(pre + col + 4);
@@ -148,10 +149,22 @@ __global__ __launch_bounds__(256) void ln_quant_rows_kernel(uint8_t* __restrict_
         s = amax / 127.0f;
         if (amax <= 5.9604644775390625e-08f) s = 1.0f;
         if (lane == 0) scale_out[row] = s;
-    } else {
+    } else if constexpr (QMODE != 3) {
         s = in_scale[0];
     }
-    if constexpr (QMODE == 2) {
+    if constexpr (QMODE == 3) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int col = (p * 64 + lane) * 8;
+            if (col < dim) {
+                uint4 o;
+                u32* ow = reinterpret_cast<u32*>(&o);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) ow[i] = Elem<Tag>::store(h[p][2 * i]) | (Elem<Tag>::store(h[p][2 * i + 1]) << 16);
+                *reinterpret_cast<uint4*>(reinterpret_cast<unsigned short*>(dst) + row_off + col) = o;
+            }
+        }
+    } else if constexpr (QMODE == 2) {
         // one set of codes per consumer of the normalised tensor (each linear has its own calibrated input scale)
         const int nout = dst_b != nullptr ? 2 : 1;
         for (int o2 = 0; o2 < nout; ++o2) {
@@ -290,6 +303,31 @@ extern "C" int lq_layernorm_mod_fp8_dual(uint8_t* dst_a, const float* input_scal
                 batch * rows_per_batch, (int)dim, rows_per_batch, eps};
     hipStream_t st = as_stream(stream);
     return dtype == LQ_F16 ? launch_ln<F16Tag, 2, 0, true>(a, st) : launch_ln<BF16Tag, 2, 0, true>(a, st);
+}
+
+extern "C" int lq_gate_residual_layernorm_mod(void* dst, void* hidden_out, const void* attn, const void* gate, const void* input,
+                                             const void* scale, const void* shift, lq_dtype_t dtype, size_t batch,
+                                             size_t rows_per_batch, size_t dim, float eps, lq_stream_t stream) {
+    const bool gated = attn != nullptr;
+    int rc = check_ln_common("lq_gate_residual_layernorm_mod", dst, input, dtype, batch * rows_per_batch, dim);
+    if (rc != LQ_OK) return rc;
+    LQ_REQUIRE(scale && shift, LQ_ERR_ARG, "lq_gate_residual_layernorm_mod: scale and shift are required");
+    LQ_REQUIRE(gated == (gate != nullptr) && gated == (hidden_out != nullptr), LQ_ERR_ARG,
+               "lq_gate_residual_layernorm_mod: attn, gate and hidden_out go together");
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(scale) % 16 == 0 && reinterpret_cast<uintptr_t>(shift) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(gate) % 16 == 0 && reinterpret_cast<uintptr_t>(attn) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(hidden_out) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0,
+               LQ_ERR_ARG, "lq_gate_residual_layernorm_mod: all tensors must be 16-byte aligned");
+    if (batch * rows_per_batch == 0) return LQ_OK;
+    hipStream_t st = as_stream(stream);
+    if (gated) {
+        LnArgs a = {static_cast<uint8_t*>(dst), hidden_out, nullptr, attn, input, gate, scale, shift, nullptr, nullptr, nullptr, nullptr,
+                    batch * rows_per_batch, (int)dim, rows_per_batch, eps};
+        return dtype == LQ_F16 ? launch_ln<F16Tag, 3, 2, true>(a, st) : launch_ln<BF16Tag, 3, 2, true>(a, st);
+    }
+    LnArgs a = {static_cast<uint8_t*>(dst), nullptr, nullptr, input, nullptr, nullptr, scale, shift, nullptr, nullptr, nullptr, nullptr,
+                batch * rows_per_batch, (int)dim, rows_per_batch, eps};
+    return dtype == LQ_F16 ? launch_ln<F16Tag, 3, 0, true>(a, st) : launch_ln<BF16Tag, 3, 0, true>(a, st);
 }
 
 extern "C" int lq_gate_residual_layernorm_mod_fp8(uint8_t* dst, void* hidden_out, const void* attn, const void* gate,

@@ -45,6 +45,8 @@ SYMBOLS = {
     "lq_layernorm_mod_fp8": (_I, [_P, _P, _P, _P, _I, _P, _Z, _Z, _Z, _F, _P]),
     "lq_layernorm_mod_fp8_dual": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _Z, _Z, _Z, _F, _P]),
     "lq_gate_residual_layernorm_mod_fp8": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _P, _Z, _Z, _Z, _F, _P]),
+    "lq_gate_residual_layernorm_mod": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _Z, _Z, _Z, _F, _P]),
+    "lq_gemm_w4a4_ex": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P]),
     "lq_gemm_w4a4_lora": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
     "lq_lora_down": (_I, [_P, _I, _P, _P, _I, _I, _I, _I, _P]),
     "lq_cast_f32": (_I, [_P, _I, _P, _Z, _P]),
@@ -57,6 +59,14 @@ SYMBOLS = {
     "lq_gemm_profile_workspace": (_Z, [_I, _I, _I, _I]),
     "lq_gemm_profile": (_I, [_I, _I, _I, _I, _P, _Z, C.POINTER(_I), C.POINTER(_F), _P]),
 }
+
+
+
+class Epilogue(C.Structure):
+    """lq_epilogue_t of include/lyraquant.h."""
+    _fields_ = [("gelu", _I), ("addend", _P), ("gate", _P), ("rows_per_gate", _Z), ("residual", _P), ("C_fp8", _P),
+                ("ldc_fp8", _Z), ("C_fp8_scale", _P)]
+
 
 _lib = None
 

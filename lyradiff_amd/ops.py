@@ -8,6 +8,8 @@ torch.ops.lyradiff.* custom operators.
 """
 from __future__ import annotations
 
+import ctypes as C
+
 import torch
 
 from . import lib as _l
@@ -235,6 +237,32 @@ def gate_residual_layernorm_mod_fp8(attn, gate, x, scale, shift, input_scale, ep
     return q, hidden_out
 
 
+def gate_residual_layernorm_mod(x, scale, shift, attn=None, gate=None, eps: float = 1e-6, hidden_out=None):
+    """adaLN (1+scale)*LN(h)+shift as a 16-bit tensor, h = x or, with attn and gate, x + gate*attn (also returned).
+    x, attn [B,S,D]; gate, scale, shift [B,D].  Returns norm, or (norm, hidden) when gated."""
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    _chk(scale, "scale", (x.dtype,))
+    _chk(shift, "shift", (x.dtype,))
+    if x.dim() != 3 or tuple(scale.shape) != (x.shape[0], x.shape[2]) or scale.shape != shift.shape:
+        raise ValueError("x must be [B,S,D] and scale, shift [B,D]")
+    if (attn is None) != (gate is None):
+        raise ValueError("attn and gate go together")
+    out = torch.empty_like(x)
+    if attn is not None:
+        _chk(attn, "attn", (x.dtype,))
+        _chk(gate, "gate", (x.dtype,))
+        if attn.shape != x.shape or gate.shape != scale.shape:
+            raise ValueError("attn must be [B,S,D] and gate [B,D]")
+        if hidden_out is None:
+            hidden_out = torch.empty_like(x)
+        _chk(hidden_out, "hidden_out", (x.dtype,))
+    _l.check(_l.load().lq_gate_residual_layernorm_mod(_ptr(out), _ptr(hidden_out) if attn is not None else None, _ptr(attn),
+                                                      _ptr(gate), _ptr(x), _ptr(scale), _ptr(shift), _DT[x.dtype], x.shape[0],
+                                                      x.shape[1], x.shape[2], float(eps), _stream()),
+             "lq_gate_residual_layernorm_mod")
+    return (out, hidden_out) if attn is not None else out
+
+
 # ---- FP8 -------------------------------------------------------------------------------------------
 
 def fp8_amax_scale(x, scale=None):
@@ -443,9 +471,14 @@ def load_lora(weight, lora, alpha: float):
     return weight
 
 
-def w4a4_linear(a_words, w_rows32, sA, sB, bias=None, out_dtype=torch.bfloat16, group: int = 64, lora_act=None, lora_up=None):
+def w4a4_linear(a_words, w_rows32, sA, sB, bias=None, out_dtype=torch.bfloat16, group: int = 64, lora_act=None, lora_up=None,
+                gelu: int = 0, addend=None, gate=None, residual=None, rows_per_gate: int = 1, out_fp8_scale=None,
+                out_fp8=None, col_offset: int = 0, want_output: bool = True, out=None):
     """W4A4 GEMM: a_words int32 [M,K/8], w_rows32 uint8 [N,K/2] (rows32), scales [M,G] / [N,G].
-    lora_act [M,R] and lora_up [N,R] (fp16 or bf16, R a multiple of 16) add the low-rank branch."""
+    lora_act [M,R] and lora_up [N,R] (fp16 or bf16, R a multiple of 16) add the low-rank branch.
+    Epilogue options, in this order: gelu (1: on fp32, 2: on the T-rounded value), addend [M,N] (T(T(y)+addend)),
+    gate + residual (T(T(T(y)*gate[row // rows_per_gate]) + residual)), out_fp8_scale (e4m3 codes of the result, into
+    columns [col_offset, col_offset+N) of out_fp8 when given; want_output=False skips the 16-bit output)."""
     _chk(a_words, "a_words", (torch.int32,))
     _chk(w_rows32, "w_rows32", (torch.uint8, torch.int8))
     _chk(sA, "sA", (torch.float32, torch.float16))
@@ -467,11 +500,38 @@ def w4a4_linear(a_words, w_rows32, sA, sB, bias=None, out_dtype=torch.bfloat16, 
         if lora_act.shape[0] != m or tuple(lora_up.shape) != (n, rank):
             raise ValueError("lora_act must be [M,R] and lora_up [N,R]")
         lora_dt = _DT[lora_act.dtype]
-    c = torch.empty((m, n), dtype=out_dtype, device=a_words.device)
-    _l.check(_l.load().lq_gemm_w4a4_lora(_ptr(c), _DT[out_dtype], _ptr(a_words), _ptr(w_rows32), _ptr(sA), _ptr(sB),
-                                         _DT[sA.dtype], _ptr(bias), _ptr(lora_act), _ptr(lora_up), lora_dt, rank, m, n, k,
-                                         group, _stream()), "lq_gemm_w4a4_lora")
-    return c
+    epi = None
+    c8 = None
+    if gelu or addend is not None or gate is not None or out_fp8_scale is not None:
+        for name, t in (("addend", addend), ("gate", gate), ("residual", residual)):
+            if t is not None:
+                _chk(t, name, (out_dtype,))
+        if (gate is None) != (residual is None):
+            raise ValueError("gate and residual go together")
+        if gate is not None and (residual.numel() != m * n or rows_per_gate <= 0 or
+                                 gate.numel() != ((m + rows_per_gate - 1) // rows_per_gate) * n):
+            raise ValueError("residual must be [M,N] and gate [ceil(M/rows_per_gate), N]")
+        if addend is not None and addend.numel() != m * n:
+            raise ValueError("addend must be [M,N]")
+        epi = _l.Epilogue(int(gelu), _ptr(addend), _ptr(gate), int(rows_per_gate), _ptr(residual), None, 0, None)
+        if out_fp8_scale is not None:
+            _chk(out_fp8_scale, "out_fp8_scale", (torch.float32,))
+            c8 = out_fp8 if out_fp8 is not None else torch.empty((m, n), dtype=torch.uint8, device=a_words.device)
+            _chk(c8, "out_fp8", (torch.uint8,))
+            if c8.dim() != 2 or c8.shape[0] != m or col_offset < 0 or col_offset + n > c8.shape[1]:
+                raise ValueError("out_fp8 must be [M, W] with col_offset + N <= W")
+            epi.C_fp8, epi.ldc_fp8, epi.C_fp8_scale = c8.data_ptr() + col_offset, c8.shape[1], _ptr(out_fp8_scale)
+    if not want_output and c8 is None:
+        raise ValueError("want_output=False needs out_fp8_scale")
+    c = (out if out is not None else torch.empty((m, n), dtype=out_dtype, device=a_words.device)) if want_output else None
+    if c is not None:
+        _chk(c, "out", (out_dtype,))
+    _l.check(_l.load().lq_gemm_w4a4_ex(_ptr(c), _DT[out_dtype], _ptr(a_words), _ptr(w_rows32), _ptr(sA), _ptr(sB),
+                                       _DT[sA.dtype], _ptr(bias), _ptr(lora_act), _ptr(lora_up), lora_dt, rank, m, n, k,
+                                       group, C.byref(epi) if epi is not None else None, _stream()), "lq_gemm_w4a4_ex")
+    if c8 is None:
+        return c
+    return (c, c8) if want_output else c8
 
 
 def lora_down(x, lora_down_w, out_dtype=None):

@@ -273,3 +273,116 @@ def test_flux_single_mlp_fp8_block(ops, dev):
     # move the projection by (a few 2^-4 relative steps of single terms), on top of the stated tolerance
     assert_close_tol(to_np_f32(out).reshape(-1, d), ref.astype(np.float32), "flux single-block mlp",
                      abs_floor=2.0 ** -6 * (np.abs(to_np_f32(x).reshape(-1, d)) + np.abs(ref)) + 0.02)
+
+
+# ---- W4A4 linears with the same epilogues (FLUX INT4 blocks) ---------------------------------------------------------
+def _w4a4_operands(ops, dev, m, n, k, seed, dt, rank=32):
+    g = rng_t(seed)
+    t = TORCH_DT[dt]
+    x = torch.randn(m, k, generator=g).to(t).to(dev)
+    w = (0.05 * torch.randn(n, k, generator=g)).to(t).to(dev)
+    qa, sa = ops.w4a4_quant(x, None, torch.float32)
+    qw, sw = ops.w4a4_quant(w, None, torch.float32)
+    wr = ops.repack_weight(qw.view(torch.uint8).view(n, k // 2))
+    bias = (0.1 * torch.randn(n, generator=g)).to(t).to(dev)
+    la = (0.3 * torch.randn(m, rank, generator=g)).to(t).to(dev)
+    lu = (0.1 * torch.randn(n, rank, generator=g)).to(t).to(dev)
+    return qa, sa, wr, sw, bias, la, lu
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("m,n,k,rpg", [(4608, 256, 512, 4608), (300, 128, 256, 77), (64, 3072, 128, 64)])
+def test_gemm_w4a4_epilogue_options_match_the_unfused_sequence(ops, dev, dt, m, n, k, rpg):
+    qa, sa, wr, sw, bias, la, lu = _w4a4_operands(ops, dev, m, n, k, 500 + m + n, dt)
+    g = rng_t(m + 7 * n)
+    t = TORCH_DT[dt]
+    gate = torch.randn((m + rpg - 1) // rpg, n, generator=g).to(t).to(dev)
+    res = (2 * torch.randn(m, n, generator=g)).to(t).to(dev)
+    add = torch.randn(m, n, generator=g).to(t).to(dev)
+    s_out = torch.tensor([0.02], dtype=torch.float32, device=dev)
+    plain = ops.w4a4_linear(qa, wr, sa, sw, bias, t, 64, la, lu)
+    p32 = to_np_f32(plain)
+    # addend, then gate and residual: every step rounded to T
+    joined = O.round_to(p32 + to_np_f32(add), dt)
+    want = O.gate_residual(joined, to_np_f32(gate), to_np_f32(res), rpg, dt)
+    got = ops.w4a4_linear(qa, wr, sa, sw, bias, t, 64, la, lu, addend=add, gate=gate, residual=res, rows_per_gate=rpg)
+    assert np.array_equal(to_np_f32(got), want)
+    assert np.array_equal(to_np_f32(ops.w4a4_linear(qa, wr, sa, sw, bias, t, 64, la, lu, addend=add)), joined)
+    # e4m3 codes of the plain output, next to the output and alone, dense and into a column block
+    c, codes = ops.w4a4_linear(qa, wr, sa, sw, bias, t, 64, la, lu, out_fp8_scale=s_out)
+    ref_codes = O.fp8_scale_cast(p32, s_out.cpu().numpy()[0], True)
+    assert torch.equal(c, plain) and np.array_equal(codes.cpu().numpy(), ref_codes)
+    wide = torch.full((m, n + 96), 0x11, dtype=torch.uint8, device=dev)
+    only = ops.w4a4_linear(qa, wr, sa, sw, bias, t, 64, la, lu, out_fp8_scale=s_out, out_fp8=wide, col_offset=32, want_output=False)
+    got_wide = only.cpu().numpy()
+    assert np.array_equal(got_wide[:, 32:32 + n], ref_codes) and (got_wide[:, :32] == 0x11).all() and (got_wide[:, 32 + n:] == 0x11).all()
+    # GELU of the rounded output: tolerance (hardware exp / reciprocal in the kernel)
+    gl = to_np_f32(ops.w4a4_linear(qa, wr, sa, sw, bias, t, 64, la, lu, gelu=2))
+    ref = O.cat_gelu(np.zeros((m, 0), np.float32), p32, dt)
+    ulp = 2.0 ** (-7 if dt == "bf16" else -10)
+    assert np.all(np.abs(gl - ref) <= ulp * np.abs(ref) + 1e-6)
+
+
+def _int4_state(prefix, n, k, g, rank=32, bias=True):
+    """Host-side W4A4 weight container entries with the reference's key names."""
+    w = 0.05 * torch.randn(n, k, generator=g)
+    wv = w.view(n, k // 64, 64)
+    sc = wv.abs().amax(dim=2) / 7.0
+    q = torch.clamp(torch.round(wv / sc[..., None]), -8, 7).to(torch.int16).view(n, k)
+    packed = ((q[:, 0::2] & 0xF) | ((q[:, 1::2] & 0xF) << 4)).to(torch.uint8).view(torch.int8)
+    sd = {prefix + "packed_weight": packed.contiguous(), prefix + "weight_scale": sc.float().contiguous(),
+          prefix + "smooth": (0.5 + torch.rand(k, generator=g)).float(),
+          prefix + "lora_up": (0.05 * torch.randn(n, rank, generator=g)).bfloat16(),
+          prefix + "lora_down": (0.05 * torch.randn(rank, k, generator=g)).bfloat16()}
+    if bias:
+        sd[prefix + "bias"] = (0.1 * torch.randn(n, generator=g)).bfloat16()
+    return sd
+
+
+def test_flux_attn_post_int4_block(ops, dev):
+    from lyradiff_amd import flux_int4 as F
+
+    b, s, d = 2, 192, 256
+    g = rng_t(61)
+    sd = _int4_state("p.net.0.proj.", 4 * d, d, g)
+    sd.update(_state_dict({"net.2": (d, 4 * d)}, 62))
+    sd["p.net.2_input_scale"] = torch.tensor([3.0 / 448])
+    w = F.load_flux_attn_post_int4(sd, "p.", d, torch.bfloat16, dev)
+    x = torch.randn(b, s, d, generator=g).bfloat16().to(dev)
+    attn = torch.randn(b, s, d, generator=g).bfloat16().to(dev)
+    msa = (0.5 * torch.randn(6, b, d, generator=g)).bfloat16().to(dev)
+    out = F.flux_attn_post_int4(x, attn, msa, w)
+    # the reference's sequence with this library's unfused kernels and T-rounded torch ops
+    hidden = x + msa[2][:, None, :] * attn
+    norm = ops.gate_residual_layernorm_mod(hidden, msa[4], msa[3])
+    assert torch.equal(norm, ops.gate_residual_layernorm_mod(x, msa[4], msa[3], attn, msa[2])[0])
+    inner = w.gelu_proj.forward(norm.view(b * s, d))                              # GEMM + low-rank + bias
+    inner = torch.nn.functional.gelu(inner.float(), approximate="tanh").bfloat16()
+    q2 = ops.fp8_scale_cast(inner, w.ff_linear.input_scale)
+    ff = ops.fp8_linear(q2, w.ff_linear.weight_rows32, w.ff_linear.input_scale, w.ff_linear.weight_scale, w.ff_linear.bias,
+                        out_dtype=torch.bfloat16)
+    seq = hidden + msa[5][:, None, :] * ff.view(b, s, d)
+    # differences come only from the GELU flavour (codes one e4m3 step apart in a few places)
+    assert_close_tol(to_np_f32(out).reshape(-1, d), to_np_f32(seq).reshape(-1, d), "flux int4 attn-post block",
+                     abs_floor=2.0 ** -6 * (np.abs(to_np_f32(hidden).reshape(-1, d)) + np.abs(to_np_f32(seq).reshape(-1, d))) + 0.02)
+
+
+def test_flux_single_mlp_int4_block(ops, dev):
+    from lyradiff_amd import flux_int4 as F
+
+    b, s, d, ms = 2, 160, 256, 4
+    g = rng_t(71)
+    sd = _int4_state("p.proj_mlp.", ms * d, d, g)
+    sd.update(_int4_state("p.proj_out.linears.0.", d, d, g))
+    sd.update(_int4_state("p.proj_out.linears.1.linear.", d, ms * d, g, bias=False))
+    w = F.load_flux_single_mlp_int4(sd, "p.", d, ms, torch.bfloat16, dev)
+    x, norm, attn = (torch.randn(b, s, d, generator=g).bfloat16().to(dev) for _ in range(3))
+    gate = (0.5 * torch.randn(b, d, generator=g)).bfloat16().to(dev)
+    out = F.flux_single_mlp_int4(x, norm, attn, gate, w)
+    m = b * s
+    mlp = torch.nn.functional.gelu(w.proj_mlp.forward(norm.view(m, d)).float(), approximate="tanh").bfloat16()
+    h1 = w.proj_out_1.forward(attn.view(m, d))
+    h2 = w.proj_out_2.forward(mlp)
+    seq = x + gate[:, None, :] * (h1 + h2).view(b, s, d)
+    assert_close_tol(to_np_f32(out).reshape(-1, d), to_np_f32(seq).reshape(-1, d), "flux int4 single-block tail",
+                     abs_floor=2.0 ** -6 * (np.abs(to_np_f32(x).reshape(-1, d)) + np.abs(to_np_f32(seq).reshape(-1, d))) + 0.03)
