@@ -227,6 +227,22 @@ int lq_gemm_fp8_codes(uint8_t* C_fp8, size_t ldc, const float* C_fp8_scale, lq_d
 int lq_fp8_scale_cast_2d(uint8_t* dst, size_t dst_ld, const void* src, size_t src_ld, lq_dtype_t dtype,
                          const float* scale, int invert, size_t rows, size_t cols, lq_stream_t stream);
 
+/* Weight-only quantized GEMM (W8A16 / W4A16 with per-output-channel scales):
+ *   C[m,n] = T( f32(scale[n]) * sum_k A[m,k]*q[k,n] [+ f32(bias[n])] ),  fp32 accumulation
+ * A, C, scale, bias of `dtype` (F16 or BF16); B_prepared from lq_repack_weight_only.  n % 32 == 0, k % 64 == 0.
+ * Replaces CutlassFpAIntBGemmRunner<T, uint8_t | uint4b_t, PER_COLUMN_SCALE_ONLY>::gemm (A, B, weight_scales, [biases,]
+ * C, m, n, k, ...) (kernels/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm.h:27-130).  The reference multiplies every
+ * dequantised weight by the scale in T inside the main loop; here the scale is applied once per output. */
+int lq_gemm_weight_only(void* C, const void* A, lq_dtype_t dtype, const uint8_t* B_prepared, lq_weight_kind_t kind,
+                        const void* scales, const void* bias, int m, int n, int k, lq_stream_t stream);
+
+/* One-time preparation of a weight-only weight: src_kn is the row-major [k, n] matrix of signed codes as
+ * symmetric_quantize leaves it before preprocessing ("unprocessed_quantized_weight": int8, or for INT4 [k, n/2] bytes
+ * with column 2j in the low nibble; kernels/cutlass_kernels/cutlass_preprocessors.cpp:532-631).  dst (k*n bytes for
+ * INT8, k*n/2 for INT4) receives the layout lq_gemm_weight_only reads; the role of preprocess_weights_for_mixed_gemm
+ * (cutlass_preprocessors.cpp:484-530), whose own layout is specific to NVIDIA's mma fragments. */
+int lq_repack_weight_only(uint8_t* dst, const int8_t* src_kn, lq_weight_kind_t kind, size_t k, size_t n, lq_stream_t stream);
+
 /* SmoothQuant smoothing vector, device side (calibration time).  The reference consumes a precomputed
  * pre_quant_scale from nvidia-modelopt (lyradiff/convert_model_scripts/convert_sd_quant_model.py:199,340); these two
  * calls produce it in the closed form its benchmark configuration states:

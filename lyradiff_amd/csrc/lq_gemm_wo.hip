@@ -1,0 +1,330 @@
+// Weight-only quantized GEMM (W8A16 / W4A16, per-output-channel scales):
+//     C[m,n] = T( scale[n] * sum_k A[m,k] * q[k,n] [+ bias[n]] )
+// with 16-bit activations, int8 or int4 weights and fp32 accumulation on v_mfma_f32_32x32x16_{f16,bf16}.
+// Reference: CutlassFpAIntBGemmRunner (kernels/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm.h:27-130 of lyraDiff,
+// PER_COLUMN_SCALE_ONLY) on weights produced by symmetric_quantize + preprocess_weights_for_mixed_gemm
+// (kernels/cutlass_kernels/cutlass_preprocessors.cpp:484-631).  That preprocessing (row permutation, column-major
+// tile interleave, +128/+8 bias, nibble interleave) is specific to NVIDIA's mma fragments; the counterpart here is
+// lq_repack_weight_only, which keeps its contract -- a one-time bijection of the [k, n] integer matrix -- and
+// produces the layout this kernel reads:
+//   * transposed to [n, k] and stored as UNSIGNED codes u = q + 128 (int8) or u = q + 8 (int4), so that a code
+//     can be ORed into the mantissa of a 16-bit float (1024 + u is 0x6400 | u in fp16) and the offset removed by
+//     one packed subtraction: one or two vector operations per pair of weights instead of a convert per weight;
+//   * int4: the eight codes of a dword sit in nibble order k0 k2 k4 k6 k1 k3 k5 k7 (low to high), so that masking
+//     with 0x000F000F after shifts of 0/4/8/12 bits yields the pairs (k0,k1) (k2,k3) (k4,k5) (k6,k7) directly;
+//   * then the rows32 chunking of the other GEMMs (16-byte chunk c of 32 consecutive output channels contiguous),
+//     which makes every LDS fragment read a conflict-free 16-byte access.
+// The scale is applied once per output in the epilogue (the reference multiplies every dequantised weight by the
+// scale in T inside the main loop, which rounds each weight; results agree to that rounding).
+//
+// Tiling: 256x128 outputs per workgroup of four wavefronts (2x2), 128x64 per wavefront (eight 32x32 MFMA tiles:
+// every converted weight fragment is used by four MFMAs), k-tile 64, two LDS stages filled from registers
+// (activations XOR-swizzled, weights copied as they lie), the next tile's global loads in flight during the MFMAs.
+#include "lq_common.h"
+
+namespace lq {
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+
+template <int CH> __device__ __forceinline__ int wo_swizzle(int row) {  // 8 chunks of 16 bytes per activation row
+    return ((row >> 1) & 7) ^ ((row & 1) << 2);
+}
+
+// eight consecutive-k weights of one output channel as 16-bit floats (four dwords), from unsigned codes
+template <bool F16, bool W4> struct WoCvt;
+template <> struct WoCvt<true, false> {  // fp16 <- uint8: d0 holds k0..k3, d1 holds k4..k7
+    static __device__ __forceinline__ void run(u32 d0, u32 d1, u32* o) {
+        const h2_t off = {(_Float16)1152.0f, (_Float16)1152.0f};
+        const u32 p[4] = {__builtin_amdgcn_perm(0x64646464u, d0, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, d0, 0x04030402u),
+                          __builtin_amdgcn_perm(0x64646464u, d1, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, d1, 0x04030402u)};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = __builtin_bit_cast(u32, __builtin_bit_cast(h2_t, p[i]) - off);
+    }
+};
+template <> struct WoCvt<true, true> {  // fp16 <- uint4: d0 holds k0..k7 in the interleaved nibble order
+    static __device__ __forceinline__ void run(u32 d0, u32, u32* o) {
+        const h2_t off = {(_Float16)1032.0f, (_Float16)1032.0f};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const u32 p = ((d0 >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
+            o[i] = __builtin_bit_cast(u32, __builtin_bit_cast(h2_t, p) - off);
+        }
+    }
+};
+template <> struct WoCvt<false, false> {  // bf16 <- uint8 (through fp32: bf16 cannot hold 1024 + u)
+    static __device__ __forceinline__ void run(u32 d0, u32 d1, u32* o) {
+        const u32 d[2] = {d0, d1};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const u32 w = d[i >> 1] >> (16 * (i & 1));
+            o[i] = pack2_bf16((float)(w & 0xFFu) - 128.0f, (float)((w >> 8) & 0xFFu) - 128.0f);
+        }
+    }
+};
+template <> struct WoCvt<false, true> {  // bf16 <- uint4
+    static __device__ __forceinline__ void run(u32 d0, u32, u32* o) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const u32 w = d0 >> (4 * i);
+            o[i] = pack2_bf16((float)(w & 0xFu) - 8.0f, (float)((w >> 16) & 0xFu) - 8.0f);
+        }
+    }
+};
+
+template <typename Tag, bool W4>
+__global__ __launch_bounds__(256, 2) void wo_gemm_kernel(void* __restrict__ C, const void* __restrict__ A,
+                                                         const uint8_t* __restrict__ B, const void* __restrict__ scales,
+                                                         const void* __restrict__ bias, int m, int n, int k, int tiles_m,
+                                                         int tiles_n) {
+    constexpr bool F16 = std::is_same<Tag, F16Tag>::value;
+    constexpr int BM = 256, BN = 128, BK = 64, TM = 128, TN = 64, MT = 4, NT = 2;
+    constexpr int A_BYTES = BM * BK * 2;                 // 32 KiB
+    constexpr int BCH = W4 ? 2 : 4;                      // 16-byte weight chunks per row per k-tile
+    constexpr int B_BYTES = BN * BCH * 16;               // 8 or 4 KiB
+    constexpr int STAGE = A_BYTES + B_BYTES;
+    constexpr int A_LD = A_BYTES / 16 / 256;             // 16-byte loads per thread per tile (8)
+    constexpr int B_LD = B_BYTES / 16 / 256;             // 2 or 1
+    static_assert(B_LD * 256 * 16 == B_BYTES, "weight stage is a whole number of 16-byte loads per thread");
+    extern __shared__ __attribute__((aligned(16))) char wo_smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    // consecutive workgroup ids of one XCD (ids congruent modulo 8) walk down a column of tiles, so that an XCD's
+    // L2 keeps one weight panel and streams activations
+    int bid = blockIdx.x;
+    const int total = tiles_m * tiles_n, per_xcd = total / 8;
+    if (bid < per_xcd * 8) bid = (bid & 7) * per_xcd + (bid >> 3);
+    const int tm = bid % tiles_m, tn = bid / tiles_m;
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int ktiles = k / BK;
+    const size_t a_pitch = (size_t)k * 2;
+    const size_t b_row_bytes = W4 ? (size_t)k / 2 : (size_t)k;
+    const size_t b_blk = b_row_bytes * 32;  // bytes per block of 32 output channels
+    const int row_last = m - 1 - m0, blk_last = n / 32 - 1 - n0 / 32;
+
+    // ---- global -> register -> LDS plan (32-bit per-lane offsets from wavefront-uniform tile bases) -------------
+    const char* a_tile = static_cast<const char*>(A) + (size_t)m0 * a_pitch;
+    const char* b_tile = reinterpret_cast<const char*>(B) + (size_t)(n0 / 32) * b_blk;
+    u32 a_voff[A_LD];
+    const int a_r0 = tid >> 3, a_c = tid & 7;
+    // row i*32 + a_r0 of the tile: the swizzle only looks at the low four row bits, so it is the same for every i
+    const int a_dst0 = a_r0 * 128 + ((a_c ^ wo_swizzle<8>(a_r0)) << 4);
+#pragma unroll
+    for (int i = 0; i < A_LD; ++i) a_voff[i] = (u32)min(i * 32 + a_r0, row_last) * (u32)a_pitch + a_c * 16;
+    u32 b_voff[B_LD];
+#pragma unroll
+    for (int i = 0; i < B_LD; ++i) {
+        const int slot = i * 256 + tid;  // [block of 32 channels][chunk][row in block]
+        const int blk = slot / (BCH * 32), within = slot % (BCH * 32);
+        b_voff[i] = (u32)((size_t)min(blk, blk_last) * b_blk) + within * 16;
+    }
+    v4i ra[A_LD], rb[B_LD];
+#define LQ_WO_FETCH(KT)                                                                                          \
+    do {                                                                                                         \
+        const char* ga = a_tile + (size_t)(KT) * (BK * 2);                                                       \
+        const char* gb = b_tile + (size_t)(KT) * (BCH * 512);                                                    \
+        _Pragma("unroll") for (int i = 0; i < A_LD; ++i) ra[i] = *reinterpret_cast<const v4i*>(ga + a_voff[i]);  \
+        _Pragma("unroll") for (int i = 0; i < B_LD; ++i) rb[i] = *reinterpret_cast<const v4i*>(gb + b_voff[i]);  \
+    } while (0)
+#define LQ_WO_STASH(STAGE_IDX)                                                                                            \
+    do {                                                                                                                  \
+        char* s = wo_smem + (STAGE_IDX) * STAGE;                                                                          \
+        _Pragma("unroll") for (int i = 0; i < A_LD; ++i) *reinterpret_cast<v4i*>(s + a_dst0 + i * (32 * 128)) = ra[i];    \
+        _Pragma("unroll") for (int i = 0; i < B_LD; ++i) *reinterpret_cast<v4i*>(s + A_BYTES + (i * 256 + tid) * 16) = rb[i]; \
+    } while (0)
+
+    v16f acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    const int lr = lane & 31, lh = lane >> 5;
+    const int xrow = wm * TM + lr;
+    const int xsw = wo_swizzle<8>(xrow);  // unchanged by +32*i
+    auto compute = [&](int stage) {
+        const char* sa = wo_smem + stage * STAGE;
+        const char* sb = sa + A_BYTES + (wn * NT) * (BCH * 512) + lr * 16;
+        uint4 w4raw[NT];  // int4: one 16-byte read holds the lane's 32 weights of the whole k-tile
+        if constexpr (W4) {
+#pragma unroll
+            for (int j = 0; j < NT; ++j) w4raw[j] = *reinterpret_cast<const uint4*>(sb + j * (BCH * 512) + lh * 512);
+        }
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {  // two MFMA k-steps per weight chunk read (int8) / per pair of dwords (int4)
+            u32 wfrag[NT][2][4];
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                if constexpr (W4) {
+                    WoCvt<F16, true>::run(half ? w4raw[j].z : w4raw[j].x, 0u, wfrag[j][0]);
+                    WoCvt<F16, true>::run(half ? w4raw[j].w : w4raw[j].y, 0u, wfrag[j][1]);
+                } else {
+                    const uint4 d = *reinterpret_cast<const uint4*>(sb + j * (BCH * 512) + (half * 2 + lh) * 512);
+                    WoCvt<F16, false>::run(d.x, d.y, wfrag[j][0]);
+                    WoCvt<F16, false>::run(d.z, d.w, wfrag[j][1]);
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                // activation chunk that holds the same eight k as wfrag[.][s]
+                const int chunk = W4 ? lh * 4 + half * 2 + s : half * 4 + lh * 2 + s;
+#pragma unroll
+                for (int i = 0; i < MT; ++i) {
+                    const uint4 x = *reinterpret_cast<const uint4*>(sa + (xrow + i * 32) * 128 + ((chunk ^ xsw) << 4));
+#pragma unroll
+                    for (int j = 0; j < NT; ++j) {
+                        const uint4 w = make_uint4(wfrag[j][s][0], wfrag[j][s][1], wfrag[j][s][2], wfrag[j][s][3]);
+                        if constexpr (F16)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, w), __builtin_bit_cast(v8h, x), acc[i][j], 0, 0, 0);
+                        else
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, w), __builtin_bit_cast(v8bf, x), acc[i][j], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    };
+
+    LQ_WO_FETCH(0);
+    LQ_WO_STASH(0);
+    __syncthreads();
+    // The prefetch is unconditional (past the end it re-reads the last tile into the stage nobody reads again): with
+    // a branch around it the compiler parks the prefetch registers in scratch memory and the overlap is lost.
+    for (int kt = 0; kt < ktiles; ++kt) {
+        LQ_WO_FETCH(min(kt + 1, ktiles - 1));
+        compute(kt & 1);
+        LQ_WO_STASH((kt + 1) & 1);
+        __syncthreads();
+    }
+#undef LQ_WO_FETCH
+#undef LQ_WO_STASH
+
+    // ---- epilogue: weights were the first MFMA operand, so a lane holds one activation row (lr) and, per tile,
+    // four runs of four consecutive output channels: 8-byte stores -------------------------------------------------
+    const int mrow0 = m0 + wm * TM + lr;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const int nb = n0 + wn * TN + j * 32;
+        float sc[16], bs[16];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            const int nn = nb + q4 * 8 + lh * 4;
+            const bool ok = nn < n;
+            uint2 sv = make_uint2(0, 0), bv = make_uint2(0, 0);
+            if (ok) sv = *reinterpret_cast<const uint2*>(static_cast<const unsigned short*>(scales) + nn);
+            if (ok && bias != nullptr) bv = *reinterpret_cast<const uint2*>(static_cast<const unsigned short*>(bias) + nn);
+            sc[q4 * 4] = Elem<Tag>::load(sv.x & 0xFFFFu); sc[q4 * 4 + 1] = Elem<Tag>::load(sv.x >> 16);
+            sc[q4 * 4 + 2] = Elem<Tag>::load(sv.y & 0xFFFFu); sc[q4 * 4 + 3] = Elem<Tag>::load(sv.y >> 16);
+            bs[q4 * 4] = Elem<Tag>::load(bv.x & 0xFFFFu); bs[q4 * 4 + 1] = Elem<Tag>::load(bv.x >> 16);
+            bs[q4 * 4 + 2] = Elem<Tag>::load(bv.y & 0xFFFFu); bs[q4 * 4 + 3] = Elem<Tag>::load(bv.y >> 16);
+        }
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const int mr = mrow0 + i * 32;
+            if (mr >= m) continue;
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const int nn = nb + q4 * 8 + lh * 4;
+                if (nn >= n) continue;
+                float y[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    y[e] = acc[i][j][q4 * 4 + e] * sc[q4 * 4 + e];
+                    if (bias != nullptr) y[e] = y[e] + bs[q4 * 4 + e];
+                }
+                uint2 o;
+                if constexpr (F16) { o.x = pack2_f16(y[0], y[1]); o.y = pack2_f16(y[2], y[3]); }
+                else { o.x = pack2_bf16(y[0], y[1]); o.y = pack2_bf16(y[2], y[3]); }
+                *reinterpret_cast<uint2*>(static_cast<unsigned short*>(C) + (size_t)mr * n + nn) = o;
+            }
+        }
+    }
+}
+
+// ---- one-time weight preparation: [k, n] signed codes (int8, or int4 pairs packed along n, low nibble = even
+// column) -> the layout described at the top.  One thread per 16-byte destination chunk. ---------------------------
+template <bool W4>
+__global__ __launch_bounds__(256) void wo_repack_kernel(uint8_t* __restrict__ dst, const int8_t* __restrict__ src, size_t k, size_t n) {
+    const size_t row_bytes = W4 ? k / 2 : k, kc_count = row_bytes / 16, total = n * kc_count;
+    for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = t & 31, rest = t >> 5, kc = rest % kc_count, nb = rest / kc_count;
+        const size_t col = nb * 32 + r;
+        u32 w[4] = {0, 0, 0, 0};
+        if constexpr (W4) {
+            const size_t kbase = kc * 32;  // 32 weights per chunk
+            const uint8_t* s = reinterpret_cast<const uint8_t*>(src) + col / 2;
+            const int sh = (col & 1) * 4;
+#pragma unroll
+            for (int e = 0; e < 32; ++e) {
+                const u32 code = ((((u32)s[(kbase + e) * (n / 2)] >> sh) & 0xFu) + 8u) & 0xFu;  // two's complement nibble + 8
+                const int j = e & 7, pos = (j & 1) * 4 + (j >> 1);                             // k0 k2 k4 k6 | k1 k3 k5 k7
+                w[e >> 3] |= code << (4 * pos);
+            }
+        } else {
+            const size_t kbase = kc * 16;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) w[e >> 2] |= (u32)(uint8_t)(src[(kbase + e) * n + col] + 128) << (8 * (e & 3));
+        }
+        *reinterpret_cast<uint4*>(dst + t * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
+}  // namespace lq
+
+using namespace lq;
+
+extern "C" int lq_repack_weight_only(uint8_t* dst, const int8_t* src_kn, lq_weight_kind_t kind, size_t k, size_t n,
+                                     lq_stream_t stream) {
+    LQ_REQUIRE(dst && src_kn, LQ_ERR_ARG, "lq_repack_weight_only: null pointer");
+    LQ_REQUIRE(kind == LQ_W_INT8 || kind == LQ_W_INT4, LQ_ERR_UNSUPPORTED, "lq_repack_weight_only: kind must be INT8 or INT4");
+    LQ_REQUIRE(n % 32 == 0 && k % 64 == 0 && n > 0 && k > 0, LQ_ERR_SHAPE,
+               "lq_repack_weight_only: need n %% 32 == 0 and k %% 64 == 0 (k=%zu n=%zu)", k, n);
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(dst) % 16 == 0, LQ_ERR_ARG, "lq_repack_weight_only: dst must be 16-byte aligned");
+    const size_t chunks = n * ((kind == LQ_W_INT4 ? k / 2 : k) / 16);
+    const unsigned blocks = (unsigned)std::min<size_t>((chunks + 255) / 256, 65535);
+    if (kind == LQ_W_INT4) hipLaunchKernelGGL((wo_repack_kernel<true>), dim3(blocks), dim3(256), 0, as_stream(stream), dst, src_kn, k, n);
+    else hipLaunchKernelGGL((wo_repack_kernel<false>), dim3(blocks), dim3(256), 0, as_stream(stream), dst, src_kn, k, n);
+    return check_launch("wo_repack");
+}
+
+extern "C" int lq_gemm_weight_only(void* C, const void* A, lq_dtype_t dtype, const uint8_t* B_prepared, lq_weight_kind_t kind,
+                                   const void* scales, const void* bias, int m, int n, int k, lq_stream_t stream) {
+    LQ_REQUIRE(C && A && B_prepared && scales, LQ_ERR_ARG, "lq_gemm_weight_only: null pointer");
+    LQ_REQUIRE(dtype == LQ_F16 || dtype == LQ_BF16, LQ_ERR_UNSUPPORTED, "lq_gemm_weight_only: activations must be F16 or BF16");
+    LQ_REQUIRE(kind == LQ_W_INT8 || kind == LQ_W_INT4, LQ_ERR_UNSUPPORTED, "lq_gemm_weight_only: kind must be INT8 or INT4");
+    LQ_REQUIRE(m >= 0 && n > 0 && k > 0 && n % 32 == 0 && k % 64 == 0, LQ_ERR_SHAPE,
+               "lq_gemm_weight_only: need n %% 32 == 0 and k %% 64 == 0 (m=%d n=%d k=%d)", m, n, k);
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B_prepared) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(C) % 8 == 0 && reinterpret_cast<uintptr_t>(scales) % 8 == 0 &&
+                   reinterpret_cast<uintptr_t>(bias) % 8 == 0,
+               LQ_ERR_ARG, "lq_gemm_weight_only: A and B must be 16-byte, C, scales and bias 8-byte aligned");
+    if (m == 0) return LQ_OK;
+    const int tiles_m = (m + 255) / 256, tiles_n = (n + 127) / 128;
+    const bool w4 = kind == LQ_W_INT4;
+    const size_t lds = 2 * (size_t)(256 * 64 * 2 + 128 * (w4 ? 2 : 4) * 16);
+    dim3 grid((unsigned)(tiles_m * tiles_n)), block(256);
+    hipStream_t st = as_stream(stream);
+#define LQ_WO_GO(TAG, W4V)                                                                                              \
+    do {                                                                                                                \
+        static bool attr_done = false;                                                                                  \
+        if (!attr_done) {                                                                                               \
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&wo_gemm_kernel<TAG, W4V>),                           \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {              \
+                set_error("lq_gemm_weight_only: cannot raise the dynamic LDS limit to %zu bytes", lds);                 \
+                return LQ_ERR_HIP;                                                                                      \
+            }                                                                                                           \
+            attr_done = true;                                                                                           \
+        }                                                                                                               \
+        hipLaunchKernelGGL((wo_gemm_kernel<TAG, W4V>), grid, block, lds, st, C, A, B_prepared, scales, bias, m, n, k,   \
+                           tiles_m, tiles_n);                                                                           \
+    } while (0)
+    if (dtype == LQ_F16) {
+        if (w4) LQ_WO_GO(F16Tag, true); else LQ_WO_GO(F16Tag, false);
+    } else {
+        if (w4) LQ_WO_GO(BF16Tag, true); else LQ_WO_GO(BF16Tag, false);
+    }
+#undef LQ_WO_GO
+    return check_launch("gemm_weight_only");
+}

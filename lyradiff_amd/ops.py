@@ -460,6 +460,35 @@ def fp8_scale_cast_into(x, scale, out, col_offset: int = 0, invert: bool = True)
     return out
 
 
+def repack_weight_only(q_kn, kind: str):
+    """One-time preparation of a weight-only weight.  q_kn: int8 [K, N] signed codes, or for kind "int4" int8
+    [K, N/2] with column 2j in the low nibble (the reference's unprocessed_quantized_weight).  Returns the uint8
+    tensor [N, K] / [N, K/2] that weight_only_linear reads."""
+    _chk(q_kn, "q_kn", (torch.int8,))
+    k = q_kn.shape[0]
+    n = q_kn.shape[1] * (2 if kind == "int4" else 1)
+    out = torch.empty((n, k // 2 if kind == "int4" else k), dtype=torch.uint8, device=q_kn.device)
+    _l.check(_l.load().lq_repack_weight_only(_ptr(out), _ptr(q_kn), _KINDS[kind], k, n, _stream()), "lq_repack_weight_only")
+    return out
+
+
+def weight_only_linear(x, w_prepared, scales, bias=None, kind: str = "int8"):
+    """W8A16 / W4A16 linear: x [M, K] fp16/bf16, w_prepared from repack_weight_only, scales and bias [N] of x.dtype."""
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    _chk(w_prepared, "w_prepared", (torch.uint8,))
+    _chk(scales, "scales", (x.dtype,))
+    if bias is not None:
+        _chk(bias, "bias", (x.dtype,))
+    m, k = x.shape
+    n = w_prepared.shape[0]
+    if w_prepared.shape[1] != (k // 2 if kind == "int4" else k) or scales.numel() != n:
+        raise ValueError("shape mismatch between x, w_prepared and scales")
+    c = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    _l.check(_l.load().lq_gemm_weight_only(_ptr(c), _ptr(x), _DT[x.dtype], _ptr(w_prepared), _KINDS[kind], _ptr(scales),
+                                           _ptr(bias), m, n, k, _stream()), "lq_gemm_weight_only")
+    return c
+
+
 def load_lora(weight, lora, alpha: float):
     """invokeLoadLora: weight += lora * alpha in the tensors' dtype, in place; returns weight."""
     _chk(weight, "weight", _FLOATS)

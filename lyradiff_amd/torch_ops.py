@@ -18,7 +18,8 @@ from . import ops as _ops
 
 _lib_op = torch.library.custom_op
 NAMES = ("sq_quant", "sq_quant_dynamic", "geglu_int8_dynamic", "int8_linear", "fp8_quant", "fp8_scale_cast", "fp8_linear",
-         "w4a4_quant", "w4a4_linear", "repack_weight")
+         "w4a4_quant", "w4a4_linear", "repack_weight", "lora_down", "layernorm_mod_fp8", "gate_residual_layernorm_mod_fp8",
+         "fp8_linear_codes", "fp8_linear_gated", "flux_attn_post_fp8", "flux_single_mlp_fp8")
 
 
 @_lib_op("lyradiff::sq_quant", mutates_args=())
@@ -129,3 +130,93 @@ def repack_weight(w_bytes: Tensor) -> Tensor:
 @repack_weight.register_fake
 def _(w_bytes):
     return torch.empty_like(w_bytes)
+
+
+@_lib_op("lyradiff::lora_down", mutates_args=())
+def lora_down(x: Tensor, lora_down_w: Tensor) -> Tensor:
+    return _ops.lora_down(x, lora_down_w)
+
+
+@lora_down.register_fake
+def _(x, lora_down_w):
+    return x.new_empty((x.shape[0], lora_down_w.shape[0]))
+
+
+@_lib_op("lyradiff::layernorm_mod_fp8", mutates_args=())
+def layernorm_mod_fp8(x: Tensor, scale: Tensor, shift: Tensor, input_scale: Tensor, eps: float = 1e-6) -> Tensor:
+    return _ops.layernorm_mod_fp8(x, scale, shift, input_scale, eps)
+
+
+@layernorm_mod_fp8.register_fake
+def _(x, scale, shift, input_scale, eps=1e-6):
+    return x.new_empty(x.shape, dtype=torch.uint8)
+
+
+@_lib_op("lyradiff::gate_residual_layernorm_mod_fp8", mutates_args=())
+def gate_residual_layernorm_mod_fp8(attn: Tensor, gate: Tensor, x: Tensor, scale: Tensor, shift: Tensor, input_scale: Tensor,
+                                    eps: float = 1e-6) -> Tuple[Tensor, Tensor]:
+    return _ops.gate_residual_layernorm_mod_fp8(attn, gate, x, scale, shift, input_scale, eps)
+
+
+@gate_residual_layernorm_mod_fp8.register_fake
+def _(attn, gate, x, scale, shift, input_scale, eps=1e-6):
+    return x.new_empty(x.shape, dtype=torch.uint8), torch.empty_like(x)
+
+
+@_lib_op("lyradiff::fp8_linear_codes", mutates_args=())
+def fp8_linear_codes(a_q: Tensor, w_rows32: Tensor, a_scale: Tensor, b_scale: Tensor, bias: Optional[Tensor],
+                     out_fp8_scale: Tensor, gelu: int = 0, round_dtype: torch.dtype = torch.bfloat16) -> Tensor:
+    return _ops.fp8_linear_codes(a_q, w_rows32, a_scale, b_scale, bias, out_fp8_scale, gelu, round_dtype)
+
+
+@fp8_linear_codes.register_fake
+def _(a_q, w_rows32, a_scale, b_scale, bias, out_fp8_scale, gelu=0, round_dtype=torch.bfloat16):
+    return a_q.new_empty((a_q.shape[0], w_rows32.shape[0]), dtype=torch.uint8)
+
+
+@_lib_op("lyradiff::fp8_linear_gated", mutates_args=())
+def fp8_linear_gated(a_q: Tensor, w_rows32: Tensor, a_scale: Tensor, b_scale: Tensor, bias: Optional[Tensor], gate: Tensor,
+                     residual: Tensor, rows_per_gate: int) -> Tensor:
+    return _ops.fp8_linear_gated(a_q, w_rows32, a_scale, b_scale, bias, gate, residual, rows_per_gate)
+
+
+@fp8_linear_gated.register_fake
+def _(a_q, w_rows32, a_scale, b_scale, bias, gate, residual, rows_per_gate):
+    return residual.new_empty((a_q.shape[0], w_rows32.shape[0]))
+
+
+# ---- block level: the FP8 feed-forward halves of the FLUX blocks as single operators --------------------------------
+# Weights travel as flat tensor lists (rows32 codes, weight scale, input scale, bias per linear), the form a
+# torch-side module keeps after loading a state dict with lyradiff_amd.flux_fp8.load_*.
+def _fp8_lin(w: Tensor, ws: Tensor, s_in: Tensor, b: Tensor):
+    from .weights import FP8Linear
+
+    return FP8Linear(w, ws, s_in, b)
+
+
+@_lib_op("lyradiff::flux_attn_post_fp8", mutates_args=())
+def flux_attn_post_fp8(x: Tensor, attn_output: Tensor, msa: Tensor, w1: Tensor, w1_scale: Tensor, in1_scale: Tensor, b1: Tensor,
+                       w2: Tensor, w2_scale: Tensor, in2_scale: Tensor, b2: Tensor) -> Tensor:
+    from . import flux_fp8 as F
+
+    return F.flux_attn_post_fp8(x, attn_output, msa, F.FluxAttnPostFP8Weights(_fp8_lin(w1, w1_scale, in1_scale, b1),
+                                                                              _fp8_lin(w2, w2_scale, in2_scale, b2)))
+
+
+@flux_attn_post_fp8.register_fake
+def _(x, attn_output, msa, w1, w1_scale, in1_scale, b1, w2, w2_scale, in2_scale, b2):
+    return torch.empty_like(x)
+
+
+@_lib_op("lyradiff::flux_single_mlp_fp8", mutates_args=())
+def flux_single_mlp_fp8(x: Tensor, norm_hidden: Tensor, attn_output: Tensor, gate: Tensor, wm: Tensor, wm_scale: Tensor,
+                        inm_scale: Tensor, bm: Tensor, wo: Tensor, wo_scale: Tensor, ino_scale: Tensor, bo: Tensor) -> Tensor:
+    from . import flux_fp8 as F
+
+    return F.flux_single_mlp_fp8(x, norm_hidden, attn_output, gate,
+                                 F.FluxSingleMlpFP8Weights(_fp8_lin(wm, wm_scale, inm_scale, bm), _fp8_lin(wo, wo_scale, ino_scale, bo)))
+
+
+@flux_single_mlp_fp8.register_fake
+def _(x, norm_hidden, attn_output, gate, wm, wm_scale, inm_scale, bm, wo, wo_scale, ino_scale, bo):
+    return torch.empty_like(x)

@@ -207,3 +207,23 @@ def unpack_int4_packed_tensor_to_int8(weight: torch.Tensor) -> torch.Tensor:
     lo, hi = b & 0xF, b >> 4
     lo, hi = torch.where(lo > 7, lo - 16, lo), torch.where(hi > 7, hi - 16, hi)
     return torch.stack((lo, hi), dim=-1).reshape(*weight.shape[:-1], weight.shape[-1] * 2).to(torch.int8)
+
+
+def symmetric_quantize_last_axis_of_batched_matrix(weight: torch.Tensor, bits: int = 8):
+    """Per-column symmetric weight-only quantisation of a CPU [K, N] (or [E, K, N]) fp16/bf16/fp32 weight
+    (symmetric_quantize, src/lyradiff/kernels/cutlass_kernels/cutlass_preprocessors.cpp:532-631, exposed as
+    lyrallms::symmetric_quantize_last_axis_of_batched_matrix, WeightOnlyQuantOps.cc:120-215): scale = max|w| / 2^(bits-1)
+    per column, q = clip(round-half-away(w / scale)).  Returns (unprocessed codes int8 -- int4 packed two per byte
+    along N, low nibble first --, scales in the weight's dtype); prepare the codes for the GEMM with
+    ops.repack_weight_only on the device."""
+    if weight.is_cuda or weight.dim() not in (2, 3) or bits not in (4, 8):
+        raise ValueError("weight must be a CPU tensor of 2 or 3 dimensions, bits 4 or 8")
+    w = weight.float()
+    half = float(1 << (bits - 1))
+    col = w.abs().amax(dim=-2) * (1.0 / half)
+    r = w / col.unsqueeze(-2)
+    r = torch.sign(r) * torch.floor(r.abs() + 0.5)
+    q = torch.nan_to_num(r, nan=0.0).clamp(-half, half - 1).to(torch.int8)
+    if bits == 4:
+        q = pack_int8_tensor_to_packed_int4(q.contiguous())
+    return q.contiguous(), col.to(weight.dtype)

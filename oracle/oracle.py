@@ -21,6 +21,8 @@ closed forms / exhaustive tables / brute force in tests/test_oracle_*.py:
                         reference's closed-source cuBLASLt)            (pinned to tolerance)
   gate_residual         exact rational arithmetic rounded once per op  (pinned)
   cat_gelu              concatenation + the pinned gelu_tanh_f32        (pinned)
+  weight_only_quantize  hand-computed columns, extremes, ties away      (pinned)
+  weight_only_gemm_f64  naive loops                                     (pinned to tolerance)
 
 The calibration that produces SmoothQuant `pre_quant_scale` in the reference lives in
 nvidia-modelopt (absent): parity unpinned, replaced by the closed form in smooth_vector().
@@ -543,6 +545,49 @@ def w4a4_gemm_lora_f64(y32, lora_act, lora_up, bias=None, out_dtype: str = "bf16
     if bias is not None:
         y = y + np.asarray(bias, dtype=np.float64)[None, :]
     return round_to(y.astype(F32), out_dtype)
+
+
+# ----------------------------------------------------------------------------------------
+# weight-only quantisation (W8A16 / W4A16): symmetric_quantize
+#      (kernels/cutlass_kernels/cutlass_preprocessors.cpp:532-631) and the contract of
+#      CutlassFpAIntBGemmRunner::gemm (kernels/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm.h:27-130)
+# ----------------------------------------------------------------------------------------
+
+
+def weight_only_quantize(w_kn, bits: int, dtype: str):
+    """Per-column symmetric quantisation of a [k, n] weight: scale_f = max_k|w| * (1 / 2^(bits-1)) in fp32,
+    q = clip(round_half_away(w / scale_f), -2^(bits-1), 2^(bits-1)-1); the stored scale is T(scale_f).
+    Returns (q int8 [k, n], scale [n] as fp32 values of T)."""
+    w = np.asarray(w_kn, dtype=F32)
+    half = 1 << (bits - 1)
+    col = (np.abs(w).max(axis=0).astype(F32) * F32(1.0 / half)).astype(F32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        r = (w / col[None, :]).astype(F32)
+    r = np.sign(r) * np.floor(np.abs(r) + F32(0.5))  # C round(): halves away from zero
+    r = np.where(np.isnan(r), F32(0.0), r)           # an all-zero column: 0/0, (int8_t)NaN is taken as 0
+    q = np.clip(r, -half, half - 1).astype(np.int8)
+    return q, round_to(col, dtype)
+
+
+def weight_only_gemm_f64(a, q_kn, scale, bias=None, out_dtype: str = "f16") -> np.ndarray:
+    """T( scale[n] * sum_k a[m,k]*q[k,n] [+ bias[n]] ) evaluated in fp64 (the reference dequantises each weight to
+    T(q*scale) first and sums in an order its tensor-core tiling fixes: tolerance reference)."""
+    y = (np.asarray(a, dtype=np.float64) @ np.asarray(q_kn, dtype=np.float64)) * np.asarray(scale, dtype=np.float64)[None, :]
+    if bias is not None:
+        y = y + np.asarray(bias, dtype=np.float64)[None, :]
+    return round_to(y.astype(F32), out_dtype)
+
+
+def weight_only_prepared(q_kn, bits: int) -> np.ndarray:
+    """The byte matrix [n, k*bits/8] lq_repack_weight_only produces before its rows32 chunking: transposed unsigned
+    codes u = q + 2^(bits-1); int4: the eight codes of a dword in nibble order k0 k2 k4 k6 k1 k3 k5 k7."""
+    q = np.asarray(q_kn, dtype=np.int16).T  # [n, k]
+    if bits == 8:
+        return (q + 128).astype(np.uint8)
+    u = (q + 8).astype(np.uint32).reshape(q.shape[0], -1, 8)
+    pos = np.array([0, 4, 1, 5, 2, 6, 3, 7], dtype=np.uint32)  # nibble that holds k_j
+    words = (u << (4 * pos)[None, None, :]).sum(axis=2).astype(np.uint32)
+    return np.ascontiguousarray(words).view(np.uint8).reshape(q.shape[0], -1)
 
 
 # ----------------------------------------------------------------------------------------

@@ -1,0 +1,81 @@
+"""GPU parity of the weight-only (W8A16 / W4A16) GEMM and its weight preparation, through the C ABI.
+
+The preparation is a bijection of integer codes: compared bit for bit with the oracle's restatement of the layout.
+The GEMM accumulates exact products (a 16-bit float times a small integer) in fp32 in an order of its own; it is
+compared with the fp64 evaluation of the contract within 1e-2 relative / 2 fp16 ULP, plus a few fp32 ULPs of the sum of
+the |terms| where the terms cancel."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from tests.helpers import TORCH_DT, assert_close_tol, rng_t, to_np_f32
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops(dev):
+    from lyradiff_amd import ops as _ops
+
+    return _ops
+
+
+def _pack_n(q_kn):
+    """[K, N] int8 codes in [-8, 7] -> [K, N/2] bytes, column 2j in the low nibble."""
+    q = q_kn.astype(np.int16)
+    return ((q[:, 0::2] & 0xF) | ((q[:, 1::2] & 0xF) << 4)).astype(np.uint8).view(np.int8)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("k,n", [(64, 32), (192, 160), (3072, 1280)])
+def test_repack_weight_only_layout(ops, dev, bits, k, n):
+    rng = np.random.default_rng(k + n + bits)
+    half = 1 << (bits - 1)
+    q = rng.integers(-half, half, (k, n)).astype(np.int8)
+    src = torch.from_numpy(q if bits == 8 else _pack_n(q)).to(dev)
+    got = ops.repack_weight_only(src, "int8" if bits == 8 else "int4").cpu().numpy()
+    want = O.repack_rows32(O.weight_only_prepared(q, bits))
+    assert got.size == want.size and np.array_equal(got.reshape(-1), want.reshape(-1))
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("m,n,k,with_bias", [(256, 128, 64, True), (300, 160, 192, False), (1, 32, 128, True),
+                                             (1024, 1280, 1280, True), (777, 3072, 512, True)])
+def test_weight_only_gemm(ops, dev, dt, bits, m, n, k, with_bias):
+    from lyradiff_amd.weights import symmetric_quantize_last_axis_of_batched_matrix as squant
+
+    g = rng_t(m + n + k + bits)
+    t = TORCH_DT[dt]
+    w = (0.05 * torch.randn(k, n, generator=g)).to(t)
+    x = torch.randn(m, k, generator=g).to(t)
+    bias = (0.2 * torch.randn(n, generator=g)).to(t) if with_bias else None
+    codes, scales = squant(w, bits)
+    q_ref, s_ref = O.weight_only_quantize(to_np_f32(w), bits, dt)
+    unpacked = codes.numpy() if bits == 8 else None
+    if bits == 4:  # unpack along N for the comparison
+        b = codes.numpy().view(np.uint8).astype(np.int16)
+        lo, hi = b & 0xF, b >> 4
+        unpacked = np.stack([np.where(lo > 7, lo - 16, lo), np.where(hi > 7, hi - 16, hi)], axis=-1).reshape(k, n).astype(np.int8)
+    assert np.array_equal(unpacked, q_ref) and np.array_equal(to_np_f32(scales), s_ref)
+    kind = "int8" if bits == 8 else "int4"
+    wp = ops.repack_weight_only(codes.to(dev), kind)
+    y = ops.weight_only_linear(x.to(dev), wp, scales.to(dev), bias.to(dev) if with_bias else None, kind)
+    ref = O.weight_only_gemm_f64(to_np_f32(x), q_ref, s_ref, to_np_f32(bias) if with_bias else None, dt)
+    floor = 4e-6 * (np.abs(to_np_f32(x)).astype(np.float64) @ np.abs(q_ref.astype(np.float64))) * s_ref.astype(np.float64)[None, :]
+    if dt == "bf16":  # the output's own rounding: one bf16 ULP is 8 fp16 ULPs
+        floor = floor + 2.0 ** -8 * np.abs(ref.astype(np.float64))
+    assert_close_tol(to_np_f32(y), ref, f"weight-only {kind} {dt}", abs_floor=floor)
+
+
+def test_weight_only_argument_checks(ops, dev):
+    from lyradiff_amd.lib import LyraQuantError
+
+    x = torch.zeros(8, 96, dtype=torch.float16, device=dev)  # k = 96 is not a multiple of 64
+    w = torch.zeros(32, 96, dtype=torch.uint8, device=dev)
+    s = torch.ones(32, dtype=torch.float16, device=dev)
+    with pytest.raises(LyraQuantError, match="k %% 64|k % 64"):
+        ops.weight_only_linear(x, w, s)
+    with pytest.raises(TypeError):
+        ops.weight_only_linear(x.float(), w, s)

@@ -416,3 +416,38 @@ def test_cat_gelu_and_fused_gate_layernorm_oracle():
     q, h = O.gate_residual_layernorm_mod_fp8(a, g, x, sc, sh, [0.03], 3, "bf16")
     assert np.array_equal(h, O.gate_residual(a, g, x, 3, "bf16"))
     assert np.array_equal(q, O.layernorm_mod_fp8(h, sc, sh, [0.03], 3, "bf16"))
+
+
+def test_weight_only_quantize_and_layout_oracle():
+    # hand-computed: column 0 has amax 2.0 -> scale 2/128; 2.0 -> 128 -> clipped to 127, -2.0 -> -128, ties go away
+    w = np.array([[2.0, 0.7, 0.0], [-2.0, -0.35, 0.0], [0.0234375, 0.1, 0.0], [-0.0234375, 0.0, 0.0]], np.float32)
+    q, s = O.weight_only_quantize(w, 8, "f16")
+    assert q[:, 0].tolist() == [127, -128, 2, -2]          # 0.0234375 / (2/128) = 1.5 -> 2 (away from zero), not 2 by ties-to-even alone: -1.5 -> -2
+    assert q[:, 2].tolist() == [0, 0, 0, 0] and s[2] == 0  # all-zero column
+    assert s[0] == np.float32(2.0 / 128) and q[:, 1].tolist() == [127, -64, 18, 0]
+    q4, s4 = O.weight_only_quantize(w, 4, "f16")
+    assert q4[:, 0].tolist() == [7, -8, 0, 0] and s4[0] == np.float32(0.25)
+    assert q4[:, 1].tolist() == [7, -4, 1, 0]              # 0.1 / 0.0875 = 1.14 -> 1
+    # 2.5-type ties: w / scale = 2.5 -> 3 (C round), rint would give 2
+    w2 = np.array([[128.0], [2.5], [-2.5], [0.5]], np.float32)
+    assert O.weight_only_quantize(w2, 8, "f16")[0][:, 0].tolist() == [127, 3, -3, 1]
+    # prepared layout: transposed, unsigned, int4 nibble order k0 k2 k4 k6 k1 k3 k5 k7
+    qk = np.arange(-8, 8, dtype=np.int8).reshape(16, 1)  # one channel, k = 16
+    p = O.weight_only_prepared(qk, 4)
+    assert p.shape == (1, 8)
+    words = p.view(np.uint32)[0]
+    assert [(int(words[0]) >> (4 * i)) & 0xF for i in range(8)] == [0, 2, 4, 6, 1, 3, 5, 7]       # codes u = q + 8 of k0..k7 are 0..7
+    assert [(int(words[1]) >> (4 * i)) & 0xF for i in range(8)] == [8, 10, 12, 14, 9, 11, 13, 15]
+    p8 = O.weight_only_prepared(np.array([[-128, 0], [127, -1]], np.int8), 8)
+    assert p8.tolist() == [[0, 255], [128, 127]]
+    # the GEMM contract against naive loops
+    rng = np.random.default_rng(41)
+    a = O.round_to(rng.standard_normal((3, 8)).astype(np.float32), "f16")
+    qq = rng.integers(-128, 128, (8, 5)).astype(np.int8)
+    sc = O.round_to(rng.random(5).astype(np.float32) * 0.01, "f16")
+    b = O.round_to(rng.standard_normal(5).astype(np.float32), "f16")
+    y = O.weight_only_gemm_f64(a, qq, sc, b, "f32")
+    for i in range(3):
+        for j in range(5):
+            ref = sum(float(a[i, t]) * int(qq[t, j]) for t in range(8)) * float(sc[j]) + float(b[j])
+            assert abs(float(y[i, j]) - ref) <= 1e-6 * max(1.0, abs(ref))

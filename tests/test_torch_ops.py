@@ -43,6 +43,23 @@ def test_shape_inference_without_a_gpu(tops):
         y4 = torch.ops.lyradiff.w4a4_linear(qa, w4, sa, sa[:3072], None)
         assert y4.shape == (4608, 3072) and y4.dtype == torch.bfloat16
         assert torch.ops.lyradiff.repack_weight(w4).shape == w4.shape
+        # FLUX FP8 block pieces
+        xs = torch.empty(2, 2304, 3072, dtype=torch.bfloat16, device=dev)
+        mod = torch.empty(2, 3072, dtype=torch.bfloat16, device=dev)
+        one = torch.empty(1, dtype=torch.float32, device=dev)
+        codes, hidden = torch.ops.lyradiff.gate_residual_layernorm_mod_fp8(xs, mod, xs, mod, mod, one)
+        assert codes.shape == xs.shape and codes.dtype == torch.uint8 and hidden.shape == xs.shape and hidden.dtype == xs.dtype
+        assert torch.ops.lyradiff.layernorm_mod_fp8(xs, mod, mod, one).dtype == torch.uint8
+        c2 = torch.ops.lyradiff.fp8_linear_codes(qf, wf, sf, sf, None, one, 1)
+        assert c2.shape == (4608, 12288) and c2.dtype == torch.uint8
+        wd = torch.empty(3072, 12288, dtype=torch.uint8, device=dev)
+        yg = torch.ops.lyradiff.fp8_linear_gated(c2, wd, one, one, None, mod[:1], xb, 4608)
+        assert yg.shape == (4608, 3072) and yg.dtype == torch.bfloat16
+        msa = torch.empty(6, 2, 3072, dtype=torch.bfloat16, device=dev)
+        b1, b2 = torch.empty(12288, dtype=torch.bfloat16, device=dev), torch.empty(3072, dtype=torch.bfloat16, device=dev)
+        out = torch.ops.lyradiff.flux_attn_post_fp8(xs, xs, msa, wf, one, one, b1, wd, one, one, b2)
+        assert out.shape == xs.shape and out.dtype == xs.dtype
+        assert torch.ops.lyradiff.lora_down(xb, torch.empty(32, 3072, dtype=torch.bfloat16, device=dev)).shape == (4608, 32)
 
 
 def test_host_tensors_are_rejected(tops):
@@ -77,3 +94,27 @@ def test_operators_match_direct_wrappers(tops, dev):
     assert torch.equal(torch.ops.lyradiff.w4a4_linear(qa, w4, sa, sa[:128].contiguous(), None),
                        ops.w4a4_linear(qa, w4, sa, sa[:128].contiguous(), None))
     assert np.isfinite(torch.ops.lyradiff.fp8_scale_cast(xb, sf).float().cpu().numpy()).all()
+
+
+@pytest.mark.gpu
+def test_block_operators_match_the_python_functions(tops, dev):
+    from lyradiff_amd import flux_fp8 as F
+
+    g = torch.Generator().manual_seed(9)
+    b, s, d = 1, 160, 256
+    bf = lambda *shape, sc=1.0: (sc * torch.randn(*shape, generator=g)).bfloat16()
+    sd = {"p.net.0.proj.weight": bf(4 * d, d, sc=0.03), "p.net.0.proj.bias": bf(4 * d, sc=0.1),
+          "p.net.2.weight": bf(d, 4 * d, sc=0.03), "p.net.2.bias": bf(d, sc=0.1),
+          "p.net.0.proj_input_scale": torch.tensor([5.0 / 448]), "p.net.2_input_scale": torch.tensor([2.0 / 448]),
+          "p.proj_mlp.weight": bf(4 * d, d, sc=0.03), "p.proj_mlp.bias": bf(4 * d, sc=0.1),
+          "p.proj_out.weight": bf(d, 5 * d, sc=0.03), "p.proj_out.bias": bf(d, sc=0.1),
+          "p.proj_mlp_input_scale": torch.tensor([5.0 / 448]), "p.proj_out_input_scale": torch.tensor([4.0 / 448])}
+    wp, ws = F.load_flux_attn_post_fp8(sd, "p.", d, torch.bfloat16, dev), F.load_flux_single_mlp_fp8(sd, "p.", d, 4, torch.bfloat16, dev)
+    x, attn, norm = bf(b, s, d).to(dev), bf(b, s, d).to(dev), bf(b, s, d).to(dev)
+    msa = bf(6, b, d, sc=0.5).to(dev)
+    flat = lambda l: (l.weight_rows32, l.weight_scale, l.input_scale, l.bias)
+    got = torch.ops.lyradiff.flux_attn_post_fp8(x, attn, msa, *flat(wp.gelu_proj), *flat(wp.ff_linear))
+    assert torch.equal(got, F.flux_attn_post_fp8(x, attn, msa, wp))
+    gate = msa[2].contiguous()
+    got = torch.ops.lyradiff.flux_single_mlp_fp8(x, norm, attn, gate, *flat(ws.proj_mlp), *flat(ws.proj_out))
+    assert torch.equal(got, F.flux_single_mlp_fp8(x, norm, attn, gate, ws))
