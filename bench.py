@@ -266,6 +266,16 @@ def extra_kernels(torch, ops, dev):
     pre = (torch.rand(d, generator=g) + 0.5).to(dev)
     us = timeit(lambda: ops.geglu_int8_dynamic(x, b, pre))
     res[f"geglu_int8_{m}x{d}"] = {"us": round(us, 2), "GB/s": round(5.0 * m * d / us / 1e3, 1)}
+    # weight-only GEMM (16-bit activations, int8 / int4 weights) at the FLUX up-projection shape
+    m, n, k = 4608, 12288, 3072
+    for dt, name in ((torch.float16, "f16"), (torch.bfloat16, "bf16")):
+        x = torch.randn(m, k, generator=g).to(dt).to(dev)
+        sc = (torch.rand(n, generator=g) * 0.01).to(dt).to(dev)
+        for kind in ("int8", "int4"):
+            q = torch.randint(-128, 128, (k, n if kind == "int8" else n // 2), generator=g, dtype=torch.int8).to(dev)
+            wp = ops.repack_weight_only(q, kind)
+            us = timeit(lambda: ops.weight_only_linear(x, wp, sc, None, kind), iters=20, warm=3)
+            res[f"gemm_weight_only_{kind}_{name}_{m}x{n}x{k}"] = {"us": round(us, 2), "TFLOP/s": round(2.0 * m * n * k / us / 1e6, 1)}
     res.update(flux_block_times(torch, ops, dev, timeit))
     return res
 

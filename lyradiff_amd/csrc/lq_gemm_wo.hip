@@ -20,7 +20,7 @@
 // Tiling: 256x128 outputs per workgroup of four wavefronts (2x2), 128x64 per wavefront (eight 32x32 MFMA tiles:
 // every converted weight fragment is used by four MFMAs), k-tile 64, two LDS stages filled from registers
 // (activations XOR-swizzled, weights copied as they lie), the next tile's global loads in flight during the MFMAs.
-#include "lq_common.h"
+#include "lq_gemm_core.h"
 
 namespace lq {
 
@@ -73,23 +73,29 @@ template <> struct WoCvt<false, true> {  // bf16 <- uint4
     }
 };
 
-template <typename Tag, bool W4>
-__global__ __launch_bounds__(256, 2) void wo_gemm_kernel(void* __restrict__ C, const void* __restrict__ A,
-                                                         const uint8_t* __restrict__ B, const void* __restrict__ scales,
-                                                         const void* __restrict__ bias, int m, int n, int k, int tiles_m,
-                                                         int tiles_n) {
+// WN = 2: 256x128 outputs, four wavefronts, two workgroups per CU.  WN = 4: 256x256 outputs, eight wavefronts, one
+// workgroup per CU (more operand reuse per LDS byte; the choice for large problems).
+template <typename Tag, bool W4, int WN, int NSTAGE>
+__global__ __launch_bounds__(128 * WN, (WN == 2 ? 2 : 1)) void wo_gemm_kernel(void* __restrict__ C, const void* __restrict__ A,
+                                                                              const uint8_t* __restrict__ B,
+                                                                              const void* __restrict__ scales,
+                                                                              const void* __restrict__ bias, int m, int n, int k,
+                                                                              int tiles_m, int tiles_n) {
     constexpr bool F16 = std::is_same<Tag, F16Tag>::value;
-    constexpr int BM = 256, BN = 128, BK = 64, TM = 128, TN = 64, MT = 4, NT = 2;
+    constexpr int NW = 2 * WN, BM = 256, BN = 64 * WN, BK = 64, TM = 128, TN = 64, MT = 4, NT = 2;
     constexpr int A_BYTES = BM * BK * 2;                 // 32 KiB
     constexpr int BCH = W4 ? 2 : 4;                      // 16-byte weight chunks per row per k-tile
-    constexpr int B_BYTES = BN * BCH * 16;               // 8 or 4 KiB
+    constexpr int B_BYTES = BN * BCH * 16;
     constexpr int STAGE = A_BYTES + B_BYTES;
-    constexpr int A_LD = A_BYTES / 16 / 256;             // 16-byte loads per thread per tile (8)
-    constexpr int B_LD = B_BYTES / 16 / 256;             // 2 or 1
-    static_assert(B_LD * 256 * 16 == B_BYTES, "weight stage is a whole number of 16-byte loads per thread");
+    constexpr int A_DMA = A_BYTES / 1024 / NW;           // 1 KiB transfers per wavefront per tile
+    constexpr int B_DMA = B_BYTES / 1024 / NW;
+    constexpr int PER_TILE = A_DMA + B_DMA;
+    static_assert(A_DMA * NW * 1024 == A_BYTES && B_DMA * NW * 1024 == B_BYTES && B_DMA >= 1, "stage / wavefront mismatch");
+    static_assert(PER_TILE * NSTAGE < 64, "vmcnt is a 6-bit counter");
     extern __shared__ __attribute__((aligned(16))) char wo_smem[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
     // consecutive workgroup ids of one XCD (ids congruent modulo 8) walk down a column of tiles, so that an XCD's
     // L2 keeps one weight panel and streams activations
     int bid = blockIdx.x;
@@ -102,37 +108,35 @@ __global__ __launch_bounds__(256, 2) void wo_gemm_kernel(void* __restrict__ C, c
     const size_t b_row_bytes = W4 ? (size_t)k / 2 : (size_t)k;
     const size_t b_blk = b_row_bytes * 32;  // bytes per block of 32 output channels
     const int row_last = m - 1 - m0, blk_last = n / 32 - 1 - n0 / 32;
+    const u32 smem_base = (u32)(uintptr_t)(__attribute__((address_space(3))) char*)wo_smem;
 
-    // ---- global -> register -> LDS plan (32-bit per-lane offsets from wavefront-uniform tile bases) -------------
+    // ---- global -> LDS transfers without registers: lane l of a transfer lands at (transfer base) + 16*l, so the
+    // XOR swizzle of the activation tile is applied by choosing WHICH global chunk each lane fetches ----------------
     const char* a_tile = static_cast<const char*>(A) + (size_t)m0 * a_pitch;
     const char* b_tile = reinterpret_cast<const char*>(B) + (size_t)(n0 / 32) * b_blk;
-    u32 a_voff[A_LD];
-    const int a_r0 = tid >> 3, a_c = tid & 7;
-    // row i*32 + a_r0 of the tile: the swizzle only looks at the low four row bits, so it is the same for every i
-    const int a_dst0 = a_r0 * 128 + ((a_c ^ wo_swizzle<8>(a_r0)) << 4);
+    u32 a_voff[A_DMA], b_voff[B_DMA];
 #pragma unroll
-    for (int i = 0; i < A_LD; ++i) a_voff[i] = (u32)min(i * 32 + a_r0, row_last) * (u32)a_pitch + a_c * 16;
-    u32 b_voff[B_LD];
+    for (int i = 0; i < A_DMA; ++i) {
+        const int slot = (wave * A_DMA + i) * 64 + lane;  // 16-byte slot of the activation stage: [row][8 chunks]
+        const int row = slot >> 3, c = (slot & 7) ^ wo_swizzle<8>(row);
+        a_voff[i] = (u32)min(row, row_last) * (u32)a_pitch + c * 16;
+    }
 #pragma unroll
-    for (int i = 0; i < B_LD; ++i) {
-        const int slot = i * 256 + tid;  // [block of 32 channels][chunk][row in block]
+    for (int i = 0; i < B_DMA; ++i) {
+        const int slot = (wave * B_DMA + i) * 64 + lane;  // [block of 32 channels][chunk][row in block], as in memory
         const int blk = slot / (BCH * 32), within = slot % (BCH * 32);
         b_voff[i] = (u32)((size_t)min(blk, blk_last) * b_blk) + within * 16;
     }
-    v4i ra[A_LD], rb[B_LD];
-#define LQ_WO_FETCH(KT)                                                                                          \
-    do {                                                                                                         \
-        const char* ga = a_tile + (size_t)(KT) * (BK * 2);                                                       \
-        const char* gb = b_tile + (size_t)(KT) * (BCH * 512);                                                    \
-        _Pragma("unroll") for (int i = 0; i < A_LD; ++i) ra[i] = *reinterpret_cast<const v4i*>(ga + a_voff[i]);  \
-        _Pragma("unroll") for (int i = 0; i < B_LD; ++i) rb[i] = *reinterpret_cast<const v4i*>(gb + b_voff[i]);  \
-    } while (0)
-#define LQ_WO_STASH(STAGE_IDX)                                                                                            \
-    do {                                                                                                                  \
-        char* s = wo_smem + (STAGE_IDX) * STAGE;                                                                          \
-        _Pragma("unroll") for (int i = 0; i < A_LD; ++i) *reinterpret_cast<v4i*>(s + a_dst0 + i * (32 * 128)) = ra[i];    \
-        _Pragma("unroll") for (int i = 0; i < B_LD; ++i) *reinterpret_cast<v4i*>(s + A_BYTES + (i * 256 + tid) * 16) = rb[i]; \
-    } while (0)
+    auto issue = [&](int kt, int stage) {
+        const char* ga = a_tile + (size_t)kt * (BK * 2);
+        const char* gb = b_tile + (size_t)kt * (BCH * 512);
+        const u32 sa = smem_base + stage * STAGE + wave * (A_DMA * 1024);
+        const u32 sb = smem_base + stage * STAGE + A_BYTES + wave * (B_DMA * 1024);
+#pragma unroll
+        for (int i = 0; i < A_DMA; ++i) dma16(ga, a_voff[i], sa + i * 1024);
+#pragma unroll
+        for (int i = 0; i < B_DMA; ++i) dma16(gb, b_voff[i], sb + i * 1024);
+    };
 
     v16f acc[MT][NT];
 #pragma unroll
@@ -187,19 +191,19 @@ __global__ __launch_bounds__(256, 2) void wo_gemm_kernel(void* __restrict__ C, c
         }
     };
 
-    LQ_WO_FETCH(0);
-    LQ_WO_STASH(0);
-    __syncthreads();
-    // The prefetch is unconditional (past the end it re-reads the last tile into the stage nobody reads again): with
-    // a branch around it the compiler parks the prefetch registers in scratch memory and the overlap is lost.
+    // Tile t lives in stage t % NSTAGE.  Every iteration issues exactly one tile of transfers (past the end it
+    // re-fetches the last tile into a stage nobody reads again), so the vmcnt threshold is a compile-time value:
+    // when at most (NSTAGE-2) tiles of this wavefront's transfers are outstanding, its part of tile kt has landed;
+    // after the barrier everybody's has, and everybody has finished reading the stage that is re-armed next.
+#pragma unroll
+    for (int t = 0; t < NSTAGE - 1; ++t) issue(min(t, ktiles - 1), t);
     for (int kt = 0; kt < ktiles; ++kt) {
-        LQ_WO_FETCH(min(kt + 1, ktiles - 1));
-        compute(kt & 1);
-        LQ_WO_STASH((kt + 1) & 1);
+        wait_vmcnt<PER_TILE*(NSTAGE - 2)>();
         __syncthreads();
+        issue(min(kt + NSTAGE - 1, ktiles - 1), (kt + NSTAGE - 1) % NSTAGE);
+        compute(kt % NSTAGE);
     }
-#undef LQ_WO_FETCH
-#undef LQ_WO_STASH
+    wait_vmcnt<0>();  // nothing in flight towards LDS when the workgroup ends
 
     // ---- epilogue: weights were the first MFMA operand, so a lane holds one activation row (lr) and, per tile,
     // four runs of four consecutive output channels: 8-byte stores -------------------------------------------------
@@ -301,30 +305,40 @@ extern "C" int lq_gemm_weight_only(void* C, const void* A, lq_dtype_t dtype, con
                    reinterpret_cast<uintptr_t>(bias) % 8 == 0,
                LQ_ERR_ARG, "lq_gemm_weight_only: A and B must be 16-byte, C, scales and bias 8-byte aligned");
     if (m == 0) return LQ_OK;
-    const int tiles_m = (m + 255) / 256, tiles_n = (n + 127) / 128;
     const bool w4 = kind == LQ_W_INT4;
-    const size_t lds = 2 * (size_t)(256 * 64 * 2 + 128 * (w4 ? 2 : 4) * 16);
-    dim3 grid((unsigned)(tiles_m * tiles_n)), block(256);
+    // 256x256 tiles (eight wavefronts, three stages) once they give every CU work; 256x128 tiles otherwise
+    const long big_tiles = (long)((m + 255) / 256) * ((n + 255) / 256);
+    const bool big = big_tiles >= 192;
     hipStream_t st = as_stream(stream);
-#define LQ_WO_GO(TAG, W4V)                                                                                              \
+#define LQ_WO_GO(TAG, W4V, WNV, NST)                                                                                    \
     do {                                                                                                                \
+        constexpr size_t lds = (size_t)(NST) * (256 * 64 * 2 + 64 * (WNV) * ((W4V) ? 2 : 4) * 16);                      \
         static bool attr_done = false;                                                                                  \
         if (!attr_done) {                                                                                               \
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&wo_gemm_kernel<TAG, W4V>),                           \
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&wo_gemm_kernel<TAG, W4V, WNV, NST>),                 \
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {              \
                 set_error("lq_gemm_weight_only: cannot raise the dynamic LDS limit to %zu bytes", lds);                 \
                 return LQ_ERR_HIP;                                                                                      \
             }                                                                                                           \
             attr_done = true;                                                                                           \
         }                                                                                                               \
-        hipLaunchKernelGGL((wo_gemm_kernel<TAG, W4V>), grid, block, lds, st, C, A, B_prepared, scales, bias, m, n, k,   \
-                           tiles_m, tiles_n);                                                                           \
+        const int tiles_m = (m + 255) / 256, tiles_n = (n + 64 * (WNV) - 1) / (64 * (WNV));                             \
+        hipLaunchKernelGGL((wo_gemm_kernel<TAG, W4V, WNV, NST>), dim3((unsigned)(tiles_m * tiles_n)), dim3(128 * (WNV)), \
+                           lds, st, C, A, B_prepared, scales, bias, m, n, k, tiles_m, tiles_n);                         \
     } while (0)
-    if (dtype == LQ_F16) {
-        if (w4) LQ_WO_GO(F16Tag, true); else LQ_WO_GO(F16Tag, false);
-    } else {
-        if (w4) LQ_WO_GO(BF16Tag, true); else LQ_WO_GO(BF16Tag, false);
-    }
+#define LQ_WO_KIND(TAG)                                       \
+    do {                                                      \
+        if (big) {                                            \
+            if (w4) LQ_WO_GO(TAG, true, 4, 3);                \
+            else LQ_WO_GO(TAG, false, 4, 3);                  \
+        } else {                                              \
+            if (w4) LQ_WO_GO(TAG, true, 2, 2);                \
+            else LQ_WO_GO(TAG, false, 2, 2);                  \
+        }                                                     \
+    } while (0)
+    if (dtype == LQ_F16) LQ_WO_KIND(F16Tag);
+    else LQ_WO_KIND(BF16Tag);
+#undef LQ_WO_KIND
 #undef LQ_WO_GO
     return check_launch("gemm_weight_only");
 }
