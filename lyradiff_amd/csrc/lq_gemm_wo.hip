@@ -32,44 +32,52 @@ template <int CH> __device__ __forceinline__ int wo_swizzle(int row) {  // 8 chu
     return ((row >> 1) & 7) ^ ((row & 1) << 2);
 }
 
-// eight consecutive-k weights of one output channel as 16-bit floats (four dwords), from unsigned codes
+// eight consecutive-k weights of one output channel as 16-bit floats (one 16-byte MFMA operand), from unsigned codes
 template <bool F16, bool W4> struct WoCvt;
 template <> struct WoCvt<true, false> {  // fp16 <- uint8: d0 holds k0..k3, d1 holds k4..k7
-    static __device__ __forceinline__ void run(u32 d0, u32 d1, u32* o) {
+    static __device__ __forceinline__ v4i run(u32 d0, u32 d1) {
+        v4i o;
         const h2_t off = {(_Float16)1152.0f, (_Float16)1152.0f};
         const u32 p[4] = {__builtin_amdgcn_perm(0x64646464u, d0, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, d0, 0x04030402u),
                           __builtin_amdgcn_perm(0x64646464u, d1, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, d1, 0x04030402u)};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = __builtin_bit_cast(u32, __builtin_bit_cast(h2_t, p[i]) - off);
+        for (int i = 0; i < 4; ++i) o[i] = __builtin_bit_cast(int, __builtin_bit_cast(h2_t, p[i]) - off);
+        return o;
     }
 };
 template <> struct WoCvt<true, true> {  // fp16 <- uint4: d0 holds k0..k7 in the interleaved nibble order
-    static __device__ __forceinline__ void run(u32 d0, u32, u32* o) {
+    static __device__ __forceinline__ v4i run(u32 d0, u32) {
+        v4i o;
         const h2_t off = {(_Float16)1032.0f, (_Float16)1032.0f};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const u32 p = ((d0 >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
-            o[i] = __builtin_bit_cast(u32, __builtin_bit_cast(h2_t, p) - off);
+            o[i] = __builtin_bit_cast(int, __builtin_bit_cast(h2_t, p) - off);
         }
+        return o;
     }
 };
 template <> struct WoCvt<false, false> {  // bf16 <- uint8 (through fp32: bf16 cannot hold 1024 + u)
-    static __device__ __forceinline__ void run(u32 d0, u32 d1, u32* o) {
+    static __device__ __forceinline__ v4i run(u32 d0, u32 d1) {
+        v4i o;
         const u32 d[2] = {d0, d1};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const u32 w = d[i >> 1] >> (16 * (i & 1));
-            o[i] = pack2_bf16((float)(w & 0xFFu) - 128.0f, (float)((w >> 8) & 0xFFu) - 128.0f);
+            o[i] = (int)pack2_bf16((float)(w & 0xFFu) - 128.0f, (float)((w >> 8) & 0xFFu) - 128.0f);
         }
+        return o;
     }
 };
 template <> struct WoCvt<false, true> {  // bf16 <- uint4
-    static __device__ __forceinline__ void run(u32 d0, u32, u32* o) {
+    static __device__ __forceinline__ v4i run(u32 d0, u32) {
+        v4i o;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const u32 w = d0 >> (4 * i);
-            o[i] = pack2_bf16((float)(w & 0xFu) - 8.0f, (float)((w >> 16) & 0xFu) - 8.0f);
+            o[i] = (int)pack2_bf16((float)(w & 0xFu) - 8.0f, (float)((w >> 16) & 0xFu) - 8.0f);
         }
+        return o;
     }
 };
 
@@ -149,46 +157,68 @@ __global__ __launch_bounds__(128 * WN, (WN == 2 ? 2 : 1)) void wo_gemm_kernel(vo
     const int lr = lane & 31, lh = lane >> 5;
     const int xrow = wm * TM + lr;
     const int xsw = wo_swizzle<8>(xrow);  // unchanged by +32*i
+    // One k-tile = 16 steps (half, s, i): one 16-byte activation fragment and NT MFMAs each.  Fragments are read two
+    // steps ahead of their use and the order "read, NT MFMAs" is pinned with scheduling barriers, so that the matrix
+    // pipe does not wait for an LDS round trip at every step; the weights of the second half are converted while
+    // the MFMAs of the first half run.
     auto compute = [&](int stage) {
         const char* sa = wo_smem + stage * STAGE;
         const char* sb = sa + A_BYTES + (wn * NT) * (BCH * 512) + lr * 16;
-        uint4 w4raw[NT];  // int4: one 16-byte read holds the lane's 32 weights of the whole k-tile
-        if constexpr (W4) {
+        auto xptr = [&](int t) -> const v4i* {
+            const int half = t >> 3, s2 = (t >> 2) & 1, i = t & 3;
+            const int chunk = W4 ? lh * 4 + half * 2 + s2 : half * 4 + lh * 2 + s2;
+            return reinterpret_cast<const v4i*>(sa + (xrow + i * 32) * 128 + ((chunk ^ xsw) << 4));
+        };
+        v4i wraw[2][NT];  // int8: one 16-byte chunk per half; int4: one chunk for the whole tile (kept in wraw[0])
 #pragma unroll
-            for (int j = 0; j < NT; ++j) w4raw[j] = *reinterpret_cast<const uint4*>(sb + j * (BCH * 512) + lh * 512);
+        for (int j = 0; j < NT; ++j) {
+            if constexpr (W4) wraw[0][j] = *reinterpret_cast<const v4i*>(sb + j * (BCH * 512) + lh * 512);
+            else {
+                wraw[0][j] = *reinterpret_cast<const v4i*>(sb + j * (BCH * 512) + lh * 512);
+                wraw[1][j] = *reinterpret_cast<const v4i*>(sb + j * (BCH * 512) + (2 + lh) * 512);
+            }
         }
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {  // two MFMA k-steps per weight chunk read (int8) / per pair of dwords (int4)
-            u32 wfrag[NT][2][4];
+        v4i xb[3];
+        xb[0] = *xptr(0);
+        xb[1] = *xptr(1);
+        v4i wfrag[2][NT][2];
+        auto convert = [&](int half) {
 #pragma unroll
             for (int j = 0; j < NT; ++j) {
                 if constexpr (W4) {
-                    WoCvt<F16, true>::run(half ? w4raw[j].z : w4raw[j].x, 0u, wfrag[j][0]);
-                    WoCvt<F16, true>::run(half ? w4raw[j].w : w4raw[j].y, 0u, wfrag[j][1]);
+                    wfrag[half][j][0] = WoCvt<F16, true>::run((u32)(half ? wraw[0][j][2] : wraw[0][j][0]), 0u);
+                    wfrag[half][j][1] = WoCvt<F16, true>::run((u32)(half ? wraw[0][j][3] : wraw[0][j][1]), 0u);
                 } else {
-                    const uint4 d = *reinterpret_cast<const uint4*>(sb + j * (BCH * 512) + (half * 2 + lh) * 512);
-                    WoCvt<F16, false>::run(d.x, d.y, wfrag[j][0]);
-                    WoCvt<F16, false>::run(d.z, d.w, wfrag[j][1]);
+                    wfrag[half][j][0] = WoCvt<F16, false>::run((u32)wraw[half][j][0], (u32)wraw[half][j][1]);
+                    wfrag[half][j][1] = WoCvt<F16, false>::run((u32)wraw[half][j][2], (u32)wraw[half][j][3]);
                 }
             }
+        };
+        convert(0);
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                // activation chunk that holds the same eight k as wfrag[.][s]
-                const int chunk = W4 ? lh * 4 + half * 2 + s : half * 4 + lh * 2 + s;
+        for (int t = 0; t < 16; ++t) {
+            const int half = t >> 3, s2 = (t >> 2) & 1, i = t & 3;
+            if (t + 2 < 16) xb[(t + 2) % 3] = *xptr(t + 2);
+            if (t == 2) convert(1);
+            const v4i x = xb[t % 3];
 #pragma unroll
-                for (int i = 0; i < MT; ++i) {
-                    const uint4 x = *reinterpret_cast<const uint4*>(sa + (xrow + i * 32) * 128 + ((chunk ^ xsw) << 4));
-#pragma unroll
-                    for (int j = 0; j < NT; ++j) {
-                        const uint4 w = make_uint4(wfrag[j][s][0], wfrag[j][s][1], wfrag[j][s][2], wfrag[j][s][3]);
-                        if constexpr (F16)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, w), __builtin_bit_cast(v8h, x), acc[i][j], 0, 0, 0);
-                        else
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, w), __builtin_bit_cast(v8bf, x), acc[i][j], 0, 0, 0);
-                    }
-                }
+            for (int j = 0; j < NT; ++j) {
+                const v4i w = wfrag[half][j][s2];
+                if constexpr (F16)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, w), __builtin_bit_cast(v8h, x), acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, w), __builtin_bit_cast(v8bf, x), acc[i][j], 0, 0, 0);
             }
         }
+        // pin the order: the weight chunks and the first two fragments, then (NT MFMAs, one LDS read) x 14, then the
+        // MFMAs of the last two steps
+        __builtin_amdgcn_sched_group_barrier(0x100, (W4 ? NT : 2 * NT) + 2, 0);  // DS reads
+#pragma unroll
+        for (int t = 0; t < 14; ++t) {
+            __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);  // MFMA
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // DS read
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * NT, 0);
     };
 
     // Tile t lives in stage t % NSTAGE.  Every iteration issues exactly one tile of transfers (past the end it
