@@ -33,11 +33,13 @@ template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
 
 using namespace lq;
 
+// LQ_OK: go on; 1: m == 0, nothing to do (pointers of empty tensors may be null); negative: error
 static int fp8_check(const char* what, const void* C, const uint8_t* A, const uint8_t* B, const float* a_scale, const float* b_scale,
                      const void* bias, const void* residual, int m, int n, int k) {
-    LQ_REQUIRE(A && B && a_scale && b_scale, LQ_ERR_ARG, "%s: null pointer", what);
     LQ_REQUIRE(m >= 0 && n > 0 && k > 0 && n % 32 == 0 && k % 64 == 0, LQ_ERR_SHAPE,
                "%s: need n %% 32 == 0 and k %% 64 == 0 (m=%d n=%d k=%d)", what, m, n, k);
+    if (m == 0) return 1;
+    LQ_REQUIRE(A && B && a_scale && b_scale, LQ_ERR_ARG, "%s: null pointer", what);
     LQ_REQUIRE(reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(C) % 16 == 0 && reinterpret_cast<uintptr_t>(bias) % 8 == 0 &&
                    reinterpret_cast<uintptr_t>(residual) % 16 == 0,
@@ -59,9 +61,9 @@ extern "C" int lq_gemm_fp8_ex(void* C, lq_dtype_t out_dtype, const uint8_t* A, c
                               const float* a_scale, const float* b_scale, const void* bias, int gelu,
                               const void* residual, float beta, int m, int n, int k, float* out_scale, uint8_t* C_fp8,
                               const float* C_fp8_scale, lq_stream_t stream) {
-    LQ_REQUIRE(C || C_fp8, LQ_ERR_ARG, "lq_gemm_fp8: null pointer");
     int rc = fp8_check("lq_gemm_fp8", C, A, B_rows32, a_scale, b_scale, bias, residual, m, n, k);
-    if (rc != LQ_OK) return rc;
+    if (rc != LQ_OK) return rc > 0 ? LQ_OK : rc;
+    LQ_REQUIRE(C || C_fp8, LQ_ERR_ARG, "lq_gemm_fp8: null pointer");
     LQ_REQUIRE((C_fp8 == nullptr) == (C_fp8_scale == nullptr), LQ_ERR_ARG, "lq_gemm_fp8: C_fp8 and C_fp8_scale go together");
     LQ_REQUIRE(reinterpret_cast<uintptr_t>(C_fp8) % 4 == 0, LQ_ERR_ARG, "lq_gemm_fp8: C_fp8 must be 4-byte aligned");
     LQ_REQUIRE(gelu >= 0 && gelu <= 2, LQ_ERR_ARG, "lq_gemm_fp8: gelu must be 0, 1 or 2");
@@ -77,7 +79,7 @@ extern "C" int lq_gemm_fp8_ex(void* C, lq_dtype_t out_dtype, const uint8_t* A, c
 extern "C" int lq_gemm_fp8(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32,
                            const float* a_scale, const float* b_scale, const void* bias, int gelu,
                            const void* residual, float beta, int m, int n, int k, lq_stream_t stream) {
-    LQ_REQUIRE(C != nullptr, LQ_ERR_ARG, "lq_gemm_fp8: null pointer");
+    LQ_REQUIRE(C != nullptr || m == 0, LQ_ERR_ARG, "lq_gemm_fp8: null pointer");
     return lq_gemm_fp8_ex(C, out_dtype, A, B_rows32, a_scale, b_scale, bias, gelu, residual, beta, m, n, k, nullptr, nullptr,
                           nullptr, stream);
 }
@@ -85,9 +87,9 @@ extern "C" int lq_gemm_fp8(void* C, lq_dtype_t out_dtype, const uint8_t* A, cons
 extern "C" int lq_gemm_fp8_gated(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32,
                                  const float* a_scale, const float* b_scale, const void* bias, const void* gate,
                                  size_t rows_per_gate, const void* residual, int m, int n, int k, lq_stream_t stream) {
-    LQ_REQUIRE(C && gate && residual, LQ_ERR_ARG, "lq_gemm_fp8_gated: null pointer");
     int rc = fp8_check("lq_gemm_fp8_gated", C, A, B_rows32, a_scale, b_scale, bias, residual, m, n, k);
-    if (rc != LQ_OK) return rc;
+    if (rc != LQ_OK) return rc > 0 ? LQ_OK : rc;
+    LQ_REQUIRE(C && gate && residual, LQ_ERR_ARG, "lq_gemm_fp8_gated: null pointer");
     LQ_REQUIRE(rows_per_gate > 0, LQ_ERR_SHAPE, "lq_gemm_fp8_gated: rows_per_gate must be positive");
     LQ_REQUIRE(reinterpret_cast<uintptr_t>(gate) % 16 == 0, LQ_ERR_ARG, "lq_gemm_fp8_gated: gate must be 16-byte aligned");
     if (m == 0) return LQ_OK;
@@ -101,13 +103,13 @@ extern "C" int lq_gemm_fp8_gated(void* C, lq_dtype_t out_dtype, const uint8_t* A
 extern "C" int lq_gemm_fp8_codes(uint8_t* C_fp8, size_t ldc, const float* C_fp8_scale, lq_dtype_t round_dtype,
                                  const uint8_t* A, const uint8_t* B_rows32, const float* a_scale, const float* b_scale,
                                  const void* bias, int gelu, int m, int n, int k, lq_stream_t stream) {
-    LQ_REQUIRE(C_fp8 && C_fp8_scale, LQ_ERR_ARG, "lq_gemm_fp8_codes: null pointer");
+    LQ_REQUIRE(gelu >= 0 && gelu <= 2, LQ_ERR_ARG, "lq_gemm_fp8_codes: gelu must be 0, 1 or 2");
+    LQ_REQUIRE(ldc >= (size_t)(n > 0 ? n : 0) && ldc % 4 == 0, LQ_ERR_SHAPE, "lq_gemm_fp8_codes: need ldc >= n and ldc %% 4 == 0 (ldc=%zu n=%d)", ldc, n);
     int rc = fp8_check("lq_gemm_fp8_codes", nullptr, A, B_rows32, a_scale, b_scale, bias, nullptr, m, n, k);
-    if (rc != LQ_OK) return rc;
+    if (rc != LQ_OK) return rc > 0 ? LQ_OK : rc;
+    LQ_REQUIRE(C_fp8 && C_fp8_scale, LQ_ERR_ARG, "lq_gemm_fp8_codes: null pointer");
     LQ_REQUIRE(ldc >= (size_t)n && ldc % 4 == 0 && reinterpret_cast<uintptr_t>(C_fp8) % 4 == 0, LQ_ERR_SHAPE,
                "lq_gemm_fp8_codes: need ldc >= n, ldc %% 4 == 0 and a 4-byte aligned destination (ldc=%zu n=%d)", ldc, n);
-    LQ_REQUIRE(gelu >= 0 && gelu <= 2, LQ_ERR_ARG, "lq_gemm_fp8_codes: gelu must be 0, 1 or 2");
-    if (m == 0) return LQ_OK;
     GemmParams p = {};
     p.A = A; p.B = B_rows32; p.bias = bias; p.a_scale = a_scale; p.b_scale = b_scale; p.gelu = gelu;
     p.C8 = C_fp8; p.c8_scale = C_fp8_scale; p.ldc8 = ldc;

@@ -234,12 +234,11 @@ template <typename Tag, int QMODE, int RESID, bool MOD> static int launch_ln(con
 }
 
 static int check_ln_common(const char* what, const void* dst, const void* src, lq_dtype_t dtype, size_t rows, size_t dim) {
-    LQ_REQUIRE(dst && src, LQ_ERR_ARG, "%s: null pointer", what);
+    LQ_REQUIRE((dst && src) || rows == 0, LQ_ERR_ARG, "%s: null pointer", what);
     LQ_REQUIRE(dtype == LQ_F16 || dtype == LQ_BF16, LQ_ERR_UNSUPPORTED, "%s: activations must be F16 or BF16", what);
     LQ_REQUIRE(dim > 0 && dim % 8 == 0 && dim <= 6144, LQ_ERR_SHAPE, "%s: need dim %% 8 == 0 and dim <= 6144 (dim=%zu)", what, dim);
     LQ_REQUIRE(reinterpret_cast<uintptr_t>(dst) % 8 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0, LQ_ERR_ARG,
                "%s: src must be 16-byte and dst 8-byte aligned", what);
-    (void)rows;
     return LQ_OK;
 }
 
@@ -294,6 +293,7 @@ extern "C" int lq_layernorm_mod_fp8_dual(uint8_t* dst_a, const float* input_scal
                                          size_t rows_per_batch, size_t dim, float eps, lq_stream_t stream) {
     int rc = check_ln_common("lq_layernorm_mod_fp8_dual", dst_a, src, dtype, batch * rows_per_batch, dim);
     if (rc != LQ_OK) return rc;
+    if (batch * rows_per_batch == 0) return LQ_OK;
     LQ_REQUIRE(dst_b && scale && shift && input_scale_a && input_scale_b, LQ_ERR_ARG, "lq_layernorm_mod_fp8_dual: null pointer");
     LQ_REQUIRE(reinterpret_cast<uintptr_t>(scale) % 16 == 0 && reinterpret_cast<uintptr_t>(shift) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(dst_b) % 8 == 0,
@@ -311,6 +311,7 @@ extern "C" int lq_gate_residual_layernorm_mod(void* dst, void* hidden_out, const
     const bool gated = attn != nullptr;
     int rc = check_ln_common("lq_gate_residual_layernorm_mod", dst, input, dtype, batch * rows_per_batch, dim);
     if (rc != LQ_OK) return rc;
+    if (batch * rows_per_batch == 0) return LQ_OK;
     LQ_REQUIRE(scale && shift, LQ_ERR_ARG, "lq_gate_residual_layernorm_mod: scale and shift are required");
     LQ_REQUIRE(gated == (gate != nullptr) && gated == (hidden_out != nullptr), LQ_ERR_ARG,
                "lq_gate_residual_layernorm_mod: attn, gate and hidden_out go together");
@@ -336,6 +337,7 @@ extern "C" int lq_gate_residual_layernorm_mod_fp8(uint8_t* dst, void* hidden_out
                                                   float eps, lq_stream_t stream) {
     int rc = check_ln_common("lq_gate_residual_layernorm_mod_fp8", dst, attn, dtype, batch * rows_per_batch, dim);
     if (rc != LQ_OK) return rc;
+    if (batch * rows_per_batch == 0) return LQ_OK;
     LQ_REQUIRE(hidden_out && gate && input && scale && shift && input_scale, LQ_ERR_ARG,
                "lq_gate_residual_layernorm_mod_fp8: null pointer");
     LQ_REQUIRE(reinterpret_cast<uintptr_t>(scale) % 16 == 0 && reinterpret_cast<uintptr_t>(shift) % 16 == 0 &&

@@ -386,3 +386,38 @@ def test_flux_single_mlp_int4_block(ops, dev):
     seq = x + gate[:, None, :] * (h1 + h2).view(b, s, d)
     assert_close_tol(to_np_f32(out).reshape(-1, d), to_np_f32(seq).reshape(-1, d), "flux int4 single-block tail",
                      abs_floor=2.0 ** -6 * (np.abs(to_np_f32(x).reshape(-1, d)) + np.abs(to_np_f32(seq).reshape(-1, d))) + 0.03)
+
+
+def test_new_entry_points_reject_bad_arguments_and_accept_empty_inputs(ops, dev):
+    """Error paths return a status and a message (nothing is launched); zero rows is a no-op."""
+    from lyradiff_amd.lib import LyraQuantError
+
+    qa, sa, wr, _, sw, bias = _fp8_operands(ops, dev, 64, 128, 64, 3, "bf16")
+    gate = torch.ones(1, 128, dtype=torch.bfloat16, device=dev)
+    res = torch.zeros(64, 128, dtype=torch.bfloat16, device=dev)
+    s_out = torch.tensor([0.02], dtype=torch.float32, device=dev)
+    with pytest.raises(ValueError):  # gate has the wrong number of rows for rows_per_gate
+        ops.fp8_linear_gated(qa, wr, sa, sw, bias, gate, res, 16)
+    with pytest.raises(LyraQuantError, match="gelu"):
+        ops.fp8_linear_codes(qa, wr, sa, sw, bias, s_out, gelu=3)
+    with pytest.raises(ValueError):  # destination too narrow for the column offset
+        ops.fp8_linear_codes(qa, wr, sa, sw, bias, s_out, out=torch.empty(64, 160, dtype=torch.uint8, device=dev), col_offset=64)
+    with pytest.raises(LyraQuantError, match="ldc"):  # row pitch not a multiple of 4
+        ops.fp8_linear_codes(qa, wr, sa, sw, bias, s_out, out=torch.empty(64, 130, dtype=torch.uint8, device=dev))
+    with pytest.raises(TypeError):
+        ops.fp8_linear_gated(qa, wr, sa, sw, bias, gate.half(), res, 64)
+    # zero rows: no launch, empty results
+    e = torch.empty(0, 64, dtype=torch.uint8, device=dev)
+    assert ops.fp8_linear_codes(e, wr, sa, sw, bias, s_out).shape == (0, 128)
+    assert ops.fp8_linear_gated(e, wr, sa, sw, bias, gate[:0], res[:0], 1).shape == (0, 128)
+    x0 = torch.empty(2, 0, 128, dtype=torch.bfloat16, device=dev)
+    mod = torch.zeros(2, 128, dtype=torch.bfloat16, device=dev)
+    q, h = ops.gate_residual_layernorm_mod_fp8(x0, mod, x0, mod, mod, s_out)
+    assert q.shape == (2, 0, 128) and h.shape == (2, 0, 128)
+    # NaN and infinity travel through the gate/residual epilogue and the codes as in the unfused kernels
+    qa2 = qa.clone()
+    sa_nan = torch.tensor([float("nan")], dtype=torch.float32, device=dev)
+    y = ops.fp8_linear_gated(qa2, wr, sa_nan, sw, bias, gate, res, 64)
+    assert torch.isnan(y).all()
+    codes = ops.fp8_linear_codes(qa2, wr, sa_nan, sw, bias, s_out)
+    assert ((codes & 0x7F) == 0x7F).all()
