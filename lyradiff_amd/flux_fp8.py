@@ -67,6 +67,33 @@ def load_flux_single_mlp_fp8(src, prefix: str, dim: int, mlp_scale: int = 4, dty
         load_fp8_linear(src, prefix, "proj_out", dim, (mlp_scale + 1) * dim, dtype, device, keep_master))
 
 
+def load_ada_fp8_layernorm(src, prefix: str, dim: int, n_chunks: int, dtype=torch.bfloat16, device="cuda",
+                           keep_master: bool = False) -> FP8Linear:
+    """Keys prefix + "linear" + {".weight", ".bias", "_input_scale"}, weight [n_chunks*D, D]
+    (AdaFP8LayerNormWeight.cc:36-92; the blocks pass prefix + "norm1." / "norm1_context." / "norm.")."""
+    return load_fp8_linear(src, prefix, "linear", n_chunks * dim, dim, dtype, device, keep_master)
+
+
+def ada_fp8_layernorm(x: torch.Tensor, temb: torch.Tensor, linear: FP8Linear, n_chunks: int, code_scales=(),
+                      switch_scale: bool = False, eps: float = 1e-6):
+    """AdaFP8LayerNorm<T>::forward (layers/ada_layer_norm/AdaFP8LayerNorm.cc:93-205): msa = FP8 linear of the
+    (already SiLU'd) time embedding, stored [n_chunks, B, D]; output = (1 + msa[1]) * LayerNorm(x) + msa[0]
+    (msa[0]/msa[1] swapped with switch_scale).  x [B, S, D], temb [B, D].
+    code_scales: () -> the 16-bit normalised tensor as the reference writes it; one or two fp32 [1] input scales ->
+    the e4m3 codes for the FP8 linears that consume it instead (cast fused, no 16-bit tensor).
+    Returns (norm | codes | (codes_a, codes_b), msa)."""
+    b, s, d = x.shape
+    q = ops.fp8_scale_cast(temb.reshape(b, d), linear.input_scale)
+    flat = ops.fp8_linear(q, linear.weight_rows32, linear.input_scale, linear.weight_scale, linear.bias, out_dtype=x.dtype)
+    msa = flat.view(b, n_chunks, d).transpose(0, 1).contiguous() if b > 1 else flat.view(n_chunks, 1, d)  # invokeTranspose102
+    shift, scale = (msa[1], msa[0]) if switch_scale else (msa[0], msa[1])
+    if len(code_scales) == 0:
+        return ops.gate_residual_layernorm_mod(x, scale, shift, eps=eps), msa
+    if len(code_scales) == 1:
+        return ops.layernorm_mod_fp8(x, scale, shift, code_scales[0], eps), msa
+    return ops.layernorm_mod_fp8_dual(x, scale, shift, code_scales[0], code_scales[1], eps), msa
+
+
 def flux_attn_post_fp8(x: torch.Tensor, attn_output: torch.Tensor, msa: torch.Tensor, w: FluxAttnPostFP8Weights,
                        eps: float = 1e-6) -> torch.Tensor:
     """x, attn_output [B, S, D]; msa [6, B, D] -> output [B, S, D] in three launches."""

@@ -421,3 +421,40 @@ def test_new_entry_points_reject_bad_arguments_and_accept_empty_inputs(ops, dev)
     assert torch.isnan(y).all()
     codes = ops.fp8_linear_codes(qa2, wr, sa_nan, sw, bias, s_out)
     assert ((codes & 0x7F) == 0x7F).all()
+
+
+@pytest.mark.parametrize("batch", [1, 3])
+def test_ada_fp8_layernorm(ops, dev, batch):
+    from lyradiff_amd import flux_fp8 as F
+
+    s, d, nch = 96, 256, 6
+    g = rng_t(80 + batch)
+    sd = _state_dict({"linear": (nch * d, d)}, 81)
+    sd["p.linear_input_scale"] = torch.tensor([4.0 / 448])
+    lin = F.load_ada_fp8_layernorm(sd, "p.", d, nch, torch.bfloat16, dev)
+    x = torch.randn(batch, s, d, generator=g).bfloat16().to(dev)
+    temb = torch.randn(batch, d, generator=g).bfloat16().to(dev)
+    norm, msa = F.ada_fp8_layernorm(x, temb, lin, nch)
+    assert msa.shape == (nch, batch, d) and norm.shape == x.shape
+    # msa against the oracle's FP8 GEMM contract on the same codes, chunk-major
+    q = O.fp8_scale_cast(to_np_f32(temb), float(lin.input_scale.cpu()[0]), True)
+    wq = ops.unpack_weight(lin.weight_rows32).cpu().numpy()
+    ref = O.fp8_gemm(q, wq, lin.input_scale.cpu().numpy(), lin.weight_scale.cpu().numpy(), to_np_f32(lin.bias), out_dtype="bf16")
+    ref = ref.reshape(batch, nch, d).transpose(1, 0, 2)
+    assert_close_tol(to_np_f32(msa), ref, "ada layernorm msa", abs_floor=2.0 ** -8 * np.abs(ref) + 1e-3)
+    # the normalised tensor and its fused-cast forms all come from the same kernel arithmetic
+    s1 = torch.tensor([0.02], dtype=torch.float32, device=dev)
+    s2 = torch.tensor([0.03], dtype=torch.float32, device=dev)
+    assert torch.equal(norm, ops.gate_residual_layernorm_mod(x, msa[1].contiguous(), msa[0].contiguous()))
+    c1, _ = F.ada_fp8_layernorm(x, temb, lin, nch, (s1,))
+    assert torch.equal(c1, ops.fp8_scale_cast(norm, s1))
+    (ca, cb), _ = F.ada_fp8_layernorm(x, temb, lin, nch, (s1, s2))
+    assert torch.equal(ca, c1) and torch.equal(cb, ops.fp8_scale_cast(norm, s2))
+    sw, _ = F.ada_fp8_layernorm(x, temb, lin, nch, switch_scale=True)
+    assert torch.equal(sw, ops.gate_residual_layernorm_mod(x, msa[0].contiguous(), msa[1].contiguous()))
+    # 16-bit output against the oracle's adaLN (statistics order differs: one ULP of T)
+    y = to_np_f32(norm).reshape(-1, d)
+    n = O._ln_normalised(to_np_f32(x).reshape(-1, d), 1e-6)
+    bidx = np.arange(batch * s) // s
+    want = O.round_to(O.round_to(O.round_to(to_np_f32(msa[1])[bidx] + 1.0, "bf16") * O.round_to(n, "bf16"), "bf16") + to_np_f32(msa[0])[bidx], "bf16")
+    assert (y != want).mean() < 0.02 and np.all(np.abs(y - want) <= 2.0 ** -7 * (np.abs(want) + np.abs(to_np_f32(msa[0])[bidx]) + 1.0))
