@@ -125,3 +125,74 @@ def flux_single_mlp_fp8(x: torch.Tensor, norm_hidden, attn_output: torch.Tensor,
     out = ops.fp8_linear_gated(q2, w.proj_out.weight_rows32, w.proj_out.input_scale, w.proj_out.weight_scale,
                                w.proj_out.bias, gate, x.view(m, d), rows_per_gate=s)
     return out.view(b, s, d)
+
+
+# ---- whole blocks around a caller-supplied attention --------------------------------------------------------------------
+# Everything the reference's FP8 blocks run through a quantized linear is here; `attention` is the caller's function
+# for the part in between (q/k RMSNorm, rotary embedding, scaled-dot-product attention), which is not quantized.
+
+@dataclass
+class FluxSingleBlockFP8Weights:
+    norm: FP8Linear      # prefix + "norm.linear"  [3D, D]
+    to_qkv: FP8Linear    # prefix + "attn.to_qkv"  [3D, D]
+    mlp: FluxSingleMlpFP8Weights
+
+
+@dataclass
+class FluxDoubleBlockFP8Weights:
+    norm1: FP8Linear           # prefix + "norm1.linear"          [6D, D]
+    norm1_context: FP8Linear   # prefix + "norm1_context.linear"  [6D, D]
+    to_qkv: FP8Linear          # prefix + "attn.to_qkv"
+    to_added_qkv: FP8Linear    # prefix + "attn.to_added_qkv"
+    to_out: FP8Linear          # prefix + "attn.to_out.0"
+    to_add_out: FP8Linear      # prefix + "attn.to_add_out"
+    ff: FluxAttnPostFP8Weights          # prefix + "ff."
+    ff_context: FluxAttnPostFP8Weights  # prefix + "ff_context."
+
+
+def load_flux_single_block_fp8(src, prefix: str, dim: int, mlp_scale: int = 4, dtype=torch.bfloat16, device="cuda",
+                               keep_master: bool = False) -> FluxSingleBlockFP8Weights:
+    """FluxSingleTransformerFP8BlockWeight::loadWeights (FluxSingleTransformerFP8BlockWeight.cc:94-121)."""
+    return FluxSingleBlockFP8Weights(load_ada_fp8_layernorm(src, prefix + "norm.", dim, 3, dtype, device, keep_master),
+                                     load_fp8_linear(src, prefix + "attn.", "to_qkv", 3 * dim, dim, dtype, device, keep_master),
+                                     load_flux_single_mlp_fp8(src, prefix, dim, mlp_scale, dtype, device, keep_master))
+
+
+def load_flux_double_block_fp8(src, prefix: str, dim: int, dtype=torch.bfloat16, device="cuda",
+                               keep_master: bool = False) -> FluxDoubleBlockFP8Weights:
+    """FluxTransformerFP8BlockWeight::loadWeights (FluxTransformerFP8BlockWeight.cc:78-91) and
+    FluxAttentionFP8ProcessorWeight::loadWeights (FluxAttentionFP8ProcessorWeight.cc:113-138)."""
+    lin = lambda name, n, k: load_fp8_linear(src, prefix + "attn.", name, n, k, dtype, device, keep_master)
+    return FluxDoubleBlockFP8Weights(load_ada_fp8_layernorm(src, prefix + "norm1.", dim, 6, dtype, device, keep_master),
+                                     load_ada_fp8_layernorm(src, prefix + "norm1_context.", dim, 6, dtype, device, keep_master),
+                                     lin("to_qkv", 3 * dim, dim), lin("to_added_qkv", 3 * dim, dim), lin("to_out.0", dim, dim),
+                                     lin("to_add_out", dim, dim),
+                                     load_flux_attn_post_fp8(src, prefix + "ff.", dim, dtype, device, keep_master),
+                                     load_flux_attn_post_fp8(src, prefix + "ff_context.", dim, dtype, device, keep_master))
+
+
+def _linear_from_codes(lin: FP8Linear, codes: torch.Tensor, dtype) -> torch.Tensor:
+    m = codes.numel() // codes.shape[-1]
+    y = ops.fp8_linear(codes.view(m, codes.shape[-1]), lin.weight_rows32, lin.input_scale, lin.weight_scale, lin.bias, out_dtype=dtype)
+    return y.view(*codes.shape[:-1], y.shape[-1])
+
+
+def flux_single_block_fp8(x: torch.Tensor, temb: torch.Tensor, w: FluxSingleBlockFP8Weights, attention) -> torch.Tensor:
+    """FluxSingleTransformerFP8Block<T>::forward (FluxSingleTransformerFP8Block.cc:163-291).  x [B, S, D], temb [B, D]
+    (SiLU already applied); attention(qkv [B, S, 3D]) -> [B, S, D].  One adaLN read yields the codes for to_qkv and for
+    proj_mlp; five launches besides the attention."""
+    (c_qkv, c_mlp), msa = ada_fp8_layernorm(x, temb, w.norm, 3, (w.to_qkv.input_scale, w.mlp.proj_mlp.input_scale))
+    attn_out = attention(_linear_from_codes(w.to_qkv, c_qkv, x.dtype))
+    return flux_single_mlp_fp8(x, c_mlp, attn_out.contiguous(), msa[2].contiguous(), w.mlp)
+
+
+def flux_double_block_fp8(x: torch.Tensor, context: torch.Tensor, temb: torch.Tensor, w: FluxDoubleBlockFP8Weights, attention):
+    """FluxTransformerFP8Block<T>::forward (FluxTransformerFP8Block.cc:159-262) with FluxAttentionFP8Processor
+    (FluxAttentionFP8Processor.cc:165-360).  attention(qkv [B, S, 3D], context_qkv [B, Sc, 3D]) -> (attn [B, S, D],
+    context_attn [B, Sc, D]).  Returns (output, context_output)."""
+    c, msa = ada_fp8_layernorm(x, temb, w.norm1, 6, (w.to_qkv.input_scale,))
+    cc, cmsa = ada_fp8_layernorm(context, temb, w.norm1_context, 6, (w.to_added_qkv.input_scale,))
+    attn, cattn = attention(_linear_from_codes(w.to_qkv, c, x.dtype), _linear_from_codes(w.to_added_qkv, cc, x.dtype))
+    a_out = w.to_out.forward(attn.contiguous())
+    c_out = w.to_add_out.forward(cattn.contiguous())
+    return flux_attn_post_fp8(x, a_out, msa, w.ff), flux_attn_post_fp8(context, c_out, cmsa, w.ff_context)

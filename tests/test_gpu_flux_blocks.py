@@ -458,3 +458,53 @@ def test_ada_fp8_layernorm(ops, dev, batch):
     bidx = np.arange(batch * s) // s
     want = O.round_to(O.round_to(O.round_to(to_np_f32(msa[1])[bidx] + 1.0, "bf16") * O.round_to(n, "bf16"), "bf16") + to_np_f32(msa[0])[bidx], "bf16")
     assert (y != want).mean() < 0.02 and np.all(np.abs(y - want) <= 2.0 ** -7 * (np.abs(want) + np.abs(to_np_f32(msa[0])[bidx]) + 1.0))
+
+
+def _toy_attention(heads):
+    """q/k/v split + scaled-dot-product attention in fp32 torch: stands in for the caller's (unquantized) attention."""
+    def run(qkv):
+        b, s, d3 = qkv.shape
+        d = d3 // 3
+        q, k, v = (t.reshape(b, s, heads, d // heads).transpose(1, 2).float() for t in qkv.split(d, dim=-1))
+        o = torch.nn.functional.scaled_dot_product_attention(q, k, v)
+        return o.transpose(1, 2).reshape(b, s, d).to(qkv.dtype)
+    return run
+
+
+def test_whole_fp8_blocks_around_a_caller_supplied_attention(ops, dev):
+    from lyradiff_amd import flux_fp8 as F
+
+    b, s, sc, d = 2, 96, 32, 256
+    g = rng_t(91)
+    names = {"norm.linear": (3 * d, d), "attn.to_qkv": (3 * d, d), "proj_mlp": (4 * d, d), "proj_out": (d, 5 * d),
+             "norm1.linear": (6 * d, d), "norm1_context.linear": (6 * d, d), "attn.to_added_qkv": (3 * d, d),
+             "attn.to_out.0": (d, d), "attn.to_add_out": (d, d), "ff.net.0.proj": (4 * d, d), "ff.net.2": (d, 4 * d),
+             "ff_context.net.0.proj": (4 * d, d), "ff_context.net.2": (d, 4 * d)}
+    sd = _state_dict(names, 92)
+    for n in names:
+        sd[f"p.{n}_input_scale"] = torch.tensor([5.0 / 448])
+    x = torch.randn(b, s, d, generator=g).bfloat16().to(dev)
+    ctx = torch.randn(b, sc, d, generator=g).bfloat16().to(dev)
+    temb = torch.randn(b, d, generator=g).bfloat16().to(dev)
+    att = _toy_attention(4)
+    # single block == the same steps called one by one
+    ws = F.load_flux_single_block_fp8(sd, "p.", d, 4, torch.bfloat16, dev)
+    out = F.flux_single_block_fp8(x, temb, ws, att)
+    norm, msa = F.ada_fp8_layernorm(x, temb, ws.norm, 3)
+    qkv = ws.to_qkv.forward(norm)
+    want = F.flux_single_mlp_fp8(x, norm, att(qkv), msa[2].contiguous(), ws.mlp)
+    assert out.shape == x.shape and torch.equal(out, want) and torch.isfinite(out.float()).all()
+    # double block likewise, both streams
+    wd = F.load_flux_double_block_fp8(sd, "p.", d, torch.bfloat16, dev)
+
+    def joint(qkv, cqkv):
+        o = att(torch.cat([cqkv, qkv], dim=1))
+        return o[:, cqkv.shape[1]:], o[:, :cqkv.shape[1]]
+
+    o1, o2 = F.flux_double_block_fp8(x, ctx, temb, wd, joint)
+    n1, m1 = F.ada_fp8_layernorm(x, temb, wd.norm1, 6)
+    n2, m2 = F.ada_fp8_layernorm(ctx, temb, wd.norm1_context, 6)
+    a1, a2 = joint(wd.to_qkv.forward(n1), wd.to_added_qkv.forward(n2))
+    w1 = F.flux_attn_post_fp8(x, wd.to_out.forward(a1.contiguous()), m1, wd.ff)
+    w2 = F.flux_attn_post_fp8(ctx, wd.to_add_out.forward(a2.contiguous()), m2, wd.ff_context)
+    assert torch.equal(o1, w1) and torch.equal(o2, w2) and o2.shape == ctx.shape
