@@ -136,10 +136,11 @@ struct I32Tag {};
 // GELU for the fused FP8 epilogue: hardware exp2 / reciprocal (the reference's counterpart is
 // cuBLASLt's GELU epilogue, utils/cublasMMWrapper.cc:1195-1199, whose arithmetic is not visible).
 __device__ __forceinline__ float gelu_fast(float x) {
-    float inner = 0.7978845608028654f * (x + 0.044715f * x * x * x);
-    float e = __builtin_amdgcn_exp2f(inner * 2.8853900817779268f);  // exp(2*inner)
-    float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);        // tanh(inner); e=inf -> 1
-    return 0.5f * x * (1.0f + t);
+    // 0.5 x (1 + tanh(u)) = x / (1 + exp(-2u)),  u = sqrt(2/pi) (x + 0.044715 x^3);  -2u log2(e) = x (A + B x^2)
+    constexpr float A = -2.0f * 0.7978845608028654f * 1.4426950408889634f, B = A * 0.044715f;
+    const float t = x * (A + B * (x * x));
+    const float e = __builtin_amdgcn_exp2f(t);             // exp(-2u): 0 for large x, inf for very negative x
+    return x * __builtin_amdgcn_rcpf(1.0f + e);            // x, resp. -0
 }
 
 // Four floats -> four e4m3 codes, round-to-nearest-even, saturating to +-448, NaN -> 0x7F | sign (the cast kernel's rule).
@@ -601,64 +602,70 @@ struct GemmKernel {
                     arow_l[i] = p.alpha_row[p.per_token ? min(m0 + wm * TM + i * 32 + lr, p.m - 1) : 0];
             }
         }
+        // The row loop exists in a few specialisations, chosen once per workgroup: which optional steps run
+        // (PLAIN: scales and bias; ACT: also GELU and/or the running maximum; GENERAL: every option, checked at run
+        // time) and whether the tile lies entirely inside C (no bounds checks).  Strip rows are read four at a time
+        // so that their LDS latencies overlap, and the specialisations keep the per-row code free of branches.
+        constexpr int E_PLAIN = 0, E_ACT = 1, E_GENERAL = 2;
+        int emode = E_PLAIN;
+        if constexpr (kExtras) {
+            if (p.addend != nullptr || p.residual != nullptr || p.gate != nullptr || p.C8 != nullptr || p.C == nullptr) emode = E_GENERAL;
+            else if (p.gelu != 0 || p.out_scale != nullptr) emode = E_ACT;
+        }
+        const bool tile_full = m0 + BM <= p.m && n0 + BN <= p.n;
+        const bool has_bias = p.bias != nullptr;
+        auto band_rows = [&](auto i_c, auto mode_c, auto full_c) {
+            constexpr int i = decltype(i_c)::value;
+            constexpr int MODE = decltype(mode_c)::value;
+            constexpr bool FULL = decltype(full_c)::value;
+            constexpr int NITER = 32 / RPI, NB = 4;
+            static_assert(NITER % NB == 0, "strip rows are processed four at a time");
+            const int mrow0 = m0 + wm * TM + i * 32 + out_row;
+            const size_t idx0 = (size_t)mrow0 * p.n + out_n, rstep = (size_t)RPI * p.n;
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
+            for (int tb = 0; tb < NITER; tb += NB) {
+                v4i raw[NB];
+                float arv[NB];
 #pragma unroll
-            for (int j = 0; j < NT; ++j)
-#pragma unroll
-                for (int q4 = 0; q4 < 4; ++q4) {
-                    char* spot = strip + lr * PITCH + (j * 32 + q4 * 8 + lh * 4) * 4;
-                    if constexpr (W4)
-                        *reinterpret_cast<float4*>(spot) = make_float4(res[i][j][q4 * 4], res[i][j][q4 * 4 + 1],
-                                                                       res[i][j][q4 * 4 + 2], res[i][j][q4 * 4 + 3]);
-                    else if constexpr (KIND == K_FP8)
-                        *reinterpret_cast<float4*>(spot) = make_float4(acc[i][j][q4 * 4], acc[i][j][q4 * 4 + 1],
-                                                                       acc[i][j][q4 * 4 + 2], acc[i][j][q4 * 4 + 3]);
-                    else
-                        *reinterpret_cast<int4*>(spot) = make_int4(acc[i][j][q4 * 4], acc[i][j][q4 * 4 + 1],
-                                                                   acc[i][j][q4 * 4 + 2], acc[i][j][q4 * 4 + 3]);
+                for (int u = 0; u < NB; ++u) {
+                    const int row = (tb + u) * RPI + out_row;
+                    raw[u] = *reinterpret_cast<const v4i*>(strip + row * PITCH + (lane % LPR) * 16);
+                    if constexpr (KIND == K_INT8 && !kI32) arv[u] = *reinterpret_cast<const float*>(strip + row * PITCH + TN * 4);
                 }
-            if constexpr (KIND == K_INT8 && !kI32) {
-                if (lh == 0) *reinterpret_cast<float*>(strip + lr * PITCH + TN * 4) = arow_l[i];
-            }
-            // strip -> registers with rows contiguous, math, store (the wavefront's own LDS accesses
-            // complete in order, so no barrier is needed inside the wavefront)
 #pragma unroll
-            for (int t = 0; t < 32 / RPI; ++t) {
-                const int row = t * RPI + out_row;
-                const int mo = m0 + wm * TM + i * 32 + row;
-                const char* src = strip + row * PITCH + (lane % LPR) * 16;
-                const bool ok = mo < p.m && n_ok;
-                const size_t idx = (size_t)mo * p.n + out_n;
-                if constexpr (kI32) {
-                    int4 v = *reinterpret_cast<const int4*>(src);
-                    if (ok) *reinterpret_cast<int4*>(static_cast<int*>(p.C) + idx) = v;
-                } else {
-                    float y[4];
-                    if constexpr (KIND == K_INT8) {
-                        int4 v = *reinterpret_cast<const int4*>(src);
-                        const float ar = *reinterpret_cast<const float*>(strip + row * PITCH + TN * 4);
-                        const int vi[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            y[e] = (float)vi[e] * (acol4[e] * ar);
-                            if (p.bias != nullptr) y[e] = y[e] + bias4[e];
-                        }
+                for (int u = 0; u < NB; ++u) {
+                    const int t = tb + u;
+                    const int mo = mrow0 + t * RPI;
+                    const bool ok = FULL || (mo < p.m && n_ok);
+                    const size_t idx = idx0 + (size_t)t * rstep;
+                    if constexpr (kI32) {
+                        if (ok) *reinterpret_cast<v4i*>(static_cast<int*>(p.C) + idx) = raw[u];
                     } else {
-                        float4 v = *reinterpret_cast<const float4*>(src);
-                        const float vf[4] = {v.x, v.y, v.z, v.w};
+                        float y[4];
+                        if constexpr (KIND == K_INT8) {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            y[e] = (KIND == K_FP8) ? vf[e] * alpha : vf[e];
-                            if (p.bias != nullptr) y[e] = y[e] + bias4[e];
-                            if constexpr (kExtras) {
-                                if (p.gelu) {
+                            for (int e = 0; e < 4; ++e) {
+                                y[e] = (float)raw[u][e] * (acol4[e] * arv[u]);
+                                if (has_bias) y[e] = y[e] + bias4[e];
+                            }
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const float vf = __int_as_float(raw[u][e]);
+                                y[e] = (KIND == K_FP8) ? vf * alpha : vf;
+                                if (has_bias) y[e] = y[e] + bias4[e];
+                            }
+                        }
+                        if constexpr (kExtras && MODE != E_PLAIN) {
+                            if (p.gelu) {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) {
                                     if (p.gelu == 2) y[e] = round_through<OutTag>(y[e]);
                                     y[e] = gelu_fast(y[e]);
                                 }
                             }
                         }
-                        if constexpr (kExtras) {
+                        if constexpr (kExtras && MODE == E_GENERAL) {
                             if (p.addend != nullptr && ok) {  // T( T(y) + addend ): a second linear's output joined in T
                                 float aa[4];
                                 OutStore<OutTag>::load4(p.addend, idx, aa);
@@ -679,21 +686,72 @@ struct GemmKernel {
                                 }
                             }
                         }
-                    }
-                    if constexpr (kExtras) {
-                        if (ok) {
-                            if (p.out_scale != nullptr)
-                                out_amax = fmaxf(fmaxf(out_amax, fmaxf(fabsf(y[0]), fabsf(y[1]))), fmaxf(fabsf(y[2]), fabsf(y[3])));
-                            if (p.C8 != nullptr) {  // the codes the separate cast kernel would produce from the T-rounded output
-                                float t[4];
+                        if constexpr (kExtras && MODE != E_PLAIN) {
+                            if (ok) {
+                                if (p.out_scale != nullptr)
+                                    out_amax = fmaxf(fmaxf(out_amax, fmaxf(fabsf(y[0]), fabsf(y[1]))), fmaxf(fabsf(y[2]), fabsf(y[3])));
+                                if constexpr (MODE == E_GENERAL) {
+                                    if (p.C8 != nullptr) {  // the codes the separate cast kernel would produce from the T-rounded output
+                                        float tq[4];
 #pragma unroll
-                                for (int e = 0; e < 4; ++e) t[e] = round_through<OutTag>(y[e]) * c8_inv;
-                                *reinterpret_cast<u32*>(p.C8 + (size_t)mo * p.ldc8 + out_n) = e4m3x4(t[0], t[1], t[2], t[3]);
+                                        for (int e = 0; e < 4; ++e) tq[e] = round_through<OutTag>(y[e]) * c8_inv;
+                                        *reinterpret_cast<u32*>(p.C8 + (size_t)mo * p.ldc8 + out_n) = e4m3x4(tq[0], tq[1], tq[2], tq[3]);
+                                    }
+                                }
                             }
                         }
+                        if constexpr (kExtras && MODE == E_GENERAL) {
+                            if (ok && p.C != nullptr) OutStore<OutTag>::store4(p.C, idx, y);
+                        } else {
+                            if (ok) OutStore<OutTag>::store4(p.C, idx, y);
+                        }
                     }
-                    if (ok && p.C != nullptr) OutStore<OutTag>::store4(p.C, idx, y);
                 }
+            }
+        };
+        // one fully unrolled pass over the wavefront's MT bands per specialisation (the accumulators must stay
+        // statically indexed, so the specialisation is chosen outside the band loop)
+        auto all_bands = [&](auto mode_c, auto full_c) {
+            auto one_band = [&](auto i_c) {
+                constexpr int i = decltype(i_c)::value;
+#pragma unroll
+                for (int j = 0; j < NT; ++j)
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; ++q4) {
+                        char* spot = strip + lr * PITCH + (j * 32 + q4 * 8 + lh * 4) * 4;
+                        if constexpr (W4)
+                            *reinterpret_cast<float4*>(spot) = make_float4(res[i][j][q4 * 4], res[i][j][q4 * 4 + 1],
+                                                                           res[i][j][q4 * 4 + 2], res[i][j][q4 * 4 + 3]);
+                        else if constexpr (KIND == K_FP8)
+                            *reinterpret_cast<float4*>(spot) = make_float4(acc[i][j][q4 * 4], acc[i][j][q4 * 4 + 1],
+                                                                           acc[i][j][q4 * 4 + 2], acc[i][j][q4 * 4 + 3]);
+                        else
+                            *reinterpret_cast<int4*>(spot) = make_int4(acc[i][j][q4 * 4], acc[i][j][q4 * 4 + 1],
+                                                                       acc[i][j][q4 * 4 + 2], acc[i][j][q4 * 4 + 3]);
+                    }
+                if constexpr (KIND == K_INT8 && !kI32) {
+                    if (lh == 0) *reinterpret_cast<float*>(strip + lr * PITCH + TN * 4) = arow_l[i];
+                }
+                // strip -> registers with rows contiguous, math, store (the wavefront's own LDS accesses
+                // complete in order, so no barrier is needed inside the wavefront)
+                band_rows(i_c, mode_c, full_c);
+            };
+            one_band(std::integral_constant<int, 0>{});
+            if constexpr (MT > 1) one_band(std::integral_constant<int, 1>{});
+            if constexpr (MT > 2) one_band(std::integral_constant<int, 2>{});
+            if constexpr (MT > 3) one_band(std::integral_constant<int, 3>{});
+            static_assert(MT <= 4, "at most four 32-row bands per wavefront");
+        };
+        {
+            using std::integral_constant;
+            if (tile_full) {
+                if (emode == E_PLAIN) all_bands(integral_constant<int, E_PLAIN>{}, std::true_type{});
+                else if (emode == E_ACT) all_bands(integral_constant<int, E_ACT>{}, std::true_type{});
+                else all_bands(integral_constant<int, E_GENERAL>{}, std::true_type{});
+            } else {
+                if (emode == E_PLAIN) all_bands(integral_constant<int, E_PLAIN>{}, std::false_type{});
+                else if (emode == E_ACT) all_bands(integral_constant<int, E_ACT>{}, std::false_type{});
+                else all_bands(integral_constant<int, E_GENERAL>{}, std::false_type{});
             }
         }
         if constexpr (kExtras) {
