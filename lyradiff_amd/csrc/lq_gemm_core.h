@@ -603,14 +603,19 @@ struct GemmKernel {
             }
         }
         // The row loop exists in a few specialisations, chosen once per workgroup: which optional steps run
-        // (PLAIN: scales and bias; ACT: also GELU and/or the running maximum; GENERAL: every option, checked at run
-        // time) and whether the tile lies entirely inside C (no bounds checks).  Strip rows are read four at a time
-        // so that their LDS latencies overlap, and the specialisations keep the per-row code free of branches.
-        constexpr int E_PLAIN = 0, E_ACT = 1, E_GENERAL = 2;
-        int emode = E_PLAIN;
-        if constexpr (kExtras) {
-            if (p.addend != nullptr || p.residual != nullptr || p.gate != nullptr || p.C8 != nullptr || p.C == nullptr) emode = E_GENERAL;
-            else if (p.gelu != 0 || p.out_scale != nullptr) emode = E_ACT;
+        // (PLAIN: scales and bias; ACT: also GELU and/or the running maximum; CODES: optional GELU, e4m3 codes
+        // instead of C; GATED: gate and residual; GENERAL: every option, checked at run time) and whether the tile lies
+        // entirely inside C (no bounds checks).  Strip rows are read four at a time so that their LDS latencies
+        // overlap, and the specialisations keep the per-row code free of branches.
+        constexpr int E_PLAIN = 0, E_ACT = 1, E_CODES = 2, E_GATED = 3, E_GENERAL = 4;
+        constexpr bool kSpecialise = kExtras && ESZ == 2;  // fp32 outputs take the general path only (build time)
+        int emode = kExtras ? E_GENERAL : E_PLAIN;
+        if constexpr (kSpecialise) {
+            const bool join = p.addend != nullptr || p.residual != nullptr || p.gate != nullptr;
+            if (!join && p.C8 == nullptr && p.C != nullptr) emode = (p.gelu != 0 || p.out_scale != nullptr) ? E_ACT : E_PLAIN;
+            else if (!join && p.C8 != nullptr && p.C == nullptr && p.out_scale == nullptr) emode = E_CODES;
+            else if (p.gate != nullptr && p.residual != nullptr && p.addend == nullptr && p.C8 == nullptr && p.C != nullptr &&
+                     p.gelu == 0 && p.out_scale == nullptr) emode = E_GATED;
         }
         const bool tile_full = m0 + BM <= p.m && n0 + BN <= p.n;
         const bool has_bias = p.bias != nullptr;
@@ -618,6 +623,7 @@ struct GemmKernel {
             constexpr int i = decltype(i_c)::value;
             constexpr int MODE = decltype(mode_c)::value;
             constexpr bool FULL = decltype(full_c)::value;
+            constexpr bool GEN = MODE == E_GENERAL;
             constexpr int NITER = 32 / RPI, NB = 4;
             static_assert(NITER % NB == 0, "strip rows are processed four at a time");
             const int mrow0 = m0 + wm * TM + i * 32 + out_row;
@@ -656,7 +662,7 @@ struct GemmKernel {
                                 if (has_bias) y[e] = y[e] + bias4[e];
                             }
                         }
-                        if constexpr (kExtras && MODE != E_PLAIN) {
+                        if constexpr (kExtras && (MODE == E_ACT || MODE == E_CODES || GEN)) {
                             if (p.gelu) {
 #pragma unroll
                                 for (int e = 0; e < 4; ++e) {
@@ -665,17 +671,19 @@ struct GemmKernel {
                                 }
                             }
                         }
-                        if constexpr (kExtras && MODE == E_GENERAL) {
+                        if constexpr (kExtras && GEN) {
                             if (p.addend != nullptr && ok) {  // T( T(y) + addend ): a second linear's output joined in T
                                 float aa[4];
                                 OutStore<OutTag>::load4(p.addend, idx, aa);
 #pragma unroll
                                 for (int e = 0; e < 4; ++e) y[e] = round_through<OutTag>(round_through<OutTag>(y[e]) + aa[e]);
                             }
-                            if (p.residual != nullptr && ok) {
+                        }
+                        if constexpr (kExtras && (MODE == E_GATED || GEN)) {
+                            if ((MODE == E_GATED || p.residual != nullptr) && ok) {
                                 float rr[4];
                                 OutStore<OutTag>::load4(p.residual, idx, rr);
-                                if (p.gate != nullptr) {
+                                if (MODE == E_GATED || p.gate != nullptr) {
                                     if (!gate_uniform) OutStore<OutTag>::load4(p.gate, ((size_t)mo / p.gate_rows) * (size_t)p.n + out_n, gate4);
 #pragma unroll
                                     for (int e = 0; e < 4; ++e)
@@ -686,23 +694,21 @@ struct GemmKernel {
                                 }
                             }
                         }
-                        if constexpr (kExtras && MODE != E_PLAIN) {
-                            if (ok) {
-                                if (p.out_scale != nullptr)
-                                    out_amax = fmaxf(fmaxf(out_amax, fmaxf(fabsf(y[0]), fabsf(y[1]))), fmaxf(fabsf(y[2]), fabsf(y[3])));
-                                if constexpr (MODE == E_GENERAL) {
-                                    if (p.C8 != nullptr) {  // the codes the separate cast kernel would produce from the T-rounded output
-                                        float tq[4];
+                        if constexpr (kExtras && (MODE == E_ACT || GEN)) {
+                            if (ok && p.out_scale != nullptr)
+                                out_amax = fmaxf(fmaxf(out_amax, fmaxf(fabsf(y[0]), fabsf(y[1]))), fmaxf(fabsf(y[2]), fabsf(y[3])));
+                        }
+                        if constexpr (kExtras && (MODE == E_CODES || GEN)) {
+                            if (ok && (MODE == E_CODES || p.C8 != nullptr)) {  // the codes the cast kernel would produce from the T-rounded output
+                                float tq[4];
 #pragma unroll
-                                        for (int e = 0; e < 4; ++e) tq[e] = round_through<OutTag>(y[e]) * c8_inv;
-                                        *reinterpret_cast<u32*>(p.C8 + (size_t)mo * p.ldc8 + out_n) = e4m3x4(tq[0], tq[1], tq[2], tq[3]);
-                                    }
-                                }
+                                for (int e = 0; e < 4; ++e) tq[e] = round_through<OutTag>(y[e]) * c8_inv;
+                                *reinterpret_cast<u32*>(p.C8 + (size_t)mo * p.ldc8 + out_n) = e4m3x4(tq[0], tq[1], tq[2], tq[3]);
                             }
                         }
-                        if constexpr (kExtras && MODE == E_GENERAL) {
+                        if constexpr (GEN) {
                             if (ok && p.C != nullptr) OutStore<OutTag>::store4(p.C, idx, y);
-                        } else {
+                        } else if constexpr (MODE != E_CODES) {
                             if (ok) OutStore<OutTag>::store4(p.C, idx, y);
                         }
                     }
@@ -744,14 +750,24 @@ struct GemmKernel {
         };
         {
             using std::integral_constant;
-            if (tile_full) {
-                if (emode == E_PLAIN) all_bands(integral_constant<int, E_PLAIN>{}, std::true_type{});
-                else if (emode == E_ACT) all_bands(integral_constant<int, E_ACT>{}, std::true_type{});
-                else all_bands(integral_constant<int, E_GENERAL>{}, std::true_type{});
+            if constexpr (kSpecialise) {
+                if (emode == E_GENERAL) all_bands(integral_constant<int, E_GENERAL>{}, std::false_type{});
+                else if (tile_full) {
+                    if (emode == E_PLAIN) all_bands(integral_constant<int, E_PLAIN>{}, std::true_type{});
+                    else if (emode == E_ACT) all_bands(integral_constant<int, E_ACT>{}, std::true_type{});
+                    else if (emode == E_CODES) all_bands(integral_constant<int, E_CODES>{}, std::true_type{});
+                    else all_bands(integral_constant<int, E_GATED>{}, std::true_type{});
+                } else {
+                    if (emode == E_PLAIN) all_bands(integral_constant<int, E_PLAIN>{}, std::false_type{});
+                    else if (emode == E_ACT) all_bands(integral_constant<int, E_ACT>{}, std::false_type{});
+                    else if (emode == E_CODES) all_bands(integral_constant<int, E_CODES>{}, std::false_type{});
+                    else all_bands(integral_constant<int, E_GATED>{}, std::false_type{});
+                }
+            } else if constexpr (kExtras) {
+                all_bands(integral_constant<int, E_GENERAL>{}, std::false_type{});
             } else {
-                if (emode == E_PLAIN) all_bands(integral_constant<int, E_PLAIN>{}, std::false_type{});
-                else if (emode == E_ACT) all_bands(integral_constant<int, E_ACT>{}, std::false_type{});
-                else all_bands(integral_constant<int, E_GENERAL>{}, std::false_type{});
+                if (tile_full) all_bands(integral_constant<int, E_PLAIN>{}, std::true_type{});
+                else all_bands(integral_constant<int, E_PLAIN>{}, std::false_type{});
             }
         }
         if constexpr (kExtras) {
