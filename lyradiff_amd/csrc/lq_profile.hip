@@ -2,7 +2,7 @@
 // operands and records the fastest in the per-shape cache.  Stands in for
 // GemmPluginProfiler::profileTactics / profileTacticForProblem of lyraDiff
 // (layers/gemm_utils/GemmProfiler.cc:78-127,161-265): same idea (warm-up runs, timed runs between two
-// events, keep the minimum), but the caller owns the temporary memory and nothing is allocated here.
+// events, keep the minimum; here in interleaved rounds), but the caller owns the temporary memory and nothing is allocated here.
 #include "lq_common.h"
 
 namespace lq {
@@ -107,24 +107,34 @@ extern "C" int lq_gemm_profile(lq_weight_kind_t kind, int m, int n, int k, void*
     hipEvent_t ev0, ev1;
     LQ_REQUIRE(hipEventCreate(&ev0) == hipSuccess && hipEventCreate(&ev1) == hipSuccess, LQ_ERR_HIP,
                "lq_gemm_profile: cannot create events");
-    constexpr int kWarmup = 2, kRuns = 5;
+    // Candidates are timed in interleaved rounds and each keeps its fastest round: on a power-limited part the clock
+    // drifts over consecutive launches by more than the candidates differ, and a block of back-to-back runs per
+    // candidate would rank them by when they ran.
+    constexpr int kRounds = 5, kRuns = 3, kMaxTactics = 16;
+    float best_of[kMaxTactics];
+    bool usable[kMaxTactics];
+    for (int t = 0; t < kMaxTactics; ++t) { best_of[t] = 0.0f; usable[t] = t < count; }
+    for (int round = 0; round < kRounds + 1; ++round) {  // round 0 is the warm-up
+        for (int t = 0; t < count && t < kMaxTactics; ++t) {
+            if (!usable[t]) continue;
+            tl_forced_tactic = t;
+            bool ok = hipEventRecord(ev0, st) == hipSuccess;
+            for (int i = 0; i < kRuns && ok; ++i) ok = run_once() == LQ_OK;
+            if (ok) ok = hipEventRecord(ev1, st) == hipSuccess && hipEventSynchronize(ev1) == hipSuccess;
+            float ms = 0.0f;
+            if (ok) ok = hipEventElapsedTime(&ms, ev0, ev1) == hipSuccess;
+            if (!ok) {
+                (void)hipGetLastError();  // a configuration that cannot run this shape is skipped, as in the reference
+                usable[t] = false;
+                continue;
+            }
+            if (round > 0 && (best_of[t] == 0.0f || ms < best_of[t])) best_of[t] = ms;
+        }
+    }
     int best = -1;
     float best_ms = 0.0f;
-    for (int t = 0; t < count; ++t) {
-        tl_forced_tactic = t;
-        bool ok = true;
-        for (int i = 0; i < kWarmup && ok; ++i) ok = run_once() == LQ_OK;
-        if (ok) ok = hipEventRecord(ev0, st) == hipSuccess;
-        for (int i = 0; i < kRuns && ok; ++i) ok = run_once() == LQ_OK;
-        if (ok) ok = hipEventRecord(ev1, st) == hipSuccess && hipEventSynchronize(ev1) == hipSuccess;
-        float ms = 0.0f;
-        if (ok) ok = hipEventElapsedTime(&ms, ev0, ev1) == hipSuccess;
-        if (!ok) {
-            (void)hipGetLastError();  // a configuration that cannot run this shape is skipped, as in the reference
-            continue;
-        }
-        if (best < 0 || ms < best_ms) { best = t; best_ms = ms; }
-    }
+    for (int t = 0; t < count && t < kMaxTactics; ++t)
+        if (usable[t] && best_of[t] > 0.0f && (best < 0 || best_of[t] < best_ms)) { best = t; best_ms = best_of[t]; }
     tl_forced_tactic = -1;
     (void)hipEventDestroy(ev0);
     (void)hipEventDestroy(ev1);
