@@ -156,33 +156,80 @@ __device__ __forceinline__ int rne_sat_s4(float x) {
     return (int)r;
 }
 
+// float -> int32 as the hardware defines it: round toward zero, saturate, NaN -> 0 (a C++ cast leaves
+// out-of-range and NaN operands undefined)
+__device__ __forceinline__ int cvt_i32_sat(float x) {
+    int r;
+    asm("v_cvt_i32_f32_e32 %0, %1" : "=v"(r) : "v"(x));
+    return r;
+}
+
 // q[i] = clamp(rint(t[i] / s), LO, HI) (NaN -> 0) for eight values, bit-identical to the IEEE
 // division but normally computed from r ~ 1/s (within 1 ulp):  |t*r - t/s| <= 2.5*2^-24*|t/s| and
 // |fl(t/s) - t/s| <= 2^-24*|t/s|, so whenever |t*r| < 512 both lie within 1.1e-4 of the true quotient;
 // if t*r is at least 2e-4 away from every tie (|t*r - rint(t*r)| <= 0.4998) the true quotient, its
 // fp32 rounding and t*r all round to the same integer.  Beyond 512 in magnitude everything saturates.
-// If any of the eight values fails the test (or is NaN/inf, or the caller flags the scale as
-// unsafe for a reciprocal), the whole octet is redone with true divisions: one rarely taken branch.
+// If any of the eight values fails the test (or the caller flags the scale as unsafe for a
+// reciprocal), the whole octet is redone with true divisions: one rarely taken branch.
 template <int LO, int HI>
 __device__ __forceinline__ void quant8(const float* t, float s, float r, bool slow, int* q) {
-    float rq[8], dev = 0.0f, nonfinite = 0.0f;
+    float rq[8], dev = 0.0f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         float qa = t[i] * r;
         rq[i] = __builtin_rintf(qa);
-        dev = fmaxf(dev, fabsf(qa - rq[i]));                   // largest distance from an integer
-        nonfinite = __builtin_fmaf(t[i], 0.0f, nonfinite);    // stays 0 unless some t is inf or NaN
+        dev = fmaxf(dev, fabsf(qa - rq[i]));  // largest distance from an integer (NaN differences drop out)
     }
-    const bool risky = slow | !(dev <= 0.4998f) | !(nonfinite == 0.0f);
+    const bool risky = slow | !(dev <= 0.4998f);
     if (__builtin_expect(risky, 0)) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            float e = t[i] / s;
-            rq[i] = (e != e) ? 0.0f : __builtin_rintf(e);
-        }
+        for (int i = 0; i < 8; ++i) rq[i] = __builtin_rintf(t[i] / s);
     }
+    // The hardware conversion saturates and turns NaN into 0, which is what the formula asks of a NaN
+    // input; +-inf (t*r and t/s alike, r being a normal positive number here) saturates like any large value.
 #pragma unroll
-    for (int i = 0; i < 8; ++i) q[i] = (int)__builtin_amdgcn_fmed3f(rq[i], (float)LO, (float)HI);
+    for (int i = 0; i < 8; ++i) {
+        const int v = cvt_i32_sat(rq[i]);
+        q[i] = v < LO ? LO : (v > HI ? HI : v);
+    }
+}
+// The dynamic per-token case: every |t[i]| <= amax and s = fl(amax / 127), so |t[i] / s| stays below 127.00002
+// and nothing needs clamping; the conversion writes its low byte straight into the packed result
+// (sub-dword destination select), which saves the clamp and the byte shuffles.  NaN -> 0 as above.
+__device__ __forceinline__ uint2 quant8_pack_unclamped(const float* t, float s, float r, bool slow) {
+    float rq[8], dev = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float qa = t[i] * r;
+        rq[i] = __builtin_rintf(qa);
+        dev = fmaxf(dev, fabsf(qa - rq[i]));
+    }
+    const bool risky = slow | !(dev <= 0.4998f);
+    if (__builtin_expect(risky, 0)) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) rq[i] = __builtin_rintf(t[i] / s);
+    }
+    uint2 o;
+    asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD" : "=v"(o.x) : "v"(rq[0]));
+    asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(o.x) : "v"(rq[1]));
+    asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(o.x) : "v"(rq[2]));
+    asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(o.x) : "v"(rq[3]));
+    asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD" : "=v"(o.y) : "v"(rq[4]));
+    asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(o.y) : "v"(rq[5]));
+    asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(o.y) : "v"(rq[6]));
+    asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(o.y) : "v"(rq[7]));
+    return o;
+}
+// t[i] = fl(x[i] * f[i]) for the eight fp16 values of a 16-byte vector: the mixed-precision fma reads the
+// half operand directly (x*f + 0 rounds once, like convert-then-multiply; a zero product loses its sign,
+// which no consumer here looks at).
+__device__ __forceinline__ void mul8_f16(const uint4& v, const float* f, float* t) {
+    const u32 w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(t[2 * i]) : "v"(w[i]), "v"(f[2 * i]));
+        asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(t[2 * i + 1]) : "v"(w[i]), "v"(f[2 * i + 1]));
+    }
 }
 // true unless |s| lies in [2^-100, 2^100]: zero, subnormal, huge, infinite and NaN scales all take the
 // exact-division path (one integer subtract and compare on the exponent field)

@@ -10,6 +10,7 @@
 // (activation), :173-223 (weights), :117-171 (dequant), kernels/quant_kernels/
 // ffn_kernels_int8.cu:102-147 (bias + GEGLU), kernels/quant_kernels/int8_utils.cuh:23-28.
 #include "lq_common.h"
+#include <type_traits>
 
 namespace lq {
 
@@ -79,15 +80,20 @@ __global__ __launch_bounds__(256) void sq_quant_rows_kernel(int8_t* __restrict__
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             int col = (p * 64 + lane) * 8;
-            unpack_raw(cur[p], t[p]);
             if constexpr (HAS_PRE) {
-                if (col < dim) {
-                    float4 a = *reinterpret_cast<const float4*>(s_pre + col);
-                    float4 b = *reinterpret_cast<const float4*>(s_pre + col + 4);
-                    const float pv[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+                // (a lane outside the row holds zeros and multiplies them by whatever LDS holds at a clamped offset)
+                const int pc = col < dim ? col : 0;
+                float4 a = *reinterpret_cast<const float4*>(s_pre + pc);
+                float4 b = *reinterpret_cast<const float4*>(s_pre + pc + 4);
+                const float pv[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+                if constexpr (std::is_same<Tag, F16Tag>::value) mul8_f16(cur[p][0], pv, t[p]);
+                else {
+                    unpack_raw(cur[p], t[p]);
 #pragma unroll
                     for (int i = 0; i < 8; ++i) t[p][i] = t[p][i] * pv[i];
                 }
+            } else {
+                unpack_raw(cur[p], t[p]);
             }
             if constexpr (MODE == 2) {
 #pragma unroll
@@ -113,11 +119,14 @@ __global__ __launch_bounds__(256) void sq_quant_rows_kernel(int8_t* __restrict__
         for (int p = 0; p < NP; ++p) {
             int col = (p * 64 + lane) * 8;
             if (col < dim) {
-                int q[8];
-                quant8<-128, 127>(t[p], s, r, slow, q);
                 uint2 o;
-                o.x = pack4_s8(q[0], q[1], q[2], q[3]);
-                o.y = pack4_s8(q[4], q[5], q[6], q[7]);
+                if constexpr (MODE == 2) o = quant8_pack_unclamped(t[p], s, r, slow);
+                else {
+                    int q[8];
+                    quant8<-128, 127>(t[p], s, r, slow, q);
+                    o.x = pack4_s8(q[0], q[1], q[2], q[3]);
+                    o.y = pack4_s8(q[4], q[5], q[6], q[7]);
+                }
                 *reinterpret_cast<uint2*>(ob + col) = o;
             }
         }
@@ -127,6 +136,93 @@ __global__ __launch_bounds__(256) void sq_quant_rows_kernel(int8_t* __restrict__
 #pragma unroll
                 for (int u = 0; u < VPP; ++u) cur[p][u] = nxt[p][u];
         }
+    }
+}
+
+// Rows longer than 1536 columns: the row is cut into 1024-column spans, one wavefront each, and a
+// workgroup of dim/1024 wavefronts (rounded up) owns one row.  A wavefront then needs at most 64
+// registers whatever the row length, so eight of them share a SIMD and the loads of one overlap the
+// arithmetic of the others; the dynamic variant exchanges the span maxima through LDS (one barrier).
+// A lane outside the row re-reads a valid octet (harmless for the maximum) and stores nothing.
+template <typename Tag, int MODE, bool HAS_PRE>
+__global__ __launch_bounds__(1024) void sq_quant_split_kernel(int8_t* __restrict__ dst, float* __restrict__ scale_out,
+                                                              const void* __restrict__ src,
+                                                              const float* __restrict__ pre,
+                                                              const float* __restrict__ in_scale, int dim) {
+    __shared__ __attribute__((aligned(16))) float red[16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const size_t row = blockIdx.x;
+    const char* rb = static_cast<const char*>(src) + row * (size_t)dim * Elem<Tag>::bytes;
+    if constexpr (MODE == 2) {
+        if (threadIdx.x < 16) red[threadIdx.x] = 0.0f;
+        __syncthreads();
+    }
+    constexpr bool kMix = HAS_PRE && std::is_same<Tag, F16Tag>::value;  // fp16 * fp32 in one instruction
+    int col[2];
+    bool valid[2];
+    float t[2][8];
+    uint4 raw[2];
+    float amax = 0.0f;
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        const int c = wave * 1024 + p * 512 + lane * 8;
+        valid[p] = c < dim;
+        col[p] = valid[p] ? c : 0;
+        if constexpr (kMix) raw[p] = *reinterpret_cast<const uint4*>(rb + (size_t)col[p] * 2);
+        else load8<Tag>(rb, col[p], t[p]);
+    }
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        if constexpr (HAS_PRE) {
+            float pv[8];
+            load8<F32Tag>(pre, col[p], pv);
+            if constexpr (kMix) mul8_f16(raw[p], pv, t[p]);
+            else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) t[p][i] = t[p][i] * pv[i];
+            }
+        }
+        if constexpr (MODE == 2) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(t[p][i]));
+        }
+    }
+    float s;
+    if constexpr (MODE == 2) {
+        amax = wave_max(amax);
+        if (lane == 0) red[wave] = amax;
+        __syncthreads();
+        const float4 a = *reinterpret_cast<const float4*>(red);
+        amax = fmaxf(fmaxf(a.x, a.y), fmaxf(a.z, a.w));
+        if (blockDim.x > 256) {  // more than four wavefronts (the same for the whole workgroup)
+            const float4 b = *reinterpret_cast<const float4*>(red + 4), c = *reinterpret_cast<const float4*>(red + 8);
+            const float4 d = *reinterpret_cast<const float4*>(red + 12);
+            amax = fmaxf(fmaxf(amax, fmaxf(fmaxf(b.x, b.y), fmaxf(b.z, b.w))),
+                         fmaxf(fmaxf(fmaxf(c.x, c.y), fmaxf(c.z, c.w)), fmaxf(fmaxf(d.x, d.y), fmaxf(d.z, d.w))));
+        }
+        s = div_by_const_fast(amax, 127.0f, 0x1.020408p-7f);
+        if (scale_out_of_range(s)) s = amax / 127.0f;
+        if (amax <= 5.9604644775390625e-08f) s = 1.0f;
+        if (threadIdx.x == 0) scale_out[row] = s;
+    } else if constexpr (MODE == 1) {
+        s = in_scale[row];
+    } else {
+        s = in_scale[0];
+    }
+    const float r = fast_recip(s);
+    const bool slow = scale_out_of_range(s);
+    int8_t* ob = dst + row * (size_t)dim;
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        uint2 o;
+        if constexpr (MODE == 2) o = quant8_pack_unclamped(t[p], s, r, slow);
+        else {
+            int q[8];
+            quant8<-128, 127>(t[p], s, r, slow, q);
+            o.x = pack4_s8(q[0], q[1], q[2], q[3]);
+            o.y = pack4_s8(q[4], q[5], q[6], q[7]);
+        }
+        if (valid[p]) *reinterpret_cast<uint2*>(ob + col[p]) = o;
     }
 }
 
@@ -180,12 +276,20 @@ static int launch_sq_quant(int8_t* dst, float* scale_out, const void* src, const
         return check_launch("sq_quant_generic");
     }
     const int np = (int)((dim + 511) / 512);
+    int d = (int)dim;
+    if (np > 3) {
+        // one wavefront per 1024 columns, one workgroup per row
+        LQ_REQUIRE(rows <= 0x7fffffffu, LQ_ERR_SHAPE, "sq_quant: %zu rows exceed the launch limit", rows);
+        dim3 grid((unsigned)rows), block(64 * ((np + 1) / 2));
+        if (pre) hipLaunchKernelGGL((sq_quant_split_kernel<Tag, MODE, true>), grid, block, 0, st, dst, scale_out, src, pre, in_scale, d);
+        else hipLaunchKernelGGL((sq_quant_split_kernel<Tag, MODE, false>), grid, block, 0, st, dst, scale_out, src, pre, in_scale, d);
+        return check_launch("sq_quant_split");
+    }
     // four rows per workgroup pass; more rows per wavefront only when there are plenty of rows
     int rpw = (int)(rows / (4 * 768));
     rpw = rpw < 1 ? 1 : (rpw > 8 ? 8 : rpw);
     const size_t blocks = (rows + 4 * (size_t)rpw - 1) / (4 * (size_t)rpw);
     dim3 grid((unsigned)blocks), block(256);
-    int d = (int)dim;
     const size_t lds = pre ? dim * sizeof(float) : 0;
 #define LQ_SQ_CASE(NPV)                                                                                             \
     do {                                                                                                            \
@@ -194,14 +298,7 @@ static int launch_sq_quant(int8_t* dst, float* scale_out, const void* src, const
     } while (0)
     if (np <= 1) LQ_SQ_CASE(1);
     else if (np <= 2) LQ_SQ_CASE(2);
-    else if (np <= 3) LQ_SQ_CASE(3);
-    else if (np <= 4) LQ_SQ_CASE(4);
-    else if (np <= 6) LQ_SQ_CASE(6);
-    else if (np <= 8) LQ_SQ_CASE(8);
-    else if (np <= 12) LQ_SQ_CASE(12);
-    else if (np <= 16) LQ_SQ_CASE(16);
-    else if (np <= 24) LQ_SQ_CASE(24);
-    else LQ_SQ_CASE(32);
+    else LQ_SQ_CASE(3);
 #undef LQ_SQ_CASE
     return check_launch("sq_quant_rows");
 }
