@@ -5,6 +5,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <type_traits>
 
 #include "lyraquant.h"
 
@@ -97,6 +98,18 @@ template <> struct Elem<F32Tag> {
 template <typename Tag> __device__ __forceinline__ float round_through(float f) {
     asm volatile("" : "+v"(f));
     return Elem<Tag>::load(Elem<Tag>::store(f));
+}
+// two values at once: for bf16 one packed conversion serves both (1.5 instead of 2 instructions per value)
+template <typename Tag> __device__ __forceinline__ void round_through2(float& a, float& b) {
+    if constexpr (std::is_same<Tag, BF16Tag>::value) {
+        asm volatile("" : "+v"(a), "+v"(b));
+        const u32 w = pack2_bf16(a, b);
+        a = __uint_as_float(w << 16);
+        b = __uint_as_float(w & 0xFFFF0000u);
+    } else {
+        a = round_through<Tag>(a);
+        b = round_through<Tag>(b);
+    }
 }
 
 // Unpack a 16-byte vector of 8 sixteen-bit values / 4 fp32 values to floats.

@@ -10,7 +10,7 @@
 //     optionally preceded by invokeFusedGateAndResidual (kernels/flux_single_transformer_block/
 //     flux_single_transformer_kernels.cu:42-65, FluxAttnPostFP8Processor.cc:112-119):
 //       x = T( T(attn * gate[b,k]) + input ), also written out (the block's second residual uses it)
-// One wavefront owns a row: the row stays in registers between the statistics and the quantisation, so the
+// A row is owned by one wavefront (by one wavefront per 1024 columns when it is longer than 1536): it stays in registers between the statistics and the quantisation, so the
 // activation is read once and only the 1-byte codes (and dst2) are written.  Mean and variance are two-pass
 // fp32 sums over the registers (the reference runs Welford updates, in T for the INT8 kernels), reduced across
 // the 64 lanes in a fixed order; rstd = 1 / sqrt(var + eps) with IEEE sqrt and division.
@@ -41,17 +41,49 @@ __device__ __forceinline__ u32 ln_nan_fix(u32 w, const float* y) {  // NaN -> 0x
 // 3: no quantisation, y stored as T (the input of a W4A4 linear, which quantises per group and also feeds its low-rank branch).
 // MOD false: y = gamma*n + beta (vectors of length dim).  MOD true: y = (1 + scale[b])*n + shift[b], b = row / rows_per_batch.
 // RESID 0: h = src.  1: h = T(T(src + residual) + bias).  2: h = T(T(src * gate[b]) + residual), gate passed as `bias`.
-template <typename Tag, int NP, int QMODE, int RESID, bool MOD>
-__global__ __launch_bounds__(256) void ln_quant_rows_kernel(uint8_t* __restrict__ dst, void* __restrict__ dst2,
+// SPLIT false: a workgroup is four wavefronts with a row each (NP passes of 512 columns, rows up to 1536 columns).
+// SPLIT true (longer rows): a workgroup owns one row, cut into 1024-column spans with a wavefront each (NP = 2), so a
+// wavefront needs about 60 registers whatever the row length and eight of them share a SIMD; the three row reductions
+// then take a step through LDS, added in wavefront order.
+template <typename Tag, int NP, int QMODE, int RESID, bool MOD, bool SPLIT>
+__global__ __launch_bounds__(SPLIT ? 384 : 256) void ln_quant_rows_kernel(uint8_t* __restrict__ dst, void* __restrict__ dst2,
                                                             float* __restrict__ scale_out, const void* __restrict__ src,
                                                             const void* __restrict__ residual, const void* __restrict__ bias,
                                                             const void* __restrict__ gamma, const void* __restrict__ beta,
                                                             const float* __restrict__ pre, const float* __restrict__ in_scale,
                                                             uint8_t* __restrict__ dst_b, const float* __restrict__ in_scale_b,
                                                             size_t rows, int dim, size_t rows_per_batch, float eps) {
+    __shared__ __attribute__((aligned(16))) float red[3][8];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const size_t row = (size_t)blockIdx.x * 4 + wave;
-    if (row >= rows) return;
+    const size_t row = SPLIT ? (size_t)blockIdx.x : (size_t)blockIdx.x * 4 + wave;
+    const int cbase = SPLIT ? wave * 1024 : 0;
+    if constexpr (SPLIT) {
+        if (threadIdx.x < 24) red[threadIdx.x >> 3][threadIdx.x & 7] = 0.0f;
+        __syncthreads();
+    } else {
+        if (row >= rows) return;
+    }
+    // sum / max over the whole row from per-wavefront results (slot k of the LDS array is used once)
+    auto row_sum = [&](float v, int k) -> float {
+        v = wave_sum(v);
+        if constexpr (SPLIT) {
+            if (lane == 0) red[k][wave] = v;
+            __syncthreads();
+            const float4 a = *reinterpret_cast<const float4*>(red[k]), b = *reinterpret_cast<const float4*>(red[k] + 4);
+            v = ((((a.x + a.y) + a.z) + a.w) + b.x) + b.y;
+        }
+        return v;
+    };
+    auto row_max = [&](float v, int k) -> float {
+        v = wave_max(v);
+        if constexpr (SPLIT) {
+            if (lane == 0) red[k][wave] = v;
+            __syncthreads();
+            const float4 a = *reinterpret_cast<const float4*>(red[k]), b = *reinterpret_cast<const float4*>(red[k] + 4);
+            v = fmaxf(fmaxf(fmaxf(a.x, a.y), fmaxf(a.z, a.w)), fmaxf(b.x, b.y));
+        }
+        return v;
+    };
     const size_t row_off = row * (size_t)dim;
     const unsigned short* xs = static_cast<const unsigned short*>(src) + row_off;
     const size_t mod_off = (MOD || RESID == 2) ? (row / rows_per_batch) * (size_t)dim : 0;
@@ -61,7 +93,7 @@ __global__ __launch_bounds__(256) void ln_quant_rows_kernel(uint8_t* __restrict_
     float sum = 0.0f;
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
-        const int col = (p * 64 + lane) * 8;
+        const int col = cbase + (p * 64 + lane) * 8;
 #pragma unroll
         for (int i = 0; i < 8; ++i) h[p][i] = 0.0f;
         if (col < dim) {
@@ -92,41 +124,63 @@ __global__ __launch_bounds__(256) void ln_quant_rows_kernel(uint8_t* __restrict_
             for (int i = 0; i < 8; ++i) sum += h[p][i];
         }
     }
-    const float mean = wave_sum(sum) / (float)dim;
-    float sq = 0.0f;
+    // the modulation vectors are requested before the reductions, whose barriers no load may cross
+    // (without them the compiler places these loads itself)
+    uint4 graw[NP], braw[NP];
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
-        const int col = (p * 64 + lane) * 8;
+        const int col = cbase + (p * 64 + lane) * 8;
+        graw[p] = braw[p] = make_uint4(0, 0, 0, 0);
+        if (SPLIT && col < dim) {
+            graw[p] = *reinterpret_cast<const uint4*>(gs + col);
+            braw[p] = *reinterpret_cast<const uint4*>(bs + col);
+        }
+    }
+    const float mean = row_sum(sum, 0) / (float)dim;
+    float sq = 0.0f;  // from here on h holds the deviations from the mean
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        const int col = cbase + (p * 64 + lane) * 8;
         if (col < dim) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const float d = h[p][i] - mean;
-                sq += d * d;
+                h[p][i] = h[p][i] - mean;
+                sq = __builtin_fmaf(h[p][i], h[p][i], sq);
             }
         }
     }
-    const float var = wave_sum(sq) / (float)dim;
+    const float var = row_sum(sq, 1) / (float)dim;
     const float rstd = 1.0f / __builtin_sqrtf(var + eps);
     // normalise, modulate, round to T; for the int8 modes apply the smoothing vector and collect the row amax
     float amax = 0.0f;
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
-        const int col = (p * 64 + lane) * 8;
+        const int col = cbase + (p * 64 + lane) * 8;
         if (col < dim) {
             float g[8], b[8];
-            unpack8<Tag>(*reinterpret_cast<const uint4*>(gs + col), g);
-            unpack8<Tag>(*reinterpret_cast<const uint4*>(bs + col), b);
+            if constexpr (!SPLIT) {
+                graw[p] = *reinterpret_cast<const uint4*>(gs + col);
+                braw[p] = *reinterpret_cast<const uint4*>(bs + col);
+            }
+            unpack8<Tag>(graw[p], g);
+            unpack8<Tag>(braw[p], b);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float n = (h[p][i] - mean) * rstd;
-                float y;
+            for (int i = 0; i < 8; i += 2) {
+                float n0 = h[p][i] * rstd, n1 = h[p][i + 1] * rstd;
+                float y0, y1;
                 if constexpr (MOD) {
-                    const float a = round_through<Tag>(g[i] + 1.0f);
-                    y = round_through<Tag>(round_through<Tag>(a * round_through<Tag>(n)) + b[i]);
+                    float a0 = g[i] + 1.0f, a1 = g[i + 1] + 1.0f;
+                    round_through2<Tag>(a0, a1);
+                    round_through2<Tag>(n0, n1);
+                    y0 = a0 * n0, y1 = a1 * n1;
+                    round_through2<Tag>(y0, y1);
+                    y0 = y0 + b[i], y1 = y1 + b[i + 1];
                 } else {
-                    y = round_through<Tag>(g[i] * n + b[i]);
+                    y0 = g[i] * n0 + b[i], y1 = g[i + 1] * n1 + b[i + 1];
                 }
-                h[p][i] = y;
+                round_through2<Tag>(y0, y1);
+                h[p][i] = y0;
+                h[p][i + 1] = y1;
             }
             if constexpr (QMODE < 2) {
                 if (pre != nullptr) {
@@ -145,17 +199,17 @@ __global__ __launch_bounds__(256) void ln_quant_rows_kernel(uint8_t* __restrict_
     }
     float s = 1.0f;
     if constexpr (QMODE == 1) {
-        amax = wave_max(amax);
+        amax = row_max(amax, 2);
         s = amax / 127.0f;
         if (amax <= 5.9604644775390625e-08f) s = 1.0f;
-        if (lane == 0) scale_out[row] = s;
+        if (threadIdx.x == (SPLIT ? 0 : wave * 64)) scale_out[row] = s;
     } else if constexpr (QMODE != 3) {
         s = in_scale[0];
     }
     if constexpr (QMODE == 3) {
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
-            const int col = (p * 64 + lane) * 8;
+            const int col = cbase + (p * 64 + lane) * 8;
             if (col < dim) {
                 uint4 o;
                 u32* ow = reinterpret_cast<u32*>(&o);
@@ -172,7 +226,7 @@ __global__ __launch_bounds__(256) void ln_quant_rows_kernel(uint8_t* __restrict_
         const float inv = 1.0f / (o2 ? in_scale_b[0] : s);
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
-            const int col = (p * 64 + lane) * 8;
+            const int col = cbase + (p * 64 + lane) * 8;
             if (col < dim) {
                 float v[8];
                 float nanp = 0.0f;
@@ -197,13 +251,16 @@ __global__ __launch_bounds__(256) void ln_quant_rows_kernel(uint8_t* __restrict_
         const bool slow = scale_out_of_range(s);
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
-            const int col = (p * 64 + lane) * 8;
+            const int col = cbase + (p * 64 + lane) * 8;
             if (col < dim) {
-                int q[8];
-                quant8<-128, 127>(h[p], s, r, slow, q);
                 uint2 o;
-                o.x = pack4_s8(q[0], q[1], q[2], q[3]);
-                o.y = pack4_s8(q[4], q[5], q[6], q[7]);
+                if constexpr (QMODE == 1) o = quant8_pack_unclamped(h[p], s, r, slow);
+                else {
+                    int q[8];
+                    quant8<-128, 127>(h[p], s, r, slow, q);
+                    o.x = pack4_s8(q[0], q[1], q[2], q[3]);
+                    o.y = pack4_s8(q[4], q[5], q[6], q[7]);
+                }
                 *reinterpret_cast<uint2*>(dst + row_off + col) = o;
             }
         }
@@ -218,17 +275,20 @@ struct LnArgs {
 
 template <typename Tag, int QMODE, int RESID, bool MOD> static int launch_ln(const LnArgs& a, hipStream_t st) {
     const int np = (a.dim + 511) / 512;
+    if (np > 3) {
+        LQ_REQUIRE(a.rows <= 0x7fffffffu, LQ_ERR_SHAPE, "layernorm: %zu rows exceed the launch limit", a.rows);
+        dim3 grid((unsigned)a.rows), block(64 * ((np + 1) / 2));
+        hipLaunchKernelGGL((ln_quant_rows_kernel<Tag, 2, QMODE, RESID, MOD, true>), grid, block, 0, st, a.dst, a.dst2, a.scale_out,
+                           a.src, a.residual, a.bias, a.gamma, a.beta, a.pre, a.in_scale, a.dst_b, a.in_scale_b, a.rows, a.dim, a.rows_per_batch, a.eps);
+        return check_launch("layernorm_quant");
+    }
     dim3 grid((unsigned)((a.rows + 3) / 4)), block(256);
 #define LQ_LN_CASE(NPV)                                                                                              \
-    hipLaunchKernelGGL((ln_quant_rows_kernel<Tag, NPV, QMODE, RESID, MOD>), grid, block, 0, st, a.dst, a.dst2, a.scale_out, \
+    hipLaunchKernelGGL((ln_quant_rows_kernel<Tag, NPV, QMODE, RESID, MOD, false>), grid, block, 0, st, a.dst, a.dst2, a.scale_out, \
                        a.src, a.residual, a.bias, a.gamma, a.beta, a.pre, a.in_scale, a.dst_b, a.in_scale_b, a.rows, a.dim, a.rows_per_batch, a.eps)
     if (np <= 1) LQ_LN_CASE(1);
     else if (np <= 2) LQ_LN_CASE(2);
-    else if (np <= 3) LQ_LN_CASE(3);
-    else if (np <= 4) LQ_LN_CASE(4);
-    else if (np <= 6) LQ_LN_CASE(6);
-    else if (np <= 8) LQ_LN_CASE(8);
-    else LQ_LN_CASE(12);
+    else LQ_LN_CASE(3);
 #undef LQ_LN_CASE
     return check_launch("layernorm_quant");
 }

@@ -113,7 +113,8 @@ def sq_dynamic_scale(x, pre) -> np.ndarray:
     (convert_sd_quant_model.py:137-150): amax <= 2^-24 -> scale 1 (q is 0 either way).
     `amax / 127.0` is a double division narrowed to float == correctly rounded fp32 division."""
     t = sq_smoothed(x, pre)
-    amax = np.fmax.reduce(np.abs(t), axis=1).astype(F32)  # fmax: a NaN operand is dropped, as CUDA's max does
+    # fmax: a NaN operand is dropped, as CUDA's max does; the running maximum starts at 0 (an all-NaN row gives 0)
+    amax = np.fmax.reduce(np.abs(t), axis=1, initial=F32(0)).astype(F32)
     s = amax / F32(127.0)
     return np.where(amax <= F32(2.0 ** -24), F32(1.0), s).astype(F32)
 

@@ -28,7 +28,7 @@ def close_codes(got, ref, what):
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
-@pytest.mark.parametrize("rows,dim", [(1024, 1280), (4096, 640), (77, 320), (4608, 3072), (5, 6144)])
+@pytest.mark.parametrize("rows,dim", [(1024, 1280), (4096, 640), (77, 320), (4608, 3072), (5, 6144), (33, 2056), (7, 4104)])
 @pytest.mark.parametrize("dynamic", [False, True])
 def test_layernorm_int8(ops, dev, dt, rows, dim, dynamic):
     g = rng_t(rows + dim)
@@ -71,7 +71,7 @@ def test_fused_residual_bias_layernorm_int8(ops, dev, dt, with_bias):
 
 
 @pytest.mark.parametrize("dt", ["bf16", "f16"])
-@pytest.mark.parametrize("batch,seq,dim", [(2, 2304, 3072), (1, 512, 3072), (3, 50, 768)])
+@pytest.mark.parametrize("batch,seq,dim", [(2, 2304, 3072), (1, 512, 3072), (3, 50, 768), (2, 37, 2568)])
 def test_layernorm_mod_fp8(ops, dev, dt, batch, seq, dim):
     g = rng_t(batch + seq + dim)
     t = TORCH_DT[dt]

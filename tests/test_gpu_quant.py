@@ -19,7 +19,7 @@ def ops(dev):
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
-@pytest.mark.parametrize("m,k", [(1024, 1280), (37, 640), (5, 8), (3, 2560), (64, 12288), (7, 1283)])
+@pytest.mark.parametrize("m,k", [(1024, 1280), (37, 640), (5, 8), (3, 2560), (64, 12288), (7, 1283), (301, 3072), (19, 2056), (3, 16384)])
 def test_sq_dynamic_quant(ops, dev, dt, m, k):
     x = make_outlier_acts(m, k, min(8, k), 20.0, TORCH_DT[dt], 1000 + m + k)
     pre = (torch.rand(k, generator=rng_t(7)) * 1.5 + 0.25).float()
@@ -31,6 +31,23 @@ def test_sq_dynamic_quant(ops, dev, dt, m, k):
     q2, s2 = ops.sq_quant_dynamic(x.to(dev), None)
     q2_ref, s2_ref = O.sq_dynamic_quant(to_np_f32(x), None)
     assert np.array_equal(s2.cpu().numpy(), s2_ref) and np.array_equal(q2.cpu().numpy(), q2_ref)
+
+
+@pytest.mark.parametrize("k", [64, 2080])
+def test_sq_dynamic_nan_and_inf_rows(ops, dev, k):
+    """NaN never enters the row maximum and quantises to 0; a row holding an infinity gets an infinite scale,
+    its finite elements become 0 and inf/inf = NaN becomes 0 as well (the oracle's IEEE arithmetic decides)."""
+    x = torch.randn(6, k, generator=rng_t(k)) * 3
+    x[1, 5] = float("nan")
+    x[2, 7] = float("inf")
+    x[3, 9] = float("-inf"); x[3, 11] = float("nan")
+    x[4, :] = float("nan")
+    x[5, k - 1] = float("nan"); x[5, k - 2] = 1e30
+    for pre in (None, (torch.rand(k, generator=rng_t(3)) + 0.5).float()):
+        q, s = ops.sq_quant_dynamic(x.to(dev), None if pre is None else pre.to(dev))
+        q_ref, s_ref = O.sq_dynamic_quant(x.numpy(), None if pre is None else pre.numpy())
+        assert np.array_equal(s.cpu().numpy(), s_ref, equal_nan=True)
+        assert np.array_equal(q.cpu().numpy(), q_ref)
 
 
 def test_sq_dynamic_zero_rows(ops, dev):
@@ -46,8 +63,9 @@ def test_sq_dynamic_zero_rows(ops, dev):
 
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
 @pytest.mark.parametrize("per_token", [False, True])
-def test_sq_static_quant(ops, dev, dt, per_token):
-    m, k = 300, 1280
+@pytest.mark.parametrize("k", [1280, 3080])
+def test_sq_static_quant(ops, dev, dt, per_token, k):
+    m = 300
     x = make_outlier_acts(m, k, 8, 20.0, TORCH_DT[dt], 5)
     pre = (torch.rand(k, generator=rng_t(8)) + 0.5).float()
     # a static scale small enough that saturation to -128 / 127 happens
@@ -58,11 +76,12 @@ def test_sq_static_quant(ops, dev, dt, per_token):
     assert np.array_equal(q.cpu().numpy(), q_ref)
 
 
-def test_sq_quant_ties_and_specials(ops, dev):
+@pytest.mark.parametrize("reps", [4, 130])  # 64 columns (one wavefront per row) and 2080 (row split over wavefronts)
+def test_sq_quant_ties_and_specials(ops, dev, reps):
     # exact half-integers, saturation edges, NaN and inf, with s = 1 and a power-of-two s
     vals = [0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 126.5, 127.5, -127.5, -128.5, 300.0, -300.0,
             float("nan"), float("inf"), float("-inf"), 0.0]
-    x = torch.tensor(vals * 4, dtype=torch.float32).reshape(1, -1)
+    x = torch.tensor(vals * reps, dtype=torch.float32).reshape(1, -1)
     for s in (1.0, 0.5, 3.0):
         sc = torch.tensor([s], dtype=torch.float32)
         q = ops.sq_quant(x.to(dev), None, sc.to(dev), False)
