@@ -184,7 +184,9 @@ __device__ __forceinline__ int cvt_i32_sat(float x) {
 // fp32 rounding and t*r all round to the same integer.  Beyond 512 in magnitude everything saturates.
 // If any of the eight values fails the test (or the caller flags the scale as unsafe for a
 // reciprocal), the whole octet is redone with true divisions: one rarely taken branch.
-template <int LO, int HI>
+// CLAMP false: the caller guarantees |t[i]| <= LIMIT * s * (1 + 2^-20) with LIMIT = HI (a scale derived from the maximum of
+// these very values), so rint(t/s) cannot leave [LO, HI] and the clamp is skipped.
+template <int LO, int HI, bool CLAMP = true>
 __device__ __forceinline__ void quant8(const float* t, float s, float r, bool slow, int* q) {
     float rq[8], dev = 0.0f;
 #pragma unroll
@@ -203,7 +205,7 @@ __device__ __forceinline__ void quant8(const float* t, float s, float r, bool sl
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int v = cvt_i32_sat(rq[i]);
-        q[i] = v < LO ? LO : (v > HI ? HI : v);
+        q[i] = CLAMP ? (v < LO ? LO : (v > HI ? HI : v)) : v;
     }
 }
 // The dynamic per-token case: every |t[i]| <= amax and s = fl(amax / 127), so |t[i] / s| stays below 127.00002

@@ -124,10 +124,14 @@ __global__ __launch_bounds__(256) void w4a4_quant_kernel(u32* __restrict__ q_wor
             }
             const float r = fast_recip(s);
             int q[8];
-            quant8<-8, 7>(v, s, r, slow, q);
-            u32 word = (u32)q[0] & 0xFu;
+            // fp32 scale: s = fl(absmax / 7) bounds every |v / s| by 7.000001, no clamp needed.  An fp16 scale may have been
+            // rounded down by a large factor in the subnormal range, so those results are clamped.
+            quant8<-8, 7, F16_SCALE>(v, s, r, slow, q);
+            // nibble i of the word = low four bits of q[i]: each step shifts the word right by four and
+            // enters the next value's low nibble at the top (one v_alignbit_b32 per element)
+            u32 word = 0;
 #pragma unroll
-            for (int i = 1; i < 8; ++i) word = (word & ~(0xFu << (4 * i))) | (((u32)q[i] << (4 * i)) & (0xFu << (4 * i)));
+            for (int i = 0; i < 8; ++i) word = __builtin_amdgcn_alignbit((u32)q[i], word, 4);
             if (col < k) {
                 q_words[(size_t)row * (k >> 3) + (col >> 3)] = word;
                 if ((lane & 7) == 0) {

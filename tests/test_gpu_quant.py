@@ -149,6 +149,28 @@ def test_w4a4_quant(ops, dev, dt, sdt, m, k):
         assert np.array_equal(q.cpu().numpy().view(np.uint32), q_ref)
 
 
+@pytest.mark.parametrize("sdt", ["f32", "f16"])
+@pytest.mark.parametrize("k", [256, 3072])
+def test_w4a4_quant_special_groups(ops, dev, sdt, k):
+    """Groups holding NaN or infinity, and groups so small that an fp16 scale is subnormal (rounded down by a large
+    factor, so the quotients exceed 7 and must saturate) or zero."""
+    g = rng_t(k)
+    x = torch.randn(8, k, generator=g)
+    x[0, 3] = float("nan")
+    x[1, 70] = float("inf")
+    x[2, 130] = float("-inf"); x[2, 131] = float("nan")
+    x[3, :64] = torch.randn(64, generator=g) * 1.1e-7   # absmax/7 between fp16 subnormal steps
+    x[4, :64] = torch.randn(64, generator=g) * 3e-9     # fp16 scale underflows to zero
+    x[5, 64:128] = torch.randn(64, generator=g) * 2.5e-7
+    x[6, :64] = 1e-30
+    smooth = (torch.rand(k, generator=g) * 1.5 + 0.5).float()
+    for sm in (None, smooth):
+        q, s = ops.w4a4_quant(x.to(dev), None if sm is None else sm.to(dev), TORCH_DT[sdt])
+        q_ref, s_ref = O.w4a4_quant(x.numpy(), None if sm is None else sm.numpy(), 64, sdt)
+        assert np.array_equal(s.cpu().float().numpy(), s_ref, equal_nan=True)
+        assert np.array_equal(q.cpu().numpy().view(np.uint32), q_ref)
+
+
 def test_repack_roundtrip(ops, dev):
     w = torch.randint(-128, 128, (1280, 640), dtype=torch.int8)
     p = ops.repack_weight(w.to(dev))
