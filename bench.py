@@ -250,12 +250,12 @@ def extra_kernels(torch, ops, dev):
     sm = (torch.rand(k, generator=g) + 0.5).to(dev)
     us = timeit(lambda: ops.w4a4_quant(x, sm))
     res[f"w4a4_quant_{m}x{k}"] = {"us": round(us, 2), "GB/s": round((2.5 * m * k + 4.0 * m * k / 64) / us / 1e3, 1)}
-    for (m, k) in [(1024, 1280), (4096, 640)]:
+    for (m, k) in [(1024, 1280), (4096, 640), (4608, 3072), (4608, 12288)]:
         x = torch.randn(m, k, generator=g).half().to(dev)
         pre = (torch.rand(k, generator=g) + 0.5).to(dev)
         us = timeit(lambda: ops.sq_quant_dynamic(x, pre))
         res[f"sq_dynamic_quant_{m}x{k}"] = {"us": round(us, 2), "GB/s": round((3.0 * m * k + 4 * m + 4 * k) / us / 1e3, 1)}
-    for (m, k) in [(4096, 1280), (4096, 640)]:
+    for (m, k) in [(4096, 1280), (4096, 640), (4608, 3072)]:
         x = torch.randn(m, k, generator=g).half().to(dev)
         gb = torch.randn(k, generator=g).half().to(dev)
         us = timeit(lambda: ops.layernorm_int8(x, gb, gb, None, None))
