@@ -7,6 +7,7 @@
 // reduces in registers -> wavefront shuffles -> LDS and issues one atomic per workgroup, and
 // the cast kernel moves 32 B in / 16 B out per lane per step.
 #include "lq_common.h"
+#include <atomic>
 
 namespace lq {
 
@@ -320,33 +321,36 @@ __global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_
     }
 }
 
+static std::atomic<unsigned> g_next_slot{0};  // one round-robin counter for every element type and host thread
+
 // Returns LQ_OK when the fused launch was issued, 1 when the caller should fall back to the
 // three-kernel sequence (unaligned buffers, or the occupancy query failed).
 template <typename Tag>
 static int launch_amax_cast_coop(uint8_t* dst, float* scale_out, const void* src, size_t n, hipStream_t st) {
-    static int blocks_per_cu = -1, num_cu = 0;
-    static unsigned next_slot = 0;
     constexpr int KEEP = 8;
     auto kern = fp8_amax_cast_coop_kernel<Tag, KEEP>;
     if (reinterpret_cast<uintptr_t>(src) % 16 != 0 || reinterpret_cast<uintptr_t>(dst) % 16 != 0) return 1;
-    if (blocks_per_cu < 0) {
+    struct Capacity { int blocks_per_cu = 0, num_cu = 0; };
+    // queried once (thread-safe initialisation of a function-local static)
+    static const Capacity cap = [&] {
+        Capacity c;
         int dev = 0, occ = 0;
         hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess ||
-            hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, kCoopThreads, 0) != hipSuccess || occ < 1) {
-            blocks_per_cu = 0;
-        } else {
-            blocks_per_cu = occ > 2 ? 2 : occ;
-            num_cu = prop.multiProcessorCount;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+            hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, kCoopThreads, 0) == hipSuccess && occ >= 1) {
+            c.blocks_per_cu = occ > 2 ? 2 : occ;
+            c.num_cu = prop.multiProcessorCount;
         }
         (void)hipGetLastError();
-    }
+        return c;
+    }();
+    const int blocks_per_cu = cap.blocks_per_cu, num_cu = cap.num_cu;
     if (blocks_per_cu == 0) return 1;
     int grid = blocks_per_cu * num_cu;
     if (grid > kCoopMaxBlocks) grid = kCoopMaxBlocks;
     size_t need = (n / Chunk16<Tag>::elems + kCoopThreads - 1) / kCoopThreads;
     if ((size_t)grid > need) grid = need ? (int)need : 1;
-    int slot = (int)(next_slot++ % kCoopSlots);
+    int slot = (int)(g_next_slot.fetch_add(1, std::memory_order_relaxed) % kCoopSlots);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kCoopThreads), 0, st, dst, scale_out, src, n, slot);
     return check_launch("fp8_amax_cast_fused");
 }
