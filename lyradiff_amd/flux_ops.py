@@ -1,0 +1,200 @@
+"""Block-level FLUX ops with the interface of the reference's torch custom classes.
+
+`FluxTransformerBlockOp` / `FluxSingleTransformerBlockOp` mirror the classes the reference registers in
+src/lyradiff/th_op/pybind.cc:66-96 (constructor arguments, initialize, forward, reload_model_from_state_dict,
+load_lora_by_name, clear_lora: th_op/flux_transformer_block/FluxTransformerBlockOp.cc:6-107 and
+th_op/flux_single_transformer_block/FluxSingleTransformerBlockOp.cc:6-98), so that the reference's Python wrappers
+(lyradiff/lyradiff_model/lyradiff_flux_transformer_model_v2.py:67-168) can hold one of these instead of a
+`torch.classes.lyradiff.*` object.  Every quantized linear, every adaLN / gate / residual step and every activation
+quantisation runs on this library's HIP kernels (flux_fp8.py); the attention core between the QKV projection and the
+output projection -- per-head RMSNorm of q and k, rotary embedding, softmax attention -- is not part of the
+quantized-linear path and is plain PyTorch here (`flux_attention_core`).
+
+Supported quant levels: FP8_W8A8 and FP8_W8A8_FULL.  Any other level raises at construction.
+"""
+from __future__ import annotations
+
+from enum import Enum
+from typing import Mapping, Optional, Sequence
+
+import torch
+
+from . import flux_fp8 as F
+
+
+class LyraQuantLevel(Enum):
+    """lyradiff/lyradiff_model/lyradiff_utils.py:4-13."""
+    NONE = 0
+    FP8_W8A8 = 1
+    FP8_W8A8_FULL = 2
+    FP8_WEIGHT_ONLY = 3
+    INT8_SMOOTH_QUANT_LEVEL1 = 4
+    INT8_SMOOTH_QUANT_LEVEL2 = 5
+    INT8_SMOOTH_QUANT_LEVEL3 = 6
+    INT4_W4A4 = 7
+    INT4_W4A4_FULL = 8
+
+
+_DTYPES = {"fp16": torch.float16, "bf16": torch.bfloat16}
+
+
+def _rms_norm_rope(qkv: torch.Tensor, norm_q: torch.Tensor, norm_k: torch.Tensor, rope: torch.Tensor, heads: int,
+                   eps: float = 1e-6):
+    """qkv [B, S, 3*H*Dh] -> q, k, v [B, H, S, Dh] with q and k RMS-normalised per head and rotated.
+
+    Follows fuseRmsNormCatAndRope / fuseRmsNormAndRope (src/lyradiff/kernels/rope/flux_apply_rope.cu:74-156): mean of
+    squares and the scaling by its inverse root in fp32, the result rounded to T, multiplied by the norm weight in T,
+    then each pair (x, y) of adjacent elements becomes (x*r00 + y*r01, x*r10 + y*r11) with the 2x2 matrices of
+    `rope` [B or 1, S, Dh/2, 2, 2].  v passes through.
+    """
+    b, s, d3 = qkv.shape
+    dh = d3 // (3 * heads)
+    q, k, v = qkv.view(b, s, 3, heads, dh).unbind(2)
+    rope = rope.reshape(-1, s, 1, dh // 2, 2, 2).to(qkv.dtype)
+
+    def one(t, w):
+        f = t.float()
+        n = (f * torch.rsqrt(f.pow(2).mean(-1, keepdim=True) + eps)).to(t.dtype) * w.to(t.dtype)
+        p = n.view(b, s, heads, dh // 2, 1, 2)
+        return (p * rope).sum(-1).view(b, s, heads, dh)
+
+    return one(q, norm_q).transpose(1, 2), one(k, norm_k).transpose(1, 2), v.transpose(1, 2)
+
+
+def flux_attention_core(qkv: torch.Tensor, norm_q: torch.Tensor, norm_k: torch.Tensor, rope_emb: torch.Tensor, heads: int,
+                        context_qkv: Optional[torch.Tensor] = None, norm_added_q: Optional[torch.Tensor] = None,
+                        norm_added_k: Optional[torch.Tensor] = None):
+    """The part of FluxAttentionFP8Processor::forward (FluxAttentionFP8Processor.cc:232-291) and
+    FluxSingleAttentionFP8Processor::forward (FluxSingleAttentionFP8Processor.cc:183-213) between the QKV and the output
+    projections.  With `context_qkv` the text tokens come first in the joint sequence (`rope_emb` covers text + image) and
+    (image [B, S, D], text [B, Sc, D]) is returned; without it a single [B, S, D] tensor."""
+    b, s, d3 = qkv.shape
+    d = d3 // 3
+    if context_qkv is None:
+        q, k, v = _rms_norm_rope(qkv, norm_q, norm_k, rope_emb, heads)
+    else:
+        sc = context_qkv.shape[1]
+        rope_emb = rope_emb.reshape(-1, sc + s, d // heads // 2, 2, 2)
+        parts = [_rms_norm_rope(context_qkv, norm_added_q, norm_added_k, rope_emb[:, :sc], heads),
+                 _rms_norm_rope(qkv, norm_q, norm_k, rope_emb[:, sc:], heads)]
+        q, k, v = (torch.cat([parts[0][i], parts[1][i]], dim=2) for i in range(3))
+    o = torch.nn.functional.scaled_dot_product_attention(q, k, v)
+    o = o.transpose(1, 2).reshape(b, -1, d)
+    if context_qkv is None:
+        return o
+    return o[:, sc:], o[:, :sc]
+
+
+def _get(src: Mapping, name: str, shape, dtype) -> torch.Tensor:
+    if name not in src:
+        raise KeyError(f"Cannot find a tensor of name {name}")
+    t = src[name]
+    if tuple(t.shape) != tuple(shape) or t.dtype != dtype:
+        raise ValueError(f"{name}: got {tuple(t.shape)} {t.dtype}, expected {tuple(shape)} {dtype}")
+    return t
+
+
+class _BlockOpBase:
+    def __init__(self, inference_dtype: str, embedding_dim: int, embedding_head_num: int, embedding_head_dim: int,
+                 mlp_scale: int, quant_level: int):
+        if inference_dtype not in _DTYPES:
+            raise ValueError("wrong inference_dtype")  # the reference throws on anything but fp32 / fp16 / bf16
+        level = LyraQuantLevel(int(quant_level))
+        if level not in (LyraQuantLevel.FP8_W8A8, LyraQuantLevel.FP8_W8A8_FULL):
+            raise NotImplementedError(f"quant level {level.name}: only the FP8 blocks are built on this library")
+        if embedding_dim != embedding_head_num * embedding_head_dim:
+            raise ValueError("embedding_dim must equal embedding_head_num * embedding_head_dim")
+        self.inference_dtype = inference_dtype
+        self.dtype = _DTYPES[inference_dtype]
+        self.dim, self.heads, self.head_dim, self.mlp_scale = embedding_dim, embedding_head_num, embedding_head_dim, mlp_scale
+        self.quant_level = level
+        self.weights = None
+        self.device = "cuda"
+
+    def initialize(self, lyradiff_context=None) -> None:
+        """The reference creates its stream, cuBLAS wrapper and allocator here; nothing of the kind is needed."""
+
+    def _check(self, name: str, t: torch.Tensor) -> None:  # CHECK_TH_CUDA, CHECK_CONTIGUOUS, dtype TORCH_CHECK
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} must be a CUDA tensor")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous")
+        if t.dtype != self.dtype:
+            raise RuntimeError(f"{name} dtype should be {self.dtype}")
+
+    def _loaded(self):
+        if self.weights is None:
+            raise RuntimeError("reload_model_from_state_dict has not been called")
+        return self.weights
+
+    def _fp8_linears(self):
+        raise NotImplementedError
+
+    def load_lora_by_name(self, lora_name: Sequence[str], lora_weights: torch.Tensor, lora_strength: float) -> None:
+        """Merges `lora_strength * lora_weights` into the named linear's 16-bit master copy and re-quantises it
+        (FP8LoraWeight::load_lora, IFLoraWeight.h:79-128).  `lora_name` is the path the reference walks through its
+        lora_layer_map / lora_weight_map (IFLoraWeight.h:146-168): ["attn", "to_qkv"], ["attn", "to_out.0"],
+        ["ff", "net.0.proj"], ["norm1", "linear"], ["proj_mlp"], ...  An unknown name raises (the reference prints a
+        message and goes on)."""
+        key = ".".join(lora_name)
+        lin = self._fp8_linears().get(key)
+        if lin is None:
+            raise KeyError(f"no FP8 linear named {key} in this block")
+        lin.load_lora(lora_weights.to(self.device), float(lora_strength))
+
+    def clear_lora(self) -> None:
+        for lin in self._fp8_linears().values():
+            lin.clear_lora()
+
+
+class FluxTransformerBlockOp(_BlockOpBase):
+    """Double-stream FLUX block (FluxTransformerFP8Block.cc:159-262)."""
+
+    def reload_model_from_state_dict(self, prefix: str, weights: Mapping[str, torch.Tensor], device: str = "cpu") -> None:
+        """Keys as FluxTransformerFP8BlockWeight::loadWeightsFromCache / FluxAttentionFP8ProcessorWeight::loadWeightsFromCache
+        read them (FluxAttentionFP8ProcessorWeight.cc:194-260): the linears' `.weight`, `.bias`, `_input_scale`, and
+        `attn.norm_q.weight`, `attn.norm_k.weight`, `attn.norm_added_q.weight`, `attn.norm_added_k.weight`.  `device` names
+        where the tensors of `weights` live, as in the reference; they end up on the GPU either way."""
+        self.weights = F.load_flux_double_block_fp8(weights, prefix, self.dim, self.dtype, self.device, keep_master=True)
+        self.norms = [_get(weights, prefix + f"attn.{n}.weight", (self.head_dim,), self.dtype).to(self.device)
+                      for n in ("norm_q", "norm_k", "norm_added_q", "norm_added_k")]
+
+    def _fp8_linears(self):
+        w = self._loaded()
+        return {"norm1.linear": w.norm1, "norm1_context.linear": w.norm1_context, "attn.to_qkv": w.to_qkv,
+                "attn.to_added_qkv": w.to_added_qkv, "attn.to_out.0": w.to_out, "attn.to_add_out": w.to_add_out,
+                "ff.net.0.proj": w.ff.gelu_proj, "ff.net.2": w.ff.ff_linear,
+                "ff_context.net.0.proj": w.ff_context.gelu_proj, "ff_context.net.2": w.ff_context.ff_linear}
+
+    def forward(self, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor, rope_emb: torch.Tensor,
+                temb_emb: torch.Tensor):
+        """Returns [hidden_states_out, encoder_hidden_states_out] (FluxTransformerBlockOp.h:186-235)."""
+        w = self._loaded()
+        for n, t in (("hidden_states", hidden_states), ("encoder_hidden_states", encoder_hidden_states),
+                     ("rope_emb", rope_emb), ("temb_emb", temb_emb)):
+            self._check(n, t)
+        nq, nk, naq, nak = self.norms
+        core = lambda qkv, cqkv: flux_attention_core(qkv, nq, nk, rope_emb, self.heads, cqkv, naq, nak)
+        out, ctx = F.flux_double_block_fp8(hidden_states, encoder_hidden_states, temb_emb, w, core)
+        return [out, ctx]
+
+
+class FluxSingleTransformerBlockOp(_BlockOpBase):
+    """Single-stream FLUX block (FluxSingleTransformerFP8Block.cc:163-291)."""
+
+    def reload_model_from_state_dict(self, prefix: str, weights: Mapping[str, torch.Tensor], device: str = "cpu") -> None:
+        self.weights = F.load_flux_single_block_fp8(weights, prefix, self.dim, self.mlp_scale, self.dtype, self.device,
+                                                    keep_master=True)
+        self.norms = [_get(weights, prefix + f"attn.{n}.weight", (self.head_dim,), self.dtype).to(self.device)
+                      for n in ("norm_q", "norm_k")]
+
+    def _fp8_linears(self):
+        w = self._loaded()
+        return {"norm.linear": w.norm, "attn.to_qkv": w.to_qkv, "proj_mlp": w.mlp.proj_mlp, "proj_out": w.mlp.proj_out}
+
+    def forward(self, hidden_states: torch.Tensor, rope_emb: torch.Tensor, temb_emb: torch.Tensor) -> torch.Tensor:
+        w = self._loaded()
+        for n, t in (("hidden_states", hidden_states), ("rope_emb", rope_emb), ("temb_emb", temb_emb)):
+            self._check(n, t)
+        nq, nk = self.norms
+        return F.flux_single_block_fp8(hidden_states, temb_emb, w, lambda qkv: flux_attention_core(qkv, nq, nk, rope_emb, self.heads))

@@ -198,12 +198,12 @@ def test_fp8_linear_lora_requantise_and_clear(ops, dev):
         load_fp8_linear(sd, "blk.", "net.2", d_out, d_in, torch.bfloat16, dev).load_lora(delta, 1.0)
 
 
-def _state_dict(names_shapes, seed, scale_w=0.03):
+def _state_dict(names_shapes, seed, scale_w=0.03, prefix="p."):
     g = rng_t(seed)
     sd = {}
     for name, (n, k) in names_shapes.items():
-        sd[f"p.{name}.weight"] = (scale_w * torch.randn(n, k, generator=g)).bfloat16()
-        sd[f"p.{name}.bias"] = (0.1 * torch.randn(n, generator=g)).bfloat16()
+        sd[f"{prefix}{name}.weight"] = (scale_w * torch.randn(n, k, generator=g)).bfloat16()
+        sd[f"{prefix}{name}.bias"] = (0.1 * torch.randn(n, generator=g)).bfloat16()
     return sd
 
 
@@ -508,3 +508,127 @@ def test_whole_fp8_blocks_around_a_caller_supplied_attention(ops, dev):
     w1 = F.flux_attn_post_fp8(x, wd.to_out.forward(a1.contiguous()), m1, wd.ff)
     w2 = F.flux_attn_post_fp8(ctx, wd.to_add_out.forward(a2.contiguous()), m2, wd.ff_context)
     assert torch.equal(o1, w1) and torch.equal(o2, w2) and o2.shape == ctx.shape
+
+
+def _rope_table(b, s, dh, seed):
+    """[B, S, Dh/2, 2, 2] rotation matrices [[cos, -sin], [sin, cos]] as FLUX's EmbedND produces them."""
+    ang = torch.rand(b, s, dh // 2, generator=rng_t(seed)) * 6.28
+    return torch.stack([torch.cos(ang), -torch.sin(ang), torch.sin(ang), torch.cos(ang)], dim=-1).reshape(b, s, dh // 2, 2, 2)
+
+
+def _attention_reference(qkv, cqkv, norms, rope, heads):
+    """Independent fp64 restatement: RMSNorm per head, rotation written with complex numbers, softmax attention."""
+    def prep(t, wq, wk, rp):
+        b, s, d3 = t.shape
+        dh = d3 // 3 // heads
+        q, k, v = t.double().view(b, s, 3, heads, dh).unbind(2)
+        rot = torch.complex(rp[..., 0, 0].double(), rp[..., 1, 0].double()).unsqueeze(2)  # cos + i sin, [B, S, 1, Dh/2]
+
+        def one(x, w):
+            n = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6) * w.double()
+            z = torch.view_as_complex(n.reshape(b, s, heads, dh // 2, 2).contiguous()) * rot
+            return torch.view_as_real(z).reshape(b, s, heads, dh)
+
+        return one(q, wq), one(k, wk), v
+
+    s, sc = qkv.shape[1], (cqkv.shape[1] if cqkv is not None else 0)
+    if cqkv is None:
+        q, k, v = prep(qkv, norms[0], norms[1], rope)
+    else:
+        a = prep(cqkv, norms[2], norms[3], rope[:, :sc])
+        c = prep(qkv, norms[0], norms[1], rope[:, sc:])
+        q, k, v = (torch.cat([a[i], c[i]], dim=1) for i in range(3))
+    w = torch.softmax(torch.einsum("bshd,bthd->bhst", q, k) / q.shape[-1] ** 0.5, dim=-1)
+    o = torch.einsum("bhst,bthd->bshd", w, v).reshape(q.shape[0], sc + s, -1)
+    return (o[:, sc:], o[:, :sc]) if cqkv is not None else o
+
+
+def test_flux_attention_core_matches_an_independent_restatement(dev):
+    from lyradiff_amd.flux_ops import flux_attention_core
+
+    b, s, sc, heads, dh = 2, 80, 24, 4, 64
+    d = heads * dh
+    g = rng_t(301)
+    qkv = torch.randn(b, s, 3 * d, generator=g).bfloat16()
+    cqkv = torch.randn(b, sc, 3 * d, generator=g).bfloat16()
+    norms = [(1 + 0.2 * torch.randn(dh, generator=g)).bfloat16() for _ in range(4)]
+    rope = _rope_table(b, sc + s, dh, 302).bfloat16()
+    got, cgot = flux_attention_core(qkv.to(dev), norms[0].to(dev), norms[1].to(dev), rope.to(dev), heads, cqkv.to(dev),
+                                    norms[2].to(dev), norms[3].to(dev))
+    want, cwant = _attention_reference(qkv, cqkv, norms, rope, heads)
+    # bf16 q/k/v and a bf16 output: a few units of 2^-8 relative to the magnitude of v
+    assert (got.cpu().double() - want).abs().max() < 0.05 and (cgot.cpu().double() - cwant).abs().max() < 0.05
+    single = flux_attention_core(qkv.to(dev), norms[0].to(dev), norms[1].to(dev), rope[:, sc:].contiguous().to(dev), heads)
+    assert (single.cpu().double() - _attention_reference(qkv, None, norms, rope[:, sc:], heads)).abs().max() < 0.05
+
+
+def test_flux_block_ops_have_the_reference_interface(ops, dev):
+    """torch.classes.lyradiff.FluxTransformerBlockOp / FluxSingleTransformerBlockOp call sites
+    (lyradiff_flux_transformer_model_v2.py:77-168): constructor, initialize, reload_model_from_state_dict, forward,
+    load_lora_by_name, clear_lora; outputs equal the block functions driven with the same attention core."""
+    from lyradiff_amd import flux_fp8 as F
+    from lyradiff_amd import flux_ops as FO
+
+    b, s, sc, heads, dh = 2, 96, 32, 4, 64
+    d = heads * dh
+    g = rng_t(311)
+    names = {"norm.linear": (3 * d, d), "attn.to_qkv": (3 * d, d), "proj_mlp": (4 * d, d), "proj_out": (d, 5 * d),
+             "norm1.linear": (6 * d, d), "norm1_context.linear": (6 * d, d), "attn.to_added_qkv": (3 * d, d),
+             "attn.to_out.0": (d, d), "attn.to_add_out": (d, d), "ff.net.0.proj": (4 * d, d), "ff.net.2": (d, 4 * d),
+             "ff_context.net.0.proj": (4 * d, d), "ff_context.net.2": (d, 4 * d)}
+    sd = _state_dict(names, 312, prefix="transformer_blocks.3.")
+    sd.update(_state_dict(names, 313, prefix="single_transformer_blocks.5."))
+    for pre in ("transformer_blocks.3.", "single_transformer_blocks.5."):
+        for n in names:
+            sd[f"{pre}{n}_input_scale"] = torch.tensor([5.0 / 448])
+        for n in ("norm_q", "norm_k", "norm_added_q", "norm_added_k"):
+            sd[f"{pre}attn.{n}.weight"] = (1 + 0.1 * torch.randn(dh, generator=g)).bfloat16()
+    x = torch.randn(b, s, d, generator=g).bfloat16().to(dev)
+    ctx = torch.randn(b, sc, d, generator=g).bfloat16().to(dev)
+    temb = torch.randn(b, d, generator=g).bfloat16().to(dev)
+    rope = _rope_table(b, sc + s, dh, 314).bfloat16().to(dev)
+
+    op = FO.FluxTransformerBlockOp("bf16", d, heads, dh, 6, FO.LyraQuantLevel.FP8_W8A8.value)
+    op.initialize(None)
+    with pytest.raises(RuntimeError):
+        op.forward(x, ctx, rope, temb)  # nothing loaded yet
+    op.reload_model_from_state_dict("transformer_blocks.3.", sd, "cpu")
+    res = op.forward(x, ctx, rope, temb)
+    assert isinstance(res, list) and res[0].shape == x.shape and res[1].shape == ctx.shape
+    wd = F.load_flux_double_block_fp8(sd, "transformer_blocks.3.", d, torch.bfloat16, dev)
+    nq, nk, naq, nak = (sd[f"transformer_blocks.3.attn.{n}.weight"].to(dev) for n in ("norm_q", "norm_k", "norm_added_q", "norm_added_k"))
+    w1, w2 = F.flux_double_block_fp8(x, ctx, temb, wd, lambda a, c: FO.flux_attention_core(a, nq, nk, rope, heads, c, naq, nak))
+    assert torch.equal(res[0], w1) and torch.equal(res[1], w2) and torch.isfinite(w1.float()).all()
+    # LoRA: merging a delta changes the output, clearing it restores the original bit for bit
+    delta = (0.05 * torch.randn(3 * d, d, generator=g)).bfloat16()
+    op.load_lora_by_name(["attn", "to_qkv"], delta, 0.8)
+    assert not torch.equal(op.forward(x, ctx, rope, temb)[0], res[0])
+    op.clear_lora()
+    again = op.forward(x, ctx, rope, temb)
+    assert torch.equal(again[0], res[0]) and torch.equal(again[1], res[1])
+    with pytest.raises(KeyError):
+        op.load_lora_by_name(["attn", "nope"], delta, 1.0)
+    # argument checks of the reference's forward
+    with pytest.raises(RuntimeError):
+        op.forward(x.float(), ctx, rope, temb)
+    with pytest.raises(RuntimeError):
+        op.forward(x.cpu(), ctx, rope, temb)
+    with pytest.raises(RuntimeError):
+        op.forward(x.transpose(0, 1), ctx, rope, temb)
+    # unsupported levels and dtypes fail at construction
+    with pytest.raises(NotImplementedError):
+        FO.FluxTransformerBlockOp("bf16", d, heads, dh, 6, FO.LyraQuantLevel.NONE.value)
+    with pytest.raises(ValueError):
+        FO.FluxSingleTransformerBlockOp("int8", d, heads, dh, 4, 1)
+    with pytest.raises(KeyError):
+        FO.FluxSingleTransformerBlockOp("bf16", d, heads, dh, 4, 2).reload_model_from_state_dict("missing.", sd, "cpu")
+
+    sop = FO.FluxSingleTransformerBlockOp("bf16", d, heads, dh, 4, FO.LyraQuantLevel.FP8_W8A8_FULL.value)
+    sop.initialize(None)
+    sop.reload_model_from_state_dict("single_transformer_blocks.5.", sd, "cpu")
+    xs = torch.cat([ctx, x], dim=1).contiguous()
+    y = sop.forward(xs, rope, temb)
+    ws = F.load_flux_single_block_fp8(sd, "single_transformer_blocks.5.", d, 4, torch.bfloat16, dev)
+    snq, snk = (sd[f"single_transformer_blocks.5.attn.{n}.weight"].to(dev) for n in ("norm_q", "norm_k"))
+    want = F.flux_single_block_fp8(xs, temb, ws, lambda a: FO.flux_attention_core(a, snq, snk, rope, heads))
+    assert y.shape == xs.shape and torch.equal(y, want) and torch.isfinite(y.float()).all()

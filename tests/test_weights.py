@@ -118,6 +118,21 @@ def test_int4_pack_helpers_match_the_oracle_packing():
         W.pack_int8_tensor_to_packed_int4(torch.tensor([[8, 0]], dtype=torch.int8))
 
 
+def test_flux_block_op_constructor_checks():
+    """The constructors of the block classes validate their arguments without touching a GPU."""
+    from lyradiff_amd import flux_ops as FO
+
+    assert [l.value for l in FO.LyraQuantLevel] == list(range(9))
+    op = FO.FluxSingleTransformerBlockOp("fp16", 256, 4, 64, 4, 2)
+    assert op.dtype == torch.float16 and op.quant_level is FO.LyraQuantLevel.FP8_W8A8_FULL
+    with pytest.raises(RuntimeError, match="reload_model_from_state_dict"):
+        op.clear_lora()
+    with pytest.raises(ValueError):
+        FO.FluxTransformerBlockOp("bf16", 256, 4, 60, 6, 1)  # dim != heads * head_dim
+    with pytest.raises(NotImplementedError):
+        FO.FluxTransformerBlockOp("bf16", 256, 4, 64, 6, FO.LyraQuantLevel.INT4_W4A4.value)
+
+
 @pytest.mark.gpu
 def test_smooth_vector_on_device(dev):
     from lyradiff_amd import ops
