@@ -22,11 +22,13 @@ kernels.  Attention (QKV, rotary, flash attention) stays with the caller.
 from __future__ import annotations
 
 from dataclasses import dataclass
+from typing import Union
 
 import torch
 
 from . import ops
-from .weights import FP8Linear, W4A4Linear, load_fp8_linear, load_w4a4_linear
+from .flux_fp8 import ada_fp8_layernorm, load_ada_fp8_layernorm
+from .weights import FP8Linear, W4A4Linear, _source, load_fp8_linear, load_w4a4_linear
 
 
 @dataclass
@@ -87,3 +89,99 @@ def flux_single_mlp_int4(x: torch.Tensor, norm_hidden: torch.Tensor, attn_output
     h1 = _w4a4(w.proj_out_1, attn_output.view(m, d))
     out = _w4a4(w.proj_out_2, mlp, addend=h1, gate=gate, residual=x.view(m, d), rows_per_gate=s)
     return out.view(b, s, d)
+
+
+# ---- whole INT4 blocks around a caller-supplied attention core ------------------------------------------------------
+@dataclass
+class AdaLinear16:
+    """The 16-bit adaLN linear of quant level INT4_W4A4 (AdaLayerNormWeight, keys prefix + "linear.weight" / ".bias"); level
+    INT4_W4A4_FULL holds an FP8Linear in its place (AdaFP8LayerNormWeight)."""
+    weight: torch.Tensor  # T [n_chunks*D, D]
+    bias: torch.Tensor    # T [n_chunks*D]
+
+
+def _load_ada(src, prefix: str, dim: int, n_chunks: int, full: bool, dtype, device) -> Union[FP8Linear, AdaLinear16]:
+    if full:
+        return load_ada_fp8_layernorm(src, prefix, dim, n_chunks, dtype, device)
+    get = _source(src)
+    return AdaLinear16(get(prefix + "linear.weight", (n_chunks * dim, dim), dtype).to(device),
+                       get(prefix + "linear.bias", (n_chunks * dim,), dtype).to(device))
+
+
+def ada_layernorm_int4(x: torch.Tensor, temb: torch.Tensor, linear: Union[FP8Linear, AdaLinear16], n_chunks: int,
+                       eps: float = 1e-6):
+    """AdaLayerNorm / AdaFP8LayerNorm in front of the W4A4 linears: returns (norm_hidden 16-bit [B, S, D], msa [n_chunks, B, D]).
+    The 16-bit adaLN linear of level INT4_W4A4 is not a quantized linear and runs as a plain PyTorch matmul."""
+    if isinstance(linear, FP8Linear):
+        return ada_fp8_layernorm(x, temb, linear, n_chunks, (), eps=eps)
+    b, s, d = x.shape
+    flat = torch.nn.functional.linear(temb.reshape(b, d), linear.weight, linear.bias)
+    msa = flat.view(b, n_chunks, d).transpose(0, 1).contiguous()
+    return ops.gate_residual_layernorm_mod(x, msa[1], msa[0], eps=eps), msa
+
+
+@dataclass
+class FluxSingleBlockInt4Weights:
+    norm: Union[FP8Linear, AdaLinear16]  # prefix + "norm.linear"
+    to_qkv: W4A4Linear                   # prefix + "attn.to_qkv."  [3D, D], bias
+    mlp: FluxSingleMlpInt4Weights
+
+
+@dataclass
+class FluxDoubleBlockInt4Weights:
+    norm1: Union[FP8Linear, AdaLinear16]          # prefix + "norm1.linear"
+    norm1_context: Union[FP8Linear, AdaLinear16]  # prefix + "norm1_context.linear"
+    to_qkv: W4A4Linear        # prefix + "attn.to_qkv."
+    to_added_qkv: W4A4Linear  # prefix + "attn.to_added_qkv."
+    to_out: W4A4Linear        # prefix + "attn.to_out.0."
+    to_add_out: W4A4Linear    # prefix + "attn.to_add_out."
+    ff: FluxAttnPostInt4Weights          # prefix + "ff."
+    ff_context: FluxAttnPostInt4Weights  # prefix + "ff_context."
+
+
+def load_flux_single_block_int4(src, prefix: str, dim: int, mlp_scale: int = 4, full: bool = True, dtype=torch.bfloat16,
+                                device="cuda", lora_rank: int = 32) -> FluxSingleBlockInt4Weights:
+    """FluxSingleTransformerInt4BlockWeight (FluxSingleTransformerInt4BlockWeight.cc:24-37,79-83) and
+    FluxSingleAttentionInt4ProcessorWeight::loadWeights (:66-78).  full: quant level INT4_W4A4_FULL (FP8 adaLN linear)."""
+    return FluxSingleBlockInt4Weights(_load_ada(src, prefix + "norm.", dim, 3, full, dtype, device),
+                                      load_w4a4_linear(src, prefix + "attn.to_qkv.", 3 * dim, dim, lora_rank, True, dtype, device),
+                                      load_flux_single_mlp_int4(src, prefix, dim, mlp_scale, dtype, device, lora_rank))
+
+
+def load_flux_double_block_int4(src, prefix: str, dim: int, full: bool = True, dtype=torch.bfloat16, device="cuda",
+                                lora_rank: int = 32) -> FluxDoubleBlockInt4Weights:
+    """FluxTransformerInt4BlockWeight (FluxTransformerInt4BlockWeight.cc:27-39,86-90) and
+    FluxAttentionInt4ProcessorWeight (FluxAttentionInt4ProcessorWeight.cc:22-25,63-66)."""
+    lin = lambda name, n: load_w4a4_linear(src, prefix + "attn." + name + ".", n, dim, lora_rank, True, dtype, device)
+    return FluxDoubleBlockInt4Weights(_load_ada(src, prefix + "norm1.", dim, 6, full, dtype, device),
+                                      _load_ada(src, prefix + "norm1_context.", dim, 6, full, dtype, device),
+                                      lin("to_qkv", 3 * dim), lin("to_added_qkv", 3 * dim), lin("to_out.0", dim),
+                                      lin("to_add_out", dim),
+                                      load_flux_attn_post_int4(src, prefix + "ff.", dim, dtype, device, lora_rank),
+                                      load_flux_attn_post_int4(src, prefix + "ff_context.", dim, dtype, device, lora_rank))
+
+
+def _w4a4_3d(lin: W4A4Linear, x: torch.Tensor) -> torch.Tensor:
+    y = _w4a4(lin, x.reshape(-1, x.shape[-1]))
+    return y.view(*x.shape[:-1], y.shape[-1])
+
+
+def flux_single_block_int4(x: torch.Tensor, temb: torch.Tensor, w: FluxSingleBlockInt4Weights, attention) -> torch.Tensor:
+    """FluxSingleTransformerInt4Block<T>::forward (FluxSingleTransformerInt4Block.cc:178-316): adaLN, W4A4 QKV projection
+    (its bias added in the GEMM epilogue; the reference adds it in a pass of its own), attention(qkv [B, S, 3D]) -> [B, S, D],
+    then the feed-forward tail."""
+    norm, msa = ada_layernorm_int4(x, temb, w.norm, 3)
+    attn_out = attention(_w4a4_3d(w.to_qkv, norm))
+    return flux_single_mlp_int4(x, norm, attn_out.contiguous(), msa[2].contiguous(), w.mlp)
+
+
+def flux_double_block_int4(x: torch.Tensor, context: torch.Tensor, temb: torch.Tensor, w: FluxDoubleBlockInt4Weights, attention):
+    """FluxTransformerInt4Block<T>::forward (FluxTransformerInt4Block.cc:159-246) with FluxAttentionInt4Processor
+    (FluxAttentionInt4Processor.cc:206-331).  attention(qkv, context_qkv) -> (attn [B, S, D], context_attn [B, Sc, D]).
+    Returns (output, context_output)."""
+    n, msa = ada_layernorm_int4(x, temb, w.norm1, 6)
+    nc, cmsa = ada_layernorm_int4(context, temb, w.norm1_context, 6)
+    attn, cattn = attention(_w4a4_3d(w.to_qkv, n), _w4a4_3d(w.to_added_qkv, nc))
+    a_out = _w4a4_3d(w.to_out, attn.contiguous())
+    c_out = _w4a4_3d(w.to_add_out, cattn.contiguous())
+    return flux_attn_post_int4(x, a_out, msa, w.ff), flux_attn_post_int4(context, c_out, cmsa, w.ff_context)

@@ -10,7 +10,8 @@ quantisation runs on this library's HIP kernels (flux_fp8.py); the attention cor
 output projection -- per-head RMSNorm of q and k, rotary embedding, softmax attention -- is not part of the
 quantized-linear path and is plain PyTorch here (`flux_attention_core`).
 
-Supported quant levels: FP8_W8A8 and FP8_W8A8_FULL.  Any other level raises at construction.
+Supported quant levels: FP8_W8A8, FP8_W8A8_FULL, INT4_W4A4 and INT4_W4A4_FULL (W4A4 linears with their low-rank branch,
+th_op/flux_transformer_block/FluxTransformerBlockOp.h:165-182).  Any other level raises at construction.
 """
 from __future__ import annotations
 
@@ -20,6 +21,7 @@ from typing import Mapping, Optional, Sequence
 import torch
 
 from . import flux_fp8 as F
+from . import flux_int4 as I4
 
 
 class LyraQuantLevel(Enum):
@@ -100,8 +102,10 @@ class _BlockOpBase:
         if inference_dtype not in _DTYPES:
             raise ValueError("wrong inference_dtype")  # the reference throws on anything but fp32 / fp16 / bf16
         level = LyraQuantLevel(int(quant_level))
-        if level not in (LyraQuantLevel.FP8_W8A8, LyraQuantLevel.FP8_W8A8_FULL):
-            raise NotImplementedError(f"quant level {level.name}: only the FP8 blocks are built on this library")
+        if level not in (LyraQuantLevel.FP8_W8A8, LyraQuantLevel.FP8_W8A8_FULL, LyraQuantLevel.INT4_W4A4,
+                         LyraQuantLevel.INT4_W4A4_FULL):
+            raise NotImplementedError(f"quant level {level.name}: only the FP8 and INT4 blocks are built on this library")
+        self.int4 = level in (LyraQuantLevel.INT4_W4A4, LyraQuantLevel.INT4_W4A4_FULL)
         if embedding_dim != embedding_head_num * embedding_head_dim:
             raise ValueError("embedding_dim must equal embedding_head_num * embedding_head_dim")
         self.inference_dtype = inference_dtype
@@ -137,14 +141,18 @@ class _BlockOpBase:
         ["ff", "net.0.proj"], ["norm1", "linear"], ["proj_mlp"], ...  An unknown name raises (the reference prints a
         message and goes on)."""
         key = ".".join(lora_name)
+        if self.int4:  # the reference's INT4 block weights register no LoRA targets (FluxTransformerInt4BlockWeight.cc:41-45)
+            raise KeyError(f"no LoRA target named {key}: the INT4 blocks carry their low-rank branch in the checkpoint")
         lin = self._fp8_linears().get(key)
         if lin is None:
             raise KeyError(f"no FP8 linear named {key} in this block")
         lin.load_lora(lora_weights.to(self.device), float(lora_strength))
 
     def clear_lora(self) -> None:
-        for lin in self._fp8_linears().values():
-            lin.clear_lora()
+        self._loaded()
+        if not self.int4:
+            for lin in self._fp8_linears().values():
+                lin.clear_lora()
 
 
 class FluxTransformerBlockOp(_BlockOpBase):
@@ -155,7 +163,11 @@ class FluxTransformerBlockOp(_BlockOpBase):
         read them (FluxAttentionFP8ProcessorWeight.cc:194-260): the linears' `.weight`, `.bias`, `_input_scale`, and
         `attn.norm_q.weight`, `attn.norm_k.weight`, `attn.norm_added_q.weight`, `attn.norm_added_k.weight`.  `device` names
         where the tensors of `weights` live, as in the reference; they end up on the GPU either way."""
-        self.weights = F.load_flux_double_block_fp8(weights, prefix, self.dim, self.dtype, self.device, keep_master=True)
+        if self.int4:
+            self.weights = I4.load_flux_double_block_int4(weights, prefix, self.dim, self.quant_level is LyraQuantLevel.INT4_W4A4_FULL,
+                                                          self.dtype, self.device)
+        else:
+            self.weights = F.load_flux_double_block_fp8(weights, prefix, self.dim, self.dtype, self.device, keep_master=True)
         self.norms = [_get(weights, prefix + f"attn.{n}.weight", (self.head_dim,), self.dtype).to(self.device)
                       for n in ("norm_q", "norm_k", "norm_added_q", "norm_added_k")]
 
@@ -175,7 +187,8 @@ class FluxTransformerBlockOp(_BlockOpBase):
             self._check(n, t)
         nq, nk, naq, nak = self.norms
         core = lambda qkv, cqkv: flux_attention_core(qkv, nq, nk, rope_emb, self.heads, cqkv, naq, nak)
-        out, ctx = F.flux_double_block_fp8(hidden_states, encoder_hidden_states, temb_emb, w, core)
+        block = I4.flux_double_block_int4 if self.int4 else F.flux_double_block_fp8
+        out, ctx = block(hidden_states, encoder_hidden_states, temb_emb, w, core)
         return [out, ctx]
 
 
@@ -183,8 +196,12 @@ class FluxSingleTransformerBlockOp(_BlockOpBase):
     """Single-stream FLUX block (FluxSingleTransformerFP8Block.cc:163-291)."""
 
     def reload_model_from_state_dict(self, prefix: str, weights: Mapping[str, torch.Tensor], device: str = "cpu") -> None:
-        self.weights = F.load_flux_single_block_fp8(weights, prefix, self.dim, self.mlp_scale, self.dtype, self.device,
-                                                    keep_master=True)
+        if self.int4:
+            self.weights = I4.load_flux_single_block_int4(weights, prefix, self.dim, self.mlp_scale,
+                                                          self.quant_level is LyraQuantLevel.INT4_W4A4_FULL, self.dtype, self.device)
+        else:
+            self.weights = F.load_flux_single_block_fp8(weights, prefix, self.dim, self.mlp_scale, self.dtype, self.device,
+                                                        keep_master=True)
         self.norms = [_get(weights, prefix + f"attn.{n}.weight", (self.head_dim,), self.dtype).to(self.device)
                       for n in ("norm_q", "norm_k")]
 
@@ -197,4 +214,5 @@ class FluxSingleTransformerBlockOp(_BlockOpBase):
         for n, t in (("hidden_states", hidden_states), ("rope_emb", rope_emb), ("temb_emb", temb_emb)):
             self._check(n, t)
         nq, nk = self.norms
-        return F.flux_single_block_fp8(hidden_states, temb_emb, w, lambda qkv: flux_attention_core(qkv, nq, nk, rope_emb, self.heads))
+        block = I4.flux_single_block_int4 if self.int4 else F.flux_single_block_fp8
+        return block(hidden_states, temb_emb, w, lambda qkv: flux_attention_core(qkv, nq, nk, rope_emb, self.heads))

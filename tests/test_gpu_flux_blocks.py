@@ -632,3 +632,75 @@ def test_flux_block_ops_have_the_reference_interface(ops, dev):
     snq, snk = (sd[f"single_transformer_blocks.5.attn.{n}.weight"].to(dev) for n in ("norm_q", "norm_k"))
     want = F.flux_single_block_fp8(xs, temb, ws, lambda a: FO.flux_attention_core(a, snq, snk, rope, heads))
     assert y.shape == xs.shape and torch.equal(y, want) and torch.isfinite(y.float()).all()
+
+
+@pytest.mark.parametrize("full", [True, False])
+def test_flux_int4_block_ops(ops, dev, full):
+    """Quant levels INT4_W4A4 (16-bit adaLN linear) and INT4_W4A4_FULL (FP8 adaLN linear) of the block classes: the op output
+    equals the block function driven with the same attention core, and the block function equals its steps one by one."""
+    from lyradiff_amd import flux_fp8 as F8
+    from lyradiff_amd import flux_int4 as F
+    from lyradiff_amd import flux_ops as FO
+
+    b, s, sc, heads, dh = 1, 128, 64, 4, 64
+    d = heads * dh
+    g = rng_t(401)
+    level = FO.LyraQuantLevel.INT4_W4A4_FULL if full else FO.LyraQuantLevel.INT4_W4A4
+    sd = {}
+    for pre, ada in (("transformer_blocks.0.", ("norm1.linear", "norm1_context.linear")), ("single_transformer_blocks.0.", ("norm.linear",))):
+        chunks = 6 if len(ada) == 2 else 3
+        sd.update(_state_dict({a: (chunks * d, d) for a in ada}, 402, prefix=pre))
+        for a in ada:
+            sd[f"{pre}{a}_input_scale"] = torch.tensor([4.0 / 448])
+        for n in ("norm_q", "norm_k", "norm_added_q", "norm_added_k"):
+            sd[f"{pre}attn.{n}.weight"] = (1 + 0.1 * torch.randn(dh, generator=g)).bfloat16()
+    for name, n in (("attn.to_qkv.", 3 * d), ("attn.to_added_qkv.", 3 * d), ("attn.to_out.0.", d), ("attn.to_add_out.", d)):
+        sd.update(_int4_state("transformer_blocks.0." + name, n, d, g))
+    for ff in ("ff.", "ff_context."):
+        sd.update(_int4_state(f"transformer_blocks.0.{ff}net.0.proj.", 4 * d, d, g))
+        sd.update(_state_dict({f"{ff}net.2": (d, 4 * d)}, 403, prefix="transformer_blocks.0."))
+        sd[f"transformer_blocks.0.{ff}net.2_input_scale"] = torch.tensor([3.0 / 448])
+    sd.update(_int4_state("single_transformer_blocks.0.attn.to_qkv.", 3 * d, d, g))
+    sd.update(_int4_state("single_transformer_blocks.0.proj_mlp.", 4 * d, d, g))
+    sd.update(_int4_state("single_transformer_blocks.0.proj_out.linears.0.", d, d, g))
+    sd.update(_int4_state("single_transformer_blocks.0.proj_out.linears.1.linear.", d, 4 * d, g, bias=False))
+    x = torch.randn(b, s, d, generator=g).bfloat16().to(dev)
+    ctx = torch.randn(b, sc, d, generator=g).bfloat16().to(dev)
+    temb = torch.randn(b, d, generator=g).bfloat16().to(dev)
+    rope = _rope_table(b, sc + s, dh, 404).bfloat16().to(dev)
+
+    op = FO.FluxTransformerBlockOp("bf16", d, heads, dh, 6, level.value)
+    op.initialize(None)
+    op.reload_model_from_state_dict("transformer_blocks.0.", sd, "cpu")
+    res = op.forward(x, ctx, rope, temb)
+    w = F.load_flux_double_block_int4(sd, "transformer_blocks.0.", d, full, torch.bfloat16, dev)
+    assert isinstance(w.norm1, F8.FP8Linear) == full
+    nq, nk, naq, nak = (sd[f"transformer_blocks.0.attn.{n}.weight"].to(dev) for n in ("norm_q", "norm_k", "norm_added_q", "norm_added_k"))
+    core = lambda a, c: FO.flux_attention_core(a, nq, nk, rope, heads, c, naq, nak)
+    o1, o2 = F.flux_double_block_int4(x, ctx, temb, w, core)
+    assert torch.equal(res[0], o1) and torch.equal(res[1], o2) and torch.isfinite(o1.float()).all() and torch.isfinite(o2.float()).all()
+    # the same steps one by one
+    n1, m1 = F.ada_layernorm_int4(x, temb, w.norm1, 6)
+    n2, m2 = F.ada_layernorm_int4(ctx, temb, w.norm1_context, 6)
+    if not full:  # the 16-bit adaLN linear is a plain matmul: msa = temb . W^T + b, chunk c of batch j at [c, j]
+        want = torch.nn.functional.linear(temb, w.norm1.weight, w.norm1.bias).view(b, 6, d).transpose(0, 1)
+        assert torch.equal(m1, want)
+    a1, a2 = core(w.to_qkv.forward(n1), w.to_added_qkv.forward(n2))
+    w1 = F.flux_attn_post_int4(x, w.to_out.forward(a1.contiguous()), m1, w.ff)
+    w2 = F.flux_attn_post_int4(ctx, w.to_add_out.forward(a2.contiguous()), m2, w.ff_context)
+    assert torch.equal(o1, w1) and torch.equal(o2, w2)
+    with pytest.raises(KeyError):
+        op.load_lora_by_name(["attn", "to_qkv"], torch.zeros(3 * d, d).bfloat16(), 1.0)
+    op.clear_lora()
+
+    sop = FO.FluxSingleTransformerBlockOp("bf16", d, heads, dh, 4, level.value)
+    sop.reload_model_from_state_dict("single_transformer_blocks.0.", sd, "cpu")
+    xs = torch.cat([ctx, x], dim=1).contiguous()
+    y = sop.forward(xs, rope, temb)
+    ws = F.load_flux_single_block_int4(sd, "single_transformer_blocks.0.", d, 4, full, torch.bfloat16, dev)
+    snq, snk = (sd[f"single_transformer_blocks.0.attn.{n}.weight"].to(dev) for n in ("norm_q", "norm_k"))
+    score = lambda a: FO.flux_attention_core(a, snq, snk, rope, heads)
+    assert torch.equal(y, F.flux_single_block_int4(xs, temb, ws, score)) and torch.isfinite(y.float()).all()
+    ns, ms = F.ada_layernorm_int4(xs, temb, ws.norm, 3)
+    want = F.flux_single_mlp_int4(xs, ns, score(ws.to_qkv.forward(ns)).contiguous(), ms[2].contiguous(), ws.mlp)
+    assert torch.equal(y, want)

@@ -124,13 +124,14 @@ def test_flux_block_op_constructor_checks():
 
     assert [l.value for l in FO.LyraQuantLevel] == list(range(9))
     op = FO.FluxSingleTransformerBlockOp("fp16", 256, 4, 64, 4, 2)
-    assert op.dtype == torch.float16 and op.quant_level is FO.LyraQuantLevel.FP8_W8A8_FULL
+    assert op.dtype == torch.float16 and op.quant_level is FO.LyraQuantLevel.FP8_W8A8_FULL and not op.int4
+    assert FO.FluxTransformerBlockOp("bf16", 256, 4, 64, 6, 8).int4
     with pytest.raises(RuntimeError, match="reload_model_from_state_dict"):
         op.clear_lora()
     with pytest.raises(ValueError):
         FO.FluxTransformerBlockOp("bf16", 256, 4, 60, 6, 1)  # dim != heads * head_dim
     with pytest.raises(NotImplementedError):
-        FO.FluxTransformerBlockOp("bf16", 256, 4, 64, 6, FO.LyraQuantLevel.INT4_W4A4.value)
+        FO.FluxTransformerBlockOp("bf16", 256, 4, 64, 6, FO.LyraQuantLevel.INT8_SMOOTH_QUANT_LEVEL1.value)
 
 
 @pytest.mark.gpu
