@@ -300,7 +300,37 @@ def extra_kernels(torch, ops, dev):
             us = timeit(lambda: ops.weight_only_linear(x, wp, sc, None, kind), iters=20, warm=3)
             res[f"gemm_weight_only_{kind}_{name}_{m}x{n}x{k}"] = {"us": round(us, 2), "TFLOP/s": round(2.0 * m * n * k / us / 1e6, 1)}
     res.update(flux_block_times(torch, ops, dev, timeit))
+    res.update(flux_linear_chain_1280(torch, ops, dev, timeit))
     return res
+
+
+def flux_linear_chain_1280(torch, ops, dev, timeit):
+    """BASELINE.json configs[4]: the FP8 linears of a FLUX double-stream block at 1280x1280 (M = 6912 tokens), each preceded
+    by the fused amax + cast of its bf16 input: QKV 3072->9216, out-proj 3072->3072, MLP 3072->12288 (GELU) ->3072.  The
+    four linears run on independent synthetic inputs of the right shapes (the attention between them is not part of the
+    path); the MLP pair is chained through the GEMM-epilogue scale as in the headline step."""
+    m, d = 6912, 3072
+    g = torch.Generator().manual_seed(1005)
+    lin = {}
+    for name, n, k in (("qkv", 3 * d, d), ("out", d, d), ("up", 4 * d, d), ("down", d, 4 * d)):
+        wq, sw = ops.fp8_quant((torch.randn(n, k, generator=g) * 0.02).bfloat16().to(dev))
+        lin[name] = (ops.repack_weight(wq), sw, (torch.randn(n, generator=g) * 0.02).bfloat16().to(dev))
+        ops.gemm_profile("fp8", m, n, k, dev)
+    xs = [torch.randn(m, d, generator=g).bfloat16().to(dev) for _ in range(3)]
+    sh = torch.zeros(1, dtype=torch.float32, device=dev)
+
+    def chain():
+        for name, x in (("qkv", xs[0]), ("out", xs[1])):
+            q, s = ops.fp8_quant(x)
+            ops.fp8_linear(q, lin[name][0], s, lin[name][1], lin[name][2])
+        q, s = ops.fp8_quant(xs[2])
+        sh.zero_()
+        h = ops.fp8_linear(q, lin["up"][0], s, lin["up"][1], lin["up"][2], True, None, 0.0, torch.bfloat16, out_scale=sh)
+        return ops.fp8_linear(ops.fp8_scale_cast(h, sh), lin["down"][0], sh, lin["down"][1], lin["down"][2])
+
+    us = timeit(chain, iters=20, warm=3)
+    flop = 2.0 * m * d * (3 * d + d + 4 * d + 4 * d)
+    return {"flux_double_block_fp8_linear_chain_6912": {"us": round(us, 2), "TFLOP/s": round(flop / us / 1e6, 1)}}
 
 
 def flux_block_times(torch, ops, dev, timeit):
