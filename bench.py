@@ -301,7 +301,38 @@ def extra_kernels(torch, ops, dev):
             res[f"gemm_weight_only_{kind}_{name}_{m}x{n}x{k}"] = {"us": round(us, 2), "TFLOP/s": round(2.0 * m * n * k / us / 1e6, 1)}
     res.update(flux_block_times(torch, ops, dev, timeit))
     res.update(flux_linear_chain_1280(torch, ops, dev, timeit))
+    res.update(sdxl_geglu_ffn_chain(torch, ops, dev, timeit))
     return res
+
+
+def sdxl_geglu_ffn_chain(torch, ops, dev, timeit):
+    """BASELINE.json configs[1]: the SDXL GEGLU feed-forward with INT8 W8A8 linears at 1024x1024 (M = 4096 tokens of the
+    64x64 latent stage): per-token quantisation, up GEMM 640 -> 5120, bias + GEGLU -> per-token INT8, down GEMM 2560 -> 640."""
+    m, d = 4096, 640
+    g = torch.Generator().manual_seed(1002)
+    x = torch.randn(m, d, generator=g).half()
+    x[:, torch.randperm(d, generator=g)[:6]] *= 15.0
+    x = x.to(dev)
+    w_up = ops.repack_weight(torch.randint(-127, 128, (8 * d, d), generator=g, dtype=torch.int8).to(dev))
+    w_dn = ops.repack_weight(torch.randint(-127, 128, (d, 4 * d), generator=g, dtype=torch.int8).to(dev))
+    s_up = (torch.rand(8 * d, generator=g) * 9e-3 + 1e-3).to(dev)
+    s_dn = (torch.rand(d, generator=g) * 9e-3 + 1e-3).to(dev)
+    b_up = (torch.randn(8 * d, generator=g) * 0.02).half().to(dev)
+    b_dn = (torch.randn(d, generator=g) * 0.02).half().to(dev)
+    pre1 = (torch.rand(d, generator=g) + 0.5).to(dev)
+    pre2 = (torch.rand(4 * d, generator=g) + 0.5).to(dev)
+    for (n, k) in ((8 * d, d), (d, 4 * d)):
+        ops.gemm_profile("int8", m, n, k, dev)
+
+    def chain():
+        q, s = ops.sq_quant_dynamic(x, pre1)
+        up = ops.int8_linear(q, w_up, s_up, s, None, torch.float16)
+        q2, s2 = ops.geglu_int8_dynamic(up, b_up, pre2)
+        return ops.int8_linear(q2, w_dn, s_dn, s2, b_dn, torch.float16)
+
+    us = timeit(chain, iters=30, warm=5)
+    ops_total = 2.0 * m * (8 * d * d + d * 4 * d)
+    return {"sdxl_geglu_ffn_int8_chain_4096": {"us": round(us, 2), "TOP/s": round(ops_total / us / 1e6, 1)}}
 
 
 def flux_linear_chain_1280(torch, ops, dev, timeit):
