@@ -359,16 +359,57 @@ __global__ __launch_bounds__(256) void int8_weight_quant_kernel(float* __restric
 }
 
 // ---- bias + GEGLU -> INT8 (ffn_kernels_int8.cu:102-147) ----------------------------------------------
+// The gate factor  gate(g) = T( g * T( 0.5 * (1 + tanh(0.79788 * (g + 0.044715 * T(g * T(g*g))))) ) )  depends only on the
+// 16-bit value g, and its evaluation (a tanh built from basic IEEE operations, so that a CPU restatement reproduces it bit
+// for bit) is about 70 of the kernel's 85 vector instructions per element.  For fp16 and bf16 inputs the factor is
+// therefore tabulated: a small kernel in front of every call evaluates the formula once for each 16-bit pattern with
+// 2^-12 <= |g| < 8 (30720 fp16 / 3840 bf16 patterns) into a table in device memory, every workgroup of the main kernel copies
+// the table into LDS and looks the factor up.  Outside that range the inner factor T(0.5 * (1 + tanh(...))) is a constant:
+// 0.5 for |g| < 2^-12 (the deviation from 0.5 is below half a unit in the last place of T), 1 for g >= 8 and 0 for g <= -8
+// (the tanh is +-1 in fp32 there), so gate(g) = T(g * c) with that constant -- the formula's own last step; infinities and
+// NaN follow the same expressions.  tests/test_oracle_pins.py checks these three constants against the formula for every
+// 16-bit pattern outside the table.  The table's contents never change; concurrent calls that rebuild it write the same bytes.
+template <typename Tag> __device__ __forceinline__ float geglu_gate(float g) {
+    const float cube = round_through<Tag>(g * round_through<Tag>(g * g));
+    const float cdf = 0.5f * (1.0f + tanh_basic(0.7978845608028654f * (g + 0.044715f * cube)));
+    return round_through<Tag>(g * round_through<Tag>(cdf));
+}
+template <typename Tag> struct GateTable;
+template <> struct GateTable<F16Tag> { static constexpr u32 LO = 0x0C00u, COUNT = 0x4800u - 0x0C00u; };   // 2^-12 .. 8
+template <> struct GateTable<BF16Tag> { static constexpr u32 LO = 0x3980u, COUNT = 0x4100u - 0x3980u; };
+__device__ __attribute__((aligned(16))) unsigned short g_gate_table_f16[2 * GateTable<F16Tag>::COUNT];
+__device__ __attribute__((aligned(16))) unsigned short g_gate_table_bf16[2 * GateTable<BF16Tag>::COUNT];
+template <typename Tag> __device__ __forceinline__ unsigned short* gate_table() {
+    if constexpr (std::is_same<Tag, F16Tag>::value) return g_gate_table_f16;
+    else return g_gate_table_bf16;
+}
+template <typename Tag> __global__ __launch_bounds__(256) void geglu_table_kernel() {
+    constexpr u32 COUNT = GateTable<Tag>::COUNT;
+    const u32 i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= 2 * COUNT) return;
+    const u32 bits = (GateTable<Tag>::LO + (i % COUNT)) | (i >= COUNT ? 0x8000u : 0u);
+    gate_table<Tag>()[i] = (unsigned short)Elem<Tag>::store(geglu_gate<Tag>(Elem<Tag>::load(bits)));
+}
+
 // One wavefront per row; the row of `dim` products h*g stays in registers (NP passes of 512).
-template <typename Tag, int NP, bool DYNAMIC>
-__global__ __launch_bounds__(256) void geglu_int8_kernel(int8_t* __restrict__ dst, float* __restrict__ scale_out,
+template <typename Tag, int NP, bool DYNAMIC, int THREADS>
+__global__ __launch_bounds__(THREADS) void geglu_int8_kernel(int8_t* __restrict__ dst, float* __restrict__ scale_out,
                                                          const void* __restrict__ hidden,
                                                          const void* __restrict__ bias,
                                                          const float* __restrict__ pre,
                                                          const float* __restrict__ in_scale, size_t rows, int dim) {
+    constexpr bool TABLE = Elem<Tag>::bytes == 2;
+    extern __shared__ __attribute__((aligned(16))) unsigned short s_gate[];
+    if constexpr (TABLE) {
+        const unsigned short* tab = gate_table<Tag>();
+        for (u32 i = threadIdx.x * 8; i < 2 * GateTable<Tag>::COUNT; i += blockDim.x * 8)
+            *reinterpret_cast<uint4*>(s_gate + i) = *reinterpret_cast<const uint4*>(tab + i);
+        __syncthreads();
+    }
     const int lane = threadIdx.x & 63;
-    const size_t wave = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const size_t nwaves = (size_t)gridDim.x * 4;
+    const size_t wpb = blockDim.x >> 6;  // wavefronts (= rows in flight) per workgroup
+    const size_t wave = (size_t)blockIdx.x * wpb + (threadIdx.x >> 6);
+    const size_t nwaves = (size_t)gridDim.x * wpb;
     for (size_t row = wave; row < rows; row += nwaves) {
         const char* rb = static_cast<const char*>(hidden) + row * (size_t)dim * 2 * Elem<Tag>::bytes;
         float t[NP][8];
@@ -377,7 +418,7 @@ __global__ __launch_bounds__(256) void geglu_int8_kernel(int8_t* __restrict__ ds
         for (int p = 0; p < NP; ++p) {
             int col = (p * 64 + lane) * 8;
             if (col < dim) {
-                float h[8], g[8], pv[8];
+                float h[8], g[8], pv[8], gel[8];
                 load8<Tag>(rb, col, h);
                 load8<Tag>(rb, col + dim, g);
                 if (bias != nullptr) {
@@ -393,12 +434,26 @@ __global__ __launch_bounds__(256) void geglu_int8_kernel(int8_t* __restrict__ ds
 #pragma unroll
                 for (int i = 0; i < 8; ++i) pv[i] = 1.0f;
                 if (pre != nullptr) load8<F32Tag>(pre, col, pv);
+                if constexpr (TABLE) {
+                    constexpr u32 LO = GateTable<Tag>::LO, COUNT = GateTable<Tag>::COUNT;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const u32 bits = Elem<Tag>::store(g[i]);  // exact: g is a T value
+                        const u32 off = (bits & 0x7FFFu) - LO;    // wraps to a huge number below the table
+                        const bool in = off < COUNT, neg = (bits & 0x8000u) != 0;
+                        const float looked_up = Elem<Tag>::load(s_gate[(in ? off : 0u) + (neg ? COUNT : 0u)]);
+                        // outside the table the inner factor is a constant (a branch for this rare case measured slower)
+                        const float c = (bits & 0x7FFFu) < LO ? 0.5f : (neg ? 0.0f : 1.0f);
+                        const float outside = round_through<Tag>(g[i] * c);
+                        gel[i] = in ? looked_up : outside;
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) gel[i] = geglu_gate<Tag>(g[i]);
+                }
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    float cube = round_through<Tag>(g[i] * round_through<Tag>(g[i] * g[i]));
-                    float cdf = 0.5f * (1.0f + tanh_basic(0.7978845608028654f * (g[i] + 0.044715f * cube)));
-                    float gel = round_through<Tag>(g[i] * round_through<Tag>(cdf));
-                    float prod = round_through<Tag>(h[i] * gel);
+                    float prod = round_through<Tag>(h[i] * gel[i]);
                     t[p][i] = prod * pv[i];
                     amax = fmaxf(amax, fabsf(t[p][i]));
                 }
@@ -442,11 +497,34 @@ static int launch_geglu(int8_t* dst, float* scale_out, const void* hidden, const
                    (pre == nullptr || reinterpret_cast<uintptr_t>(pre) % 16 == 0),
                LQ_ERR_ARG, "geglu_int8: pointers must be 16-byte aligned");
     const int np = (int)((dim + 511) / 512);
-    size_t blocks = (rows + 3) / 4;
-    dim3 grid((unsigned)(blocks < 65535 ? blocks : 65535)), block(256);
+    size_t lds = 0, threads = 256, cap = 65535;
+    if constexpr (Elem<Tag>::bytes == 2) {
+        // the gate table, rebuilt in front of every call (no state to initialise, nothing for a captured graph to miss);
+        // every workgroup stages it once, so the grid is a few workgroups per CU that walk the rows.  The fp16 table
+        // (60 KB) allows two workgroups per CU: those have eight wavefronts each.
+        constexpr unsigned entries = 2 * GateTable<Tag>::COUNT;
+        hipLaunchKernelGGL((geglu_table_kernel<Tag>), dim3((entries + 255) / 256), dim3(256), 0, st);
+        lds = entries * sizeof(unsigned short);
+        threads = (lds > 32768 && np <= 10) ? 512 : 256;  // (the 16-pass form needs all 256 registers of a 256-thread workgroup)
+        cap = 256 * (lds > 32768 ? 2 : 8);
+    }
+    size_t blocks = (rows + threads / 64 - 1) / (threads / 64);
+    if (blocks > cap) blocks = cap;
+    dim3 grid((unsigned)blocks), block((unsigned)threads);
     int d = (int)dim;
-#define LQ_GG_CASE(NPV) \
-    hipLaunchKernelGGL((geglu_int8_kernel<Tag, NPV, DYNAMIC>), grid, block, 0, st, dst, scale_out, hidden, bias, pre, in_scale, rows, d)
+#define LQ_GG_CASE(NPV)                                                                                                  \
+    do {                                                                                                                 \
+        auto kern = threads == 512 ? geglu_int8_kernel<Tag, NPV, DYNAMIC, (NPV <= 10 ? 512 : 256)>                       \
+                                   : geglu_int8_kernel<Tag, NPV, DYNAMIC, 256>;                                          \
+        if (lds > 48 * 1024) {                                                                                           \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+            if (e != hipSuccess) {                                                                                       \
+                set_error("geglu_int8: cannot raise the LDS limit to %zu bytes: %s", lds, hipGetErrorString(e));         \
+                return LQ_ERR_HIP;                                                                                       \
+            }                                                                                                            \
+        }                                                                                                                \
+        hipLaunchKernelGGL(kern, grid, block, lds, st, dst, scale_out, hidden, bias, pre, in_scale, rows, d);            \
+    } while (0)
     if (np <= 2) LQ_GG_CASE(2);
     else if (np <= 3) LQ_GG_CASE(3);
     else if (np <= 5) LQ_GG_CASE(5);

@@ -107,6 +107,33 @@ def test_geglu_int8(ops, dev, dt, with_bias):
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+def test_geglu_int8_gate_values_outside_the_table(ops, dev, dt):
+    """Gate inputs below 2^-12, at the table's two ends, beyond 8, subnormal, infinite and NaN (the HIP kernel looks the gate
+    factor up for 2^-12 <= |g| < 8 and uses its constant forms elsewhere), with and without a bias."""
+    m, d = 64, 1024
+    g = rng_t(23)
+    x = (torch.randn(m, 2 * d, generator=g) * 1.5)
+    gate = x[:, d:]
+    gate[:, 0::7] *= 1e-4
+    gate[:, 1::11] *= 20.0
+    gate[0, :12] = torch.tensor([2.0 ** -12, -2.0 ** -12, 8.0, -8.0, 7.99, -7.99, 2.4e-4, -2.4e-4, 6e-8, -6e-8, 0.0, -0.0])
+    gate[1, :4] = torch.tensor([float("inf"), float("-inf"), float("nan"), 65504.0])
+    x = x.to(TORCH_DT[dt])
+    xn = to_np_f32(x)
+    pre = (torch.rand(d, generator=g) + 0.5).float()
+    for bias in (None, (torch.randn(2 * d, generator=g) * 1e-3).to(TORCH_DT[dt])):
+        bn = None if bias is None else to_np_f32(bias)
+        bd = None if bias is None else bias.to(dev)
+        sc = torch.tensor([0.05], dtype=torch.float32)
+        with np.errstate(all="ignore"):
+            q_ref = O.geglu_int8(xn, bn, pre.numpy(), sc.numpy(), dt)
+            qd_ref, sd_ref = O.geglu_int8_dynamic(xn, bn, pre.numpy(), dt)
+        assert np.array_equal(ops.geglu_int8(x.to(dev), bd, pre.to(dev), sc.to(dev)).cpu().numpy(), q_ref)
+        qd, sd = ops.geglu_int8_dynamic(x.to(dev), bd, pre.to(dev))
+        assert np.array_equal(sd.cpu().numpy(), sd_ref, equal_nan=True) and np.array_equal(qd.cpu().numpy(), qd_ref)
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("n", [4608 * 3072, 1000003, 17, 4096])
 def test_fp8_amax_cast(ops, dev, dt, n):
     x = (torch.randn(n, generator=rng_t(n % 1000)) * 3).to(TORCH_DT[dt])

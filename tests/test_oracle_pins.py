@@ -451,3 +451,27 @@ def test_weight_only_quantize_and_layout_oracle():
         for j in range(5):
             ref = sum(float(a[i, t]) * int(qq[t, j]) for t in range(8)) * float(sc[j]) + float(b[j])
             assert abs(float(y[i, j]) - ref) <= 1e-6 * max(1.0, abs(ref))
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+def test_geglu_gate_is_constant_times_g_outside_the_tabulated_range(dt):
+    """The HIP GEGLU kernel tabulates gate(g) = T(g * T(0.5 * (1 + tanh(...)))) for 2^-12 <= |g| < 8 and uses T(g * c) outside,
+    c = 0.5 below the range, 1 for g >= 8, 0 for g <= -8.  Every 16-bit pattern outside the range is checked against the
+    formula (infinities and NaN included)."""
+    bits = np.arange(65536, dtype=np.uint32)
+    if dt == "f16":
+        g = bits.astype(np.uint16).view(np.float16).astype(np.float32)
+    else:
+        g = (bits << 16).view(np.float32)
+    a = np.abs(g)
+    outside = ~((a >= 2.0 ** -12) & (a < 8.0))  # NaN compares false both ways: outside
+    go = g[outside]
+    with np.errstate(all="ignore"):
+        x = np.stack([np.ones_like(go), go], axis=1)  # h = 1: T(1 * gate) = gate
+        want = O.geglu_product(x, None, dt)[:, 0]
+        c = np.where(np.abs(go) < 2.0 ** -12, np.float32(0.5), np.where(np.signbit(go), np.float32(0.0), np.float32(1.0)))
+        got = O.round_to((go * c).astype(np.float32), dt)
+    assert outside.sum() > 20000
+    same = (want == got) | (np.isnan(want) & np.isnan(got))
+    assert same.all(), f"{(~same).sum()} patterns differ, first g = {go[~same][:4]}"
+    assert np.array_equal(np.signbit(want[~np.isnan(want)]), np.signbit(got[~np.isnan(got)]))
