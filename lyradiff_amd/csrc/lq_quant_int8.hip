@@ -436,16 +436,21 @@ __global__ __launch_bounds__(THREADS) void geglu_int8_kernel(int8_t* __restrict_
                 if (pre != nullptr) load8<F32Tag>(pre, col, pv);
                 if constexpr (TABLE) {
                     constexpr u32 LO = GateTable<Tag>::LO, COUNT = GateTable<Tag>::COUNT;
+                    bool in[8], all_in = true;
 #pragma unroll
                     for (int i = 0; i < 8; ++i) {
                         const u32 bits = Elem<Tag>::store(g[i]);  // exact: g is a T value
                         const u32 off = (bits & 0x7FFFu) - LO;    // wraps to a huge number below the table
-                        const bool in = off < COUNT, neg = (bits & 0x8000u) != 0;
-                        const float looked_up = Elem<Tag>::load(s_gate[(in ? off : 0u) + (neg ? COUNT : 0u)]);
-                        // outside the table the inner factor is a constant (a branch for this rare case measured slower)
-                        const float c = (bits & 0x7FFFu) < LO ? 0.5f : (neg ? 0.0f : 1.0f);
-                        const float outside = round_through<Tag>(g[i] * c);
-                        gel[i] = in ? looked_up : outside;
+                        in[i] = off < COUNT;
+                        all_in = all_in && in[i];
+                        gel[i] = Elem<Tag>::load(s_gate[(in[i] ? off : 0u) + ((bits & 0x8000u) ? COUNT : 0u)]);
+                    }
+                    if (__builtin_expect(!all_in, 0)) {  // rare: outside the table the inner factor is a constant
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) {
+                            const float c = fabsf(g[i]) < 1.0f ? 0.5f : (g[i] < 0.0f ? 0.0f : 1.0f);  // below the table : beyond it
+                            if (!in[i]) gel[i] = round_through<Tag>(g[i] * c);
+                        }
                     }
                 } else {
 #pragma unroll
