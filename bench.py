@@ -302,6 +302,51 @@ def extra_kernels(torch, ops, dev):
     res.update(flux_block_times(torch, ops, dev, timeit))
     res.update(flux_linear_chain_1280(torch, ops, dev, timeit))
     res.update(sdxl_geglu_ffn_chain(torch, ops, dev, timeit))
+    res.update(flux_whole_blocks(torch, dev, timeit))
+    return res
+
+
+def flux_whole_blocks(torch, dev, timeit):
+    """Whole FLUX blocks at 1024x1024 (4096 image + 512 text tokens, d = 3072, 24 heads) through the block classes with the
+    reference's interface, FP8 level: every linear, adaLN, gate and residual on this library's kernels, the attention core
+    (q/k RMSNorm, rotary embedding, softmax attention) in PyTorch.  Random weights; informative only."""
+    from lyradiff_amd import flux_ops as FO
+
+    d, heads, dh, s, sc = 3072, 24, 128, 4096, 512
+    g = torch.Generator().manual_seed(88)
+
+    def state(prefix, names, norms):
+        sd = {}
+        for name, (n, k) in names.items():
+            sd[f"{prefix}{name}.weight"] = (torch.randn(n, k, generator=g) * 0.02).bfloat16()
+            sd[f"{prefix}{name}.bias"] = (torch.randn(n, generator=g) * 0.02).bfloat16()
+            sd[f"{prefix}{name}_input_scale"] = torch.tensor([6.0 / 448])
+        for n in norms:
+            sd[f"{prefix}attn.{n}.weight"] = torch.ones(dh).bfloat16()
+        return sd
+
+    dbl = {"norm1.linear": (6 * d, d), "norm1_context.linear": (6 * d, d), "attn.to_qkv": (3 * d, d), "attn.to_added_qkv": (3 * d, d),
+           "attn.to_out.0": (d, d), "attn.to_add_out": (d, d), "ff.net.0.proj": (4 * d, d), "ff.net.2": (d, 4 * d),
+           "ff_context.net.0.proj": (4 * d, d), "ff_context.net.2": (d, 4 * d)}
+    sgl = {"norm.linear": (3 * d, d), "attn.to_qkv": (3 * d, d), "proj_mlp": (4 * d, d), "proj_out": (d, 5 * d)}
+    x = torch.randn(1, s, d, generator=g).bfloat16().to(dev)
+    ctx = torch.randn(1, sc, d, generator=g).bfloat16().to(dev)
+    temb = torch.randn(1, d, generator=g).bfloat16().to(dev)
+    ang = torch.rand(1, sc + s, dh // 2, generator=g) * 6.28
+    rope = torch.stack([ang.cos(), -ang.sin(), ang.sin(), ang.cos()], dim=-1).reshape(1, sc + s, dh // 2, 2, 2).bfloat16().to(dev)
+    res = {}
+    op = FO.FluxTransformerBlockOp("bf16", d, heads, dh, 6, FO.LyraQuantLevel.FP8_W8A8.value)
+    op.reload_model_from_state_dict("b.", state("b.", dbl, ("norm_q", "norm_k", "norm_added_q", "norm_added_k")), "cpu")
+    us = timeit(lambda: op.forward(x, ctx, rope, temb), iters=10, warm=3)
+    lin = 2.0 * d * d * ((s + sc) * (3 + 1 + 8))
+    res["flux_double_block_fp8_whole_1024"] = {"us": round(us, 1), "linear_TFLOP/s": round(lin / us / 1e6, 1)}
+    del op
+    sop = FO.FluxSingleTransformerBlockOp("bf16", d, heads, dh, 4, FO.LyraQuantLevel.FP8_W8A8.value)
+    sop.reload_model_from_state_dict("b.", state("b.", sgl, ("norm_q", "norm_k")), "cpu")
+    xs = torch.cat([ctx, x], dim=1).contiguous()
+    us = timeit(lambda: sop.forward(xs, rope, temb), iters=10, warm=3)
+    lin = 2.0 * d * d * (s + sc) * (3 + 4 + 5)
+    res["flux_single_block_fp8_whole_1024"] = {"us": round(us, 1), "linear_TFLOP/s": round(lin / us / 1e6, 1)}
     return res
 
 
