@@ -521,12 +521,14 @@ static int launch_geglu(int8_t* dst, float* scale_out, const void* hidden, const
     do {                                                                                                                 \
         auto kern = threads == 512 ? geglu_int8_kernel<Tag, NPV, DYNAMIC, (NPV <= 10 ? 512 : 256)>                       \
                                    : geglu_int8_kernel<Tag, NPV, DYNAMIC, 256>;                                          \
-        if (lds > 48 * 1024) {                                                                                           \
+        static bool raised = false; /* raising the dynamic LDS limit is idempotent; a race only repeats it */           \
+        if (lds > 48 * 1024 && !raised) {                                                                                \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
             if (e != hipSuccess) {                                                                                       \
                 set_error("geglu_int8: cannot raise the LDS limit to %zu bytes: %s", lds, hipGetErrorString(e));         \
                 return LQ_ERR_HIP;                                                                                       \
             }                                                                                                            \
+            raised = true;                                                                                               \
         }                                                                                                                \
         hipLaunchKernelGGL(kern, grid, block, lds, st, dst, scale_out, hidden, bias, pre, in_scale, rows, d);            \
     } while (0)
