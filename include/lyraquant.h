@@ -358,6 +358,21 @@ int lq_lora_down(void* out, lq_dtype_t out_dtype, const void* x, const void* lor
  * (invokeCudaD2DcpyConvert<T, float>, utils/memory_utils.cu:398-402). */
 int lq_cast_f32(void* dst, lq_dtype_t dst_dtype, const float* src, size_t n, lq_stream_t stream);
 
+/* Between the QKV projections and the attention of a FLUX block: per-head RMSNorm of q and k, rotary embedding, and the
+ * concatenation [text tokens, image tokens] -- invokeFusedRmsNormCatAndRope and (context_seq = 0) invokeFusedRmsNormAndRope
+ * (kernels/rope/flux_apply_rope.h; kernels/rope/flux_apply_rope.cu:74-156,291-319; call sites
+ * layers/flux_attention_processor/FluxAttentionFP8Processor.cc:232-245,
+ * layers/flux_single_attention_processor/FluxSingleAttentionFP8Processor.cc:183-193).
+ *   qkv [batch, seq, 3, heads, head_dim], context_qkv [batch, context_seq, 3, heads, head_dim] (or NULL with context_seq 0),
+ *   out [batch, context_seq + seq, 3, heads, head_dim]: the flash-attention input of the reference (its nhidden_buffer),
+ *   norm_qk / norm_added_qk [2 * head_dim]: the q weights then the k weights (qk_norm_weight, encoder_qk_norm_weight),
+ *   rope [.., context_seq + seq, head_dim / 2, 2, 2] with rope_batch_stride elements between batches (0: one table for all).
+ * q and k:  n = T(x * (1 / sqrt(mean(x^2) + eps))) * w  in T, then every pair (n0, n1) -> (T(T(n0*r00) + T(n1*r01)),
+ * T(T(n0*r10) + T(n1*r11)));  v is copied.  dtype F16 or BF16 for every tensor; head_dim 64 or 128. */
+int lq_rmsnorm_rope(void* out, const void* qkv, const void* context_qkv, const void* norm_qk, const void* norm_added_qk,
+                    const void* rope, size_t rope_batch_stride, lq_dtype_t dtype, int batch, int seq, int context_seq,
+                    int heads, int head_dim, float eps, lq_stream_t stream);
+
 /* dst[i] = T( dst[i] + T( src[i] * T(alpha) ) ): merges a full-rank LoRA delta into a 16-bit (or fp32) weight
  * (invokeLoadLora, kernels/lora/load_lora.h + load_lora.cu:6-14,92-96).  An FP8 weight is re-quantised after the
  * merge the way FP8LoraWeight::load_lora / clear_lora do (interface/IFLoraWeight.h:79-128): restore the 16-bit

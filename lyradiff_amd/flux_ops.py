@@ -6,9 +6,9 @@ load_lora_by_name, clear_lora: th_op/flux_transformer_block/FluxTransformerBlock
 th_op/flux_single_transformer_block/FluxSingleTransformerBlockOp.cc:6-98), so that the reference's Python wrappers
 (lyradiff/lyradiff_model/lyradiff_flux_transformer_model_v2.py:67-168) can hold one of these instead of a
 `torch.classes.lyradiff.*` object.  Every quantized linear, every adaLN / gate / residual step and every activation
-quantisation runs on this library's HIP kernels (flux_fp8.py); the attention core between the QKV projection and the
-output projection -- per-head RMSNorm of q and k, rotary embedding, softmax attention -- is not part of the
-quantized-linear path and is plain PyTorch here (`flux_attention_core`).
+quantisation runs on this library's HIP kernels (flux_fp8.py), as do the per-head RMSNorm of q and k and the rotary
+embedding behind the QKV projection (lq_rmsnorm_rope); the softmax attention itself is not part of the quantized-linear
+path and is PyTorch's (`flux_attention_core`).
 
 Supported quant levels: FP8_W8A8, FP8_W8A8_FULL, INT4_W4A4 and INT4_W4A4_FULL (W4A4 linears with their low-rank branch,
 th_op/flux_transformer_block/FluxTransformerBlockOp.h:165-182).  Any other level raises at construction.
@@ -22,6 +22,7 @@ import torch
 
 from . import flux_fp8 as F
 from . import flux_int4 as I4
+from . import ops
 
 
 class LyraQuantLevel(Enum):
@@ -40,48 +41,23 @@ class LyraQuantLevel(Enum):
 _DTYPES = {"fp16": torch.float16, "bf16": torch.bfloat16}
 
 
-def _rms_norm_rope(qkv: torch.Tensor, norm_q: torch.Tensor, norm_k: torch.Tensor, rope: torch.Tensor, heads: int,
-                   eps: float = 1e-6):
-    """qkv [B, S, 3*H*Dh] -> q, k, v [B, H, S, Dh] with q and k RMS-normalised per head and rotated.
-
-    Follows fuseRmsNormCatAndRope / fuseRmsNormAndRope (src/lyradiff/kernels/rope/flux_apply_rope.cu:74-156): mean of
-    squares and the scaling by its inverse root in fp32, the result rounded to T, multiplied by the norm weight in T,
-    then each pair (x, y) of adjacent elements becomes (x*r00 + y*r01, x*r10 + y*r11) with the 2x2 matrices of
-    `rope` [B or 1, S, Dh/2, 2, 2].  v passes through.
-    """
-    b, s, d3 = qkv.shape
-    dh = d3 // (3 * heads)
-    q, k, v = qkv.view(b, s, 3, heads, dh).unbind(2)
-    rope = rope.reshape(-1, s, 1, dh // 2, 2, 2).to(qkv.dtype)
-
-    def one(t, w):
-        f = t.float()
-        n = (f * torch.rsqrt(f.pow(2).mean(-1, keepdim=True) + eps)).to(t.dtype) * w.to(t.dtype)
-        p = n.view(b, s, heads, dh // 2, 1, 2)
-        return (p * rope).sum(-1).view(b, s, heads, dh)
-
-    return one(q, norm_q).transpose(1, 2), one(k, norm_k).transpose(1, 2), v.transpose(1, 2)
-
-
 def flux_attention_core(qkv: torch.Tensor, norm_q: torch.Tensor, norm_k: torch.Tensor, rope_emb: torch.Tensor, heads: int,
                         context_qkv: Optional[torch.Tensor] = None, norm_added_q: Optional[torch.Tensor] = None,
                         norm_added_k: Optional[torch.Tensor] = None):
     """The part of FluxAttentionFP8Processor::forward (FluxAttentionFP8Processor.cc:232-291) and
     FluxSingleAttentionFP8Processor::forward (FluxSingleAttentionFP8Processor.cc:183-213) between the QKV and the output
-    projections.  With `context_qkv` the text tokens come first in the joint sequence (`rope_emb` covers text + image) and
-    (image [B, S, D], text [B, Sc, D]) is returned; without it a single [B, S, D] tensor."""
+    projections: q/k RMSNorm per head, rotary embedding and the [text, image] concatenation in one HIP kernel
+    (ops.rmsnorm_rope = invokeFusedRmsNormCatAndRope), then softmax attention (PyTorch) on its [B, S, 3, H, Dh] output.
+    With `context_qkv` (image [B, S, D], text [B, Sc, D]) is returned; without it a single [B, S, D] tensor."""
     b, s, d3 = qkv.shape
     d = d3 // 3
-    if context_qkv is None:
-        q, k, v = _rms_norm_rope(qkv, norm_q, norm_k, rope_emb, heads)
-    else:
-        sc = context_qkv.shape[1]
-        rope_emb = rope_emb.reshape(-1, sc + s, d // heads // 2, 2, 2)
-        parts = [_rms_norm_rope(context_qkv, norm_added_q, norm_added_k, rope_emb[:, :sc], heads),
-                 _rms_norm_rope(qkv, norm_q, norm_k, rope_emb[:, sc:], heads)]
-        q, k, v = (torch.cat([parts[0][i], parts[1][i]], dim=2) for i in range(3))
+    sc = 0 if context_qkv is None else context_qkv.shape[1]
+    added = None if context_qkv is None else torch.cat([norm_added_q, norm_added_k])
+    cat = ops.rmsnorm_rope(qkv.contiguous(), torch.cat([norm_q, norm_k]), rope_emb.contiguous(), heads,
+                           None if context_qkv is None else context_qkv.contiguous(), added)
+    q, k, v = (cat[:, :, i].transpose(1, 2) for i in range(3))  # [B, H, Sc + S, Dh] views
     o = torch.nn.functional.scaled_dot_product_attention(q, k, v)
-    o = o.transpose(1, 2).reshape(b, -1, d)
+    o = o.transpose(1, 2).reshape(b, sc + s, d)
     if context_qkv is None:
         return o
     return o[:, sc:], o[:, :sc]

@@ -578,6 +578,35 @@ def lora_down(x, lora_down_w, out_dtype=None):
     return out
 
 
+def rmsnorm_rope(qkv, norm_qk, rope, heads: int, context_qkv=None, norm_added_qk=None, eps: float = 1e-6):
+    """invokeFusedRmsNormCatAndRope / invokeFusedRmsNormAndRope: qkv [B, S, 3*H*Dh] (context_qkv [B, Sc, 3*H*Dh], text tokens,
+    placed first) -> [B, Sc + S, 3, H, Dh] with q and k RMS-normalised per head, scaled by norm_qk / norm_added_qk ([2*Dh]: q
+    weights then k weights) and rotated by the 2x2 matrices of rope [B or 1, Sc + S, Dh/2, 2, 2]; v copied."""
+    _chk(qkv, "qkv", (torch.float16, torch.bfloat16))
+    b, s, d3 = qkv.shape
+    if d3 % (3 * heads):
+        raise ValueError("the last dimension of qkv must be 3 * heads * head_dim")
+    dh = d3 // (3 * heads)
+    sc = 0
+    for name, t in (("norm_qk", norm_qk), ("rope", rope), ("context_qkv", context_qkv), ("norm_added_qk", norm_added_qk)):
+        if t is not None:
+            _chk(t, name, (qkv.dtype,))
+    if context_qkv is not None:
+        if norm_added_qk is None or context_qkv.shape[0] != b or context_qkv.shape[2] != d3:
+            raise ValueError("context_qkv needs norm_added_qk and the batch and width of qkv")
+        sc = context_qkv.shape[1]
+    if norm_qk.numel() != 2 * dh or (norm_added_qk is not None and norm_added_qk.numel() != 2 * dh):
+        raise ValueError("norm weights must hold 2 * head_dim elements (q then k)")
+    per_batch = (sc + s) * dh * 2
+    if rope.numel() not in (per_batch, b * per_batch):
+        raise ValueError("rope must be [B or 1, Sc + S, head_dim / 2, 2, 2]")
+    out = torch.empty((b, sc + s, 3, heads, dh), dtype=qkv.dtype, device=qkv.device)
+    _l.check(_l.load().lq_rmsnorm_rope(_ptr(out), _ptr(qkv), _ptr(context_qkv), _ptr(norm_qk), _ptr(norm_added_qk), _ptr(rope),
+                                       per_batch if rope.numel() != per_batch else 0, _DT[qkv.dtype], b, s, sc, heads, dh, eps,
+                                       _stream()), "lq_rmsnorm_rope")
+    return out
+
+
 _KINDS = {"int8": _l.LQ_W_INT8, "fp8": _l.LQ_W_FP8, "int4": _l.LQ_W_INT4}
 
 

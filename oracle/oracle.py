@@ -611,3 +611,42 @@ def repack_rows32(w_bytes) -> np.ndarray:
 def unpack_rows32(packed, n: int, kb: int) -> np.ndarray:
     p = np.asarray(packed, dtype=np.uint8).reshape(n // 32, kb // 16, 32, 16)
     return np.ascontiguousarray(p.transpose(0, 2, 1, 3)).reshape(n, kb)
+
+
+# ----------------------------------------------------------------------------------------
+# q/k RMSNorm + rotary embedding + [text, image] concatenation in front of the FLUX attention
+# (kernels/rope/flux_apply_rope.cu:74-156: fuseRmsNormCatAndRope; :159-289 for the variants without the concatenation)
+# ----------------------------------------------------------------------------------------
+
+
+def rmsnorm_rope(qkv, context_qkv, norm_qk, norm_added_qk, rope, heads: int, dtype: str, eps: float = 1e-6) -> np.ndarray:
+    """qkv [B, S, 3*H*Dh], context_qkv [B, Sc, 3*H*Dh] or None, norm_* [2*Dh] (q then k), rope [B or 1, Sc+S, Dh/2, 2, 2],
+    all holding T values -> [B, Sc+S, 3, H, Dh].  q, k: n = T(x / sqrt(mean(x^2) + eps)) (statistics in fp64 narrowed to fp32:
+    a kernel with its own fp32 summation order agrees to one ULP of T), m = T(n * w), then every pair
+    (m0, m1) -> (T(T(m0*r00) + T(m1*r01)), T(T(m0*r10) + T(m1*r11))); v copied; text tokens first."""
+    x = np.asarray(qkv, dtype=F32)
+    b, s, d3 = x.shape
+    dh = d3 // (3 * heads)
+    parts = []
+    if context_qkv is not None:
+        parts.append((np.asarray(context_qkv, dtype=F32), np.asarray(norm_added_qk, dtype=F32)))
+    parts.append((x, np.asarray(norm_qk, dtype=F32)))
+    total = sum(p[0].shape[1] for p in parts)
+    r = np.broadcast_to(np.asarray(rope, dtype=F32).reshape(-1, total, 1, dh // 2, 2, 2), (b, total, heads, dh // 2, 2, 2))
+    out = np.empty((b, total, 3, heads, dh), dtype=F32)
+    at = 0
+    for t, w in parts:
+        n = t.shape[1]
+        t5 = t.reshape(b, n, 3, heads, dh)
+        out[:, at:at + n, 2] = t5[:, :, 2]
+        for c in (0, 1):
+            v = t5[:, :, c]
+            ms = ((v.astype(np.float64) ** 2).sum(-1, keepdims=True) / dh).astype(F32)
+            inv = (F32(1.0) / np.sqrt((ms + F32(eps)).astype(F32))).astype(F32)
+            m = round_to(round_to(v * inv, dtype) * w[c * dh:(c + 1) * dh], dtype).reshape(b, n, heads, dh // 2, 2)
+            rr = r[:, at:at + n]
+            y0 = round_to(round_to(m[..., 0] * rr[..., 0, 0], dtype) + round_to(m[..., 1] * rr[..., 0, 1], dtype), dtype)
+            y1 = round_to(round_to(m[..., 0] * rr[..., 1, 0], dtype) + round_to(m[..., 1] * rr[..., 1, 1], dtype), dtype)
+            out[:, at:at + n, c] = np.stack([y0, y1], axis=-1).reshape(b, n, heads, dh)
+        at += n
+    return out

@@ -704,3 +704,34 @@ def test_flux_int4_block_ops(ops, dev, full):
     ns, ms = F.ada_layernorm_int4(xs, temb, ws.norm, 3)
     want = F.flux_single_mlp_int4(xs, ns, score(ws.to_qkv.forward(ns)).contiguous(), ms[2].contiguous(), ws.mlp)
     assert torch.equal(y, want)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("b,s,sc,heads,dh", [(2, 70, 21, 3, 128), (1, 33, 0, 2, 64), (2, 5, 9, 24, 128)])
+def test_rmsnorm_rope_against_the_oracle(ops, dev, dt, b, s, sc, heads, dh):
+    """lq_rmsnorm_rope (invokeFusedRmsNormCatAndRope / invokeFusedRmsNormAndRope): v and the layout bit for bit; q and k within one
+    ULP of T per rounding step of the oracle (the mean of squares is summed in the kernel's own fp32 order), at most 2 % of the
+    elements differing at all; rope given per batch and shared by the batch."""
+    t = TORCH_DT[dt]
+    g = rng_t(b * 1000 + s + dh)
+    d3 = 3 * heads * dh
+    qkv = (torch.randn(b, s, d3, generator=g) * 1.7).to(t)
+    cqkv = (torch.randn(b, sc, d3, generator=g) * 0.8).to(t) if sc else None
+    nqk = (1 + 0.2 * torch.randn(2 * dh, generator=g)).to(t)
+    naqk = (1 + 0.2 * torch.randn(2 * dh, generator=g)).to(t) if sc else None
+    for rope_b in (b, 1):
+        rope = _rope_table(rope_b, sc + s, dh, 77 + rope_b).to(t)
+        out = ops.rmsnorm_rope(qkv.to(dev), nqk.to(dev), rope.to(dev), heads, None if cqkv is None else cqkv.to(dev),
+                               None if naqk is None else naqk.to(dev))
+        want = O.rmsnorm_rope(to_np_f32(qkv), None if cqkv is None else to_np_f32(cqkv), to_np_f32(nqk),
+                              None if naqk is None else to_np_f32(naqk), to_np_f32(rope), heads, dt)
+        got = to_np_f32(out)
+        assert got.shape == want.shape == (b, sc + s, 3, heads, dh)
+        assert np.array_equal(got[:, :, 2], want[:, :, 2])
+        ulp = 2.0 ** (-8 if dt == "bf16" else -11)
+        diff = np.abs(got[:, :, :2] - want[:, :, :2])
+        mag = np.abs(want[:, :, :2]).reshape(b, sc + s, 2, heads, dh // 2, 2).sum(-1, keepdims=True).repeat(2, -1).reshape(diff.shape)
+        assert np.all(diff <= 3 * ulp * mag + 1e-6), f"max excess {(diff - 3 * ulp * mag).max()}"
+        assert (diff != 0).mean() < 0.02
+    with pytest.raises(Exception):
+        ops.rmsnorm_rope(qkv.to(dev)[..., :-8].contiguous(), nqk.to(dev), rope.to(dev), heads)

@@ -475,3 +475,37 @@ def test_geglu_gate_is_constant_times_g_outside_the_tabulated_range(dt):
     same = (want == got) | (np.isnan(want) & np.isnan(got))
     assert same.all(), f"{(~same).sum()} patterns differ, first g = {go[~same][:4]}"
     assert np.array_equal(np.signbit(want[~np.isnan(want)]), np.signbit(got[~np.isnan(got)]))
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+def test_rmsnorm_rope_oracle_special_cases(dt):
+    """Identity rotation reduces the step to a per-head RMSNorm (compared with a plain fp64 evaluation), a quarter turn swaps
+    the two elements of every pair exactly, any rotation preserves the norm of the normalised vector (= sqrt(Dh) for unit
+    weights), v is copied and the text tokens come first."""
+    rng = np.random.default_rng(5)
+    b, s, sc, heads, dh = 2, 7, 3, 2, 64
+    q = O.round_to(rng.standard_normal((b, s, 3 * heads * dh)).astype(np.float32) * 2, dt)
+    c = O.round_to(rng.standard_normal((b, sc, 3 * heads * dh)).astype(np.float32), dt)
+    w = O.round_to(1 + 0.1 * rng.standard_normal(2 * dh).astype(np.float32), dt)
+    wa = O.round_to(1 + 0.1 * rng.standard_normal(2 * dh).astype(np.float32), dt)
+    eye = np.broadcast_to(np.eye(2, dtype=np.float32), (1, sc + s, dh // 2, 2, 2))
+    out = O.rmsnorm_rope(q, c, w, wa, eye, heads, dt)
+    assert out.shape == (b, sc + s, 3, heads, dh)
+    q5, c5 = q.reshape(b, s, 3, heads, dh), c.reshape(b, sc, 3, heads, dh)
+    assert np.array_equal(out[:, sc:, 2], q5[:, :, 2]) and np.array_equal(out[:, :sc, 2], c5[:, :, 2])
+    ulp = 2.0 ** (-8 if dt == "bf16" else -11)
+    for part, src, wt in ((out[:, sc:], q5, w), (out[:, :sc], c5, wa)):
+        for ci in (0, 1):
+            v = src[:, :, ci].astype(np.float64)
+            want = v / np.sqrt((v ** 2).mean(-1, keepdims=True) + 1e-6) * wt[ci * dh:(ci + 1) * dh]
+            assert np.all(np.abs(part[:, :, ci] - want) <= 2.5 * ulp * np.abs(want) + 2e-7)  # two roundings to T (fp16 subnormals below 6e-5)
+    quarter = np.broadcast_to(np.array([[0, -1], [1, 0]], dtype=np.float32), (b, sc + s, dh // 2, 2, 2))
+    turned = O.rmsnorm_rope(q, c, w, wa, quarter, heads, dt)
+    pairs, tp = out[:, :, :2].reshape(b, sc + s, 2, heads, dh // 2, 2), turned[:, :, :2].reshape(b, sc + s, 2, heads, dh // 2, 2)
+    assert np.array_equal(tp[..., 0], -pairs[..., 1]) and np.array_equal(tp[..., 1], pairs[..., 0])
+    ang = rng.uniform(0, 6.28, (1, sc + s, dh // 2))
+    rot = O.round_to(np.stack([np.cos(ang), -np.sin(ang), np.sin(ang), np.cos(ang)], -1).reshape(1, sc + s, dh // 2, 2, 2).astype(np.float32), dt)
+    ones = np.ones(2 * dh, dtype=np.float32)
+    y = O.rmsnorm_rope(q, None, ones, None, rot[:, sc:], heads, dt)
+    norms = np.sqrt((y[:, :, :2].astype(np.float64) ** 2).sum(-1))
+    assert np.all(np.abs(norms - np.sqrt(dh)) < (0.03 if dt == "bf16" else 0.005) * np.sqrt(dh))
