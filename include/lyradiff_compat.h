@@ -161,6 +161,26 @@ void invokeLayerNormWithShiftAndScaleFP8(fp8_e4m3_t* dst, const T* src, const T*
                   "invokeLayerNormWithShiftAndScaleFP8");
 }
 
+// ---- kernels/rope/flux_apply_rope.h:18-28,58-72 ---------------------------------------------------------------
+// q/k RMSNorm per head + rotary embedding (+ the [encoder, hidden] concatenation) in front of the attention;
+// out / input are [batch, seq, 3, head_num, head_dim], scale is [2 * head_dim] (q then k), rope_emb is indexed per batch.
+template <typename T>
+void invokeFusedRmsNormAndRope(T* out, const T* input, const T* scale, const T* rope_emb, float eps, int batch_size, int seq_len,
+                               int head_num, int head_dim, hipStream_t stream) {
+    detail::check(lq_rmsnorm_rope(out, input, nullptr, scale, nullptr, rope_emb, (size_t)seq_len * head_dim * 2,
+                                  detail::DType<T>::value, batch_size, seq_len, 0, head_num, head_dim, eps, stream),
+                  "invokeFusedRmsNormAndRope");
+}
+template <typename T>
+void invokeFusedRmsNormCatAndRope(T* out, const T* hidden, const T* encoder_hidden, const T* hidden_rms_scale,
+                                  const T* encoder_rms_scale, const T* rope_emb, float eps, int batch_size, int hidden_seq_len,
+                                  int encoder_seq_len, int head_num, int head_dim, hipStream_t stream) {
+    detail::check(lq_rmsnorm_rope(out, hidden, encoder_hidden, hidden_rms_scale, encoder_rms_scale, rope_emb,
+                                  (size_t)(hidden_seq_len + encoder_seq_len) * head_dim * 2, detail::DType<T>::value, batch_size,
+                                  hidden_seq_len, encoder_seq_len, head_num, head_dim, eps, stream),
+                  "invokeFusedRmsNormCatAndRope");
+}
+
 // ---- kernels/w4a4_gemm/w4a4_gemm.h:6-30 ------------------------------------------------------------------
 // Quantises A [m,k] (bf16) to group-64 int4 words + fp32 group scales and, when Bptr (lora down, bf16
 // [n = rank, k]) is given, writes the fp32 down projection A . B^T to Cptr [m, n].  The reference ADDS its

@@ -176,5 +176,56 @@ int main() {
             return 3;
         }
     }
+    // ---------------- invokeFusedRmsNormCatAndRope / invokeFusedRmsNormAndRope -----------------------------------------
+    // Exactly checkable cases of the reference call (FluxAttentionFP8Processor.cc:232-245): a quarter-turn rope with unit
+    // norm weights swaps each normalised pair (x, y) -> (-y, x); v is copied; the text rows come first; the single-stream
+    // launcher agrees with the concatenating one on the same rows.
+    {
+        const int B = 2, S = 9, SC = 5, H = 3, DH = 128, T = S + SC;
+        auto hid = rand_bf16((size_t)B * S * 3 * H * DH, 3.0f, seed), enc = rand_bf16((size_t)B * SC * 3 * H * DH, 3.0f, seed);
+        std::vector<bf16> ones(2 * DH, bf16(1.0f)), eye((size_t)B * T * DH * 2), quarter((size_t)B * T * DH * 2);
+        for (size_t i = 0; i < eye.size(); i += 4) {
+            eye[i] = bf16(1.0f); eye[i + 1] = bf16(0.0f); eye[i + 2] = bf16(0.0f); eye[i + 3] = bf16(1.0f);
+            quarter[i] = bf16(0.0f); quarter[i + 1] = bf16(-1.0f); quarter[i + 2] = bf16(1.0f); quarter[i + 3] = bf16(0.0f);
+        }
+        bf16 *dh = upload(hid), *de = upload(enc), *d1 = upload(ones), *deye = upload(eye), *dq = upload(quarter), *o1, *o2, *o3;
+        const size_t n_out = (size_t)B * T * 3 * H * DH;
+        CK(hipMalloc(&o1, n_out * 2)); CK(hipMalloc(&o2, n_out * 2)); CK(hipMalloc(&o3, (size_t)B * S * 3 * H * DH * 2));
+        try {
+            invokeFusedRmsNormCatAndRope<bf16>(o1, dh, de, d1, d1, deye, 1e-6f, B, S, SC, H, DH, st);
+            invokeFusedRmsNormCatAndRope<bf16>(o2, dh, de, d1, d1, dq, 1e-6f, B, S, SC, H, DH, st);
+            invokeFusedRmsNormAndRope<bf16>(o3, dh, d1, deye, 1e-6f, B, S, H, DH, st);  // rope rows 0..S-1 of each batch: identity too
+            CK(hipStreamSynchronize(st));
+            auto a = download(o1, n_out), q = download(o2, n_out), single = download(o3, (size_t)B * S * 3 * H * DH);
+            int bad = 0;
+            for (int b = 0; b < B; ++b)
+                for (int t = 0; t < T; ++t)
+                    for (int c = 0; c < 3; ++c)
+                        for (int h = 0; h < H; ++h)
+                            for (int e = 0; e < DH; e += 2) {
+                                const size_t o = ((((size_t)b * T + t) * 3 + c) * H + h) * DH + e;
+                                const std::vector<bf16>& src = t < SC ? enc : hid;
+                                const size_t si = ((((size_t)b * (t < SC ? SC : S) + (t < SC ? t : t - SC)) * 3 + c) * H + h) * DH + e;
+                                if (c == 2) {
+                                    bad += (float)a[o] != (float)src[si] || (float)a[o + 1] != (float)src[si + 1];
+                                } else {
+                                    bad += (float)q[o] != -(float)a[o + 1] || (float)q[o + 1] != (float)a[o];
+                                    if (t >= SC) {
+                                        const size_t so = ((((size_t)b * S + (t - SC)) * 3 + c) * H + h) * DH + e;
+                                        bad += (float)single[so] != (float)a[o] || (float)single[so + 1] != (float)a[o + 1];
+                                    }
+                                }
+                            }
+            // RMS of a normalised head is 1
+            double ss = 0;
+            for (int e = 0; e < DH; ++e) ss += (double)(float)a[e] * (float)a[e];
+            bad += std::fabs(std::sqrt(ss / DH) - 1.0) > 0.01;
+            std::printf("invokeFusedRmsNormCatAndRope<bf16>: B=%d S=%d Sc=%d H=%d Dh=%d, %d mismatches\n", B, S, SC, H, DH, bad);
+            failures += bad != 0;
+        } catch (const std::exception& e) {
+            std::printf("exception: %s\n", e.what());
+            return 3;
+        }
+    }
     return failures == 0 ? 0 : 1;
 }

@@ -28,11 +28,11 @@ def test_cpp_layer_types(dev):
 
 
 def test_cpp_flux_fp8_types(dev):
-    """FluxAttnPostFP8Processor / FluxSingleTransformerFP8Mlp / FP8LoraWeight (include/lyradiff_layers.h): each fused
+    """FluxAttnPostFP8Processor / FluxSingleTransformerFP8Mlp / FP8LoraWeight (include/lyradiff_layers.h) and the rope launchers: each fused
     forward equals the reference's launch sequence run step by step, bit for bit."""
     exe = os.path.join(ROOT, "tests", "cpp", "flux_fp8_check")
     assert os.path.exists(exe), "build it with `python -m lyradiff_amd.build` (prebuilt binaries travel to the GPU box)"
     r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count(" 0 mismatches") == 3
+    assert r.stdout.count(" 0 mismatches") == 4
