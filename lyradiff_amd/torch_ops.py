@@ -19,7 +19,7 @@ from . import ops as _ops
 _lib_op = torch.library.custom_op
 NAMES = ("sq_quant", "sq_quant_dynamic", "geglu_int8_dynamic", "int8_linear", "fp8_quant", "fp8_scale_cast", "fp8_linear",
          "w4a4_quant", "w4a4_linear", "repack_weight", "lora_down", "layernorm_mod_fp8", "gate_residual_layernorm_mod_fp8",
-         "fp8_linear_codes", "fp8_linear_gated", "flux_attn_post_fp8", "flux_single_mlp_fp8")
+         "fp8_linear_codes", "fp8_linear_gated", "flux_attn_post_fp8", "flux_single_mlp_fp8", "rmsnorm_rope")
 
 
 @_lib_op("lyradiff::sq_quant", mutates_args=())
@@ -140,6 +140,18 @@ def lora_down(x: Tensor, lora_down_w: Tensor) -> Tensor:
 @lora_down.register_fake
 def _(x, lora_down_w):
     return x.new_empty((x.shape[0], lora_down_w.shape[0]))
+
+
+@_lib_op("lyradiff::rmsnorm_rope", mutates_args=())
+def rmsnorm_rope(qkv: Tensor, norm_qk: Tensor, rope: Tensor, heads: int, context_qkv: Optional[Tensor] = None,
+                 norm_added_qk: Optional[Tensor] = None, eps: float = 1e-6) -> Tensor:
+    return _ops.rmsnorm_rope(qkv, norm_qk, rope, heads, context_qkv, norm_added_qk, eps)
+
+
+@rmsnorm_rope.register_fake
+def _(qkv, norm_qk, rope, heads, context_qkv=None, norm_added_qk=None, eps=1e-6):
+    sc = 0 if context_qkv is None else context_qkv.shape[1]
+    return qkv.new_empty((qkv.shape[0], sc + qkv.shape[1], 3, heads, qkv.shape[2] // (3 * heads)))
 
 
 @_lib_op("lyradiff::layernorm_mod_fp8", mutates_args=())
