@@ -335,6 +335,12 @@ def flux_whole_blocks(torch, dev, timeit):
     ang = torch.rand(1, sc + s, dh // 2, generator=g) * 6.28
     rope = torch.stack([ang.cos(), -ang.sin(), ang.sin(), ang.cos()], dim=-1).reshape(1, sc + s, dh // 2, 2, 2).bfloat16().to(dev)
     res = {}
+    from lyradiff_amd import ops as _ops
+    qkv = torch.randn(1, s, 3 * d, generator=g).bfloat16().to(dev)
+    cqkv = torch.randn(1, sc, 3 * d, generator=g).bfloat16().to(dev)
+    nqk = torch.ones(2 * dh).bfloat16().to(dev)
+    us = timeit(lambda: _ops.rmsnorm_rope(qkv, nqk, rope, heads, cqkv, nqk))
+    res["rmsnorm_rope_cat_4608x72x128"] = {"us": round(us, 2), "GB/s": round(2 * 2.0 * (s + sc) * 3 * d / us / 1e3, 1)}
     op = FO.FluxTransformerBlockOp("bf16", d, heads, dh, 6, FO.LyraQuantLevel.FP8_W8A8.value)
     op.reload_model_from_state_dict("b.", state("b.", dbl, ("norm_q", "norm_k", "norm_added_q", "norm_added_k")), "cpu")
     us = timeit(lambda: op.forward(x, ctx, rope, temb), iters=10, warm=3)
