@@ -88,7 +88,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path shards by token rows without "
-              "collectives; see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+              "collectives, so N GPUs are N independent copies of this run). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     import torch

@@ -3,10 +3,17 @@
 // that the reference computes inside its quantisation kernel with float atomics
 // (kernels/w4a4_gemm/w4a4_gemm.cu:769-953 of lyraDiff, `reduce_add` into a zeroed fp32 buffer, followed by a
 // separate float -> T conversion, layers/w4a4_gemm_block/W4A4Gemm.cc:138-150).  Here it is a skinny GEMM of its
-// own: a workgroup owns 32 rows and all of K, its eight wavefronts take interleaved 64-wide slices of K, the
+// own: a workgroup owns up to 32 rows and all of K, its eight wavefronts take interleaved 64-wide slices of K, the
 // partial 32 x rank blocks meet in LDS and are added in wavefront order -- no atomics, so the result does not
 // depend on scheduling -- and the output is written once, already in the requested type.  It reads x from HBM
 // only if the quantisation kernel that ran just before did not leave it in the caches.
+// The matrix instruction wants a lane to hold eight consecutive k of ONE row, so loading its operands straight
+// from memory makes every load instruction touch 32 different cache lines and use a quarter of each; the cache's
+// tag rate, not bandwidth or latency, then sets the time (about 10 us whatever m is).  A slice therefore takes the
+// coalesced route: a load instruction fetches eight whole 128-byte lines (eight lanes per row), the wavefront
+// parks the slice in its private, bank-swizzled LDS block and reads the fragments back from there.  The launch
+// spreads the rows over every CU: a workgroup takes ceil(m / CUs) rows when that is fewer than 32 (the unused
+// rows of the 32-row matrix instruction repeat the last one, which costs no memory traffic).
 #include "lq_common.h"
 
 namespace lq {
@@ -23,46 +30,85 @@ template <bool F16> __device__ __forceinline__ v16f_t mfma16(const v4i& a, const
 // NR: rank / 32.  OUT: 0 fp32, 1 fp16, 2 bf16.
 template <bool F16, int NR, int OUT>
 __global__ __launch_bounds__(512) void lora_down_kernel(void* __restrict__ out, const unsigned short* __restrict__ x,
-                                                        const unsigned short* __restrict__ down, int m, int k) {
+                                                        const unsigned short* __restrict__ down, int m, int k, int rows_per_wg) {
     constexpr int W = 8;                    // wavefronts per workgroup, each takes every eighth 64-wide slice of K
-    __shared__ float part[W - 1][NR][16][64];  // partial blocks of wavefronts 1..7
+    constexpr int WAVE_STAGE = (1 + NR) * 4096;  // one slice of x and of `down`: 32 rows x 128 bytes each
+    constexpr int PART_BYTES = (W - 1) * NR * 16 * 64 * 4;
+    __shared__ __attribute__((aligned(16))) char smem[W * WAVE_STAGE > PART_BYTES ? W * WAVE_STAGE : PART_BYTES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int row0 = blockIdx.x * 32;
+    const int row0 = blockIdx.x * rows_per_wg;
     const int lr = lane & 31, lh = lane >> 5;
-    const unsigned short* xrow = x + (size_t)min(row0 + lr, m - 1) * k + lh * 8;
-    const unsigned short* drow = down + (size_t)lr * k + lh * 8;
+    char* stage = smem + wave * WAVE_STAGE;
+    // memory side: lane -> (row 8*i + lane/8, 16-byte chunk lane%8); LDS side: chunk c of row r sits at chunk
+    // slot c ^ ((r >> 1) & 7), which keeps both the 16-lane write groups and the 16-lane read groups conflict-free
+    const int gr = lane >> 3, gc = lane & 7;
+    const unsigned short* xg[4];
+    const unsigned short* dg[4];
+    int wofs[4], rofs[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = i * 8 + gr;
+        xg[i] = x + (size_t)min(row0 + min(r, rows_per_wg - 1), m - 1) * k + gc * 8;
+        dg[i] = down + (size_t)r * k + gc * 8;
+        wofs[i] = r * 128 + ((gc ^ ((r >> 1) & 7)) << 4);
+        rofs[i] = lr * 128 + (((2 * i + lh) ^ ((lr >> 1) & 7)) << 4);  // matrix step i: k = 16 i + 8 lh .. + 8
+    }
     v16f_t acc[NR];
 #pragma unroll
     for (int r = 0; r < NR; ++r)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[r][v] = 0.0f;
-    // a wavefront's slice: 64 consecutive k (four MFMA steps, one 128-byte line per row), every eighth slice.
-    // The operands of the next slice are requested before the matrix instructions of the current one, so the
-    // memory latency of a slice is hidden behind the previous slice's arithmetic and the other wavefronts.
-    v4i xf[2][4], df[2][NR][4];
+    // The lines of the next slice are requested before the current slice goes through LDS and the matrix
+    // instructions, so their latency is hidden behind that work and the other wavefronts.
+    constexpr int NBUF = 2;  // the slice on its way through LDS and the one requested behind it (deeper queues measured no faster)
+    v4i gx[NBUF][4], gd[NBUF][NR][4];
     auto load_slice = [&](int k0, int buf) {
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            xf[buf][s] = *reinterpret_cast<const v4i*>(xrow + k0 + s * 16);
+        for (int i = 0; i < 4; ++i) {
+            gx[buf][i] = *reinterpret_cast<const v4i*>(xg[i] + k0);
 #pragma unroll
-            for (int r = 0; r < NR; ++r) df[buf][r][s] = *reinterpret_cast<const v4i*>(drow + (size_t)r * 32 * k + k0 + s * 16);
+            for (int r = 0; r < NR; ++r) gd[buf][r][i] = *reinterpret_cast<const v4i*>(dg[i] + (size_t)r * 32 * k + k0);
         }
     };
     auto compute_slice = [&](int buf) {
 #pragma unroll
-        for (int s = 0; s < 4; ++s)
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<v4i*>(stage + wofs[i]) = gx[buf][i];
 #pragma unroll
-            for (int r = 0; r < NR; ++r) acc[r] = mfma16<F16>(df[buf][r][s], xf[buf][s], acc[r]);
+            for (int r = 0; r < NR; ++r) *reinterpret_cast<v4i*>(stage + (1 + r) * 4096 + wofs[i]) = gd[buf][r][i];
+        }
+        // the wavefront's LDS accesses complete in program order; the fence only keeps the compiler from
+        // moving the reads of other lanes' data above the writes
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const v4i xf = *reinterpret_cast<const v4i*>(stage + rofs[s]);
+#pragma unroll
+            for (int r = 0; r < NR; ++r)
+                acc[r] = mfma16<F16>(*reinterpret_cast<const v4i*>(stage + (1 + r) * 4096 + rofs[s]), xf, acc[r]);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
     };
+    constexpr int STEP = 64 * W;
     int k0 = wave * 64;
-    if (k0 < k) load_slice(k0, 0);
-    for (; k0 < k; k0 += 2 * 64 * W) {
-        if (k0 + 64 * W < k) load_slice(k0 + 64 * W, 1);
-        compute_slice(0);
-        if (k0 + 64 * W >= k) break;
-        if (k0 + 2 * 64 * W < k) load_slice(k0 + 2 * 64 * W, 0);
-        compute_slice(1);
+#pragma unroll
+    for (int b = 0; b < NBUF - 1; ++b)
+        if (k0 + b * STEP < k) load_slice(k0 + b * STEP, b);
+    // the buffers rotate with a period of NBUF slices; the loop body is unrolled over one period so that every
+    // buffer index is a compile-time constant (the lines in flight must stay in registers)
+    for (; k0 < k; k0 += NBUF * STEP) {
+#pragma unroll
+        for (int b = 0; b < NBUF; ++b) {
+            if (k0 + b * STEP < k) {
+                if (k0 + (b + NBUF - 1) * STEP < k) load_slice(k0 + (b + NBUF - 1) * STEP, (b + NBUF - 1) % NBUF);
+                compute_slice(b);
+            }
+        }
     }
+    __syncthreads();  // every wavefront is done with its operand block: the partial sums may overwrite them
+    float(*part)[NR][16][64] = reinterpret_cast<float(*)[NR][16][64]>(smem);  // partial blocks of wavefronts 1..7
     if (wave != 0) {
 #pragma unroll
         for (int r = 0; r < NR; ++r)
@@ -78,7 +124,7 @@ __global__ __launch_bounds__(512) void lora_down_kernel(void* __restrict__ out, 
         for (int v = 0; v < 16; ++v)
 #pragma unroll
             for (int w = 0; w < W - 1; ++w) acc[r][v] += part[w][r][v][lane];  // wavefront order: 0, 1, ..., 7
-        if (row < m) {
+        if (row < m && lr < rows_per_wg) {
             // result layout of the 32x32 MFMA: this lane holds row (= x row) lr and rank indices 8*(v/4) + 4*lh + v%4
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
@@ -98,13 +144,19 @@ __global__ __launch_bounds__(512) void lora_down_kernel(void* __restrict__ out, 
 }
 
 template <bool F16, int NR> static int launch_lora_down(void* out, lq_dtype_t out_dtype, const void* x, const void* down, int m, int k, hipStream_t st) {
-    dim3 grid((unsigned)((m + 31) / 32)), block(512);
+    static const int num_cu = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        return n;
+    }();
+    const int rpw = std::min(32, std::max(8, (m + num_cu - 1) / num_cu));
+    dim3 grid((unsigned)((m + rpw - 1) / rpw)), block(512);
     const unsigned short* xs = static_cast<const unsigned short*>(x);
     const unsigned short* ds = static_cast<const unsigned short*>(down);
     switch (out_dtype) {
-        case LQ_F32: hipLaunchKernelGGL((lora_down_kernel<F16, NR, 0>), grid, block, 0, st, out, xs, ds, m, k); break;
-        case LQ_F16: hipLaunchKernelGGL((lora_down_kernel<F16, NR, 1>), grid, block, 0, st, out, xs, ds, m, k); break;
-        case LQ_BF16: hipLaunchKernelGGL((lora_down_kernel<F16, NR, 2>), grid, block, 0, st, out, xs, ds, m, k); break;
+        case LQ_F32: hipLaunchKernelGGL((lora_down_kernel<F16, NR, 0>), grid, block, 0, st, out, xs, ds, m, k, rpw); break;
+        case LQ_F16: hipLaunchKernelGGL((lora_down_kernel<F16, NR, 1>), grid, block, 0, st, out, xs, ds, m, k, rpw); break;
+        case LQ_BF16: hipLaunchKernelGGL((lora_down_kernel<F16, NR, 2>), grid, block, 0, st, out, xs, ds, m, k, rpw); break;
         default: set_error("lq_lora_down: unsupported output dtype %d", (int)out_dtype); return LQ_ERR_UNSUPPORTED;
     }
     return check_launch("lq_lora_down");
