@@ -383,7 +383,22 @@ def sdxl_geglu_ffn_chain(torch, ops, dev, timeit):
 
     us = timeit(chain, iters=30, warm=5)
     ops_total = 2.0 * m * (8 * d * d + d * 4 * d)
-    return {"sdxl_geglu_ffn_int8_chain_4096": {"us": round(us, 2), "TOP/s": round(ops_total / us / 1e6, 1)}}
+    res = {"sdxl_geglu_ffn_int8_chain_4096": {"us": round(us, 2), "TOP/s": round(ops_total / us / 1e6, 1)}}
+    # The same five launches replayed from a HIP graph: the eager figure above is bounded by the host's per-launch cost
+    # (the kernels take 3-10 us each), the replay shows what the kernels themselves need.
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        chain()
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        y_static = chain()
+    torch.cuda.synchronize()
+    us_g = timeit(graph.replay, iters=50, warm=5)
+    if not torch.equal(y_static, chain()):
+        raise RuntimeError("graph replay of the SDXL INT8 chain differs from the eager result")
+    res["sdxl_geglu_ffn_int8_chain_4096_graph_replay"] = {"us": round(us_g, 2), "TOP/s": round(ops_total / us_g / 1e6, 1)}
+    return res
 
 
 def flux_linear_chain_1280(torch, ops, dev, timeit):
