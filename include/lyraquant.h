@@ -81,7 +81,9 @@ int lq_int8_weight_quant(float* scale_out, int8_t* q_out, const void* weight, lq
  * q = sat_s8(rne(f32(h*g) * pre[k] / in_scale[0])); adds and products rounded to T as the
  * reference does.  bias may be NULL.  Replaces invokeFusedAddBiasGegluInt8O<T>
  * (kernels/quant_kernels/ffn_kernels_int8.h:12-21, ffn_kernels_int8.cu:102-237); lifts its
- * dim in {1280,2560,5120} limit to any dim % 8 == 0.  T in {F16, BF16, F32}. */
+ * dim in {1280,2560,5120} limit to any dim % 8 == 0.  T in {F16, BF16, F32}.
+ * The first F16 / BF16 call on a device builds a constant lookup table on `stream` and waits for that
+ * one kernel (later calls never block); under stream capture it records the table kernel instead. */
 int lq_geglu_int8(int8_t* dst, const void* hidden, const void* bias, lq_dtype_t dtype,
                   const float* pre_quant_scale, const float* input_quant_scale, size_t rows, size_t dim,
                   lq_stream_t stream);

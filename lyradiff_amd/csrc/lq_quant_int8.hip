@@ -9,6 +9,8 @@
 // Formulas follow the lyraDiff reference: kernels/quant_kernels/quant_kernels.cu:51-115
 // (activation), :173-223 (weights), :117-171 (dequant), kernels/quant_kernels/
 // ffn_kernels_int8.cu:102-147 (bias + GEGLU), kernels/quant_kernels/int8_utils.cuh:23-28.
+#include <atomic>
+
 #include "lq_common.h"
 #include <type_traits>
 
@@ -362,13 +364,13 @@ __global__ __launch_bounds__(256) void int8_weight_quant_kernel(float* __restric
 // The gate factor  gate(g) = T( g * T( 0.5 * (1 + tanh(0.79788 * (g + 0.044715 * T(g * T(g*g))))) ) )  depends only on the
 // 16-bit value g, and its evaluation (a tanh built from basic IEEE operations, so that a CPU restatement reproduces it bit
 // for bit) is about 70 of the kernel's 85 vector instructions per element.  For fp16 and bf16 inputs the factor is
-// therefore tabulated: a small kernel in front of every call evaluates the formula once for each 16-bit pattern with
+// therefore tabulated: a small kernel, run once per device (ensure_gate_table), evaluates the formula for each 16-bit pattern with
 // 2^-12 <= |g| < 8 (30720 fp16 / 3840 bf16 patterns) into a table in device memory, every workgroup of the main kernel copies
 // the table into LDS and looks the factor up.  Outside that range the inner factor T(0.5 * (1 + tanh(...))) is a constant:
 // 0.5 for |g| < 2^-12 (the deviation from 0.5 is below half a unit in the last place of T), 1 for g >= 8 and 0 for g <= -8
 // (the tanh is +-1 in fp32 there), so gate(g) = T(g * c) with that constant -- the formula's own last step; infinities and
 // NaN follow the same expressions.  tests/test_oracle_pins.py checks these three constants against the formula for every
-// 16-bit pattern outside the table.  The table's contents never change; concurrent calls that rebuild it write the same bytes.
+// 16-bit pattern outside the table.  The table's contents never change; concurrent first calls that build it write the same bytes.
 template <typename Tag> __device__ __forceinline__ float geglu_gate(float g) {
     const float cube = round_through<Tag>(g * round_through<Tag>(g * g));
     const float cdf = 0.5f * (1.0f + tanh_basic(0.7978845608028654f * (g + 0.044715f * cube)));
@@ -493,6 +495,33 @@ __global__ __launch_bounds__(THREADS) void geglu_int8_kernel(int8_t* __restrict_
     }
 }
 
+// The gate table holds constants, so it is built once per device and element type: the first call on a device
+// launches the table kernel on the caller's stream and waits for it (the only blocking step of the entry point, once
+// per process), after which calls on any stream find it complete.  While the stream is being captured into a graph
+// nothing may block: the table kernel then simply becomes part of the graph, and the device stays unmarked.
+template <typename Tag> static int ensure_gate_table(hipStream_t st) {
+    static std::atomic<unsigned> built{0};  // one bit per device ordinal; devices beyond 31 rebuild on every call
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 32;
+    const unsigned bit = (dev >= 0 && dev < 32) ? 1u << dev : 0u;
+    if (bit != 0 && (built.load(std::memory_order_acquire) & bit) != 0) return LQ_OK;
+    constexpr unsigned entries = 2 * GateTable<Tag>::COUNT;
+    hipLaunchKernelGGL((geglu_table_kernel<Tag>), dim3((entries + 255) / 256), dim3(256), 0, st);
+    if (int rc = check_launch("geglu_int8 gate table"); rc != LQ_OK) return rc;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess) {
+        (void)hipGetLastError();  // e.g. the null stream while another stream captures: treat as capturing
+        return LQ_OK;
+    }
+    if (cs != hipStreamCaptureStatusNone || bit == 0) return LQ_OK;
+    if (hipStreamSynchronize(st) != hipSuccess) {
+        set_error("geglu_int8: waiting for the gate table failed: %s", hipGetErrorString(hipGetLastError()));
+        return LQ_ERR_HIP;
+    }
+    built.fetch_or(bit, std::memory_order_release);
+    return LQ_OK;
+}
+
 template <typename Tag, bool DYNAMIC>
 static int launch_geglu(int8_t* dst, float* scale_out, const void* hidden, const void* bias, const float* pre,
                         const float* in_scale, size_t rows, size_t dim, hipStream_t st) {
@@ -504,11 +533,10 @@ static int launch_geglu(int8_t* dst, float* scale_out, const void* hidden, const
     const int np = (int)((dim + 511) / 512);
     size_t lds = 0, threads = 256, cap = 65535;
     if constexpr (Elem<Tag>::bytes == 2) {
-        // the gate table, rebuilt in front of every call (no state to initialise, nothing for a captured graph to miss);
-        // every workgroup stages it once, so the grid is a few workgroups per CU that walk the rows.  The fp16 table
-        // (60 KB) allows two workgroups per CU: those have eight wavefronts each.
+        // every workgroup stages the gate table once, so the grid is a few workgroups per CU that walk the rows.  The
+        // fp16 table (60 KB) allows two workgroups per CU: those have eight wavefronts each.
         constexpr unsigned entries = 2 * GateTable<Tag>::COUNT;
-        hipLaunchKernelGGL((geglu_table_kernel<Tag>), dim3((entries + 255) / 256), dim3(256), 0, st);
+        if (int rc = ensure_gate_table<Tag>(st); rc != LQ_OK) return rc;
         lds = entries * sizeof(unsigned short);
         threads = (lds > 32768 && np <= 10) ? 512 : 256;  // (the 16-pass form needs all 256 registers of a 256-thread workgroup)
         cap = 256 * (lds > 32768 ? 2 : 8);

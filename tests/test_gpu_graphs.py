@@ -94,3 +94,42 @@ def test_sdxl_int8_ffn_chain_replays_exactly(ops, dev):
     e1.record()
     torch.cuda.synchronize()
     print(f"SDXL INT8 FFN chain, graph replay: {e0.elapsed_time(e1) / 20 * 1e3:.1f} us per chain")
+
+
+_FIRST_CALL_UNDER_CAPTURE = r"""
+import sys, torch
+sys.path.insert(0, sys.argv[1])
+from lyradiff_amd import ops
+from oracle import oracle as O
+dev = torch.device("cuda:0")
+g = torch.Generator().manual_seed(11)
+x = (torch.randn(96, 2 * 640, generator=g) * 2).half().to(dev)
+side = torch.cuda.Stream()
+graph = torch.cuda.CUDAGraph()
+with torch.cuda.graph(graph, stream=side):   # the process's very first GEGLU call: the gate table is not built yet
+    q_static, s_static = ops.geglu_int8_dynamic(x, None, None)
+for i in range(3):
+    graph.replay()
+    torch.cuda.synchronize()
+    q_ref, s_ref = O.geglu_int8_dynamic(x.float().cpu().numpy(), None, None, "f16")
+    assert (q_static.cpu().numpy() == q_ref).all() and (s_static.cpu().numpy() == s_ref).all(), i
+    x.copy_(torch.roll(x, 1, 0))
+q_eager, s_eager = ops.geglu_int8_dynamic(x, None, None)   # first eager call: builds the table for good
+graph.replay()
+torch.cuda.synchronize()
+assert torch.equal(q_eager, q_static) and torch.equal(s_eager, s_static)
+print("capture-first ok")
+"""
+
+
+def test_geglu_first_call_inside_a_capture(dev):
+    """The GEGLU gate table is built by the first call on a device.  When that call is being captured into a graph it must
+    not block: the table kernel is recorded into the graph instead, and replays are exact.  Needs a process of its own (in
+    this one the table exists already)."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", _FIRST_CALL_UNDER_CAPTURE, root], capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0 and "capture-first ok" in r.stdout, r.stdout + r.stderr
