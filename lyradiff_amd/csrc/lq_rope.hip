@@ -107,7 +107,7 @@ extern "C" int lq_rmsnorm_rope(void* out, const void* qkv, const void* context_q
                    reinterpret_cast<uintptr_t>(context_qkv) % 8 == 0 && reinterpret_cast<uintptr_t>(norm_qk) % 8 == 0 &&
                    reinterpret_cast<uintptr_t>(norm_added_qk) % 8 == 0 && reinterpret_cast<uintptr_t>(rope) % 16 == 0 &&
                    rope_batch_stride % 8 == 0,
-               LQ_ERR_ARG, "lq_rmsnorm_rope: tensors must be 8-byte aligned, rope (and its batch stride in bytes) 16-byte aligned");
+               LQ_ERR_ARG, "lq_rmsnorm_rope: tensors must be 8-byte aligned, rope 16-byte aligned and its batch stride a multiple of 8 elements");
     const size_t tokens = (size_t)batch * ((size_t)seq + context_seq);
     LQ_REQUIRE(tokens <= 0x7fffffffu, LQ_ERR_SHAPE, "lq_rmsnorm_rope: too many tokens for one launch");
     dim3 grid((unsigned)tokens), block(256);
