@@ -33,7 +33,15 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream():
+    """Handle of the current HIP stream of the current device.  The private accessors skip the Stream object and the
+    device-index normalisation of torch.cuda.current_stream() (2.8 -> 0.4 us per call); without them the public path is used."""
+    if _raw_stream is not None and _raw_device is not None:
+        return _raw_stream(_raw_device())
     return torch.cuda.current_stream().cuda_stream
 
 
