@@ -225,7 +225,8 @@ def test_profiler_fills_the_shape_cache(ops, dev, tactic_guard):
 
 # ---- W4A4 low-rank branch ------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dt", ["bf16", "f16"])
-@pytest.mark.parametrize("m,k,rank", [(300, 3072, 32), (4608, 3072, 32), (70, 256, 64)])
+# rows per workgroup follow m: 8 (m = 5, 70, 300), 18 (4608), 27 (6912), 32 with a ragged last workgroup (9000)
+@pytest.mark.parametrize("m,k,rank", [(300, 3072, 32), (4608, 3072, 32), (70, 256, 64), (5, 64, 32), (6912, 3072, 32), (9000, 1024, 64)])
 def test_lora_down(ops, dev, dt, m, k, rank):
     g = rng_t(m + k + rank)
     x = torch.randn(m, k, generator=g).to(TORCH_DT[dt])
