@@ -353,6 +353,42 @@ def flux_whole_blocks(torch, dev, timeit):
     us = timeit(lambda: sop.forward(xs, rope, temb), iters=10, warm=3)
     lin = 2.0 * d * d * (s + sc) * (3 + 4 + 5)
     res["flux_single_block_fp8_whole_1024"] = {"us": round(us, 1), "linear_TFLOP/s": round(lin / us / 1e6, 1)}
+    del sop
+
+    # The same blocks at level INT4_W4A4_FULL: W4A4 linears with their rank-32 low-rank branch (random codes and scales in
+    # the reference's container layout), FP8 adaLN and ff.net.2 linears.
+    def w4(prefix, n, k, bias=True):
+        sd = {prefix + "packed_weight": torch.randint(-128, 128, (n, k // 2), generator=g, dtype=torch.int8),
+              prefix + "weight_scale": torch.rand(n, k // 64, generator=g) * 4e-3 + 1e-3,
+              prefix + "smooth": torch.rand(k, generator=g) + 0.5,
+              prefix + "lora_up": (0.05 * torch.randn(n, 32, generator=g)).bfloat16(),
+              prefix + "lora_down": (0.05 * torch.randn(32, k, generator=g)).bfloat16()}
+        if bias:
+            sd[prefix + "bias"] = (0.02 * torch.randn(n, generator=g)).bfloat16()
+        return sd
+
+    level = FO.LyraQuantLevel.INT4_W4A4_FULL.value
+    sd = state("b.", {k: v for k, v in dbl.items() if k.startswith("norm1") or k.endswith("net.2")},
+               ("norm_q", "norm_k", "norm_added_q", "norm_added_k"))
+    for name, n in (("attn.to_qkv.", 3 * d), ("attn.to_added_qkv.", 3 * d), ("attn.to_out.0.", d), ("attn.to_add_out.", d),
+                    ("ff.net.0.proj.", 4 * d), ("ff_context.net.0.proj.", 4 * d)):
+        sd.update(w4("b." + name, n, d))
+    op = FO.FluxTransformerBlockOp("bf16", d, heads, dh, 6, level)
+    op.reload_model_from_state_dict("b.", sd, "cpu")
+    us = timeit(lambda: op.forward(x, ctx, rope, temb), iters=10, warm=3)
+    lin = 2.0 * d * d * ((s + sc) * (3 + 1 + 8))
+    res["flux_double_block_int4_whole_1024"] = {"us": round(us, 1), "linear_TOP/s": round(lin / us / 1e6, 1)}
+    del op, sd
+    sd = state("b.", {"norm.linear": (3 * d, d)}, ("norm_q", "norm_k"))
+    sd.update(w4("b.attn.to_qkv.", 3 * d, d))
+    sd.update(w4("b.proj_mlp.", 4 * d, d))
+    sd.update(w4("b.proj_out.linears.0.", d, d))
+    sd.update(w4("b.proj_out.linears.1.linear.", d, 4 * d, bias=False))
+    sop = FO.FluxSingleTransformerBlockOp("bf16", d, heads, dh, 4, level)
+    sop.reload_model_from_state_dict("b.", sd, "cpu")
+    us = timeit(lambda: sop.forward(xs, rope, temb), iters=10, warm=3)
+    lin = 2.0 * d * d * (s + sc) * (3 + 4 + 5)
+    res["flux_single_block_int4_whole_1024"] = {"us": round(us, 1), "linear_TOP/s": round(lin / us / 1e6, 1)}
     return res
 
 
