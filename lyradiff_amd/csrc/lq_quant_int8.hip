@@ -393,9 +393,12 @@ template <typename Tag> __global__ __launch_bounds__(256) void geglu_table_kerne
     gate_table<Tag>()[i] = (unsigned short)Elem<Tag>::store(geglu_gate<Tag>(Elem<Tag>::load(bits)));
 }
 
-// One wavefront per row; the row of `dim` products h*g stays in registers (NP passes of 512).
-template <typename Tag, int NP, bool DYNAMIC, int THREADS>
-__global__ __launch_bounds__(THREADS) void geglu_int8_kernel(int8_t* __restrict__ dst, float* __restrict__ scale_out,
+// SW wavefronts per row (1, or 2 for wide rows: half the registers per lane, so twice the wavefronts per SIMD); a
+// wavefront's share of the row's `dim` products h*g stays in registers (NP passes of 512 columns).  With SW = 2 the two
+// halves of a row meet in LDS for the row maximum; the row loop then has the same trip count in every wavefront of the
+// workgroup, because it contains a workgroup barrier.
+template <typename Tag, int NP, bool DYNAMIC, int THREADS, int SW>
+__global__ __launch_bounds__(THREADS, (SW == 2 && THREADS == 512) ? 4 : 1) void geglu_int8_kernel(int8_t* __restrict__ dst, float* __restrict__ scale_out,
                                                          const void* __restrict__ hidden,
                                                          const void* __restrict__ bias,
                                                          const float* __restrict__ pre,
@@ -408,18 +411,24 @@ __global__ __launch_bounds__(THREADS) void geglu_int8_kernel(int8_t* __restrict_
             *reinterpret_cast<uint4*>(s_gate + i) = *reinterpret_cast<const uint4*>(tab + i);
         __syncthreads();
     }
-    const int lane = threadIdx.x & 63;
-    const size_t wpb = blockDim.x >> 6;  // wavefronts (= rows in flight) per workgroup
-    const size_t wave = (size_t)blockIdx.x * wpb + (threadIdx.x >> 6);
-    const size_t nwaves = (size_t)gridDim.x * wpb;
-    for (size_t row = wave; row < rows; row += nwaves) {
-        const char* rb = static_cast<const char*>(hidden) + row * (size_t)dim * 2 * Elem<Tag>::bytes;
+    __shared__ float s_half_max[2][THREADS / 64];  // SW = 2: each wavefront's maximum over its half row, by loop parity
+    const int lane = threadIdx.x & 63, wave_in_wg = threadIdx.x >> 6;
+    const size_t wpb = blockDim.x >> 6;  // wavefronts per workgroup; wpb / SW rows in flight
+    const size_t team = ((size_t)blockIdx.x * wpb + wave_in_wg) / SW;  // the wavefronts 2t, 2t+1 of a workgroup share a row
+    const size_t nteams = (size_t)gridDim.x * wpb / SW;
+    const int cbase = (SW == 2 && (wave_in_wg & 1)) ? NP * 512 : 0;
+    const size_t trips = (rows + nteams - 1) / nteams;
+    for (size_t trip = 0; trip < trips; ++trip) {
+        const size_t row = team + trip * nteams;
+        const bool live = row < rows;
+        if (SW == 1 && !live) break;
+        const char* rb = static_cast<const char*>(hidden) + (live ? row : 0) * (size_t)dim * 2 * Elem<Tag>::bytes;
         float t[NP][8];
         float amax = 0.0f;
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
-            int col = (p * 64 + lane) * 8;
-            if (col < dim) {
+            int col = cbase + (p * 64 + lane) * 8;
+            if (col < dim && live) {
                 float h[8], g[8], pv[8], gel[8];
                 load8<Tag>(rb, col, h);
                 load8<Tag>(rb, col + dim, g);
@@ -472,18 +481,23 @@ __global__ __launch_bounds__(THREADS) void geglu_int8_kernel(int8_t* __restrict_
         float s;
         if constexpr (DYNAMIC) {
             amax = wave_max(amax);
+            if constexpr (SW == 2) {
+                if (lane == 0) s_half_max[trip & 1][wave_in_wg] = amax;
+                __syncthreads();  // one barrier per trip: the next trip writes the other parity
+                amax = fmaxf(amax, s_half_max[trip & 1][wave_in_wg ^ 1]);
+            }
             s = (amax <= 5.9604644775390625e-08f) ? 1.0f : amax / 127.0f;
-            if (lane == 0) scale_out[row] = s;
+            if (lane == 0 && cbase == 0 && live) scale_out[row] = s;
         } else {
             s = in_scale[0];
         }
         const float r = 1.0f / s;
         const bool slow = recip_unsafe(s, r);
-        int8_t* ob = dst + row * (size_t)dim;
+        int8_t* ob = dst + (live ? row : 0) * (size_t)dim;
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
-            int col = (p * 64 + lane) * 8;
-            if (col < dim) {
+            int col = cbase + (p * 64 + lane) * 8;
+            if (col < dim && live) {
                 int q[8];
                 quant8<-128, 127>(t[p], s, r, slow, q);
                 uint2 o;
@@ -530,7 +544,10 @@ static int launch_geglu(int8_t* dst, float* scale_out, const void* hidden, const
                    (bias == nullptr || reinterpret_cast<uintptr_t>(bias) % 16 == 0) &&
                    (pre == nullptr || reinterpret_cast<uintptr_t>(pre) % 16 == 0),
                LQ_ERR_ARG, "geglu_int8: pointers must be 16-byte aligned");
-    const int np = (int)((dim + 511) / 512);
+    const int np_row = (int)((dim + 511) / 512);
+    // rows of 2561..5120 columns go to two wavefronts each (the 5120-wide rows of SDXL: 10 passes -> 5, half the registers)
+    const int sw = (np_row > 5 && np_row <= 10) ? 2 : 1;
+    const int np = (np_row + sw - 1) / sw;
     size_t lds = 0, threads = 256, cap = 65535;
     if constexpr (Elem<Tag>::bytes == 2) {
         // every workgroup stages the gate table once, so the grid is a few workgroups per CU that walk the rows.  The
@@ -541,14 +558,20 @@ static int launch_geglu(int8_t* dst, float* scale_out, const void* hidden, const
         threads = (lds > 32768 && np <= 10) ? 512 : 256;  // (the 16-pass form needs all 256 registers of a 256-thread workgroup)
         cap = 256 * (lds > 32768 ? 2 : 8);
     }
-    size_t blocks = (rows + threads / 64 - 1) / (threads / 64);
+    const size_t rows_per_wg = threads / 64 / sw;
+    size_t blocks = (rows + rows_per_wg - 1) / rows_per_wg;
     if (blocks > cap) blocks = cap;
     dim3 grid((unsigned)blocks), block((unsigned)threads);
     int d = (int)dim;
-#define LQ_GG_CASE(NPV)                                                                                                  \
+#define LQ_GG_CASE(NPV) \
+    do {                \
+        if (sw == 2) LQ_GG_GO(NPV, ((NPV == 3 || NPV == 5) ? 2 : 1)); /* split rows need 3..5 passes per wavefront */ \
+        else LQ_GG_GO(NPV, 1);                                                                                        \
+    } while (0)
+#define LQ_GG_GO(NPV, SWV)                                                                                               \
     do {                                                                                                                 \
-        auto kern = threads == 512 ? geglu_int8_kernel<Tag, NPV, DYNAMIC, (NPV <= 10 ? 512 : 256)>                       \
-                                   : geglu_int8_kernel<Tag, NPV, DYNAMIC, 256>;                                          \
+        auto kern = threads == 512 ? geglu_int8_kernel<Tag, NPV, DYNAMIC, (NPV <= 10 ? 512 : 256), SWV>                  \
+                                   : geglu_int8_kernel<Tag, NPV, DYNAMIC, 256, SWV>;                                     \
         static bool raised = false; /* raising the dynamic LDS limit is idempotent; a race only repeats it */           \
         if (lds > 48 * 1024 && !raised) {                                                                                \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
@@ -566,6 +589,7 @@ static int launch_geglu(int8_t* dst, float* scale_out, const void* hidden, const
     else if (np <= 10) LQ_GG_CASE(10);
     else LQ_GG_CASE(16);
 #undef LQ_GG_CASE
+#undef LQ_GG_GO
     return check_launch("geglu_int8");
 }
 

@@ -107,6 +107,28 @@ def test_geglu_int8(ops, dev, dt, with_bias):
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("m,d", [(37, 5120), (2051, 2568), (5, 4096), (9, 8192), (3, 5128)])
+def test_geglu_int8_wide_rows(ops, dev, dt, m, d):
+    """Rows of 2561..5120 columns are shared by two wavefronts (row maximum exchanged through LDS); wider ones take the
+    one-wavefront form again.  Row counts that leave wavefront pairs idle in the last trip, widths that leave the second
+    wavefront a ragged or almost empty half, a maximum that sits in either half."""
+    g = rng_t(m + d)
+    x = (torch.randn(m, 2 * d, generator=g) * 1.5)
+    x[0::2, 7] *= 9.0            # row maximum in the first half of the value columns
+    x[1::2, d - 3] *= 9.0        # ... and in the last columns
+    x = x.to(TORCH_DT[dt])
+    bias = (torch.randn(2 * d, generator=g) * 0.1).to(TORCH_DT[dt])
+    pre = (torch.rand(d, generator=g) + 0.5).float()
+    xn, bn = to_np_f32(x), to_np_f32(bias)
+    q, s = ops.geglu_int8_dynamic(x.to(dev), bias.to(dev), pre.to(dev))
+    q_ref, s_ref = O.geglu_int8_dynamic(xn, bn, pre.numpy(), dt)
+    assert np.array_equal(s.cpu().numpy(), s_ref) and np.array_equal(q.cpu().numpy(), q_ref)
+    sc = torch.tensor([0.04], dtype=torch.float32)
+    q2 = ops.geglu_int8(x.to(dev), None, None, sc.to(dev))
+    assert np.array_equal(q2.cpu().numpy(), O.geglu_int8(xn, None, None, sc.numpy(), dt))
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
 def test_geglu_int8_gate_values_outside_the_table(ops, dev, dt):
     """Gate inputs below 2^-12, at the table's two ends, beyond 8, subnormal, infinite and NaN (the HIP kernel looks the gate
     factor up for 2^-12 <= |g| < 8 and uses its constant forms elsewhere), with and without a bias."""
