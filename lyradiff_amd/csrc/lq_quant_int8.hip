@@ -556,7 +556,10 @@ static int launch_geglu(int8_t* dst, float* scale_out, const void* hidden, const
         if (int rc = ensure_gate_table<Tag>(st); rc != LQ_OK) return rc;
         lds = entries * sizeof(unsigned short);
         threads = (lds > 32768 && np <= 10) ? 512 : 256;  // (the 16-pass form needs all 256 registers of a 256-thread workgroup)
-        cap = 256 * (lds > 32768 ? 2 : 8);
+        // one 16-wavefront workgroup per CU instead of two of eight halves the table traffic; it pays when every CU gets
+        // a full workgroup of whole rows (17.2 against 18.1 us at 4096 x 2560) and costs when rows are few or shared
+        if (threads == 512 && sw == 1 && np <= 5 && rows >= 256 * 16) threads = 1024;
+        cap = 256 * (lds > 32768 ? (threads == 1024 ? 1 : 2) : 8);
     }
     const size_t rows_per_wg = threads / 64 / sw;
     size_t blocks = (rows + rows_per_wg - 1) / rows_per_wg;
@@ -570,8 +573,9 @@ static int launch_geglu(int8_t* dst, float* scale_out, const void* hidden, const
     } while (0)
 #define LQ_GG_GO(NPV, SWV)                                                                                               \
     do {                                                                                                                 \
-        auto kern = threads == 512 ? geglu_int8_kernel<Tag, NPV, DYNAMIC, (NPV <= 10 ? 512 : 256), SWV>                  \
-                                   : geglu_int8_kernel<Tag, NPV, DYNAMIC, 256, SWV>;                                     \
+        auto kern = threads == 1024 ? geglu_int8_kernel<Tag, NPV, DYNAMIC, (NPV <= 5 ? 1024 : 256), SWV>                 \
+                    : threads == 512 ? geglu_int8_kernel<Tag, NPV, DYNAMIC, (NPV <= 10 ? 512 : 256), SWV>                \
+                                     : geglu_int8_kernel<Tag, NPV, DYNAMIC, 256, SWV>;                                   \
         static bool raised = false; /* raising the dynamic LDS limit is idempotent; a race only repeats it */           \
         if (lds > 48 * 1024 && !raised) {                                                                                \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
