@@ -15,7 +15,8 @@ Inputs and (pre-quantised, rows32-repacked) weights are resident in HBM before t
 `value` is the GEMM work of the step (2*M*N*K summed over both GEMMs) divided by the wall time of
 the whole step, quant kernels included.  The JSON line also carries:
   roofline      the dominant kernel (up-projection FP8 GEMM) priced against the dense FP8 MFMA peak
-                from HIP-event timings taken inside the timed steps, on the launch stream;
+                from HIP-event timings taken inside the timed steps, on the launch stream (every
+                --event-every-th step carries the markers: they are not free, see --help);
   cpu_baseline  the same math (dequantise e4m3 -> fp32 matmul -> scale/bias/GELU) through PyTorch
                 CPU on the host cores (oracle port; a reported baseline only);
   kernels       per-kernel averages of the same timed steps (GEMM TFLOP/s, act-quant GB/s);
@@ -85,6 +86,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=M)
     ap.add_argument("--extra", action="store_true", help="also time the INT8 / W4A4 / SDXL-shape kernels")
+    ap.add_argument("--event-every", type=int, default=5,
+                    help="bracket every kernel with HIP events on every N-th timed step; the five markers of such a step "
+                         "cost the GPU 15-20 us (387-393 us per step with N=1, 370-373 us with none), so the per-kernel "
+                         "figures come from a sample of the timed steps")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path shards by token rows without "
@@ -151,7 +156,7 @@ def main():
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        y = step(i, record=True)
+        y = step(i, record=(i % max(1, args.event_every) == 0))
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
 
@@ -183,6 +188,7 @@ def main():
                                "-> act-quant -> GEMM 12288->3072 (+bias), bf16 in/out (BASELINE.json configs[2])",
                    "tokens": M, "d_model": D, "d_ff": H, "profiled_tactics": tactics},
         "roofline": roofline, "kernels": kernels,
+        "kernel_timing": f"HIP events around each kernel on {len(marks)} of the {args.steps} timed steps",
     }
     if not args.no_cpu:
         cb, y_cpu = cpu_baseline(torch, x, w_up, w_dn, b_up, b_dn, args.cpu_rows)
