@@ -576,7 +576,8 @@ static int launch_geglu(int8_t* dst, float* scale_out, const void* hidden, const
         auto kern = threads == 1024 ? geglu_int8_kernel<Tag, NPV, DYNAMIC, (NPV <= 5 ? 1024 : 256), SWV>                 \
                     : threads == 512 ? geglu_int8_kernel<Tag, NPV, DYNAMIC, (NPV <= 10 ? 512 : 256), SWV>                \
                                      : geglu_int8_kernel<Tag, NPV, DYNAMIC, 256, SWV>;                                   \
-        static bool raised = false; /* raising the dynamic LDS limit is idempotent; a race only repeats it */           \
+        static bool raised_by_size[3] = {false, false, false}; /* one flag per kernel; idempotent, a race only repeats it */ \
+        bool& raised = raised_by_size[threads == 1024 ? 2 : threads == 512 ? 1 : 0];                                     \
         if (lds > 48 * 1024 && !raised) {                                                                                \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
             if (e != hipSuccess) {                                                                                       \
