@@ -146,85 +146,104 @@ __global__ __launch_bounds__(256) void sq_quant_rows_kernel(int8_t* __restrict__
 // registers whatever the row length, so eight of them share a SIMD and the loads of one overlap the
 // arithmetic of the others; the dynamic variant exchanges the span maxima through LDS (one barrier).
 // A lane outside the row re-reads a valid octet (harmless for the maximum) and stores nothing.
-template <typename Tag, int MODE, bool HAS_PRE>
+template <typename Tag, int MODE, bool HAS_PRE, int R>
 __global__ __launch_bounds__(1024) void sq_quant_split_kernel(int8_t* __restrict__ dst, float* __restrict__ scale_out,
                                                               const void* __restrict__ src,
                                                               const float* __restrict__ pre,
-                                                              const float* __restrict__ in_scale, int dim) {
-    __shared__ __attribute__((aligned(16))) float red[16];
+                                                              const float* __restrict__ in_scale, size_t rows, int dim) {
+    // R rows per workgroup (1 or 2): with two, a wavefront's share of the smoothing vector -- twice the bytes of its share
+    // of an fp16 row -- is loaded once for both rows.
+    __shared__ __attribute__((aligned(16))) float red[R][16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const size_t row = blockIdx.x;
-    const char* rb = static_cast<const char*>(src) + row * (size_t)dim * Elem<Tag>::bytes;
+    const size_t row0 = (size_t)blockIdx.x * R;
     if constexpr (MODE == 2) {
-        if (threadIdx.x < 16) red[threadIdx.x] = 0.0f;
+        if (threadIdx.x < 16 * R) red[threadIdx.x / 16][threadIdx.x % 16] = 0.0f;
         __syncthreads();
     }
     constexpr bool kMix = HAS_PRE && std::is_same<Tag, F16Tag>::value;  // fp16 * fp32 in one instruction
     int col[2];
     bool valid[2];
-    float t[2][8];
-    uint4 raw[2];
-    float amax = 0.0f;
+    bool live[R];
+    float t[R][2][8];
+    uint4 raw[R][2];
+    float amax[R];
 #pragma unroll
-    for (int p = 0; p < 2; ++p) {
-        const int c = wave * 1024 + p * 512 + lane * 8;
-        valid[p] = c < dim;
-        col[p] = valid[p] ? c : 0;
-        if constexpr (kMix) raw[p] = *reinterpret_cast<const uint4*>(rb + (size_t)col[p] * 2);
-        else load8<Tag>(rb, col[p], t[p]);
+    for (int rr = 0; rr < R; ++rr) {
+        live[rr] = row0 + rr < rows;  // the last workgroup of an odd row count repeats its first row (stores masked)
+        const char* rb = static_cast<const char*>(src) + (live[rr] ? row0 + rr : row0) * (size_t)dim * Elem<Tag>::bytes;
+        amax[rr] = 0.0f;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const int c = wave * 1024 + p * 512 + lane * 8;
+            valid[p] = c < dim;
+            col[p] = valid[p] ? c : 0;
+            if constexpr (kMix) raw[rr][p] = *reinterpret_cast<const uint4*>(rb + (size_t)col[p] * 2);
+            else load8<Tag>(rb, col[p], t[rr][p]);
+        }
     }
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
-        if constexpr (HAS_PRE) {
-            float pv[8];
-            load8<F32Tag>(pre, col[p], pv);
-            if constexpr (kMix) mul8_f16(raw[p], pv, t[p]);
-            else {
+        float pv[8];
+        if constexpr (HAS_PRE) load8<F32Tag>(pre, col[p], pv);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) t[p][i] = t[p][i] * pv[i];
+        for (int rr = 0; rr < R; ++rr) {
+            if constexpr (HAS_PRE) {
+                if constexpr (kMix) mul8_f16(raw[rr][p], pv, t[rr][p]);
+                else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) t[rr][p][i] = t[rr][p][i] * pv[i];
+                }
+            }
+            if constexpr (MODE == 2) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) amax[rr] = fmaxf(amax[rr], fabsf(t[rr][p][i]));
             }
         }
-        if constexpr (MODE == 2) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(t[p][i]));
-        }
     }
-    float s;
+    float s[R];
     if constexpr (MODE == 2) {
-        amax = wave_max(amax);
-        if (lane == 0) red[wave] = amax;
-        __syncthreads();
-        const float4 a = *reinterpret_cast<const float4*>(red);
-        amax = fmaxf(fmaxf(a.x, a.y), fmaxf(a.z, a.w));
-        if (blockDim.x > 256) {  // more than four wavefronts (the same for the whole workgroup)
-            const float4 b = *reinterpret_cast<const float4*>(red + 4), c = *reinterpret_cast<const float4*>(red + 8);
-            const float4 d = *reinterpret_cast<const float4*>(red + 12);
-            amax = fmaxf(fmaxf(amax, fmaxf(fmaxf(b.x, b.y), fmaxf(b.z, b.w))),
-                         fmaxf(fmaxf(fmaxf(c.x, c.y), fmaxf(c.z, c.w)), fmaxf(fmaxf(d.x, d.y), fmaxf(d.z, d.w))));
-        }
-        s = div_by_const_fast(amax, 127.0f, 0x1.020408p-7f);
-        if (scale_out_of_range(s)) s = amax / 127.0f;
-        if (amax <= 5.9604644775390625e-08f) s = 1.0f;
-        if (threadIdx.x == 0) scale_out[row] = s;
-    } else if constexpr (MODE == 1) {
-        s = in_scale[row];
-    } else {
-        s = in_scale[0];
-    }
-    const float r = fast_recip(s);
-    const bool slow = scale_out_of_range(s);
-    int8_t* ob = dst + row * (size_t)dim;
 #pragma unroll
-    for (int p = 0; p < 2; ++p) {
-        uint2 o;
-        if constexpr (MODE == 2) o = quant8_pack_unclamped(t[p], s, r, slow);
-        else {
-            int q[8];
-            quant8<-128, 127>(t[p], s, r, slow, q);
-            o.x = pack4_s8(q[0], q[1], q[2], q[3]);
-            o.y = pack4_s8(q[4], q[5], q[6], q[7]);
+        for (int rr = 0; rr < R; ++rr) {
+            amax[rr] = wave_max(amax[rr]);
+            if (lane == 0) red[rr][wave] = amax[rr];
         }
-        if (valid[p]) *reinterpret_cast<uint2*>(ob + col[p]) = o;
+        __syncthreads();
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            const float4 a = *reinterpret_cast<const float4*>(red[rr]);
+            float m = fmaxf(fmaxf(a.x, a.y), fmaxf(a.z, a.w));
+            if (blockDim.x > 256) {  // more than four wavefronts (the same for the whole workgroup)
+                const float4 b = *reinterpret_cast<const float4*>(red[rr] + 4), c = *reinterpret_cast<const float4*>(red[rr] + 8);
+                const float4 d = *reinterpret_cast<const float4*>(red[rr] + 12);
+                m = fmaxf(fmaxf(m, fmaxf(fmaxf(b.x, b.y), fmaxf(b.z, b.w))),
+                          fmaxf(fmaxf(fmaxf(c.x, c.y), fmaxf(c.z, c.w)), fmaxf(fmaxf(d.x, d.y), fmaxf(d.z, d.w))));
+            }
+            s[rr] = div_by_const_fast(m, 127.0f, 0x1.020408p-7f);
+            if (scale_out_of_range(s[rr])) s[rr] = m / 127.0f;
+            if (m <= 5.9604644775390625e-08f) s[rr] = 1.0f;
+            if (threadIdx.x == 0 && live[rr]) scale_out[row0 + rr] = s[rr];
+        }
+    } else {
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) s[rr] = MODE == 1 ? in_scale[live[rr] ? row0 + rr : row0] : in_scale[0];
+    }
+#pragma unroll
+    for (int rr = 0; rr < R; ++rr) {
+        const float r = fast_recip(s[rr]);
+        const bool slow = scale_out_of_range(s[rr]);
+        int8_t* ob = dst + (row0 + rr) * (size_t)dim;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            uint2 o;
+            if constexpr (MODE == 2) o = quant8_pack_unclamped(t[rr][p], s[rr], r, slow);
+            else {
+                int q[8];
+                quant8<-128, 127>(t[rr][p], s[rr], r, slow, q);
+                o.x = pack4_s8(q[0], q[1], q[2], q[3]);
+                o.y = pack4_s8(q[4], q[5], q[6], q[7]);
+            }
+            if (valid[p] && live[rr]) *reinterpret_cast<uint2*>(ob + col[p]) = o;
+        }
     }
 }
 
@@ -282,9 +301,15 @@ static int launch_sq_quant(int8_t* dst, float* scale_out, const void* src, const
     if (np > 3) {
         // one wavefront per 1024 columns, one workgroup per row
         LQ_REQUIRE(rows <= 0x7fffffffu, LQ_ERR_SHAPE, "sq_quant: %zu rows exceed the launch limit", rows);
-        dim3 grid((unsigned)rows), block(64 * ((np + 1) / 2));
-        if (pre) hipLaunchKernelGGL((sq_quant_split_kernel<Tag, MODE, true>), grid, block, 0, st, dst, scale_out, src, pre, in_scale, d);
-        else hipLaunchKernelGGL((sq_quant_split_kernel<Tag, MODE, false>), grid, block, 0, st, dst, scale_out, src, pre, in_scale, d);
+        dim3 block(64 * ((np + 1) / 2));
+        if (pre && dim >= 2048) {  // long rows with a smoothing vector: two rows per workgroup share its loads
+            dim3 grid((unsigned)((rows + 1) / 2));
+            hipLaunchKernelGGL((sq_quant_split_kernel<Tag, MODE, true, 2>), grid, block, 0, st, dst, scale_out, src, pre, in_scale, rows, d);
+        } else {
+            dim3 grid((unsigned)rows);
+            if (pre) hipLaunchKernelGGL((sq_quant_split_kernel<Tag, MODE, true, 1>), grid, block, 0, st, dst, scale_out, src, pre, in_scale, rows, d);
+            else hipLaunchKernelGGL((sq_quant_split_kernel<Tag, MODE, false, 1>), grid, block, 0, st, dst, scale_out, src, pre, in_scale, rows, d);
+        }
         return check_launch("sq_quant_split");
     }
     // four rows per workgroup pass; more rows per wavefront only when there are plenty of rows
