@@ -350,6 +350,9 @@ __global__ __launch_bounds__(256) void sq_dequant_kernel(void* __restrict__ dst,
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         size_t r = i / dim, c = i - r * dim;
         float y = ((float)src[i] * in_scale[PER_TOKEN ? r : 0]) * w_scale[c];
+        // pin the fp32 product: otherwise the second multiply and the conversion become one mixed-precision
+        // instruction that rounds the exact product straight to fp16 (one rounding instead of the specified two)
+        asm volatile("" : "+v"(y));
         u32 b = Elem<Tag>::store(y);
         if constexpr (Elem<Tag>::bytes == 2) static_cast<unsigned short*>(dst)[i] = (unsigned short)b;
         else static_cast<u32*>(dst)[i] = b;

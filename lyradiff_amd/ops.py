@@ -116,6 +116,12 @@ def sq_dequant(acc, input_quant_scale, weight_quant_scale, per_token: bool = Fal
     _chk(weight_quant_scale, "weight_quant_scale", (torch.float32,))
     n = acc.shape[-1]
     rows = acc.numel() // n if n else 0
+    if weight_quant_scale.numel() != n:
+        raise ValueError("weight_quant_scale must have N elements")
+    if input_quant_scale.numel() < (rows if per_token else 1):
+        raise ValueError("input_quant_scale must have one element per row when per_token, at least one otherwise")
+    if out_dtype not in _FLOATS:
+        raise TypeError("out_dtype must be float16, bfloat16 or float32")
     y = torch.empty(acc.shape, dtype=out_dtype, device=acc.device)
     _l.check(_l.load().lq_sq_output_dequant(_ptr(y), _DT[out_dtype], _ptr(acc), _ptr(input_quant_scale),
                                             _ptr(weight_quant_scale), int(per_token), rows, n, _stream()),
@@ -128,7 +134,11 @@ def int8_weight_quant(w, pre_quant_scale=None):
     _chk(w, "w", _FLOATS)
     if pre_quant_scale is not None:
         _chk(pre_quant_scale, "pre_quant_scale", (torch.float32,))
+    if w.dim() != 2:
+        raise ValueError("w must be a matrix [N, K]")
     n, k = w.shape
+    if pre_quant_scale is not None and pre_quant_scale.numel() != k:
+        raise ValueError("pre_quant_scale must have K elements")
     q = torch.empty((n, k), dtype=torch.int8, device=w.device)
     s = torch.empty(n, dtype=torch.float32, device=w.device)
     _l.check(_l.load().lq_int8_weight_quant(_ptr(s), _ptr(q), _ptr(w), _DT[w.dtype], _ptr(pre_quant_scale), n, k,

@@ -80,6 +80,53 @@ int main() {
         }
     }
     std::printf("int8 path (invokeSqDynamicPerTokenQuant + runGemmInt8): %d mismatches\n", bad);
+    // ---------------- INT8 loader route: invokeGetINT8WeightScale, then the unfused invokeSqOutputDequant -------------
+    std::vector<__half> hwf(n * k);
+    std::vector<float> fwf(n * k);
+    for (int i = 0; i < n * k; ++i) { hwf[i] = __float2half(0.2f * lcg(seed)); fwf[i] = __half2float(hwf[i]); }
+    for (int j = 0; j < k; ++j) { hwf[5 * k + j] = __float2half(0.0f); fwf[5 * k + j] = 0.0f; }  // a zero row: scale 0, codes 0
+    __half *dwf, *ddq;
+    int8_t* dwq;
+    float* dwqs;
+    int32_t* dacc;
+    CK(hipMalloc(&dwf, n * k * 2)); CK(hipMalloc(&dwq, n * k)); CK(hipMalloc(&dwqs, n * 4));
+    CK(hipMalloc(&dacc, m * n * 4)); CK(hipMalloc(&ddq, m * n * 2));
+    CK(hipMemcpy(dwf, hwf.data(), n * k * 2, hipMemcpyHostToDevice));
+    std::vector<int32_t> hacc(m * n);
+    for (int i = 0; i < m * n; ++i) hacc[i] = (int32_t)(6.0e6f * lcg(seed));
+    CK(hipMemcpy(dacc, hacc.data(), m * n * 4, hipMemcpyHostToDevice));
+    try {
+        invokeGetINT8WeightScale<__half>(dwqs, dwq, dwf, dpre, n, k, st);
+        invokeSqOutputDequant<__half>(ddq, dacc, dscale, dws, QuantMode::useSmoothQuant(true, true), 1, m, n, st);
+    } catch (const std::exception& e) {
+        std::printf("exception: %s\n", e.what());
+        return 3;
+    }
+    CK(hipStreamSynchronize(st));
+    std::vector<int8_t> hwq(n * k);
+    std::vector<float> hwqs(n);
+    std::vector<__half> hdq(m * n);
+    CK(hipMemcpy(hwq.data(), dwq, n * k, hipMemcpyDeviceToHost));
+    CK(hipMemcpy(hwqs.data(), dwqs, n * 4, hipMemcpyDeviceToHost));
+    CK(hipMemcpy(hdq.data(), ddq, m * n * 2, hipMemcpyDeviceToHost));
+    int badw = 0;
+    for (int i = 0; i < n; ++i) {
+        float amax = 0.f;
+        for (int j = 0; j < k; ++j) amax = std::fmax(amax, std::fabs(fwf[i * k + j] / pre[j]));
+        float s = amax / 127.0f;
+        if (s != hwqs[i]) ++badw;
+        for (int j = 0; j < k; ++j) {
+            float r = std::rint((fwf[i * k + j] / pre[j]) / s);
+            int want = std::isnan(r) ? 0 : (int)std::fmin(std::fmax(r, -128.f), 127.f);
+            if (want != (int)hwq[i * k + j]) ++badw;
+        }
+    }
+    for (int i = 0; i < m; ++i)
+        for (int j = 0; j < n; ++j) {
+            float y = ((float)hacc[i * n + j] * hs[i]) * wscale[j];
+            if (__half2float(__float2half(y)) != __half2float(hdq[i * n + j])) ++badw;
+        }
+    std::printf("int8 loader route (invokeGetINT8WeightScale + invokeSqOutputDequant): %d mismatches\n", badw);
     // ---------------- FP8: weight scale + cast + GemmWithResidualAndBias (bf16 out) ----------------------
     std::vector<hip_bfloat16> bx(m * k), bw(n * k);
     std::vector<float> fbx(m * k), fbw(n * k);
@@ -127,5 +174,5 @@ int main() {
         threw = std::string(e.what()).find("[lyradiff Error]") == 0;
     }
     std::printf("bad shape raises std::runtime_error with the reference's prefix: %s\n", threw ? "yes" : "no");
-    return (bad == 0 && bad8 == 0 && threw) ? 0 : 1;
+    return (bad == 0 && badw == 0 && bad8 == 0 && threw) ? 0 : 1;
 }

@@ -1,0 +1,92 @@
+"""Records what MI355X's FP8 matrix instruction returns for single-step (K = 64) products, through the library's own
+FP8 GEMM with unit scales and fp32 output (one v_mfma_f32_32x32x64_f8f6f4 per output, accumulator starting at zero),
+plus two-step (K = 128) cases for the accumulation between steps.  Run on the GPU box:
+
+    python tests/golden/record_mfma_fp8.py gpurun_out/mfma_fp8_recorded.npz
+
+The result is committed as tests/golden/mfma_fp8_recorded.npz; tests/test_oracle_pins.py checks oracle.fp8_mfma_dot_model
+against it on the CPU.  Inputs are seeded, so a re-run reproduces the file."""
+import os
+import sys
+
+import numpy as np
+import torch
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))))
+from lyradiff_amd import ops  # noqa: E402
+from oracle import oracle as O  # noqa: E402
+
+
+def hw(a, b):
+    dev = torch.device("cuda:0")
+    qa, qb = O.e4m3_encode(a), O.e4m3_encode(b)
+    assert np.array_equal(O.e4m3_decode(qa), a) and np.array_equal(O.e4m3_decode(qb), b), "operands must be e4m3 numbers"
+    one = torch.ones(1, dtype=torch.float32, device=dev)
+    y = ops.fp8_linear(torch.from_numpy(qa).to(dev), ops.repack_weight(torch.from_numpy(qb).to(dev)), one, one, None, False,
+                       None, 0.0, torch.float32)
+    return y.cpu().numpy()
+
+
+def cases():
+    rng = np.random.default_rng(20250)
+    out = {}
+    for spread in (0, 4, 8):  # random signs and mantissas, exponents spread over 2^(+-spread)
+        x = rng.standard_normal((32, 64)) * np.exp2(rng.integers(-spread, spread + 1, (32, 64)))
+        w = rng.standard_normal((32, 64)) * np.exp2(rng.integers(-spread, spread + 1, (32, 64)))
+        out[f"rand{spread}"] = (O.e4m3_decode(O.e4m3_encode(np.clip(x, -448, 448).astype(np.float32))),
+                                O.e4m3_decode(O.e4m3_encode(np.clip(w, -448, 448).astype(np.float32))))
+    # one large product at k = p, one small product 2^(8-j) (row j) at k = q: where does the small one stop counting?
+    for p, q in ((0, 1), (3, 4), (7, 8), (0, 63), (15, 16)):
+        a = np.zeros((32, 64), np.float32)
+        b = np.ones((32, 64), np.float32)
+        a[:, p] = 256.0
+        for j in range(32):
+            a[j, q] = 2.0 ** max(-9, 8 - j)
+        out[f"big{p}_small{q}"] = (a, b)
+    # truncation, not rounding: small = mantissa * 2^(8-j), both signs
+    for name, mant in (("m175", 1.75), ("m125", 1.25), ("neg175", -1.75)):
+        a = np.zeros((32, 64), np.float32)
+        b = np.ones((32, 64), np.float32)
+        a[:, 0] = 256.0
+        for j in range(32):
+            a[j, 1] = mant * 2.0 ** max(-6, 8 - j)
+        out[f"trunc_{name}"] = (a, b)
+    # 63 equal small products next to one large one
+    a = np.zeros((32, 64), np.float32)
+    b = np.ones((32, 64), np.float32)
+    a[:, 0] = 256.0
+    for j in range(32):
+        a[j, 1:] = 2.0 ** max(-9, 8 - j)
+    out["big_plus_63_small"] = (a, b)
+    # the exponent that aligns a group is the sum of the operands' exponents, not the product's: 1.5 * 1.5 = 2.25
+    a = np.zeros((32, 64), np.float32)
+    b = np.ones((32, 64), np.float32)
+    a[:, 0] = 1.5 * 128.0
+    b[:, 0] = 1.5
+    for j in range(32):
+        a[j, 1] = 2.0 ** max(-9, 8 - j)
+    out["mantissa_carry"] = (a, b)
+    # subnormal operands
+    a = np.zeros((32, 64), np.float32)
+    b = np.ones((32, 64), np.float32)
+    a[:, 0] = 2.0 ** -9 * np.arange(1, 33).clip(1, 7)
+    b[:, 0] = 2.0 ** -9 * 3
+    a[:, 1] = 2.0 ** -7
+    b[:, 1] = 2.0 ** -6
+    out["subnormal"] = (a, b)
+    # two steps (K = 128): accumulation of the second step onto the first
+    for spread in (4, 8):
+        x = rng.standard_normal((32, 128)) * np.exp2(rng.integers(-spread, spread + 1, (32, 128)))
+        w = rng.standard_normal((32, 128)) * np.exp2(rng.integers(-spread, spread + 1, (32, 128)))
+        out[f"rand{spread}_k128"] = (O.e4m3_decode(O.e4m3_encode(np.clip(x, -448, 448).astype(np.float32))),
+                                     O.e4m3_decode(O.e4m3_encode(np.clip(w, -448, 448).astype(np.float32))))
+    return out
+
+
+if __name__ == "__main__":
+    dst = sys.argv[1] if len(sys.argv) > 1 else "gpurun_out/mfma_fp8_recorded.npz"
+    rec = {}
+    for name, (a, b) in cases().items():
+        rec[name + "__a"], rec[name + "__b"], rec[name + "__y"] = O.e4m3_encode(a), O.e4m3_encode(b), hw(a, b)
+    np.savez_compressed(dst, **rec)
+    print("wrote", dst, len(rec) // 3, "cases")

@@ -270,3 +270,101 @@ def test_golden_vectors_on_gpu(ops, dev):
     # rows32 repack
     p = ops.repack_weight(torch.from_numpy(G["rows32_src"]).to(dev))
     assert np.array_equal(p.cpu().numpy().reshape(-1), G["rows32_dst"])
+
+
+# ---- per-output-channel weight quantisation on the device (invokeGetINT8WeightScale, quant_kernels.cu:173-223,270-312) ---
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("with_pre", [True, False])
+@pytest.mark.parametrize("n,k", [(1280, 1280), (640, 2560), (33, 8), (5, 4099)])
+def test_int8_weight_quant_device(ops, dev, dt, with_pre, n, k):
+    g = rng_t(300 + n + k)
+    w = (torch.randn(n, k, generator=g) * 0.05).to(TORCH_DT[dt])
+    w[n // 2] = 0  # zero row: amax 0, scale 0, 0/0 = NaN -> code 0
+    w[1, k - 1] = -w[1].abs().max() * 2  # the row maximum on a negative element: -127, never -128
+    pre = (torch.rand(k, generator=g) * 2.7 + 0.3).float() if with_pre else None
+    q, s = ops.int8_weight_quant(w.to(dev), None if pre is None else pre.to(dev))
+    q_ref, s_ref = O.int8_weight_quant_device(to_np_f32(w), None if pre is None else pre.numpy())
+    assert np.array_equal(s.cpu().numpy(), s_ref)
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+    assert s_ref[n // 2] == 0.0 and not q_ref[n // 2].any()
+    assert np.array_equal(np.abs(q_ref[np.arange(n) != n // 2].astype(np.int32)).max(axis=1), np.full(n - 1, 127))
+    if not with_pre:
+        assert q_ref[1, k - 1] == -127
+
+
+def test_int8_weight_quant_device_specials_and_many_rows(ops, dev):
+    """NaN never enters the row maximum and quantises to 0, an infinity makes the scale infinite (finite/inf = 0,
+    inf/inf = NaN -> 0), an all-NaN row has scale 0; more rows than one grid dimension holds (d_out > 65535)."""
+    k = 72
+    w = torch.randn(70001, k, generator=rng_t(12))
+    w[0, 3] = float("nan")
+    w[1, 5] = float("inf")
+    w[2, :] = float("nan")
+    w[3, 6] = float("-inf"); w[3, 9] = float("nan")
+    w[70000, k - 1] = 1e30
+    pre = (torch.rand(k, generator=rng_t(13)) + 0.5).float()
+    for p in (None, pre):
+        q, s = ops.int8_weight_quant(w.to(dev), None if p is None else p.to(dev))
+        with np.errstate(invalid="ignore"):
+            q_ref, s_ref = O.int8_weight_quant_device(w.numpy(), None if p is None else p.numpy())
+        assert np.array_equal(s.cpu().numpy(), s_ref, equal_nan=True)
+        assert np.array_equal(q.cpu().numpy(), q_ref)
+    assert np.isinf(s_ref[1]) and not q_ref[1].any() and s_ref[2] == 0.0 and not q_ref[2].any()
+    with pytest.raises(ValueError):
+        ops.int8_weight_quant(w[:4].to(dev), pre[:8].to(dev))
+
+
+def test_int8_weight_quant_feeds_the_gemm(ops, dev):
+    """The reference's loader path: fp16 weight -> device quantiser (dividing by pre_quant_scale) -> INT8 GEMM with the
+    per-channel scales it produced (layers/basic_transformer/BasicTransformerInt8BlockWeight.cc, quant_kernels.cu:270-312)."""
+    m, n, k = 96, 320, 640
+    g = rng_t(77)
+    x = make_outlier_acts(m, k, 6, 15.0, torch.float16, 78)
+    w = (torch.randn(n, k, generator=g) * 0.03).half()
+    pre = (torch.rand(k, generator=g) * 1.5 + 0.5).float()
+    qw, sw = ops.int8_weight_quant(w.to(dev), pre.to(dev))
+    qx, sx = ops.sq_quant_dynamic(x.to(dev), pre.to(dev))
+    y = ops.int8_linear(qx, ops.repack_weight(qw), sw, sx, None, torch.float16)
+    qw_ref, sw_ref = O.int8_weight_quant_device(to_np_f32(w), pre.numpy())
+    qx_ref, sx_ref = O.sq_dynamic_quant(to_np_f32(x), pre.numpy())
+    y_ref = O.int8_epilogue(O.gemm_i8_acc(qx_ref, qw_ref), sw_ref, sx_ref, None, "f16")
+    assert np.array_equal(to_np_f32(y), y_ref)
+    # and the quantised product approximates the unquantised one: (x*pre) . (w/pre) = x . w
+    full = to_np_f32(x).astype(np.float64) @ to_np_f32(w).astype(np.float64).T
+    assert np.sqrt(((y_ref - full) ** 2).mean()) < 0.08 * np.sqrt((full ** 2).mean())
+
+
+# ---- unfused dequant (invokeSqOutputDequant, quant_kernels.cu:117-171,250-268) -------------------------------------------
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("per_token", [False, True])
+@pytest.mark.parametrize("m,n", [(1024, 1280), (37, 642), (3, 2)])
+def test_sq_output_dequant(ops, dev, dt, per_token, m, n):
+    g = rng_t(500 + m + n)
+    acc = torch.randint(-(2 ** 22), 2 ** 22, (m, n), generator=g, dtype=torch.int32)
+    acc[0, 0] = 2 ** 24 + 1  # not an fp32 number: the int -> float conversion rounds
+    acc[m - 1, n - 1] = -(2 ** 24) - 3
+    s_in = (torch.rand(m if per_token else 1, generator=g) * 4e-2 + 1e-2).float()
+    s_w = (torch.rand(n, generator=g) * 9e-3 + 1e-3).float()
+    y = ops.sq_dequant(acc.to(dev), s_in.to(dev), s_w.to(dev), per_token, TORCH_DT[dt])
+    y_ref = O.sq_output_dequant(acc.numpy(), s_in.numpy(), s_w.numpy(), per_token, dt)
+    assert np.array_equal(to_np_f32(y), y_ref)
+    if dt == "f32":  # the order (acc*s_in)*s_w is visible in fp32: the fused epilogue's (s_w*s_in)*acc differs somewhere
+        other = acc.numpy().astype(np.float32) * (s_w.numpy()[None, :] * (s_in.numpy()[:, None] if per_token else s_in.numpy()[0]))
+        assert m * n < 1000 or (other != y_ref).any()
+    with pytest.raises(ValueError):
+        ops.sq_dequant(acc.to(dev), s_in.to(dev), s_w[:-1].to(dev), per_token, TORCH_DT[dt])
+
+
+def test_int32_gemm_then_unfused_dequant_matches_the_two_step_reference(ops, dev):
+    """cublasMMWrapper's int32-output GEMM followed by invokeSqOutputDequant, the reference's unfused route."""
+    m, n, k = 64, 128, 256
+    g = rng_t(31)
+    a = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int8)
+    w = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8)
+    s_in = (torch.rand(m, generator=g) * 4e-2 + 1e-2).float()
+    s_w = (torch.rand(n, generator=g) * 9e-3 + 1e-3).float()
+    acc = ops.int8_linear(a.to(dev), ops.repack_weight(w.to(dev)), None, None, None, torch.int32)
+    y = ops.sq_dequant(acc, s_in.to(dev), s_w.to(dev), True, torch.float16)
+    acc_ref = O.gemm_i8_acc(a.numpy(), w.numpy())
+    assert np.array_equal(acc.cpu().numpy(), acc_ref)
+    assert np.array_equal(to_np_f32(y), O.sq_output_dequant(acc_ref, s_in.numpy(), s_w.numpy(), True, "f16"))

@@ -6,7 +6,7 @@ import torch
 
 from oracle import oracle as O
 from oracle import oracle_c as OC
-from tests.helpers import assert_close_tol, rng_t, to_np_f32
+from tests.helpers import assert_close_tol, check_fp8_gemm, rng_t, to_np_f32
 
 
 def write_bin(path, t):
@@ -73,8 +73,7 @@ def test_fp8_linear_from_state_dict(dev):
     y = lin.forward(x.to(dev), gelu=True)
     qa = O.fp8_scale_cast(to_np_f32(x), np.float32(0.012), True)
     ref = O.fp8_gemm(qa, qw, 0.012, sw, to_np_f32(sd["blk.net.0.proj.bias"]), True, None, 0.0, "bf16")
-    mag = np.abs(O.e4m3_decode(qa)).astype(np.float64) @ np.abs(O.e4m3_decode(qw)).astype(np.float64).T
-    assert_close_tol(to_np_f32(y), ref, "fp8 linear from state dict", abs_floor=2.0 ** -13 * mag * 0.012 * float(sw) + 2e-6)
+    check_fp8_gemm(to_np_f32(y), ref, qa, qw, 0.012, sw, "bf16", "fp8 linear from state dict", extra_abs=2e-6)
 
 
 @pytest.mark.gpu
@@ -147,9 +146,13 @@ def test_smooth_vector_on_device(dev):
     aw = ops.col_absmax(w.to(dev))
     assert np.array_equal(ax.cpu().numpy(), np.abs(to_np_f32(x)).max(axis=0))
     assert np.array_equal(aw.cpu().numpy(), np.abs(w.numpy()).max(axis=0))
-    pre, s = ops.smooth_vector(ax, aw, 0.5)
-    s_ref = O.smooth_vector(to_np_f32(x), w.numpy(), 0.5)
-    assert np.allclose(s.cpu().numpy(), s_ref, rtol=2e-6) and np.allclose(pre.cpu().numpy(), 1.0 / s_ref, rtol=3e-6)
+    for alpha in (0.8, 0.25, 1.0, 0.0, 0.5):  # 0.8 is the reference's default (convert_sd_quant_model.py:340)
+        pre, s = ops.smooth_vector(ax, aw, alpha)
+        s_ref = O.smooth_vector(to_np_f32(x), w.numpy(), alpha)
+        assert np.allclose(s.cpu().numpy(), s_ref, rtol=2e-6) and np.allclose(pre.cpu().numpy(), 1.0 / s_ref, rtol=3e-6)
+    # hand-computed values at an asymmetric exponent: 16^0.75 / 256^0.25 = 8 / 4 (a swapped exponent gives 2 / 64)
+    p2, s2 = ops.smooth_vector(torch.full((8,), 16.0, device=dev), torch.full((8,), 256.0, device=dev), 0.75)
+    assert np.allclose(s2.cpu().numpy(), 2.0, rtol=2e-6) and np.allclose(p2.cpu().numpy(), 0.5, rtol=2e-6)
     # the vector does its job: the smoothed activation has a flatter column profile
     t = to_np_f32(x) * pre.cpu().numpy()[None, :]
     assert np.abs(t).max(axis=0).max() / np.median(np.abs(t).max(axis=0)) < 0.3 * np.abs(to_np_f32(x)).max(axis=0).max() / np.median(np.abs(to_np_f32(x)).max(axis=0))
