@@ -113,6 +113,20 @@ int lq_fp8_scale_cast(uint8_t* dst, const void* src, lq_dtype_t dtype, const flo
  * those of the two functions above.  Overwrites scale_out (no zero-init needed). */
 int lq_fp8_amax_cast(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t n,
                      lq_stream_t stream);
+/* How lq_fp8_amax_cast runs: normally one launch whose workgroups meet at a grid-wide barrier in statically allocated
+ * device memory; each stream owns one of 16 barrier slots per device (work of one stream runs in order), so calls on
+ * up to 16 streams may be in flight together.  Under stream capture, on further streams and for unaligned buffers it
+ * runs three scratch-free kernels instead (zero the scale, atomic-max pass, cast pass).  The barrier assumes the grid
+ * becomes resident; when kernels of OTHER streams hold the device for longer than its bounded wait (~0.1 s), the
+ * launch gives up, writes a NaN scale and raises a flag:
+ * lq_fp8_amax_cast_status() returns 0 if no such time-out happened on the current device since the last call, 1 if
+ * one did (flag cleared; lq_last_error() explains), negative on a HIP error.  It copies 4 bytes from the device and
+ * therefore waits for the null stream; call it after synchronising the streams that quantised.  No reference
+ * counterpart. */
+int lq_fp8_amax_cast_status(void);
+/* The barrier slot (0..15) `stream` owns on the current device, assigned on first use; -1 when all 16 are taken (calls
+ * on that stream then run the scratch-free kernels); negative status on a HIP error.  For diagnostics and tests. */
+int lq_fp8_amax_cast_slot(lq_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * W4A4 group-wise INT4 activation quantisation

@@ -8,6 +8,7 @@
 // the cast kernel moves 32 B in / 16 B out per lane per step.
 #include "lq_common.h"
 #include <atomic>
+#include <mutex>
 
 namespace lq {
 
@@ -166,62 +167,129 @@ __global__ __launch_bounds__(256) void fp8_amax_scalar_kernel(float* __restrict_
 
 __global__ void fill_f32_kernel(float* p, float v) { p[0] = v; }
 
+// ---- device scratch of the dynamic (amax + cast) quantiser --------------------------------------------------------
+// One statically allocated block per GPU (each device that loads this library holds its own copy until the process
+// ends): the time-out flag and the barrier slots of the one-launch kernel.  Static device memory starts zeroed, and
+// every launch leaves its counters at zero again.
+// Host code never uses the array's name as an address: device_scratch() asks the runtime for the device address once
+// per device (hipGetSymbolAddress) and the kernels receive that pointer as an argument.
+constexpr int kCoopThreads = 512;
+constexpr int kCoopMaxBlocks = 1024;
+constexpr int kCoopSlots = 16;
+struct CounterLine {  // one counter per 128-byte line: polls of one word must not queue behind atomics on another
+    unsigned count;
+    unsigned pad[31];
+};
+struct CoopSlot {
+    CounterLine group[8];
+    CounterLine top;
+    CounterLine flag;
+    float partials[kCoopMaxBlocks];
+};
+struct FusedScratch {
+    unsigned timeout;
+    unsigned pad[63];
+    CoopSlot coop[kCoopSlots];
+};
+static __device__ __align__(256) unsigned char scratch[sizeof(FusedScratch)];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<FusedScratch*> g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device (nullptr, with the error message set, on failure).
+static FusedScratch* device_scratch(int* dev_out = nullptr) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        set_error("fp8 quantiser: cannot identify the current device (%d)", dev);
+        return nullptr;
+    }
+    if (dev_out) *dev_out = dev;
+    FusedScratch* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p) return p;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+    if (p) return p;
+    void* addr = nullptr;
+    hipError_t e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || addr == nullptr) {
+        (void)hipGetLastError();
+        set_error("fp8 quantiser: hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+        return nullptr;
+    }
+    p = static_cast<FusedScratch*>(addr);
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+    return p;
+}
+
+// A stream owns one barrier slot for the life of the process (work of one stream runs in order, so its launches never
+// overlap); streams beyond kCoopSlots get none and use the scratch-free kernel sequence.
+struct StreamSlots {
+    hipStream_t stream[kCoopSlots];
+    int used = 0;
+};
+static StreamSlots g_stream_slots[kMaxDevices];
+static std::mutex g_slot_mutex;
+static int slot_for_stream(int dev, hipStream_t st) {
+    std::lock_guard<std::mutex> lock(g_slot_mutex);
+    StreamSlots& t = g_stream_slots[dev];
+    for (int i = 0; i < t.used; ++i)
+        if (t.stream[i] == st) return i;
+    if (t.used == kCoopSlots) return -1;
+    t.stream[t.used] = st;
+    return t.used++;
+}
+
 // Fused dynamic per-tensor quantisation in ONE launch: every thread keeps up to KEEP 16-element
 // chunks of its slice in registers while the tensor-wide absmax is formed (workgroup partials ->
 // grid-wide barrier -> every workgroup reduces the partials), then casts from registers, so the
 // source is read from HBM once (3 bytes moved per element: the algorithmic minimum).  Chunks
 // beyond KEEP are re-read in the second phase (from L2 / Infinity Cache when they fit).
 //
-// The grid never exceeds what the device holds at once (CUs x resident workgroups), so every
-// workgroup is running when the barrier is reached.  The barrier re-arms itself (safe to replay from
-// a HIP graph); the wait is bounded,
-// so that even a starved grid terminates: on time-out the kernel raises g_amax_timeout and the
-// scale it writes is NaN, which poisons the output visibly instead of hanging the device.
-// Launches that overlap in time must use different slots: the host hands slots out round-robin.
-constexpr int kCoopThreads = 512;
-constexpr int kCoopMaxBlocks = 1024;
-constexpr int kCoopSlots = 16;
-__device__ float g_amax_partials[kCoopSlots][kCoopMaxBlocks];
-__device__ unsigned g_amax_group_count[kCoopSlots][8];
-__device__ unsigned g_amax_top_count[kCoopSlots];
-__device__ unsigned g_amax_flag[kCoopSlots];
-__device__ unsigned g_amax_timeout;
+// The grid never exceeds what the device holds at once (CUs x resident workgroups), so every workgroup is running when
+// the barrier is reached -- provided nothing else occupies the device; when another stream's kernels hold CUs the
+// late workgroups start once those retire, and the wait is bounded so that even a starved grid terminates: on
+// time-out the kernel raises the time-out flag (lq_fp8_amax_cast_status reports it) and the scale it writes is NaN,
+// which poisons the output visibly instead of hanging the device.  The barrier re-arms itself.  Launches that may
+// overlap in time use different slots: a slot belongs to one stream, and the path is not taken under stream capture
+// (a captured launch could later replay on any stream).
 
 // Two-level arrive counter (workgroup ids congruent modulo 8 share a counter, so at most G/8 atomics
 // hit one address; the last arriver of a group bumps the top counter, the last group flips the flag
-// everybody polls).  Counters are cleared by their last arriver, so the barrier re-arms itself and can
-// be replayed from a HIP graph.  Only relaxed device-scope atomics are used for the hand-over -- no
-// release/acquire fences, which on this multi-die part would write back / invalidate whole L2s -- and
-// the partial maxima travel through the same kind of atomics; a workgroup-scope release fence (a plain
-// wait for outstanding memory operations) orders the partial store before the arrival.
+// everybody polls).  Counters are cleared by their last arriver.  Only relaxed device-scope atomics are used for the
+// hand-over -- no release/acquire fences, which on this multi-die part would write back / invalidate whole L2s.  The
+// partial maximum is published with a device-scope atomic store and the thread then waits explicitly (s_waitcnt vmcnt(0):
+// on this architecture stores count in vmcnt) for its acknowledgement before the arrival is counted.
 // Returns false on time-out.
-__device__ __forceinline__ bool grid_barrier(int slot) {
+__device__ __forceinline__ bool grid_barrier(CoopSlot* slot, unsigned* timeout, float partial) {
     __shared__ int ok;
     __syncthreads();
     if (threadIdx.x == 0) {
         const unsigned G = gridDim.x, grp = blockIdx.x & 7;
         const unsigned in_group = (G - grp + 7) / 8, ngroups = G < 8 ? G : 8;
-        const unsigned f0 = __hip_atomic_load(&g_amax_flag[slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        unsigned x = __hip_atomic_fetch_add(&g_amax_group_count[slot][grp], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned f0 = __hip_atomic_load(&slot->flag.count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&slot->partials[blockIdx.x], partial, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the device-scope (write-through) store has been acknowledged
+        unsigned x = __hip_atomic_fetch_add(&slot->group[grp].count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (x == in_group - 1) {
-            __hip_atomic_store(&g_amax_group_count[slot][grp], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            unsigned t = __hip_atomic_fetch_add(&g_amax_top_count[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&slot->group[grp].count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            unsigned t = __hip_atomic_fetch_add(&slot->top.count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (t == ngroups - 1) {
-                __hip_atomic_store(&g_amax_top_count[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                __hip_atomic_store(&g_amax_flag[slot], f0 + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&slot->top.count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // counters are zero again before anyone is released
+                __hip_atomic_store(&slot->flag.count, f0 + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
         int good = 0;
-        for (int spin = 0; spin < (1 << 22); ++spin) {
-            if (__hip_atomic_load(&g_amax_flag[slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != f0) {
+        for (int spin = 0; spin < (1 << 18); ++spin) {
+            if (__hip_atomic_load(&slot->flag.count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != f0) {
                 good = 1;
                 break;
             }
             __builtin_amdgcn_s_sleep(1);
         }
-        if (!good) __hip_atomic_store(&g_amax_timeout, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (!good) __hip_atomic_store(timeout, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         ok = good;
     }
     __syncthreads();
@@ -232,9 +300,9 @@ template <typename Tag, int KEEP>
 __global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_t* __restrict__ dst,
                                                                           float* __restrict__ scale_out,
                                                                           const void* __restrict__ src, size_t n,
-                                                                          int slot) {
+                                                                          CoopSlot* slot, unsigned* timeout) {
     constexpr int E = Chunk16<Tag>::elems;
-    constexpr int V = Elem<Tag>::bytes == 2 ? 2 : 2;  // uint4 vectors per chunk (32 bytes either way)
+    constexpr int V = 2;  // uint4 vectors per chunk (32 bytes for every element type)
     const size_t nchunks = n / E;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -274,13 +342,12 @@ __global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_
     amax = wave_max(amax);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
     __syncthreads();
+    float wg_max = 0.0f;
     if (threadIdx.x == 0) {
-        float m = 0.0f;
 #pragma unroll
-        for (int i = 0; i < kCoopThreads / 64; ++i) m = fmaxf(m, red[i]);
-        __hip_atomic_store(&g_amax_partials[slot][blockIdx.x], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int i = 0; i < kCoopThreads / 64; ++i) wg_max = fmaxf(wg_max, red[i]);
     }
-    const bool arrived = grid_barrier(slot);
+    const bool arrived = grid_barrier(slot, timeout, wg_max);
     // Only the raw 16-byte vectors live across the barrier: the empty asm makes them new values to the compiler, which
     // would otherwise keep the unpacked fp32 copies of the first phase as well (twice the registers, half the occupancy).
 #pragma unroll
@@ -290,7 +357,7 @@ __global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_
             asm volatile("" : "+v"(keep[it][u].x), "+v"(keep[it][u].y), "+v"(keep[it][u].z), "+v"(keep[it][u].w));
     float m = 0.0f;
     for (int i = threadIdx.x; i < (int)gridDim.x; i += kCoopThreads)
-        m = fmaxf(m, __hip_atomic_load(&g_amax_partials[slot][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        m = fmaxf(m, __hip_atomic_load(&slot->partials[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
     m = wave_max(m);
     __syncthreads();
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
@@ -328,10 +395,9 @@ __global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_
     }
 }
 
-static std::atomic<unsigned> g_next_slot{0};  // one round-robin counter for every element type and host thread
-
-// Returns LQ_OK when the fused launch was issued, 1 when the caller should fall back to the
-// three-kernel sequence (unaligned buffers, or the occupancy query failed).
+// Returns LQ_OK when the fused launch was issued, 1 when the caller should fall back to the scratch-free
+// kernel sequence (unaligned buffers, stream capture, no barrier slot left for this stream, occupancy query failed),
+// a negative status on an error.
 // KEEP = 8 chunks of 32 bytes (64 registers) stay in each thread's registers across the barrier: with two workgroups
 // per CU that holds a tensor of up to 33.5 M sixteen-bit elements on 256 CUs; the rest of a larger one is read twice.
 template <typename Tag>
@@ -339,13 +405,23 @@ static int launch_amax_cast_coop(uint8_t* dst, float* scale_out, const void* src
     constexpr int KEEP = 8;
     auto kern = fp8_amax_cast_coop_kernel<Tag, KEEP>;
     if (reinterpret_cast<uintptr_t>(src) % 16 != 0 || reinterpret_cast<uintptr_t>(dst) % 16 != 0) return 1;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return 1;
+    }
+    int dev = 0;
+    FusedScratch* ws = device_scratch(&dev);
+    if (ws == nullptr) return LQ_ERR_HIP;
+    const int slot = slot_for_stream(dev, st);
+    if (slot < 0) return 1;
     struct Capacity { int blocks_per_cu = 0, num_cu = 0; };
     // queried once (thread-safe initialisation of a function-local static)
     static const Capacity cap = [&] {
         Capacity c;
-        int dev = 0, occ = 0;
+        int occ = 0;
         hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+        if (hipGetDeviceProperties(&prop, dev) == hipSuccess &&
             hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, kCoopThreads, 0) == hipSuccess && occ >= 1) {
             c.blocks_per_cu = occ > 2 ? 2 : occ;
             c.num_cu = prop.multiProcessorCount;
@@ -361,8 +437,7 @@ static int launch_amax_cast_coop(uint8_t* dst, float* scale_out, const void* src
     int grid = (need <= (size_t)KEEP * num_cu ? 1 : blocks_per_cu) * num_cu;
     if (grid > kCoopMaxBlocks) grid = kCoopMaxBlocks;
     if ((size_t)grid > need) grid = need ? (int)need : 1;
-    int slot = (int)(g_next_slot.fetch_add(1, std::memory_order_relaxed) % kCoopSlots);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kCoopThreads), 0, st, dst, scale_out, src, n, slot);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kCoopThreads), 0, st, dst, scale_out, src, n, &ws->coop[slot], &ws->timeout);
     return check_launch("fp8_amax_cast_fused");
 }
 
@@ -451,12 +526,42 @@ extern "C" int lq_fp8_amax_cast(uint8_t* dst, float* scale_out, const void* src,
             case LQ_F32: rc = launch_amax_cast_coop<F32Tag>(dst, scale_out, src, n, as_stream(stream)); break;
             default: set_error("lq_fp8_amax_cast: unsupported dtype %d", (int)dtype); return LQ_ERR_UNSUPPORTED;
         }
-        if (rc == LQ_OK) return LQ_OK;
+        if (rc <= 0) return rc;
     }
+    // scratch-free sequence: safe under stream capture and for any number of concurrent streams
     hipLaunchKernelGGL(fill_f32_kernel, dim3(1), dim3(1), 0, as_stream(stream), scale_out, 0.0f);
     int rc = check_launch("fp8_amax_cast(fill)");
     if (rc != LQ_OK || n == 0) return rc;
     rc = lq_fp8_amax_scale(scale_out, src, dtype, n, stream);
     if (rc != LQ_OK) return rc;
     return lq_fp8_scale_cast(dst, src, dtype, scale_out, 1, n, stream);
+}
+
+extern "C" int lq_fp8_amax_cast_slot(lq_stream_t stream) {
+    int dev = 0;
+    if (device_scratch(&dev) == nullptr) return LQ_ERR_HIP;
+    return slot_for_stream(dev, as_stream(stream));
+}
+
+extern "C" int lq_fp8_amax_cast_status(void) {
+    FusedScratch* ws = device_scratch();
+    if (ws == nullptr) return LQ_ERR_HIP;
+    unsigned flag = 0;
+    hipError_t e = hipMemcpy(&flag, &ws->timeout, sizeof(flag), hipMemcpyDeviceToHost);
+    if (e == hipSuccess && flag != 0) {
+        const unsigned zero = 0;
+        e = hipMemcpy(&ws->timeout, &zero, sizeof(zero), hipMemcpyHostToDevice);
+    }
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        set_error("lq_fp8_amax_cast_status: %s", hipGetErrorString(e));
+        return LQ_ERR_HIP;
+    }
+    if (flag != 0) {
+        set_error("lq_fp8_amax_cast: a one-launch quantisation timed out at its grid barrier since the last status call "
+                  "(its scale is NaN); another stream's kernels held the device -- serialise the streams or quantise with "
+                  "lq_fp8_amax_scale + lq_fp8_scale_cast");
+        return 1;
+    }
+    return 0;
 }

@@ -9,7 +9,9 @@ import ctypes as C
 import os
 
 PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.environ.get("LYRA_LIB_PATH_AMD", os.path.join(PKG, "liblyraquant.so"))
+# LYRA_LIB_PATH is the variable the reference's Python wrapper reads (lyradiff/__init__.py:4-5); LYRA_LIB_PATH_AMD wins
+# when both are set (a machine that also carries the reference's CUDA build)
+LIB_PATH = os.environ.get("LYRA_LIB_PATH_AMD") or os.environ.get("LYRA_LIB_PATH") or os.path.join(PKG, "liblyraquant.so")
 
 LQ_F32, LQ_F16, LQ_BF16, LQ_I32 = 0, 1, 2, 3
 LQ_W_INT8, LQ_W_FP8, LQ_W_INT4 = 0, 1, 2
@@ -28,6 +30,8 @@ SYMBOLS = {
     "lq_fp8_amax_scale": (_I, [_P, _P, _I, _Z, _P]),
     "lq_fp8_scale_cast": (_I, [_P, _P, _I, _P, _I, _Z, _P]),
     "lq_fp8_amax_cast": (_I, [_P, _P, _P, _I, _Z, _P]),
+    "lq_fp8_amax_cast_status": (_I, []),
+    "lq_fp8_amax_cast_slot": (_I, [_P]),
     "lq_w4a4_quantize": (_I, [_P, _P, _I, _P, _I, _P, _I, _I, _I, _P]),
     "lq_weight_row_bytes": (_Z, [_I, _Z]),
     "lq_repack_rows32": (_I, [_P, _P, _Z, _Z, _P]),

@@ -314,6 +314,15 @@ def fp8_quant(x):
     return q, s
 
 
+def fp8_amax_cast_status() -> bool:
+    """True when a one-launch fp8_quant on the current device timed out at its grid barrier since the last call (its
+    scale is NaN).  Copies 4 bytes from the device: synchronise the quantising streams first."""
+    rc = _l.load().lq_fp8_amax_cast_status()
+    if rc < 0:
+        _l.check(rc, "lq_fp8_amax_cast_status")
+    return rc == 1
+
+
 # ---- W4A4 ------------------------------------------------------------------------------------------
 
 def w4a4_quant(x, smooth=None, scale_dtype=torch.float32, group: int = 64):

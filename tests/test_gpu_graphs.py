@@ -1,7 +1,8 @@
 """The quantized-linear chains under HIP graph capture: every kernel is stream-ordered and allocation-free, so a chain
 whose buffers come from the graph's private pool can be captured once and replayed.  Replays are interleaved with eager
-work and synchronisations and every replay is compared bit for bit with the eager result (the fused FP8 quantisation
-re-arms its own grid barrier, no memset node is involved)."""
+work and synchronisations and every replay is compared bit for bit with the eager result (under capture the dynamic FP8
+quantiser records its three barrier-free kernels instead of the one-launch kernel with the grid barrier; no memset node is
+involved)."""
 import numpy as np
 import pytest
 import torch

@@ -272,6 +272,37 @@ def test_golden_vectors_on_gpu(ops, dev):
     assert np.array_equal(p.cpu().numpy().reshape(-1), G["rows32_dst"])
 
 
+def test_fp8_amax_cast_stream_slots_fallback_and_status(ops, dev):
+    """The one-launch dynamic quantiser meets at a grid barrier in a slot that belongs to the calling stream; at most 16
+    streams per device get one, the others run the scratch-free kernel sequence.  Both routes give the oracle's codes and
+    scale, and after normal runs the time-out status reads clean."""
+    import ctypes as C
+
+    from lyradiff_amd import lib as L
+
+    lib = L.load()
+    streams = [torch.cuda.Stream() for _ in range(20)]
+    slots = [lib.lq_fp8_amax_cast_slot(C.c_void_p(st.cuda_stream)) for st in streams]
+    assert all(-1 <= v < 16 for v in slots)
+    owned = [v for v in slots if v >= 0]
+    assert len(set(owned)) == len(owned) and slots.count(-1) >= 4  # distinct slots; 20 streams cannot all have one
+    if -1 in slots:
+        assert all(v == -1 for v in slots[slots.index(-1):])  # once they run out they stay out
+    assert [lib.lq_fp8_amax_cast_slot(C.c_void_p(st.cuda_stream)) for st in streams] == slots  # stable per stream
+    x = (torch.randn(300, 1024, generator=rng_t(3)) * 3).bfloat16()
+    q_ref, s_ref = O.fp8_amax_cast(to_np_f32(x))
+    xd = x.to(dev)
+    torch.cuda.synchronize()
+    outs = []
+    for st in (streams[0], streams[-1]):  # one with a slot (unless earlier tests used them up), one without
+        with torch.cuda.stream(st):
+            outs.append(ops.fp8_quant(xd))
+    torch.cuda.synchronize()
+    for q, s in outs:
+        assert s.item() == float(s_ref) and np.array_equal(q.cpu().numpy(), q_ref)
+    assert ops.fp8_amax_cast_status() is False
+
+
 # ---- per-output-channel weight quantisation on the device (invokeGetINT8WeightScale, quant_kernels.cu:173-223,270-312) ---
 @pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("with_pre", [True, False])
