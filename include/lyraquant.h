@@ -128,6 +128,19 @@ int lq_fp8_amax_cast_status(void);
  * on that stream then run the scratch-free kernels); negative status on a HIP error.  For diagnostics and tests. */
 int lq_fp8_amax_cast_slot(lq_stream_t stream);
 
+/* lq_fp8_amax_cast for callers that cannot allocate or tolerate a kernel that waits: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Two launches, no barrier:
+ * a partial-maximum pass whose workgroups leave their maxima and a ticket counter in a static device array
+ * (119 KiB per GPU, held until the process ends; its address is looked up once per device on first use) -- the
+ * workgroup drawing the last ticket writes scale_out[0] = max|x| / 448 and re-arms the counter -- then the cast pass.
+ * Same results as lq_fp8_amax_cast, bit for bit.  Calls no allocating routine.  n from 1 to
+ * lq_fp8_amax_cast_static_max_elems() (2^28: 8192 partial maxima of 32768 elements), src and dst 16-byte aligned;
+ * anything else is rejected with LQ_ERR_SHAPE / LQ_ERR_ARG.  All calls on one GPU share the one array: calls that
+ * overlap in time (different streams, or a graph replay next to eager calls) race -- serialise them. */
+int lq_fp8_amax_cast_static(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t n,
+                            lq_stream_t stream);
+size_t lq_fp8_amax_cast_static_max_elems(void);
+
 /* ---------------------------------------------------------------------------------------------
  * W4A4 group-wise INT4 activation quantisation
  * ------------------------------------------------------------------------------------------- */

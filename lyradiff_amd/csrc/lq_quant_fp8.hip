@@ -169,13 +169,16 @@ __global__ void fill_f32_kernel(float* p, float v) { p[0] = v; }
 
 // ---- device scratch of the dynamic (amax + cast) quantiser --------------------------------------------------------
 // One statically allocated block per GPU (each device that loads this library holds its own copy until the process
-// ends): the time-out flag and the barrier slots of the one-launch kernel.  Static device memory starts zeroed, and
-// every launch leaves its counters at zero again.
+// ends): the time-out flag and the barrier slots of the one-launch kernel, and the partial maxima + ticket counter of
+// the two-launch kernel pair.  Static device memory starts zeroed, and every user leaves its counters at zero again.
 // Host code never uses the array's name as an address: device_scratch() asks the runtime for the device address once
 // per device (hipGetSymbolAddress) and the kernels receive that pointer as an argument.
 constexpr int kCoopThreads = 512;
 constexpr int kCoopMaxBlocks = 1024;
 constexpr int kCoopSlots = 16;
+constexpr size_t kTicketSlab = 32768;     // elements per workgroup of the partial-maximum pass
+constexpr size_t kTicketMaxSlabs = 8192;  // partial maxima the scratch holds => at most 2^28 elements per call
+constexpr int kTicketGroups = 16;         // first-level ticket counters, one 128-byte line each
 struct CounterLine {  // one counter per 128-byte line: polls of one word must not queue behind atomics on another
     unsigned count;
     unsigned pad[31];
@@ -186,10 +189,16 @@ struct CoopSlot {
     CounterLine flag;
     float partials[kCoopMaxBlocks];
 };
+struct TicketRegion {
+    CounterLine group[kTicketGroups];
+    CounterLine top;
+    float partials[kTicketMaxSlabs];
+};
 struct FusedScratch {
     unsigned timeout;
     unsigned pad[63];
     CoopSlot coop[kCoopSlots];
+    TicketRegion ticket;
 };
 static __device__ __align__(256) unsigned char scratch[sizeof(FusedScratch)];
 
@@ -441,6 +450,80 @@ static int launch_amax_cast_coop(uint8_t* dst, float* scale_out, const void* src
     return check_launch("fp8_amax_cast_fused");
 }
 
+// ---- two launches, no barrier: partial maxima + ticket, then the cast ------------------------------------------------
+// Workgroup b reduces elements [b * kTicketSlab, (b+1) * kTicketSlab) to one partial maximum in the scratch block and
+// takes a ticket; the workgroup that draws the last ticket reduces all partials, writes scale_out[0] = max / 448 and
+// puts the ticket counters back to zero.  Nobody waits for anybody, so the kernel is safe under any scheduling, under
+// stream capture and in graph replays; the cast kernel that follows re-reads the source (from the Infinity Cache when
+// it fits).  All calls on one device share the one scratch block: calls that overlap in time race.
+template <typename Tag>
+__global__ __launch_bounds__(256) void fp8_amax_ticket_kernel(TicketRegion* __restrict__ ws, float* __restrict__ scale_out,
+                                                              const void* __restrict__ x, size_t n) {
+    constexpr int E = Chunk16<Tag>::elems;
+    constexpr int PER_THREAD = (int)(kTicketSlab / E / 256);  // chunks per thread: all requested before the first is used
+    const size_t nchunks = n / E;
+    const size_t c0 = (size_t)blockIdx.x * (kTicketSlab / E) + threadIdx.x;
+    uint4 v[PER_THREAD][2];
+#pragma unroll
+    for (int it = 0; it < PER_THREAD; ++it) {
+        const size_t c = c0 + (size_t)it * 256;
+        v[it][0] = make_uint4(0, 0, 0, 0);
+        v[it][1] = make_uint4(0, 0, 0, 0);
+        if (c < nchunks) {
+            const uint4* p = reinterpret_cast<const uint4*>(static_cast<const char*>(x) + c * 32);
+            v[it][0] = p[0];
+            v[it][1] = p[1];
+        }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int it = 0; it < PER_THREAD; ++it) {
+        float f[16];
+        if constexpr (Elem<Tag>::bytes == 2) { unpack8<Tag>(v[it][0], f); unpack8<Tag>(v[it][1], f + 8); }
+        else { f[0] = __uint_as_float(v[it][0].x); f[1] = __uint_as_float(v[it][0].y); f[2] = __uint_as_float(v[it][0].z); f[3] = __uint_as_float(v[it][0].w);
+               f[4] = __uint_as_float(v[it][1].x); f[5] = __uint_as_float(v[it][1].y); f[6] = __uint_as_float(v[it][1].z); f[7] = __uint_as_float(v[it][1].w); }
+#pragma unroll
+        for (int i = 0; i < E; ++i) amax = fmaxf(amax, fabsf(f[i]));
+    }
+    if (blockIdx.x == gridDim.x - 1) {  // fewer than E trailing elements
+        size_t i = nchunks * E + threadIdx.x;
+        if (i < n) amax = fmaxf(amax, fabsf(load_one<Tag>(x, i)));
+    }
+    __shared__ float red[4];
+    __shared__ int last;
+    amax = wave_max(amax);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const float m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        __hip_atomic_store(&ws->partials[blockIdx.x], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // acknowledged at device scope before the ticket is drawn
+        // two-level ticket (same-address atomics serialise): workgroups congruent modulo kTicketGroups share a counter,
+        // the last of a group puts it back to zero and draws from the top counter
+        const unsigned G = gridDim.x, grp = blockIdx.x % kTicketGroups;
+        const unsigned in_group = (G - grp + kTicketGroups - 1) / kTicketGroups, ngroups = G < kTicketGroups ? G : kTicketGroups;
+        int is_last = 0;
+        if (__hip_atomic_fetch_add(&ws->group[grp].count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == in_group - 1) {
+            __hip_atomic_store(&ws->group[grp].count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            is_last = __hip_atomic_fetch_add(&ws->top.count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ngroups - 1;
+        }
+        last = is_last;
+    }
+    __syncthreads();
+    if (!last) return;
+    float m = 0.0f;
+    for (unsigned i = threadIdx.x; i < gridDim.x; i += 256)
+        m = fmaxf(m, __hip_atomic_load(&ws->partials[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    m = wave_max(m);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        scale_out[0] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])) / 448.0f;
+        __hip_atomic_store(&ws->top.count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 static unsigned stream_grid(size_t n, int elems_per_thread) {
     size_t blocks = (n / elems_per_thread + 255) / 256;
     const size_t cap = 256 * 8;  // 8 workgroups of 4 wavefronts per CU keep HBM busy
@@ -468,6 +551,15 @@ static int launch_cast(uint8_t* dst, const void* src, const float* scale, int in
         hipLaunchKernelGGL((fp8_cast_scalar_kernel<Tag>), dim3(stream_grid(n, 4)), dim3(256), 0, st, dst, src, scale, invert, n);
     }
     return check_launch("fp8_cast");
+}
+
+// Partial-maximum pass of the two-launch quantiser on the scratch block `ws` (16-byte aligned x).
+template <typename Tag>
+static int launch_amax_ticket(TicketRegion* ws, float* scale_out, const void* x, size_t n, hipStream_t st) {
+    size_t slabs = (n + kTicketSlab - 1) / kTicketSlab;
+    if (slabs == 0) slabs = 1;
+    hipLaunchKernelGGL((fp8_amax_ticket_kernel<Tag>), dim3((unsigned)slabs), dim3(256), 0, st, ws, scale_out, x, n);
+    return check_launch("fp8_amax_ticket");
 }
 
 }  // namespace lq
@@ -537,11 +629,36 @@ extern "C" int lq_fp8_amax_cast(uint8_t* dst, float* scale_out, const void* src,
     return lq_fp8_scale_cast(dst, src, dtype, scale_out, 1, n, stream);
 }
 
+extern "C" int lq_fp8_amax_cast_static(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t n,
+                                       lq_stream_t stream) {
+    LQ_REQUIRE(dst && scale_out && src, LQ_ERR_ARG, "lq_fp8_amax_cast_static: null pointer");
+    LQ_REQUIRE(dtype == LQ_F16 || dtype == LQ_BF16 || dtype == LQ_F32, LQ_ERR_UNSUPPORTED,
+               "lq_fp8_amax_cast_static: unsupported dtype %d", (int)dtype);
+    LQ_REQUIRE(n >= 1 && n <= lq_fp8_amax_cast_static_max_elems(), LQ_ERR_SHAPE,
+               "lq_fp8_amax_cast_static: n=%zu outside 1..%zu (the static scratch holds %zu partial maxima of %zu elements)",
+               n, lq_fp8_amax_cast_static_max_elems(), kTicketMaxSlabs, kTicketSlab);
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0, LQ_ERR_ARG,
+               "lq_fp8_amax_cast_static: src and dst must be 16-byte aligned");
+    FusedScratch* ws = device_scratch();
+    if (ws == nullptr) return LQ_ERR_HIP;
+    hipStream_t st = as_stream(stream);
+    int rc;
+    switch (dtype) {
+        case LQ_F16: rc = launch_amax_ticket<F16Tag>(&ws->ticket, scale_out, src, n, st); break;
+        case LQ_BF16: rc = launch_amax_ticket<BF16Tag>(&ws->ticket, scale_out, src, n, st); break;
+        default: rc = launch_amax_ticket<F32Tag>(&ws->ticket, scale_out, src, n, st); break;
+    }
+    if (rc != LQ_OK) return rc;
+    return lq_fp8_scale_cast(dst, src, dtype, scale_out, 1, n, stream);
+}
+
 extern "C" int lq_fp8_amax_cast_slot(lq_stream_t stream) {
     int dev = 0;
     if (device_scratch(&dev) == nullptr) return LQ_ERR_HIP;
     return slot_for_stream(dev, as_stream(stream));
 }
+
+extern "C" size_t lq_fp8_amax_cast_static_max_elems(void) { return kTicketSlab * kTicketMaxSlabs; }
 
 extern "C" int lq_fp8_amax_cast_status(void) {
     FusedScratch* ws = device_scratch();

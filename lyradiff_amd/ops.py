@@ -323,6 +323,19 @@ def fp8_amax_cast_status() -> bool:
     return rc == 1
 
 
+def fp8_quant_static(x, q_out, scale_out):
+    """fp8_quant into caller-owned outputs through lq_fp8_amax_cast_static: two launches, no barrier, no allocation
+    (scratch in a static device array shared by every call on the GPU: do not overlap calls)."""
+    _chk(x, "x", _FLOATS)
+    _chk(q_out, "q_out", (torch.uint8,))
+    _chk(scale_out, "scale_out", (torch.float32,))
+    if q_out.numel() != x.numel() or scale_out.numel() < 1:
+        raise ValueError("q_out must have as many elements as x, scale_out at least one")
+    _l.check(_l.load().lq_fp8_amax_cast_static(_ptr(q_out), _ptr(scale_out), _ptr(x), _DT[x.dtype], x.numel(), _stream()),
+             "lq_fp8_amax_cast_static")
+    return q_out, scale_out
+
+
 # ---- W4A4 ------------------------------------------------------------------------------------------
 
 def w4a4_quant(x, smooth=None, scale_dtype=torch.float32, group: int = 64):
