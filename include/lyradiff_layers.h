@@ -4,12 +4,16 @@
 // that takes LoRA deltas (FP8LoraWeight) and the FP8 feed-forward halves of the FLUX blocks,
 // with the reference's names, members and call shapes (paths relative to the reference's
 // src/lyradiff/), so that reference-style layer code compiles against liblyraquant.so.
+// Weight files: loadWeightFromBin reads the reference's raw .bin files (one tensor per file, elements of the stated
+// file type, converted to the member's type on the way in) and every weight class has loadWeights(prefix, file_type)
+// next to loadWeightsFromCache.
 //
-// Not built: file loading (loadWeights from .bin files) and the npy/torch tensor readers of Tensor.
+// Not built: the npy/torch tensor readers of Tensor.
 #pragma once
 
 #include <cstdlib>
 #include <cstring>
+#include <fstream>
 #include <initializer_list>
 #include <sstream>
 #include <unordered_map>
@@ -224,6 +228,67 @@ enum LyraQuantType {
     INT8_SMOOTH_QUANT_LEVEL2 = 5, INT8_SMOOTH_QUANT_LEVEL3 = 6, INT4_W4A4 = 7, INT4_W4A4_FULL = 8,
 };
 
+// ---- utils/cuda_utils.h:37-43 and utils/memory_utils.cu:250-360 ------------------------------------------------------
+enum FtCudaDataType { FP32 = 0, FP16 = 1, BF16 = 2, INT8 = 3, FP8 = 4 };
+
+namespace detail {
+template <typename T> struct HostCast;  // element conversions of loadWeightFromBin (round to nearest even, as the
+template <> struct HostCast<float> {    // reference's device-side invokeCudaD2DcpyConvert does)
+    static float from(float v) { return v; }
+    static float to(float v) { return v; }
+};
+template <> struct HostCast<__half> {
+    static __half from(float v) { return __float2half(v); }
+    static float to(__half v) { return __half2float(v); }
+};
+template <> struct HostCast<hip_bfloat16> {
+    static hip_bfloat16 from(float v) { return hip_bfloat16(v); }
+    static float to(hip_bfloat16 v) { return static_cast<float>(v); }
+};
+template <> struct HostCast<int8_t> {  // never converted (INT8 files load into int8_t members only); keeps the generic code well-formed
+    static int8_t from(float v) { return static_cast<int8_t>(v); }
+    static float to(int8_t v) { return static_cast<float>(v); }
+};
+template <typename T_IN> inline bool read_bin(const std::string& filename, size_t count, std::vector<T_IN>& host) {
+    std::ifstream in(filename, std::ios::in | std::ios::binary);
+    if (!in.is_open()) return false;
+    host.resize(count);
+    in.read(reinterpret_cast<char*>(host.data()), static_cast<std::streamsize>(sizeof(T_IN) * count));
+    return static_cast<size_t>(in.gcount()) == sizeof(T_IN) * count;
+}
+}  // namespace detail
+
+// Reads shape[0] (* shape[1]) elements of `model_file_type` from `filename` into device memory at `ptr`, converting
+// them to T (loadWeightFromBin, utils/memory_utils.cu:336-360).  The reference only logs a warning when a file is
+// missing or short and leaves the weight unset; here that throws LyraException, since a linear with a missing weight
+// cannot produce a valid result.  Synchronous (hipMemcpy), like the reference's cudaH2Dcpy.
+template <typename T>
+int loadWeightFromBin(T* ptr, std::vector<size_t> shape, std::string filename, FtCudaDataType model_file_type = FtCudaDataType::FP32) {
+    LYRA_CHECK_WITH_INFO(shape.size() >= 1 && shape.size() <= 2, "loadWeightFromBin: shape should have one or two dims");
+    const size_t count = shape[0] * (shape.size() == 2 ? shape[1] : 1);
+    if (count == 0) return 0;
+    std::vector<T> out(count);
+    auto convert = [&](auto tag) {
+        using T_IN = decltype(tag);
+        std::vector<T_IN> host;
+        LYRA_CHECK_WITH_INFO(detail::read_bin<T_IN>(filename, count, host), "file " + filename + " cannot be opened or is too short, loading model fails");
+        if constexpr (std::is_same<T, T_IN>::value) out.swap(host);
+        else if constexpr (std::is_same<T, int8_t>::value || std::is_same<T_IN, int8_t>::value)
+            LYRA_CHECK_WITH_INFO(false, "loadWeightFromBin: INT8 files load into int8_t members only");
+        else
+            for (size_t i = 0; i < count; ++i) out[i] = detail::HostCast<T>::from(detail::HostCast<T_IN>::to(host[i]));
+    };
+    switch (model_file_type) {
+        case FtCudaDataType::FP32: convert(float{}); break;
+        case FtCudaDataType::FP16: convert(__half{}); break;
+        case FtCudaDataType::BF16: convert(hip_bfloat16{}); break;
+        case FtCudaDataType::INT8: convert(int8_t{}); break;
+        default: LYRA_CHECK_WITH_INFO(false, "loadWeightFromBin: does not support FtCudaDataType=" + std::to_string(static_cast<int>(model_file_type)));
+    }
+    LYRA_CHECK_WITH_INFO(hipMemcpy(ptr, out.data(), sizeof(T) * count, hipMemcpyHostToDevice) == hipSuccess, "loadWeightFromBin: copy to the device failed");
+    return 0;
+}
+
 // ---- layers/w4a4_gemm_block/W4A4GemmWeight.h:7-45, W4A4GemmWeight.cc:31-83 -----------------------------------------
 // Device-resident weights of one W4A4 linear.  `packed_weight` holds the [d_out, d_in/2] nibble matrix in
 // the rows32 layout the GEMM reads; loadWeightsFromCache takes the reference's row-major bytes and
@@ -301,6 +366,32 @@ public:
         ok = ok && hipStreamSynchronize(stream) == hipSuccess;
         (void)hipFree(staging);
         LYRA_CHECK_WITH_INFO(ok, std::string("W4A4GemmWeight::loadWeightsFromCache failed: ") + lq_last_error());
+    }
+    // The reference's raw files prefix + {packed_weight, weight_scale, lora_up, lora_down, smooth, bias}.bin
+    // (W4A4GemmWeight.cc:65-83): int8 / fp32 files as they are, the 16-bit members converted from model_file_type;
+    // the nibble matrix is repacked to rows32 once, as loadWeightsFromCache does.
+    virtual void loadWeights(const std::string prefix, FtCudaDataType model_file_type) {
+        if (!is_maintain_buffer) mallocWeights();
+        const size_t wbytes = d_out_ * d_in_ / 2;
+        int8_t* staging = nullptr;
+        LYRA_CHECK_WITH_INFO(hipMalloc(reinterpret_cast<void**>(&staging), wbytes) == hipSuccess, "W4A4GemmWeight: staging allocation failed");
+        try {
+            loadWeightFromBin<int8_t>(staging, {wbytes}, prefix + "packed_weight.bin", FtCudaDataType::INT8);
+        } catch (...) {
+            (void)hipFree(staging);
+            throw;
+        }
+        bool ok = lq_repack_rows32(reinterpret_cast<uint8_t*>(packed_weight), reinterpret_cast<const uint8_t*>(staging), d_out_, d_in_ / 2, 0) == LQ_OK &&
+                  hipStreamSynchronize(0) == hipSuccess;
+        (void)hipFree(staging);
+        LYRA_CHECK_WITH_INFO(ok, std::string("W4A4GemmWeight::loadWeights: repack failed: ") + lq_last_error());
+        loadWeightFromBin<float>(weight_scale, {d_out_ * group_num_}, prefix + "weight_scale.bin", FtCudaDataType::FP32);
+        if (lora_rank_ > 0) {
+            loadWeightFromBin<T>(lora_up, {d_out_ * lora_rank_}, prefix + "lora_up.bin", model_file_type);
+            loadWeightFromBin<T>(lora_down, {d_in_ * lora_rank_}, prefix + "lora_down.bin", model_file_type);
+        }
+        loadWeightFromBin<float>(smooth, {d_in_}, prefix + "smooth.bin", FtCudaDataType::FP32);
+        if (has_bias_) loadWeightFromBin<T>(bias, {d_out_}, prefix + "bias.bin", model_file_type);
     }
     size_t lora_rank() const { return lora_rank_; }
     size_t d_out() const { return d_out_; }
@@ -473,6 +564,17 @@ template <typename T> struct FP8LinearStore {
         LYRA_CHECK_WITH_INFO(ok, "FP8 weight copy failed for " + prefix + name);
         FP8LoraWeight<T>({d_out, d_in}, weight, weight_scale, weight_h).quantise(allocator);
     }
+    // MACROLoadFP8WeightFromBin (utils/common_macro_def.h:66-75): prefix + name + {".weight.bin", ".bias.bin",
+    // "_input_scale.bin"}; the 16-bit weight becomes the host master copy and is quantised on the device with a fresh
+    // per-tensor scale (the staging buffer of the macro is the pool buffer FP8LoraWeight uses).
+    void load_bin(const std::string& prefix, const std::string& name, FtCudaDataType model_file_type, IAllocator* allocator) {
+        T* tmp = static_cast<T*>(allocator->reMallocWithName("global_shared_weight_buffer_", sizeof(T) * d_out * d_in, false));
+        loadWeightFromBin<T>(tmp, {d_out * d_in}, prefix + name + ".weight.bin", model_file_type);
+        LYRA_CHECK_WITH_INFO(hipMemcpy(weight_h, tmp, sizeof(T) * d_out * d_in, hipMemcpyDeviceToHost) == hipSuccess, "FP8 master copy failed for " + prefix + name);
+        loadWeightFromBin<T>(bias, {d_out}, prefix + name + ".bias.bin", model_file_type);
+        loadWeightFromBin<float>(input_scale, {1}, prefix + name + "_input_scale.bin", FtCudaDataType::FP32);
+        FP8LoraWeight<T>({d_out, d_in}, weight, weight_scale, weight_h).quantise(allocator);
+    }
 };
 }  // namespace detail
 
@@ -519,6 +621,12 @@ public:
         if (!is_maintain_buffer) mallocWeights();
         gelu_.load(prefix, "net.0.proj", weights, memcpyKind, allocator_);
         ff_.load(prefix, "net.2", weights, memcpyKind, allocator_);
+    }
+    // FluxAttnPostFP8ProcessorWeight.cc:70-89: the raw files of the two feed-forward linears
+    virtual void loadWeights(const std::string prefix, FtCudaDataType model_file_type) {
+        if (!is_maintain_buffer) mallocWeights();
+        gelu_.load_bin(prefix, "net.0.proj", model_file_type, allocator_);
+        ff_.load_bin(prefix, "net.2", model_file_type, allocator_);
     }
     size_t embedding_dim() const { return embedding_dim_; }
 
@@ -651,6 +759,12 @@ public:
         if (!is_maintain_buffer) mallocWeights();
         mlp_.load(prefix, "proj_mlp", weights, memcpyKind, allocator_);
         out_.load(prefix, "proj_out", weights, memcpyKind, allocator_);
+    }
+    // FluxSingleTransformerFP8BlockWeight.cc:99-122 (the two linears this class owns)
+    virtual void loadWeights(const std::string prefix, FtCudaDataType model_file_type) {
+        if (!is_maintain_buffer) mallocWeights();
+        mlp_.load_bin(prefix, "proj_mlp", model_file_type, allocator_);
+        out_.load_bin(prefix, "proj_out", model_file_type, allocator_);
     }
     size_t embedding_dim() const { return embedding_dim_; }
     size_t mlp_scale() const { return mlp_scale_; }

@@ -32,11 +32,12 @@ chunks 2..5 are gate_msa, shift_mlp, scale_mlp, gate_mlp; for the single block c
 from __future__ import annotations
 
 from dataclasses import dataclass
+from typing import Union
 
 import torch
 
 from . import ops
-from .weights import FP8Linear, load_fp8_linear
+from .weights import FP8Linear, _source, load_fp8_linear
 
 
 @dataclass
@@ -74,7 +75,26 @@ def load_ada_fp8_layernorm(src, prefix: str, dim: int, n_chunks: int, dtype=torc
     return load_fp8_linear(src, prefix, "linear", n_chunks * dim, dim, dtype, device, keep_master)
 
 
-def ada_fp8_layernorm(x: torch.Tensor, temb: torch.Tensor, linear: FP8Linear, n_chunks: int, code_scales=(),
+@dataclass
+class AdaLinear16:
+    """The 16-bit adaLN linear of the quant levels FP8_W8A8 and INT4_W4A4 (AdaLayerNormWeight, keys prefix +
+    "linear.weight" / ".bias"; the blocks take this branch unless the level is ..._FULL,
+    FluxTransformerFP8Block.cc:203-211); the _FULL levels hold an FP8Linear in its place (AdaFP8LayerNormWeight)."""
+    weight: torch.Tensor  # T [n_chunks*D, D]
+    bias: torch.Tensor    # T [n_chunks*D]
+
+
+def load_ada_layernorm(src, prefix: str, dim: int, n_chunks: int, full: bool, dtype=torch.bfloat16, device="cuda",
+                       keep_master: bool = False) -> Union[FP8Linear, AdaLinear16]:
+    """full: the level's adaLN linear is FP8 (keys with `_input_scale`); otherwise a plain 16-bit linear."""
+    if full:
+        return load_ada_fp8_layernorm(src, prefix, dim, n_chunks, dtype, device, keep_master)
+    get = _source(src)
+    return AdaLinear16(get(prefix + "linear.weight", (n_chunks * dim, dim), dtype).to(device),
+                       get(prefix + "linear.bias", (n_chunks * dim,), dtype).to(device))
+
+
+def ada_fp8_layernorm(x: torch.Tensor, temb: torch.Tensor, linear: Union[FP8Linear, AdaLinear16], n_chunks: int, code_scales=(),
                       switch_scale: bool = False, eps: float = 1e-6):
     """AdaFP8LayerNorm<T>::forward (layers/ada_layer_norm/AdaFP8LayerNorm.cc:93-205): msa = FP8 linear of the
     (already SiLU'd) time embedding, stored [n_chunks, B, D]; output = (1 + msa[1]) * LayerNorm(x) + msa[0]
@@ -83,8 +103,11 @@ def ada_fp8_layernorm(x: torch.Tensor, temb: torch.Tensor, linear: FP8Linear, n_
     the e4m3 codes for the FP8 linears that consume it instead (cast fused, no 16-bit tensor).
     Returns (norm | codes | (codes_a, codes_b), msa)."""
     b, s, d = x.shape
-    q = ops.fp8_scale_cast(temb.reshape(b, d), linear.input_scale)
-    flat = ops.fp8_linear(q, linear.weight_rows32, linear.input_scale, linear.weight_scale, linear.bias, out_dtype=x.dtype)
+    if isinstance(linear, AdaLinear16):  # not a quantized linear: a plain 16-bit matmul (AdaLayerNorm.cc)
+        flat = torch.nn.functional.linear(temb.reshape(b, d), linear.weight, linear.bias)
+    else:
+        q = ops.fp8_scale_cast(temb.reshape(b, d), linear.input_scale)
+        flat = ops.fp8_linear(q, linear.weight_rows32, linear.input_scale, linear.weight_scale, linear.bias, out_dtype=x.dtype)
     msa = flat.view(b, n_chunks, d).transpose(0, 1).contiguous() if b > 1 else flat.view(n_chunks, 1, d)  # invokeTranspose102
     shift, scale = (msa[1], msa[0]) if switch_scale else (msa[0], msa[1])
     if len(code_scales) == 0:
@@ -133,15 +156,15 @@ def flux_single_mlp_fp8(x: torch.Tensor, norm_hidden, attn_output: torch.Tensor,
 
 @dataclass
 class FluxSingleBlockFP8Weights:
-    norm: FP8Linear      # prefix + "norm.linear"  [3D, D]
+    norm: Union[FP8Linear, AdaLinear16]  # prefix + "norm.linear"  [3D, D]
     to_qkv: FP8Linear    # prefix + "attn.to_qkv"  [3D, D]
     mlp: FluxSingleMlpFP8Weights
 
 
 @dataclass
 class FluxDoubleBlockFP8Weights:
-    norm1: FP8Linear           # prefix + "norm1.linear"          [6D, D]
-    norm1_context: FP8Linear   # prefix + "norm1_context.linear"  [6D, D]
+    norm1: Union[FP8Linear, AdaLinear16]          # prefix + "norm1.linear"          [6D, D]
+    norm1_context: Union[FP8Linear, AdaLinear16]  # prefix + "norm1_context.linear"  [6D, D]
     to_qkv: FP8Linear          # prefix + "attn.to_qkv"
     to_added_qkv: FP8Linear    # prefix + "attn.to_added_qkv"
     to_out: FP8Linear          # prefix + "attn.to_out.0"
@@ -151,20 +174,21 @@ class FluxDoubleBlockFP8Weights:
 
 
 def load_flux_single_block_fp8(src, prefix: str, dim: int, mlp_scale: int = 4, dtype=torch.bfloat16, device="cuda",
-                               keep_master: bool = False) -> FluxSingleBlockFP8Weights:
-    """FluxSingleTransformerFP8BlockWeight::loadWeights (FluxSingleTransformerFP8BlockWeight.cc:94-121)."""
-    return FluxSingleBlockFP8Weights(load_ada_fp8_layernorm(src, prefix + "norm.", dim, 3, dtype, device, keep_master),
+                               keep_master: bool = False, full: bool = True) -> FluxSingleBlockFP8Weights:
+    """FluxSingleTransformerFP8BlockWeight::loadWeights (FluxSingleTransformerFP8BlockWeight.cc:94-121).
+    full: quant level FP8_W8A8_FULL (FP8 adaLN linear); False: level FP8_W8A8 (16-bit adaLN linear)."""
+    return FluxSingleBlockFP8Weights(load_ada_layernorm(src, prefix + "norm.", dim, 3, full, dtype, device, keep_master),
                                      load_fp8_linear(src, prefix + "attn.", "to_qkv", 3 * dim, dim, dtype, device, keep_master),
                                      load_flux_single_mlp_fp8(src, prefix, dim, mlp_scale, dtype, device, keep_master))
 
 
 def load_flux_double_block_fp8(src, prefix: str, dim: int, dtype=torch.bfloat16, device="cuda",
-                               keep_master: bool = False) -> FluxDoubleBlockFP8Weights:
+                               keep_master: bool = False, full: bool = True) -> FluxDoubleBlockFP8Weights:
     """FluxTransformerFP8BlockWeight::loadWeights (FluxTransformerFP8BlockWeight.cc:78-91) and
     FluxAttentionFP8ProcessorWeight::loadWeights (FluxAttentionFP8ProcessorWeight.cc:113-138)."""
     lin = lambda name, n, k: load_fp8_linear(src, prefix + "attn.", name, n, k, dtype, device, keep_master)
-    return FluxDoubleBlockFP8Weights(load_ada_fp8_layernorm(src, prefix + "norm1.", dim, 6, dtype, device, keep_master),
-                                     load_ada_fp8_layernorm(src, prefix + "norm1_context.", dim, 6, dtype, device, keep_master),
+    return FluxDoubleBlockFP8Weights(load_ada_layernorm(src, prefix + "norm1.", dim, 6, full, dtype, device, keep_master),
+                                     load_ada_layernorm(src, prefix + "norm1_context.", dim, 6, full, dtype, device, keep_master),
                                      lin("to_qkv", 3 * dim, dim), lin("to_added_qkv", 3 * dim, dim), lin("to_out.0", dim, dim),
                                      lin("to_add_out", dim, dim),
                                      load_flux_attn_post_fp8(src, prefix + "ff.", dim, dtype, device, keep_master),

@@ -27,8 +27,8 @@ from typing import Union
 import torch
 
 from . import ops
-from .flux_fp8 import ada_fp8_layernorm, load_ada_fp8_layernorm
-from .weights import FP8Linear, W4A4Linear, _source, load_fp8_linear, load_w4a4_linear
+from .flux_fp8 import AdaLinear16, ada_fp8_layernorm, load_ada_layernorm
+from .weights import FP8Linear, W4A4Linear, load_fp8_linear, load_w4a4_linear
 
 
 @dataclass
@@ -92,32 +92,15 @@ def flux_single_mlp_int4(x: torch.Tensor, norm_hidden: torch.Tensor, attn_output
 
 
 # ---- whole INT4 blocks around a caller-supplied attention core ------------------------------------------------------
-@dataclass
-class AdaLinear16:
-    """The 16-bit adaLN linear of quant level INT4_W4A4 (AdaLayerNormWeight, keys prefix + "linear.weight" / ".bias"); level
-    INT4_W4A4_FULL holds an FP8Linear in its place (AdaFP8LayerNormWeight)."""
-    weight: torch.Tensor  # T [n_chunks*D, D]
-    bias: torch.Tensor    # T [n_chunks*D]
-
-
 def _load_ada(src, prefix: str, dim: int, n_chunks: int, full: bool, dtype, device) -> Union[FP8Linear, AdaLinear16]:
-    if full:
-        return load_ada_fp8_layernorm(src, prefix, dim, n_chunks, dtype, device)
-    get = _source(src)
-    return AdaLinear16(get(prefix + "linear.weight", (n_chunks * dim, dim), dtype).to(device),
-                       get(prefix + "linear.bias", (n_chunks * dim,), dtype).to(device))
+    return load_ada_layernorm(src, prefix, dim, n_chunks, full, dtype, device)
 
 
 def ada_layernorm_int4(x: torch.Tensor, temb: torch.Tensor, linear: Union[FP8Linear, AdaLinear16], n_chunks: int,
                        eps: float = 1e-6):
     """AdaLayerNorm / AdaFP8LayerNorm in front of the W4A4 linears: returns (norm_hidden 16-bit [B, S, D], msa [n_chunks, B, D]).
     The 16-bit adaLN linear of level INT4_W4A4 is not a quantized linear and runs as a plain PyTorch matmul."""
-    if isinstance(linear, FP8Linear):
-        return ada_fp8_layernorm(x, temb, linear, n_chunks, (), eps=eps)
-    b, s, d = x.shape
-    flat = torch.nn.functional.linear(temb.reshape(b, d), linear.weight, linear.bias)
-    msa = flat.view(b, n_chunks, d).transpose(0, 1).contiguous()
-    return ops.gate_residual_layernorm_mod(x, msa[1], msa[0], eps=eps), msa
+    return ada_fp8_layernorm(x, temb, linear, n_chunks, (), eps=eps)
 
 
 @dataclass

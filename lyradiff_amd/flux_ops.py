@@ -23,6 +23,7 @@ import torch
 from . import flux_fp8 as F
 from . import flux_int4 as I4
 from . import ops
+from . import weights as W
 
 
 class LyraQuantLevel(Enum):
@@ -61,15 +62,6 @@ def flux_attention_core(qkv: torch.Tensor, norm_q: torch.Tensor, norm_k: torch.T
     if context_qkv is None:
         return o
     return o[:, sc:], o[:, :sc]
-
-
-def _get(src: Mapping, name: str, shape, dtype) -> torch.Tensor:
-    if name not in src:
-        raise KeyError(f"Cannot find a tensor of name {name}")
-    t = src[name]
-    if tuple(t.shape) != tuple(shape) or t.dtype != dtype:
-        raise ValueError(f"{name}: got {tuple(t.shape)} {t.dtype}, expected {tuple(shape)} {dtype}")
-    return t
 
 
 class _BlockOpBase:
@@ -120,7 +112,7 @@ class _BlockOpBase:
         if self.int4:  # the reference's INT4 block weights register no LoRA targets (FluxTransformerInt4BlockWeight.cc:41-45)
             raise KeyError(f"no LoRA target named {key}: the INT4 blocks carry their low-rank branch in the checkpoint")
         lin = self._fp8_linears().get(key)
-        if lin is None:
+        if lin is None or not isinstance(lin, W.FP8Linear):
             raise KeyError(f"no FP8 linear named {key} in this block")
         lin.load_lora(lora_weights.to(self.device), float(lora_strength))
 
@@ -128,7 +120,8 @@ class _BlockOpBase:
         self._loaded()
         if not self.int4:
             for lin in self._fp8_linears().values():
-                lin.clear_lora()
+                if isinstance(lin, W.FP8Linear):
+                    lin.clear_lora()
 
 
 class FluxTransformerBlockOp(_BlockOpBase):
@@ -139,12 +132,23 @@ class FluxTransformerBlockOp(_BlockOpBase):
         read them (FluxAttentionFP8ProcessorWeight.cc:194-260): the linears' `.weight`, `.bias`, `_input_scale`, and
         `attn.norm_q.weight`, `attn.norm_k.weight`, `attn.norm_added_q.weight`, `attn.norm_added_k.weight`.  `device` names
         where the tensors of `weights` live, as in the reference; they end up on the GPU either way."""
+        self._load(prefix, weights)
+
+    def reload_model_from_bin(self, model_path: str, model_dtype: str) -> None:
+        """FluxTransformerBlockOp::reload_model_from_bin (th_op/flux_transformer_block/FluxTransformerBlockOp.h:239-258):
+        `model_path` is the prefix of the block's raw .bin files (model_path + "attn.to_qkv.weight.bin", ...), with the
+        same tensor names as the state dict; `model_dtype` is the element type the 16-bit tensors were written in."""
+        self._load(model_path, W.BinFiles("", model_dtype))
+
+    def _load(self, prefix: str, src) -> None:
         if self.int4:
-            self.weights = I4.load_flux_double_block_int4(weights, prefix, self.dim, self.quant_level is LyraQuantLevel.INT4_W4A4_FULL,
+            self.weights = I4.load_flux_double_block_int4(src, prefix, self.dim, self.quant_level is LyraQuantLevel.INT4_W4A4_FULL,
                                                           self.dtype, self.device)
         else:
-            self.weights = F.load_flux_double_block_fp8(weights, prefix, self.dim, self.dtype, self.device, keep_master=True)
-        self.norms = [_get(weights, prefix + f"attn.{n}.weight", (self.head_dim,), self.dtype).to(self.device)
+            self.weights = F.load_flux_double_block_fp8(src, prefix, self.dim, self.dtype, self.device, keep_master=True,
+                                                        full=self.quant_level is LyraQuantLevel.FP8_W8A8_FULL)
+        get = W._source(src)
+        self.norms = [get(prefix + f"attn.{n}.weight", (self.head_dim,), self.dtype).to(self.device)
                       for n in ("norm_q", "norm_k", "norm_added_q", "norm_added_k")]
 
     def _fp8_linears(self):
@@ -172,14 +176,21 @@ class FluxSingleTransformerBlockOp(_BlockOpBase):
     """Single-stream FLUX block (FluxSingleTransformerFP8Block.cc:163-291)."""
 
     def reload_model_from_state_dict(self, prefix: str, weights: Mapping[str, torch.Tensor], device: str = "cpu") -> None:
+        self._load(prefix, weights)
+
+    def reload_model_from_bin(self, model_path: str, model_dtype: str) -> None:
+        """FluxSingleTransformerBlockOp::reload_model_from_bin: raw .bin files named model_path + tensor name + ".bin"."""
+        self._load(model_path, W.BinFiles("", model_dtype))
+
+    def _load(self, prefix: str, src) -> None:
         if self.int4:
-            self.weights = I4.load_flux_single_block_int4(weights, prefix, self.dim, self.mlp_scale,
+            self.weights = I4.load_flux_single_block_int4(src, prefix, self.dim, self.mlp_scale,
                                                           self.quant_level is LyraQuantLevel.INT4_W4A4_FULL, self.dtype, self.device)
         else:
-            self.weights = F.load_flux_single_block_fp8(weights, prefix, self.dim, self.mlp_scale, self.dtype, self.device,
-                                                        keep_master=True)
-        self.norms = [_get(weights, prefix + f"attn.{n}.weight", (self.head_dim,), self.dtype).to(self.device)
-                      for n in ("norm_q", "norm_k")]
+            self.weights = F.load_flux_single_block_fp8(src, prefix, self.dim, self.mlp_scale, self.dtype, self.device,
+                                                        keep_master=True, full=self.quant_level is LyraQuantLevel.FP8_W8A8_FULL)
+        get = W._source(src)
+        self.norms = [get(prefix + f"attn.{n}.weight", (self.head_dim,), self.dtype).to(self.device) for n in ("norm_q", "norm_k")]
 
     def _fp8_linears(self):
         w = self._loaded()

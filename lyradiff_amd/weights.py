@@ -44,8 +44,31 @@ def read_bin(path: str, shape, dtype: torch.dtype) -> torch.Tensor:
     return t.view(torch.bfloat16) if dtype == torch.bfloat16 else t
 
 
+class BinFiles:
+    """The reference's raw weight files under `root` (file name = root + tensor name + ".bin"), with the element type
+    the files of the 16-bit members were written in (`model_dtype` "fp32", "fp16" or "bf16": the FtCudaDataType argument
+    of loadWeights).  Members the reference always stores as fp32 or int8 (scales, smoothing vectors, packed codes) are
+    read as such; 16-bit members are converted from the file type to the requested type with round-to-nearest-even, as
+    loadWeightFromBin does (utils/memory_utils.cu:295-360)."""
+
+    _FILE = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}
+
+    def __init__(self, root: str, model_dtype: str = "fp32"):
+        if model_dtype not in self._FILE:
+            raise ValueError("wrong model_dtype")  # the reference: std::invalid_argument("wrong model_dtype")
+        self.root, self.file_dtype = root, self._FILE[model_dtype]
+
+    def __call__(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        path = self.root + name + ".bin"
+        if dtype in (torch.float16, torch.bfloat16):
+            return read_bin(path, shape, self.file_dtype).to(dtype)
+        return read_bin(path, shape, dtype)
+
+
 def _source(src) -> Callable[[str, tuple, torch.dtype], torch.Tensor]:
-    """`src` is a directory of .bin files or a mapping name -> tensor (a state dict)."""
+    """`src` is a directory of .bin files, a BinFiles object or a mapping name -> tensor (a state dict)."""
+    if isinstance(src, BinFiles):
+        return src
     if isinstance(src, Mapping):
         def get(name, shape, dtype):
             if name not in src:

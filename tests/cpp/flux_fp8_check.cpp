@@ -5,6 +5,7 @@
 // steps.  Exit code 0 when every check passes; one line per check.  Built by lyradiff_amd/build.py, run by
 // tests/test_gpu_compat.py.
 #include <cmath>
+#include <unistd.h>
 #include <cstdio>
 #include <cstdlib>
 #include <vector>
@@ -126,6 +127,32 @@ int main() {
             const int restored = count_diff(download(dout, M * D), got);
             std::printf("FP8LoraWeight load/clear: %d outputs changed by the merge, %d mismatches after clear\n", changed, restored);
             failures += changed == 0 || restored != 0;
+
+            // the same weights from the reference's raw .bin files (loadWeights: MACROLoadFP8WeightFromBin), stored as bf16
+            char dir_tmpl[] = "/tmp/lq_fp8_XXXXXX";
+            const char* dir = mkdtemp(dir_tmpl);
+            if (dir == nullptr) { std::printf("mkdtemp failed\n"); return 2; }
+            const std::string fprefix = std::string(dir) + "/ff.";
+            const char* names[6] = {"net.0.proj.weight.bin", "net.0.proj.bias.bin", "net.0.proj_input_scale.bin",
+                                    "net.2.weight.bin", "net.2.bias.bin", "net.2_input_scale.bin"};
+            const void* datas[6] = {w1.data(), b1.data(), &s_in1, w2.data(), b2.data(), &s_in2};
+            const size_t sizes[6] = {w1.size() * 2, b1.size() * 2, 4, w2.size() * 2, b2.size() * 2, 4};
+            bool wrote = true;
+            for (int i = 0; i < 6; ++i) {
+                std::FILE* f = std::fopen((fprefix + names[i]).c_str(), "wb");
+                wrote = wrote && f != nullptr && std::fwrite(datas[i], 1, sizes[i], f) == sizes[i];
+                if (f) std::fclose(f);
+            }
+            FluxAttnPostFP8ProcessorWeight<bf16> from_files(D, LyraQuantType::FP8_W8A8, &allocator);
+            from_files.loadWeights(fprefix, FtCudaDataType::BF16);
+            CK(hipMemset(dout, 0, M * D * 2));
+            proc.forward(&out, &in, &from_files);
+            CK(hipStreamSynchronize(st));
+            const int badf = (wrote ? 0 : 1) + count_diff(download(dout, M * D), got);
+            std::printf("FluxAttnPostFP8ProcessorWeight::loadWeights from .bin files: %d mismatches\n", badf);
+            failures += badf != 0;
+            for (int i = 0; i < 6; ++i) std::remove((fprefix + names[i]).c_str());
+            rmdir(dir);
         } catch (const std::exception& e) {
             std::printf("exception: %s\n", e.what());
             return 3;

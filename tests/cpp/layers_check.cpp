@@ -3,6 +3,7 @@
 // Exit code 0 when every check passes; one line per check.  Built by lyradiff_amd/build.py, run by
 // tests/test_gpu_compat.py.
 #include <cmath>
+#include <unistd.h>
 #include <cstdio>
 #include <cstdlib>
 #include <vector>
@@ -164,6 +165,52 @@ int main() {
             }
             std::printf("W4A4Gemm<bf16>::forward with the low-rank branch: %d outliers\n", outliers);
             failures += outliers != 0;
+            // ---- the same weights from the reference's raw .bin files (W4A4GemmWeight::loadWeights): the 16-bit members
+            // are stored as fp32 files and converted on the way in; the forward must equal the cache-loaded layer's, bit for bit
+            {
+                char dir_tmpl[] = "/tmp/lq_w4a4_XXXXXX";
+                const char* dir = mkdtemp(dir_tmpl);
+                if (dir == nullptr) { std::printf("mkdtemp failed\n"); return 2; }
+                const std::string prefix = std::string(dir) + "/blk.";
+                auto dump = [&](const char* name, const void* data, size_t bytes) {
+                    std::FILE* f = std::fopen((prefix + name).c_str(), "wb");
+                    bool ok = f != nullptr && std::fwrite(data, 1, bytes, f) == bytes;
+                    if (f) std::fclose(f);
+                    return ok;
+                };
+                bool wrote = dump("packed_weight.bin", wpacked.data(), wpacked.size()) && dump("weight_scale.bin", ws.data(), ws.size() * 4) &&
+                             dump("smooth.bin", smooth.data(), smooth.size() * 4) && dump("bias.bin", biasf.data(), biasf.size() * 4) &&
+                             dump("lora_down.bin", down.data(), down.size() * 4) && dump("lora_up.bin", up.data(), up.size() * 4);
+                std::vector<hip_bfloat16> y2(m * n);
+                bool missing_throws = false;
+                try {
+                    W4A4GemmWeight<hip_bfloat16> wf(n, k, R, true, 64, LyraQuantType::INT4_W4A4, &allocator);
+                    wf.loadWeights(prefix, FtCudaDataType::FP32);
+                    W4A4Gemm<hip_bfloat16> layer(n, k, R, true, 64, st, nullptr, &allocator, false);
+                    TensorMap in({{"input", Tensor(MEMORY_GPU, TYPE_BF16, {(size_t)m, (size_t)k}, dx)}});
+                    TensorMap out({{"output", Tensor(MEMORY_GPU, TYPE_BF16, {(size_t)m, (size_t)n}, dy)}});
+                    CK(hipMemset(dy, 0, m * n * 2));
+                    layer.forward(&out, &in, &wf);
+                    CK(hipStreamSynchronize(st));
+                    CK(hipMemcpy(y2.data(), dy, m * n * 2, hipMemcpyDeviceToHost));
+                    try {
+                        wf.loadWeights(prefix + "absent.", FtCudaDataType::FP32);
+                    } catch (const LyraException&) {
+                        missing_throws = true;
+                    }
+                } catch (const std::exception& e) {
+                    std::printf("exception: %s\n", e.what());
+                    return 3;
+                }
+                int badf = wrote ? 0 : 1;
+                for (int i = 0; i < m * n; ++i) badf += (float)y2[i] != (float)y[i];
+                std::printf("W4A4GemmWeight::loadWeights from .bin files: %d mismatches, a missing file raises LyraException: %s\n",
+                            badf, missing_throws ? "yes" : "no");
+                failures += badf != 0 || !missing_throws;
+                for (const char* nm : {"packed_weight.bin", "weight_scale.bin", "smooth.bin", "bias.bin", "lora_down.bin", "lora_up.bin"})
+                    std::remove((prefix + nm).c_str());
+                rmdir(dir);
+            }
             allocator.freeWithName("W4A4Gemm_lora_down_res_buffer2");
         }
         bool threw = false;

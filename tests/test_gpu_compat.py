@@ -24,7 +24,7 @@ def test_cpp_layer_types(dev):
     r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count("0 mismatches") == 2 and r.stdout.count(": yes") == 2 and "0 outliers" in r.stdout
+    assert r.stdout.count("0 mismatches") == 3 and r.stdout.count(": yes") == 3 and "0 outliers" in r.stdout
 
 
 def test_cpp_flux_fp8_types(dev):
@@ -35,4 +35,4 @@ def test_cpp_flux_fp8_types(dev):
     r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count(" 0 mismatches") == 4
+    assert r.stdout.count(" 0 mismatches") == 5

@@ -595,7 +595,7 @@ def test_flux_block_ops_have_the_reference_interface(ops, dev):
     op.reload_model_from_state_dict("transformer_blocks.3.", sd, "cpu")
     res = op.forward(x, ctx, rope, temb)
     assert isinstance(res, list) and res[0].shape == x.shape and res[1].shape == ctx.shape
-    wd = F.load_flux_double_block_fp8(sd, "transformer_blocks.3.", d, torch.bfloat16, dev)
+    wd = F.load_flux_double_block_fp8(sd, "transformer_blocks.3.", d, torch.bfloat16, dev, full=False)  # level FP8_W8A8: 16-bit adaLN linear
     nq, nk, naq, nak = (sd[f"transformer_blocks.3.attn.{n}.weight"].to(dev) for n in ("norm_q", "norm_k", "norm_added_q", "norm_added_k"))
     w1, w2 = F.flux_double_block_fp8(x, ctx, temb, wd, lambda a, c: FO.flux_attention_core(a, nq, nk, rope, heads, c, naq, nak))
     assert torch.equal(res[0], w1) and torch.equal(res[1], w2) and torch.isfinite(w1.float()).all()
@@ -632,6 +632,117 @@ def test_flux_block_ops_have_the_reference_interface(ops, dev):
     snq, snk = (sd[f"single_transformer_blocks.5.attn.{n}.weight"].to(dev) for n in ("norm_q", "norm_k"))
     want = F.flux_single_block_fp8(xs, temb, ws, lambda a: FO.flux_attention_core(a, snq, snk, rope, heads))
     assert y.shape == xs.shape and torch.equal(y, want) and torch.isfinite(y.float()).all()
+
+
+_BLOCK_LINEARS = lambda d: {"norm.linear": (3 * d, d), "attn.to_qkv": (3 * d, d), "proj_mlp": (4 * d, d), "proj_out": (d, 5 * d),
+                            "norm1.linear": (6 * d, d), "norm1_context.linear": (6 * d, d), "attn.to_added_qkv": (3 * d, d),
+                            "attn.to_out.0": (d, d), "attn.to_add_out": (d, d), "ff.net.0.proj": (4 * d, d), "ff.net.2": (d, 4 * d),
+                            "ff_context.net.0.proj": (4 * d, d), "ff_context.net.2": (d, 4 * d)}
+
+
+def _block_state(d, dh, seed, prefixes):
+    """Weights large enough that every branch of the block matters as much as the residual stream (gates, scales and
+    shifts of order one): a mis-wired block then differs by tens of per cent, not by a rounding error."""
+    g = rng_t(seed)
+    sd = {}
+    for i, pre in enumerate(prefixes):
+        sd.update(_state_dict(_BLOCK_LINEARS(d), seed + 1 + i, scale_w=0.06, prefix=pre))
+        for n in _BLOCK_LINEARS(d):
+            sd[f"{pre}{n}_input_scale"] = torch.tensor([6.0 / 448])
+        for n in ("norm_q", "norm_k", "norm_added_q", "norm_added_k"):
+            sd[f"{pre}attn.{n}.weight"] = (1 + 0.1 * torch.randn(dh, generator=g)).bfloat16()
+    return sd
+
+
+def _rel(a, b):
+    return float((a.double() - b.double()).norm() / b.double().norm())
+
+
+@pytest.mark.parametrize("level", ["FP8_W8A8_FULL", "FP8_W8A8"])
+def test_flux_block_ops_against_an_independent_fp64_restatement(ops, dev, level):
+    """FluxTransformerBlockOp.forward and FluxSingleTransformerBlockOp.forward against oracle/flux_blocks_f64.py, an fp64
+    restatement of the reference's block code that shares nothing with lyradiff_amd/flux_fp8.py.  The outputs agree to
+    within the noise of e4m3 codes that flip on 16-bit rounding differences; every deliberately mis-wired variant of the
+    restatement (scale/shift swapped, wrong msa chunk, image tokens first, projections swapped, a dropped residual, the
+    concatenation of the single block reversed) is many times further away."""
+    from lyradiff_amd import flux_ops as FO
+    from oracle import flux_blocks_f64 as FB
+
+    b, s, sc, heads, dh = 2, 96, 32, 4, 64
+    d = heads * dh
+    full = level == "FP8_W8A8_FULL"
+    g = rng_t(401)
+    sd = _block_state(d, dh, 402, ("transformer_blocks.0.", "single_transformer_blocks.0."))
+    x = torch.randn(b, s, d, generator=g).bfloat16()
+    ctx = torch.randn(b, sc, d, generator=g).bfloat16()
+    temb = torch.randn(b, d, generator=g).bfloat16()
+    rope = _rope_table(b, sc + s, dh, 403).bfloat16()
+
+    op = FO.FluxTransformerBlockOp("bf16", d, heads, dh, 4, FO.LyraQuantLevel[level].value)
+    op.reload_model_from_state_dict("transformer_blocks.0.", sd, "cpu")
+    out, cout = op.forward(x.to(dev), ctx.to(dev), rope.to(dev), temb.to(dev))
+    want, cwant = FB.flux_double_block(sd, "transformer_blocks.0.", x, ctx, temb, rope, heads, "bf16", full)
+    e1, e2 = _rel(out.cpu(), want), _rel(cout.cpu(), cwant)
+    print(f"double block {level}: relative L2 distance to the fp64 restatement {e1:.4f} (image), {e2:.4f} (text)")
+    assert e1 < 0.04 and e2 < 0.04
+    for w in ("swap_scale_shift", "image_first", "swap_mlp_scale_shift", "swap_gates", "no_second_residual", "swap_out_projections"):
+        bad, cbad = FB.flux_double_block(sd, "transformer_blocks.0.", x, ctx, temb, rope, heads, "bf16", full, wiring=(w,))
+        assert _rel(out.cpu(), bad) > 4 * max(e1, 0.02) and _rel(cout.cpu(), cbad) > 4 * max(e2, 0.02), w
+
+    sop = FO.FluxSingleTransformerBlockOp("bf16", d, heads, dh, 4, FO.LyraQuantLevel[level].value)
+    sop.reload_model_from_state_dict("single_transformer_blocks.0.", sd, "cpu")
+    xs = torch.cat([ctx, x], dim=1).contiguous()
+    y = sop.forward(xs.to(dev), rope.to(dev), temb.to(dev))
+    ywant = FB.flux_single_block(sd, "single_transformer_blocks.0.", xs, temb, rope, heads, "bf16", full)
+    e3 = _rel(y.cpu(), ywant)
+    print(f"single block {level}: relative L2 distance to the fp64 restatement {e3:.4f}")
+    assert e3 < 0.04
+    for w in ("swap_scale_shift", "mlp_first", "gate_is_chunk0"):
+        assert _rel(y.cpu(), FB.flux_single_block(sd, "single_transformer_blocks.0.", xs, temb, rope, heads, "bf16", full, wiring=(w,))) > 4 * max(e3, 0.02), w
+
+
+@pytest.mark.parametrize("file_dtype", ["fp32", "fp16"])
+def test_flux_block_ops_reload_model_from_bin(ops, dev, tmp_path, file_dtype):
+    """reload_model_from_bin(model_path, model_dtype) (th_op/flux_transformer_block/FluxTransformerBlockOp.h:239-258): the
+    block's tensors as raw files model_path + name + ".bin", 16-bit members written in `model_dtype` and converted on
+    the way in, scales as fp32.  With fp32 files (exact for bf16 values) the outputs equal those of the state-dict route bit for bit;
+    with fp16 files the weights are rounded to fp16 and back, and the op equals a state-dict load of those rounded weights."""
+    from lyradiff_amd import flux_ops as FO
+
+    b, s, sc, heads, dh = 1, 64, 32, 4, 64
+    d = heads * dh
+    sd = _block_state(d, dh, 412, ("transformer_blocks.7.", "single_transformer_blocks.9."))
+    ft = {"fp32": torch.float32, "fp16": torch.float16}[file_dtype]
+    sd_files = {}
+    for k, v in sd.items():
+        if v.dtype == torch.bfloat16:
+            v.to(ft).numpy().tofile(str(tmp_path / (k + ".bin")))
+            sd_files[k] = v.to(ft).bfloat16()
+        else:
+            v.numpy().tofile(str(tmp_path / (k + ".bin")))
+            sd_files[k] = v
+    g = rng_t(413)
+    x = torch.randn(b, s, d, generator=g).bfloat16().to(dev)
+    ctx = torch.randn(b, sc, d, generator=g).bfloat16().to(dev)
+    temb = torch.randn(b, d, generator=g).bfloat16().to(dev)
+    rope = _rope_table(b, sc + s, dh, 414).bfloat16().to(dev)
+    for level in (FO.LyraQuantLevel.FP8_W8A8_FULL, FO.LyraQuantLevel.FP8_W8A8):
+        a = FO.FluxTransformerBlockOp("bf16", d, heads, dh, 4, level.value)
+        a.reload_model_from_state_dict("transformer_blocks.7.", sd_files, "cpu")
+        f = FO.FluxTransformerBlockOp("bf16", d, heads, dh, 4, level.value)
+        f.reload_model_from_bin(str(tmp_path) + "/transformer_blocks.7.", file_dtype)
+        ra, rf = a.forward(x, ctx, rope, temb), f.forward(x, ctx, rope, temb)
+        assert torch.equal(ra[0], rf[0]) and torch.equal(ra[1], rf[1])
+    sa = FO.FluxSingleTransformerBlockOp("bf16", d, heads, dh, 4, FO.LyraQuantLevel.FP8_W8A8_FULL.value)
+    sa.reload_model_from_state_dict("single_transformer_blocks.9.", sd_files, "cpu")
+    sf = FO.FluxSingleTransformerBlockOp("bf16", d, heads, dh, 4, FO.LyraQuantLevel.FP8_W8A8_FULL.value)
+    sf.reload_model_from_bin(str(tmp_path) + "/single_transformer_blocks.9.", file_dtype)
+    xs = torch.cat([ctx, x], dim=1).contiguous()
+    assert torch.equal(sa.forward(xs, rope, temb), sf.forward(xs, rope, temb))
+    with pytest.raises(ValueError):
+        sf.reload_model_from_bin(str(tmp_path) + "/single_transformer_blocks.9.", "int8")  # the reference: "wrong model_dtype"
+    with pytest.raises((FileNotFoundError, ValueError, OSError)):
+        sf.reload_model_from_bin(str(tmp_path) + "/absent.", "fp32")
 
 
 @pytest.mark.parametrize("full", [True, False])

@@ -733,3 +733,87 @@ def test_fp8_mfma_step_bound_dominates_the_model_error():
     exact = a.astype(np.float64) @ b.astype(np.float64).T
     z = O.fp8_mfma_dot_model(a, b).astype(np.float64)
     assert (z <= exact * (1 + 2.0 ** -23)).all() and (z >= exact * (1 - 2.0 ** -10)).all()
+
+
+# ---- fp64 restatement of the FLUX blocks (oracle/flux_blocks_f64.py) ----------------------------------------------------
+def test_flux_block_restatement_closed_forms():
+    """The parts against library routines, and the wiring against cases that can be worked out by hand: with every weight
+    matrix zero a linear returns its bias, so each msa chunk, gate and residual can be set independently."""
+    from oracle import flux_blocks_f64 as FB
+
+    g = torch.Generator().manual_seed(5)
+    b, s, sc, heads, dh = 2, 6, 3, 2, 8
+    d = heads * dh
+    x = torch.randn(b, s, d, generator=g).bfloat16()
+    ctx = torch.randn(b, sc, d, generator=g).bfloat16()
+    temb = torch.randn(b, d, generator=g).bfloat16()
+    # parts
+    assert torch.allclose(FB.layer_norm(x), torch.nn.functional.layer_norm(x.double(), (d,), eps=1e-6), atol=1e-12)
+    assert torch.allclose(FB.gelu_tanh(x), torch.nn.functional.gelu(x.double(), approximate="tanh"), atol=1e-12)
+    w = (0.1 * torch.randn(24, d, generator=g)).bfloat16()
+    bias = torch.randn(24, generator=g).bfloat16()
+    y = FB.fp8_linear(x, w, bias, 0.02)
+    qa = O.fp8_scale_cast(x.reshape(-1, d).float().numpy(), np.float32(0.02), True)
+    qw, sw = O.fp8_amax_cast(w.float().numpy())
+    ref = O.fp8_gemm(qa, qw, np.float32(0.02), sw, bias.float().numpy(), out_dtype="f32")  # the pinned contract
+    assert np.allclose(y.reshape(-1, 24).numpy(), ref, rtol=1e-6, atol=1e-6)
+    # rotary embedding: identity rotation leaves the RMS-normalised vector, a quarter turn maps (n0, n1) to (-n1, n0)
+    t = torch.randn(b, s, 3 * d, generator=g).bfloat16()
+    ones = torch.ones(dh)
+    eye = torch.tensor([[1.0, 0.0], [0.0, 1.0]]).expand(b, s, dh // 2, 2, 2)
+    q, k, v = FB.qk_norm_rope(t, ones, ones, eye, heads)
+    q0 = t.double().view(b, s, 3, heads, dh)[:, :, 0]
+    assert torch.allclose(q, q0 / torch.sqrt((q0 ** 2).mean(-1, keepdim=True) + 1e-6), atol=1e-12)
+    assert torch.equal(v, t.double().view(b, s, 3, heads, dh)[:, :, 2])
+    quarter = torch.tensor([[0.0, -1.0], [1.0, 0.0]]).expand(b, s, dh // 2, 2, 2)
+    q90, _, _ = FB.qk_norm_rope(t, ones, ones, quarter, heads)
+    pairs, pairs90 = q.reshape(b, s, heads, dh // 2, 2), q90.reshape(b, s, heads, dh // 2, 2)
+    assert torch.allclose(pairs90[..., 0], -pairs[..., 1]) and torch.allclose(pairs90[..., 1], pairs[..., 0])
+    # attention of one token with itself returns its value vector
+    one_tok = FB.softmax_attention(q[:, :1], k[:, :1], v[:, :1])
+    assert torch.allclose(one_tok, v[:, :1].reshape(b, 1, d))
+
+    # wiring: all weight matrices (as good as) zero
+    names = {"norm.linear": (3 * d, d), "attn.to_qkv": (3 * d, d), "proj_mlp": (4 * d, d), "proj_out": (d, 5 * d),
+             "norm1.linear": (6 * d, d), "norm1_context.linear": (6 * d, d), "attn.to_added_qkv": (3 * d, d),
+             "attn.to_out.0": (d, d), "attn.to_add_out": (d, d), "ff.net.0.proj": (4 * d, d), "ff.net.2": (d, 4 * d),
+             "ff_context.net.0.proj": (4 * d, d), "ff_context.net.2": (d, 4 * d)}
+    sd = {}
+    for nme, (n, kk) in names.items():
+        sd[f"p.{nme}.weight"] = torch.zeros(n, kk).bfloat16()
+        sd[f"p.{nme}.weight"][0, 0] = 2.0 ** -100  # an all-zero tensor has the per-tensor scale 0 and quantises to NaN; 1e-30 vanishes in every T sum
+        sd[f"p.{nme}.bias"] = torch.zeros(n).bfloat16()
+        sd[f"p.{nme}_input_scale"] = torch.tensor([0.02])
+    for nme in ("norm_q", "norm_k", "norm_added_q", "norm_added_k"):
+        sd[f"p.attn.{nme}.weight"] = torch.ones(dh).bfloat16()
+    rope = eye.repeat(1, 1, 1, 1, 1)[:, :1].expand(b, sc + s, dh // 2, 2, 2)
+    o, c = FB.flux_double_block(sd, "p.", x, ctx, temb, rope, heads)
+    assert torch.equal(o, x.double()) and torch.equal(c, ctx.double())  # every gate is zero: both streams pass through
+    # gate_msa is chunk 2 and gate_mlp chunk 5 of norm1's output; to_out's bias and net.2's bias are what they gate
+    sd["p.norm1.linear.bias"][2 * d:3 * d] = 1.0
+    sd["p.norm1.linear.bias"][5 * d:6 * d] = 2.0
+    sd["p.attn.to_out.0.bias"][:] = 0.5
+    sd["p.ff.net.2.bias"][:] = 0.25
+    o, c = FB.flux_double_block(sd, "p.", x, ctx, temb, rope, heads)
+    assert torch.equal(o, FB._round(FB._round(x.double() + 0.5, "bf16") + 0.5, "bf16")) and torch.equal(c, ctx.double())
+    # the text stream has its own modulation (norm1_context) and its own projections
+    sd["p.norm1_context.linear.bias"][2 * d:3 * d] = -1.0
+    sd["p.attn.to_add_out.bias"][:] = 0.125
+    o2, c2 = FB.flux_double_block(sd, "p.", x, ctx, temb, rope, heads)
+    assert torch.equal(o2, o) and torch.equal(c2, FB._round(ctx.double() - 0.125, "bf16"))
+    # scale is chunk 1 and shift chunk 0: with scale = -1 the normalised tensor is the shift alone, so to_qkv (whose weight
+    # is now the identity on a constant input) sees a constant; swapping the two would feed LayerNorm(x) * (1 + 3) - 1
+    sd["p.norm1.linear.bias"][0 * d:1 * d] = 3.0
+    sd["p.norm1.linear.bias"][1 * d:2 * d] = -1.0
+    assert torch.equal(FB.modulate(x, FB.ada_msa(sd, "p.norm1.", temb, 6, "bf16", True)[1], FB.ada_msa(sd, "p.norm1.", temb, 6, "bf16", True)[0], "bf16"),
+                       torch.full((b, s, d), 3.0, dtype=torch.float64))
+    # single block: out = x + gate (chunk 2) * (proj_out bias); proj_out consumes [attn, gelu(mlp)] in that order
+    xs = torch.cat([ctx, x], dim=1)
+    sd["p.norm.linear.bias"][2 * d:3 * d] = 2.0
+    sd["p.proj_out.bias"][:] = 0.25
+    ys = FB.flux_single_block(sd, "p.", xs, temb, rope, heads)
+    assert torch.equal(ys, FB._round(xs.double() + 0.5, "bf16"))
+    sd["p.proj_out.weight"][:, :d] = torch.eye(d).bfloat16()  # picks the attention columns of the concatenation
+    sd["p.attn.to_qkv.bias"][2 * d:] = 0.75                    # v = 0.75 everywhere -> attention output 0.75
+    ys = FB.flux_single_block(sd, "p.", xs, temb, rope, heads)
+    assert torch.allclose(ys, FB._round(xs.double() + 2.0 * (0.75 + 0.25), "bf16"), atol=0.15)  # e4m3 noise on 0.75 / 0.02 only
