@@ -78,6 +78,20 @@ def cpu_baseline(torch, x, w_up, w_dn, b_up, b_dn, rows):
                       f"on dequantised e4m3 ({dt:.1f} s)"}, y
 
 
+def profiled_traffic():
+    """HBM-side bytes per launch of the roofline kernel from the committed rocprofv3 --pmc summary (a line
+    `roofline.traffic_bytes_per_launch = <number>`); (None, None) when the summary is not there."""
+    import re
+
+    rel = "profiles/bench_flux_mlp_fp8_hbm_traffic.md"
+    try:
+        with open(os.path.join(ROOT, rel)) as f:
+            m = re.search(r"roofline\.traffic_bytes_per_launch\s*=\s*([0-9.eE+]+)", f.read())
+        return (float(m.group(1)), rel) if m else (None, None)
+    except OSError:
+        return None, None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -151,6 +165,27 @@ def main():
             marks.append(e)
         return y
 
+    # Set-up, before the W warm-up steps: bring the device out of idle.  From an idle start the power management needs about
+    # 30 ms of load before it gives the compute units their sustained clock (the same GEMM takes 198 us on its first launches
+    # and 163 us from the 150th on); a serving process is past that point after its first image, a 25-step benchmark that
+    # starts cold would measure the ramp.  The chain is run until two consecutive groups of ten steps agree to 1.5 % (at
+    # most 400 steps); what it took is reported as `settle_ms`.
+    settle_t0 = time.perf_counter()
+    prev, settled_after = None, 0
+    for grp in range(40):
+        a, b = ev(), ev()
+        a.record()
+        for i in range(10):
+            step(i)
+        b.record()
+        torch.cuda.synchronize()
+        cur = a.elapsed_time(b)
+        settled_after = (grp + 1) * 10
+        if prev is not None and abs(cur - prev) <= 0.015 * prev:
+            break
+        prev = cur
+    settle_ms = (time.perf_counter() - settle_t0) * 1e3
+
     for i in range(args.warmup):
         y = step(i)
     torch.cuda.synchronize()
@@ -165,19 +200,87 @@ def main():
     value = flops_step / (dt / args.steps) / 1e12
     per = {n: sum(m[k].elapsed_time(m[k + 1]) for m in marks) / len(marks) * 1e3 for k, n in enumerate(names)}  # us
     gemm_flops = 2.0 * M * D * H
+
+    # ---- after the timed region: each kernel alone, launched back to back between ONE pair of events (no marker
+    # between launches, so no launch gap inside the figure), on the same rotating inputs
+    def batched(fn, n=20):
+        fn(0)
+        torch.cuda.synchronize()
+        a, b = ev(), ev()
+        a.record()
+        for i in range(n):
+            fn(i)
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / n * 1e3
+
+    qx0, sx0 = ops.fp8_quant(xs[0])
+    sh0 = torch.zeros(1, dtype=torch.float32, device=dev)
+    h0 = ops.fp8_linear(qx0, wp_up, sx0, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh0)
+    qh0 = ops.fp8_scale_cast(h0, sh0)
+    alone = {
+        "quant_x": batched(lambda i: ops.fp8_quant(xs[i % n_rot])),
+        "gemm_up": batched(lambda i: ops.fp8_linear(qx0, wp_up, sx0, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh0)),
+        "quant_h": batched(lambda i: ops.fp8_scale_cast(h0, sh0)),
+        "gemm_down": batched(lambda i: ops.fp8_linear(qh0, wp_dn, sh0, s_dn, bd, False, None, 0.0, torch.bfloat16)),
+    }
+    # the power argument, checkable from this line: the SAME up-projection kernel on all-zero operands (no switching in
+    # the matrix pipe, so the clock is not pulled down), and the shader clock a probe on a second stream sees while the
+    # kernel runs on random and on zero operands (idle clock for reference)
+    zq, zw = torch.zeros_like(qx0), torch.zeros_like(wp_up)
+    zeros_us = batched(lambda i: ops.fp8_linear(zq, zw, sx0, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh0))
+
+    def clock_under(fn, n=6):
+        side = torch.cuda.Stream()
+        torch.cuda.synchronize()
+        for i in range(2):
+            fn(i)  # the kernel under study is running before the probe starts
+        with torch.cuda.stream(side):
+            t = ops.shader_clock_probe(int(0.6 * n * alone["gemm_up"]), 8, side)
+        for i in range(n):
+            fn(i)
+        torch.cuda.synchronize()
+        t = t.cpu().double()
+        return round(float((0.1 * t[:, 0] / t[:, 1]).median()), 3)
+
+    clocks = {
+        "idle": clock_under(lambda i: None),
+        "up_gemm_random_operands": clock_under(lambda i: ops.fp8_linear(qx0, wp_up, sx0, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh0)),
+        "up_gemm_zero_operands": clock_under(lambda i: ops.fp8_linear(zq, zw, sx0, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh0)),
+    }
+    del zq, zw
+    vendor = None
+    try:  # the vendor library's plain FP8 GEMM on the same operands (no bias, GELU or amax), for scale only
+        a8, one = qx0.view(torch.float8_e4m3fn), torch.ones((), device=dev)
+        w8 = ops.unpack_weight(wp_up).view(torch.float8_e4m3fn)
+        vendor = round(batched(lambda i: torch._scaled_mm(a8, w8.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)), 2)
+        del w8
+    except Exception:  # not every PyTorch build exposes it
+        pass
+
     kernels = {
-        "gemm_up_fp8_4608x12288x3072": {"us": round(per["gemm_up"], 2), "TFLOP/s": round(gemm_flops / per["gemm_up"] / 1e6, 1)},
-        "gemm_down_fp8_4608x3072x12288": {"us": round(per["gemm_down"], 2), "TFLOP/s": round(gemm_flops / per["gemm_down"] / 1e6, 1)},
-        "fp8_amax_cast_4608x3072": {"us": round(per["quant_x"], 2), "GB/s": round(3.0 * M * D / per["quant_x"] / 1e3, 1)},
-        "fp8_cast_with_gemm_scale_4608x12288": {"us": round(per["quant_h"], 2), "GB/s": round(3.0 * M * H / per["quant_h"] / 1e3, 1)},
+        "gemm_up_fp8_4608x12288x3072": {"us_in_step_incl_launch_gap": round(per["gemm_up"], 2), "us_back_to_back": round(alone["gemm_up"], 2),
+                                        "TFLOP/s": round(gemm_flops / alone["gemm_up"] / 1e6, 1)},
+        "gemm_down_fp8_4608x3072x12288": {"us_in_step_incl_launch_gap": round(per["gemm_down"], 2), "us_back_to_back": round(alone["gemm_down"], 2),
+                                          "TFLOP/s": round(gemm_flops / alone["gemm_down"] / 1e6, 1)},
+        "fp8_amax_cast_4608x3072": {"us_in_step_incl_launch_gap": round(per["quant_x"], 2), "us_back_to_back": round(alone["quant_x"], 2),
+                                    "GB/s": round(3.0 * M * D / alone["quant_x"] / 1e3, 1)},
+        "fp8_cast_with_gemm_scale_4608x12288": {"us_in_step_incl_launch_gap": round(per["quant_h"], 2), "us_back_to_back": round(alone["quant_h"], 2),
+                                                "GB/s": round(3.0 * M * H / alone["quant_h"] / 1e3, 1)},
     }
     achieved = gemm_flops / per["gemm_up"] / 1e6
+    traffic, traffic_src = profiled_traffic()
     roofline = {"bound": "mfma", "kernel": "lq::gemm_kernel<fp8> 4608x12288x3072 (bias+GELU, bf16 out)",
                 "achieved": round(achieved, 1), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / FP8_PEAK_TFLOPS, 4),
-                # HBM-side bytes per launch of this kernel: rocprofv3 --pmc FETCH_SIZE (x2.0, the factor a plain copy of known
-                # size gives on this part) + WRITE_SIZE (x1.0), measured with this very command line; see profiles/
-                "traffic": 4.66e8, "traffic_unit": "bytes per launch (algorithmic: 1.65e8)"}
+                "timing": f"HIP events around the kernel on {len(marks)} of the {args.steps} timed steps, on the launch stream",
+                # HBM-side bytes per launch of this kernel: not measured in this run -- taken from the committed rocprofv3
+                # --pmc summary (FETCH_SIZE x2.0, the factor a plain copy of known size gives on this part, + WRITE_SIZE)
+                "traffic": traffic, "traffic_unit": "bytes per launch (algorithmic: 1.65e8)", "traffic_source": traffic_src,
+                "same_kernel_all_zero_operands": {"us": round(zeros_us, 2), "TFLOP/s": round(gemm_flops / zeros_us / 1e6, 1),
+                                                  "frac": round(gemm_flops / zeros_us / 1e6 / FP8_PEAK_TFLOPS, 4)},
+                "shader_clock_ghz": clocks,
+                "vendor_fp8_gemm_same_operands_us": vendor}
 
     out = {
         "metric": "W8A8/FP8 GEMM TOPS at FLUX shapes (% MFMA peak); act-quant HBM GB/s",
@@ -186,9 +289,12 @@ def main():
         "dtype": "fp8_e4m3", "data": "synthetic",
         "config": {"workload": "FLUX DiT MLP FP8 e4m3 per-tensor, M=4608: act-quant -> GEMM 3072->12288 (+bias, GELU) "
                                "-> act-quant -> GEMM 12288->3072 (+bias), bf16 in/out (BASELINE.json configs[2])",
-                   "tokens": M, "d_model": D, "d_ff": H, "profiled_tactics": tactics},
+                   "tokens": M, "d_model": D, "d_ff": H, "profiled_tactics": tactics,
+                   "settle_steps_before_warmup": settled_after, "settle_ms": round(settle_ms, 1)},
         "roofline": roofline, "kernels": kernels,
-        "kernel_timing": f"HIP events around each kernel on {len(marks)} of the {args.steps} timed steps",
+        "kernel_timing": f"us_in_step_incl_launch_gap: HIP events around each kernel on {len(marks)} of the {args.steps} timed steps "
+                         "(the event markers and the gap to the next launch are inside); us_back_to_back: 20 launches of the "
+                         "kernel alone between one pair of events, after the timed region (rates are computed from these)",
     }
     if not args.no_cpu:
         cb, y_cpu = cpu_baseline(torch, x, w_up, w_dn, b_up, b_dn, args.cpu_rows)

@@ -444,6 +444,13 @@ size_t lq_gemm_profile_workspace(lq_weight_kind_t kind, int m, int n, int k);
 int lq_gemm_profile(lq_weight_kind_t kind, int m, int n, int k, void* workspace, size_t workspace_bytes,
                     int* best_tactic, float* best_us, lq_stream_t stream);
 
+/* Measurement aid (no reference counterpart): `probes` one-wavefront workgroups each record, into
+ * out_ticks[2*i] and out_ticks[2*i+1], how far the shader clock counter and the constant 100 MHz counter advanced
+ * while they idled for `microseconds`.  100 MHz * out[2i] / out[2i+1] is the clock the compute units ran at during that
+ * window; launched on a second stream next to a kernel it tells the clock that kernel was given (the matrix kernels
+ * are power-limited on random operands).  Enqueued on `stream`, returns immediately; 1 <= probes <= 1024. */
+int lq_shader_clock_probe(uint64_t* out_ticks, int probes, unsigned microseconds, lq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

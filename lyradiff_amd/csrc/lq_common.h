@@ -178,14 +178,18 @@ __device__ __forceinline__ int cvt_i32_sat(float x) {
 }
 
 // q[i] = clamp(rint(t[i] / s), LO, HI) (NaN -> 0) for eight values, bit-identical to the IEEE
-// division but normally computed from r ~ 1/s (within 1 ulp):  |t*r - t/s| <= 2.5*2^-24*|t/s| and
-// |fl(t/s) - t/s| <= 2^-24*|t/s|, so whenever |t*r| < 512 both lie within 1.1e-4 of the true quotient;
-// if t*r is at least 2e-4 away from every tie (|t*r - rint(t*r)| <= 0.4998) the true quotient, its
-// fp32 rounding and t*r all round to the same integer.  Beyond 512 in magnitude everything saturates.
-// If any of the eight values fails the test (or the caller flags the scale as unsafe for a
-// reciprocal), the whole octet is redone with true divisions: one rarely taken branch.
+// division but normally computed from r ~ 1/s (within 1 ulp).  With Q = t/s the exact quotient:
+// |fl(t*r) - Q| <= (2^-23 + 2^-24)|Q| (reciprocal error, one rounding) and |fl(t/s) - Q| <= 2^-24 |Q|, together
+// 2.4e-7 |Q|.  Only ties up to HI - 0.5 in magnitude can change the clamped result (beyond them both candidates
+// saturate to the same bound), and there |Q| <= HI + 1: if t*r is more than tie_margin<HI>() = 2 * 2.4e-7 * (HI + 1)
+// away from every tie, the true quotient, its fp32 rounding and t*r all round to the same integer.
+// If any of the eight values fails the test (or the caller flags the scale as unsafe for a reciprocal), the whole
+// octet is redone with true divisions.  The branch is taken by a wavefront when ANY lane asks for it, so the width
+// of the margin is the frequency of the slow path: with the margin of 2e-4 first used here one step in five ran the
+// eight divisions (64 lanes x 8 values x 4e-4); with the bound above it is one in 17 for int8 and one in 250 for int4.
 // CLAMP false: the caller guarantees |t[i]| <= LIMIT * s * (1 + 2^-20) with LIMIT = HI (a scale derived from the maximum of
 // these very values), so rint(t/s) cannot leave [LO, HI] and the clamp is skipped.
+template <int HI> __device__ __forceinline__ constexpr float tie_margin() { return 2.0f * 2.4e-7f * (float)(HI + 1); }
 template <int LO, int HI, bool CLAMP = true>
 __device__ __forceinline__ void quant8(const float* t, float s, float r, bool slow, int* q) {
     float rq[8], dev = 0.0f;
@@ -195,7 +199,7 @@ __device__ __forceinline__ void quant8(const float* t, float s, float r, bool sl
         rq[i] = __builtin_rintf(qa);
         dev = fmaxf(dev, fabsf(qa - rq[i]));  // largest distance from an integer (NaN differences drop out)
     }
-    const bool risky = slow | !(dev <= 0.4998f);
+    const bool risky = slow | !(dev <= 0.5f - tie_margin<HI>());
     if (__builtin_expect(risky, 0)) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) rq[i] = __builtin_rintf(t[i] / s);
@@ -219,7 +223,7 @@ __device__ __forceinline__ uint2 quant8_pack_unclamped(const float* t, float s, 
         rq[i] = __builtin_rintf(qa);
         dev = fmaxf(dev, fabsf(qa - rq[i]));
     }
-    const bool risky = slow | !(dev <= 0.4998f);
+    const bool risky = slow | !(dev <= 0.5f - tie_margin<127>());
     if (__builtin_expect(risky, 0)) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) rq[i] = __builtin_rintf(t[i] / s);
@@ -261,8 +265,7 @@ __device__ __forceinline__ float div_by_const_fast(float a, float D, float Y) {
     float rem = __builtin_fmaf(-q0, D, a);
     return __builtin_fmaf(rem, Y, q0);
 }
-// reciprocal good to 1 ulp (hardware v_rcp_f32): enough for quant8's argument, whose margin of 2e-4
-// covers 2.5*2^-24*512 + 2^-24*512 = 1.1e-4
+// reciprocal good to 1 ulp (hardware v_rcp_f32): what quant8's error bound assumes
 __device__ __forceinline__ float fast_recip(float s) { return __builtin_amdgcn_rcpf(s); }
 
 // true when 1/s cannot be trusted as a reciprocal (zero, subnormal, infinite or NaN scale)

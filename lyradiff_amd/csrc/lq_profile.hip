@@ -49,9 +49,34 @@ static ProfileLayout profile_layout(lq_weight_kind_t kind, int m, int n, int k) 
     return L;
 }
 
+// One wavefront per workgroup reads the shader clock counter (s_memtime: ticks of the clock the compute units run at,
+// which follows the power management) and the constant 100 MHz counter (s_memrealtime), idles with s_sleep until
+// `realtime_ticks` of the latter have passed, and reads both again.  Launched on one stream while a kernel under study
+// runs on another, the ratio of the two differences is the clock that kernel was actually given.
+__global__ __launch_bounds__(64) void clock_probe_kernel(unsigned long long* out, unsigned long long realtime_ticks) {
+    if (threadIdx.x != 0) return;
+    const unsigned long long c0 = __builtin_readcyclecounter(), r0 = wall_clock64();
+    unsigned long long r1 = r0;
+    for (int spin = 0; spin < (1 << 24) && r1 - r0 < realtime_ticks; ++spin) {  // bounded: ends by itself in any case
+        __builtin_amdgcn_s_sleep(32);
+        r1 = wall_clock64();
+    }
+    const unsigned long long c1 = __builtin_readcyclecounter();
+    out[2 * blockIdx.x] = c1 - c0;
+    out[2 * blockIdx.x + 1] = r1 - r0;
+}
+
 }  // namespace lq
 
 using namespace lq;
+
+extern "C" int lq_shader_clock_probe(uint64_t* out_ticks, int probes, unsigned microseconds, lq_stream_t stream) {
+    LQ_REQUIRE(out_ticks != nullptr && probes >= 1 && probes <= 1024, LQ_ERR_ARG, "lq_shader_clock_probe: need 1..1024 probes and an output buffer");
+    LQ_REQUIRE(microseconds >= 1 && microseconds <= 100000, LQ_ERR_ARG, "lq_shader_clock_probe: 1..100000 microseconds");
+    hipLaunchKernelGGL(clock_probe_kernel, dim3((unsigned)probes), dim3(64), 0, as_stream(stream),
+                       reinterpret_cast<unsigned long long*>(out_ticks), (unsigned long long)microseconds * 100ull);
+    return check_launch("lq_shader_clock_probe");
+}
 
 extern "C" size_t lq_gemm_profile_workspace(lq_weight_kind_t kind, int m, int n, int k) {
     if (m <= 0 || n <= 0 || k <= 0 || lq_gemm_tactic_count(kind) < 0) return 0;

@@ -26,16 +26,6 @@ __global__ __launch_bounds__(256) void w4a4_quant_kernel(u32* __restrict__ q_wor
     const int ng = k >> 6;
     const int part = blockIdx.x % parts, rowblock = blockIdx.x / parts;
     const int cbase = part * SPAN;
-    if constexpr (SMOOTH == 1) {
-        for (int c = threadIdx.x * 4; c < SPAN && cbase + c < k; c += 1024) {
-            float4 d = *reinterpret_cast<const float4*>(smooth + cbase + c);
-            *reinterpret_cast<float4*>(s_dy + c) = d;
-            *reinterpret_cast<float4*>(s_dy + SPAN + c) = make_float4(1.0f / d.x, 1.0f / d.y, 1.0f / d.z, 1.0f / d.w);
-        }
-        __syncthreads();
-    }
-    // Raw row data is double buffered in registers: the loads of the wavefront's next row are in
-    // flight while the current row is quantised.
     constexpr int VPP = Elem<Tag>::bytes == 2 ? 1 : 2;  // 16-byte vectors per 8 elements
     auto load_raw = [&](int row, uint4 (*raw)[VPP]) {
         const char* rb = static_cast<const char*>(x) + (size_t)row * k * Elem<Tag>::bytes;
@@ -49,6 +39,21 @@ __global__ __launch_bounds__(256) void w4a4_quant_kernel(u32* __restrict__ q_wor
             }
         }
     };
+    // The wavefront's first row is requested before the smoothing vector is staged, so that the two memory latencies
+    // (row from HBM, vector from L2) run side by side instead of one after the other.
+    const int row0 = rowblock * 4 * rows_per_wave + wave;
+    uint4 cur[NP][VPP], nxt[NP][VPP];
+    if (row0 < m) load_raw(row0, cur);
+    if constexpr (SMOOTH == 1) {
+        for (int c = threadIdx.x * 4; c < SPAN && cbase + c < k; c += 1024) {
+            float4 d = *reinterpret_cast<const float4*>(smooth + cbase + c);
+            *reinterpret_cast<float4*>(s_dy + c) = d;
+            *reinterpret_cast<float4*>(s_dy + SPAN + c) = make_float4(1.0f / d.x, 1.0f / d.y, 1.0f / d.z, 1.0f / d.w);
+        }
+        __syncthreads();
+    }
+    // Raw row data is double buffered in registers: the loads of the wavefront's next row are in
+    // flight while the current row is quantised.
     auto unpack_raw = [&](const uint4* r, float* o) {
         if constexpr (Elem<Tag>::bytes == 2) unpack8<Tag>(r[0], o);
         else {
@@ -56,9 +61,6 @@ __global__ __launch_bounds__(256) void w4a4_quant_kernel(u32* __restrict__ q_wor
             o[4] = __uint_as_float(r[VPP - 1].x); o[5] = __uint_as_float(r[VPP - 1].y); o[6] = __uint_as_float(r[VPP - 1].z); o[7] = __uint_as_float(r[VPP - 1].w);
         }
     };
-    const int row0 = rowblock * 4 * rows_per_wave + wave;
-    uint4 cur[NP][VPP], nxt[NP][VPP];
-    if (row0 < m) load_raw(row0, cur);
     for (int j = 0; j < rows_per_wave; ++j) {
         const int row = row0 + 4 * j;
         if (row >= m) break;

@@ -67,6 +67,7 @@ SYMBOLS = {
     "lq_gemm_get_shape_tactic": (_I, [_I, _I, _I, _I]),
     "lq_gemm_profile_workspace": (_Z, [_I, _I, _I, _I]),
     "lq_gemm_profile": (_I, [_I, _I, _I, _I, _P, _Z, C.POINTER(_I), C.POINTER(_F), _P]),
+    "lq_shader_clock_probe": (_I, [_P, _I, C.c_uint, _P]),
 }
 
 

@@ -679,6 +679,16 @@ def gemm_profile(kind: str, m: int, n: int, k: int, device=None):
     return best.value, us.value
 
 
+def shader_clock_probe(microseconds: int, probes: int = 8, stream=None):
+    """Enqueues lq_shader_clock_probe on `stream` (a torch stream; default: the current one) and returns the int64 tensor
+    [probes, 2] it will fill with (shader clock ticks, 100 MHz ticks); after synchronising,
+    0.1 * t[:, 0] / t[:, 1] is the clock in GHz the compute units ran at during the window."""
+    out = torch.zeros((probes, 2), dtype=torch.int64, device="cuda")
+    st = _stream() if stream is None else stream.cuda_stream
+    _l.check(_l.load().lq_shader_clock_probe(_ptr(out), int(probes), int(microseconds), st), "lq_shader_clock_probe")
+    return out
+
+
 def gemm_shape_tactic(kind: str, m: int, n: int, k: int, tactic=None) -> int:
     """Reads (tactic=None) or writes the per-shape tactic cache; -1 removes an entry / means no entry."""
     lib = _l.load()
