@@ -1,4 +1,5 @@
-"""Builds liblyraquant.so (hand-written HIP for gfx950 behind the C ABI of include/lyraquant.h).
+"""Builds liblyraquant.so (hand-written HIP for gfx950 behind the C ABI of include/lyraquant.h) and libth_lyradiff.so
+(the torch custom classes over it).
 
     python -m lyradiff_amd.build [--force]
 
@@ -63,7 +64,33 @@ def build(force: bool = False, jobs: int | None = None) -> str:
         if r.returncode != 0:
             raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
     build_compat_check(force)
+    build_torch_classes(force)
     return LIB
+
+
+TH_LIB = os.path.join(PKG, "libth_lyradiff.so")
+
+
+def build_torch_classes(force: bool = False) -> str:
+    """Compiles th_op/th_lyradiff.cpp (torch.classes.lyradiff.*, host code only) against PyTorch's headers and links it to
+    liblyraquant.so next to it."""
+    import torch
+
+    src = os.path.join(PKG, "th_op", "th_lyradiff.cpp")
+    newest = max(os.path.getmtime(f) for f in (src, LIB, os.path.join(ROOT, "include", "lyraquant.h")))
+    if not force and os.path.exists(TH_LIB) and os.path.getmtime(TH_LIB) >= newest:
+        return TH_LIB
+    tdir = os.path.dirname(torch.__file__)
+    cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O2", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", "-Wno-deprecated-declarations",
+           "-I", os.path.join(ROOT, "include"), "-I", os.path.join(tdir, "include"),
+           "-I", os.path.join(tdir, "include", "torch", "csrc", "api", "include"), "-I", "/opt/rocm/include",
+           src, "-o", TH_LIB, "-L", os.path.join(tdir, "lib"), "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip",
+           "-L", PKG, "-llyraquant", "-Wl,-rpath,$ORIGIN"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"libth_lyradiff.so build failed:\n{r.stdout}\n{r.stderr}")
+    return TH_LIB
 
 
 def build_compat_check(force: bool = False) -> list:

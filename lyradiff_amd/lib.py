@@ -9,9 +9,43 @@ import ctypes as C
 import os
 
 PKG = os.path.dirname(os.path.abspath(__file__))
-# LYRA_LIB_PATH is the variable the reference's Python wrapper reads (lyradiff/__init__.py:4-5); LYRA_LIB_PATH_AMD wins
-# when both are set (a machine that also carries the reference's CUDA build)
-LIB_PATH = os.environ.get("LYRA_LIB_PATH_AMD") or os.environ.get("LYRA_LIB_PATH") or os.path.join(PKG, "liblyraquant.so")
+
+
+def _paths():
+    """(C-ABI library, torch custom-class library).  LYRA_LIB_PATH is the variable the reference's Python wrapper hands to
+    torch.classes.load_library (lyradiff/__init__.py:4-5): here it names libth_lyradiff.so, and liblyraquant.so is taken
+    from the same directory (the class library links it by $ORIGIN); a LYRA_LIB_PATH that names liblyraquant.so itself is
+    accepted too.  LYRA_LIB_PATH_AMD names liblyraquant.so directly and wins (a machine that also carries the reference's
+    CUDA build).  Without either, the in-tree build."""
+    ref = os.environ.get("LYRA_LIB_PATH")
+    th = os.path.join(PKG, "libth_lyradiff.so")
+    abi = os.path.join(PKG, "liblyraquant.so")
+    if ref:
+        if os.path.basename(ref).startswith("liblyraquant"):
+            abi, th = ref, os.path.join(os.path.dirname(ref), "libth_lyradiff.so")
+        else:
+            th, abi = ref, os.path.join(os.path.dirname(os.path.abspath(ref)), "liblyraquant.so")
+    return os.environ.get("LYRA_LIB_PATH_AMD") or abi, th
+
+
+LIB_PATH, TH_LIB_PATH = _paths()
+_th_loaded = False
+
+
+def load_torch_classes():
+    """torch.classes.load_library on libth_lyradiff.so: registers torch.classes.lyradiff.FluxTransformerBlockOp,
+    FluxSingleTransformerBlockOp and LyraDiffCommonContext (th_op/th_lyradiff.cpp).  Fails loudly when the library is missing."""
+    global _th_loaded
+    if not _th_loaded:
+        import torch
+
+        if not os.path.exists(TH_LIB_PATH):
+            raise ImportError(f"{TH_LIB_PATH} not found: run `python -m lyradiff_amd.build` (there is no Python fallback behind "
+                              "torch.classes.lyradiff)")
+        torch.classes.load_library(TH_LIB_PATH)
+        _th_loaded = True
+    return TH_LIB_PATH
+
 
 LQ_F32, LQ_F16, LQ_BF16, LQ_I32 = 0, 1, 2, 3
 LQ_W_INT8, LQ_W_FP8, LQ_W_INT4 = 0, 1, 2

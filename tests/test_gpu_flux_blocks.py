@@ -745,18 +745,9 @@ def test_flux_block_ops_reload_model_from_bin(ops, dev, tmp_path, file_dtype):
         sf.reload_model_from_bin(str(tmp_path) + "/absent.", "fp32")
 
 
-@pytest.mark.parametrize("full", [True, False])
-def test_flux_int4_block_ops(ops, dev, full):
-    """Quant levels INT4_W4A4 (16-bit adaLN linear) and INT4_W4A4_FULL (FP8 adaLN linear) of the block classes: the op output
-    equals the block function driven with the same attention core, and the block function equals its steps one by one."""
-    from lyradiff_amd import flux_fp8 as F8
-    from lyradiff_amd import flux_int4 as F
-    from lyradiff_amd import flux_ops as FO
-
-    b, s, sc, heads, dh = 1, 128, 64, 4, 64
-    d = heads * dh
-    g = rng_t(401)
-    level = FO.LyraQuantLevel.INT4_W4A4_FULL if full else FO.LyraQuantLevel.INT4_W4A4
+def _int4_block_state(d, dh, g):
+    """State dict of one double ("transformer_blocks.0.") and one single ("single_transformer_blocks.0.") INT4 block in the
+    reference's container layout; the adaLN linears carry FP8 input scales, which the non-FULL level ignores."""
     sd = {}
     for pre, ada in (("transformer_blocks.0.", ("norm1.linear", "norm1_context.linear")), ("single_transformer_blocks.0.", ("norm.linear",))):
         chunks = 6 if len(ada) == 2 else 3
@@ -775,6 +766,22 @@ def test_flux_int4_block_ops(ops, dev, full):
     sd.update(_int4_state("single_transformer_blocks.0.proj_mlp.", 4 * d, d, g))
     sd.update(_int4_state("single_transformer_blocks.0.proj_out.linears.0.", d, d, g))
     sd.update(_int4_state("single_transformer_blocks.0.proj_out.linears.1.linear.", d, 4 * d, g, bias=False))
+    return sd
+
+
+@pytest.mark.parametrize("full", [True, False])
+def test_flux_int4_block_ops(ops, dev, full):
+    """Quant levels INT4_W4A4 (16-bit adaLN linear) and INT4_W4A4_FULL (FP8 adaLN linear) of the block classes: the op output
+    equals the block function driven with the same attention core, and the block function equals its steps one by one."""
+    from lyradiff_amd import flux_fp8 as F8
+    from lyradiff_amd import flux_int4 as F
+    from lyradiff_amd import flux_ops as FO
+
+    b, s, sc, heads, dh = 1, 128, 64, 4, 64
+    d = heads * dh
+    g = rng_t(401)
+    level = FO.LyraQuantLevel.INT4_W4A4_FULL if full else FO.LyraQuantLevel.INT4_W4A4
+    sd = _int4_block_state(d, dh, g)
     x = torch.randn(b, s, d, generator=g).bfloat16().to(dev)
     ctx = torch.randn(b, sc, d, generator=g).bfloat16().to(dev)
     temb = torch.randn(b, d, generator=g).bfloat16().to(dev)
