@@ -11,6 +11,11 @@
 
 namespace lq {
 
+// A tensor of at least this many bytes that a kernel touches exactly once (the 16-bit output of a GEMM that a cast pass
+// consumes, the input of that cast pass) is moved with nontemporal loads / stores: streaming it through the 256 MB last-level
+// cache would displace the operands the GEMMs around it re-read.
+constexpr size_t kStreamBytes = (size_t)64 << 20;
+
 // ---- error plumbing ---------------------------------------------------------------------------
 void set_error(const char* fmt, ...);  // stores the message for lq_last_error() (thread local)
 extern int g_tactic_int8, g_tactic_fp8, g_tactic_w4a4;  // process-wide forced tile configuration, -1 = none

@@ -50,6 +50,11 @@ struct GemmParams {
     uint8_t* C8;            // optional: e4m3 codes of C with a given (static) scale, written next to or instead of C
     const float* c8_scale;  // scale of C8: C8 = e4m3(f32(T(y)) * (1 / c8_scale[0]))
     size_t ldc8;            // row pitch of C8 in bytes (n when the codes are dense)
+    // C is written with nontemporal stores: set for an output that is read once, by one streaming pass (the cast of a
+    // dynamic-scale chain: out_scale given), and is too large to share the 256 MB last-level cache with the operands of
+    // the GEMM after it.  Measured on the FLUX MLP chain (113 MB hidden tensor): up + cast + down 340-353 -> 319-330 us
+    // together with the nontemporal loads of the cast.
+    int stream_c;
     // gelu: 0 none, 1 on the fp32 value, 2 on the value rounded to T first (the activation applied by a separate
     // kernel to a stored T tensor)
     // gate: C = T( T( T(y) * gate[m / gate_rows, n] ) + residual[m, n] ), the roundings of a GEMM that stores T
@@ -95,6 +100,9 @@ __device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, i
     tn = in_band / rows;
 }
 
+// store4_stream: the same store with the nontemporal hint, for an output that one streaming pass reads once (see
+// GemmParams::stream_c): its lines then do not displace the next kernel's operands from the last-level cache
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
 template <typename OutTag> struct OutStore;
 template <> struct OutStore<F16Tag> {
     static __device__ __forceinline__ void store4(void* C, size_t idx, const float* y) {
@@ -102,6 +110,10 @@ template <> struct OutStore<F16Tag> {
         o.x = pack2_f16(y[0], y[1]);
         o.y = pack2_f16(y[2], y[3]);
         *reinterpret_cast<uint2*>(static_cast<unsigned short*>(C) + idx) = o;
+    }
+    static __device__ __forceinline__ void store4_stream(void* C, size_t idx, const float* y) {
+        const u32x2_t o = {pack2_f16(y[0], y[1]), pack2_f16(y[2], y[3])};
+        __builtin_nontemporal_store(o, reinterpret_cast<u32x2_t*>(static_cast<unsigned short*>(C) + idx));
     }
     static __device__ __forceinline__ void load4(const void* P, size_t idx, float* y) {
         uint2 v = *reinterpret_cast<const uint2*>(static_cast<const unsigned short*>(P) + idx);
@@ -116,6 +128,10 @@ template <> struct OutStore<BF16Tag> {
         o.y = pack2_bf16(y[2], y[3]);
         *reinterpret_cast<uint2*>(static_cast<unsigned short*>(C) + idx) = o;
     }
+    static __device__ __forceinline__ void store4_stream(void* C, size_t idx, const float* y) {
+        const u32x2_t o = {pack2_bf16(y[0], y[1]), pack2_bf16(y[2], y[3])};
+        __builtin_nontemporal_store(o, reinterpret_cast<u32x2_t*>(static_cast<unsigned short*>(C) + idx));
+    }
     static __device__ __forceinline__ void load4(const void* P, size_t idx, float* y) {
         uint2 v = *reinterpret_cast<const uint2*>(static_cast<const unsigned short*>(P) + idx);
         y[0] = bf16_bits_to_f32(v.x & 0xFFFF); y[1] = bf16_bits_to_f32(v.x >> 16);
@@ -126,6 +142,7 @@ template <> struct OutStore<F32Tag> {
     static __device__ __forceinline__ void store4(void* C, size_t idx, const float* y) {
         *reinterpret_cast<float4*>(static_cast<float*>(C) + idx) = make_float4(y[0], y[1], y[2], y[3]);
     }
+    static __device__ __forceinline__ void store4_stream(void* C, size_t idx, const float* y) { store4(C, idx, y); }
     static __device__ __forceinline__ void load4(const void* P, size_t idx, float* y) {
         float4 v = *reinterpret_cast<const float4*>(static_cast<const float*>(P) + idx);
         y[0] = v.x; y[1] = v.y; y[2] = v.z; y[3] = v.w;
@@ -708,6 +725,11 @@ struct GemmKernel {
                         }
                         if constexpr (GEN) {
                             if (ok && p.C != nullptr) OutStore<OutTag>::store4(p.C, idx, y);
+                        } else if constexpr (kExtras && MODE == E_ACT) {
+                            if (ok) {
+                                if (p.stream_c) OutStore<OutTag>::store4_stream(p.C, idx, y);
+                                else OutStore<OutTag>::store4(p.C, idx, y);
+                            }
                         } else if constexpr (MODE != E_CODES) {
                             if (ok) OutStore<OutTag>::store4(p.C, idx, y);
                         }

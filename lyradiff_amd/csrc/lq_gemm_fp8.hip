@@ -73,6 +73,8 @@ extern "C" int lq_gemm_fp8_ex(void* C, lq_dtype_t out_dtype, const uint8_t* A, c
     p.gelu = gelu; p.residual = (beta != 0.0f) ? residual : nullptr; p.beta = beta;
     p.out_scale = out_scale; p.C8 = C_fp8; p.c8_scale = C_fp8_scale; p.ldc8 = (size_t)n;
     p.m = m; p.n = n; p.k = k; p.kb = k;
+    // with out_scale the 16-bit output exists to be cast once with that scale; a large one bypasses the cache on its way out
+    p.stream_c = out_scale != nullptr && C != nullptr && (size_t)m * (size_t)n * (out_dtype == LQ_F32 ? 4 : 2) >= kStreamBytes;
     return fp8_dispatch("lq_gemm_fp8", p, out_dtype, stream);
 }
 

@@ -16,11 +16,19 @@ template <typename Tag> struct Chunk16 {  // 16 consecutive elements of a 16-bit
     static constexpr int elems = Elem<Tag>::bytes == 2 ? 16 : 8;
 };
 
-template <typename Tag>
+template <typename Tag, bool NT = false>
 __device__ __forceinline__ void load_elems(const void* base, size_t idx, float* o) {
     if constexpr (Elem<Tag>::bytes == 2) {
-        const uint4* p = reinterpret_cast<const uint4*>(static_cast<const char*>(base) + idx * 2);
-        uint4 a = p[0], b = p[1];
+        uint4 a, b;
+        if constexpr (NT) {  // read-once input of a large cast: do not keep its lines in the caches
+            typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+            const u32x4_t* p = reinterpret_cast<const u32x4_t*>(static_cast<const char*>(base) + idx * 2);
+            const u32x4_t a4 = __builtin_nontemporal_load(p), b4 = __builtin_nontemporal_load(p + 1);
+            a = make_uint4(a4.x, a4.y, a4.z, a4.w), b = make_uint4(b4.x, b4.y, b4.z, b4.w);
+        } else {
+            const uint4* p = reinterpret_cast<const uint4*>(static_cast<const char*>(base) + idx * 2);
+            a = p[0], b = p[1];
+        }
         unpack8<Tag>(a, o);
         unpack8<Tag>(b, o + 8);
     } else {
@@ -94,7 +102,7 @@ __global__ __launch_bounds__(256) void fp8_amax_kernel(float* __restrict__ scale
     }
 }
 
-template <typename Tag>
+template <typename Tag, bool NT>
 __global__ __launch_bounds__(256) void fp8_cast_kernel(uint8_t* __restrict__ dst, const void* __restrict__ src,
                                                        const float* __restrict__ scale, int invert, size_t n) {
     constexpr int E = Chunk16<Tag>::elems;
@@ -103,7 +111,7 @@ __global__ __launch_bounds__(256) void fp8_cast_kernel(uint8_t* __restrict__ dst
     const size_t nchunks = n / E;
     for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < nchunks; c += (size_t)gridDim.x * blockDim.x) {
         float v[16];
-        load_elems<Tag>(src, c * E, v);
+        load_elems<Tag, NT>(src, c * E, v);
         u32 w[4];
 #pragma unroll
         for (int i = 0; i < E / 4; ++i)
@@ -546,7 +554,10 @@ template <typename Tag> static int launch_amax(float* scale, const void* x, size
 template <typename Tag>
 static int launch_cast(uint8_t* dst, const void* src, const float* scale, int invert, size_t n, hipStream_t st) {
     if (reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0) {
-        hipLaunchKernelGGL((fp8_cast_kernel<Tag>), dim3(stream_grid(n, Chunk16<Tag>::elems)), dim3(256), 0, st, dst, src, scale, invert, n);
+        if (n * Elem<Tag>::bytes >= kStreamBytes)
+            hipLaunchKernelGGL((fp8_cast_kernel<Tag, true>), dim3(stream_grid(n, Chunk16<Tag>::elems)), dim3(256), 0, st, dst, src, scale, invert, n);
+        else
+            hipLaunchKernelGGL((fp8_cast_kernel<Tag, false>), dim3(stream_grid(n, Chunk16<Tag>::elems)), dim3(256), 0, st, dst, src, scale, invert, n);
     } else {
         hipLaunchKernelGGL((fp8_cast_scalar_kernel<Tag>), dim3(stream_grid(n, 4)), dim3(256), 0, st, dst, src, scale, invert, n);
     }
