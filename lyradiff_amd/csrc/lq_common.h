@@ -132,7 +132,9 @@ template <typename Tag> __device__ __forceinline__ void unpack8(const uint4& v, 
 // quad_perm [1,0,3,2] and [2,3,0,1] exchange with the lanes at distance 1 and 2, row_half_mirror
 // and row_mirror bring in the other quad / the other half of the row.
 template <int CTRL> __device__ __forceinline__ int dpp_i32(int v) {
-    return __builtin_amdgcn_update_dpp(v, v, CTRL, 0xF, 0xF, false);
+    // every lane has a valid source under these swizzles, so the "old" operand never shows; passing 0 instead of v
+    // leaves the move free to fold into the instruction that uses it (v_max_i32_dpp: one instruction per step, not three)
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
 }
 // max over aligned groups of 8 consecutive lanes of a NON-NEGATIVE float (or +NaN pattern), result in
 // every lane of the group.  Non-negative floats order like their bit patterns, so the steps run as

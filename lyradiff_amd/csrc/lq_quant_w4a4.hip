@@ -12,8 +12,13 @@ namespace lq {
 // SMOOTH 0: no smoothing vector; 1: the divisors d of the workgroup's column range and their correctly
 // rounded reciprocals y = fl(1/d) are computed once per workgroup into LDS and shared by the rows of
 // its four wavefronts.
-template <typename Tag, int NP, bool F16_SCALE, int SMOOTH>
-__global__ __launch_bounds__(256) void w4a4_quant_kernel(u32* __restrict__ q_words, void* __restrict__ scales,
+// WAVES: wavefronts (= rows in flight) per workgroup.  The staging of the smoothing vector costs a workgroup one IEEE division
+// per column of its range whatever its size, so sixteen rows per workgroup would pay a quarter of what four pay -- measured
+// slower all the same (15.4 against 14.7 us at 4608x3072 from HBM: sixteen wavefronts wait at one barrier for the staging's
+// load and division chain, where small workgroups on a CU are in different phases), so four it stays.
+// FULL: k is a multiple of the column range, no lane is ever out of range.
+template <typename Tag, int NP, bool F16_SCALE, int SMOOTH, int WAVES = 4, bool FULL = false>
+__global__ __launch_bounds__(WAVES * 64) void w4a4_quant_kernel(u32* __restrict__ q_words, void* __restrict__ scales,
                                                          const void* __restrict__ x,
                                                          const float* __restrict__ smooth, int m, int k,
                                                          int rows_per_wave, int parts) {
@@ -34,18 +39,18 @@ __global__ __launch_bounds__(256) void w4a4_quant_kernel(u32* __restrict__ q_wor
             int col = cbase + (p * 64 + lane) * 8;
 #pragma unroll
             for (int u = 0; u < VPP; ++u) {
-                raw[p][u] = make_uint4(0, 0, 0, 0);
-                if (col < k) raw[p][u] = *reinterpret_cast<const uint4*>(rb + (size_t)col * Elem<Tag>::bytes + u * 16);
+                if constexpr (!FULL) raw[p][u] = make_uint4(0, 0, 0, 0);
+                if (FULL || col < k) raw[p][u] = *reinterpret_cast<const uint4*>(rb + (size_t)col * Elem<Tag>::bytes + u * 16);
             }
         }
     };
     // The wavefront's first row is requested before the smoothing vector is staged, so that the two memory latencies
     // (row from HBM, vector from L2) run side by side instead of one after the other.
-    const int row0 = rowblock * 4 * rows_per_wave + wave;
+    const int row0 = rowblock * WAVES * rows_per_wave + wave;
     uint4 cur[NP][VPP], nxt[NP][VPP];
     if (row0 < m) load_raw(row0, cur);
     if constexpr (SMOOTH == 1) {
-        for (int c = threadIdx.x * 4; c < SPAN && cbase + c < k; c += 1024) {
+        for (int c = threadIdx.x * 4; c < SPAN && cbase + c < k; c += WAVES * 256) {
             float4 d = *reinterpret_cast<const float4*>(smooth + cbase + c);
             *reinterpret_cast<float4*>(s_dy + c) = d;
             *reinterpret_cast<float4*>(s_dy + SPAN + c) = make_float4(1.0f / d.x, 1.0f / d.y, 1.0f / d.z, 1.0f / d.w);
@@ -62,10 +67,10 @@ __global__ __launch_bounds__(256) void w4a4_quant_kernel(u32* __restrict__ q_wor
         }
     };
     for (int j = 0; j < rows_per_wave; ++j) {
-        const int row = row0 + 4 * j;
+        const int row = row0 + WAVES * j;
         if (row >= m) break;
-        const bool has_next = j + 1 < rows_per_wave && row + 4 < m;
-        if (has_next) load_raw(row + 4, nxt);
+        const bool has_next = j + 1 < rows_per_wave && row + WAVES < m;
+        if (has_next) load_raw(row + WAVES, nxt);
         const char* rb = static_cast<const char*>(x) + (size_t)row * k * Elem<Tag>::bytes;
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
@@ -82,7 +87,7 @@ __global__ __launch_bounds__(256) void w4a4_quant_kernel(u32* __restrict__ q_wor
                 // patterns of |v| so that an inf or NaN anywhere in the group also takes the exact path.
                 float dv[8], yv[8];
                 {
-                    const int cc = col < k ? col - cbase : 0;
+                    const int cc = (FULL || col < k) ? col - cbase : 0;
                     float4 a = *reinterpret_cast<const float4*>(s_dy + cc), b = *reinterpret_cast<const float4*>(s_dy + cc + 4);
                     float4 c = *reinterpret_cast<const float4*>(s_dy + SPAN + cc), d = *reinterpret_cast<const float4*>(s_dy + SPAN + cc + 4);
                     dv[0] = a.x; dv[1] = a.y; dv[2] = a.z; dv[3] = a.w; dv[4] = b.x; dv[5] = b.y; dv[6] = b.z; dv[7] = b.w;
@@ -134,7 +139,7 @@ __global__ __launch_bounds__(256) void w4a4_quant_kernel(u32* __restrict__ q_wor
             u32 word = 0;
 #pragma unroll
             for (int i = 0; i < 8; ++i) word = __builtin_amdgcn_alignbit((u32)q[i], word, 4);
-            if (col < k) {
+            if (FULL || col < k) {
                 q_words[(size_t)row * (k >> 3) + (col >> 3)] = word;
                 if ((lane & 7) == 0) {
                     size_t si = (size_t)row * ng + (col >> 6);
@@ -197,6 +202,15 @@ extern "C" int lq_w4a4_quantize(uint32_t* q_words, void* scales, lq_dtype_t scal
     const bool f16s = scale_dtype == LQ_F16;
     const int smode = smooth == nullptr ? 0 : 1;
     const size_t lds = smode == 1 ? 2 * (size_t)np * 512 * sizeof(float) : 0;
+    // long rows whose length is a whole number of column ranges (FLUX: 3072): no range checks
+    if (smode == 1 && np == 2 && k % 1024 == 0 && x_dtype != LQ_F32) {
+#define LQ_W4_FULL(TAG, F16S) \
+    hipLaunchKernelGGL((w4a4_quant_kernel<TAG, 2, F16S, 1, 4, true>), grid, block, lds, st, q_words, scales, x, smooth, m, k, rpw, parts)
+        if (x_dtype == LQ_F16) { if (f16s) LQ_W4_FULL(F16Tag, true); else LQ_W4_FULL(F16Tag, false); }
+        else { if (f16s) LQ_W4_FULL(BF16Tag, true); else LQ_W4_FULL(BF16Tag, false); }
+#undef LQ_W4_FULL
+        return check_launch("w4a4_quantize");
+    }
 #define LQ_W4_LAUNCH2(TAG, NPV, F16S, SM) \
     hipLaunchKernelGGL((w4a4_quant_kernel<TAG, NPV, F16S, SM>), grid, block, lds, st, q_words, scales, x, smooth, m, k, rpw, parts)
 #define LQ_W4_LAUNCH(TAG, NPV)                                                     \
