@@ -425,6 +425,11 @@ def extra_kernels(torch, ops, dev):
             wp = ops.repack_weight_only(q, kind)
             us = timeit(lambda: ops.weight_only_linear(x, wp, sc, None, kind), iters=20, warm=3)
             res[f"gemm_weight_only_{kind}_{name}_{m}x{n}x{k}"] = {"us": round(us, 2), "TFLOP/s": round(2.0 * m * n * k / us / 1e6, 1)}
+            if kind == "int4":  # group-wise scales and zero points (group 128), dequantised per weight in the main loop
+                gs = (torch.rand(k // 128, n, generator=g) * 0.01).to(dt).to(dev)
+                gz = (torch.randn(k // 128, n, generator=g) * 0.01).to(dt).to(dev)
+                us = timeit(lambda: ops.weight_only_linear_grouped(x, wp, gs, gz, None, kind, 128), iters=20, warm=3)
+                res[f"gemm_weight_only_{kind}_g128_zeros_{name}_{m}x{n}x{k}"] = {"us": round(us, 2), "TFLOP/s": round(2.0 * m * n * k / us / 1e6, 1)}
     res.update(flux_block_times(torch, ops, dev, timeit))
     res.update(flux_linear_chain_1280(torch, ops, dev, timeit))
     res.update(sdxl_geglu_ffn_chain(torch, ops, dev, timeit))

@@ -230,6 +230,16 @@ inline void repackWeight(void* dst_rows32, const void* src_row_major, lq_weight_
 // A configuration is one of the library's tile configurations; tile_config = -1 means "choose"
 // (ChooseWithHeuristic).  split_k_factor and stages are carried for source compatibility only: the
 // reference's launcher never applies split-k either (int8_gemm_template.h:146-148).
+// ---- kernels/cutlass_extensions/include/cutlass_extensions/weight_only_quant_op.h:9-25 ------------------------
+namespace cutlass {
+enum class WeightOnlyQuantOp { UNDEFINED, PER_COLUMN_SCALE_ONLY, FINEGRAINED_SCALE_ONLY, FINEGRAINED_SCALE_AND_ZEROS };
+constexpr bool isFinegrained(WeightOnlyQuantOp op) {
+    return op == WeightOnlyQuantOp::FINEGRAINED_SCALE_AND_ZEROS || op == WeightOnlyQuantOp::FINEGRAINED_SCALE_ONLY;
+}
+constexpr bool hasZero(WeightOnlyQuantOp op) { return op == WeightOnlyQuantOp::FINEGRAINED_SCALE_AND_ZEROS; }
+struct uint4b_t {};  // tag for 4-bit weights (two per byte); only used as a template argument here
+}  // namespace cutlass
+
 namespace cutlass_extensions {
 struct CutlassGemmConfig {
     int tile_config = -1;
@@ -273,6 +283,43 @@ public:
         for (int t = 0; t < lq_gemm_tactic_count(LQ_W_INT8); ++t) configs.emplace_back(t, 1, -1);
         return configs;
     }
+};
+
+// ---- kernels/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm.h:25-180 (weight-only W8A16 / W4A16) ---------------------
+// B is the buffer lq_repack_weight_only made from the unprocessed codes (same size as the reference's preprocessed
+// weight); scales [n] for PER_COLUMN_SCALE_ONLY, scales and zero points [k / group_size, n] for the FINEGRAINED ops.
+// The alpha overloads, the fp8 activation form and the split-k workspace of the reference are not carried.
+template <typename ActivationType, typename WeightType, cutlass::WeightOnlyQuantOp QuantOp>
+class CutlassFpAIntBGemmRunner {
+    static_assert(std::is_same<WeightType, uint8_t>::value || std::is_same<WeightType, cutlass::uint4b_t>::value,
+                  "WeightType must be uint8_t or cutlass::uint4b_t");
+    static constexpr lq_weight_kind_t kKind = std::is_same<WeightType, uint8_t>::value ? LQ_W_INT8 : LQ_W_INT4;
+
+public:
+    void gemm(void const* A, void const* B, void const* weight_scales, void* C, int m, int n, int k,
+              cutlass_extensions::CutlassGemmConfig /*gemmConfig*/, char* /*workspace_ptr*/, const size_t /*workspace_bytes*/,
+              hipStream_t stream) {
+        static_assert(QuantOp == cutlass::WeightOnlyQuantOp::PER_COLUMN_SCALE_ONLY, "per-column overload");
+        detail::check(lq_gemm_weight_only(C, A, detail::DType<ActivationType>::value, static_cast<const uint8_t*>(B), kKind,
+                                          weight_scales, nullptr, m, n, k, stream),
+                      "CutlassFpAIntBGemmRunner::gemm");
+    }
+    void gemm(void const* A, void const* B, void const* weight_scales, void const* weight_zero_points, void const* biases, void* C,
+              int m, int n, int k, int const group_size, cutlass_extensions::CutlassGemmConfig /*gemmConfig*/,
+              char* /*workspace_ptr*/, const size_t /*workspace_bytes*/, hipStream_t stream) {
+        int status;
+        if (QuantOp == cutlass::WeightOnlyQuantOp::PER_COLUMN_SCALE_ONLY)
+            status = lq_gemm_weight_only(C, A, detail::DType<ActivationType>::value, static_cast<const uint8_t*>(B), kKind,
+                                         weight_scales, biases, m, n, k, stream);
+        else
+            status = lq_gemm_weight_only_grouped(C, A, detail::DType<ActivationType>::value, static_cast<const uint8_t*>(B), kKind,
+                                                 weight_scales,
+                                                 QuantOp == cutlass::WeightOnlyQuantOp::FINEGRAINED_SCALE_AND_ZEROS ? weight_zero_points : nullptr,
+                                                 biases, m, n, k, group_size, stream);
+        detail::check(status, "CutlassFpAIntBGemmRunner::gemm");
+    }
+    size_t getWorkspaceSize(int const, int const, int const) { return 0; }
+    std::vector<cutlass_extensions::CutlassGemmConfig> getConfigs() const { return {cutlass_extensions::CutlassGemmConfig(0, 1, -1)}; }
 };
 }  // namespace cutlass_kernels
 

@@ -265,6 +265,20 @@ int lq_fp8_scale_cast_2d(uint8_t* dst, size_t dst_ld, const void* src, size_t sr
 int lq_gemm_weight_only(void* C, const void* A, lq_dtype_t dtype, const uint8_t* B_prepared, lq_weight_kind_t kind,
                         const void* scales, const void* bias, int m, int n, int k, lq_stream_t stream);
 
+/* The same GEMM with group-wise ("fine-grained") scales and optional zero points along k:
+ *   C[m,n] = T( sum_k A[m,k] * w[k,n] [+ f32(bias[n])] ),  w[k,n] the dequantised weight formed in T per element:
+ *     F16:   w = T( T(q[k,n] * scale[k/g, n]) + zero[k/g, n] )      (multiply, then add: two roundings)
+ *     BF16:  w = T( q[k,n] * scale[k/g, n] + zero[k/g, n] )         (one fused multiply-add)
+ *   and w = T(q * scale) for both when `zeros` is NULL; q is the signed code (the +128 / +8 of the prepared layout removed).
+ * scales and zeros are row-major [k / group_size, n] of `dtype`; group_size 64 or 128, k % group_size == 0.
+ * Replaces CutlassFpAIntBGemmRunner<T, uint8_t | uint4b_t, FINEGRAINED_SCALE_ONLY | FINEGRAINED_SCALE_AND_ZEROS>::gemm(A, B,
+ * weight_scales, weight_zero_points, biases, C, m, n, k, group_size, ...) (kernels/cutlass_kernels/fpA_intB_gemm/
+ * fpA_intB_gemm.h:58-85); the per-element arithmetic is that of its MmaTensorOpDequantizer
+ * (kernels/cutlass_extensions/include/cutlass_extensions/gemm/warp/mma_tensorop_dequantizer.h:150-222,370-390). */
+int lq_gemm_weight_only_grouped(void* C, const void* A, lq_dtype_t dtype, const uint8_t* B_prepared, lq_weight_kind_t kind,
+                                const void* scales, const void* zeros, const void* bias, int m, int n, int k, int group_size,
+                                lq_stream_t stream);
+
 /* One-time preparation of a weight-only weight: src_kn is the row-major [k, n] matrix of signed codes as
  * symmetric_quantize leaves it before preprocessing ("unprocessed_quantized_weight": int8, or for INT4 [k, n/2] bytes
  * with column 2j in the low nibble; kernels/cutlass_kernels/cutlass_preprocessors.cpp:532-631).  dst (k*n bytes for

@@ -17,6 +17,13 @@
 // The scale is applied once per output in the epilogue (the reference multiplies every dequantised weight by the
 // scale in T inside the main loop, which rounds each weight; results agree to that rounding).
 //
+// Group-wise ("fine-grained") scales, with or without zero points (FINEGRAINED_SCALE_ONLY / FINEGRAINED_SCALE_AND_ZEROS,
+// group 64 or 128 along k, scales and zeros [k / group, n] of T): every dequantised weight is formed in T inside the main
+// loop as the reference's MmaTensorOpDequantizer does (cutlass_extensions/gemm/warp/mma_tensorop_dequantizer.h:150-222,
+// 370-390): fp16  w = T(T(q * s) + z)  (multiply, then add, one packed instruction each);  bf16  w = T(fma(q, s, z))
+// (evaluated in fp32 and rounded once to bf16; q * s is exact in fp32).  The k-tile of 64 lies inside one group; the
+// scales (and zeros) of the tile's output channels travel to LDS with the operands (one 4-byte transfer per lane).
+//
 // Tiling: 256x128 outputs per workgroup of four wavefronts (2x2), 128x64 per wavefront (eight 32x32 MFMA tiles:
 // every converted weight fragment is used by four MFMAs), k-tile 64, two LDS stages filled from registers
 // (activations XOR-swizzled, weights copied as they lie), the next tile's global loads in flight during the MFMAs.
@@ -32,50 +39,63 @@ template <int CH> __device__ __forceinline__ int wo_swizzle(int row) {  // 8 chu
     return ((row >> 1) & 7) ^ ((row & 1) << 2);
 }
 
-// eight consecutive-k weights of one output channel as 16-bit floats (one 16-byte MFMA operand), from unsigned codes
-template <bool F16, bool W4> struct WoCvt;
-template <> struct WoCvt<true, false> {  // fp16 <- uint8: d0 holds k0..k3, d1 holds k4..k7
-    static __device__ __forceinline__ v4i run(u32 d0, u32 d1) {
+// eight consecutive-k weights of one output channel as 16-bit floats (one 16-byte MFMA operand), from unsigned codes.
+// G = 0: the bare integer values (the per-channel scale is applied to the sums); 1: times the group's scale; 2: times the
+// scale plus the zero point.  s2 / z2: the scale and zero of the lane's channel, as a pair of fp16 (fp16 path) or as fp32
+// bit patterns (bf16 path).
+template <bool F16, bool W4, int G> struct WoCvt;
+template <int G> __device__ __forceinline__ int wo_apply_h2(h2_t q, u32 s2, u32 z2) {
+    if constexpr (G >= 1) q = q * __builtin_bit_cast(h2_t, s2);   // v_pk_mul_f16: T(q * s)
+    if constexpr (G == 2) q = q + __builtin_bit_cast(h2_t, z2);   // v_pk_add_f16: T(. + z)
+    return __builtin_bit_cast(int, q);
+}
+template <int G> __device__ __forceinline__ float wo_apply_f32(float q, u32 s, u32 z) {
+    if constexpr (G == 1) return q * __uint_as_float(s);                                      // exact in fp32
+    if constexpr (G == 2) return __builtin_fmaf(q, __uint_as_float(s), __uint_as_float(z));
+    return q;
+}
+template <int G> struct WoCvt<true, false, G> {  // fp16 <- uint8: d0 holds k0..k3, d1 holds k4..k7
+    static __device__ __forceinline__ v4i run(u32 d0, u32 d1, u32 s2, u32 z2) {
         v4i o;
         const h2_t off = {(_Float16)1152.0f, (_Float16)1152.0f};
         const u32 p[4] = {__builtin_amdgcn_perm(0x64646464u, d0, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, d0, 0x04030402u),
                           __builtin_amdgcn_perm(0x64646464u, d1, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, d1, 0x04030402u)};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = __builtin_bit_cast(int, __builtin_bit_cast(h2_t, p[i]) - off);
+        for (int i = 0; i < 4; ++i) o[i] = wo_apply_h2<G>(__builtin_bit_cast(h2_t, p[i]) - off, s2, z2);
         return o;
     }
 };
-template <> struct WoCvt<true, true> {  // fp16 <- uint4: d0 holds k0..k7 in the interleaved nibble order
-    static __device__ __forceinline__ v4i run(u32 d0, u32) {
+template <int G> struct WoCvt<true, true, G> {  // fp16 <- uint4: d0 holds k0..k7 in the interleaved nibble order
+    static __device__ __forceinline__ v4i run(u32 d0, u32, u32 s2, u32 z2) {
         v4i o;
         const h2_t off = {(_Float16)1032.0f, (_Float16)1032.0f};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const u32 p = ((d0 >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
-            o[i] = __builtin_bit_cast(int, __builtin_bit_cast(h2_t, p) - off);
+            o[i] = wo_apply_h2<G>(__builtin_bit_cast(h2_t, p) - off, s2, z2);
         }
         return o;
     }
 };
-template <> struct WoCvt<false, false> {  // bf16 <- uint8 (through fp32: bf16 cannot hold 1024 + u)
-    static __device__ __forceinline__ v4i run(u32 d0, u32 d1) {
+template <int G> struct WoCvt<false, false, G> {  // bf16 <- uint8 (through fp32: bf16 cannot hold 1024 + u)
+    static __device__ __forceinline__ v4i run(u32 d0, u32 d1, u32 s, u32 z) {
         v4i o;
         const u32 d[2] = {d0, d1};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const u32 w = d[i >> 1] >> (16 * (i & 1));
-            o[i] = (int)pack2_bf16((float)(w & 0xFFu) - 128.0f, (float)((w >> 8) & 0xFFu) - 128.0f);
+            o[i] = (int)pack2_bf16(wo_apply_f32<G>((float)(w & 0xFFu) - 128.0f, s, z), wo_apply_f32<G>((float)((w >> 8) & 0xFFu) - 128.0f, s, z));
         }
         return o;
     }
 };
-template <> struct WoCvt<false, true> {  // bf16 <- uint4
-    static __device__ __forceinline__ v4i run(u32 d0, u32) {
+template <int G> struct WoCvt<false, true, G> {  // bf16 <- uint4
+    static __device__ __forceinline__ v4i run(u32 d0, u32, u32 s, u32 z) {
         v4i o;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const u32 w = d0 >> (4 * i);
-            o[i] = (int)pack2_bf16((float)(w & 0xFu) - 8.0f, (float)((w >> 16) & 0xFu) - 8.0f);
+            o[i] = (int)pack2_bf16(wo_apply_f32<G>((float)(w & 0xFu) - 8.0f, s, z), wo_apply_f32<G>((float)((w >> 16) & 0xFu) - 8.0f, s, z));
         }
         return o;
     }
@@ -83,21 +103,24 @@ template <> struct WoCvt<false, true> {  // bf16 <- uint4
 
 // WN = 2: 256x128 outputs, four wavefronts, two workgroups per CU.  WN = 4: 256x256 outputs, eight wavefronts, one
 // workgroup per CU (more operand reuse per LDS byte; the choice for large problems).
-template <typename Tag, bool W4, int WN, int NSTAGE>
+// GROUPED 0: scales [n], applied to the sums; 1: scales [k / group, n] applied to every weight; 2: scales and zeros.
+template <typename Tag, bool W4, int WN, int NSTAGE, int GROUPED = 0>
 __global__ __launch_bounds__(128 * WN, (WN == 2 ? 2 : 1)) void wo_gemm_kernel(void* __restrict__ C, const void* __restrict__ A,
                                                                               const uint8_t* __restrict__ B,
                                                                               const void* __restrict__ scales,
+                                                                              const void* __restrict__ zeros,
                                                                               const void* __restrict__ bias, int m, int n, int k,
-                                                                              int tiles_m, int tiles_n) {
+                                                                              int tiles_m, int tiles_n, int tiles_per_group) {
     constexpr bool F16 = std::is_same<Tag, F16Tag>::value;
     constexpr int NW = 2 * WN, BM = 256, BN = 64 * WN, BK = 64, TM = 128, TN = 64, MT = 4, NT = 2;
     constexpr int A_BYTES = BM * BK * 2;                 // 32 KiB
     constexpr int BCH = W4 ? 2 : 4;                      // 16-byte weight chunks per row per k-tile
     constexpr int B_BYTES = BN * BCH * 16;
-    constexpr int STAGE = A_BYTES + B_BYTES;
+    constexpr int SZ_BYTES = GROUPED ? 1024 : 0;          // scales of the tile's BN channels at +0, zeros at +512
+    constexpr int STAGE = A_BYTES + B_BYTES + SZ_BYTES;
     constexpr int A_DMA = A_BYTES / 1024 / NW;           // 1 KiB transfers per wavefront per tile
     constexpr int B_DMA = B_BYTES / 1024 / NW;
-    constexpr int PER_TILE = A_DMA + B_DMA;
+    constexpr int PER_TILE = A_DMA + B_DMA + GROUPED;     // + one 4-byte-per-lane transfer for the scales, one for the zeros
     static_assert(A_DMA * NW * 1024 == A_BYTES && B_DMA * NW * 1024 == B_BYTES && B_DMA >= 1, "stage / wavefront mismatch");
     static_assert(PER_TILE * NSTAGE < 64, "vmcnt is a 6-bit counter");
     extern __shared__ __attribute__((aligned(16))) char wo_smem[];
@@ -135,6 +158,10 @@ __global__ __launch_bounds__(128 * WN, (WN == 2 ? 2 : 1)) void wo_gemm_kernel(vo
         const int blk = slot / (BCH * 32), within = slot % (BCH * 32);
         b_voff[i] = (u32)((size_t)min(blk, blk_last) * b_blk) + within * 16;
     }
+    // group scales / zeros: lane l of a transfer fetches the pair of channels (2l, 2l+1) of its half of the tile's
+    // columns; BN / 128 wavefronts cover the tile, the others repeat them (same bytes to the same place)
+    const int sz_part = BN == 256 ? (wave & 1) : 0;
+    const u32 sz_voff = (u32)min(n0 + sz_part * 128 + 2 * lane, n - 2) * 2u;
     auto issue = [&](int kt, int stage) {
         const char* ga = a_tile + (size_t)kt * (BK * 2);
         const char* gb = b_tile + (size_t)kt * (BCH * 512);
@@ -144,6 +171,12 @@ __global__ __launch_bounds__(128 * WN, (WN == 2 ? 2 : 1)) void wo_gemm_kernel(vo
         for (int i = 0; i < A_DMA; ++i) dma16(ga, a_voff[i], sa + i * 1024);
 #pragma unroll
         for (int i = 0; i < B_DMA; ++i) dma16(gb, b_voff[i], sb + i * 1024);
+        if constexpr (GROUPED >= 1) {
+            const size_t grow = (size_t)(kt / tiles_per_group) * (size_t)n * 2;
+            const u32 ss = smem_base + stage * STAGE + A_BYTES + B_BYTES + sz_part * 256;
+            dma4(static_cast<const char*>(scales) + grow, sz_voff, ss);
+            if constexpr (GROUPED == 2) dma4(static_cast<const char*>(zeros) + grow, sz_voff, ss + 512);
+        }
     };
 
     v16f acc[MT][NT];
@@ -178,6 +211,21 @@ __global__ __launch_bounds__(128 * WN, (WN == 2 ? 2 : 1)) void wo_gemm_kernel(vo
                 wraw[1][j] = *reinterpret_cast<const v4i*>(sb + j * (BCH * 512) + (2 + lh) * 512);
             }
         }
+        // the scale (and zero) of the lane's output channel in each of its NT column tiles: a pair of fp16, or fp32 bits
+        u32 gs[NT], gz[NT];
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            gs[j] = gz[j] = 0;
+            if constexpr (GROUPED >= 1) {
+                const char* szp = sa + A_BYTES + B_BYTES + ((wn * NT + j) * 32 + lr) * 2;
+                const u32 sv = *reinterpret_cast<const unsigned short*>(szp);
+                gs[j] = F16 ? (sv | (sv << 16)) : (sv << 16);
+                if constexpr (GROUPED == 2) {
+                    const u32 zv = *reinterpret_cast<const unsigned short*>(szp + 512);
+                    gz[j] = F16 ? (zv | (zv << 16)) : (zv << 16);
+                }
+            }
+        }
         v4i xb[3];
         xb[0] = *xptr(0);
         xb[1] = *xptr(1);
@@ -186,11 +234,11 @@ __global__ __launch_bounds__(128 * WN, (WN == 2 ? 2 : 1)) void wo_gemm_kernel(vo
 #pragma unroll
             for (int j = 0; j < NT; ++j) {
                 if constexpr (W4) {
-                    wfrag[half][j][0] = WoCvt<F16, true>::run((u32)(half ? wraw[0][j][2] : wraw[0][j][0]), 0u);
-                    wfrag[half][j][1] = WoCvt<F16, true>::run((u32)(half ? wraw[0][j][3] : wraw[0][j][1]), 0u);
+                    wfrag[half][j][0] = WoCvt<F16, true, GROUPED>::run((u32)(half ? wraw[0][j][2] : wraw[0][j][0]), 0u, gs[j], gz[j]);
+                    wfrag[half][j][1] = WoCvt<F16, true, GROUPED>::run((u32)(half ? wraw[0][j][3] : wraw[0][j][1]), 0u, gs[j], gz[j]);
                 } else {
-                    wfrag[half][j][0] = WoCvt<F16, false>::run((u32)wraw[half][j][0], (u32)wraw[half][j][1]);
-                    wfrag[half][j][1] = WoCvt<F16, false>::run((u32)wraw[half][j][2], (u32)wraw[half][j][3]);
+                    wfrag[half][j][0] = WoCvt<F16, false, GROUPED>::run((u32)wraw[half][j][0], (u32)wraw[half][j][1], gs[j], gz[j]);
+                    wfrag[half][j][1] = WoCvt<F16, false, GROUPED>::run((u32)wraw[half][j][2], (u32)wraw[half][j][3], gs[j], gz[j]);
                 }
             }
         };
@@ -212,7 +260,7 @@ __global__ __launch_bounds__(128 * WN, (WN == 2 ? 2 : 1)) void wo_gemm_kernel(vo
         }
         // pin the order: the weight chunks and the first two fragments, then (NT MFMAs, one LDS read) x 14, then the
         // MFMAs of the last two steps
-        __builtin_amdgcn_sched_group_barrier(0x100, (W4 ? NT : 2 * NT) + 2, 0);  // DS reads
+        __builtin_amdgcn_sched_group_barrier(0x100, (W4 ? NT : 2 * NT) + 2 + GROUPED * NT, 0);  // DS reads
 #pragma unroll
         for (int t = 0; t < 14; ++t) {
             __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);  // MFMA
@@ -247,7 +295,7 @@ __global__ __launch_bounds__(128 * WN, (WN == 2 ? 2 : 1)) void wo_gemm_kernel(vo
             const int nn = nb + q4 * 8 + lh * 4;
             const bool ok = nn < n;
             uint2 sv = make_uint2(0, 0), bv = make_uint2(0, 0);
-            if (ok) sv = *reinterpret_cast<const uint2*>(static_cast<const unsigned short*>(scales) + nn);
+            if (ok && GROUPED == 0) sv = *reinterpret_cast<const uint2*>(static_cast<const unsigned short*>(scales) + nn);
             if (ok && bias != nullptr) bv = *reinterpret_cast<const uint2*>(static_cast<const unsigned short*>(bias) + nn);
             sc[q4 * 4] = Elem<Tag>::load(sv.x & 0xFFFFu); sc[q4 * 4 + 1] = Elem<Tag>::load(sv.x >> 16);
             sc[q4 * 4 + 2] = Elem<Tag>::load(sv.y & 0xFFFFu); sc[q4 * 4 + 3] = Elem<Tag>::load(sv.y >> 16);
@@ -265,7 +313,7 @@ __global__ __launch_bounds__(128 * WN, (WN == 2 ? 2 : 1)) void wo_gemm_kernel(vo
                 float y[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    y[e] = acc[i][j][q4 * 4 + e] * sc[q4 * 4 + e];
+                    y[e] = GROUPED == 0 ? acc[i][j][q4 * 4 + e] * sc[q4 * 4 + e] : acc[i][j][q4 * 4 + e];
                     if (bias != nullptr) y[e] = y[e] + bs[q4 * 4 + e];
                 }
                 uint2 o;
@@ -323,29 +371,21 @@ extern "C" int lq_repack_weight_only(uint8_t* dst, const int8_t* src_kn, lq_weig
     return check_launch("wo_repack");
 }
 
-extern "C" int lq_gemm_weight_only(void* C, const void* A, lq_dtype_t dtype, const uint8_t* B_prepared, lq_weight_kind_t kind,
-                                   const void* scales, const void* bias, int m, int n, int k, lq_stream_t stream) {
-    LQ_REQUIRE(C && A && B_prepared && scales, LQ_ERR_ARG, "lq_gemm_weight_only: null pointer");
-    LQ_REQUIRE(dtype == LQ_F16 || dtype == LQ_BF16, LQ_ERR_UNSUPPORTED, "lq_gemm_weight_only: activations must be F16 or BF16");
-    LQ_REQUIRE(kind == LQ_W_INT8 || kind == LQ_W_INT4, LQ_ERR_UNSUPPORTED, "lq_gemm_weight_only: kind must be INT8 or INT4");
-    LQ_REQUIRE(m >= 0 && n > 0 && k > 0 && n % 32 == 0 && k % 64 == 0, LQ_ERR_SHAPE,
-               "lq_gemm_weight_only: need n %% 32 == 0 and k %% 64 == 0 (m=%d n=%d k=%d)", m, n, k);
-    LQ_REQUIRE(reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B_prepared) % 16 == 0 &&
-                   reinterpret_cast<uintptr_t>(C) % 8 == 0 && reinterpret_cast<uintptr_t>(scales) % 8 == 0 &&
-                   reinterpret_cast<uintptr_t>(bias) % 8 == 0,
-               LQ_ERR_ARG, "lq_gemm_weight_only: A and B must be 16-byte, C, scales and bias 8-byte aligned");
-    if (m == 0) return LQ_OK;
+static int wo_launch(void* C, const void* A, lq_dtype_t dtype, const uint8_t* B_prepared, lq_weight_kind_t kind, const void* scales,
+                     const void* zeros, const void* bias, int m, int n, int k, int group_size, lq_stream_t stream) {
     const bool w4 = kind == LQ_W_INT4;
+    const int grouped = group_size == 0 ? 0 : (zeros == nullptr ? 1 : 2);
+    const int tiles_per_group = group_size == 0 ? 1 : group_size / 64;
     // 256x256 tiles (eight wavefronts, three stages) once they give every CU work; 256x128 tiles otherwise
     const long big_tiles = (long)((m + 255) / 256) * ((n + 255) / 256);
     const bool big = big_tiles >= 192;
     hipStream_t st = as_stream(stream);
-#define LQ_WO_GO(TAG, W4V, WNV, NST)                                                                                    \
+#define LQ_WO_GO(TAG, W4V, WNV, NST, GRP)                                                                               \
     do {                                                                                                                \
-        constexpr size_t lds = (size_t)(NST) * (256 * 64 * 2 + 64 * (WNV) * ((W4V) ? 2 : 4) * 16);                      \
+        constexpr size_t lds = (size_t)(NST) * (256 * 64 * 2 + 64 * (WNV) * ((W4V) ? 2 : 4) * 16 + ((GRP) ? 1024 : 0)); \
         static bool attr_done = false;                                                                                  \
         if (!attr_done) {                                                                                               \
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&wo_gemm_kernel<TAG, W4V, WNV, NST>),                 \
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&wo_gemm_kernel<TAG, W4V, WNV, NST, GRP>),            \
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {              \
                 set_error("lq_gemm_weight_only: cannot raise the dynamic LDS limit to %zu bytes", lds);                 \
                 return LQ_ERR_HIP;                                                                                      \
@@ -353,22 +393,64 @@ extern "C" int lq_gemm_weight_only(void* C, const void* A, lq_dtype_t dtype, con
             attr_done = true;                                                                                           \
         }                                                                                                               \
         const int tiles_m = (m + 255) / 256, tiles_n = (n + 64 * (WNV) - 1) / (64 * (WNV));                             \
-        hipLaunchKernelGGL((wo_gemm_kernel<TAG, W4V, WNV, NST>), dim3((unsigned)(tiles_m * tiles_n)), dim3(128 * (WNV)), \
-                           lds, st, C, A, B_prepared, scales, bias, m, n, k, tiles_m, tiles_n);                         \
+        hipLaunchKernelGGL((wo_gemm_kernel<TAG, W4V, WNV, NST, GRP>), dim3((unsigned)(tiles_m * tiles_n)),              \
+                           dim3(128 * (WNV)), lds, st, C, A, B_prepared, scales, zeros, bias, m, n, k, tiles_m, tiles_n, \
+                           tiles_per_group);                                                                            \
     } while (0)
-#define LQ_WO_KIND(TAG)                                       \
-    do {                                                      \
-        if (big) {                                            \
-            if (w4) LQ_WO_GO(TAG, true, 4, 3);                \
-            else LQ_WO_GO(TAG, false, 4, 3);                  \
-        } else {                                              \
-            if (w4) LQ_WO_GO(TAG, true, 2, 2);                \
-            else LQ_WO_GO(TAG, false, 2, 2);                  \
-        }                                                     \
+#define LQ_WO_SIZE(TAG, W4V, GRP)                  \
+    do {                                           \
+        if (big) LQ_WO_GO(TAG, W4V, 4, 3, GRP);    \
+        else LQ_WO_GO(TAG, W4V, 2, 2, GRP);        \
     } while (0)
-    if (dtype == LQ_F16) LQ_WO_KIND(F16Tag);
-    else LQ_WO_KIND(BF16Tag);
+#define LQ_WO_KIND(TAG, GRP)                       \
+    do {                                           \
+        if (w4) LQ_WO_SIZE(TAG, true, GRP);        \
+        else LQ_WO_SIZE(TAG, false, GRP);          \
+    } while (0)
+#define LQ_WO_GRP(TAG)                             \
+    do {                                           \
+        if (grouped == 0) LQ_WO_KIND(TAG, 0);      \
+        else if (grouped == 1) LQ_WO_KIND(TAG, 1); \
+        else LQ_WO_KIND(TAG, 2);                   \
+    } while (0)
+    if (dtype == LQ_F16) LQ_WO_GRP(F16Tag);
+    else LQ_WO_GRP(BF16Tag);
+#undef LQ_WO_GRP
 #undef LQ_WO_KIND
+#undef LQ_WO_SIZE
 #undef LQ_WO_GO
     return check_launch("gemm_weight_only");
+}
+
+static int wo_check(const char* what, void* C, const void* A, lq_dtype_t dtype, const uint8_t* B_prepared, lq_weight_kind_t kind,
+                    const void* scales, const void* zeros, const void* bias, int m, int n, int k) {
+    LQ_REQUIRE(C && A && B_prepared && scales, LQ_ERR_ARG, "%s: null pointer", what);
+    LQ_REQUIRE(dtype == LQ_F16 || dtype == LQ_BF16, LQ_ERR_UNSUPPORTED, "%s: activations must be F16 or BF16", what);
+    LQ_REQUIRE(kind == LQ_W_INT8 || kind == LQ_W_INT4, LQ_ERR_UNSUPPORTED, "%s: kind must be INT8 or INT4", what);
+    LQ_REQUIRE(m >= 0 && n > 0 && k > 0 && n % 32 == 0 && k % 64 == 0, LQ_ERR_SHAPE,
+               "%s: need n %% 32 == 0 and k %% 64 == 0 (m=%d n=%d k=%d)", what, m, n, k);
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B_prepared) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(C) % 8 == 0 && reinterpret_cast<uintptr_t>(scales) % 8 == 0 &&
+                   reinterpret_cast<uintptr_t>(zeros) % 8 == 0 && reinterpret_cast<uintptr_t>(bias) % 8 == 0,
+               LQ_ERR_ARG, "%s: A and B must be 16-byte, C, scales, zeros and bias 8-byte aligned", what);
+    return LQ_OK;
+}
+
+extern "C" int lq_gemm_weight_only(void* C, const void* A, lq_dtype_t dtype, const uint8_t* B_prepared, lq_weight_kind_t kind,
+                                   const void* scales, const void* bias, int m, int n, int k, lq_stream_t stream) {
+    int rc = wo_check("lq_gemm_weight_only", C, A, dtype, B_prepared, kind, scales, nullptr, bias, m, n, k);
+    if (rc != LQ_OK) return rc;
+    if (m == 0) return LQ_OK;
+    return wo_launch(C, A, dtype, B_prepared, kind, scales, nullptr, bias, m, n, k, 0, stream);
+}
+
+extern "C" int lq_gemm_weight_only_grouped(void* C, const void* A, lq_dtype_t dtype, const uint8_t* B_prepared,
+                                           lq_weight_kind_t kind, const void* scales, const void* zeros, const void* bias, int m,
+                                           int n, int k, int group_size, lq_stream_t stream) {
+    int rc = wo_check("lq_gemm_weight_only_grouped", C, A, dtype, B_prepared, kind, scales, zeros, bias, m, n, k);
+    if (rc != LQ_OK) return rc;
+    LQ_REQUIRE((group_size == 64 || group_size == 128) && k % group_size == 0, LQ_ERR_SHAPE,
+               "lq_gemm_weight_only_grouped: group_size must be 64 or 128 and divide k (group_size=%d k=%d)", group_size, k);
+    if (m == 0) return LQ_OK;
+    return wo_launch(C, A, dtype, B_prepared, kind, scales, zeros, bias, m, n, k, group_size, stream);
 }

@@ -80,6 +80,7 @@ SYMBOLS = {
     "lq_fp8_scale_cast_2d": (_I, [_P, _Z, _P, _Z, _I, _P, _I, _Z, _Z, _P]),
     "lq_gemm_w4a4": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P]),
     "lq_gemm_weight_only": (_I, [_P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _P]),
+    "lq_gemm_weight_only_grouped": (_I, [_P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _P]),
     "lq_repack_weight_only": (_I, [_P, _P, _I, _Z, _Z, _P]),
     "lq_col_absmax": (_I, [_P, _P, _I, _Z, _Z, _P]),
     "lq_smooth_vector": (_I, [_P, _P, _P, _P, _F, _Z, _P]),

@@ -529,6 +529,30 @@ def weight_only_linear(x, w_prepared, scales, bias=None, kind: str = "int8"):
     return c
 
 
+def weight_only_linear_grouped(x, w_prepared, scales, zeros=None, bias=None, kind: str = "int8", group_size: int = 128):
+    """W8A16 / W4A16 linear with group-wise scales [K / group_size, N] and optional zero points of the same shape (the
+    reference's FINEGRAINED_SCALE_ONLY / FINEGRAINED_SCALE_AND_ZEROS): every weight is dequantised in x.dtype,
+    w = q * scale (+ zero), before it is multiplied."""
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    _chk(w_prepared, "w_prepared", (torch.uint8,))
+    _chk(scales, "scales", (x.dtype,))
+    for name, t in (("zeros", zeros), ("bias", bias)):
+        if t is not None:
+            _chk(t, name, (x.dtype,))
+    m, k = x.shape
+    n = w_prepared.shape[0]
+    if group_size not in (64, 128) or k % group_size:
+        raise ValueError("group_size must be 64 or 128 and divide K")
+    if w_prepared.shape[1] != (k // 2 if kind == "int4" else k) or tuple(scales.shape) != (k // group_size, n) or \
+            (zeros is not None and zeros.shape != scales.shape) or (bias is not None and bias.numel() != n):
+        raise ValueError("shape mismatch between x, w_prepared, scales [K/group, N], zeros and bias")
+    c = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    _l.check(_l.load().lq_gemm_weight_only_grouped(_ptr(c), _ptr(x), _DT[x.dtype], _ptr(w_prepared), _KINDS[kind], _ptr(scales),
+                                                   _ptr(zeros), _ptr(bias), m, n, k, int(group_size), _stream()),
+             "lq_gemm_weight_only_grouped")
+    return c
+
+
 def load_lora(weight, lora, alpha: float):
     """invokeLoadLora: weight += lora * alpha in the tensors' dtype, in place; returns weight."""
     _chk(weight, "weight", _FLOATS)

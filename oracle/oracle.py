@@ -75,6 +75,19 @@ def round_to(x, dtype: str) -> np.ndarray:
     raise ValueError(dtype)
 
 
+def round_f64_to(x, dtype: str) -> np.ndarray:
+    """Round an fp64 array ONCE to `dtype` (as fp32 values): fp64 -> fp32 with round-to-odd, then the usual nearest-even
+    step, which cannot double-round because fp32 carries more than two extra bits over fp16 / bf16."""
+    x = np.asarray(x, dtype=np.float64)
+    with np.errstate(over="ignore", invalid="ignore"):
+        t = x.astype(F32)
+        inexact = np.isfinite(t) & (t.astype(np.float64) != x)
+        over = np.abs(t.astype(np.float64)) > np.abs(x)
+        tz = np.where(over, np.nextafter(t, F32(0)), t).astype(F32)
+    bits = tz.view(np.uint32) | inexact.astype(np.uint32)
+    return round_to(bits.view(F32), dtype)
+
+
 # ----------------------------------------------------------------------------------------
 # a1  float_to_int8_rn  (kernels/quant_kernels/int8_utils.cuh:23-28)
 # ----------------------------------------------------------------------------------------
@@ -645,6 +658,33 @@ def weight_only_gemm_f64(a, q_kn, scale, bias=None, out_dtype: str = "f16") -> n
     if bias is not None:
         y = y + np.asarray(bias, dtype=np.float64)[None, :]
     return round_to(y.astype(F32), out_dtype)
+
+
+def weight_only_dequant_grouped(q_kn, scales, zeros, group: int, dtype: str) -> np.ndarray:
+    """The dequantised weight [k, n] of the group-wise weight-only GEMM as fp32 values of T, with the roundings of the
+    reference's MmaTensorOpDequantizer (kernels/cutlass_extensions/include/cutlass_extensions/gemm/warp/
+    mma_tensorop_dequantizer.h): fp16 `plus(mul(q, scale), zero)`, two roundings (:370-390); bf16 `__hfma2(q, scale,
+    zero)`, one rounding (:200-222); `mul` alone without zero points.  scales, zeros: [k / group, n] values of T."""
+    q = np.asarray(q_kn, dtype=np.float64)
+    s = np.repeat(np.asarray(scales, dtype=np.float64), group, axis=0)
+    if zeros is None:
+        return round_to((q * s).astype(F32), dtype)          # q * s is exact in fp32: at most 8 + 11 significant bits
+    z = np.repeat(np.asarray(zeros, dtype=np.float64), group, axis=0)
+    if dtype == "f16":
+        return round_to((round_to((q * s).astype(F32), dtype).astype(np.float64) + z).astype(F32), dtype)
+    # bf16: the exact q * s + z rounded once.  The sum is formed in fp64 (exact: both terms have few significant bits
+    # unless their exponents are more than 29 apart, when the small one cannot matter) and rounded to bf16 directly.
+    return round_f64_to(q * s + z, dtype)
+
+
+def weight_only_gemm_grouped_f64(a, q_kn, scales, zeros, bias, group: int, dtype: str) -> np.ndarray:
+    """T( sum_k a[m,k] * w[k,n] [+ bias[n]] ) in fp64 over the T-rounded dequantised weights (tolerance reference: the
+    reference sums in an order its tensor-core tiling fixes)."""
+    w = weight_only_dequant_grouped(q_kn, scales, zeros, group, dtype).astype(np.float64)
+    y = np.asarray(a, dtype=np.float64) @ w
+    if bias is not None:
+        y = y + np.asarray(bias, dtype=np.float64)[None, :]
+    return round_to(y.astype(F32), dtype)
 
 
 def weight_only_prepared(q_kn, bits: int) -> np.ndarray:

@@ -165,6 +165,52 @@ int main() {
             if (std::fabs(got - ref) > 0.1 * std::fabs(ref) + 0.05) ++bad8;  // e4m3 operands (3 mantissa bits): noise ~0.01 rms here
         }
     std::printf("fp8 path (GetFP8WeightScale + ScaleCpyConvert + GemmWithResidualAndBias): %d outliers\n", bad8);
+    // ---------------- weight-only W4A16 with group-wise scales and zero points: CutlassFpAIntBGemmRunner ----------------
+    // (fpA_intB_gemm.h:58-85; every dequantised weight is T(T(q * s) + z) for fp16, so a host loop reproduces it)
+    int badwo = 0;
+    {
+        const int wk = 256, wn = 64, wm = 48, grp = 128;
+        std::vector<int8_t> codes(wk * wn / 2);
+        std::vector<int> qv(wk * wn);
+        for (int i = 0; i < wk * wn; ++i) qv[i] = (int)(15.9f * (lcg(seed) + 0.5f)) - 8;
+        for (int r = 0; r < wk; ++r)
+            for (int c = 0; c < wn; c += 2)
+                codes[r * (wn / 2) + c / 2] = (int8_t)((qv[r * wn + c] & 0xF) | ((qv[r * wn + c + 1] & 0xF) << 4));
+        std::vector<__half> hs(wk / grp * wn), hz(wk / grp * wn), ha(wm * wk), hb(wn);
+        for (auto& v : hs) v = __float2half(0.01f + 0.02f * (lcg(seed) + 0.5f));
+        for (auto& v : hz) v = __float2half(0.1f * lcg(seed));
+        for (auto& v : ha) v = __float2half(2.0f * lcg(seed));
+        for (auto& v : hb) v = __float2half(lcg(seed));
+        int8_t* dcodes; uint8_t* dprep; __half *ds, *dz, *da, *db, *dc;
+        CK(hipMalloc(&dcodes, codes.size())); CK(hipMalloc(&dprep, codes.size())); CK(hipMalloc(&ds, hs.size() * 2));
+        CK(hipMalloc(&dz, hz.size() * 2)); CK(hipMalloc(&da, ha.size() * 2)); CK(hipMalloc(&db, hb.size() * 2)); CK(hipMalloc(&dc, wm * wn * 2));
+        CK(hipMemcpy(dcodes, codes.data(), codes.size(), hipMemcpyHostToDevice));
+        CK(hipMemcpy(ds, hs.data(), hs.size() * 2, hipMemcpyHostToDevice)); CK(hipMemcpy(dz, hz.data(), hz.size() * 2, hipMemcpyHostToDevice));
+        CK(hipMemcpy(da, ha.data(), ha.size() * 2, hipMemcpyHostToDevice)); CK(hipMemcpy(db, hb.data(), hb.size() * 2, hipMemcpyHostToDevice));
+        try {
+            detail::check(lq_repack_weight_only(dprep, dcodes, LQ_W_INT4, wk, wn, st), "lq_repack_weight_only");
+            cutlass_kernels::CutlassFpAIntBGemmRunner<__half, cutlass::uint4b_t, cutlass::WeightOnlyQuantOp::FINEGRAINED_SCALE_AND_ZEROS> runner;
+            runner.gemm(da, dprep, ds, dz, db, dc, wm, wn, wk, grp, runner.getConfigs()[0], nullptr, runner.getWorkspaceSize(wm, wn, wk), st);
+        } catch (const std::exception& e) {
+            std::printf("exception: %s\n", e.what());
+            return 4;
+        }
+        CK(hipStreamSynchronize(st));
+        std::vector<__half> hc(wm * wn);
+        CK(hipMemcpy(hc.data(), dc, wm * wn * 2, hipMemcpyDeviceToHost));
+        for (int i = 0; i < wm; ++i)
+            for (int j = 0; j < wn; ++j) {
+                double ref = (double)__half2float(hb[j]), mag = 0;
+                for (int p = 0; p < wk; ++p) {
+                    const float qs = __half2float(__float2half((float)qv[p * wn + j] * __half2float(hs[(p / grp) * wn + j])));
+                    const float w = __half2float(__float2half(qs + __half2float(hz[(p / grp) * wn + j])));
+                    ref += (double)__half2float(ha[i * wk + p]) * (double)w;
+                    mag += std::fabs((double)__half2float(ha[i * wk + p]) * (double)w);
+                }
+                if (std::fabs((double)__half2float(hc[i * wn + j]) - ref) > 2e-3 * std::fabs(ref) + 1e-5 * mag + 1e-4) ++badwo;
+            }
+    }
+    std::printf("weight-only path (lq_repack_weight_only + CutlassFpAIntBGemmRunner, group scales and zeros): %d mismatches\n", badwo);
     // error convention: exception with the reference's prefix
     bool threw = false;
     try {
@@ -174,5 +220,5 @@ int main() {
         threw = std::string(e.what()).find("[lyradiff Error]") == 0;
     }
     std::printf("bad shape raises std::runtime_error with the reference's prefix: %s\n", threw ? "yes" : "no");
-    return (bad == 0 && badw == 0 && bad8 == 0 && threw) ? 0 : 1;
+    return (bad == 0 && badw == 0 && bad8 == 0 && badwo == 0 && threw) ? 0 : 1;
 }

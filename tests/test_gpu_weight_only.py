@@ -69,6 +69,81 @@ def test_weight_only_gemm(ops, dev, dt, bits, m, n, k, with_bias):
     assert_close_tol(to_np_f32(y), ref, f"weight-only {kind} {dt}", abs_floor=floor)
 
 
+def _grouped_case(k, n, bits, group, dt, with_zeros, seed):
+    """Random codes with group-wise scales of varied magnitude and (optionally) zero points, all values of T."""
+    rng = np.random.default_rng(seed)
+    half = 1 << (bits - 1)
+    q = rng.integers(-half, half, (k, n)).astype(np.int8)
+    t = TORCH_DT[dt]
+    scales = torch.from_numpy((0.002 + 0.02 * rng.random((k // group, n))).astype(np.float32)).to(t)
+    zeros = torch.from_numpy((0.05 * rng.standard_normal((k // group, n))).astype(np.float32)).to(t) if with_zeros else None
+    return q, scales, zeros
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("with_zeros", [False, True])
+@pytest.mark.parametrize("group", [64, 128])
+def test_weight_only_grouped_dequantised_weights(ops, dev, dt, bits, with_zeros, group):
+    """With the identity as activation every output is one dequantised weight (all other products are exact zeros), so the
+    kernel's per-element arithmetic is visible: bit-exact against the reference's rounding sequence for fp16 (multiply, then
+    add) and for the scale-only forms; for bf16 with zero points the kernel rounds the fp32 fused multiply-add to bf16, which
+    differs from the single rounding by one bf16 step when the fp32 result falls on a bf16 midpoint (counted, < 1e-3)."""
+    k, n = 256, 160
+    q, scales, zeros = _grouped_case(k, n, bits, group, dt, with_zeros, 100 * bits + group + with_zeros)
+    kind = "int8" if bits == 8 else "int4"
+    wp = ops.repack_weight_only(torch.from_numpy(q if bits == 8 else _pack_n(q)).to(dev), kind)
+    eye = torch.eye(k, dtype=TORCH_DT[dt]).to(dev)
+    got = to_np_f32(ops.weight_only_linear_grouped(eye, wp, scales.to(dev), None if zeros is None else zeros.to(dev), None, kind, group))
+    want = O.weight_only_dequant_grouped(q, to_np_f32(scales), None if zeros is None else to_np_f32(zeros), group, dt)
+    if dt == "bf16" and with_zeros:
+        diff = got != want
+        assert diff.mean() < 1e-3 and np.all(np.abs(got - want)[diff] <= 2.0 ** -7 * np.abs(want)[diff])
+    else:
+        assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("bits,with_zeros,group", [(8, False, 128), (8, True, 64), (4, True, 128), (4, False, 64)])
+@pytest.mark.parametrize("m,n,k,with_bias", [(256, 128, 128, True), (300, 160, 384, False), (1, 32, 128, True),
+                                             (1024, 1280, 1280, True), (777, 3072, 512, True)])
+def test_weight_only_gemm_grouped(ops, dev, dt, bits, with_zeros, group, m, n, k, with_bias):
+    g = rng_t(m + n + k + bits + group)
+    t = TORCH_DT[dt]
+    q, scales, zeros = _grouped_case(k, n, bits, group, dt, with_zeros, m + n + k)
+    x = torch.randn(m, k, generator=g).to(t)
+    bias = (0.2 * torch.randn(n, generator=g)).to(t) if with_bias else None
+    kind = "int8" if bits == 8 else "int4"
+    wp = ops.repack_weight_only(torch.from_numpy(q if bits == 8 else _pack_n(q)).to(dev), kind)
+    y = ops.weight_only_linear_grouped(x.to(dev), wp, scales.to(dev), None if zeros is None else zeros.to(dev),
+                                       None if bias is None else bias.to(dev), kind, group)
+    zs = None if zeros is None else to_np_f32(zeros)
+    ref = O.weight_only_gemm_grouped_f64(to_np_f32(x), q, to_np_f32(scales), zs, None if bias is None else to_np_f32(bias), group, dt)
+    w = np.abs(O.weight_only_dequant_grouped(q, to_np_f32(scales), zs, group, dt)).astype(np.float64)
+    ax = np.abs(to_np_f32(x)).astype(np.float64)
+    floor = 4e-6 * (ax @ w)
+    if dt == "bf16":  # the output's own rounding, and a weight that is one bf16 step off where the fp32 fma double-rounds
+        floor = floor + 2.0 ** -8 * np.abs(ref.astype(np.float64)) + (2.0 ** -7 * ax.max(axis=1)[:, None] * w.max(axis=0)[None, :] if with_zeros else 0.0)
+    assert_close_tol(to_np_f32(y), ref, f"weight-only grouped {kind} {dt} g{group} zeros={with_zeros}", abs_floor=floor)
+
+
+def test_weight_only_grouped_argument_checks(ops, dev):
+    from lyradiff_amd.lib import LyraQuantError
+
+    x = torch.zeros(8, 128, dtype=torch.float16, device=dev)
+    w = torch.zeros(32, 128, dtype=torch.uint8, device=dev)
+    with pytest.raises(ValueError, match="group_size"):
+        ops.weight_only_linear_grouped(x, w, torch.ones(4, 32, dtype=torch.float16, device=dev), group_size=32)
+    with pytest.raises(ValueError, match="shape mismatch"):
+        ops.weight_only_linear_grouped(x, w, torch.ones(2, 32, dtype=torch.float16, device=dev), group_size=128)
+    lib = __import__("lyradiff_amd.lib", fromlist=["load"]).load()
+    s = torch.ones(1, 32, dtype=torch.float16, device=dev)
+    c = torch.empty(8, 32, dtype=torch.float16, device=dev)
+    rc = lib.lq_gemm_weight_only_grouped(c.data_ptr(), x.data_ptr(), 1, w.data_ptr(), 0, s.data_ptr(), None, None, 8, 32, 128, 96, None)
+    assert rc < 0 and b"group_size must be 64 or 128" in lib.lq_last_error()
+    assert LyraQuantError is not None
+
+
 def test_weight_only_argument_checks(ops, dev):
     from lyradiff_amd.lib import LyraQuantError
 

@@ -817,3 +817,84 @@ def test_flux_block_restatement_closed_forms():
     sd["p.attn.to_qkv.bias"][2 * d:] = 0.75                    # v = 0.75 everywhere -> attention output 0.75
     ys = FB.flux_single_block(sd, "p.", xs, temb, rope, heads)
     assert torch.allclose(ys, FB._round(xs.double() + 2.0 * (0.75 + 0.25), "bf16"), atol=0.15)  # e4m3 noise on 0.75 / 0.02 only
+
+
+def _rn(fr, sig_bits, emin):
+    """Exact rational -> nearest value with `sig_bits` significant bits (ties to even), subnormals below 2**emin."""
+    from fractions import Fraction
+    import math
+
+    fr = Fraction(fr)
+    if fr == 0:
+        return Fraction(0)
+    e = math.floor(math.log2(abs(fr)))
+    while Fraction(2) ** e > abs(fr):
+        e -= 1
+    while Fraction(2) ** (e + 1) <= abs(fr):
+        e += 1
+    q = Fraction(2) ** (max(e, emin) - (sig_bits - 1))
+    nq = fr / q
+    fl = nq.numerator // nq.denominator
+    r = nq - fl
+    if r > Fraction(1, 2) or (r == Fraction(1, 2) and fl % 2 == 1):
+        fl += 1
+    return fl * q
+
+
+def test_round_f64_to_rounds_once_vs_rational_arithmetic():
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal(3000) * np.exp(rng.uniform(-15, 15, 3000))
+    b = O.round_to(x.astype(np.float32), "bf16").astype(np.float64)
+    mid = b + 2.0 ** (np.floor(np.log2(np.abs(b))) - 8)  # exact bf16 midpoints: where rounding twice goes wrong
+    xs = np.concatenate([x, mid, mid * (1 + 2.0 ** -40), mid * (1 - 2.0 ** -40)])
+    got16, gotb = O.round_f64_to(xs, "f16"), O.round_f64_to(xs, "bf16")
+    for v, g16, gb in zip(xs[::5], got16[::5], gotb[::5]):
+        assert float(_rn(float(v), 8, -126)) == float(gb)
+        if 2.0 ** -14 < abs(v) < 60000:
+            assert float(_rn(float(v), 11, -14)) == float(g16)
+    # the case that distinguishes it from rounding through fp32: 1 + 2^-8 + 2^-30 is above the bf16 midpoint
+    assert O.round_f64_to(np.array([1 + 2.0 ** -8 + 2.0 ** -30]), "bf16")[0] == np.float32(1 + 2.0 ** -7)
+    assert O.round_to(np.array([1 + 2.0 ** -8 + 2.0 ** -30], dtype=np.float32), "bf16")[0] == np.float32(1.0)
+
+
+@pytest.mark.parametrize("dt,sig,emin", [("f16", 11, -14), ("bf16", 8, -126)])
+def test_weight_only_dequant_grouped_vs_rational_arithmetic(dt, sig, emin):
+    """The reference's per-element dequantisation (mma_tensorop_dequantizer.h): fp16 multiplies, rounds, adds, rounds; bf16
+    uses one fused multiply-add; each group of `group` consecutive k has its own row of scales and zeros."""
+    from fractions import Fraction
+
+    rng = np.random.default_rng(11)
+    k, n, group = 128, 6, 64
+    q = rng.integers(-128, 128, (k, n)).astype(np.int8)
+    s = O.round_to((0.003 + 0.05 * rng.random((k // group, n))).astype(np.float32), dt)
+    z = O.round_to((0.3 * rng.standard_normal((k // group, n))).astype(np.float32), dt)
+    got = O.weight_only_dequant_grouped(q, s, z, group, dt)
+    got_s = O.weight_only_dequant_grouped(q, s, None, group, dt)
+    fused_differs = 0
+    for kk in range(k):
+        for nn in range(n):
+            qs = Fraction(int(q[kk, nn])) * Fraction(float(s[kk // group, nn]))
+            zz = Fraction(float(z[kk // group, nn]))
+            two = _rn(_rn(qs, sig, emin) + zz, sig, emin)
+            one = _rn(qs + zz, sig, emin)
+            assert float(got[kk, nn]) == float(two if dt == "f16" else one)
+            assert float(got_s[kk, nn]) == float(_rn(qs, sig, emin))
+            fused_differs += two != one
+    assert fused_differs > 0  # the two orders are distinguishable on this input
+    # the group row matters: the next group's scales give other values
+    assert not np.array_equal(got_s[:group], O.weight_only_dequant_grouped(q, s[::-1].copy(), None, group, dt)[:group])
+
+
+def test_weight_only_gemm_grouped_reduces_to_the_per_column_form():
+    rng = np.random.default_rng(12)
+    m, k, n, group = 5, 256, 8, 128
+    a = O.round_to(rng.standard_normal((m, k)).astype(np.float32), "f16")
+    q = rng.integers(-8, 8, (k, n)).astype(np.int8)
+    col = (2.0 ** rng.integers(-9, -3, n)).astype(np.float32)  # powers of two: T(q * s) is exact
+    bias = O.round_to(rng.standard_normal(n).astype(np.float32), "f16")
+    grouped = O.weight_only_gemm_grouped_f64(a, q, np.tile(col, (k // group, 1)), None, bias, group, "f16")
+    assert np.array_equal(grouped, O.weight_only_gemm_f64(a, q, col, bias, "f16"))
+    zeros = np.tile(O.round_to(rng.standard_normal(n).astype(np.float32) * 0.25, "f16"), (k // group, 1))
+    with_z = O.weight_only_gemm_grouped_f64(a, q, np.tile(col, (k // group, 1)), zeros, None, group, "f16")
+    w = O.weight_only_dequant_grouped(q, np.tile(col, (k // group, 1)), zeros, group, "f16").astype(np.float64)
+    assert np.array_equal(with_z, O.round_to((a.astype(np.float64) @ w).astype(np.float32), "f16"))
