@@ -198,3 +198,40 @@ def test_int4_block_classes_equal_the_python_ops(classes, ops, dev, level):
     xs = torch.cat([ctx, x], dim=1).contiguous()
     y = sop.forward(xs, rope, temb)
     assert torch.equal(y, spy.forward(xs, rope, temb)) and torch.isfinite(y.float()).all()
+
+
+@pytest.mark.gpu
+def test_int4_block_classes_reload_model_from_bin_and_fp16(classes, ops, dev, tmp_path):
+    """The INT4 checkpoints as raw files (packed codes int8, scales and smoothing vectors fp32, 16-bit members in the model
+    file type) give the same bits as the state-dict route; an fp16 block runs and equals the Python class."""
+    from lyradiff_amd import flux_ops as FO
+
+    b, s, sc, heads, dh = 2, 64, 32, 4, 64
+    d = heads * dh
+    sd = _int4_block_state(d, dh, rng_t(431))
+    for k, v in sd.items():
+        (v.float().numpy() if v.dtype == torch.bfloat16 else v.numpy()).tofile(str(tmp_path / (k + ".bin")))
+    x, ctx, temb, rope = _fp8_inputs(dev, b, s, sc, heads, dh, 531)
+    for level in (8, 7):
+        a = classes.FluxTransformerBlockOp("bf16", d, heads, dh, 6, level)
+        a.reload_model_from_state_dict("transformer_blocks.0.", sd, "cpu")
+        f = classes.FluxTransformerBlockOp("bf16", d, heads, dh, 6, level)
+        f.reload_model_from_bin(str(tmp_path) + "/transformer_blocks.0.", "fp32")
+        ra, rf = a.forward(x, ctx, rope, temb), f.forward(x, ctx, rope, temb)
+        assert torch.equal(ra[0], rf[0]) and torch.equal(ra[1], rf[1])
+    xs = torch.cat([ctx, x], dim=1).contiguous()
+    sa = classes.FluxSingleTransformerBlockOp("bf16", d, heads, dh, 4, 8)
+    sa.reload_model_from_state_dict("single_transformer_blocks.0.", sd, "cpu")
+    sf = classes.FluxSingleTransformerBlockOp("bf16", d, heads, dh, 4, 8)
+    sf.reload_model_from_bin(str(tmp_path) + "/single_transformer_blocks.0.", "fp32")
+    assert torch.equal(sa.forward(xs, rope, temb), sf.forward(xs, rope, temb))
+    # fp16 inference dtype, FP8 level, batch of two
+    sd16 = {k: (v.half() if v.dtype == torch.bfloat16 else v) for k, v in _block_state(d, dh, 432, ("t.", "s.")).items()}
+    op = classes.FluxSingleTransformerBlockOp("fp16", d, heads, dh, 4, 2)
+    op.reload_model_from_state_dict("s.", sd16, "cpu")
+    py = FO.FluxSingleTransformerBlockOp("fp16", d, heads, dh, 4, 2)
+    py.reload_model_from_state_dict("s.", sd16, "cpu")
+    y = op.forward(xs.half(), rope.half(), temb.half())
+    assert torch.equal(y, py.forward(xs.half(), rope.half(), temb.half())) and torch.isfinite(y.float()).all()
+    with pytest.raises(RuntimeError, match="hidden_states dtype should be"):
+        op.forward(xs, rope.half(), temb.half())
