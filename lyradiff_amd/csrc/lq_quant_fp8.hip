@@ -314,7 +314,7 @@ __device__ __forceinline__ bool grid_barrier(CoopSlot* slot, unsigned* timeout, 
 }
 
 template <typename Tag, int KEEP>
-__global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_t* __restrict__ dst,
+__global__ __launch_bounds__(kCoopThreads, (KEEP > 8 ? 4 : 1)) void fp8_amax_cast_coop_kernel(uint8_t* __restrict__ dst,
                                                                           float* __restrict__ scale_out,
                                                                           const void* __restrict__ src, size_t n,
                                                                           CoopSlot* slot, unsigned* timeout) {
@@ -417,10 +417,28 @@ __global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_
 // a negative status on an error.
 // KEEP = 8 chunks of 32 bytes (64 registers) stay in each thread's registers across the barrier: with two workgroups
 // per CU that holds a tensor of up to 33.5 M sixteen-bit elements on 256 CUs; the rest of a larger one is read twice.
+template <typename Tag, int KEEP> struct CoopCapacity {
+    int blocks_per_cu = 0, num_cu = 0;
+    static const CoopCapacity& get(int dev) {  // queried once (thread-safe initialisation of a function-local static)
+        static const CoopCapacity cap = [dev] {
+            CoopCapacity c;
+            int occ = 0;
+            hipDeviceProp_t prop;
+            if (hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+                hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, fp8_amax_cast_coop_kernel<Tag, KEEP>, kCoopThreads, 0) == hipSuccess &&
+                occ >= 1) {
+                c.blocks_per_cu = occ > 2 ? 2 : occ;
+                c.num_cu = prop.multiProcessorCount;
+            }
+            (void)hipGetLastError();
+            return c;
+        }();
+        return cap;
+    }
+};
+
 template <typename Tag>
 static int launch_amax_cast_coop(uint8_t* dst, float* scale_out, const void* src, size_t n, hipStream_t st) {
-    constexpr int KEEP = 8;
-    auto kern = fp8_amax_cast_coop_kernel<Tag, KEEP>;
     if (reinterpret_cast<uintptr_t>(src) % 16 != 0 || reinterpret_cast<uintptr_t>(dst) % 16 != 0) return 1;
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
@@ -432,29 +450,30 @@ static int launch_amax_cast_coop(uint8_t* dst, float* scale_out, const void* src
     if (ws == nullptr) return LQ_ERR_HIP;
     const int slot = slot_for_stream(dev, st);
     if (slot < 0) return 1;
-    struct Capacity { int blocks_per_cu = 0, num_cu = 0; };
-    // queried once (thread-safe initialisation of a function-local static)
-    static const Capacity cap = [&] {
-        Capacity c;
-        int occ = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-            hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, kCoopThreads, 0) == hipSuccess && occ >= 1) {
-            c.blocks_per_cu = occ > 2 ? 2 : occ;
-            c.num_cu = prop.multiProcessorCount;
-        }
-        (void)hipGetLastError();
-        return c;
-    }();
+    const CoopCapacity<Tag, 8>& cap = CoopCapacity<Tag, 8>::get(dev);
     const int blocks_per_cu = cap.blocks_per_cu, num_cu = cap.num_cu;
     if (blocks_per_cu == 0) return 1;
     // One workgroup per CU while the tensor fits in their registers (fewer parties at the barrier: 15.4 us against 17.0
     // at 4608x3072), two for a larger one (more of it stays in registers: 39.6 us against 46.3 at 4608x12288).
     size_t need = (n / Chunk16<Tag>::elems + kCoopThreads - 1) / kCoopThreads;
-    int grid = (need <= (size_t)KEEP * num_cu ? 1 : blocks_per_cu) * num_cu;
+    // A tensor that two workgroups per CU cannot hold with 8 chunks per thread (more than 33.5 M sixteen-bit elements)
+    // takes the form with 10 chunks, 80 of the 128 registers a lane may use at that occupancy (12 spill): 42 M elements stay in
+    // registers and less of the tensor is read twice.
+    if (need > (size_t)8 * 2 * num_cu) {
+        const CoopCapacity<Tag, 10>& cap12 = CoopCapacity<Tag, 10>::get(dev);
+        if (cap12.blocks_per_cu == 2) {
+            int grid = 2 * num_cu;
+            if (grid > kCoopMaxBlocks) grid = kCoopMaxBlocks;
+            hipLaunchKernelGGL((fp8_amax_cast_coop_kernel<Tag, 10>), dim3(grid), dim3(kCoopThreads), 0, st, dst, scale_out, src, n,
+                               &ws->coop[slot], &ws->timeout);
+            return check_launch("fp8_amax_cast_fused");
+        }
+    }
+    int grid = (need <= (size_t)8 * num_cu ? 1 : blocks_per_cu) * num_cu;
     if (grid > kCoopMaxBlocks) grid = kCoopMaxBlocks;
     if ((size_t)grid > need) grid = need ? (int)need : 1;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kCoopThreads), 0, st, dst, scale_out, src, n, &ws->coop[slot], &ws->timeout);
+    hipLaunchKernelGGL((fp8_amax_cast_coop_kernel<Tag, 8>), dim3(grid), dim3(kCoopThreads), 0, st, dst, scale_out, src, n,
+                       &ws->coop[slot], &ws->timeout);
     return check_launch("fp8_amax_cast_fused");
 }
 

@@ -156,7 +156,7 @@ def test_geglu_int8_gate_values_outside_the_table(ops, dev, dt):
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
-@pytest.mark.parametrize("n", [4608 * 3072, 1000003, 17, 4096])
+@pytest.mark.parametrize("n", [4608 * 3072, 1000003, 17, 4096, 35000003])  # the last: more than two workgroups per CU hold with 8 chunks
 def test_fp8_amax_cast(ops, dev, dt, n):
     x = (torch.randn(n, generator=rng_t(n % 1000)) * 3).to(TORCH_DT[dt])
     q, s = ops.fp8_quant(x.to(dev))
