@@ -281,6 +281,13 @@ def main():
                                                   "frac": round(gemm_flops / zeros_us / 1e6 / FP8_PEAK_TFLOPS, 4)},
                 "shader_clock_ghz": clocks,
                 "vendor_fp8_gemm_same_operands_us": vendor}
+    # what the matrix pipes can deliver at the clock the device sustains under this kernel: CUs x 8192 FP8 FLOP per clock
+    # (the published 5.0 PFLOP/s is 256 CUs at 2.4 GHz); `frac` above stays relative to the published peak
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    ghz = (clocks or {}).get("up_gemm_random_operands") if isinstance(clocks, dict) else None
+    if ghz:
+        at_clock = cus * 8192 * ghz / 1e3
+        roofline["peak_at_sustained_clock"] = {"compute_units": cus, "TFLOP/s": round(at_clock, 1), "frac": round(achieved / at_clock, 4)}
 
     out = {
         "metric": "W8A8/FP8 GEMM TOPS at FLUX shapes (% MFMA peak); act-quant HBM GB/s",

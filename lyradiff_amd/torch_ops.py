@@ -232,3 +232,63 @@ def flux_single_mlp_fp8(x: Tensor, norm_hidden: Tensor, attn_output: Tensor, gat
 @flux_single_mlp_fp8.register_fake
 def _(x, norm_hidden, attn_output, gate, wm, wm_scale, inm_scale, bm, wo, wo_scale, ino_scale, bo):
     return torch.empty_like(x)
+
+
+# ---- torch.ops.lyrallms.*: the weight-only utility operators of the reference -----------------------------------------
+# (torch::RegisterOperators("lyrallms::...") in src/lyradiff/layers/gemm_utils/WeightOnlyQuantOps.cc:326-351: CPU tensors in,
+# CPU tensors out, used by conversion scripts).  quant_type is torch.int8 or torch.quint4x2 as there (:30-60).  The
+# "processed" weight is this library's prepared layout (lq_repack_weight_only, a device kernel: the tensor makes a round
+# trip to the GPU), the counterpart of the reference's NVIDIA-specific interleave.
+_LLM = ("symmetric_quantize_last_axis_of_batched_matrix", "_symmetric_quantize_last_axis_of_batched_matrix",
+        "preprocess_weights_for_mixed_gemm", "pack_int8_tensor_to_packed_int4", "unpack_int4_packed_tensor_to_int8")
+
+
+def _bits(quant_type: torch.dtype) -> int:
+    if quant_type == torch.int8:
+        return 8
+    if quant_type == torch.quint4x2:
+        return 4
+    raise RuntimeError("Must be int4 or int8 quantization")  # check_quant_type_allowed, WeightOnlyQuantOps.cc:30-37
+
+
+def _prepare(q_unprocessed: Tensor, bits: int) -> Tensor:
+    if q_unprocessed.dim() == 3:
+        return torch.stack([_prepare(w, bits) for w in q_unprocessed])
+    return _ops.repack_weight_only(q_unprocessed.cuda(), "int8" if bits == 8 else "int4").cpu().view(torch.int8)
+
+
+@_lib_op("lyrallms::pack_int8_tensor_to_packed_int4", mutates_args=(), device_types="cpu")
+def llm_pack_int4(weight: Tensor) -> Tensor:
+    from .weights import pack_int8_tensor_to_packed_int4
+
+    return pack_int8_tensor_to_packed_int4(weight)
+
+
+@_lib_op("lyrallms::unpack_int4_packed_tensor_to_int8", mutates_args=(), device_types="cpu")
+def llm_unpack_int4(weight: Tensor) -> Tensor:
+    from .weights import unpack_int4_packed_tensor_to_int8
+
+    return unpack_int4_packed_tensor_to_int8(weight)
+
+
+@_lib_op("lyrallms::preprocess_weights_for_mixed_gemm", mutates_args=(), device_types="cpu")
+def llm_preprocess(row_major_quantized_weight: Tensor, quant_type: torch.dtype) -> Tensor:
+    if row_major_quantized_weight.dtype != torch.int8:
+        raise RuntimeError("Quantized tensor must be int8 dtype")
+    return _prepare(row_major_quantized_weight.contiguous(), _bits(quant_type))
+
+
+@_lib_op("lyrallms::_symmetric_quantize_last_axis_of_batched_matrix", mutates_args=(), device_types="cpu")
+def llm_squant_all(weight: Tensor, quant_type: torch.dtype) -> list[Tensor]:
+    from .weights import symmetric_quantize_last_axis_of_batched_matrix as squant
+
+    if weight.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("Invalid datatype. Weight must be BF16/FP16")
+    bits = _bits(quant_type)
+    q, scales = squant(weight.contiguous(), bits)
+    return [q, _prepare(q, bits), scales]
+
+
+@_lib_op("lyrallms::symmetric_quantize_last_axis_of_batched_matrix", mutates_args=(), device_types="cpu")
+def llm_squant(weight: Tensor, quant_type: torch.dtype) -> list[Tensor]:
+    return list(llm_squant_all(weight, quant_type)[1:])

@@ -118,3 +118,46 @@ def test_block_operators_match_the_python_functions(tops, dev):
     gate = msa[2].contiguous()
     got = torch.ops.lyradiff.flux_single_mlp_fp8(x, norm, attn, gate, *flat(ws.proj_mlp), *flat(ws.proj_out))
     assert torch.equal(got, F.flux_single_mlp_fp8(x, norm, attn, gate, ws))
+
+
+def test_lyrallms_utility_operators_on_the_cpu(tops):
+    """torch.ops.lyrallms.* as the reference registers them (WeightOnlyQuantOps.cc:326-351): CPU tensors in and out."""
+    for name in tops._LLM:
+        assert hasattr(torch.ops.lyrallms, name), name
+    q = torch.randint(-8, 8, (2, 5, 8), generator=torch.Generator().manual_seed(3), dtype=torch.int8)
+    packed = torch.ops.lyrallms.pack_int8_tensor_to_packed_int4(q)
+    assert packed.shape == (2, 5, 4) and packed.dtype == torch.int8
+    assert torch.equal(torch.ops.lyrallms.unpack_int4_packed_tensor_to_int8(packed), q)
+    assert packed[0, 0, 0].item() == ((int(q[0, 0, 0]) & 0xF) | ((int(q[0, 0, 1]) & 0xF) << 4)) - (256 if (int(q[0, 0, 1]) & 0x8) else 0)
+    with pytest.raises(RuntimeError, match="int4 or int8"):
+        torch.ops.lyrallms.preprocess_weights_for_mixed_gemm(torch.zeros(64, 32, dtype=torch.int8), torch.float16)
+    with pytest.raises(RuntimeError, match="BF16/FP16"):
+        torch.ops.lyrallms.symmetric_quantize_last_axis_of_batched_matrix(torch.zeros(64, 32), torch.int8)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("quant_type,kind", [(torch.int8, "int8"), (torch.quint4x2, "int4")])
+def test_lyrallms_quantise_preprocess_and_gemm(tops, dev, quant_type, kind):
+    """symmetric_quantize_last_axis_of_batched_matrix -> (processed weight, scales) feeds the weight-only GEMM directly;
+    the underscore form also returns the unprocessed codes, and preprocessing those gives the same processed weight."""
+    from lyradiff_amd import ops
+    from oracle import oracle as O
+
+    g = torch.Generator().manual_seed(11)
+    k, n, m = 256, 96, 40
+    w = (0.05 * torch.randn(k, n, generator=g)).half()
+    x = torch.randn(m, k, generator=g).half()
+    processed, scales = torch.ops.lyrallms.symmetric_quantize_last_axis_of_batched_matrix(w, quant_type)
+    unprocessed, processed2, scales2 = torch.ops.lyrallms._symmetric_quantize_last_axis_of_batched_matrix(w, quant_type)
+    assert not processed.is_cuda and torch.equal(processed, processed2) and torch.equal(scales, scales2)
+    assert torch.equal(torch.ops.lyrallms.preprocess_weights_for_mixed_gemm(unprocessed, quant_type), processed)
+    bits = 8 if kind == "int8" else 4
+    q_ref, s_ref = O.weight_only_quantize(w.float().numpy(), bits, "f16")
+    assert np.array_equal(scales.float().numpy(), s_ref)
+    y = ops.weight_only_linear(x.to(dev), processed.view(torch.uint8).to(dev), scales.to(dev), None, kind)
+    ref = O.weight_only_gemm_f64(x.float().numpy(), q_ref, s_ref, None, "f16")
+    assert np.allclose(y.float().cpu().numpy(), ref, rtol=1e-2, atol=2e-3)
+    # a batch of matrices ("experts") is processed one by one
+    w3 = torch.stack([w, -w])
+    p3, s3 = torch.ops.lyrallms.symmetric_quantize_last_axis_of_batched_matrix(w3, quant_type)
+    assert p3.shape[0] == 2 and torch.equal(p3[0], processed) and torch.equal(s3[0], scales)
