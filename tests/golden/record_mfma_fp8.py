@@ -2,7 +2,7 @@
 FP8 GEMM with unit scales and fp32 output (one v_mfma_f32_32x32x64_f8f6f4 per output, accumulator starting at zero),
 plus two-step (K = 128) cases for the accumulation between steps.  Run on the GPU box:
 
-    python tests/golden/record_mfma_fp8.py gpurun_out/mfma_fp8_recorded.npz
+    python tests/golden/record_mfma_fp8.py /tmp/mfma_fp8_recorded.npz
 
 The result is committed as tests/golden/mfma_fp8_recorded.npz; tests/test_oracle_pins.py checks oracle.fp8_mfma_dot_model
 against it on the CPU.  Inputs are seeded, so a re-run reproduces the file."""
@@ -84,7 +84,7 @@ def cases():
 
 
 if __name__ == "__main__":
-    dst = sys.argv[1] if len(sys.argv) > 1 else "gpurun_out/mfma_fp8_recorded.npz"
+    dst = sys.argv[1] if len(sys.argv) > 1 else "mfma_fp8_recorded.npz"
     rec = {}
     for name, (a, b) in cases().items():
         rec[name + "__a"], rec[name + "__b"], rec[name + "__y"] = O.e4m3_encode(a), O.e4m3_encode(b), hw(a, b)
