@@ -198,6 +198,10 @@ template <int NP, int G, int... I> __device__ __forceinline__ void sched_interle
     (sched_slot<NP, G, I>(), ...);
 }
 
+#ifndef LQ_GEMM_SPREAD_TRANSFERS
+#define LQ_GEMM_SPREAD_TRANSFERS 1
+#endif
+
 template <int KIND, typename OutTag, int BM, int BN, int BKB, int WM, int WN, int NSTAGE>
 struct GemmKernel {
     static constexpr int NW = WM * WN;
@@ -313,6 +317,20 @@ struct GemmKernel {
 #pragma unroll
             for (int i = 0; i < B_DMA; ++i) dma16(gb, b_voff[i], sb + i * 1024);
             issue_scales(kt, stage);
+        };
+        // Transfers lo..hi-1 of a tile (A first, then B), for main loops that spread a tile's transfers
+        // between their MFMAs; lo and hi are compile-time values after unrolling.
+        auto issue_range = [&](int kt, int stage, int lo, int hi) {
+            const uint8_t* ga = a_base + (size_t)kt * BKB;
+            const uint8_t* gb = b_base + (size_t)kt * (BKB * 32);
+            const u32 sa = smem_base + stage * STAGE_BYTES + wave * (A_DMA * 1024);
+            const u32 sb = smem_base + stage * STAGE_BYTES + A_BYTES + wave * (B_DMA * 1024);
+#pragma unroll
+            for (int d = 0; d < A_DMA + B_DMA; ++d)
+                if (d >= lo && d < hi) {
+                    if (d < A_DMA) dma16(ga, a_voff[d < A_DMA ? d : 0], sa + d * 1024);
+                    else dma16(gb, b_voff[d >= A_DMA ? d - A_DMA : 0], sb + (d - A_DMA) * 1024);
+                }
         };
         // ---- accumulators ----------------------------------------------------------------------
         AccT acc[MT][NT];
@@ -464,9 +482,21 @@ struct GemmKernel {
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wp[buf][j][0], xp[buf][i][0], acc[i][j], 0, 0, 0);
                 }
             };
+            // With three or more stages a tile's transfers are not issued in one burst behind the barrier
+            // but spread between the MFMAs: a wavefront stalled on a full memory-instruction queue cannot
+            // feed the matrix pipe, and with one wavefront per SIMD nobody else can either.  Tile T's first
+            // N_AFTER transfers go out behind the barrier that retires tile T-NSTAGE, between the MFMAs
+            // that follow it; the rest between the MFMAs of tile T-NSTAGE+1 ahead of ITS barrier.  At the
+            // barrier of tile kt everything up to tile kt+NSTAGE-1 has been issued, so the wait for tile
+            // kt+1 leaves the same PER_TILE*(NSTAGE-2) transfers in flight as the burst scheme.
+            constexpr bool SPREAD = LQ_GEMM_SPREAD_TRANSFERS && NSTAGE >= 3;
+            constexpr int HPRE = NMFMA / 2, RPOST = NMFMA - HPRE;  // MFMAs of the last k-step ahead of / behind the barrier
+            constexpr int NPOS = KS * NMFMA, PRE = NPOS - RPOST;
+            constexpr int N_AFTER = SPREAD ? PER_TILE * RPOST / NPOS : PER_TILE, N_BEFORE = PER_TILE - N_AFTER;
             auto tile_iter = [&](int kt, auto parity) {
                 constexpr int P = decltype(parity)::value;
                 const char* sa = smem + (kt % NSTAGE) * STAGE_BYTES;
+                const int t_prev = min(kt + NSTAGE - 1, ktiles - 1), s_prev = (kt + NSTAGE - 1) % NSTAGE;
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     const int cur = (P + ks) & 1, nxt = cur ^ 1;
@@ -474,39 +504,60 @@ struct GemmKernel {
                         // MFMAs of this step interleaved with the fragment reads of the next step
 #pragma unroll
                         for (int idx = 0; idx < NMFMA; ++idx) {
+                            if constexpr (SPREAD) {
+                                const int q = ks * NMFMA + idx;
+                                issue_range(t_prev, s_prev, N_AFTER + q * N_BEFORE / PRE, N_AFTER + (q + 1) * N_BEFORE / PRE);
+                            }
 #pragma unroll
                             for (int pc = idx * NPIECE / NMFMA; pc < (idx + 1) * NPIECE / NMFMA; ++pc)
                                 load_piece(sa, ks + 1, nxt, pc);
                             do_mfma(cur, idx);
+                            if constexpr (SPREAD) __builtin_amdgcn_sched_barrier(0);
                         }
-                        sched_interleave<NPIECE, NMFMA>(std::make_integer_sequence<int, NMFMA>{});
+                        if constexpr (!SPREAD) sched_interleave<NPIECE, NMFMA>(std::make_integer_sequence<int, NMFMA>{});
                     } else {
                         // last step of the tile: half of the MFMAs go ahead of the barrier so that the matrix
-                        // pipe has queued work while the wavefront waits; the other half is interleaved with
-                        // the first fragment reads of the next tile.
-                        constexpr int H = NMFMA / 2, R = NMFMA - H;
+                        // pipe has work while the wavefront waits; the other half is interleaved with the first
+                        // fragment reads of the next tile.
 #pragma unroll
-                        for (int idx = 0; idx < H; ++idx) do_mfma(cur, idx);
+                        for (int idx = 0; idx < HPRE; ++idx) {
+                            if constexpr (SPREAD) {
+                                const int q = ks * NMFMA + idx;
+                                issue_range(t_prev, s_prev, N_AFTER + q * N_BEFORE / PRE, N_AFTER + (q + 1) * N_BEFORE / PRE);
+                            }
+                            do_mfma(cur, idx);
+                            if constexpr (SPREAD) __builtin_amdgcn_sched_barrier(0);
+                        }
                         __builtin_amdgcn_sched_barrier(0);
                         wait_vmcnt<PER_TILE*(NSTAGE - 2)>();
                         __syncthreads();
-                        issue_tile(min(kt + NSTAGE, ktiles - 1), kt % NSTAGE);
+                        const int t_next = min(kt + NSTAGE, ktiles - 1);
+                        if constexpr (!SPREAD) issue_tile(t_next, kt % NSTAGE);
                         __builtin_amdgcn_sched_barrier(0);
                         const char* sn = smem + ((kt + 1) % NSTAGE) * STAGE_BYTES;
 #pragma unroll
-                        for (int idx = 0; idx < R; ++idx) {
+                        for (int idx = 0; idx < RPOST; ++idx) {
+                            if constexpr (SPREAD) issue_range(t_next, kt % NSTAGE, idx * N_AFTER / RPOST, (idx + 1) * N_AFTER / RPOST);
 #pragma unroll
-                            for (int pc = idx * NPIECE / R; pc < (idx + 1) * NPIECE / R; ++pc) load_piece(sn, 0, nxt, pc);
-                            do_mfma(cur, H + idx);
+                            for (int pc = idx * NPIECE / RPOST; pc < (idx + 1) * NPIECE / RPOST; ++pc) load_piece(sn, 0, nxt, pc);
+                            do_mfma(cur, HPRE + idx);
+                            if constexpr (SPREAD) __builtin_amdgcn_sched_barrier(0);
                         }
-                        sched_interleave<NPIECE, R>(std::make_integer_sequence<int, R>{});
+                        if constexpr (!SPREAD) sched_interleave<NPIECE, RPOST>(std::make_integer_sequence<int, RPOST>{});
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
             };
+            if constexpr (SPREAD) {
 #pragma unroll
-            for (int s = 0; s < NSTAGE; ++s) issue_tile(min(s, ktiles - 1), s);
-            wait_vmcnt<PER_TILE*(NSTAGE - 1)>();
+                for (int s = 0; s < NSTAGE - 1; ++s) issue_tile(min(s, ktiles - 1), s);
+                issue_range(min(NSTAGE - 1, ktiles - 1), NSTAGE - 1, 0, N_AFTER);
+                wait_vmcnt<PER_TILE*(NSTAGE - 2) + N_AFTER>();
+            } else {
+#pragma unroll
+                for (int s = 0; s < NSTAGE; ++s) issue_tile(min(s, ktiles - 1), s);
+                wait_vmcnt<PER_TILE*(NSTAGE - 1)>();
+            }
             __syncthreads();
 #pragma unroll
             for (int pc = 0; pc < NPIECE; ++pc) load_piece(smem, 0, 0, pc);
@@ -812,6 +863,7 @@ struct GemmKernel {
 // The W4A4 kernel is bound by the vector ALU (three fp32 operations per output per group), so its
 // small-tile configurations ask for more resident wavefronts instead.
 template <int KIND, int BM, int BN, int BKB, int WM, int WN> constexpr int min_workgroups_per_cu() {
+    if ((BM / WM) * (BN / WN) >= 128 * 128) return 1;  // 256 accumulator registers: one wavefront per SIMD, the whole register file
     if (KIND != K_W4A4 && KIND != K_W4A4H) return 2;
     if (WM * WN > 4) return 1;
     const int wave_tile = (BM / WM) * (BN / WN);

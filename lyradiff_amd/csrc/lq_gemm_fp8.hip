@@ -14,7 +14,7 @@ template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
         const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
         // one round of 256x256 tiles when they fit the 256 CUs at once; otherwise 128x256 tiles, two workgroups
         // per CU (finer tail, one workgroup's epilogue overlaps the other's MFMA work)
-        t = t256 >= 192 ? (t256 <= 256 ? 0 : 4) : (t128 >= 192 ? 2 : 3);
+        t = t256 >= 192 ? (t256 <= 256 ? 6 : 4) : (t128 >= 192 ? 2 : 3);
         if (p.k <= 1024 && t128 >= 192) t = 2;  // short K: prologue and epilogue dominate, smaller tiles overlap them better
     }
     if (t == 1 && p.kb % 128 != 0) t = 0;  // the 128-byte k-tile needs k % 128 == 0
@@ -25,6 +25,7 @@ template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
         case 3: return launch_gemm<K_FP8, OutTag, 64, 64, 64, 2, 2, 3>(p, st);
         case 4: return launch_gemm<K_FP8, OutTag, 128, 256, 64, 2, 2, 3>(p, st);
         case 5: return launch_gemm<K_FP8, OutTag, 256, 128, 64, 2, 2, 3>(p, st);
+        case 6: return launch_gemm<K_FP8, OutTag, 256, 256, 64, 2, 2, 4>(p, st);  // one wavefront per SIMD, 128x128 wavefront tiles
         default: set_error("lq_gemm_fp8: unknown tactic %d", t); return LQ_ERR_ARG;
     }
 }

@@ -76,7 +76,7 @@ def test_shape_tactic_cache(lib):
     from lyradiff_amd import lib as L
 
     k8, k4 = L.LQ_W_INT8, L.LQ_W_INT4
-    assert lib.lq_gemm_tactic_count(k8) == 6 and lib.lq_gemm_tactic_count(L.LQ_W_FP8) == 6 and lib.lq_gemm_tactic_count(k4) == 3
+    assert lib.lq_gemm_tactic_count(k8) == 7 and lib.lq_gemm_tactic_count(L.LQ_W_FP8) == 7 and lib.lq_gemm_tactic_count(k4) == 3
     assert lib.lq_gemm_tactic_count(7) < 0
     assert lib.lq_gemm_get_shape_tactic(k8, 4096, 640, 2560) == -1
     assert lib.lq_gemm_set_shape_tactic(k8, 4096, 640, 2560, 2) == 0
