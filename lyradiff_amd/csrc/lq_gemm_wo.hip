@@ -162,22 +162,27 @@ __global__ __launch_bounds__(128 * WN, (WN == 2 ? 2 : 1)) void wo_gemm_kernel(vo
     // columns; BN / 128 wavefronts cover the tile, the others repeat them (same bytes to the same place)
     const int sz_part = BN == 256 ? (wave & 1) : 0;
     const u32 sz_voff = (u32)min(n0 + sz_part * 128 + 2 * lane, n - 2) * 2u;
-    auto issue = [&](int kt, int stage) {
+    // transfers lo..hi-1 of tile kt (activations, weights, then the group scales and zeros); lo and hi are compile-time
+    // values after unrolling
+    auto issue_range = [&](int kt, int stage, int lo, int hi) {
         const char* ga = a_tile + (size_t)kt * (BK * 2);
         const char* gb = b_tile + (size_t)kt * (BCH * 512);
         const u32 sa = smem_base + stage * STAGE + wave * (A_DMA * 1024);
         const u32 sb = smem_base + stage * STAGE + A_BYTES + wave * (B_DMA * 1024);
 #pragma unroll
-        for (int i = 0; i < A_DMA; ++i) dma16(ga, a_voff[i], sa + i * 1024);
-#pragma unroll
-        for (int i = 0; i < B_DMA; ++i) dma16(gb, b_voff[i], sb + i * 1024);
-        if constexpr (GROUPED >= 1) {
-            const size_t grow = (size_t)(kt / tiles_per_group) * (size_t)n * 2;
-            const u32 ss = smem_base + stage * STAGE + A_BYTES + B_BYTES + sz_part * 256;
-            dma4(static_cast<const char*>(scales) + grow, sz_voff, ss);
-            if constexpr (GROUPED == 2) dma4(static_cast<const char*>(zeros) + grow, sz_voff, ss + 512);
+        for (int d = 0; d < PER_TILE; ++d) {
+            if (d < lo || d >= hi) continue;
+            if (d < A_DMA) dma16(ga, a_voff[d < A_DMA ? d : 0], sa + d * 1024);
+            else if (d < A_DMA + B_DMA) dma16(gb, b_voff[d >= A_DMA && d < A_DMA + B_DMA ? d - A_DMA : 0], sb + (d - A_DMA) * 1024);
+            else {
+                const size_t grow = (size_t)(kt / tiles_per_group) * (size_t)n * 2;
+                const u32 ss = smem_base + stage * STAGE + A_BYTES + B_BYTES + sz_part * 256;
+                if (d == A_DMA + B_DMA) dma4(static_cast<const char*>(scales) + grow, sz_voff, ss);
+                else dma4(static_cast<const char*>(zeros) + grow, sz_voff, ss + 512);
+            }
         }
     };
+    auto issue = [&](int kt, int stage) { issue_range(kt, stage, 0, PER_TILE); };
 
     v16f acc[MT][NT];
 #pragma unroll
@@ -194,7 +199,9 @@ __global__ __launch_bounds__(128 * WN, (WN == 2 ? 2 : 1)) void wo_gemm_kernel(vo
     // steps ahead of their use and the order "read, NT MFMAs" is pinned with scheduling barriers, so that the matrix
     // pipe does not wait for an LDS round trip at every step; the weights of the second half are converted while
     // the MFMAs of the first half run.
-    auto compute = [&](int stage) {
+    // (with three stages the transfers of tile kt_next go out one or two at a time between the steps: a wavefront that
+    // stalls on a full memory-instruction queue cannot issue its next MFMA)
+    auto compute = [&](int stage, int kt_next, int stage_next) {
         const char* sa = wo_smem + stage * STAGE;
         const char* sb = sa + A_BYTES + (wn * NT) * (BCH * 512) + lr * 16;
         auto xptr = [&](int t) -> const v4i* {
@@ -246,6 +253,7 @@ __global__ __launch_bounds__(128 * WN, (WN == 2 ? 2 : 1)) void wo_gemm_kernel(vo
 #pragma unroll
         for (int t = 0; t < 16; ++t) {
             const int half = t >> 3, s2 = (t >> 2) & 1, i = t & 3;
+            if constexpr (NSTAGE >= 3) issue_range(kt_next, stage_next, t * PER_TILE / 16, (t + 1) * PER_TILE / 16);
             if (t + 2 < 16) xb[(t + 2) % 3] = *xptr(t + 2);
             if (t == 2) convert(1);
             const v4i x = xb[t % 3];
@@ -278,8 +286,9 @@ __global__ __launch_bounds__(128 * WN, (WN == 2 ? 2 : 1)) void wo_gemm_kernel(vo
     for (int kt = 0; kt < ktiles; ++kt) {
         wait_vmcnt<PER_TILE*(NSTAGE - 2)>();
         __syncthreads();
-        issue(min(kt + NSTAGE - 1, ktiles - 1), (kt + NSTAGE - 1) % NSTAGE);
-        compute(kt % NSTAGE);
+        // two stages: the next tile must be on its way for the whole of this one, so its transfers go out at once
+        if constexpr (NSTAGE < 3) issue(min(kt + NSTAGE - 1, ktiles - 1), (kt + NSTAGE - 1) % NSTAGE);
+        compute(kt % NSTAGE, min(kt + NSTAGE - 1, ktiles - 1), (kt + NSTAGE - 1) % NSTAGE);
     }
     wait_vmcnt<0>();  // nothing in flight towards LDS when the workgroup ends
 
