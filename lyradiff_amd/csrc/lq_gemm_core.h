@@ -198,10 +198,6 @@ template <int NP, int G, int... I> __device__ __forceinline__ void sched_interle
     (sched_slot<NP, G, I>(), ...);
 }
 
-#ifndef LQ_GEMM_SPREAD_TRANSFERS
-#define LQ_GEMM_SPREAD_TRANSFERS 1
-#endif
-
 template <int KIND, typename OutTag, int BM, int BN, int BKB, int WM, int WN, int NSTAGE>
 struct GemmKernel {
     static constexpr int NW = WM * WN;
@@ -489,7 +485,7 @@ struct GemmKernel {
             // that follow it; the rest between the MFMAs of tile T-NSTAGE+1 ahead of ITS barrier.  At the
             // barrier of tile kt everything up to tile kt+NSTAGE-1 has been issued, so the wait for tile
             // kt+1 leaves the same PER_TILE*(NSTAGE-2) transfers in flight as the burst scheme.
-            constexpr bool SPREAD = LQ_GEMM_SPREAD_TRANSFERS && NSTAGE >= 3;
+            constexpr bool SPREAD = NSTAGE >= 3;
             constexpr int HPRE = NMFMA / 2, RPOST = NMFMA - HPRE;  // MFMAs of the last k-step ahead of / behind the barrier
             constexpr int NPOS = KS * NMFMA, PRE = NPOS - RPOST;
             constexpr int N_AFTER = SPREAD ? PER_TILE * RPOST / NPOS : PER_TILE, N_BEFORE = PER_TILE - N_AFTER;

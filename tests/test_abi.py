@@ -86,7 +86,7 @@ def test_shape_tactic_cache(lib):
     assert lib.lq_gemm_get_shape_tactic(k4, 4096, 640, 2560) == -1     # another GEMM
     assert lib.lq_gemm_set_shape_tactic(k8, 3000, 640, 2560, 4) == 0   # an exact entry wins over the bucket
     assert lib.lq_gemm_get_shape_tactic(k8, 3000, 640, 2560) == 4
-    assert lib.lq_gemm_set_shape_tactic(k8, 4096, 640, 2560, 6) == -1  # tactic out of range
+    assert lib.lq_gemm_set_shape_tactic(k8, 4096, 640, 2560, lib.lq_gemm_tactic_count(k8)) == -1  # tactic out of range
     assert b"tactic" in lib.lq_last_error()
     assert lib.lq_gemm_set_shape_tactic(k8, 3000, 640, 2560, -1) == 0 and lib.lq_gemm_set_shape_tactic(k8, 4096, 640, 2560, -1) == 0
     assert lib.lq_gemm_get_shape_tactic(k8, 3000, 640, 2560) == -1
