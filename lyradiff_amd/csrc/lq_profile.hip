@@ -3,6 +3,7 @@
 // GemmPluginProfiler::profileTactics / profileTacticForProblem of lyraDiff
 // (layers/gemm_utils/GemmProfiler.cc:78-127,161-265): same idea (warm-up runs, timed runs between two
 // events, keep the minimum; here in interleaved rounds), but the caller owns the temporary memory and nothing is allocated here.
+#include <algorithm>
 #include "lq_common.h"
 
 namespace lq {
@@ -132,10 +133,28 @@ extern "C" int lq_gemm_profile(lq_weight_kind_t kind, int m, int n, int k, void*
     hipEvent_t ev0, ev1;
     LQ_REQUIRE(hipEventCreate(&ev0) == hipSuccess && hipEventCreate(&ev1) == hipSuccess, LQ_ERR_HIP,
                "lq_gemm_profile: cannot create events");
-    // Candidates are timed in interleaved rounds and each keeps its fastest round: on a power-limited part the clock
+    // Candidates are timed in interleaved rounds: on a power-limited part the clock
     // drifts over consecutive launches by more than the candidates differ, and a block of back-to-back runs per
     // candidate would rank them by when they ran.
-    constexpr int kRounds = 5, kRuns = 3, kMaxTactics = 16;
+    // Before that the built-in choice runs until two groups of ten launches agree to 1.5 % (at most 30 ms): from idle the
+    // power management needs tens of milliseconds of load to settle, and until then every candidate looks faster than it
+    // will be in a running pipeline, the power-hungry ones most of all.  A candidate's figure is the median of its rounds.
+    constexpr int kRounds = 5, kRuns = 4, kMaxTactics = 16;
+    {
+        float prev = 0.0f, spent = 0.0f;
+        for (int group = 0; group < 200 && spent < 30.0f; ++group) {
+            bool ok = hipEventRecord(ev0, st) == hipSuccess;
+            for (int i = 0; i < 10 && ok; ++i) ok = run_once() == LQ_OK;
+            float ms = 0.0f;
+            ok = ok && hipEventRecord(ev1, st) == hipSuccess && hipEventSynchronize(ev1) == hipSuccess &&
+                 hipEventElapsedTime(&ms, ev0, ev1) == hipSuccess;
+            if (!ok) { (void)hipGetLastError(); break; }
+            spent += ms;
+            if (prev > 0.0f && ms < prev * 1.015f && ms > prev * 0.985f) break;
+            prev = ms;
+        }
+    }
+    float rounds_of[kMaxTactics][kRounds];
     float best_of[kMaxTactics];
     bool usable[kMaxTactics];
     for (int t = 0; t < kMaxTactics; ++t) { best_of[t] = 0.0f; usable[t] = t < count; }
@@ -153,8 +172,13 @@ extern "C" int lq_gemm_profile(lq_weight_kind_t kind, int m, int n, int k, void*
                 usable[t] = false;
                 continue;
             }
-            if (round > 0 && (best_of[t] == 0.0f || ms < best_of[t])) best_of[t] = ms;
+            if (round > 0) rounds_of[t][round - 1] = ms;
         }
+    }
+    for (int t = 0; t < count && t < kMaxTactics; ++t) {
+        if (!usable[t]) continue;
+        std::sort(rounds_of[t], rounds_of[t] + kRounds);
+        best_of[t] = rounds_of[t][kRounds / 2];
     }
     int best = -1;
     float best_ms = 0.0f;
