@@ -266,6 +266,18 @@ def main():
         del wd8
     except Exception:  # not every PyTorch build exposes it
         pass
+    # what the matrix pipes alone sustain on this part: 16 x 300 FP8 MFMAs per wavefront on register operands, no memory or
+    # LDS traffic, one wavefront per SIMD (the layout of the down projection's kernel), on the chain's input codes and on zeros
+    pipe_only = {}
+    for name, codes in (("random_operands", qx0.view(-1)[: 1 << 22]), ("zero_operands", None)):
+        flop = [0.0]
+
+        def probe(i, codes=codes):
+            flop[0] = ops.mfma_fp8_probe(codes, 300)
+
+        us = batched(probe)
+        pipe_only[name] = {"us": round(us, 2), "TFLOP/s": round(flop[0] / us / 1e6, 1)}
+    pipe_only["random_operands"]["shader_clock_ghz"] = clock_under(lambda i: ops.mfma_fp8_probe(qx0.view(-1)[: 1 << 22], 300))
     clocks = {
         "idle": clock_under(lambda i: None),
         "up_gemm_random_operands": clock_under(lambda i: ops.fp8_linear(qx0, wp_up, sx0, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh0)),
@@ -298,6 +310,9 @@ def main():
                 "traffic": traffic, "traffic_unit": "bytes per launch (algorithmic: 1.65e8)", "traffic_source": traffic_src,
                 "same_kernel_all_zero_operands": {"us": round(zeros_us, 2), "TFLOP/s": round(gemm_flops / zeros_us / 1e6, 1),
                                                   "frac": round(gemm_flops / zeros_us / 1e6 / FP8_PEAK_TFLOPS, 4)},
+                # the same instruction stream without any memory or LDS traffic (lq_mfma_fp8_probe): on real operands the part is
+                # power limited below the published peak before a GEMM has moved a byte
+                "matrix_pipes_alone": pipe_only,
                 "shader_clock_ghz": clocks,
                 "vendor_fp8_gemm_same_operands_us": vendor}  # plain GEMMs of the vendor library, no bias / GELU / amax
     # what the matrix pipes can deliver at the clock the device sustains under this kernel: CUs x 8192 FP8 FLOP per clock

@@ -465,6 +465,14 @@ int lq_gemm_profile(lq_weight_kind_t kind, int m, int n, int k, void* workspace,
  * are power-limited on random operands).  Enqueued on `stream`, returns immediately; 1 <= probes <= 1024. */
 int lq_shader_clock_probe(uint64_t* out_ticks, int probes, unsigned microseconds, lq_stream_t stream);
 
+/* Measurement aid (no reference counterpart): one 256-thread workgroup per CU; every wavefront issues `iters` times 16
+ * independent v_mfma_f32_32x32x64_f8f6f4 (a 128x128 wavefront tile) on register operands drawn from `operand_codes` (e4m3
+ * codes, n_codes >= 4, 4-byte aligned; NULL = all-zero operands) and rotated between iterations, with no memory or LDS
+ * traffic: 2*32*32*64 * 16 * iters * 4 * *workgroups FLOP per launch.  Timed by the caller, it gives what the matrix pipes
+ * alone sustain on this part -- on real codes they are power limited well below the published peak, on zeros they are not.
+ * `sink` (4 bytes of device memory) is practically never written; *workgroups (optional) receives the grid size. */
+int lq_mfma_fp8_probe(float* sink, const uint8_t* operand_codes, size_t n_codes, int iters, int* workgroups, lq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

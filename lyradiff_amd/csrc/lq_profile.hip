@@ -79,6 +79,69 @@ extern "C" int lq_shader_clock_probe(uint64_t* out_ticks, int probes, unsigned m
     return check_launch("lq_shader_clock_probe");
 }
 
+// What the matrix pipes alone sustain: every wavefront (one per SIMD, one workgroup per CU) issues 16 independent
+// v_mfma_f32_32x32x64_f8f6f4 per iteration on operand fragments held in registers -- a 128x128 wavefront tile without any
+// memory or LDS traffic -- and rotates the fragments' registers between iterations so that the operand buses keep toggling
+// as they do in a GEMM.  With operands drawn from real e4m3 codes the part is power limited; with zeros it is not.
+__global__ __launch_bounds__(256, 1) void mfma_fp8_probe_kernel(float* sink, const uint32_t* __restrict__ src, size_t src_words, int iters) {
+    typedef int v8i_t __attribute__((ext_vector_type(8)));
+    typedef float v16f_t __attribute__((ext_vector_type(16)));
+    v8i_t a[4], b[4];
+#pragma unroll
+    for (int f = 0; f < 4; ++f)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const size_t ia = ((size_t)blockIdx.x * 8192 + (threadIdx.x + 256 * f) * 8 + i) % (src_words ? src_words : 1);
+            const size_t ib = ((size_t)blockIdx.x * 8192 + (threadIdx.x + 256 * (f + 4)) * 8 + i) % (src_words ? src_words : 1);
+            a[f][i] = src ? (int)src[ia] : 0;
+            b[f][i] = src ? (int)src[ib] : 0;
+        }
+    v16f_t acc[16];
+#pragma unroll
+    for (int t = 0; t < 16; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[t][i] = 0.0f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[i * 4 + j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[i], b[j], acc[i * 4 + j], 0, 0, 0, 0, 0, 0);
+#pragma unroll
+        for (int f = 0; f < 4; ++f) {
+            int t = a[f][0];
+#pragma unroll
+            for (int i = 0; i < 7; ++i) a[f][i] = a[f][i + 1];
+            a[f][7] = t;
+            t = b[f][7];
+#pragma unroll
+            for (int i = 7; i > 0; --i) b[f][i] = b[f][i - 1];
+            b[f][0] = t;
+        }
+    }
+    float sum = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 16; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sum += acc[t][i];
+    if (sum == 12345.678f) sink[0] = sum;  // keeps the loop alive; practically never taken
+}
+
+extern "C" int lq_mfma_fp8_probe(float* sink, const uint8_t* operand_codes, size_t n_codes, int iters, int* workgroups,
+                                 lq_stream_t stream) {
+    LQ_REQUIRE(sink != nullptr && iters >= 1 && iters <= (1 << 20), LQ_ERR_ARG, "lq_mfma_fp8_probe: need a sink and 1..2^20 iterations");
+    LQ_REQUIRE(operand_codes == nullptr || (n_codes >= 4 && reinterpret_cast<uintptr_t>(operand_codes) % 4 == 0), LQ_ERR_ARG,
+               "lq_mfma_fp8_probe: operand codes must be 4-byte aligned and at least 4 bytes");
+    int dev = 0, cus = 0;
+    LQ_REQUIRE(hipGetDevice(&dev) == hipSuccess &&
+                   hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0,
+               LQ_ERR_HIP, "lq_mfma_fp8_probe: cannot read the CU count");
+    if (workgroups) *workgroups = cus;
+    hipLaunchKernelGGL(mfma_fp8_probe_kernel, dim3((unsigned)cus), dim3(256), 0, as_stream(stream), sink,
+                       reinterpret_cast<const uint32_t*>(operand_codes), n_codes / 4, iters);
+    return check_launch("lq_mfma_fp8_probe");
+}
+
 extern "C" size_t lq_gemm_profile_workspace(lq_weight_kind_t kind, int m, int n, int k) {
     if (m <= 0 || n <= 0 || k <= 0 || lq_gemm_tactic_count(kind) < 0) return 0;
     return profile_layout(kind, m, n, k).total;

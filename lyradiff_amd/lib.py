@@ -103,6 +103,7 @@ SYMBOLS = {
     "lq_gemm_profile_workspace": (_Z, [_I, _I, _I, _I]),
     "lq_gemm_profile": (_I, [_I, _I, _I, _I, _P, _Z, C.POINTER(_I), C.POINTER(_F), _P]),
     "lq_shader_clock_probe": (_I, [_P, _I, C.c_uint, _P]),
+    "lq_mfma_fp8_probe": (_I, [_P, _P, C.c_size_t, _I, _P, _P]),
 }
 
 

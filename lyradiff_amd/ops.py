@@ -713,6 +713,22 @@ def shader_clock_probe(microseconds: int, probes: int = 8, stream=None):
     return out
 
 
+_PROBE_SINK = {}
+
+
+def mfma_fp8_probe(codes, iters: int) -> float:
+    """Enqueues lq_mfma_fp8_probe (one workgroup per CU, 16 x iters FP8 MFMAs of 32x32x64 per wavefront on register
+    operands drawn from the uint8 e4m3 tensor `codes`, or on zeros when codes is None) and returns the FLOP of the launch."""
+    dev = torch.cuda.current_device()
+    sink = _PROBE_SINK.get(dev)
+    if sink is None:
+        sink = _PROBE_SINK[dev] = torch.zeros(1, dtype=torch.float32, device="cuda")
+    wgs = C.c_int(0)
+    _l.check(_l.load().lq_mfma_fp8_probe(_ptr(sink), None if codes is None else _ptr(codes), 0 if codes is None else codes.numel(),
+                                         int(iters), C.byref(wgs), _stream()), "lq_mfma_fp8_probe")
+    return 2.0 * 32 * 32 * 64 * 16 * iters * 4 * wgs.value
+
+
 def gemm_shape_tactic(kind: str, m: int, n: int, k: int, tactic=None) -> int:
     """Reads (tactic=None) or writes the per-shape tactic cache; -1 removes an entry / means no entry."""
     lib = _l.load()
