@@ -273,6 +273,20 @@ def test_w4a4_gemm_every_tactic(ops, dev, tactic, sdt, tactic_guard):
         assert np.array_equal(y32.cpu().numpy(), ref), f"k={kk}"
 
 
+def test_matrix_pipe_probe_runs_and_reports_its_work(ops, dev):
+    """lq_mfma_fp8_probe: measurement aid; the launch completes and the FLOP count follows the CU count."""
+    import torch
+
+    codes = torch.randint(0, 120, (1 << 16,), dtype=torch.uint8, device=dev)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    for c in (codes, None):
+        flop = ops.mfma_fp8_probe(c, 8)
+        torch.cuda.synchronize()
+        assert flop == 2.0 * 32 * 32 * 64 * 16 * 8 * 4 * cus
+    with pytest.raises(Exception):
+        ops.mfma_fp8_probe(codes, 0)
+
+
 def test_profiler_fills_the_shape_cache(ops, dev, tactic_guard):
     """lq_gemm_profile picks a valid configuration, later calls of that shape use it, results stay exact."""
     m, n, k = 1000, 1280, 1280
