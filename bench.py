@@ -16,7 +16,11 @@ Inputs and (pre-quantised, rows32-repacked) weights are resident in HBM before t
 the whole step, quant kernels included.  The JSON line also carries:
   roofline      the dominant kernel (up-projection FP8 GEMM) priced against the dense FP8 MFMA peak
                 from HIP-event timings taken inside the timed steps, on the launch stream (every
-                --event-every-th step carries the markers: they are not free, see --help);
+                --event-every-th step carries the markers: they are not free, see --help); beside it, measured after the
+                timed region: the same kernel on all-zero operands, the shader clock under it, under the vendor library's
+                FP8 GEMM and idle, the vendor GEMM's time on both shapes, and `matrix_pipes_alone`: the FP8 MFMA stream
+                of a 128x128 wavefront tile on register operands without any memory traffic (what the part's power
+                limit leaves of the published peak before a GEMM has moved a byte);
   cpu_baseline  the same math (dequantise e4m3 -> fp32 matmul -> scale/bias/GELU) through PyTorch
                 CPU on the host cores (oracle port; a reported baseline only);
   kernels       per-kernel averages of the same timed steps (GEMM TFLOP/s, act-quant GB/s);
