@@ -12,11 +12,12 @@ template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
     if (t < 0) {
         const long t256 = (long)((p.m + 255) / 256) * ((p.n + 255) / 256);
         const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
-        // 256x256 tiles, one wavefront per SIMD, when their rounds on the 256 CUs are at least three quarters full (measured
-        // on the FLUX shapes at 4608 and 6912 rows: ahead of the others from 0.84 up, behind at 0.63); otherwise 128x256
-        // tiles, two workgroups per CU (finer tail, one workgroup's epilogue overlaps the other's MFMA work)
-        const long rounds256 = (t256 + 255) / 256;
-        t = t256 >= 192 ? (4 * t256 >= 3 * 256 * rounds256 ? 6 : 4) : (t128 >= 192 ? 2 : 3);
+        // 256x256 tiles, one wavefront per SIMD, when their last round on the 256 CUs is at least half full (measured on
+        // the FLUX shapes at 4608 and 6912 rows, FP8 and INT8: ahead of the others by up to 10 % then, level or up to 4 %
+        // behind otherwise); else 128x256 tiles, two workgroups per CU (finer tail, one workgroup's epilogue overlaps the
+        // other's MFMA work)
+        const long last256 = t256 % 256;
+        t = t256 >= 192 ? ((last256 == 0 || last256 >= 128) ? 6 : 4) : (t128 >= 192 ? 2 : 3);
         if (p.k <= 1024 && t128 >= 192) t = 2;  // short K: prologue and epilogue dominate, smaller tiles overlap them better
     }
     if (t == 1 && p.kb % 128 != 0) t = 0;  // the 128-byte k-tile needs k % 128 == 0
