@@ -234,6 +234,20 @@ def test_int8_gemm_every_tactic(ops, dev, tactic, k, tactic_guard):
     assert np.array_equal(to_np_f32(y), O.int8_epilogue(ref_acc, ac.numpy(), ar.numpy(), to_np_f32(bias), "f16"))
 
 
+@pytest.mark.parametrize("tactic", range(N_TACTICS["int8"]))
+@pytest.mark.parametrize("k", [64, 128, 192, 320])
+def test_int8_gemm_fewer_k_tiles_than_pipeline_stages(ops, dev, tactic, k, tactic_guard):
+    """One to five k-tiles: the pipelines of three and four stages start, re-fetch past the end and drain correctly
+    when the loop is shorter than they are deep (exact int32 sums)."""
+    m, n = 300, 288
+    g = rng_t(1700 + 10 * tactic + k)
+    a = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int8)
+    w = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8)
+    ops.gemm_set_tactic("int8", tactic)
+    acc = ops.int8_linear(a.to(dev), ops.repack_weight(w.to(dev)), None, None, None, torch.int32)
+    assert np.array_equal(acc.cpu().numpy(), O.gemm_i8_acc(a.numpy(), w.numpy()))
+
+
 @pytest.mark.parametrize("tactic", range(N_TACTICS["fp8"]))
 @pytest.mark.parametrize("k", [704, 768])
 def test_fp8_gemm_every_tactic(ops, dev, tactic, k, tactic_guard):
