@@ -221,7 +221,7 @@ extern "C" int lq_gemm_profile(lq_weight_kind_t kind, int m, int n, int k, void*
     float best_of[kMaxTactics];
     bool usable[kMaxTactics];
     for (int t = 0; t < kMaxTactics; ++t) { best_of[t] = 0.0f; usable[t] = t < count; }
-    for (int round = 0; round < kRounds + 1; ++round) {  // round 0 is the warm-up
+    for (int round = 0; round < kRounds + 1; ++round) {  // the first pass is the warm-up
         for (int t = 0; t < count && t < kMaxTactics; ++t) {
             if (!usable[t]) continue;
             tl_forced_tactic = t;
