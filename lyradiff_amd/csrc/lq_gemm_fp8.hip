@@ -21,6 +21,14 @@ template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
         if (p.k <= 1024 && t128 >= 192) t = 2;  // short K: prologue and epilogue dominate, smaller tiles overlap them better
     }
     if (t == 1 && p.kb % 128 != 0) t = 0;  // the 128-byte k-tile needs k % 128 == 0
+    // The per-shape cache is filled by timing the plain epilogue.  With one workgroup per CU nothing runs beside tactic 6's
+    // epilogue, and one that does more than scale and bias (activation, output maximum, codes, gate, residual) then costs
+    // a quarter of the kernel on a shape of several rounds of tiles (up projection 4608x12288x3072 with GELU and the output
+    // maximum: 214 us against 160 us with two 128x256 workgroups per CU).  A configuration forced by the caller is kept.
+    const bool forced = tl_forced_tactic >= 0 || g_tactic_fp8 >= 0;
+    const bool plain_epilogue = p.gelu == 0 && p.out_scale == nullptr && p.C8 == nullptr && p.gate == nullptr &&
+                                p.residual == nullptr && p.addend == nullptr;
+    if (t == 6 && !forced && !plain_epilogue && (long)((p.m + 255) / 256) * ((p.n + 255) / 256) > 256) t = 4;
     switch (t) {
         case 0: return launch_gemm<K_FP8, OutTag, 256, 256, 64, 2, 4, 3>(p, st);
         case 1: return launch_gemm<K_FP8, OutTag, 256, 256, 128, 2, 4, 2>(p, st);
