@@ -21,14 +21,16 @@ template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
         if (p.k <= 1024 && t128 >= 192) t = 2;  // short K: prologue and epilogue dominate, smaller tiles overlap them better
     }
     if (t == 1 && p.kb % 128 != 0) t = 0;  // the 128-byte k-tile needs k % 128 == 0
-    // The per-shape cache is filled by timing the plain epilogue.  With one workgroup per CU nothing runs beside tactic 6's
-    // epilogue, and one that does more than scale and bias (activation, output maximum, codes, gate, residual) then costs
-    // a quarter of the kernel on a shape of several rounds of tiles (up projection 4608x12288x3072 with GELU and the output
-    // maximum: 214 us against 160 us with two 128x256 workgroups per CU).  A configuration forced by the caller is kept.
+    // The per-shape cache is filled by timing the plain epilogue.  With one wavefront per SIMD nothing runs beside tactic 6's
+    // epilogue: one that does more than scale and bias (activation, output maximum, codes, gate, residual) costs 13-18 us
+    // per 256x256 tile there (transcendentals, or one exposed memory round trip per group of rows) and next to nothing with
+    // two wavefronts per SIMD.  Measured at 4608 rows: 12288x3072 with GELU and the output maximum 209-214 us against
+    // 153-160 us with tactic 4; 3072x12288 with gate and residual 139 us against 134 us with tactic 0, 3072x3072 55 against
+    // 48 us.  A configuration forced by the caller is kept.
     const bool forced = tl_forced_tactic >= 0 || g_tactic_fp8 >= 0;
     const bool plain_epilogue = p.gelu == 0 && p.out_scale == nullptr && p.C8 == nullptr && p.gate == nullptr &&
                                 p.residual == nullptr && p.addend == nullptr;
-    if (t == 6 && !forced && !plain_epilogue && (long)((p.m + 255) / 256) * ((p.n + 255) / 256) > 256) t = 4;
+    if (t == 6 && !forced && !plain_epilogue) t = (long)((p.m + 255) / 256) * ((p.n + 255) / 256) > 256 ? 4 : 0;
     switch (t) {
         case 0: return launch_gemm<K_FP8, OutTag, 256, 256, 64, 2, 4, 3>(p, st);
         case 1: return launch_gemm<K_FP8, OutTag, 256, 256, 128, 2, 4, 2>(p, st);
