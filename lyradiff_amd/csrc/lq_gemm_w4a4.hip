@@ -15,6 +15,10 @@ template <int KIND, typename OutTag> static int run_w4a4(GemmParams p, hipStream
     if (t < 0) {
         const long tiles = (long)((p.m + 63) / 64) * ((p.n + 127) / 128);
         t = tiles >= 768 ? 0 : 1;  // three workgroups per CU on 256 CUs
+        // 16-bit scales, short K: the 128x64 tile (same 64x32 wavefront tile, two rows of wavefronts sharing the weight
+        // stage) measured 1-6 % ahead of the 64x128 one at K = 3072 (4608x3072x3072: 91 against 97 us) and 3-4 % behind at
+        // K >= 12288; with fp32 scales the two are level
+        if (t == 0 && KIND == K_W4A4H && p.k <= 4096) t = 2;
     }
     switch (t) {
         case 0: return launch_gemm<KIND, OutTag, 64, 128, 64, 1, 4, 2>(p, st);
