@@ -17,7 +17,7 @@ template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
         // behind otherwise); else 128x256 tiles, two workgroups per CU (finer tail, one workgroup's epilogue overlaps the
         // other's MFMA work)
         const long last256 = t256 % 256;
-        t = t256 >= 192 ? ((last256 == 0 || last256 >= 128) ? 6 : 4) : (t128 >= 192 ? 2 : 3);
+        t = t256 >= 192 ? ((last256 == 0 || last256 >= 128) ? 6 : 4) : (t128 >= 128 ? 2 : 3);  // 128x128 tiles from half a round up (4096x640x2560: 14.5 against 16.3 us with 64x64)
         if (p.k <= 1024 && t128 >= 192) t = 2;  // short K: prologue and epilogue dominate, smaller tiles overlap them better
     }
     if (t == 1 && p.kb % 128 != 0) t = 0;  // the 128-byte k-tile needs k % 128 == 0
