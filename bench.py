@@ -16,7 +16,7 @@ Inputs and (pre-quantised, rows32-repacked) weights are resident in HBM before t
 the whole step, quant kernels included.  The JSON line also carries:
   roofline      the dominant kernel (up-projection FP8 GEMM) priced against the dense FP8 MFMA peak
                 from HIP-event timings taken inside the timed steps, on the launch stream (every
-                --event-every-th step carries the markers: they are not free, see --help); beside it, measured after the
+                --event-every-th step brackets one kernel: markers are not free, see --help); beside it, measured after the
                 timed region: the same kernel on all-zero operands, the shader clock under it, under the vendor library's
                 FP8 GEMM and idle, the vendor GEMM's time on both shapes, and `matrix_pipes_alone`: the FP8 MFMA stream
                 of a 128x128 wavefront tile on register operands without any memory traffic (what the part's power
@@ -104,10 +104,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=M)
     ap.add_argument("--extra", action="store_true", help="also time the INT8 / W4A4 / SDXL-shape kernels")
-    ap.add_argument("--event-every", type=int, default=5,
-                    help="bracket every kernel with HIP events on every N-th timed step; the five markers of such a step "
-                         "cost the GPU 15-20 us (387-393 us per step with N=1, 370-373 us with none), so the per-kernel "
-                         "figures come from a sample of the timed steps")
+    ap.add_argument("--event-every", type=int, default=2,
+                    help="on every N-th timed step ONE kernel is bracketed by a pair of HIP events (the up GEMM on every other "
+                         "such step, the three others in turn); markers are not free -- five of them in one step cost the "
+                         "GPU 15-20 us -- so a marked step carries two and the per-kernel figures come from a sample")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path shards by token rows without "
@@ -143,30 +143,38 @@ def main():
     s_h = [torch.zeros(1, dtype=torch.float32, device=dev) for _ in range(2)]
     ev = lambda: torch.cuda.Event(enable_timing=True)
     names = ["quant_x", "gemm_up", "quant_h", "gemm_down"]
-    marks = []
+    marks = {n: [] for n in names}
 
-    def step(i, record=False):
+    def step(i, record=None):
+        """One pass of the chain; record = index into `names` of the one kernel to bracket with a pair of events."""
         xi = xs[i % n_rot]
-        e = [ev() for _ in range(5)] if record else None
-        if record:
+        e = (ev(), ev()) if record is not None else None
+        if record == 0:
             e[0].record()
         qx, sx = ops.fp8_quant(xi)
-        if record:
+        if record == 0:
             e[1].record()
         # the up projection's epilogue also accumulates max|h|/448, the dynamic scale of h, so the quantisation
         # of h is a single cast pass (the same numbers as an amax pass over h followed by the cast)
         sh = s_h[i % 2]
         sh.zero_()
+        if record == 1:
+            e[0].record()
         h = ops.fp8_linear(qx, wp_up, sx, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh)
-        if record:
-            e[2].record()
+        if record == 1:
+            e[1].record()
+        if record == 2:
+            e[0].record()
         qh = ops.fp8_scale_cast(h, sh)
-        if record:
-            e[3].record()
+        if record == 2:
+            e[1].record()
+        if record == 3:
+            e[0].record()
         y = ops.fp8_linear(qh, wp_dn, sh, s_dn, bd, False, None, 0.0, torch.bfloat16)
-        if record:
-            e[4].record()
-            marks.append(e)
+        if record == 3:
+            e[1].record()
+        if record is not None:
+            marks[names[record]].append(e)
         return y
 
     # Set-up, before the W warm-up steps: bring the device out of idle.  From an idle start the power management needs about
@@ -194,15 +202,17 @@ def main():
         y = step(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    every = max(1, args.event_every)
+    turn = (1, 0, 1, 2, 1, 3)  # which kernel a marked step brackets: the roofline kernel every other time
     for i in range(args.steps):
-        y = step(i, record=(i % max(1, args.event_every) == 0))
+        y = step(i, record=turn[(i // every) % len(turn)] if i % every == 0 else None)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
 
     ms_per_step = dt / args.steps * 1e3
     flops_step = 2.0 * M * (D * H + H * D)
     value = flops_step / (dt / args.steps) / 1e12
-    per = {n: sum(m[k].elapsed_time(m[k + 1]) for m in marks) / len(marks) * 1e3 for k, n in enumerate(names)}  # us
+    per = {n: (sum(a.elapsed_time(b) for a, b in marks[n]) / len(marks[n]) * 1e3 if marks[n] else None) for n in names}  # us
     gemm_flops = 2.0 * M * D * H
 
     # ---- after the timed region: each kernel alone, launched back to back between ONE pair of events (no marker
@@ -293,6 +303,9 @@ def main():
         del w8
     del zq, zw
 
+    for n_ in names:  # a kernel that no marked step bracketed (very few --steps): its back-to-back time stands in
+        if per[n_] is None:
+            per[n_] = alone[n_]
     kernels = {
         "gemm_up_fp8_4608x12288x3072": {"us_in_step_incl_launch_gap": round(per["gemm_up"], 2), "us_back_to_back": round(alone["gemm_up"], 2),
                                         "TFLOP/s": round(gemm_flops / alone["gemm_up"] / 1e6, 1)},
@@ -308,7 +321,7 @@ def main():
     roofline = {"bound": "mfma", "kernel": "lq::gemm_kernel<fp8> 4608x12288x3072 (bias+GELU, bf16 out)",
                 "achieved": round(achieved, 1), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / FP8_PEAK_TFLOPS, 4),
-                "timing": f"HIP events around the kernel on {len(marks)} of the {args.steps} timed steps, on the launch stream",
+                "timing": f"a pair of HIP events around the kernel on {len(marks['gemm_up'])} of the {args.steps} timed steps, on the launch stream",
                 # HBM-side bytes per launch of this kernel: not measured in this run -- taken from the committed rocprofv3
                 # --pmc summary (FETCH_SIZE x2.0, the factor a plain copy of known size gives on this part, + WRITE_SIZE)
                 "traffic": traffic, "traffic_unit": "bytes per launch (algorithmic: 1.65e8)", "traffic_source": traffic_src,
@@ -337,8 +350,9 @@ def main():
                    "tokens": M, "d_model": D, "d_ff": H, "profiled_tactics": tactics,
                    "settle_steps_before_warmup": settled_after, "settle_ms": round(settle_ms, 1)},
         "roofline": roofline, "kernels": kernels,
-        "kernel_timing": f"us_in_step_incl_launch_gap: HIP events around each kernel on {len(marks)} of the {args.steps} timed steps "
-                         "(the event markers and the gap to the next launch are inside); us_back_to_back: 20 launches of the "
+        "kernel_timing": f"us_in_step_incl_launch_gap: a pair of HIP events around one kernel on {sum(len(v) for v in marks.values())} of the "
+                         f"{args.steps} timed steps ({', '.join(f'{n}: {len(v)}' for n, v in marks.items())}; the markers "
+                         "themselves and the gap to the next launch are inside); us_back_to_back: 20 launches of the "
                          "kernel alone between one pair of events, after the timed region (rates are computed from these)",
     }
     if not args.no_cpu:
