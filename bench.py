@@ -303,6 +303,12 @@ def main():
         del w8
     del zq, zw
 
+    # the other two GEMMs the metric names, at their FLUX 1024^2 shapes, timed like `alone` above (after the timed region):
+    # W8A8 = INT8 up projection with per-token x per-channel dequant + bias, fp16 out; W4A4 = attention projection with
+    # 16-bit group scales (BASELINE.json configs[3]), bf16 out.  Both are priced against the dense int8 MFMA peak (there
+    # is no int4 matrix instruction; the W4A4 kernel widens nibbles to int8).
+    other = other_metric_gemms(torch, ops, dev, batched)
+
     for n_ in names:  # a kernel that no marked step bracketed (very few --steps): its back-to-back time stands in
         if per[n_] is None:
             per[n_] = alone[n_]
@@ -316,6 +322,7 @@ def main():
         "fp8_cast_with_gemm_scale_4608x12288": {"us_in_step_incl_launch_gap": round(per["quant_h"], 2), "us_back_to_back": round(alone["quant_h"], 2),
                                                 "GB/s": round(3.0 * M * H / alone["quant_h"] / 1e3, 1)},
     }
+    kernels.update(other)
     achieved = gemm_flops / per["gemm_up"] / 1e6
     traffic, traffic_src = profiled_traffic()
     roofline = {"bound": "mfma", "kernel": "lq::gemm_kernel<fp8> 4608x12288x3072 (bias+GELU, bf16 out)",
@@ -369,6 +376,34 @@ def main():
     if args.extra:
         out["extra"] = extra_kernels(torch, ops, dev)
     print(json.dumps(out))
+
+
+def other_metric_gemms(torch, ops, dev, batched):
+    """INT8 W8A8 GEMM 4608x12288x3072 and W4A4 GEMM 4608x3072x3072 (16-bit group scales), random codes, back to back."""
+    g = torch.Generator().manual_seed(1003)
+    out = {}
+    m, n, k = M, H, D
+    ops.gemm_profile("int8", m, n, k, dev)
+    a = torch.randint(-127, 128, (m, k), generator=g, dtype=torch.int8).to(dev)
+    w = ops.repack_weight(torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8).to(dev))
+    ac = (torch.rand(n, generator=g) * 9e-3 + 1e-3).to(dev)
+    ar = (torch.rand(m, generator=g) * 0.05).to(dev)
+    b = (torch.randn(n, generator=g) * 0.02).half().to(dev)
+    us = batched(lambda i: ops.int8_linear(a, w, ac, ar, b, torch.float16))
+    tops = 2.0 * m * n * k / us / 1e6
+    out[f"gemm_int8_w8a8_{m}x{n}x{k}"] = {"us_back_to_back": round(us, 2), "TOP/s": round(tops, 1),
+                                          "frac_of_int8_peak": round(tops / INT8_PEAK_TOPS, 4)}
+    del a, w
+    m, n, k = M, D, D
+    aw = torch.randint(-2 ** 31, 2 ** 31 - 1, (m, k // 8), generator=g, dtype=torch.int32).to(dev)
+    ww = ops.repack_weight(torch.randint(0, 256, (n, k // 2), generator=g, dtype=torch.int32).to(torch.uint8).to(dev))
+    sa = torch.rand(m, k // 64, generator=g).half().to(dev)
+    sb = torch.rand(n, k // 64, generator=g).half().to(dev)
+    us = batched(lambda i: ops.w4a4_linear(aw, ww, sa, sb, None, torch.bfloat16))
+    tops = 2.0 * m * n * k / us / 1e6
+    out[f"gemm_w4a4_f16scales_{m}x{n}x{k}"] = {"us_back_to_back": round(us, 2), "TOP/s": round(tops, 1),
+                                               "frac_of_int8_peak": round(tops / INT8_PEAK_TOPS, 4)}
+    return out
 
 
 def extra_kernels(torch, ops, dev):
