@@ -261,14 +261,19 @@ int lq_fp8_scale_cast_2d(uint8_t* dst, size_t dst_ld, const void* src, size_t sr
  * A, C, scale, bias of `dtype` (F16 or BF16); B_prepared from lq_repack_weight_only.  n % 32 == 0, k % 64 == 0.
  * Replaces CutlassFpAIntBGemmRunner<T, uint8_t | uint4b_t, PER_COLUMN_SCALE_ONLY>::gemm (A, B, weight_scales, [biases,]
  * C, m, n, k, ...) (kernels/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm.h:27-130).  The reference multiplies every
- * dequantised weight by the scale in T inside the main loop; here the scale is applied once per output. */
+ * dequantised weight by the scale in T inside the main loop; here the scale is applied once per output.
+ * Two tile configurations: 0 = 256x256 (eight wavefronts, three stages; chosen from 192 such tiles up), 1 = 256x128 (four
+ * wavefronts, two stages); both walk k in the same order and give the same bits.  lq_gemm_set_thread_tactic(0 | 1) picks
+ * one for the calling thread's next calls (the gemm_config argument of CutlassFpAIntBGemmRunner::gemm), -1 the built-in rule. */
 int lq_gemm_weight_only(void* C, const void* A, lq_dtype_t dtype, const uint8_t* B_prepared, lq_weight_kind_t kind,
                         const void* scales, const void* bias, int m, int n, int k, lq_stream_t stream);
 
 /* The same GEMM with group-wise ("fine-grained") scales and optional zero points along k:
  *   C[m,n] = T( sum_k A[m,k] * w[k,n] [+ f32(bias[n])] ),  w[k,n] the dequantised weight formed in T per element:
  *     F16:   w = T( T(q[k,n] * scale[k/g, n]) + zero[k/g, n] )      (multiply, then add: two roundings)
- *     BF16:  w = T( q[k,n] * scale[k/g, n] + zero[k/g, n] )         (one fused multiply-add)
+ *     BF16:  w = T( f32( q[k,n] * scale[k/g, n] + zero[k/g, n] ) )  (one fused multiply-add rounded to fp32, then to bf16; the
+ *            reference's __hfma2 rounds the exact sum to bf16 once -- the two differ by one bf16 step where the fp32 value
+ *            falls on a bf16 midpoint, measured on < 1e-3 of random weights)
  *   and w = T(q * scale) for both when `zeros` is NULL; q is the signed code (the +128 / +8 of the prepared layout removed).
  * scales and zeros are row-major [k / group_size, n] of `dtype`; group_size 64 or 128, k % group_size == 0.
  * Replaces CutlassFpAIntBGemmRunner<T, uint8_t | uint4b_t, FINEGRAINED_SCALE_ONLY | FINEGRAINED_SCALE_AND_ZEROS>::gemm(A, B,

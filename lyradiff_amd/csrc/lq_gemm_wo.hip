@@ -386,8 +386,13 @@ static int wo_launch(void* C, const void* A, lq_dtype_t dtype, const uint8_t* B_
     const int grouped = group_size == 0 ? 0 : (zeros == nullptr ? 1 : 2);
     const int tiles_per_group = group_size == 0 ? 1 : group_size / 64;
     // 256x256 tiles (eight wavefronts, three stages) once they give every CU work; 256x128 tiles otherwise
+    // A tile configuration set with lq_gemm_set_thread_tactic wins: 0 = 256x256, 1 = 256x128.
     const long big_tiles = (long)((m + 255) / 256) * ((n + 255) / 256);
-    const bool big = big_tiles >= 192;
+    if (tl_forced_tactic > 1) {
+        set_error("gemm_weight_only: unknown tile configuration %d (0 = 256x256, 1 = 256x128)", tl_forced_tactic);
+        return LQ_ERR_ARG;
+    }
+    const bool big = tl_forced_tactic >= 0 ? tl_forced_tactic == 0 : big_tiles >= 192;
     hipStream_t st = as_stream(stream);
 #define LQ_WO_GO(TAG, W4V, WNV, NST, GRP)                                                                               \
     do {                                                                                                                \

@@ -681,6 +681,22 @@ def gemm_set_tactic(kind: str, tactic: int = -1) -> None:
     _l.check(_l.load().lq_gemm_set_tactic(_KINDS[kind], int(tactic)), "lq_gemm_set_tactic")
 
 
+class gemm_thread_tactic:
+    """`with gemm_thread_tactic(t):` -- the GEMM calls of this thread inside the block use tile configuration t (the per-call
+    gemmConfig argument of the reference's runners, kernels/cutlass_kernels/int8_gemm/int8_gemm.h:24-36)."""
+
+    def __init__(self, tactic: int):
+        self.tactic = int(tactic)
+
+    def __enter__(self):
+        _l.check(_l.load().lq_gemm_set_thread_tactic(self.tactic), "lq_gemm_set_thread_tactic")
+        return self
+
+    def __exit__(self, *exc):
+        _l.load().lq_gemm_set_thread_tactic(-1)
+        return False
+
+
 def gemm_tactic_count(kind: str) -> int:
     return int(_l.load().lq_gemm_tactic_count(_KINDS[kind]))
 

@@ -323,7 +323,7 @@ def test_gemm_w4a4_epilogue_options_match_the_unfused_sequence(ops, dev, dt, m, 
     assert np.all(np.abs(gl - ref) <= ulp * np.abs(ref) + 1e-6)
 
 
-def _int4_state(prefix, n, k, g, rank=32, bias=True):
+def _int4_state(prefix, n, k, g, rank=32, bias=True, lora_scale=0.05):
     """Host-side W4A4 weight container entries with the reference's key names."""
     w = 0.05 * torch.randn(n, k, generator=g)
     wv = w.view(n, k // 64, 64)
@@ -332,8 +332,8 @@ def _int4_state(prefix, n, k, g, rank=32, bias=True):
     packed = ((q[:, 0::2] & 0xF) | ((q[:, 1::2] & 0xF) << 4)).to(torch.uint8).view(torch.int8)
     sd = {prefix + "packed_weight": packed.contiguous(), prefix + "weight_scale": sc.float().contiguous(),
           prefix + "smooth": (0.5 + torch.rand(k, generator=g)).float(),
-          prefix + "lora_up": (0.05 * torch.randn(n, rank, generator=g)).bfloat16(),
-          prefix + "lora_down": (0.05 * torch.randn(rank, k, generator=g)).bfloat16()}
+          prefix + "lora_up": (lora_scale * torch.randn(n, rank, generator=g)).bfloat16(),
+          prefix + "lora_down": (lora_scale * torch.randn(rank, k, generator=g)).bfloat16()}
     if bias:
         sd[prefix + "bias"] = (0.1 * torch.randn(n, generator=g)).bfloat16()
     return sd
@@ -745,27 +745,29 @@ def test_flux_block_ops_reload_model_from_bin(ops, dev, tmp_path, file_dtype):
         sf.reload_model_from_bin(str(tmp_path) + "/absent.", "fp32")
 
 
-def _int4_block_state(d, dh, g):
+def _int4_block_state(d, dh, g, scale_w=0.03, lora_scale=0.05):
     """State dict of one double ("transformer_blocks.0.") and one single ("single_transformer_blocks.0.") INT4 block in the
     reference's container layout; the adaLN linears carry FP8 input scales, which the non-FULL level ignores."""
+    _state_dict_ = lambda names, seed, prefix: _state_dict(names, seed, scale_w=scale_w, prefix=prefix)
+    _int4_state_ = lambda prefix, n, k, g, bias=True: _int4_state(prefix, n, k, g, bias=bias, lora_scale=lora_scale)
     sd = {}
     for pre, ada in (("transformer_blocks.0.", ("norm1.linear", "norm1_context.linear")), ("single_transformer_blocks.0.", ("norm.linear",))):
         chunks = 6 if len(ada) == 2 else 3
-        sd.update(_state_dict({a: (chunks * d, d) for a in ada}, 402, prefix=pre))
+        sd.update(_state_dict_({a: (chunks * d, d) for a in ada}, 402, prefix=pre))
         for a in ada:
             sd[f"{pre}{a}_input_scale"] = torch.tensor([4.0 / 448])
         for n in ("norm_q", "norm_k", "norm_added_q", "norm_added_k"):
             sd[f"{pre}attn.{n}.weight"] = (1 + 0.1 * torch.randn(dh, generator=g)).bfloat16()
     for name, n in (("attn.to_qkv.", 3 * d), ("attn.to_added_qkv.", 3 * d), ("attn.to_out.0.", d), ("attn.to_add_out.", d)):
-        sd.update(_int4_state("transformer_blocks.0." + name, n, d, g))
+        sd.update(_int4_state_("transformer_blocks.0." + name, n, d, g))
     for ff in ("ff.", "ff_context."):
-        sd.update(_int4_state(f"transformer_blocks.0.{ff}net.0.proj.", 4 * d, d, g))
-        sd.update(_state_dict({f"{ff}net.2": (d, 4 * d)}, 403, prefix="transformer_blocks.0."))
+        sd.update(_int4_state_(f"transformer_blocks.0.{ff}net.0.proj.", 4 * d, d, g))
+        sd.update(_state_dict_({f"{ff}net.2": (d, 4 * d)}, 403, prefix="transformer_blocks.0."))
         sd[f"transformer_blocks.0.{ff}net.2_input_scale"] = torch.tensor([3.0 / 448])
-    sd.update(_int4_state("single_transformer_blocks.0.attn.to_qkv.", 3 * d, d, g))
-    sd.update(_int4_state("single_transformer_blocks.0.proj_mlp.", 4 * d, d, g))
-    sd.update(_int4_state("single_transformer_blocks.0.proj_out.linears.0.", d, d, g))
-    sd.update(_int4_state("single_transformer_blocks.0.proj_out.linears.1.linear.", d, 4 * d, g, bias=False))
+    sd.update(_int4_state_("single_transformer_blocks.0.attn.to_qkv.", 3 * d, d, g))
+    sd.update(_int4_state_("single_transformer_blocks.0.proj_mlp.", 4 * d, d, g))
+    sd.update(_int4_state_("single_transformer_blocks.0.proj_out.linears.0.", d, d, g))
+    sd.update(_int4_state_("single_transformer_blocks.0.proj_out.linears.1.linear.", d, 4 * d, g, bias=False))
     return sd
 
 
@@ -822,6 +824,72 @@ def test_flux_int4_block_ops(ops, dev, full):
     ns, ms = F.ada_layernorm_int4(xs, temb, ws.norm, 3)
     want = F.flux_single_mlp_int4(xs, ns, score(ws.to_qkv.forward(ns)).contiguous(), ms[2].contiguous(), ws.mlp)
     assert torch.equal(y, want)
+
+
+_INT4_DOUBLE_MUTATIONS = ("swap_scale_shift", "swap_mlp_scale_shift", "swap_gates", "no_second_residual", "swap_qkv_projections",
+                          "swap_out_projections", "swap_feed_forwards", "no_low_rank", "low_rank_from_smoothed", "no_gelu")
+_INT4_SINGLE_MUTATIONS = ("swap_scale_shift", "gate_is_chunk0", "mlp_from_block_input", "linears0_from_norm", "drop_linears1",
+                          "no_low_rank", "low_rank_from_smoothed")
+
+
+def check_int4_blocks_against_the_restatement(make_double, make_single, dev, full):
+    """Shared by the Python op classes (here) and the C++ torch classes (tests/test_gpu_torch_classes.py).
+
+    A 4-bit group quantiser turns a one-ULP difference in its 16-bit input (the attention output of a bf16 softmax against
+    an fp64 one) into code flips worth a seventh of the group maximum, so a correct block sits further from the fp64
+    restatement than the FP8 blocks do: measured 0.05-0.08 relative L2 when the W4A4 main product and its low-rank branch
+    contribute alike (low-rank weights of std 0.1), 0.016-0.019 when the low-rank branch -- 16-bit arithmetic, no flips --
+    dominates (std 0.2).  Both settings run; the nearest mis-wired variant measured 0.34 and 0.28 away."""
+    from oracle import flux_blocks_f64 as FB
+
+    b, s, sc, heads, dh = 2, 96, 32, 4, 64
+    d = heads * dh
+    for lora_scale, e_max, far in ((0.1, 0.10, 0.30), (0.2, 0.03, 0.25)):
+        g = rng_t(441)
+        sd = _int4_block_state(d, dh, g, scale_w=0.06, lora_scale=lora_scale)
+        x = torch.randn(b, s, d, generator=g).bfloat16()
+        ctx = torch.randn(b, sc, d, generator=g).bfloat16()
+        temb = torch.randn(b, d, generator=g).bfloat16()
+        rope = _rope_table(b, sc + s, dh, 443).bfloat16()
+        op = make_double(d, heads, dh)
+        op.reload_model_from_state_dict("transformer_blocks.0.", sd, "cpu")
+        out, cout = op.forward(x.to(dev), ctx.to(dev), rope.to(dev), temb.to(dev))
+        want, cwant = FB.flux_double_block_int4(sd, "transformer_blocks.0.", x, ctx, temb, rope, heads, "bf16", full)
+        e1, e2 = _rel(out.cpu(), want), _rel(cout.cpu(), cwant)
+        print(f"INT4 double block (full={full}, low-rank std {lora_scale}): relative L2 distance to the fp64 restatement "
+              f"{e1:.4f} (image), {e2:.4f} (text)")
+        assert e1 < e_max and e2 < e_max
+        for w in _INT4_DOUBLE_MUTATIONS:
+            bad, cbad = FB.flux_double_block_int4(sd, "transformer_blocks.0.", x, ctx, temb, rope, heads, "bf16", full, wiring=(w,))
+            r1, r2 = _rel(out.cpu(), bad), _rel(cout.cpu(), cbad)
+            assert r1 > far and r2 > far and min(r1, r2) > 3 * max(e1, e2), (w, r1, r2)
+        sop = make_single(d, heads, dh)
+        sop.reload_model_from_state_dict("single_transformer_blocks.0.", sd, "cpu")
+        xs = torch.cat([ctx, x], dim=1).contiguous()
+        y = sop.forward(xs.to(dev), rope.to(dev), temb.to(dev))
+        ywant = FB.flux_single_block_int4(sd, "single_transformer_blocks.0.", xs, temb, rope, heads, "bf16", full)
+        e3 = _rel(y.cpu(), ywant)
+        print(f"INT4 single block (full={full}, low-rank std {lora_scale}): relative L2 distance to the fp64 restatement {e3:.4f}")
+        assert e3 < e_max
+        for w in _INT4_SINGLE_MUTATIONS:
+            r3 = _rel(y.cpu(), FB.flux_single_block_int4(sd, "single_transformer_blocks.0.", xs, temb, rope, heads, "bf16", full, wiring=(w,)))
+            assert r3 > far and r3 > 3 * e3, (w, r3)
+
+
+@pytest.mark.parametrize("level", ["INT4_W4A4_FULL", "INT4_W4A4"])
+def test_flux_int4_block_ops_against_an_independent_fp64_restatement(ops, dev, level):
+    """Both INT4 levels of FluxTransformerBlockOp and FluxSingleTransformerBlockOp against the fp64 restatement of
+    FluxTransformerInt4Block / FluxAttentionInt4Processor / FluxAttnPostInt4Processor / FluxSingleTransformerInt4Block
+    (oracle/flux_blocks_f64.py), which shares nothing with lyradiff_amd/flux_int4.py.  The outputs agree to within the noise of
+    4-bit codes that flip on 16-bit rounding differences; every mis-wired variant of the restatement (a wrong msa chunk, gates
+    or projections or feed-forwards swapped, a dropped residual or projection, the low-rank branch missing or fed from the
+    smoothed input, proj_mlp or proj_out.linears.0 fed from the wrong tensor) is many times further away."""
+    from lyradiff_amd import flux_ops as FO
+
+    lv = FO.LyraQuantLevel[level].value
+    check_int4_blocks_against_the_restatement(lambda d, h, dh: FO.FluxTransformerBlockOp("bf16", d, h, dh, 4, lv),
+                                              lambda d, h, dh: FO.FluxSingleTransformerBlockOp("bf16", d, h, dh, 4, lv),
+                                              dev, level == "INT4_W4A4_FULL")
 
 
 @pytest.mark.parametrize("dt", ["bf16", "f16"])

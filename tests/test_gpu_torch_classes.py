@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from tests.helpers import rng_t
-from tests.test_gpu_flux_blocks import _block_state, _int4_block_state, _rel, _rope_table
+from tests.test_gpu_flux_blocks import _block_state, _int4_block_state, _rel, _rope_table, check_int4_blocks_against_the_restatement
 
 
 @pytest.fixture(scope="module")
@@ -198,6 +198,15 @@ def test_int4_block_classes_equal_the_python_ops(classes, ops, dev, level):
     xs = torch.cat([ctx, x], dim=1).contiguous()
     y = sop.forward(xs, rope, temb)
     assert torch.equal(y, spy.forward(xs, rope, temb)) and torch.isfinite(y.float()).all()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("level", [8, 7])
+def test_int4_block_classes_match_the_fp64_restatement(classes, ops, dev, level):
+    """The C++ classes at both INT4 levels directly against oracle/flux_blocks_f64.py, with its mis-wired variants."""
+    check_int4_blocks_against_the_restatement(lambda d, h, dh: classes.FluxTransformerBlockOp("bf16", d, h, dh, 4, level),
+                                              lambda d, h, dh: classes.FluxSingleTransformerBlockOp("bf16", d, h, dh, 4, level),
+                                              dev, level == 8)
 
 
 @pytest.mark.gpu

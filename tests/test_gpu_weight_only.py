@@ -127,6 +127,52 @@ def test_weight_only_gemm_grouped(ops, dev, dt, bits, with_zeros, group, m, n, k
     assert_close_tol(to_np_f32(y), ref, f"weight-only grouped {kind} {dt} g{group} zeros={with_zeros}", abs_floor=floor)
 
 
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("bits,grouped,group", [(8, 0, 0), (4, 0, 0), (8, 1, 64), (4, 1, 128), (8, 2, 128), (4, 2, 64)])
+@pytest.mark.parametrize("m,n,k", [(4096, 3072, 256), (4000, 3104, 384)])
+def test_weight_only_gemm_256x256_tiles(ops, dev, dt, bits, grouped, group, m, n, k):
+    """The 256x256 eight-wavefront three-stage kernels (picked from 192 such tiles up): per-channel, group-wise scale-only and
+    scale + zero-point forms, int8 and int4, n a multiple of 256 and not, ragged m; against the fp64 contract, and bit for bit
+    against the 256x128 configuration (same k order) forced through the thread tactic."""
+    g = rng_t(m + n + k + bits + group)
+    t = TORCH_DT[dt]
+    kind = "int8" if bits == 8 else "int4"
+    x = torch.randn(m, k, generator=g).to(t)
+    bias = (0.2 * torch.randn(n, generator=g)).to(t)
+    assert ((m + 255) // 256) * ((n + 255) // 256) >= 192
+    if grouped == 0:
+        rng = np.random.default_rng(m + bits)
+        half = 1 << (bits - 1)
+        q = rng.integers(-half, half, (k, n)).astype(np.int8)
+        scales = torch.from_numpy((0.002 + 0.02 * rng.random(n)).astype(np.float32)).to(t)
+        run = lambda wp: ops.weight_only_linear(x.to(dev), wp, scales.to(dev), bias.to(dev), kind)
+        ref = O.weight_only_gemm_f64(to_np_f32(x), q, to_np_f32(scales), to_np_f32(bias), dt)
+        w = np.abs(q.astype(np.float64)) * to_np_f32(scales).astype(np.float64)[None, :]
+    else:
+        q, scales, zeros = _grouped_case(k, n, bits, group, dt, grouped == 2, m + n + k)
+        run = lambda wp: ops.weight_only_linear_grouped(x.to(dev), wp, scales.to(dev), None if zeros is None else zeros.to(dev),
+                                                        bias.to(dev), kind, group)
+        zs = None if zeros is None else to_np_f32(zeros)
+        ref = O.weight_only_gemm_grouped_f64(to_np_f32(x), q, to_np_f32(scales), zs, to_np_f32(bias), group, dt)
+        w = np.abs(O.weight_only_dequant_grouped(q, to_np_f32(scales), zs, group, dt)).astype(np.float64)
+    wp = ops.repack_weight_only(torch.from_numpy(q if bits == 8 else _pack_n(q)).to(dev), kind)
+    y = run(wp)  # built-in rule: 256x256
+    with ops.gemm_thread_tactic(0):
+        y0 = run(wp)
+    with ops.gemm_thread_tactic(1):
+        y1 = run(wp)
+    assert torch.equal(y, y0), "the built-in rule did not pick the 256x256 configuration"
+    assert torch.equal(y0, y1), "256x256 and 256x128 configurations differ"
+    ax = np.abs(to_np_f32(x)).astype(np.float64)
+    floor = 4e-6 * (ax @ w)
+    if dt == "bf16":
+        floor = floor + 2.0 ** -8 * np.abs(ref.astype(np.float64)) + (2.0 ** -7 * ax.max(axis=1)[:, None] * w.max(axis=0)[None, :] if grouped == 2 else 0.0)
+    assert_close_tol(to_np_f32(y), ref, f"weight-only 256x256 {kind} {dt} grouped={grouped} g{group}", abs_floor=floor)
+    with pytest.raises(Exception, match="unknown tile configuration"):
+        with ops.gemm_thread_tactic(5):
+            run(wp)
+
+
 def test_weight_only_grouped_argument_checks(ops, dev):
     from lyradiff_amd.lib import LyraQuantError
 

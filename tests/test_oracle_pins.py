@@ -898,3 +898,110 @@ def test_weight_only_gemm_grouped_reduces_to_the_per_column_form():
     with_z = O.weight_only_gemm_grouped_f64(a, q, np.tile(col, (k // group, 1)), zeros, None, group, "f16")
     w = O.weight_only_dequant_grouped(q, np.tile(col, (k // group, 1)), zeros, group, "f16").astype(np.float64)
     assert np.array_equal(with_z, O.round_to((a.astype(np.float64) @ w).astype(np.float32), "f16"))
+
+
+def _int4_entries(prefix, n, k, g, rank=8, zero_codes=False):
+    """A W4A4 weight container with the reference's key names (W4A4GemmWeight.cc:65-83), random codes."""
+    codes = torch.zeros(n, k, dtype=torch.int16) if zero_codes else torch.randint(-8, 8, (n, k), generator=g, dtype=torch.int16)
+    packed = ((codes[:, 0::2] & 0xF) | ((codes[:, 1::2] & 0xF) << 4)).to(torch.uint8).view(torch.int8)
+    return codes, {prefix + "packed_weight": packed.contiguous(), prefix + "weight_scale": (torch.rand(n, k // 64, generator=g) * 0.02 + 0.01).float(),
+                   prefix + "smooth": (0.5 + torch.rand(k, generator=g)).float(),
+                   prefix + "lora_up": (0.25 * torch.randn(n, rank, generator=g)).bfloat16(),
+                   prefix + "lora_down": (0.25 * torch.randn(rank, k, generator=g)).bfloat16(),
+                   prefix + "bias": (0.5 * torch.randn(n, generator=g)).bfloat16()}
+
+
+def test_int4_block_restatement_parts_and_closed_forms():
+    """oracle/flux_blocks_f64.py, INT4 half.  The nibble order of the weight container against hand-spelled bytes and the
+    pinned word unpacker; the fp64 W4A4 linear against the C twin's pinned fmaf chain on the same codes (main product)
+    and against sums written out term by term (low-rank branch, which must see the RAW input, not the smoothed one); the
+    block wiring against cases that can be worked out by hand (zero codes: a W4A4 linear returns its low-rank product,
+    zero low-rank weights as well: nothing, so every bias, gate and residual can be set independently)."""
+    from oracle import flux_blocks_f64 as FB
+
+    g = torch.Generator().manual_seed(17)
+    # byte 0x8F: element 0 = 0xF = -1 (low nibble), element 1 = 0x8 = -8; byte 0x27: elements 7, 2
+    packed = torch.zeros(1, 32, dtype=torch.uint8)
+    packed[0, 0], packed[0, 1] = 0x8F, 0x27
+    w = FB.unpack_w4a4_weight(packed.view(torch.int8), torch.tensor([[0.5]]))
+    assert w.shape == (1, 64) and w[0, :4].tolist() == [-0.5, -4.0, 3.5, 1.0] and float(w[0, 4:].abs().max()) == 0.0
+    n, k, m, rank = 24, 128, 10, 8
+    codes, sd = _int4_entries("p.", n, k, g, rank)
+    words = sd["p.packed_weight"].view(torch.uint8).numpy().view(np.uint32)  # little-endian: byte j of a word = elements 2j, 2j+1
+    assert np.array_equal(O.unpack_int4(words), codes.numpy().astype(np.int8))
+    wq = FB.unpack_w4a4_weight(sd["p.packed_weight"], sd["p.weight_scale"])
+    assert torch.equal(wq, codes.double() * sd["p.weight_scale"].double().repeat_interleave(64, dim=1))
+    # main product against the pinned fp32 chain of the C twin on the same operands
+    x = torch.randn(m, k, generator=g).bfloat16()
+    y = FB.w4a4_linear(sd, "p.", x, "bf16", wiring=("no_low_rank",))
+    xa, sa = O.w4a4_quant(x.float().numpy(), sd["p.smooth"].numpy())
+    chain = OC.w4a4_gemm(xa, words, sa, sd["p.weight_scale"].numpy())
+    assert np.allclose(y.numpy(), chain, rtol=2e-6, atol=1e-6) and np.abs(chain).max() > 1.0
+    # low-rank branch term by term on sampled outputs: T(sum_k x[m,k] down[r,k]) in T, then times up[n,r], added to the main product
+    full = FB.w4a4_linear(sd, "p.", x, "bf16")
+    for (mi, ni) in ((0, 0), (3, 17), (9, 23)):
+        low = [float(O.round_to(np.full(1, sum(float(x[mi, kk]) * float(sd["p.lora_down"][r, kk]) for kk in range(k)), np.float32), "bf16")[0]) for r in range(rank)]
+        want = float(y[mi, ni]) + sum(low[r] * float(sd["p.lora_up"][ni, r]) for r in range(rank))
+        assert abs(float(full[mi, ni]) - want) < 1e-9 * (1 + abs(want))
+    wrong = FB.w4a4_linear(sd, "p.", x, "bf16", wiring=("low_rank_from_smoothed",))
+    assert float((wrong - full).abs().max()) > 0.05  # the variant that feeds x / smooth into the low-rank branch is visibly different
+
+    # ---- block wiring with zero codes and zero low-rank weights: W4A4 linears return 0, their biases are added by the callers
+    b, s, sc, heads, dh = 2, 6, 3, 2, 32
+    d = heads * dh
+    xs = torch.randn(b, s, d, generator=g).bfloat16()
+    ctx = torch.randn(b, sc, d, generator=g).bfloat16()
+    temb = torch.randn(b, d, generator=g).bfloat16()
+    sd = {}
+    for pre, chunks, adas in (("d.", 6, ("norm1.linear", "norm1_context.linear")), ("s.", 3, ("norm.linear",))):
+        for a in adas:
+            sd[f"{pre}{a}.weight"] = torch.zeros(chunks * d, d).bfloat16()
+            sd[f"{pre}{a}.bias"] = torch.zeros(chunks * d).bfloat16()
+        for nme in ("norm_q", "norm_k", "norm_added_q", "norm_added_k"):
+            sd[f"{pre}attn.{nme}.weight"] = torch.ones(dh).bfloat16()
+    w4 = {"d.attn.to_qkv.": (3 * d, d), "d.attn.to_added_qkv.": (3 * d, d), "d.attn.to_out.0.": (d, d), "d.attn.to_add_out.": (d, d),
+          "d.ff.net.0.proj.": (4 * d, d), "d.ff_context.net.0.proj.": (4 * d, d), "s.attn.to_qkv.": (3 * d, d), "s.proj_mlp.": (4 * d, d),
+          "s.proj_out.linears.0.": (d, d), "s.proj_out.linears.1.linear.": (d, 4 * d)}
+    for pre, (nn, kk) in w4.items():
+        _, e = _int4_entries(pre, nn, kk, g, 8, zero_codes=True)
+        e[pre + "lora_up"].zero_()
+        e[pre + "bias"].zero_()
+        sd.update(e)
+    for ff in ("ff.", "ff_context."):
+        sd[f"d.{ff}net.2.weight"] = torch.zeros(d, 4 * d).bfloat16()
+        sd[f"d.{ff}net.2.weight"][0, 0] = 2.0 ** -100  # an all-zero tensor would have the per-tensor scale 0
+        sd[f"d.{ff}net.2.bias"] = torch.zeros(d).bfloat16()
+        sd[f"d.{ff}net.2_input_scale"] = torch.tensor([0.02])
+    eye = torch.tensor([[1.0, 0.0], [0.0, 1.0]]).expand(b, sc + s, dh // 2, 2, 2)
+    o, c = FB.flux_double_block_int4(sd, "d.", xs, ctx, temb, eye, heads, full=False)
+    assert torch.equal(o, xs.double()) and torch.equal(c, ctx.double())  # every gate is zero
+    # gate_msa = chunk 2 gates to_out.0's output (= its bias here), gate_mlp = chunk 5 gates net.2's output (= its bias)
+    sd["d.norm1.linear.bias"][2 * d:3 * d] = 1.0
+    sd["d.norm1.linear.bias"][5 * d:6 * d] = 2.0
+    sd["d.attn.to_out.0.bias"][:] = 0.5
+    sd["d.ff.net.2.bias"][:] = 0.25
+    o, c = FB.flux_double_block_int4(sd, "d.", xs, ctx, temb, eye, heads, full=False)
+    assert torch.equal(o, FB._round(FB._round(xs.double() + 0.5, "bf16") + 0.5, "bf16")) and torch.equal(c, ctx.double())
+    sd["d.norm1_context.linear.bias"][2 * d:3 * d] = -1.0
+    sd["d.attn.to_add_out.bias"][:] = 0.125
+    o2, c2 = FB.flux_double_block_int4(sd, "d.", xs, ctx, temb, eye, heads, full=False)
+    assert torch.equal(o2, o) and torch.equal(c2, FB._round(ctx.double() - 0.125, "bf16"))
+    # single block: out = x + gate (chunk 2) * ((linears.0 + b0) + linears.1); only linears.0 has a bias
+    xcat = torch.cat([ctx, xs], dim=1)
+    assert torch.equal(FB.flux_single_block_int4(sd, "s.", xcat, temb, eye, heads, full=False), xcat.double())
+    sd["s.norm.linear.bias"][2 * d:3 * d] = 2.0
+    sd["s.proj_out.linears.0.bias"][:] = 0.75
+    y1 = FB.flux_single_block_int4(sd, "s.", xcat, temb, eye, heads, full=False)
+    assert torch.equal(y1, FB._round(xcat.double() + 1.5, "bf16"))
+    # proj_mlp's bias passes through GELU into linears.1, whose low-rank branch (codes stay zero) carries it to the output:
+    # mlp = T(gelu(1)) everywhere, low = T(4d * mlp * 2^-6), h2 = low * 2^-3 * rank  -- exact powers of two around one constant
+    sd["s.proj_mlp.bias"][:] = 1.0
+    sd["s.proj_out.linears.1.linear.lora_down"][:] = 2.0 ** -6
+    sd["s.proj_out.linears.1.linear.lora_up"][:] = 2.0 ** -3
+    mlp = float(FB._round(FB.gelu_tanh(torch.tensor([1.0])), "bf16"))
+    low = float(FB._round(torch.tensor([4 * d * mlp * 2.0 ** -6]), "bf16"))
+    h2 = float(FB._round(torch.tensor([8 * low * 2.0 ** -3]), "bf16"))
+    y2 = FB.flux_single_block_int4(sd, "s.", xcat, temb, eye, heads, full=False)
+    osum = float(FB._round(torch.tensor([0.75 + h2]), "bf16"))
+    assert torch.equal(y2, FB._round(FB._round(torch.tensor([osum * 2.0]), "bf16") + xcat.double(), "bf16"))
+    assert not torch.equal(y2, y1)
