@@ -113,33 +113,44 @@ int lq_fp8_scale_cast(uint8_t* dst, const void* src, lq_dtype_t dtype, const flo
  * those of the two functions above.  Overwrites scale_out (no zero-init needed). */
 int lq_fp8_amax_cast(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t n,
                      lq_stream_t stream);
-/* How lq_fp8_amax_cast runs: normally one launch whose workgroups meet at a grid-wide barrier in statically allocated
- * device memory; each stream owns one of 16 barrier slots per device (work of one stream runs in order), so calls on
- * up to 16 streams may be in flight together.  Under stream capture, on further streams and for unaligned buffers it
- * runs three scratch-free kernels instead (zero the scale, atomic-max pass, cast pass).  The barrier assumes the grid
- * becomes resident; when kernels of OTHER streams hold the device for longer than its bounded wait (~0.1 s), the
- * launch gives up, writes a NaN scale and raises a flag:
- * lq_fp8_amax_cast_status() returns 0 if no such time-out happened on the current device since the last call, 1 if
- * one did (flag cleared; lq_last_error() explains), negative on a HIP error.  It copies 4 bytes from the device and
- * therefore waits for the null stream; call it after synchronising the streams that quantised.  No reference
- * counterpart. */
+/* How lq_fp8_amax_cast runs: normally one launch (one 1024-thread workgroup per CU) whose workgroups exchange their
+ * maxima through statically allocated device memory; each stream owns one of 16 exchange slots per device (work of
+ * one stream runs in order), so calls on up to 16 streams may be in flight together.  Under stream capture, on the
+ * per-thread default stream, on further streams and for unaligned buffers it runs three scratch-free kernels instead
+ * (zero the scale, atomic-max pass, cast pass).  The exchange assumes the grid becomes resident; when kernels of OTHER
+ * streams hold the device for longer than its bounded wait (~0.1 s), the workgroups that gave up cast with a NaN
+ * scale, write NaN to scale_out and raise a flag:
+ * lq_fp8_amax_cast_status() returns 0 if nothing went wrong on the current device since the last call, 1 if a
+ * one-launch quantisation timed out (flag cleared; lq_last_error() explains), 2 if overlapping calls of
+ * lq_fp8_amax_cast_static corrupted its ticket counters (stays until lq_fp8_amax_cast_static_reset), negative on a HIP
+ * error.  It copies 8 bytes from the device and therefore waits for the null stream; call it after synchronising the
+ * streams that quantised.  No reference counterpart. */
 int lq_fp8_amax_cast_status(void);
-/* The barrier slot (0..15) `stream` owns on the current device, assigned on first use; -1 when all 16 are taken (calls
+/* The exchange slot (0..15) `stream` owns on the current device, assigned on first use; -1 when all 16 are taken (calls
  * on that stream then run the scratch-free kernels); negative status on a HIP error.  For diagnostics and tests. */
 int lq_fp8_amax_cast_slot(lq_stream_t stream);
+/* Gives the slot of `stream` back (call it when the stream is destroyed or done quantising, with none of its calls still
+ * running): returns the freed slot, -1 if the stream owned none.  A process that creates and destroys streams without
+ * it runs out of slots after 16 and silently takes the slower three-kernel route. */
+int lq_fp8_amax_cast_release_slot(lq_stream_t stream);
 
 /* lq_fp8_amax_cast for callers that cannot allocate or tolerate a kernel that waits: code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Two launches, no barrier:
  * a partial-maximum pass whose workgroups leave their maxima and a ticket counter in a static device array
- * (119 KiB per GPU, held until the process ends; its address is looked up once per device on first use) -- the
+ * (the static block is 115 KiB per GPU, held until the process ends; its address is looked up once per device on first use) -- the
  * workgroup drawing the last ticket writes scale_out[0] = max|x| / 448 and re-arms the counter -- then the cast pass.
  * Same results as lq_fp8_amax_cast, bit for bit.  Calls no allocating routine.  n from 1 to
  * lq_fp8_amax_cast_static_max_elems() (2^28: 8192 partial maxima of 32768 elements), src and dst 16-byte aligned;
  * anything else is rejected with LQ_ERR_SHAPE / LQ_ERR_ARG.  All calls on one GPU share the one array: calls that
- * overlap in time (different streams, or a graph replay next to eager calls) race -- serialise them. */
+ * overlap in time (different streams, or a graph replay next to eager calls) race -- serialise them.  An overlap can leave
+ * the ticket counters where no later call ever draws the last ticket (scale_out then stays unwritten while the call
+ * returns LQ_OK): a ticket that one launch alone cannot issue raises a flag that lq_fp8_amax_cast_status() reports as 2,
+ * and lq_fp8_amax_cast_static_reset (one tiny launch on `stream`, allocates nothing) puts counters and flag back to
+ * zero -- run it once the overlapping calls have finished. */
 int lq_fp8_amax_cast_static(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t n,
                             lq_stream_t stream);
 size_t lq_fp8_amax_cast_static_max_elems(void);
+int lq_fp8_amax_cast_static_reset(lq_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * W4A4 group-wise INT4 activation quantisation

@@ -33,16 +33,27 @@ def sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith((".hip", ".cpp")))
 
 
-def _deps_mtime():
-    hdrs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
-    hdrs.append(os.path.join(ROOT, "include", "lyraquant.h"))
-    return max(os.path.getmtime(h) for h in hdrs)
+def _deps_mtime(path: str, seen=None) -> float:
+    """Newest modification time among `path` and the project headers it includes, directly or not."""
+    seen = set() if seen is None else seen
+    if path in seen or not os.path.exists(path):
+        return 0.0
+    seen.add(path)
+    newest = os.path.getmtime(path)
+    with open(path, errors="replace") as f:
+        for line in f:
+            line = line.strip()
+            if line.startswith("#include \""):
+                name = line.split('"')[1]
+                for d in (os.path.dirname(path), CSRC, os.path.join(ROOT, "include")):
+                    newest = max(newest, _deps_mtime(os.path.join(d, name), seen))
+    return newest
 
 
 def _compile(src: str, force: bool) -> str:
     obj = os.path.join(OBJ, src + ".o")
     path = os.path.join(CSRC, src)
-    if not force and os.path.exists(obj) and os.path.getmtime(obj) >= max(os.path.getmtime(path), _deps_mtime()):
+    if not force and os.path.exists(obj) and os.path.getmtime(obj) >= _deps_mtime(path):
         return obj
     cmd = [HIPCC, *FLAGS, "-c", path, "-o", obj]
     if src.endswith(".cpp"):

@@ -181,8 +181,8 @@ __global__ void fill_f32_kernel(float* p, float v) { p[0] = v; }
 // the two-launch kernel pair.  Static device memory starts zeroed, and every user leaves its counters at zero again.
 // Host code never uses the array's name as an address: device_scratch() asks the runtime for the device address once
 // per device (hipGetSymbolAddress) and the kernels receive that pointer as an argument.
-constexpr int kCoopThreads = 512;
-constexpr int kCoopMaxBlocks = 1024;
+constexpr int kCoopThreads = 1024;
+constexpr int kCoopMaxBlocks = 512;
 constexpr int kCoopSlots = 16;
 constexpr size_t kTicketSlab = 32768;     // elements per workgroup of the partial-maximum pass
 constexpr size_t kTicketMaxSlabs = 8192;  // partial maxima the scratch holds => at most 2^28 elements per call
@@ -191,11 +191,15 @@ struct CounterLine {  // one counter per 128-byte line: polls of one word must n
     unsigned count;
     unsigned pad[31];
 };
+struct TaggedLine {  // one {launch number, float bits} word per 128-byte line
+    unsigned long long word;
+    unsigned long long pad[15];
+};
+// Barrier state of the one-launch quantiser.  Nothing in it is a counter: every word is {launch number << 32 | float bits},
+// written whole by one 8-byte store, so a launch that gives up leaves nothing behind that a later launch could trip over.
 struct CoopSlot {
-    CounterLine group[8];
-    CounterLine top;
-    CounterLine flag;
-    float partials[kCoopMaxBlocks];
+    unsigned long long partial[kCoopMaxBlocks];  // workgroup maxima of the launch named in the upper half
+    TaggedLine result[8];                         // the tensor maximum, one copy per group of pollers (workgroup id mod 8)
 };
 struct TicketRegion {
     CounterLine group[kTicketGroups];
@@ -203,8 +207,9 @@ struct TicketRegion {
     float partials[kTicketMaxSlabs];
 };
 struct FusedScratch {
-    unsigned timeout;
-    unsigned pad[63];
+    unsigned timeout;         // a one-launch quantisation gave up at its exchange
+    unsigned ticket_overlap;  // the two-launch quantiser drew a ticket that only overlapping calls can produce
+    unsigned pad[62];
     CoopSlot coop[kCoopSlots];
     TicketRegion ticket;
 };
@@ -240,185 +245,218 @@ static FusedScratch* device_scratch(int* dev_out = nullptr) {
     return p;
 }
 
-// A stream owns one barrier slot for the life of the process (work of one stream runs in order, so its launches never
-// overlap); streams beyond kCoopSlots get none and use the scratch-free kernel sequence.
+// A stream owns one barrier slot from its first call until lq_fp8_amax_cast_release_slot (work of one stream runs in
+// order, so its launches never overlap); streams beyond kCoopSlots get none and use the scratch-free kernel sequence.
+// Every launch on a slot carries the slot's next launch number (never 0, the value of untouched memory).
 struct StreamSlots {
     hipStream_t stream[kCoopSlots];
-    int used = 0;
+    bool taken[kCoopSlots];
+    unsigned launches[kCoopSlots];
 };
 static StreamSlots g_stream_slots[kMaxDevices];
 static std::mutex g_slot_mutex;
-static int slot_for_stream(int dev, hipStream_t st) {
+static int slot_for_stream(int dev, hipStream_t st, unsigned* launch_number = nullptr) {
     std::lock_guard<std::mutex> lock(g_slot_mutex);
     StreamSlots& t = g_stream_slots[dev];
-    for (int i = 0; i < t.used; ++i)
-        if (t.stream[i] == st) return i;
-    if (t.used == kCoopSlots) return -1;
-    t.stream[t.used] = st;
-    return t.used++;
+    int slot = -1;
+    for (int i = 0; i < kCoopSlots && slot < 0; ++i)
+        if (t.taken[i] && t.stream[i] == st) slot = i;
+    for (int i = 0; i < kCoopSlots && slot < 0; ++i)
+        if (!t.taken[i]) {
+            t.taken[i] = true;
+            t.stream[i] = st;
+            slot = i;
+        }
+    if (slot >= 0 && launch_number) {
+        if (++t.launches[slot] == 0) ++t.launches[slot];
+        *launch_number = t.launches[slot];
+    }
+    return slot;
+}
+static int release_slot(int dev, hipStream_t st) {
+    std::lock_guard<std::mutex> lock(g_slot_mutex);
+    StreamSlots& t = g_stream_slots[dev];
+    for (int i = 0; i < kCoopSlots; ++i)
+        if (t.taken[i] && t.stream[i] == st) {
+            t.taken[i] = false;  // the launch counter stays: a later owner continues the numbering
+            return i;
+        }
+    return -1;
 }
 
-// Fused dynamic per-tensor quantisation in ONE launch: every thread keeps up to KEEP 16-element
-// chunks of its slice in registers while the tensor-wide absmax is formed (workgroup partials ->
-// grid-wide barrier -> every workgroup reduces the partials), then casts from registers, so the
-// source is read from HBM once (3 bytes moved per element: the algorithmic minimum).  Chunks
-// beyond KEEP are re-read in the second phase (from L2 / Infinity Cache when they fit).
+// Fused dynamic per-tensor quantisation in ONE launch: every thread keeps up to KEEP 32-byte chunks of the tensor in
+// registers while the tensor-wide absmax is formed (workgroup maxima -> grid-wide exchange), then casts from
+// registers, so the source is read from HBM once (3 bytes moved per element: the algorithmic minimum).  Chunks beyond
+// KEEP are re-read in the second phase (from L2 / Infinity Cache when they fit).
 //
-// The grid never exceeds what the device holds at once (CUs x resident workgroups), so every workgroup is running when
-// the barrier is reached -- provided nothing else occupies the device; when another stream's kernels hold CUs the
-// late workgroups start once those retire, and the wait is bounded so that even a starved grid terminates: on
-// time-out the kernel raises the time-out flag (lq_fp8_amax_cast_status reports it) and the scale it writes is NaN,
-// which poisons the output visibly instead of hanging the device.  The barrier re-arms itself.  Launches that may
-// overlap in time use different slots: a slot belongs to one stream, and the path is not taken under stream capture
-// (a captured launch could later replay on any stream).
-
-// Two-level arrive counter (workgroup ids congruent modulo 8 share a counter, so at most G/8 atomics
-// hit one address; the last arriver of a group bumps the top counter, the last group flips the flag
-// everybody polls).  Counters are cleared by their last arriver.  Only relaxed device-scope atomics are used for the
-// hand-over -- no release/acquire fences, which on this multi-die part would write back / invalidate whole L2s.  The
-// partial maximum is published with a device-scope atomic store and the thread then waits explicitly (s_waitcnt vmcnt(0):
-// on this architecture stores count in vmcnt) for its acknowledgement before the arrival is counted.
-// Returns false on time-out.
-__device__ __forceinline__ bool grid_barrier(CoopSlot* slot, unsigned* timeout, float partial) {
-    __shared__ int ok;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const unsigned G = gridDim.x, grp = blockIdx.x & 7;
-        const unsigned in_group = (G - grp + 7) / 8, ngroups = G < 8 ? G : 8;
-        const unsigned f0 = __hip_atomic_load(&slot->flag.count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&slot->partials[blockIdx.x], partial, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the device-scope (write-through) store has been acknowledged
-        unsigned x = __hip_atomic_fetch_add(&slot->group[grp].count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (x == in_group - 1) {
-            __hip_atomic_store(&slot->group[grp].count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            unsigned t = __hip_atomic_fetch_add(&slot->top.count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (t == ngroups - 1) {
-                __hip_atomic_store(&slot->top.count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // counters are zero again before anyone is released
-                __hip_atomic_store(&slot->flag.count, f0 + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-        }
-        int good = 0;
-        for (int spin = 0; spin < (1 << 18); ++spin) {
-            if (__hip_atomic_load(&slot->flag.count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != f0) {
-                good = 1;
-                break;
-            }
-            __builtin_amdgcn_s_sleep(1);
-        }
-        if (!good) __hip_atomic_store(timeout, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        ok = good;
+// Layout: a wavefront owns 2 KiB blocks of the source; lane l holds the 16-byte pieces at l*16 and 1024 + l*16 of a
+// block (fully coalesced 1 KiB requests) and writes their codes at the matching output offsets.  Which element a lane
+// holds is free: the maximum is a reduction and the cast elementwise.  Kept pieces are fetched with nontemporal loads and
+// the codes leave with nontemporal stores: measured at 4608x3072 bf16 from HBM, in-kernel time stamps, one 1024-thread
+// workgroup per CU: load phase 7.5 -> 6.3 us with the loads marked, and 12.8 -> 11.1 us from launch to launch with the
+// stores marked as well (the 14 MB of codes no longer sit dirty in the L2s for the end-of-kernel write-back).
+//
+// Exchange: thread 0 of every workgroup stores {launch number, workgroup maximum} as one 8-byte word; workgroup 0
+// gathers the words of this launch (one per thread), reduces them and publishes {launch number, tensor maximum} in
+// eight copies; the other workgroups poll the copy of their group (workgroup id mod 8) -- 32 pollers per word.  No
+// read-modify-write, no counter to re-arm, two stores and two polls on the critical path (1.5 us against 2.2 us for a
+// two-level arrival counter with a flag), and every workgroup receives the maximum itself instead of re-reading all
+// partial maxima.  Only relaxed device-scope accesses are used -- no release/acquire fences, which on this multi-die part
+// would write back / invalidate whole L2s; a word is complete by construction.
+//
+// The grid never exceeds what the device holds at once (one workgroup per CU), so every workgroup is running when the
+// exchange starts -- provided nothing else occupies the device; when another stream's kernels hold CUs the late
+// workgroups start once those retire, and every wait is bounded so that even a starved grid terminates: a workgroup that
+// gives up raises the time-out flag (lq_fp8_amax_cast_status reports it), casts with a NaN scale and writes NaN to
+// scale_out, which poisons the output visibly instead of hanging the device.  Launches that may overlap in time use
+// different slots: a slot belongs to one stream, and the path is not taken under stream capture (a captured launch
+// could later replay on any stream) nor for the per-thread default stream (one handle, many streams).
+__device__ __forceinline__ unsigned long long poll_tagged(const unsigned long long* word, unsigned launch, bool* ok) {
+    unsigned long long v = 0;
+    int spin = 0;
+    for (; spin < (1 << 18); ++spin) {
+        v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((unsigned)(v >> 32) == launch) break;
+        __builtin_amdgcn_s_sleep(1);
     }
-    __syncthreads();
-    return ok != 0;
+    *ok = spin < (1 << 18);
+    return v;
 }
 
 template <typename Tag, int KEEP>
-__global__ __launch_bounds__(kCoopThreads, (KEEP > 8 ? 4 : 1)) void fp8_amax_cast_coop_kernel(uint8_t* __restrict__ dst,
-                                                                          float* __restrict__ scale_out,
-                                                                          const void* __restrict__ src, size_t n,
-                                                                          CoopSlot* slot, unsigned* timeout) {
-    constexpr int E = Chunk16<Tag>::elems;
-    constexpr int V = 2;  // uint4 vectors per chunk (32 bytes for every element type)
-    const size_t nchunks = n / E;
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    uint4 keep[KEEP][V];
+__global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_t* __restrict__ dst, float* __restrict__ scale_out,
+                                                                          const void* __restrict__ src, size_t n, CoopSlot* slot,
+                                                                          unsigned launch, unsigned* timeout) {
+    constexpr int E2 = Elem<Tag>::bytes == 2 ? 8 : 4;  // elements per 16-byte piece
+    constexpr int BLK = 128 * E2;                      // elements per 2 KiB block
+    typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+    typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+    const size_t nblocks = n / BLK;
+    const int lane = threadIdx.x & 63;
+    const size_t wave = ((size_t)blockIdx.x * kCoopThreads + threadIdx.x) >> 6;
+    const size_t nwaves = (size_t)gridDim.x * (kCoopThreads / 64);
+    const char* in = static_cast<const char*>(src) + lane * 16;
+    uint4 keep[KEEP][2];
     float amax = 0.0f;
-    auto chunk_amax = [&](const uint4* v) {
-        float f[16];
-        if constexpr (Elem<Tag>::bytes == 2) { unpack8<Tag>(v[0], f); unpack8<Tag>(v[1], f + 8); }
-        else { f[0] = __uint_as_float(v[0].x); f[1] = __uint_as_float(v[0].y); f[2] = __uint_as_float(v[0].z); f[3] = __uint_as_float(v[0].w);
-               f[4] = __uint_as_float(v[1].x); f[5] = __uint_as_float(v[1].y); f[6] = __uint_as_float(v[1].z); f[7] = __uint_as_float(v[1].w); }
+    auto piece_amax = [&](const uint4& v) {
+        float f[8];
+        if constexpr (E2 == 8) unpack8<Tag>(v, f);
+        else { f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y); f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w); }
 #pragma unroll
-        for (int i = 0; i < E; ++i) amax = fmaxf(amax, fabsf(f[i]));
+        for (int i = 0; i < E2; ++i) amax = fmaxf(amax, fabsf(f[i]));
     };
 #pragma unroll
     for (int it = 0; it < KEEP; ++it) {
-        size_t c = first + it * stride;
+        const size_t b = wave + it * nwaves;
         keep[it][0] = make_uint4(0, 0, 0, 0);
         keep[it][1] = make_uint4(0, 0, 0, 0);
-        if (c < nchunks) {
-            const uint4* p = reinterpret_cast<const uint4*>(static_cast<const char*>(src) + c * 32);
-            keep[it][0] = p[0];
-            keep[it][1] = p[1];
+        if (b < nblocks) {
+            const u32x4_t a = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(in + b * 2048));
+            const u32x4_t c = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(in + b * 2048 + 1024));
+            keep[it][0] = make_uint4(a.x, a.y, a.z, a.w);
+            keep[it][1] = make_uint4(c.x, c.y, c.z, c.w);
         }
     }
 #pragma unroll
-    for (int it = 0; it < KEEP; ++it) chunk_amax(keep[it]);
-    for (size_t c = first + KEEP * stride; c < nchunks; c += stride) {
-        const uint4* p = reinterpret_cast<const uint4*>(static_cast<const char*>(src) + c * 32);
-        uint4 v[2] = {p[0], p[1]};
-        chunk_amax(v);
+    for (int it = 0; it < KEEP; ++it) {
+        piece_amax(keep[it][0]);
+        piece_amax(keep[it][1]);
     }
-    if (blockIdx.x == 0) {
-        size_t i = nchunks * E + threadIdx.x;
-        if (i < n) amax = fmaxf(amax, fabsf(load_one<Tag>(src, i)));
+    for (size_t b = wave + KEEP * nwaves; b < nblocks; b += nwaves) {  // what the registers cannot hold is read twice
+        piece_amax(*reinterpret_cast<const uint4*>(in + b * 2048));
+        piece_amax(*reinterpret_cast<const uint4*>(in + b * 2048 + 1024));
     }
+    if (blockIdx.x == 0)  // fewer than BLK trailing elements
+        for (size_t i = nblocks * BLK + threadIdx.x; i < n; i += kCoopThreads) amax = fmaxf(amax, fabsf(load_one<Tag>(src, i)));
     __shared__ float red[kCoopThreads / 64];
+    __shared__ float tensor_max;
     amax = wave_max(amax);
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+    if (lane == 0) red[threadIdx.x >> 6] = amax;
     __syncthreads();
-    float wg_max = 0.0f;
     if (threadIdx.x == 0) {
+        float wg_max = 0.0f;
 #pragma unroll
         for (int i = 0; i < kCoopThreads / 64; ++i) wg_max = fmaxf(wg_max, red[i]);
+        __hip_atomic_store(&slot->partial[blockIdx.x], ((unsigned long long)launch << 32) | __float_as_uint(wg_max), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
     }
-    const bool arrived = grid_barrier(slot, timeout, wg_max);
-    // Only the raw 16-byte vectors live across the barrier: the empty asm makes them new values to the compiler, which
+    bool ok = true;
+    if (blockIdx.x == 0) {
+        float m = 0.0f;
+        for (unsigned i = threadIdx.x; i < gridDim.x; i += kCoopThreads) {
+            bool got;
+            m = fmaxf(m, __uint_as_float((unsigned)poll_tagged(&slot->partial[i], launch, &got)));
+            ok = ok && got;
+        }
+        m = wave_max(__syncthreads_and(ok) ? m : __builtin_nanf(""));  // a missing partial maximum makes the result NaN for everybody
+        __syncthreads();
+        if (lane == 0) red[threadIdx.x >> 6] = m;
+        __syncthreads();
+        m = red[0];
+#pragma unroll
+        for (int i = 1; i < kCoopThreads / 64; ++i) m = (m != m || red[i] != red[i]) ? __builtin_nanf("") : fmaxf(m, red[i]);
+        if (threadIdx.x < 8)
+            __hip_atomic_store(&slot->result[threadIdx.x].word, ((unsigned long long)launch << 32) | __float_as_uint(m), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        if (threadIdx.x == 0) tensor_max = m;
+    } else if (threadIdx.x == 0) {
+        const unsigned long long v = poll_tagged(&slot->result[blockIdx.x & 7].word, launch, &ok);
+        tensor_max = ok ? __uint_as_float((unsigned)v) : __builtin_nanf("");
+    }
+    __syncthreads();
+    const float s = tensor_max / 448.0f;  // NaN after a time-out
+    if (threadIdx.x == 0 && s != s) {
+        __hip_atomic_store(timeout, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        scale_out[0] = s;  // long after workgroup 0 wrote its value, if it had one
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) scale_out[0] = s;
+    // Only the raw 16-byte vectors live across the exchange: the empty asm makes them new values to the compiler, which
     // would otherwise keep the unpacked fp32 copies of the first phase as well (twice the registers, half the occupancy).
 #pragma unroll
     for (int it = 0; it < KEEP; ++it)
 #pragma unroll
-        for (int u = 0; u < V; ++u)
+        for (int u = 0; u < 2; ++u)
             asm volatile("" : "+v"(keep[it][u].x), "+v"(keep[it][u].y), "+v"(keep[it][u].z), "+v"(keep[it][u].w));
-    float m = 0.0f;
-    for (int i = threadIdx.x; i < (int)gridDim.x; i += kCoopThreads)
-        m = fmaxf(m, __hip_atomic_load(&slot->partials[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-    m = wave_max(m);
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
-    __syncthreads();
-    m = 0.0f;
-#pragma unroll
-    for (int i = 0; i < kCoopThreads / 64; ++i) m = fmaxf(m, red[i]);
-    const float s = arrived ? m / 448.0f : __builtin_nanf("");
-    if (blockIdx.x == 0 && threadIdx.x == 0) scale_out[0] = s;
     const float r = 1.0f / s;
-    auto chunk_cast = [&](const uint4* v, size_t c) {
-        float f[16];
-        if constexpr (Elem<Tag>::bytes == 2) { unpack8<Tag>(v[0], f); unpack8<Tag>(v[1], f + 8); }
-        else { f[0] = __uint_as_float(v[0].x); f[1] = __uint_as_float(v[0].y); f[2] = __uint_as_float(v[0].z); f[3] = __uint_as_float(v[0].w);
-               f[4] = __uint_as_float(v[1].x); f[5] = __uint_as_float(v[1].y); f[6] = __uint_as_float(v[1].z); f[7] = __uint_as_float(v[1].w); }
-        u32 w[4];
-#pragma unroll
-        for (int i = 0; i < E / 4; ++i) w[i] = cvt4_e4m3(f[4 * i] * r, f[4 * i + 1] * r, f[4 * i + 2] * r, f[4 * i + 3] * r);
-        if constexpr (E == 16) *reinterpret_cast<uint4*>(dst + c * 16) = make_uint4(w[0], w[1], w[2], w[3]);
-        else *reinterpret_cast<uint2*>(dst + c * 8) = make_uint2(w[0], w[1]);
+    uint8_t* out = dst + lane * E2;
+    auto piece_cast = [&](const uint4& v, uint8_t* o, bool stream_out) {
+        float f[8];
+        if constexpr (E2 == 8) unpack8<Tag>(v, f);
+        else { f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y); f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w); }
+        const u32 w0 = cvt4_e4m3(f[0] * r, f[1] * r, f[2] * r, f[3] * r);
+        if constexpr (E2 == 8) {
+            const u32x2_t w = {w0, cvt4_e4m3(f[4] * r, f[5] * r, f[6] * r, f[7] * r)};
+            if (stream_out) __builtin_nontemporal_store(w, reinterpret_cast<u32x2_t*>(o));
+            else *reinterpret_cast<u32x2_t*>(o) = w;
+        } else {
+            if (stream_out) __builtin_nontemporal_store(w0, reinterpret_cast<u32*>(o));
+            else *reinterpret_cast<u32*>(o) = w0;
+        }
     };
 #pragma unroll
     for (int it = 0; it < KEEP; ++it) {
-        size_t c = first + it * stride;
-        if (c < nchunks) chunk_cast(keep[it], c);
+        const size_t b = wave + it * nwaves;
+        if (b < nblocks) {
+            piece_cast(keep[it][0], out + b * BLK, true);
+            piece_cast(keep[it][1], out + b * BLK + 64 * E2, true);
+        }
     }
-    for (size_t c = first + KEEP * stride; c < nchunks; c += stride) {
-        const uint4* p = reinterpret_cast<const uint4*>(static_cast<const char*>(src) + c * 32);
-        uint4 v[2] = {p[0], p[1]};
-        chunk_cast(v, c);
+    for (size_t b = wave + KEEP * nwaves; b < nblocks; b += nwaves) {
+        piece_cast(*reinterpret_cast<const uint4*>(in + b * 2048), out + b * BLK, true);
+        piece_cast(*reinterpret_cast<const uint4*>(in + b * 2048 + 1024), out + b * BLK + 64 * E2, true);
     }
-    if (blockIdx.x == 0) {
-        size_t i = nchunks * E + threadIdx.x;
-        if (i < n) dst[i] = (uint8_t)cvt1_e4m3(load_one<Tag>(src, i) * r);
-    }
+    if (blockIdx.x == 0)
+        for (size_t i = nblocks * BLK + threadIdx.x; i < n; i += kCoopThreads) dst[i] = (uint8_t)cvt1_e4m3(load_one<Tag>(src, i) * r);
 }
 
 // Returns LQ_OK when the fused launch was issued, 1 when the caller should fall back to the scratch-free
-// kernel sequence (unaligned buffers, stream capture, no barrier slot left for this stream, occupancy query failed),
-// a negative status on an error.
-// KEEP = 8 chunks of 32 bytes (64 registers) stay in each thread's registers across the barrier: with two workgroups
-// per CU that holds a tensor of up to 33.5 M sixteen-bit elements on 256 CUs; the rest of a larger one is read twice.
+// kernel sequence (unaligned buffers, stream capture, per-thread default stream, no barrier slot left for this stream,
+// occupancy query failed), a negative status on an error.
+// One 1024-thread workgroup per CU keeps KEEP = 4, 8 or 10 chunks of 32 bytes per thread across the exchange: 16.7, 33.5 or
+// 41.9 M sixteen-bit elements on 256 CUs; the rest of a larger tensor is read twice (10 chunks are 80 of the 128 registers a
+// lane has at this occupancy, 6-8 more spill; 12 chunks spilled 60).
 template <typename Tag, int KEEP> struct CoopCapacity {
-    int blocks_per_cu = 0, num_cu = 0;
+    int num_cu = 0;
     static const CoopCapacity& get(int dev) {  // queried once (thread-safe initialisation of a function-local static)
         static const CoopCapacity cap = [dev] {
             CoopCapacity c;
@@ -426,10 +464,8 @@ template <typename Tag, int KEEP> struct CoopCapacity {
             hipDeviceProp_t prop;
             if (hipGetDeviceProperties(&prop, dev) == hipSuccess &&
                 hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, fp8_amax_cast_coop_kernel<Tag, KEEP>, kCoopThreads, 0) == hipSuccess &&
-                occ >= 1) {
-                c.blocks_per_cu = occ > 2 ? 2 : occ;
+                occ >= 1)
                 c.num_cu = prop.multiProcessorCount;
-            }
             (void)hipGetLastError();
             return c;
         }();
@@ -437,9 +473,27 @@ template <typename Tag, int KEEP> struct CoopCapacity {
     }
 };
 
+template <typename Tag, int KEEP>
+static int launch_coop_keep(uint8_t* dst, float* scale_out, const void* src, size_t n, hipStream_t st, int dev, FusedScratch* ws,
+                            size_t waves_needed) {
+    const int num_cu = CoopCapacity<Tag, KEEP>::get(dev).num_cu;
+    if (num_cu == 0) return 1;
+    unsigned launch = 0;
+    const int slot = slot_for_stream(dev, st, &launch);
+    if (slot < 0) return 1;
+    size_t grid = (waves_needed + kCoopThreads / 64 - 1) / (kCoopThreads / 64);
+    if (grid > (size_t)num_cu) grid = num_cu;
+    if (grid > kCoopMaxBlocks) grid = kCoopMaxBlocks;
+    if (grid == 0) grid = 1;
+    hipLaunchKernelGGL((fp8_amax_cast_coop_kernel<Tag, KEEP>), dim3((unsigned)grid), dim3(kCoopThreads), 0, st, dst, scale_out, src, n,
+                       &ws->coop[slot], launch, &ws->timeout);
+    return check_launch("fp8_amax_cast_fused");
+}
+
 template <typename Tag>
 static int launch_amax_cast_coop(uint8_t* dst, float* scale_out, const void* src, size_t n, hipStream_t st) {
     if (reinterpret_cast<uintptr_t>(src) % 16 != 0 || reinterpret_cast<uintptr_t>(dst) % 16 != 0) return 1;
+    if (st == hipStreamPerThread) return 1;  // one handle for every thread's own stream: its launches can overlap
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
         (void)hipGetLastError();
@@ -448,33 +502,14 @@ static int launch_amax_cast_coop(uint8_t* dst, float* scale_out, const void* src
     int dev = 0;
     FusedScratch* ws = device_scratch(&dev);
     if (ws == nullptr) return LQ_ERR_HIP;
-    const int slot = slot_for_stream(dev, st);
-    if (slot < 0) return 1;
-    const CoopCapacity<Tag, 8>& cap = CoopCapacity<Tag, 8>::get(dev);
-    const int blocks_per_cu = cap.blocks_per_cu, num_cu = cap.num_cu;
-    if (blocks_per_cu == 0) return 1;
-    // One workgroup per CU while the tensor fits in their registers (fewer parties at the barrier: 15.4 us against 17.0
-    // at 4608x3072), two for a larger one (more of it stays in registers: 39.6 us against 46.3 at 4608x12288).
-    size_t need = (n / Chunk16<Tag>::elems + kCoopThreads - 1) / kCoopThreads;
-    // A tensor that two workgroups per CU cannot hold with 8 chunks per thread (more than 33.5 M sixteen-bit elements)
-    // takes the form with 10 chunks, 80 of the 128 registers a lane may use at that occupancy (12 spill): 42 M elements stay in
-    // registers and less of the tensor is read twice.
-    if (need > (size_t)8 * 2 * num_cu) {
-        const CoopCapacity<Tag, 10>& cap12 = CoopCapacity<Tag, 10>::get(dev);
-        if (cap12.blocks_per_cu == 2) {
-            int grid = 2 * num_cu;
-            if (grid > kCoopMaxBlocks) grid = kCoopMaxBlocks;
-            hipLaunchKernelGGL((fp8_amax_cast_coop_kernel<Tag, 10>), dim3(grid), dim3(kCoopThreads), 0, st, dst, scale_out, src, n,
-                               &ws->coop[slot], &ws->timeout);
-            return check_launch("fp8_amax_cast_fused");
-        }
-    }
-    int grid = (need <= (size_t)8 * num_cu ? 1 : blocks_per_cu) * num_cu;
-    if (grid > kCoopMaxBlocks) grid = kCoopMaxBlocks;
-    if ((size_t)grid > need) grid = need ? (int)need : 1;
-    hipLaunchKernelGGL((fp8_amax_cast_coop_kernel<Tag, 8>), dim3(grid), dim3(kCoopThreads), 0, st, dst, scale_out, src, n,
-                       &ws->coop[slot], &ws->timeout);
-    return check_launch("fp8_amax_cast_fused");
+    const size_t blocks = n / (Elem<Tag>::bytes == 2 ? 1024 : 512);  // 2 KiB blocks, one per wavefront and kept chunk
+    const int num_cu = CoopCapacity<Tag, 4>::get(dev).num_cu;
+    if (num_cu == 0) return 1;
+    const size_t waves = (size_t)num_cu * (kCoopThreads / 64);
+    const size_t per_wave = (blocks + waves - 1) / waves;
+    if (per_wave <= 4) return launch_coop_keep<Tag, 4>(dst, scale_out, src, n, st, dev, ws, blocks);
+    if (per_wave <= 8) return launch_coop_keep<Tag, 8>(dst, scale_out, src, n, st, dev, ws, blocks);
+    return launch_coop_keep<Tag, 10>(dst, scale_out, src, n, st, dev, ws, blocks);
 }
 
 // ---- two launches, no barrier: partial maxima + ticket, then the cast ------------------------------------------------
@@ -485,7 +520,7 @@ static int launch_amax_cast_coop(uint8_t* dst, float* scale_out, const void* src
 // it fits).  All calls on one device share the one scratch block: calls that overlap in time race.
 template <typename Tag>
 __global__ __launch_bounds__(256) void fp8_amax_ticket_kernel(TicketRegion* __restrict__ ws, float* __restrict__ scale_out,
-                                                              const void* __restrict__ x, size_t n) {
+                                                              const void* __restrict__ x, size_t n, unsigned* __restrict__ overlap) {
     constexpr int E = Chunk16<Tag>::elems;
     constexpr int PER_THREAD = (int)(kTicketSlab / E / 256);  // chunks per thread: all requested before the first is used
     const size_t nchunks = n / E;
@@ -530,9 +565,16 @@ __global__ __launch_bounds__(256) void fp8_amax_ticket_kernel(TicketRegion* __re
         const unsigned G = gridDim.x, grp = blockIdx.x % kTicketGroups;
         const unsigned in_group = (G - grp + kTicketGroups - 1) / kTicketGroups, ngroups = G < kTicketGroups ? G : kTicketGroups;
         int is_last = 0;
-        if (__hip_atomic_fetch_add(&ws->group[grp].count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == in_group - 1) {
+        const unsigned drawn = __hip_atomic_fetch_add(&ws->group[grp].count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (drawn == in_group - 1) {
             __hip_atomic_store(&ws->group[grp].count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            is_last = __hip_atomic_fetch_add(&ws->top.count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ngroups - 1;
+            const unsigned top = __hip_atomic_fetch_add(&ws->top.count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            is_last = top == ngroups - 1;
+            if (top >= ngroups) __hip_atomic_store(overlap, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else if (drawn >= in_group) {
+            // a ticket this launch cannot have issued: another call's workgroups drew from the same counters (calls that
+            // overlap on one GPU); the counters are unusable until lq_fp8_amax_cast_static_reset puts them back to zero
+            __hip_atomic_store(overlap, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         last = is_last;
     }
@@ -585,10 +627,10 @@ static int launch_cast(uint8_t* dst, const void* src, const float* scale, int in
 
 // Partial-maximum pass of the two-launch quantiser on the scratch block `ws` (16-byte aligned x).
 template <typename Tag>
-static int launch_amax_ticket(TicketRegion* ws, float* scale_out, const void* x, size_t n, hipStream_t st) {
+static int launch_amax_ticket(TicketRegion* ws, unsigned* overlap, float* scale_out, const void* x, size_t n, hipStream_t st) {
     size_t slabs = (n + kTicketSlab - 1) / kTicketSlab;
     if (slabs == 0) slabs = 1;
-    hipLaunchKernelGGL((fp8_amax_ticket_kernel<Tag>), dim3((unsigned)slabs), dim3(256), 0, st, ws, scale_out, x, n);
+    hipLaunchKernelGGL((fp8_amax_ticket_kernel<Tag>), dim3((unsigned)slabs), dim3(256), 0, st, ws, scale_out, x, n, overlap);
     return check_launch("fp8_amax_ticket");
 }
 
@@ -674,9 +716,9 @@ extern "C" int lq_fp8_amax_cast_static(uint8_t* dst, float* scale_out, const voi
     hipStream_t st = as_stream(stream);
     int rc;
     switch (dtype) {
-        case LQ_F16: rc = launch_amax_ticket<F16Tag>(&ws->ticket, scale_out, src, n, st); break;
-        case LQ_BF16: rc = launch_amax_ticket<BF16Tag>(&ws->ticket, scale_out, src, n, st); break;
-        default: rc = launch_amax_ticket<F32Tag>(&ws->ticket, scale_out, src, n, st); break;
+        case LQ_F16: rc = launch_amax_ticket<F16Tag>(&ws->ticket, &ws->ticket_overlap, scale_out, src, n, st); break;
+        case LQ_BF16: rc = launch_amax_ticket<BF16Tag>(&ws->ticket, &ws->ticket_overlap, scale_out, src, n, st); break;
+        default: rc = launch_amax_ticket<F32Tag>(&ws->ticket, &ws->ticket_overlap, scale_out, src, n, st); break;
     }
     if (rc != LQ_OK) return rc;
     return lq_fp8_scale_cast(dst, src, dtype, scale_out, 1, n, stream);
@@ -688,17 +730,39 @@ extern "C" int lq_fp8_amax_cast_slot(lq_stream_t stream) {
     return slot_for_stream(dev, as_stream(stream));
 }
 
+extern "C" int lq_fp8_amax_cast_release_slot(lq_stream_t stream) {
+    int dev = 0;
+    if (device_scratch(&dev) == nullptr) return LQ_ERR_HIP;
+    return release_slot(dev, as_stream(stream));
+}
+
 extern "C" size_t lq_fp8_amax_cast_static_max_elems(void) { return kTicketSlab * kTicketMaxSlabs; }
+
+namespace lq {
+__global__ void ticket_reset_kernel(TicketRegion* ws, unsigned* overlap) {
+    if (threadIdx.x < kTicketGroups) ws->group[threadIdx.x].count = 0;
+    if (threadIdx.x == kTicketGroups) ws->top.count = 0;
+    if (threadIdx.x == kTicketGroups + 1) *overlap = 0;
+}
+}  // namespace lq
+
+extern "C" int lq_fp8_amax_cast_static_reset(lq_stream_t stream) {
+    FusedScratch* ws = device_scratch();
+    if (ws == nullptr) return LQ_ERR_HIP;
+    hipLaunchKernelGGL(ticket_reset_kernel, dim3(1), dim3(64), 0, as_stream(stream), &ws->ticket, &ws->ticket_overlap);
+    return check_launch("fp8_amax_cast_static_reset");
+}
 
 extern "C" int lq_fp8_amax_cast_status(void) {
     FusedScratch* ws = device_scratch();
     if (ws == nullptr) return LQ_ERR_HIP;
-    unsigned flag = 0;
-    hipError_t e = hipMemcpy(&flag, &ws->timeout, sizeof(flag), hipMemcpyDeviceToHost);
-    if (e == hipSuccess && flag != 0) {
+    unsigned flags[2] = {0, 0};
+    hipError_t e = hipMemcpy(flags, &ws->timeout, sizeof(flags), hipMemcpyDeviceToHost);
+    if (e == hipSuccess && flags[0] != 0) {
         const unsigned zero = 0;
         e = hipMemcpy(&ws->timeout, &zero, sizeof(zero), hipMemcpyHostToDevice);
     }
+    const unsigned flag = flags[0];
     if (e != hipSuccess) {
         (void)hipGetLastError();
         set_error("lq_fp8_amax_cast_status: %s", hipGetErrorString(e));
@@ -709,6 +773,12 @@ extern "C" int lq_fp8_amax_cast_status(void) {
                   "(its scale is NaN); another stream's kernels held the device -- serialise the streams or quantise with "
                   "lq_fp8_amax_scale + lq_fp8_scale_cast");
         return 1;
+    }
+    if (flags[1] != 0) {
+        set_error("lq_fp8_amax_cast_static: calls overlapped on this GPU and left the ticket counters of the static scratch in a "
+                  "state no later call can finish from (scales stay unwritten); serialise the calls and run "
+                  "lq_fp8_amax_cast_static_reset");
+        return 2;
     }
     return 0;
 }

@@ -66,6 +66,8 @@ SYMBOLS = {
     "lq_fp8_amax_cast": (_I, [_P, _P, _P, _I, _Z, _P]),
     "lq_fp8_amax_cast_status": (_I, []),
     "lq_fp8_amax_cast_slot": (_I, [_P]),
+    "lq_fp8_amax_cast_release_slot": (_I, [_P]),
+    "lq_fp8_amax_cast_static_reset": (_I, [_P]),
     "lq_fp8_amax_cast_static": (_I, [_P, _P, _P, _I, _Z, _P]),
     "lq_fp8_amax_cast_static_max_elems": (_Z, []),
     "lq_w4a4_quantize": (_I, [_P, _P, _I, _P, _I, _P, _I, _I, _I, _P]),

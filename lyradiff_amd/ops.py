@@ -315,12 +315,26 @@ def fp8_quant(x):
 
 
 def fp8_amax_cast_status() -> bool:
-    """True when a one-launch fp8_quant on the current device timed out at its grid barrier since the last call (its
-    scale is NaN).  Copies 4 bytes from the device: synchronise the quantising streams first."""
+    """True when something went wrong in a dynamic fp8 quantisation on the current device since the last call: a one-launch
+    fp8_quant timed out at its exchange (its scale is NaN), or overlapping fp8_quant_static calls corrupted the ticket
+    counters (fp8_quant_static_reset repairs them); lyradiff_amd.lib.load().lq_last_error() says which.  Copies 8 bytes from
+    the device: synchronise the quantising streams first."""
     rc = _l.load().lq_fp8_amax_cast_status()
     if rc < 0:
         _l.check(rc, "lq_fp8_amax_cast_status")
-    return rc == 1
+    return rc >= 1
+
+
+def fp8_quant_release_stream(stream=None) -> int:
+    """Gives back the exchange slot the one-launch fp8_quant holds for `stream` (default: the current stream); call it before a
+    stream that quantised is destroyed.  Returns the freed slot or -1."""
+    st = _stream() if stream is None else stream.cuda_stream
+    return int(_l.load().lq_fp8_amax_cast_release_slot(st))
+
+
+def fp8_quant_static_reset() -> None:
+    """Puts the ticket counters of fp8_quant_static back to zero on the current stream (after calls overlapped)."""
+    _l.check(_l.load().lq_fp8_amax_cast_static_reset(_stream()), "lq_fp8_amax_cast_static_reset")
 
 
 def fp8_quant_static(x, q_out, scale_out):

@@ -6,6 +6,7 @@ import pytest
 import torch
 
 from oracle import oracle as O
+from oracle import oracle_c as OC
 from tests.helpers import TORCH_DT, make_outlier_acts, rng_t, to_np_f32
 
 pytestmark = pytest.mark.gpu
@@ -300,6 +301,51 @@ def test_fp8_amax_cast_stream_slots_fallback_and_status(ops, dev):
     torch.cuda.synchronize()
     for q, s in outs:
         assert s.item() == float(s_ref) and np.array_equal(q.cpu().numpy(), q_ref)
+    assert ops.fp8_amax_cast_status() is False
+    # slots are given back: afterwards a new stream finds one again, and a stream that owns none reports -1
+    freed = [ops.fp8_quant_release_stream(st) for st in streams]
+    assert sorted(v for v in freed if v >= 0) == sorted(owned) and freed.count(-1) == slots.count(-1)
+    assert ops.fp8_quant_release_stream(streams[0]) == -1
+    fresh = torch.cuda.Stream()
+    assert lib.lq_fp8_amax_cast_slot(C.c_void_p(fresh.cuda_stream)) >= 0
+    with torch.cuda.stream(fresh):
+        q, s = ops.fp8_quant(xd)
+    torch.cuda.synchronize()
+    assert s.item() == float(s_ref) and np.array_equal(q.cpu().numpy(), q_ref)
+    assert ops.fp8_quant_release_stream(fresh) >= 0
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32"])
+@pytest.mark.parametrize("n", [4096, 5000, 1024 * 16 * 256 * 4 + 1024 + 7, 23 * 1024 * 1024 + 1000, 52 * 1024 * 1024 + 13])
+def test_fp8_amax_cast_one_launch_sizes(ops, dev, dt, n):
+    """The one-launch quantiser over its register budgets: tensors that fit with 4, 8 and 12 chunks per thread, one that does
+    not (its rest is read twice), ragged tails shorter than a 2 KiB block; codes and scale equal the oracle's, and the
+    two-launch allocation-free form gives the same bits."""
+    if dt == "f32" and n > 30 * 1024 * 1024:
+        pytest.skip("the fp32 form is covered at the smaller sizes")
+    x = (torch.randn(n, generator=rng_t(n % 1000 + 5)) * 2.5).to(TORCH_DT[dt])
+    x[n // 3] = 37.0
+    xd = x.to(dev)
+    q, s = ops.fp8_quant(xd)
+    xf = to_np_f32(x)
+    s_ref = OC.fp8_scale(xf)
+    q_ref = OC.fp8_scale_cast(xf, s_ref)
+    assert s.item() == float(s_ref)
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+    q2, s2 = torch.empty_like(q), torch.empty_like(s)
+    ops.fp8_quant_static(xd, q2, s2)
+    assert torch.equal(q, q2) and torch.equal(s, s2)
+    assert ops.fp8_amax_cast_status() is False
+
+
+def test_fp8_quant_static_reset(ops, dev):
+    """The repair call of the allocation-free quantiser: after it the status is clean and the quantiser works."""
+    x = (torch.randn(70000, generator=rng_t(9)) * 3).bfloat16().to(dev)
+    ops.fp8_quant_static_reset()
+    q, s = torch.empty(70000, dtype=torch.uint8, device=dev), torch.empty(1, device=dev)
+    ops.fp8_quant_static(x, q, s)
+    q_ref, s_ref = O.fp8_amax_cast(to_np_f32(x.cpu()))
+    assert s.item() == float(s_ref) and np.array_equal(q.cpu().numpy(), q_ref)
     assert ops.fp8_amax_cast_status() is False
 
 
