@@ -127,6 +127,45 @@ template <typename Tag> __device__ __forceinline__ void unpack8(const uint4& v, 
     }
 }
 
+// ---- streaming accesses ---------------------------------------------------------------------------
+// Nontemporal 16-byte load / 4-, 8-, 16-byte stores for tensors that a quantisation kernel touches exactly once (its
+// activation input, its codes).  Measured on the fp8 amax + cast kernel at 4608x3072 from HBM: the load phase of the
+// whole-tensor-at-once access pattern took 7.5 us with plain loads and 6.3 us with these, and the time from launch to
+// launch fell by another 1.6 us with the stores marked, because the codes no longer wait dirty in the L2s for the
+// write-back at the end of the kernel.  STREAM false gives the plain access (small tensors that the next kernel
+// reads straight from L2).
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+constexpr size_t kStreamQuantBytes = (size_t)8 << 20;  // inputs from this size on take the streaming forms
+template <bool STREAM> __device__ __forceinline__ uint4 ld16(const void* p) {
+    if constexpr (STREAM) {
+        const u32x4_t v = __builtin_nontemporal_load(static_cast<const u32x4_t*>(p));
+        return make_uint4(v.x, v.y, v.z, v.w);
+    } else {
+        return *static_cast<const uint4*>(p);
+    }
+}
+template <bool STREAM> __device__ __forceinline__ void st16(void* p, const uint4& v) {
+    if constexpr (STREAM) {
+        const u32x4_t w = {v.x, v.y, v.z, v.w};
+        __builtin_nontemporal_store(w, static_cast<u32x4_t*>(p));
+    } else {
+        *static_cast<uint4*>(p) = v;
+    }
+}
+template <bool STREAM> __device__ __forceinline__ void st8(void* p, const uint2& v) {
+    if constexpr (STREAM) {
+        const u32x2_t w = {v.x, v.y};
+        __builtin_nontemporal_store(w, static_cast<u32x2_t*>(p));
+    } else {
+        *static_cast<uint2*>(p) = v;
+    }
+}
+template <bool STREAM> __device__ __forceinline__ void st4(void* p, unsigned int v) {
+    if constexpr (STREAM) __builtin_nontemporal_store(v, static_cast<unsigned int*>(p));
+    else *static_cast<unsigned int*>(p) = v;
+}
+
 // ---- wavefront (64 lanes) reductions ------------------------------------------------------------
 // Cross-lane steps inside a row of 16 lanes use DPP operand swizzles (no LDS traffic):
 // quad_perm [1,0,3,2] and [2,3,0,1] exchange with the lanes at distance 1 and 2, row_half_mirror

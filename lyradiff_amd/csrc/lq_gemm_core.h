@@ -102,7 +102,6 @@ __device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, i
 
 // store4_stream: the same store with the nontemporal hint, for an output that one streaming pass reads once (see
 // GemmParams::stream_c): its lines then do not displace the next kernel's operands from the last-level cache
-typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
 template <typename OutTag> struct OutStore;
 template <> struct OutStore<F16Tag> {
     static __device__ __forceinline__ void store4(void* C, size_t idx, const float* y) {

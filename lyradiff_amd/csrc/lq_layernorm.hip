@@ -69,7 +69,7 @@ __device__ __forceinline__ u32 ln_nan_fix(u32 w, const float* y) {  // NaN -> 0x
 // then take a step through LDS, added in wavefront order.
 // FULL (SPLIT only): dim is a multiple of 1024, every lane of every wavefront owns valid columns in both passes: no range
 // checks and no zero-filling of unused registers (7 % of the instructions of a kernel that is bound by its vector ALU).
-template <typename Tag, int NP, int QMODE, int RESID, bool MOD, bool SPLIT, bool FULL = false>
+template <typename Tag, int NP, int QMODE, int RESID, bool MOD, bool SPLIT, bool FULL = false, bool STREAM = false>
 __global__ __launch_bounds__(SPLIT ? 384 : 256) void ln_quant_rows_kernel(uint8_t* __restrict__ dst, void* __restrict__ dst2,
                                                             float* __restrict__ scale_out, const void* __restrict__ src,
                                                             const void* __restrict__ residual, const void* __restrict__ bias,
@@ -123,7 +123,7 @@ __global__ __launch_bounds__(SPLIT ? 384 : 256) void ln_quant_rows_kernel(uint8_
 #pragma unroll
         for (int i = 0; i < 8; ++i) h[p][i] = 0.0f;
         if (FULL || col < dim) {
-            unpack8<Tag>(*reinterpret_cast<const uint4*>(xs + col), h[p]);
+            unpack8<Tag>(ld16<STREAM>(xs + col), h[p]);
             if constexpr (RESID != 0) {
                 float r[8], b[8];
                 unpack8<Tag>(*reinterpret_cast<const uint4*>(static_cast<const unsigned short*>(residual) + row_off + col), r);
@@ -268,7 +268,7 @@ __global__ __launch_bounds__(SPLIT ? 384 : 256) void ln_quant_rows_kernel(uint8_
                     o.x = ln_nan_fix(o.x, v);
                     o.y = ln_nan_fix(o.y, v + 4);
                 }
-                *reinterpret_cast<uint2*>(out + row_off + col) = o;
+                st8<STREAM>(out + row_off + col, o);
             }
         }
         }
@@ -287,7 +287,7 @@ __global__ __launch_bounds__(SPLIT ? 384 : 256) void ln_quant_rows_kernel(uint8_
                     o.x = pack4_s8(q[0], q[1], q[2], q[3]);
                     o.y = pack4_s8(q[4], q[5], q[6], q[7]);
                 }
-                *reinterpret_cast<uint2*>(dst + row_off + col) = o;
+                st8<STREAM>(dst + row_off + col, o);
             }
         }
     }
@@ -304,7 +304,12 @@ template <typename Tag, int QMODE, int RESID, bool MOD> static int launch_ln(con
     if (np > 3) {
         LQ_REQUIRE(a.rows <= 0x7fffffffu, LQ_ERR_SHAPE, "layernorm: %zu rows exceed the launch limit", a.rows);
         dim3 grid((unsigned)a.rows), block(64 * ((np + 1) / 2));
-        if (a.dim % 1024 == 0)
+        // a large activation is read once and its codes written once: streaming accesses (see ld16 / st8)
+        const bool stream_io = QMODE != 3 && a.rows * (size_t)a.dim * 2 >= kStreamQuantBytes;
+        if (a.dim % 1024 == 0 && stream_io)
+            hipLaunchKernelGGL((ln_quant_rows_kernel<Tag, 2, QMODE, RESID, MOD, true, true, true>), grid, block, 0, st, a.dst, a.dst2, a.scale_out,
+                               a.src, a.residual, a.bias, a.gamma, a.beta, a.pre, a.in_scale, a.dst_b, a.in_scale_b, a.rows, a.dim, a.rows_per_batch, a.eps, 1.0f / (float)a.dim);
+        else if (a.dim % 1024 == 0)
             hipLaunchKernelGGL((ln_quant_rows_kernel<Tag, 2, QMODE, RESID, MOD, true, true>), grid, block, 0, st, a.dst, a.dst2, a.scale_out,
                                a.src, a.residual, a.bias, a.gamma, a.beta, a.pre, a.in_scale, a.dst_b, a.in_scale_b, a.rows, a.dim, a.rows_per_batch, a.eps, 1.0f / (float)a.dim);
         else

@@ -146,7 +146,7 @@ __global__ __launch_bounds__(256) void sq_quant_rows_kernel(int8_t* __restrict__
 // registers whatever the row length, so eight of them share a SIMD and the loads of one overlap the
 // arithmetic of the others; the dynamic variant exchanges the span maxima through LDS (one barrier).
 // A lane outside the row re-reads a valid octet (harmless for the maximum) and stores nothing.
-template <typename Tag, int MODE, bool HAS_PRE, int R>
+template <typename Tag, int MODE, bool HAS_PRE, int R, bool STREAM = false>
 __global__ __launch_bounds__(1024) void sq_quant_split_kernel(int8_t* __restrict__ dst, float* __restrict__ scale_out,
                                                               const void* __restrict__ src,
                                                               const float* __restrict__ pre,
@@ -177,7 +177,8 @@ __global__ __launch_bounds__(1024) void sq_quant_split_kernel(int8_t* __restrict
             const int c = wave * 1024 + p * 512 + lane * 8;
             valid[p] = c < dim;
             col[p] = valid[p] ? c : 0;
-            if constexpr (kMix) raw[rr][p] = *reinterpret_cast<const uint4*>(rb + (size_t)col[p] * 2);
+            if constexpr (kMix) raw[rr][p] = ld16<STREAM>(rb + (size_t)col[p] * 2);
+            else if constexpr (Elem<Tag>::bytes == 2) unpack8<Tag>(ld16<STREAM>(rb + (size_t)col[p] * 2), t[rr][p]);
             else load8<Tag>(rb, col[p], t[rr][p]);
         }
     }
@@ -242,7 +243,7 @@ __global__ __launch_bounds__(1024) void sq_quant_split_kernel(int8_t* __restrict
                 o.x = pack4_s8(q[0], q[1], q[2], q[3]);
                 o.y = pack4_s8(q[4], q[5], q[6], q[7]);
             }
-            if (valid[p] && live[rr]) *reinterpret_cast<uint2*>(ob + col[p]) = o;
+            if (valid[p] && live[rr]) st8<STREAM>(ob + col[p], o);
         }
     }
 }
@@ -302,12 +303,15 @@ static int launch_sq_quant(int8_t* dst, float* scale_out, const void* src, const
         // one wavefront per 1024 columns, one workgroup per row
         LQ_REQUIRE(rows <= 0x7fffffffu, LQ_ERR_SHAPE, "sq_quant: %zu rows exceed the launch limit", rows);
         dim3 block(64 * ((np + 1) / 2));
+        const bool stream_io = rows * dim * Elem<Tag>::bytes >= kStreamQuantBytes;  // read-once input, write-once codes
         if (pre && dim >= 2048) {  // long rows with a smoothing vector: two rows per workgroup share its loads
             dim3 grid((unsigned)((rows + 1) / 2));
-            hipLaunchKernelGGL((sq_quant_split_kernel<Tag, MODE, true, 2>), grid, block, 0, st, dst, scale_out, src, pre, in_scale, rows, d);
+            if (stream_io) hipLaunchKernelGGL((sq_quant_split_kernel<Tag, MODE, true, 2, true>), grid, block, 0, st, dst, scale_out, src, pre, in_scale, rows, d);
+            else hipLaunchKernelGGL((sq_quant_split_kernel<Tag, MODE, true, 2>), grid, block, 0, st, dst, scale_out, src, pre, in_scale, rows, d);
         } else {
             dim3 grid((unsigned)rows);
             if (pre) hipLaunchKernelGGL((sq_quant_split_kernel<Tag, MODE, true, 1>), grid, block, 0, st, dst, scale_out, src, pre, in_scale, rows, d);
+            else if (stream_io) hipLaunchKernelGGL((sq_quant_split_kernel<Tag, MODE, false, 1, true>), grid, block, 0, st, dst, scale_out, src, pre, in_scale, rows, d);
             else hipLaunchKernelGGL((sq_quant_split_kernel<Tag, MODE, false, 1>), grid, block, 0, st, dst, scale_out, src, pre, in_scale, rows, d);
         }
         return check_launch("sq_quant_split");

@@ -17,7 +17,7 @@ namespace lq {
 // slower all the same (15.4 against 14.7 us at 4608x3072 from HBM: sixteen wavefronts wait at one barrier for the staging's
 // load and division chain, where small workgroups on a CU are in different phases), so four it stays.
 // FULL: k is a multiple of the column range, no lane is ever out of range.
-template <typename Tag, int NP, bool F16_SCALE, int SMOOTH, int WAVES = 4, bool FULL = false>
+template <typename Tag, int NP, bool F16_SCALE, int SMOOTH, int WAVES = 4, bool FULL = false, bool STREAM = false>
 __global__ __launch_bounds__(WAVES * 64) void w4a4_quant_kernel(u32* __restrict__ q_words, void* __restrict__ scales,
                                                          const void* __restrict__ x,
                                                          const float* __restrict__ smooth, int m, int k,
@@ -40,7 +40,7 @@ __global__ __launch_bounds__(WAVES * 64) void w4a4_quant_kernel(u32* __restrict_
 #pragma unroll
             for (int u = 0; u < VPP; ++u) {
                 if constexpr (!FULL) raw[p][u] = make_uint4(0, 0, 0, 0);
-                if (FULL || col < k) raw[p][u] = *reinterpret_cast<const uint4*>(rb + (size_t)col * Elem<Tag>::bytes + u * 16);
+                if (FULL || col < k) raw[p][u] = ld16<STREAM>(rb + (size_t)col * Elem<Tag>::bytes + u * 16);
             }
         }
     };
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(WAVES * 64) void w4a4_quant_kernel(u32* __restrict_
 #pragma unroll
             for (int i = 0; i < 8; ++i) word = __builtin_amdgcn_alignbit((u32)q[i], word, 4);
             if (FULL || col < k) {
-                q_words[(size_t)row * (k >> 3) + (col >> 3)] = word;
+                st4<STREAM>(q_words + (size_t)row * (k >> 3) + (col >> 3), word);
                 if ((lane & 7) == 0) {
                     size_t si = (size_t)row * ng + (col >> 6);
                     if constexpr (F16_SCALE) static_cast<unsigned short*>(scales)[si] = (unsigned short)f32_to_f16_bits(s);  // s is already an fp16 value
@@ -204,8 +204,12 @@ extern "C" int lq_w4a4_quantize(uint32_t* q_words, void* scales, lq_dtype_t scal
     const size_t lds = smode == 1 ? 2 * (size_t)np * 512 * sizeof(float) : 0;
     // long rows whose length is a whole number of column ranges (FLUX: 3072): no range checks
     if (smode == 1 && np == 2 && k % 1024 == 0 && x_dtype != LQ_F32) {
-#define LQ_W4_FULL(TAG, F16S) \
-    hipLaunchKernelGGL((w4a4_quant_kernel<TAG, 2, F16S, 1, 4, true>), grid, block, lds, st, q_words, scales, x, smooth, m, k, rpw, parts)
+        const bool stream_io = (size_t)m * k * 2 >= kStreamQuantBytes;  // read-once input, write-once codes
+#define LQ_W4_FULL(TAG, F16S)                                                                                                          \
+    do {                                                                                                                               \
+        if (stream_io) hipLaunchKernelGGL((w4a4_quant_kernel<TAG, 2, F16S, 1, 4, true, true>), grid, block, lds, st, q_words, scales, x, smooth, m, k, rpw, parts); \
+        else hipLaunchKernelGGL((w4a4_quant_kernel<TAG, 2, F16S, 1, 4, true, false>), grid, block, lds, st, q_words, scales, x, smooth, m, k, rpw, parts);       \
+    } while (0)
         if (x_dtype == LQ_F16) { if (f16s) LQ_W4_FULL(F16Tag, true); else LQ_W4_FULL(F16Tag, false); }
         else { if (f16s) LQ_W4_FULL(BF16Tag, true); else LQ_W4_FULL(BF16Tag, false); }
 #undef LQ_W4_FULL
