@@ -66,8 +66,8 @@ extern "C" int lq_gemm_set_thread_tactic(int tactic) {
 
 extern "C" int lq_gemm_tactic_count(lq_weight_kind_t kind) {
     switch (kind) {
-        case LQ_W_INT8: return 7;
-        case LQ_W_FP8: return 7;
+        case LQ_W_INT8: return 8;
+        case LQ_W_FP8: return 8;
         case LQ_W_INT4: return 3;
         default: lq::set_error("lq_gemm_tactic_count: bad kind %d", (int)kind); return LQ_ERR_ARG;
     }

@@ -76,6 +76,8 @@ struct GemmParams {
     int m, n, k;
     int kb;  // bytes per operand row: k (int8/fp8) or k/2 (int4)
     int tiles_m, tiles_n;
+    // persistent kernel: whole-tile rounds per workgroup and the number of half tiles in its last, split round (0: none)
+    int persist_rounds, persist_halves;
 };
 
 template <int CH> __device__ __forceinline__ int chunk_swizzle(int row) {
@@ -897,5 +899,12 @@ static int launch_gemm(GemmParams p, hipStream_t st) {
     hipLaunchKernelGGL(kern, grid, block, GK::SMEM_BYTES, st, p);
     return check_launch("gemm");
 }
+
+// Persistent one-wavefront-per-SIMD form (lq_gemm_persist.h, compiled in lq_gemm_persist.hip): LQ_OK when launched, 1 when
+// the call is not one it implements (shape with partial tiles or an odd number of k-tiles, an epilogue beyond scales and
+// bias, an output type other than fp16 / bf16) -- the caller then runs the plain configuration -- negative on an error.
+int launch_persist_fp8(const GemmParams& p, lq_dtype_t out_dtype, hipStream_t st);
+int launch_persist_int8(const GemmParams& p, lq_dtype_t out_dtype, hipStream_t st);
+int device_cu_count();  // compute units of the current device (cached per device)
 
 }  // namespace lq

@@ -7,8 +7,14 @@
 namespace lq {
 
 
+template <typename OutTag> static constexpr lq_dtype_t out_enum() {
+    return std::is_same<OutTag, F16Tag>::value ? LQ_F16 : std::is_same<OutTag, BF16Tag>::value ? LQ_BF16 : LQ_F32;
+}
+
 template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
     int t = requested_tactic(g_tactic_fp8, LQ_W_FP8, p.m, p.n, p.k);
+    const bool plain_epilogue = p.gelu == 0 && p.out_scale == nullptr && p.C8 == nullptr && p.gate == nullptr &&
+                                p.residual == nullptr && p.addend == nullptr;
     if (t < 0) {
         const long t256 = (long)((p.m + 255) / 256) * ((p.n + 255) / 256);
         const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
@@ -19,6 +25,11 @@ template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
         const long last256 = t256 % 256;
         t = t256 >= 192 ? ((last256 == 0 || last256 >= 128) ? 6 : 4) : (t128 >= 128 ? 2 : 3);  // 128x128 tiles from half a round up (4096x640x2560: 14.5 against 16.3 us with 64x64)
         if (p.k <= 1024 && t128 >= 192) t = 2;  // short K: prologue and epilogue dominate, smaller tiles overlap them better
+        // More full 256x256 tiles than CUs and nothing but scales and bias in the epilogue: the persistent form
+        // (4608x12288x3072: 134-140 us against 148 with 128x256 tiles, 6912x9216x3072: 156 against 161 with tactic 6)
+        if (plain_epilogue && t256 > device_cu_count() && p.m % 256 == 0 && p.n % 256 == 0 && p.kb % 128 == 0 && p.k > 1024 &&
+            out_enum<OutTag>() != LQ_F32)
+            t = 7;
     }
     if (t == 1 && p.kb % 128 != 0) t = 0;  // the 128-byte k-tile needs k % 128 == 0
     // The per-shape cache is filled by timing the plain epilogue.  With one wavefront per SIMD nothing runs beside tactic 6's
@@ -28,9 +39,12 @@ template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
     // 153-160 us with tactic 4; 3072x12288 with gate and residual 139 us against 134 us with tactic 0, 3072x3072 55 against
     // 48 us.  A configuration forced by the caller is kept.
     const bool forced = tl_forced_tactic >= 0 || g_tactic_fp8 >= 0;
-    const bool plain_epilogue = p.gelu == 0 && p.out_scale == nullptr && p.C8 == nullptr && p.gate == nullptr &&
-                                p.residual == nullptr && p.addend == nullptr;
-    if (t == 6 && !forced && !plain_epilogue) t = (long)((p.m + 255) / 256) * ((p.n + 255) / 256) > 256 ? 4 : 0;
+    if ((t == 6 || t == 7) && !forced && !plain_epilogue) t = (long)((p.m + 255) / 256) * ((p.n + 255) / 256) > 256 ? 4 : 0;
+    if (t == 7) {  // the persistent form of tactic 6 where it applies, tactic 6 itself elsewhere
+        const int rc = launch_persist_fp8(p, out_enum<OutTag>(), st);
+        if (rc != 1) return rc;
+        t = 6;
+    }
     switch (t) {
         case 0: return launch_gemm<K_FP8, OutTag, 256, 256, 64, 2, 4, 3>(p, st);
         case 1: return launch_gemm<K_FP8, OutTag, 256, 256, 128, 2, 4, 2>(p, st);

@@ -7,6 +7,11 @@
 namespace lq {
 
 
+template <typename OutTag> static constexpr lq_dtype_t out_enum() {
+    return std::is_same<OutTag, F16Tag>::value ? LQ_F16 : std::is_same<OutTag, BF16Tag>::value ? LQ_BF16
+                                                 : std::is_same<OutTag, F32Tag>::value ? LQ_F32 : LQ_I32;
+}
+
 template <typename OutTag> static int run_int8(GemmParams p, hipStream_t st) {
     // static tile table in place of the reference's run-time tactic profiler
     // (layers/gemm_utils/GemmProfiler.cc:78-127): largest tile that still fills the 256 CUs.
@@ -21,8 +26,17 @@ template <typename OutTag> static int run_int8(GemmParams p, hipStream_t st) {
         const long last256 = t256 % 256;
         t = t256 >= 192 ? ((last256 == 0 || last256 >= 128) ? 6 : 4) : (t128 >= 128 ? 2 : 3);  // 128x128 tiles from half a round up (4096x640x2560: 14.5 against 16.3 us with 64x64)
         if (p.k <= 1024 && t128 >= 192) t = 2;  // short K: prologue and epilogue dominate, smaller tiles overlap them better
+        // more full 256x256 tiles than CUs: the persistent form (4608x12288x3072: 153-160 us against 162-165 with 128x256 tiles)
+        if (t256 > device_cu_count() && p.m % 256 == 0 && p.n % 256 == 0 && p.kb % 128 == 0 && p.k > 1024 &&
+            (out_enum<OutTag>() == LQ_F16 || out_enum<OutTag>() == LQ_BF16))
+            t = 7;
     }
     if (t == 1 && p.kb % 128 != 0) t = 0;  // the 128-byte k-tile needs k % 128 == 0
+    if (t == 7) {  // the persistent form of tactic 6 where it applies, tactic 6 itself elsewhere
+        const int rc = launch_persist_int8(p, out_enum<OutTag>(), st);
+        if (rc != 1) return rc;
+        t = 6;
+    }
     switch (t) {
         case 0: return launch_gemm<K_INT8, OutTag, 256, 256, 64, 2, 4, 3>(p, st);
         case 1: return launch_gemm<K_INT8, OutTag, 256, 256, 128, 2, 4, 2>(p, st);

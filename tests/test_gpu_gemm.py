@@ -205,7 +205,7 @@ def test_w4a4_gemm(ops, dev, m, n, k, sdt):
 
 
 # ---- every tile configuration, forced one by one, against the same oracle -------------------------------------------
-N_TACTICS = {"int8": 7, "fp8": 7, "int4": 3}
+N_TACTICS = {"int8": 8, "fp8": 8, "int4": 3}
 
 
 @pytest.fixture
@@ -264,6 +264,51 @@ def test_fp8_gemm_every_tactic(ops, dev, tactic, k, tactic_guard):
     check_fp8_gemm(y, O.fp8_gemm(qa, qb, sa, sb, to_np_f32(bias), False, None, 0.0, "bf16"), qa, qb, sa, sb, "bf16", "fp8 tactic")
     rows = np.arange(0, m, 37)  # every tactic walks k in the same order, so each reproduces the instruction model
     check_fp8_against_instruction_model(y[rows], qa[rows], qb, sa, sb, to_np_f32(bias), "bf16", f"fp8 tactic {tactic}")
+
+
+@pytest.mark.parametrize("kind", ["int8", "fp8"])
+@pytest.mark.parametrize("m,n,k", [(512, 1024, 256),     # 8 tiles: fewer than CUs, one round, four k-tiles (two per buffer parity)
+                                   (4608, 12288, 128),   # 864 tiles: three rounds on 256 CUs and 96 left over, cut into 192 halves
+                                   (4864, 14336, 384),   # 1064 tiles: four rounds and 40 left over (80 halves)
+                                   (6912, 9216, 256),    # 972 tiles: 204 left over, more than half a round: whole tiles
+                                   (4608, 12288 + 256, 128)])  # 882 tiles: 114 left over, not a multiple of 8: whole tiles
+def test_persistent_gemm(ops, dev, kind, m, n, k, tactic_guard):
+    """Tactic 7, the persistent one-wavefront-per-SIMD kernel: every tile count class (fewer tiles than CUs, leftover tiles
+    cut into halves, leftover tiles kept whole) gives the bits of tactic 4, whose results the other tests pin to the oracle (all
+    tactics walk k in the same order); one 256-row band of the big outputs is compared with the oracle directly."""
+    g = rng_t(m + n + k)
+    rows = slice(m - 256, m)  # the last band: a half tile where the last round is split
+    if kind == "int8":
+        a = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int8)
+        w = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8)
+        ac = (torch.rand(n, generator=g) * 9e-3 + 1e-3).float()
+        ar = (torch.rand(m, generator=g) * 0.05 + 0.01).float()
+        bias = (torch.randn(n, generator=g) * 0.02).half()
+        wp = ops.repack_weight(w.to(dev))
+        run = lambda: ops.int8_linear(a.to(dev), wp, ac.to(dev), ar.to(dev), bias.to(dev), torch.float16)
+        ref = O.int8_epilogue(O.gemm_i8_acc(a[rows].numpy(), w.numpy()), ac.numpy(), ar[rows].numpy(), to_np_f32(bias), "f16")
+    else:
+        qa, sa = O.fp8_amax_cast(to_np_f32(torch.randn(m, k, generator=g).bfloat16()))
+        qb, sb = O.fp8_amax_cast(to_np_f32((torch.randn(n, k, generator=g) * 0.02).bfloat16()))
+        bias = (torch.randn(n, generator=g) * 0.1).bfloat16()
+        wp = ops.repack_weight(torch.from_numpy(qb).to(dev))
+        sad, sbd = torch.tensor([sa], dtype=torch.float32, device=dev), torch.tensor([sb], dtype=torch.float32, device=dev)
+        run = lambda: ops.fp8_linear(torch.from_numpy(qa).to(dev), wp, sad, sbd, bias.to(dev), False, None, 0.0, torch.bfloat16)
+        ref = None
+    ops.gemm_set_tactic(kind, 4)
+    want = run()
+    ops.gemm_set_tactic(kind, 7)
+    got = run()
+    again = run()
+    assert torch.equal(got, want) and torch.equal(again, want)
+    if kind == "int8":
+        assert np.array_equal(to_np_f32(got[rows]), ref)
+    else:
+        y = to_np_f32(got[rows])
+        check_fp8_gemm(y, O.fp8_gemm(qa[rows], qb, sa, sb, to_np_f32(bias), False, None, 0.0, "bf16"), qa[rows], qb, sa, sb, "bf16", "fp8 persistent")
+    ops.gemm_set_tactic(kind, -1)
+    if k > 1024:
+        assert torch.equal(run(), want)  # the built-in table takes the same kernel for these shapes
 
 
 @pytest.mark.parametrize("tactic", range(N_TACTICS["int4"]))
