@@ -256,13 +256,13 @@ def main():
     zq, zw = torch.zeros_like(qx0), torch.zeros_like(wp_up)
     zeros_us = batched(lambda i: ops.fp8_linear(zq, zw, sx0, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh0))
 
-    def clock_under(fn, n=6):
+    def clock_under(fn, per_launch_us=None, n=6):
         side = torch.cuda.Stream()
         torch.cuda.synchronize()
         for i in range(20):
             fn(i)  # the kernel under study is running, and has been for a while, before the probe starts
         with torch.cuda.stream(side):
-            t = ops.shader_clock_probe(int(0.6 * n * alone["gemm_up"]), 8, side)
+            t = ops.shader_clock_probe(int(0.6 * n * (per_launch_us or alone["gemm_up"])), 8, side)
         for i in range(n):
             fn(i)
         torch.cuda.synchronize()
@@ -280,18 +280,19 @@ def main():
         del wd8
     except Exception:  # not every PyTorch build exposes it
         pass
-    # what the matrix pipes alone sustain on this part: 16 x 300 FP8 MFMAs per wavefront on register operands, no memory or
+    # what the matrix pipes alone sustain on this part: 16 x 1000 FP8 MFMAs per wavefront on register operands, no memory or
     # LDS traffic, one wavefront per SIMD (the layout of the down projection's kernel), on the chain's input codes and on zeros
     pipe_only = {}
     for name, codes in (("random_operands", qx0.view(-1)[: 1 << 22]), ("zero_operands", None)):
         flop = [0.0]
 
         def probe(i, codes=codes):
-            flop[0] = ops.mfma_fp8_probe(codes, 300)
+            flop[0] = ops.mfma_fp8_probe(codes, 1000)
 
         us = batched(probe)
         pipe_only[name] = {"us": round(us, 2), "TFLOP/s": round(flop[0] / us / 1e6, 1)}
-    pipe_only["random_operands"]["shader_clock_ghz"] = clock_under(lambda i: ops.mfma_fp8_probe(qx0.view(-1)[: 1 << 22], 300))
+    pipe_only["random_operands"]["shader_clock_ghz"] = clock_under(lambda i: ops.mfma_fp8_probe(qx0.view(-1)[: 1 << 22], 1000), pipe_only["random_operands"]["us"])
+    pipe_only["zero_operands"]["shader_clock_ghz"] = clock_under(lambda i: ops.mfma_fp8_probe(None, 1000), pipe_only["zero_operands"]["us"])
     clocks = {
         "idle": clock_under(lambda i: None),
         "up_gemm_random_operands": clock_under(lambda i: ops.fp8_linear(qx0, wp_up, sx0, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh0)),

@@ -360,6 +360,19 @@ public:
     }
     // -1: nothing profiled for this shape, the library's built-in table applies
     int getBestConfig(int m, int n, int k) const { return mSkip ? -1 : lq_gemm_get_shape_tactic(LQ_W_INT8, m, n, k); }
+    // GemmPluginProfiler::getSerializationSize / serialize / deserialize (layers/gemm_utils/GemmProfiler.cc:26-75): the
+    // measured configurations as bytes; the library keeps one table for every shape, so the GEMM id argument of the
+    // reference is not needed.  serialize advances `buffer`, deserialize advances `data`, as the reference's do.
+    size_t getSerializationSize() const { return lq_gemm_tactics_serialized_size(); }
+    void serialize(char*& buffer) const {
+        size_t written = 0;
+        detail::check(lq_gemm_tactics_serialize(buffer, lq_gemm_tactics_serialized_size(), &written), "GemmPluginProfiler::serialize");
+        buffer += written;
+    }
+    void deserialize(char const*& data, size_t bytes) {
+        detail::check(lq_gemm_tactics_deserialize(data, bytes), "GemmPluginProfiler::deserialize");
+        data += bytes;
+    }
     QuantMode mQuantMode;
 
 private:

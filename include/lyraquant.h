@@ -442,7 +442,9 @@ int lq_load_lora(void* dst, const void* src, lq_dtype_t dtype, size_t n, float a
  * the built-in static table.  Stands in for the CutlassGemmConfig argument of
  * CutlassInt8GemmRunner<T>::gemm and the tactic cache of GemmPluginProfiler
  * (kernels/cutlass_kernels/int8_gemm/int8_gemm.h:24-39, layers/gemm_utils/GemmProfiler.cc:78-143).
- * Unknown tactic numbers make the next GEMM call fail with LQ_ERR_ARG. */
+ * Unknown tactic numbers make the next GEMM call fail with LQ_ERR_ARG.  INT8 / FP8: 0-5 tile shapes with two wavefronts
+ * per SIMD, 6 = 256x256 tiles with one wavefront per SIMD, 7 = the persistent form of 6 (one workgroup per CU walks its
+ * tiles; full 256x256 tiles, k %% 128 == 0, scales and bias only, fp16 / bf16 output -- any other call runs as 6). */
 int lq_gemm_set_tactic(lq_weight_kind_t kind, int tactic);
 
 /* Tile configuration for the GEMM calls the CALLING THREAD makes from now on (any kind), ahead of every
@@ -464,6 +466,17 @@ int lq_gemm_tactic_count(lq_weight_kind_t kind);
 int lq_gemm_set_shape_tactic(lq_weight_kind_t kind, int m, int n, int k, int tactic);
 int lq_gemm_get_shape_tactic(lq_weight_kind_t kind, int m, int n, int k);
 
+/* The per-shape tactic cache as a byte string, so that a process need not profile again what an earlier one measured
+ * on the same part: the role of GemmPluginProfiler::serialize / deserialize / getSerializationSize
+ * (layers/gemm_utils/GemmProfiler.cc:26-75; SmoothQuantGemmPlugin::serialize, layers/gemm_utils/SmoothQuantGemm.cc:177-194).
+ * Format: the four bytes "LQT1", the entry count, then {kind, m, n, k, tactic} per entry, all little-endian int32.
+ * lq_gemm_tactics_serialize writes lq_gemm_tactics_serialized_size() bytes (LQ_ERR_ARG when the buffer is smaller);
+ * lq_gemm_tactics_deserialize checks the whole table (magic, length, kinds, tactic numbers against
+ * lq_gemm_tactic_count) before it adds the entries to the cache, replacing entries of the same shape.  Host memory. */
+size_t lq_gemm_tactics_serialized_size(void);
+int lq_gemm_tactics_serialize(void* buffer, size_t buffer_bytes, size_t* written);
+int lq_gemm_tactics_deserialize(const void* data, size_t bytes);
+
 /* Set-up-time profiler, the role of GemmPluginProfiler::profileTactics
  * (layers/gemm_utils/GemmProfiler.cc:78-127,161-265): runs every tile configuration of the `kind`
  * GEMM on shape (m, n, k) with synthetic operands placed in `workspace` (caller-owned device memory
@@ -483,8 +496,8 @@ int lq_shader_clock_probe(uint64_t* out_ticks, int probes, unsigned microseconds
 
 /* Measurement aid (no reference counterpart): one 256-thread workgroup per CU; every wavefront issues `iters` times 16
  * independent v_mfma_f32_32x32x64_f8f6f4 (a 128x128 wavefront tile) on register operands drawn from `operand_codes` (e4m3
- * codes, n_codes >= 4, 4-byte aligned; NULL = all-zero operands) and rotated between iterations, with no memory or LDS
- * traffic: 2*32*32*64 * 16 * iters * 4 * *workgroups FLOP per launch.  Timed by the caller, it gives what the matrix pipes
+ * codes, n_codes >= 4096, 4-byte aligned; NULL = all-zero operands), two sets of fragments alternating, with no memory or
+ * LDS traffic and no instruction that depends on an MFMA in flight: 2*32*32*64 * 16 * iters * 4 * *workgroups FLOP per launch.  Timed by the caller, it gives what the matrix pipes
  * alone sustain on this part -- on real codes they are power limited well below the published peak, on zeros they are not.
  * `sink` (4 bytes of device memory) is practically never written; *workgroups (optional) receives the grid size. */
 int lq_mfma_fp8_probe(float* sink, const uint8_t* operand_codes, size_t n_codes, int iters, int* workgroups, lq_stream_t stream);

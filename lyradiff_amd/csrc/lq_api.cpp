@@ -91,3 +91,60 @@ extern "C" int lq_gemm_set_shape_tactic(lq_weight_kind_t kind, int m, int n, int
 extern "C" int lq_gemm_get_shape_tactic(lq_weight_kind_t kind, int m, int n, int k) {
     return lq::shape_tactic_lookup((int)kind, m, n, k);
 }
+
+// ---- the per-shape cache as a byte string: "LQT1", entry count, then {kind, m, n, k, tactic} as little-endian int32 ----
+static const unsigned kTacticsMagic = 0x3154514Cu;  // "LQT1"
+
+extern "C" size_t lq_gemm_tactics_serialized_size(void) {
+    std::shared_lock<std::shared_timed_mutex> lock(lq::g_shape_mutex);
+    return 8 + lq::g_shape_tactics.size() * 20;
+}
+
+extern "C" int lq_gemm_tactics_serialize(void* buffer, size_t buffer_bytes, size_t* written) {
+    if (buffer == nullptr) {
+        lq::set_error("lq_gemm_tactics_serialize: null buffer");
+        return LQ_ERR_ARG;
+    }
+    std::shared_lock<std::shared_timed_mutex> lock(lq::g_shape_mutex);
+    const size_t need = 8 + lq::g_shape_tactics.size() * 20;
+    if (buffer_bytes < need) {
+        lq::set_error("lq_gemm_tactics_serialize: the buffer holds %zu bytes, %zu are needed", buffer_bytes, need);
+        return LQ_ERR_ARG;
+    }
+    int* out = static_cast<int*>(buffer);
+    *out++ = (int)kTacticsMagic;
+    *out++ = (int)lq::g_shape_tactics.size();
+    for (auto const& e : lq::g_shape_tactics) {
+        *out++ = std::get<0>(e.first);
+        *out++ = std::get<1>(e.first);
+        *out++ = std::get<2>(e.first);
+        *out++ = std::get<3>(e.first);
+        *out++ = e.second;
+    }
+    if (written) *written = need;
+    return LQ_OK;
+}
+
+extern "C" int lq_gemm_tactics_deserialize(const void* data, size_t bytes) {
+    const int* in = static_cast<const int*>(data);
+    if (data == nullptr || bytes < 8 || (unsigned)in[0] != kTacticsMagic || in[1] < 0 || (size_t)in[1] > (bytes - 8) / 20) {
+        lq::set_error("lq_gemm_tactics_deserialize: not a tactic table (%zu bytes)", bytes);
+        return LQ_ERR_ARG;
+    }
+    const int count = in[1];
+    for (int i = 0; i < count; ++i) {  // validate everything before anything is stored
+        const int* e = in + 2 + 5 * i;
+        const int tactics = lq_gemm_tactic_count((lq_weight_kind_t)e[0]);
+        if (tactics < 0 || e[1] <= 0 || e[2] <= 0 || e[3] <= 0 || e[4] < 0 || e[4] >= tactics) {
+            lq::set_error("lq_gemm_tactics_deserialize: entry %d is invalid (kind %d, m %d, n %d, k %d, tactic %d)", i, e[0], e[1], e[2], e[3], e[4]);
+            return LQ_ERR_ARG;
+        }
+    }
+    std::unique_lock<std::shared_timed_mutex> lock(lq::g_shape_mutex);
+    for (int i = 0; i < count; ++i) {
+        const int* e = in + 2 + 5 * i;
+        lq::g_shape_tactics[std::make_tuple(e[0], e[1], e[2], e[3])] = e[4];
+    }
+    lq::g_shape_entries.store((int)lq::g_shape_tactics.size(), std::memory_order_relaxed);
+    return LQ_OK;
+}

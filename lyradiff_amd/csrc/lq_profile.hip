@@ -5,6 +5,7 @@
 // events, keep the minimum; here in interleaved rounds), but the caller owns the temporary memory and nothing is allocated here.
 #include <algorithm>
 #include "lq_common.h"
+#include <type_traits>
 
 namespace lq {
 
@@ -80,45 +81,54 @@ extern "C" int lq_shader_clock_probe(uint64_t* out_ticks, int probes, unsigned m
 }
 
 // What the matrix pipes alone sustain: every wavefront (one per SIMD, one workgroup per CU) issues 16 independent
-// v_mfma_f32_32x32x64_f8f6f4 per iteration on operand fragments held in registers -- a 128x128 wavefront tile without any
-// memory or LDS traffic -- and rotates the fragments' registers between iterations so that the operand buses keep toggling
-// as they do in a GEMM.  With operands drawn from real e4m3 codes the part is power limited; with zeros it is not.
+// v_mfma_f32_32x32x64_f8f6f4 per step on operand fragments held in registers -- a 128x128 wavefront tile without any
+// memory or LDS traffic.  Two sets of fragments (two k-steps' worth) alternate by unrolled index, so consecutive MFMAs never
+// read the same pair of operand registers and nothing is written between them: no instruction of the loop depends on an
+// MFMA in flight (an earlier form rotated the fragments' registers with 64 moves per step, whose destinations were sources
+// of MFMAs still executing; its matrix pipes were busy three quarters of the time).  With operands drawn from real e4m3
+// codes the part is power limited; with zeros it is not.
 __global__ __launch_bounds__(256, 1) void mfma_fp8_probe_kernel(float* sink, const uint32_t* __restrict__ src, size_t src_words, int iters) {
     typedef int v8i_t __attribute__((ext_vector_type(8)));
     typedef float v16f_t __attribute__((ext_vector_type(16)));
-    v8i_t a[4], b[4];
+    v8i_t a[2][4], b[2][4];
+    const u32 words = src_words ? (u32)(src_words > 0x40000000u ? 0x40000000u : src_words) : 1u;
+    const u32 start = (u32)(((size_t)blockIdx.x * 16384u) % words);
 #pragma unroll
-    for (int f = 0; f < 4; ++f)
+    for (int s = 0; s < 2; ++s)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const size_t ia = ((size_t)blockIdx.x * 8192 + (threadIdx.x + 256 * f) * 8 + i) % (src_words ? src_words : 1);
-            const size_t ib = ((size_t)blockIdx.x * 8192 + (threadIdx.x + 256 * (f + 4)) * 8 + i) % (src_words ? src_words : 1);
-            a[f][i] = src ? (int)src[ia] : 0;
-            b[f][i] = src ? (int)src[ib] : 0;
-        }
+        for (int f = 0; f < 4; ++f)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                // one division per thread (start); the offsets wrap by subtraction -- 128 64-bit divisions per thread took
+                // longer than a thousand MFMAs
+                u32 ia = start + (u32)s * 8192u + (threadIdx.x + 256u * f) * 8u + i;
+                u32 ib = start + (u32)s * 8192u + (threadIdx.x + 256u * (f + 4)) * 8u + i;
+                if (src) {
+                    while (ia >= words) ia -= words;
+                    while (ib >= words) ib -= words;
+                }
+                a[s][f][i] = src ? (int)src[ia] : 0;
+                b[s][f][i] = src ? (int)src[ib] : 0;
+            }
     v16f_t acc[16];
 #pragma unroll
     for (int t = 0; t < 16; ++t)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[t][i] = 0.0f;
-    for (int it = 0; it < iters; ++it) {
+    auto step = [&](auto set_c) {
+        constexpr int s = decltype(set_c)::value;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                acc[i * 4 + j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[i], b[j], acc[i * 4 + j], 0, 0, 0, 0, 0, 0);
-#pragma unroll
-        for (int f = 0; f < 4; ++f) {
-            int t = a[f][0];
-#pragma unroll
-            for (int i = 0; i < 7; ++i) a[f][i] = a[f][i + 1];
-            a[f][7] = t;
-            t = b[f][7];
-#pragma unroll
-            for (int i = 7; i > 0; --i) b[f][i] = b[f][i - 1];
-            b[f][0] = t;
-        }
+                acc[i * 4 + j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[s][i], b[s][j], acc[i * 4 + j], 0, 0, 0, 0, 0, 0);
+    };
+    int it = 0;
+    for (; it + 1 < iters; it += 2) {
+        step(std::integral_constant<int, 0>{});
+        step(std::integral_constant<int, 1>{});
     }
+    if (it < iters) step(std::integral_constant<int, 0>{});
     float sum = 0.0f;
 #pragma unroll
     for (int t = 0; t < 16; ++t)
@@ -130,8 +140,8 @@ __global__ __launch_bounds__(256, 1) void mfma_fp8_probe_kernel(float* sink, con
 extern "C" int lq_mfma_fp8_probe(float* sink, const uint8_t* operand_codes, size_t n_codes, int iters, int* workgroups,
                                  lq_stream_t stream) {
     LQ_REQUIRE(sink != nullptr && iters >= 1 && iters <= (1 << 20), LQ_ERR_ARG, "lq_mfma_fp8_probe: need a sink and 1..2^20 iterations");
-    LQ_REQUIRE(operand_codes == nullptr || (n_codes >= 4 && reinterpret_cast<uintptr_t>(operand_codes) % 4 == 0), LQ_ERR_ARG,
-               "lq_mfma_fp8_probe: operand codes must be 4-byte aligned and at least 4 bytes");
+    LQ_REQUIRE(operand_codes == nullptr || (n_codes >= 4096 && reinterpret_cast<uintptr_t>(operand_codes) % 4 == 0), LQ_ERR_ARG,
+               "lq_mfma_fp8_probe: operand codes must be 4-byte aligned and at least 4096 bytes");
     int dev = 0, cus = 0;
     LQ_REQUIRE(hipGetDevice(&dev) == hipSuccess &&
                    hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0,

@@ -99,6 +99,9 @@ SYMBOLS = {
     "lq_load_lora": (_I, [_P, _P, _I, _Z, _F, _P]),
     "lq_gemm_set_tactic": (_I, [_I, _I]),
     "lq_gemm_set_thread_tactic": (_I, [_I]),
+    "lq_gemm_tactics_serialized_size": (_Z, []),
+    "lq_gemm_tactics_serialize": (_I, [_P, _Z, _P]),
+    "lq_gemm_tactics_deserialize": (_I, [_P, _Z]),
     "lq_gemm_tactic_count": (_I, [_I]),
     "lq_gemm_set_shape_tactic": (_I, [_I, _I, _I, _I, _I]),
     "lq_gemm_get_shape_tactic": (_I, [_I, _I, _I, _I]),

@@ -711,6 +711,21 @@ class gemm_thread_tactic:
         return False
 
 
+def gemm_tactics_dumps() -> bytes:
+    """The per-shape tactic cache as bytes (GemmPluginProfiler::serialize, layers/gemm_utils/GemmProfiler.cc:26-38)."""
+    lib = _l.load()
+    size = int(lib.lq_gemm_tactics_serialized_size())
+    buf = C.create_string_buffer(size + 64)  # room for entries another thread adds in between
+    written = C.c_size_t(0)
+    _l.check(lib.lq_gemm_tactics_serialize(buf, size + 64, C.byref(written)), "lq_gemm_tactics_serialize")
+    return buf.raw[: written.value]
+
+
+def gemm_tactics_loads(data: bytes) -> None:
+    """Adds a table made by gemm_tactics_dumps to the cache (GemmPluginProfiler::deserialize, GemmProfiler.cc:40-65)."""
+    _l.check(_l.load().lq_gemm_tactics_deserialize(C.c_char_p(bytes(data)), len(data)), "lq_gemm_tactics_deserialize")
+
+
 def gemm_tactic_count(kind: str) -> int:
     return int(_l.load().lq_gemm_tactic_count(_KINDS[kind]))
 

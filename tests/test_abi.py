@@ -76,7 +76,7 @@ def test_shape_tactic_cache(lib):
     from lyradiff_amd import lib as L
 
     k8, k4 = L.LQ_W_INT8, L.LQ_W_INT4
-    assert lib.lq_gemm_tactic_count(k8) == 7 and lib.lq_gemm_tactic_count(L.LQ_W_FP8) == 7 and lib.lq_gemm_tactic_count(k4) == 3
+    assert lib.lq_gemm_tactic_count(k8) == 8 and lib.lq_gemm_tactic_count(L.LQ_W_FP8) == 8 and lib.lq_gemm_tactic_count(k4) == 3
     assert lib.lq_gemm_tactic_count(7) < 0
     assert lib.lq_gemm_get_shape_tactic(k8, 4096, 640, 2560) == -1
     assert lib.lq_gemm_set_shape_tactic(k8, 4096, 640, 2560, 2) == 0
@@ -94,3 +94,40 @@ def test_shape_tactic_cache(lib):
     assert lib.lq_gemm_profile_workspace(k8, 1024, 1280, 1280) >= 1024 * 1280 * 2 + 1024 * 1280 * 2
     assert lib.lq_gemm_profile(k8, 1024, 1280, 1280, None, 0, None, None, None) == -1
     assert b"workspace" in lib.lq_last_error()
+
+
+def test_tactic_cache_round_trips_through_bytes(lib):
+    """lq_gemm_tactics_serialize / deserialize (the reference's GemmPluginProfiler::serialize / deserialize,
+    layers/gemm_utils/GemmProfiler.cc:26-65): the table survives a round trip, a damaged or foreign table is refused whole."""
+    import struct
+
+    from lyradiff_amd import lib as L
+    from lyradiff_amd import ops
+
+    k8, kf = L.LQ_W_INT8, L.LQ_W_FP8
+    shapes = [(k8, 4608, 12288, 3072, 7), (kf, 4608, 3072, 12288, 6), (kf, 6912, 9216, 3072, 4)]
+    try:
+        for kind, m, n, k, t in shapes:
+            assert lib.lq_gemm_set_shape_tactic(kind, m, n, k, t) == 0
+        blob = ops.gemm_tactics_dumps()
+        assert blob[:4] == b"LQT1" and len(blob) == lib.lq_gemm_tactics_serialized_size() and (len(blob) - 8) % 20 == 0
+        count = struct.unpack("<i", blob[4:8])[0]
+        entries = {struct.unpack("<5i", blob[8 + 20 * i: 28 + 20 * i]) for i in range(count)}
+        assert set(shapes) <= entries
+        for kind, m, n, k, _ in shapes:
+            assert lib.lq_gemm_set_shape_tactic(kind, m, n, k, -1) == 0 and lib.lq_gemm_get_shape_tactic(kind, m, n, k) == -1
+        ops.gemm_tactics_loads(blob)
+        for kind, m, n, k, t in shapes:
+            assert lib.lq_gemm_get_shape_tactic(kind, m, n, k) == t
+        # refused: wrong magic, truncated, a tactic number the kind does not have, a bad kind; nothing of a refused table is kept
+        bad_tactic = blob[:8] + struct.pack("<5i", k8, 64, 64, 64, 99) + blob[28:]
+        bad_kind = blob[:8] + struct.pack("<5i", 42, 64, 64, 64, 0) + blob[28:]
+        for bad in (b"XXXX" + blob[4:], blob[:-4], bad_tactic, bad_kind, b""):
+            with pytest.raises(Exception):
+                ops.gemm_tactics_loads(bad)
+        assert lib.lq_gemm_get_shape_tactic(k8, 64, 64, 64) == -1
+        small = (C := __import__("ctypes")).create_string_buffer(4)
+        assert lib.lq_gemm_tactics_serialize(small, 4, None) == -1 and b"needed" in lib.lq_last_error()
+    finally:
+        for kind, m, n, k, _ in shapes:
+            lib.lq_gemm_set_shape_tactic(kind, m, n, k, -1)
