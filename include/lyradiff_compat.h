@@ -195,10 +195,13 @@ inline void invokeFusedQuantizeAndLoraDownSimple(float* Cptr, uint32_t* quantize
         throw std::runtime_error("[lyradiff Error][invokeFusedQuantizeAndLoraDownSimple] only group size 64 is supported");
     if ((Cptr == nullptr) != (Bptr == nullptr))
         throw std::runtime_error("[lyradiff Error][invokeFusedQuantizeAndLoraDownSimple] Cptr and Bptr go together");
-    detail::check(lq_w4a4_quantize(quantized_input, quantized_scale, LQ_F32, Aptr, LQ_BF16, Smoothptr, m, k, 64, stream),
-                  "invokeFusedQuantizeAndLoraDownSimple");
-    if (Bptr != nullptr)
-        detail::check(lq_lora_down(Cptr, LQ_F32, Aptr, Bptr, LQ_BF16, m, k, n, stream), "invokeFusedQuantizeAndLoraDownSimple");
+    if (Bptr != nullptr)  // one pass over A for both results, as in the reference
+        detail::check(lq_w4a4_quantize_lora_down(quantized_input, quantized_scale, LQ_F32, Cptr, LQ_F32, Aptr, LQ_BF16, Smoothptr,
+                                                 Bptr, m, k, n, 64, stream),
+                      "invokeFusedQuantizeAndLoraDownSimple");
+    else
+        detail::check(lq_w4a4_quantize(quantized_input, quantized_scale, LQ_F32, Aptr, LQ_BF16, Smoothptr, m, k, 64, stream),
+                      "invokeFusedQuantizeAndLoraDownSimple");
 }
 // utils/memory_utils.cu:398-402, the float -> T instantiations
 template <typename T_OUT>

@@ -435,13 +435,17 @@ public:
         const bool low_rank = weights->lora_up != nullptr && weights->lora_down != nullptr;
         LYRA_CHECK_WITH_INFO(!low_rank || weights->lora_rank() == lora_rank_, "W4A4Gemm: lora rank of layer and weights differ");
         allocateBuffer(m);
-        detail::check(lq_w4a4_quantize(quantized_input_buffer, input_scale_buffer, LQ_F32, input_tensor.getPtr<T>(),
-                                       detail::DType<T>::value, weights->smooth, (int)m, (int)k, (int)group_size_, stream_),
-                      "W4A4Gemm::forward quantize");
-        if (low_rank)  // down projection of the unsmoothed input, written as T directly (no fp32 detour)
-            detail::check(lq_lora_down(lora_down_res_buffer2, detail::DType<T>::value, input_tensor.getPtr<T>(), weights->lora_down,
-                                       detail::DType<T>::value, (int)m, (int)k, (int)lora_rank_, stream_),
-                          "W4A4Gemm::forward lora down");
+        if (low_rank)  // one pass over the input: quantised words and scales, and the down projection of the unsmoothed input
+                       // written as T directly (no fp32 detour)
+            detail::check(lq_w4a4_quantize_lora_down(quantized_input_buffer, input_scale_buffer, LQ_F32, lora_down_res_buffer2,
+                                                     detail::DType<T>::value, input_tensor.getPtr<T>(), detail::DType<T>::value,
+                                                     weights->smooth, weights->lora_down, (int)m, (int)k, (int)lora_rank_,
+                                                     (int)group_size_, stream_),
+                          "W4A4Gemm::forward quantize and lora down");
+        else
+            detail::check(lq_w4a4_quantize(quantized_input_buffer, input_scale_buffer, LQ_F32, input_tensor.getPtr<T>(),
+                                           detail::DType<T>::value, weights->smooth, (int)m, (int)k, (int)group_size_, stream_),
+                          "W4A4Gemm::forward quantize");
         detail::check(lq_gemm_w4a4_lora(output_tensor.getPtr<T>(), detail::DType<T>::value, quantized_input_buffer,
                                         reinterpret_cast<const uint8_t*>(weights->packed_weight), input_scale_buffer,
                                         weights->weight_scale, LQ_F32, has_bias_ ? weights->bias : nullptr,

@@ -413,6 +413,16 @@ int lq_gemm_w4a4_ex(void* C, lq_dtype_t out_dtype, const uint32_t* A_words, cons
 int lq_lora_down(void* out, lq_dtype_t out_dtype, const void* x, const void* lora_down, lq_dtype_t dtype,
                  int m, int k, int rank, lq_stream_t stream);
 
+/* Both halves of invokeFusedQuantizeAndLoraDownSimple (kernels/w4a4_gemm/w4a4_gemm.h:6-16; w4a4_gemm.cu:769-953) from ONE
+ * read of x, as the reference has it: q_words/scales exactly as lq_w4a4_quantize writes them (the same bits), lora_act
+ * [m, rank] = T_act( sum_k x[m,k] * lora_down[rank,k] ) as lq_lora_down defines it (fp32 accumulation in a fixed order; the
+ * order differs from lq_lora_down's, so the two agree to fp32 rounding of the sum, not bit for bit).
+ * One launch when x is F16/BF16, smooth is given, rank == 32, k % 128 == 0 and act_dtype is F32 or x_dtype; every other
+ * combination that the two separate entry points accept runs them one after the other inside this call. */
+int lq_w4a4_quantize_lora_down(uint32_t* q_words, void* scales, lq_dtype_t scale_dtype, void* lora_act,
+                               lq_dtype_t act_dtype, const void* x, lq_dtype_t x_dtype, const float* smooth,
+                               const void* lora_down, int m, int k, int rank, int group, lq_stream_t stream);
+
 /* dst[i] = T(src[i]), the float -> T copy between the reference's two W4A4 kernels
  * (invokeCudaD2DcpyConvert<T, float>, utils/memory_utils.cu:398-402). */
 int lq_cast_f32(void* dst, lq_dtype_t dst_dtype, const float* src, size_t n, lq_stream_t stream);

@@ -61,8 +61,10 @@ def load_flux_single_mlp_int4(src, prefix: str, dim: int, mlp_scale: int = 4, dt
 
 def _w4a4(lin: W4A4Linear, x2: torch.Tensor, **epilogue):
     """W4A4Gemm::forward (W4A4Gemm.cc:113-169) with epilogue options: quantise, low-rank down, GEMM."""
-    q, s = ops.w4a4_quant(x2, lin.smooth, torch.float32)
-    act = ops.lora_down(x2, lin.lora_down) if lin.lora_down is not None else None
+    if lin.lora_down is not None:
+        q, s, act = ops.w4a4_quant_lora_down(x2, lin.smooth, lin.lora_down, torch.float32)
+    else:
+        (q, s), act = ops.w4a4_quant(x2, lin.smooth, torch.float32), None
     return ops.w4a4_linear(q, lin.weight_rows32, s, lin.weight_scale, lin.bias, x2.dtype, 64, act,
                            lin.lora_up if act is not None else None, **epilogue)
 

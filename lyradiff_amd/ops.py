@@ -656,6 +656,27 @@ def lora_down(x, lora_down_w, out_dtype=None):
     return out
 
 
+def w4a4_quant_lora_down(x, smooth, lora_down_w, scale_dtype=torch.float32, out_dtype=None, group: int = 64):
+    """w4a4_quant and lora_down from one read of x (invokeFusedQuantizeAndLoraDownSimple, kernels/w4a4_gemm/w4a4_gemm.h:6-16):
+    returns (words int32 [M, K/8], scales [M, K/64], lora_act [M, R])."""
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    _chk(lora_down_w, "lora_down_w", (x.dtype,))
+    if smooth is not None:
+        _chk(smooth, "smooth", (torch.float32,))
+    m, k = x.shape
+    rank = lora_down_w.shape[0]
+    if lora_down_w.shape[1] != k:
+        raise ValueError("K mismatch between x and lora_down_w")
+    out_dtype = out_dtype or x.dtype
+    q = torch.empty((m, k // 8), dtype=torch.int32, device=x.device)
+    s = torch.empty((m, k // group), dtype=scale_dtype, device=x.device)
+    act = torch.empty((m, rank), dtype=out_dtype, device=x.device)
+    _l.check(_l.load().lq_w4a4_quantize_lora_down(_ptr(q), _ptr(s), _DT[scale_dtype], _ptr(act), _DT[out_dtype], _ptr(x),
+                                                  _DT[x.dtype], _ptr(smooth), _ptr(lora_down_w), m, k, rank, group, _stream()),
+             "lq_w4a4_quantize_lora_down")
+    return q, s, act
+
+
 def rmsnorm_rope(qkv, norm_qk, rope, heads: int, context_qkv=None, norm_added_qk=None, eps: float = 1e-6):
     """invokeFusedRmsNormCatAndRope / invokeFusedRmsNormAndRope: qkv [B, S, 3*H*Dh] (context_qkv [B, Sc, 3*H*Dh], text tokens,
     placed first) -> [B, Sc + S, 3, H, Dh] with q and k RMS-normalised per head, scaled by norm_qk / norm_added_qk ([2*Dh]: q

@@ -179,10 +179,10 @@ struct W4A4Linear {
         const int64_t m = x2.size(0);
         const at::ScalarType T = x2.scalar_type();
         at::Tensor q = at::empty({m, k / 8}, on_gpu(at::kInt)), s = at::empty({m, k / 64}, on_gpu(at::kFloat));
-        ok(lq_w4a4_quantize(static_cast<uint32_t*>(P(q)), P(s), LQ_F32, P(x2), lq_dt(T), PF(smooth), (int)m, (int)k, 64, cur_stream()),
-           "lq_w4a4_quantize");
         at::Tensor act = at::empty({m, rank}, on_gpu(T));
-        ok(lq_lora_down(P(act), lq_dt(T), P(x2), P(lora_down), lq_dt(T), (int)m, (int)k, (int)rank, cur_stream()), "lq_lora_down");
+        ok(lq_w4a4_quantize_lora_down(static_cast<uint32_t*>(P(q)), P(s), LQ_F32, P(act), lq_dt(T), P(x2), lq_dt(T), PF(smooth),
+                                      P(lora_down), (int)m, (int)k, (int)rank, 64, cur_stream()),
+           "lq_w4a4_quantize_lora_down");
         at::Tensor y;
         if (want_output) y = at::empty({m, n}, on_gpu(T));
         ok(lq_gemm_w4a4_ex(P(y), lq_dt(T), static_cast<const uint32_t*>(P(q)), P8(w_rows32), P(s), P(w_scale), LQ_F32, P(bias), P(act),

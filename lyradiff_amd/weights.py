@@ -158,8 +158,10 @@ class W4A4Linear:
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         k = x.shape[-1]
         x2 = x.reshape(-1, k)
-        q, s = ops.w4a4_quant(x2, self.smooth, torch.float32)
-        act = ops.lora_down(x2, self.lora_down) if self.lora_down is not None else None
+        if self.lora_down is not None:
+            q, s, act = ops.w4a4_quant_lora_down(x2, self.smooth, self.lora_down, torch.float32)
+        else:
+            (q, s), act = ops.w4a4_quant(x2, self.smooth, torch.float32), None
         y = ops.w4a4_linear(q, self.weight_rows32, s, self.weight_scale, self.bias, x.dtype, 64, act,
                             self.lora_up if act is not None else None)
         return y.reshape(*x.shape[:-1], y.shape[-1])

@@ -382,6 +382,50 @@ def test_lora_down(ops, dev, dt, m, k, rank):
     assert torch.equal(ops.lora_down(x.to(dev), down.to(dev)), y), "no atomics: repeated calls agree bit for bit"
 
 
+# One pass over x for both halves of invokeFusedQuantizeAndLoraDownSimple (kernels/w4a4_gemm/w4a4_gemm.h:6-16): words and scales are
+# the bits of the stand-alone quantiser (and so of the oracle), the low-rank result meets the stand-alone kernel's error bound.
+# Rows per workgroup follow m: 4 (m = 5, 70, 300), 18 (4608), 27 (6912), 32 with a ragged last workgroup (9000); k = 128 gives
+# seven of the eight wavefronts no slice at all, k = 1152 an uneven share; the last two cases take the two-kernel route inside the
+# call (rank 64; k not a multiple of 128).
+@pytest.mark.parametrize("dt,sdt", [("bf16", "f32"), ("f16", "f32"), ("bf16", "f16")])
+@pytest.mark.parametrize("m,k,rank", [(300, 3072, 32), (4608, 3072, 32), (70, 128, 32), (5, 1152, 32), (6912, 3072, 32), (9000, 1024, 32),
+                                      (1024, 12288, 32), (70, 256, 64), (33, 192, 32)])
+def test_w4a4_quant_and_lora_down_in_one_pass(ops, dev, dt, sdt, m, k, rank):
+    g = rng_t(m + k + rank + 1)
+    x = (torch.randn(m, k, generator=g) * (1.0 + 4.0 * torch.rand(m, 1, generator=g))).to(TORCH_DT[dt])
+    x[m // 2, : min(k, 192)] = 0  # all-zero groups
+    smooth = (0.25 + 2.0 * torch.rand(k, generator=g)).float()
+    down = (torch.randn(rank, k, generator=g) * 0.05).to(TORCH_DT[dt])
+    sdtype = torch.float32 if sdt == "f32" else torch.float16
+    xd, sd, dd = x.to(dev), smooth.to(dev), down.to(dev)
+    q, s, act32 = ops.w4a4_quant_lora_down(xd, sd, dd, sdtype, torch.float32)
+    q0, s0 = ops.w4a4_quant(xd, sd, sdtype)
+    assert torch.equal(q, q0) and torch.equal(s.view(torch.int16 if sdt == "f16" else torch.int32),
+                                              s0.view(torch.int16 if sdt == "f16" else torch.int32)), "words and scales: the stand-alone quantiser's bits"
+    if m * k <= 300 * 3072:  # and the oracle's, where it finishes quickly
+        qo, so = O.w4a4_quant(to_np_f32(x), smooth.numpy(), 64, sdt)
+        assert np.array_equal(q.cpu().numpy().view(np.uint32), qo)
+        assert np.array_equal(s.float().cpu().numpy(), so.astype(np.float32))
+    ref = O.lora_down_f64(to_np_f32(x), to_np_f32(down))
+    mag = np.abs(to_np_f32(x)).astype(np.float64) @ np.abs(to_np_f32(down)).astype(np.float64).T
+    assert np.all(np.abs(act32.cpu().numpy() - ref) <= 2.0 ** -20 * mag + 1e-30), "fp32 accumulation error beyond a few ULP of the term magnitudes"
+    q1, s1, act = ops.w4a4_quant_lora_down(xd, sd, dd, sdtype)
+    assert act.dtype == x.dtype and torch.equal(q1, q0)
+    assert_close_tol(to_np_f32(act), O.round_to(ref.astype(np.float32), dt), "low-rank result", abs_floor=2.0 ** -20 * mag)
+    q2, s2, act2 = ops.w4a4_quant_lora_down(xd, sd, dd, sdtype)
+    assert torch.equal(act2, act) and torch.equal(q2, q1) and torch.equal(s2, s1), "no atomics: repeated calls agree bit for bit"
+
+
+def test_w4a4_quant_and_lora_down_argument_checks(ops, dev):
+    x = torch.zeros(8, 128, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(ValueError):
+        ops.w4a4_quant_lora_down(x, None, torch.zeros(32, 64, dtype=torch.bfloat16, device=dev))
+    with pytest.raises(RuntimeError):  # rank 16: neither route takes it
+        ops.w4a4_quant_lora_down(x, None, torch.zeros(16, 128, dtype=torch.bfloat16, device=dev))
+    q, s, act = ops.w4a4_quant_lora_down(x[:0], None, torch.zeros(32, 128, dtype=torch.bfloat16, device=dev))
+    assert q.shape == (0, 16) and act.shape == (0, 32)
+
+
 @pytest.mark.parametrize("sdt", ["f32", "f16"])
 @pytest.mark.parametrize("m,n,k,rank,tactic", [(333, 416, 640, 32, 0), (333, 416, 640, 32, 1), (333, 416, 640, 16, 2), (512, 3072, 3072, 32, -1)])
 def test_w4a4_gemm_with_low_rank_branch(ops, dev, sdt, m, n, k, rank, tactic, tactic_guard):
