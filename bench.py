@@ -7,9 +7,13 @@ One "step" is one pass of the FLUX DiT MLP FP8 chain over one batch of synthetic
 (BASELINE.json configs[2], M=4608 tokens = 4096 image + 512 text at 1024^2):
 
     x bf16 [4608,3072]  --fp8 amax+cast-->  e4m3
-        --FP8 GEMM 3072->12288, bias + tanh-GELU fused, bf16 out-->  h [4608,12288]
-    h --fp8 cast with the dynamic scale max|h|/448 that the first GEMM's epilogue accumulated--> e4m3
+        --FP8 GEMM 3072->12288, bias fused, bf16 out, the largest output left beside it-->  u [4608,12288]
+    u --tanh-GELU, dynamic scale max|h|/448 (from the largest output: GELU is monotone there) and e4m3 cast, one pass--> e4m3
       --FP8 GEMM 12288->3072, bias, bf16 out-->  y [4608,3072]
+
+(The activation sits in the memory-bound cast pass, where the vector ALU is idle, instead of the GEMM's epilogue, where it
+costs 19-26 us: the GEMM then runs as the persistent one-wavefront-per-SIMD kernel.  `kernels` also times the up projection
+with bias + GELU + output maximum in its epilogue, the form this chain used before.)
 
 Inputs and (pre-quantised, rows32-repacked) weights are resident in HBM before the timed region.
 `value` is the GEMM work of the step (2*M*N*K summed over both GEMMs) divided by the wall time of
@@ -70,8 +74,8 @@ def cpu_baseline(torch, x, w_up, w_dn, b_up, b_dn, rows):
     t0 = time.perf_counter()
     qa, sa = O.fp8_amax_cast(xs)
     a = torch.from_numpy(O.e4m3_decode(qa))
-    h = (a @ wu.t()) * float(np.float32(sa) * np.float32(swu)) + b_up.float()
-    h = torch.nn.functional.gelu(h, approximate="tanh").to(torch.bfloat16)
+    h = ((a @ wu.t()) * float(np.float32(sa) * np.float32(swu)) + b_up.float()).to(torch.bfloat16)  # the GEMM stores bf16
+    h = torch.nn.functional.gelu(h.float(), approximate="tanh").to(torch.bfloat16)
     qh, sh = O.fp8_amax_cast(h.float().numpy())
     hh = torch.from_numpy(O.e4m3_decode(qh))
     y = ((hh @ wd.t()) * float(np.float32(sh) * np.float32(swd)) + b_dn.float()).to(torch.bfloat16)
@@ -154,18 +158,19 @@ def main():
         qx, sx = ops.fp8_quant(xi)
         if record == 0:
             e[1].record()
-        # the up projection's epilogue also accumulates max|h|/448, the dynamic scale of h, so the quantisation
-        # of h is a single cast pass (the same numbers as an amax pass over h followed by the cast)
-        sh = s_h[i % 2]
-        sh.zero_()
+        # the up projection's epilogue also leaves its largest output, from which the next pass derives max|gelu(u)|/448,
+        # the dynamic scale of h: activation and quantisation are a single pass (the same numbers as GELU, an amax pass over
+        # h and the cast)
+        um = s_h[i % 2]
+        um.zero_()
         if record == 1:
             e[0].record()
-        h = ops.fp8_linear(qx, wp_up, sx, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh)
+        u = ops.fp8_linear_max(qx, wp_up, sx, s_up, bu, um, torch.bfloat16)
         if record == 1:
             e[1].record()
         if record == 2:
             e[0].record()
-        qh = ops.fp8_scale_cast(h, sh)
+        qh, sh = ops.fp8_gelu_quant(u, um)
         if record == 2:
             e[1].record()
         if record == 3:
@@ -241,20 +246,23 @@ def main():
         return a.elapsed_time(b) / n * 1e3
 
     qx0, sx0 = ops.fp8_quant(xs[0])
-    sh0 = torch.zeros(1, dtype=torch.float32, device=dev)
-    h0 = ops.fp8_linear(qx0, wp_up, sx0, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh0)
-    qh0 = ops.fp8_scale_cast(h0, sh0)
+    um0 = torch.zeros(1, dtype=torch.float32, device=dev)
+    u0 = ops.fp8_linear_max(qx0, wp_up, sx0, s_up, bu, um0, torch.bfloat16)
+    qh0, sh0 = ops.fp8_gelu_quant(u0, um0)
     alone = {
         "quant_x": batched(lambda i: ops.fp8_quant(xs[i % n_rot])),
-        "gemm_up": batched(lambda i: ops.fp8_linear(qx0, wp_up, sx0, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh0)),
-        "quant_h": batched(lambda i: ops.fp8_scale_cast(h0, sh0)),
+        "gemm_up": batched(lambda i: ops.fp8_linear_max(qx0, wp_up, sx0, s_up, bu, um0, torch.bfloat16)),
+        "quant_h": batched(lambda i: ops.fp8_gelu_quant(u0, um0)),
         "gemm_down": batched(lambda i: ops.fp8_linear(qh0, wp_dn, sh0, s_dn, bd, False, None, 0.0, torch.bfloat16)),
     }
+    # the up projection with the activation and the output maximum in its epilogue (not part of the timed chain)
+    sg0 = torch.zeros(1, dtype=torch.float32, device=dev)
+    up_gelu_us = batched(lambda i: ops.fp8_linear(qx0, wp_up, sx0, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sg0))
     # the power argument, checkable from this line: the SAME up-projection kernel on all-zero operands (no switching in
     # the matrix pipe, so the clock is not pulled down), and the shader clock a probe on a second stream sees while the
     # kernel runs on random and on zero operands (idle clock for reference)
     zq, zw = torch.zeros_like(qx0), torch.zeros_like(wp_up)
-    zeros_us = batched(lambda i: ops.fp8_linear(zq, zw, sx0, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh0))
+    zeros_us = batched(lambda i: ops.fp8_linear_max(zq, zw, sx0, s_up, bu, um0, torch.bfloat16))
 
     def clock_under(fn, per_launch_us=None, n=6):
         side = torch.cuda.Stream()
@@ -295,8 +303,8 @@ def main():
     pipe_only["zero_operands"]["shader_clock_ghz"] = clock_under(lambda i: ops.mfma_fp8_probe(None, 1000), pipe_only["zero_operands"]["us"])
     clocks = {
         "idle": clock_under(lambda i: None),
-        "up_gemm_random_operands": clock_under(lambda i: ops.fp8_linear(qx0, wp_up, sx0, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh0)),
-        "up_gemm_zero_operands": clock_under(lambda i: ops.fp8_linear(zq, zw, sx0, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sh0)),
+        "up_gemm_random_operands": clock_under(lambda i: ops.fp8_linear_max(qx0, wp_up, sx0, s_up, bu, um0, torch.bfloat16)),
+        "up_gemm_zero_operands": clock_under(lambda i: ops.fp8_linear_max(zq, zw, sx0, s_up, bu, um0, torch.bfloat16)),
     }
     if vendor is not None:
         w8 = ops.unpack_weight(wp_up).view(torch.float8_e4m3fn)
@@ -320,13 +328,16 @@ def main():
                                           "TFLOP/s": round(gemm_flops / alone["gemm_down"] / 1e6, 1)},
         "fp8_amax_cast_4608x3072": {"us_in_step_incl_launch_gap": round(per["quant_x"], 2), "us_back_to_back": round(alone["quant_x"], 2),
                                     "GB/s": round(3.0 * M * D / alone["quant_x"] / 1e3, 1)},
-        "fp8_cast_with_gemm_scale_4608x12288": {"us_in_step_incl_launch_gap": round(per["quant_h"], 2), "us_back_to_back": round(alone["quant_h"], 2),
-                                                "GB/s": round(3.0 * M * H / alone["quant_h"] / 1e3, 1)},
+        "fp8_gelu_cast_with_gemm_max_4608x12288": {"us_in_step_incl_launch_gap": round(per["quant_h"], 2), "us_back_to_back": round(alone["quant_h"], 2),
+                                                   "GB/s": round(3.0 * M * H / alone["quant_h"] / 1e3, 1)},
+        "gemm_up_fp8_with_gelu_and_amax_epilogue_4608x12288x3072": {"us_back_to_back": round(up_gelu_us, 2),
+                                                                    "TFLOP/s": round(gemm_flops / up_gelu_us / 1e6, 1),
+                                                                    "note": "not in the timed chain: the activation in the GEMM's epilogue"},
     }
     kernels.update(other)
     achieved = gemm_flops / per["gemm_up"] / 1e6
     traffic, traffic_src = profiled_traffic()
-    roofline = {"bound": "mfma", "kernel": "lq::gemm_kernel<fp8> 4608x12288x3072 (bias+GELU, bf16 out)",
+    roofline = {"bound": "mfma", "kernel": "lq::gemm_persist_kernel<fp8> 4608x12288x3072 (bias, running maximum, bf16 out)",
                 "achieved": round(achieved, 1), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / FP8_PEAK_TFLOPS, 4),
                 "timing": f"a pair of HIP events around the kernel on {len(marks['gemm_up'])} of the {args.steps} timed steps, on the launch stream",
@@ -353,8 +364,8 @@ def main():
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp8_e4m3", "data": "synthetic",
-        "config": {"workload": "FLUX DiT MLP FP8 e4m3 per-tensor, M=4608: act-quant -> GEMM 3072->12288 (+bias, GELU) "
-                               "-> act-quant -> GEMM 12288->3072 (+bias), bf16 in/out (BASELINE.json configs[2])",
+        "config": {"workload": "FLUX DiT MLP FP8 e4m3 per-tensor, M=4608: act-quant -> GEMM 3072->12288 (+bias) "
+                               "-> GELU + act-quant -> GEMM 12288->3072 (+bias), bf16 in/out (BASELINE.json configs[2])",
                    "tokens": M, "d_model": D, "d_ff": H, "profiled_tactics": tactics,
                    "settle_steps_before_warmup": settled_after, "settle_ms": round(settle_ms, 1)},
         "roofline": roofline, "kernels": kernels,
@@ -370,8 +381,9 @@ def main():
         # by the GELU flavour of the fused epilogue and by bf16/e4m3 rounding flips, so a loose bound)
         xr = xd[: args.cpu_rows].contiguous()
         qx, sx = ops.fp8_quant(xr)
-        hg = ops.fp8_linear(qx, wp_up, sx, s_up, bu, True, None, 0.0, torch.bfloat16)
-        qh, sh = ops.fp8_quant(hg)  # the two-pass form; the timed chain's fused scale is checked equal in tests/
+        ug = ops.fp8_linear(qx, wp_up, sx, s_up, bu, False, None, 0.0, torch.bfloat16)
+        um = ug.float().max().clamp(min=0).reshape(1)
+        qh, sh = ops.fp8_gelu_quant(ug, um)  # the scale is checked equal to an amax pass over gelu(u) in tests/
         y_gpu = ops.fp8_linear(qh, wp_dn, sh, s_dn, bd, False, None, 0.0, torch.bfloat16).float().cpu()
         out["cpu_gpu_max_abs_diff"] = round((y_gpu - y_cpu.float()).abs().max().item(), 4)
     if args.extra:
@@ -667,7 +679,7 @@ def flux_linear_chain_1280(torch, ops, dev, timeit):
     """BASELINE.json configs[4]: the FP8 linears of a FLUX double-stream block at 1280x1280 (M = 6912 tokens), each preceded
     by the fused amax + cast of its bf16 input: QKV 3072->9216, out-proj 3072->3072, MLP 3072->12288 (GELU) ->3072.  The
     four linears run on independent synthetic inputs of the right shapes (the attention between them is not part of the
-    path); the MLP pair is chained through the GEMM-epilogue scale as in the headline step."""
+    path); the MLP pair is chained through the up projection's largest output as in the headline step."""
     m, d = 6912, 3072
     g = torch.Generator().manual_seed(1005)
     lin = {}
@@ -684,8 +696,9 @@ def flux_linear_chain_1280(torch, ops, dev, timeit):
             ops.fp8_linear(q, lin[name][0], s, lin[name][1], lin[name][2])
         q, s = ops.fp8_quant(xs[2])
         sh.zero_()
-        h = ops.fp8_linear(q, lin["up"][0], s, lin["up"][1], lin["up"][2], True, None, 0.0, torch.bfloat16, out_scale=sh)
-        return ops.fp8_linear(ops.fp8_scale_cast(h, sh), lin["down"][0], sh, lin["down"][1], lin["down"][2])
+        u = ops.fp8_linear_max(q, lin["up"][0], s, lin["up"][1], lin["up"][2], sh, torch.bfloat16)
+        qh, s2 = ops.fp8_gelu_quant(u, sh)
+        return ops.fp8_linear(qh, lin["down"][0], s2, lin["down"][1], lin["down"][2])
 
     us = timeit(chain, iters=20, warm=3)
     flop = 2.0 * m * d * (3 * d + d + 4 * d + 4 * d)

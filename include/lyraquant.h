@@ -237,6 +237,25 @@ int lq_gemm_fp8_ex(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_
                    const void* residual, float beta, int m, int n, int k,
                    float* out_scale, uint8_t* C_fp8, const float* C_fp8_scale, lq_stream_t stream);
 
+/* lq_gemm_fp8 without activation or residual that also joins the largest output into out_max[0]:
+ *   out_max[0] = max( out_max[0], max_{m,n} f32(C[m,n]), 0 )      (the caller zeroes it; a float >= 0)
+ * for lq_fp8_gelu_cast below, which derives the dynamic e4m3 scale of gelu(C) from it without a pass over C.  With 256-row
+ * and 256-column multiples and k % 128 == 0 this runs the persistent one-wavefront-per-SIMD kernel (the maximum costs its
+ * epilogue two instructions per four outputs, where an activation in the epilogue would cost it 13-18 us per tile). */
+int lq_gemm_fp8_max(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32, const float* a_scale,
+                    const float* b_scale, const void* bias, int m, int n, int k, float* out_max, lq_stream_t stream);
+
+/* Activation and dynamic FP8 quantisation of a stored GEMM output y [n elements] in one pass:
+ *   h = T(gelu_tanh(y))   (invokeFusedBiasAndGelu on a stored T tensor, kernels/flux_single_transformer_block/
+ *                          flux_single_transformer_kernels.cu:122-141, 194-201; the same arithmetic as gelu == 2 above)
+ *   scale_out[0] = max|h| / 448,  dst = e4m3( h * (1 / scale_out[0]) ),  h_out (optional, T) = h
+ * src_max[0] >= max(y, 0) exactly (lq_gemm_fp8_max leaves it): T(gelu(.)) is non-decreasing from 0 up, so max|h| =
+ * h(src_max) whenever src_max >= 0.5 -- the result is then bit for bit that of lq_fp8_amax_cast on h.  A tensor without a
+ * single value of 0.5 or more takes max(h(src_max), 0.171875) for max|h|: an upper bound (no |gelu| of a negative number
+ * exceeds 0.17), not the exact maximum. */
+int lq_fp8_gelu_cast(uint8_t* dst, float* scale_out, void* h_out, const void* src, lq_dtype_t dtype, size_t n,
+                     const float* src_max, lq_stream_t stream);
+
 /* lq_gemm_fp8 (no activation) whose epilogue applies FLUX's gate and second residual:
  *   C[m,n] = T( T( T(y[m,n]) * gate[m / rows_per_gate, n] ) + residual[m,n] ),  y = (sa*sb)*acc + bias[n]
  * with every rounding of the reference's sequence "GEMM stores T, then multiply and add in T": it replaces

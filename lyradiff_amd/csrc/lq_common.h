@@ -350,6 +350,16 @@ __device__ __forceinline__ float gelu_tanh(float x) {
     return x * (0.5f * (1.0f + tanh_basic(inner)));
 }
 
+// GELU for the fused FP8 epilogue: hardware exp2 / reciprocal (the reference's counterpart is
+// cuBLASLt's GELU epilogue, utils/cublasMMWrapper.cc:1195-1199, whose arithmetic is not visible).
+__device__ __forceinline__ float gelu_fast(float x) {
+    // 0.5 x (1 + tanh(u)) = x / (1 + exp(-2u)),  u = sqrt(2/pi) (x + 0.044715 x^3);  -2u log2(e) = x (A + B x^2)
+    constexpr float A = -2.0f * 0.7978845608028654f * 1.4426950408889634f, B = A * 0.044715f;
+    const float t = x * (A + B * (x * x));
+    const float e = __builtin_amdgcn_exp2f(t);             // exp(-2u): 0 for large x, inf for very negative x
+    return x * __builtin_amdgcn_rcpf(1.0f + e);            // x, resp. -0
+}
+
 static inline hipStream_t as_stream(lq_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 }  // namespace lq

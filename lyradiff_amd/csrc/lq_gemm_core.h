@@ -47,6 +47,8 @@ struct GemmParams {
     const void* residual;
     float beta;
     float* out_scale;       // optional: max(out_scale, max|C| / 448), the e4m3 scale of the output for a following cast
+    float* out_max;         // optional: max(out_max, max over T(C), 0): the largest output, for an activation + cast pass that
+                            // derives its scale from it (non-negative floats order like their bit patterns)
     uint8_t* C8;            // optional: e4m3 codes of C with a given (static) scale, written next to or instead of C
     const float* c8_scale;  // scale of C8: C8 = e4m3(f32(T(y)) * (1 / c8_scale[0]))
     size_t ldc8;            // row pitch of C8 in bytes (n when the codes are dense)
@@ -151,14 +153,14 @@ template <> struct OutStore<F32Tag> {
 };
 struct I32Tag {};
 
-// GELU for the fused FP8 epilogue: hardware exp2 / reciprocal (the reference's counterpart is
-// cuBLASLt's GELU epilogue, utils/cublasMMWrapper.cc:1195-1199, whose arithmetic is not visible).
-__device__ __forceinline__ float gelu_fast(float x) {
-    // 0.5 x (1 + tanh(u)) = x / (1 + exp(-2u)),  u = sqrt(2/pi) (x + 0.044715 x^3);  -2u log2(e) = x (A + B x^2)
-    constexpr float A = -2.0f * 0.7978845608028654f * 1.4426950408889634f, B = A * 0.044715f;
-    const float t = x * (A + B * (x * x));
-    const float e = __builtin_amdgcn_exp2f(t);             // exp(-2u): 0 for large x, inf for very negative x
-    return x * __builtin_amdgcn_rcpf(1.0f + e);            // x, resp. -0
+// The wavefront's largest output (>= 0) joins the running maximum of the call.  Rounding to T is monotone, so the maximum
+// of the rounded outputs is the rounded maximum.
+template <typename OutTag> __device__ __forceinline__ void publish_out_max(float* out_max, float wave_part, int lane) {
+    const float mx = round_through<OutTag>(wave_max(wave_part));
+    if (lane == 0) {
+        const int cur = __hip_atomic_load(reinterpret_cast<int*>(out_max), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (__float_as_int(mx) > cur) atomicMax(reinterpret_cast<int*>(out_max), __float_as_int(mx));
+    }
 }
 
 // Four floats -> four e4m3 codes, round-to-nearest-even, saturating to +-448, NaN -> 0x7F | sign (the cast kernel's rule).
@@ -639,7 +641,7 @@ struct GemmKernel {
         const int out_row = lane / LPR, out_n = n0 + wn * TN + (lane % LPR) * 4;
         const bool n_ok = out_n < p.n;
         float alpha = 1.0f, bias4[4] = {0.f, 0.f, 0.f, 0.f}, acol4[4] = {0.f, 0.f, 0.f, 0.f}, arow_l[MT];
-        float out_amax = 0.0f, c8_inv = 0.0f, gate4[4] = {0.f, 0.f, 0.f, 0.f};
+        float out_amax = 0.0f, out_pmax = 0.0f, c8_inv = 0.0f, gate4[4] = {0.f, 0.f, 0.f, 0.f};
         bool gate_uniform = true;  // every row of the wavefront's tile uses the same gate vector
         // the FP8 and W4A4 linears of the FLUX blocks share the activation / re-quantisation / gate epilogues
         constexpr bool kExtras = (KIND == K_FP8 || W4) && !kI32;
@@ -677,7 +679,7 @@ struct GemmKernel {
         int emode = kExtras ? E_GENERAL : E_PLAIN;
         if constexpr (kSpecialise) {
             const bool join = p.addend != nullptr || p.residual != nullptr || p.gate != nullptr;
-            if (!join && p.C8 == nullptr && p.C != nullptr) emode = (p.gelu != 0 || p.out_scale != nullptr) ? E_ACT : E_PLAIN;
+            if (!join && p.C8 == nullptr && p.C != nullptr) emode = (p.gelu != 0 || p.out_scale != nullptr || p.out_max != nullptr) ? E_ACT : E_PLAIN;
             else if (!join && p.C8 != nullptr && p.C == nullptr && p.out_scale == nullptr) emode = E_CODES;
             else if (p.gate != nullptr && p.residual != nullptr && p.addend == nullptr && p.C8 == nullptr && p.C != nullptr &&
                      p.gelu == 0 && p.out_scale == nullptr) emode = E_GATED;
@@ -762,6 +764,7 @@ struct GemmKernel {
                         if constexpr (kExtras && (MODE == E_ACT || GEN)) {
                             if (ok && p.out_scale != nullptr)
                                 out_amax = fmaxf(fmaxf(out_amax, fmaxf(fabsf(y[0]), fabsf(y[1]))), fmaxf(fabsf(y[2]), fabsf(y[3])));
+                            if (ok && p.out_max != nullptr) out_pmax = fmaxf(fmaxf(out_pmax, fmaxf(y[0], y[1])), fmaxf(y[2], y[3]));
                         }
                         if constexpr (kExtras && (MODE == E_CODES || GEN)) {
                             if (ok && (MODE == E_CODES || p.C8 != nullptr)) {  // the codes the cast kernel would produce from the T-rounded output
@@ -851,6 +854,7 @@ struct GemmKernel {
                     if (__float_as_int(sc) > cur) atomicMax(reinterpret_cast<int*>(p.out_scale), __float_as_int(sc));
                 }
             }
+            if (p.out_max != nullptr) publish_out_max<OutTag>(p.out_max, out_pmax, lane);
         }
     }
 };

@@ -13,6 +13,7 @@ template <typename OutTag> static constexpr lq_dtype_t out_enum() {
 
 template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
     int t = requested_tactic(g_tactic_fp8, LQ_W_FP8, p.m, p.n, p.k);
+    // scales and bias, and at most the running maximum of the outputs (two instructions per four outputs)
     const bool plain_epilogue = p.gelu == 0 && p.out_scale == nullptr && p.C8 == nullptr && p.gate == nullptr &&
                                 p.residual == nullptr && p.addend == nullptr;
     if (t < 0) {
@@ -39,6 +40,7 @@ template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
     // 153-160 us with tactic 4; 3072x12288 with gate and residual 139 us against 134 us with tactic 0, 3072x3072 55 against
     // 48 us.  A configuration forced by the caller is kept.
     const bool forced = tl_forced_tactic >= 0 || g_tactic_fp8 >= 0;
+    if (t == 6 && !forced && p.out_max != nullptr) t = (long)((p.m + 255) / 256) * ((p.n + 255) / 256) > 256 ? 4 : 0;  // outside the persistent form the running maximum takes the activation epilogue
     if ((t == 6 || t == 7) && !forced && !plain_epilogue) t = (long)((p.m + 255) / 256) * ((p.n + 255) / 256) > 256 ? 4 : 0;
     if (t == 7) {  // the persistent form of tactic 6 where it applies, tactic 6 itself elsewhere
         const int rc = launch_persist_fp8(p, out_enum<OutTag>(), st);
@@ -104,6 +106,21 @@ extern "C" int lq_gemm_fp8_ex(void* C, lq_dtype_t out_dtype, const uint8_t* A, c
     // with out_scale the 16-bit output exists to be cast once with that scale; a large one bypasses the cache on its way out
     p.stream_c = out_scale != nullptr && C != nullptr && (size_t)m * (size_t)n * (out_dtype == LQ_F32 ? 4 : 2) >= kStreamBytes;
     return fp8_dispatch("lq_gemm_fp8", p, out_dtype, stream);
+}
+
+extern "C" int lq_gemm_fp8_max(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32, const float* a_scale,
+                               const float* b_scale, const void* bias, int m, int n, int k, float* out_max, lq_stream_t stream) {
+    int rc = fp8_check("lq_gemm_fp8_max", C, A, B_rows32, a_scale, b_scale, bias, nullptr, m, n, k);
+    if (rc != LQ_OK) return rc > 0 ? LQ_OK : rc;
+    LQ_REQUIRE(C && out_max, LQ_ERR_ARG, "lq_gemm_fp8_max: null pointer");
+    GemmParams p = {};
+    p.C = C; p.A = A; p.B = B_rows32; p.bias = bias; p.a_scale = a_scale; p.b_scale = b_scale;
+    p.out_max = out_max; p.ldc8 = (size_t)n;
+    p.m = m; p.n = n; p.k = k; p.kb = k;
+    // the output exists to be read once by the activation + cast pass; a large one bypasses the cache on its way out (the
+    // two-workgroups-per-CU kernels only: the persistent kernel's counted waits do not get along with such stores)
+    p.stream_c = (size_t)m * (size_t)n * (out_dtype == LQ_F32 ? 4 : 2) >= kStreamBytes;
+    return fp8_dispatch("lq_gemm_fp8_max", p, out_dtype, stream);
 }
 
 extern "C" int lq_gemm_fp8(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32,

@@ -30,7 +30,8 @@ namespace lq {
 // 148 us with the plain epilogue -- so such calls stay with the two-workgroups-per-CU configuration.
 // MT: 32-row MFMA blocks per wavefront along M: 4 = 256x256 tiles, 2 = 128x256 tiles (the halves of the leftover tiles, see
 // launch_gemm_persist).
-template <int KIND, typename OutTag, int MT>
+// TRACK (FP8): the largest output joins p.out_max.
+template <int KIND, typename OutTag, int MT, bool TRACK = false>
 struct GemmPersist {
     static_assert(KIND == K_FP8 || KIND == K_INT8, "INT8 and FP8 only");
     static_assert(MT == 4 || MT == 2, "256- or 128-row tiles");
@@ -212,6 +213,7 @@ struct GemmPersist {
         float alpha = 1.0f;
         if constexpr (KIND == K_FP8) alpha = p.a_scale[0] * p.b_scale[0];
         const bool has_bias = p.bias != nullptr;
+        float out_pmax = 0.0f;  // TRACK: the largest output this lane has stored
         auto epilogue = [&](int tj) {
             int m0, n0;
             tile_origin(tj, m0, n0);
@@ -276,6 +278,10 @@ struct GemmPersist {
                                 else y[e] = __int_as_float(raw[u][e]) * alpha;
                                 if (has_bias) y[e] = y[e] + bias4[hj][e];
                             }
+                            // (plain stores also for an output that is read only once: nontemporal ones are acknowledged so
+                            // much later that the counted waits behind them stall the operand stream -- 4608x12288x3072: 184-195
+                            // against 140 us)
+                            if constexpr (TRACK) out_pmax = fmaxf(fmaxf(out_pmax, fmaxf(y[0], y[1])), fmaxf(y[2], y[3]));
                             OutStore<OutTag>::store4(p.C, idx, y);
                         }
                     }
@@ -343,31 +349,34 @@ struct GemmPersist {
         }
         wait_vmcnt<0>();  // the transfers past the end have landed before the LDS is reused or given back
         __syncthreads();
+        if constexpr (TRACK) publish_out_max<OutTag>(p.out_max, out_pmax, lane);
     }
 };
 
-template <int KIND, typename OutTag>
+template <int KIND, typename OutTag, bool TRACK>
 __global__ __launch_bounds__(256, 1) void gemm_persist_kernel(GemmParams p) {
     extern __shared__ __attribute__((aligned(16))) char lq_smem[];
-    GemmPersist<KIND, OutTag, 4>::run(p, lq_smem, 0);
-    if (p.persist_halves > 0) GemmPersist<KIND, OutTag, 2>::run(p, lq_smem, 1);
+    GemmPersist<KIND, OutTag, 4, TRACK>::run(p, lq_smem, 0);
+    if (p.persist_halves > 0) GemmPersist<KIND, OutTag, 2, TRACK>::run(p, lq_smem, 1);
 }
 
-// True when the persistent kernel implements this call: full 256x256 tiles, an even number of k-tiles, scales and bias only.
+// True when the persistent kernel implements this call: full 256x256 tiles, an even number of k-tiles, scales and bias only
+// (and, for FP8, the running maximum of the outputs, which costs the epilogue two instructions per four outputs).
 template <int KIND> static inline bool persist_supports(const GemmParams& p) {
     if (p.m <= 0 || p.m % 256 != 0 || p.n % 256 != 0 || p.kb % 128 != 0) return false;
     if (p.C == nullptr || p.addend != nullptr || p.gate != nullptr || p.residual != nullptr || p.C8 != nullptr || p.gelu != 0 ||
         p.out_scale != nullptr)
         return false;
+    if (p.out_max != nullptr && KIND != K_FP8) return false;
     return true;
 }
 
-template <int KIND, typename OutTag> static int launch_gemm_persist(GemmParams p, hipStream_t st) {
-    using GK = GemmPersist<KIND, OutTag, 4>;
-    if (!persist_supports<KIND>(p)) return 1;
+template <int KIND, typename OutTag, bool TRACK = false> static int launch_gemm_persist(GemmParams p, hipStream_t st) {
+    using GK = GemmPersist<KIND, OutTag, 4, TRACK>;
+    if (!persist_supports<KIND>(p) || TRACK != (p.out_max != nullptr)) return 1;
     p.tiles_m = p.m / 256;
     p.tiles_n = p.n / 256;
-    auto kern = gemm_persist_kernel<KIND, OutTag>;
+    auto kern = gemm_persist_kernel<KIND, OutTag, TRACK>;
     static bool attr_done = false;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, GK::SMEM_BYTES);

@@ -125,6 +125,67 @@ __global__ __launch_bounds__(256) void fp8_cast_kernel(uint8_t* __restrict__ dst
     }
 }
 
+// Activation and dynamic quantisation of a stored GEMM output in one pass: h = T(gelu(y)) (the tanh-GELU that the reference
+// applies to a stored T tensor, invokeFusedBiasAndGelu, kernels/flux_single_transformer_block/flux_single_transformer_kernels.cu:
+// 122-141), codes = e4m3(h / scale), scale = max|h| / 448.  The maximum needs no pass over the tensor: the GEMM that wrote y
+// also left ymax = max(y, 0) (lq_gemm_fp8_max), T(gelu(.)) is non-decreasing on the values of T from 0 up (checked value by
+// value in the tests), so max|h| = h(ymax) as soon as that beats the largest |h| any negative y can give (0.17 at y = -0.75);
+// the kernel takes that route from ymax >= 0.5 (h = 0.345).  Below that -- a tensor without a single output of 0.5 or more --
+// the scale comes from the bound max(h(ymax), kGeluNegBound) instead of the exact maximum.
+constexpr float kGeluNegBound = 0.171875f;  // >= |gelu(y)| for every y < 0; a value of fp16 and bf16
+template <typename Tag, bool NT, bool WANT_H>
+__global__ __launch_bounds__(256) void fp8_gelu_cast_kernel(uint8_t* __restrict__ dst, float* __restrict__ scale_out,
+                                                            void* __restrict__ h_out, const void* __restrict__ src,
+                                                            const float* __restrict__ src_max, size_t n) {
+    constexpr int E = Chunk16<Tag>::elems;
+    const float ym = round_through<Tag>(fmaxf(src_max[0], 0.0f));
+    float amax = round_through<Tag>(gelu_fast(ym));
+    if (!(ym >= 0.5f)) amax = fmaxf(amax, kGeluNegBound);
+    const float s = amax / 448.0f;
+    const float r = 1.0f / s;
+    if (blockIdx.x == 0 && threadIdx.x == 0) scale_out[0] = s;
+    const size_t nchunks = n / E;
+    for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < nchunks; c += (size_t)gridDim.x * blockDim.x) {
+        float v[16];
+        load_elems<Tag, NT>(src, c * E, v);
+#pragma unroll
+        for (int i = 0; i < E; i += 2) {
+            v[i] = gelu_fast(v[i]);
+            v[i + 1] = gelu_fast(v[i + 1]);
+            round_through2<Tag>(v[i], v[i + 1]);
+        }
+        if constexpr (WANT_H) {
+            if constexpr (Elem<Tag>::bytes == 2) {
+                u32 hw[E / 2];
+#pragma unroll
+                for (int i = 0; i < E / 2; ++i) hw[i] = Elem<Tag>::store(v[2 * i]) | (Elem<Tag>::store(v[2 * i + 1]) << 16);
+                *reinterpret_cast<uint4*>(static_cast<char*>(h_out) + c * 32) = make_uint4(hw[0], hw[1], hw[2], hw[3]);
+                *reinterpret_cast<uint4*>(static_cast<char*>(h_out) + c * 32 + 16) = make_uint4(hw[4], hw[5], hw[6], hw[7]);
+            } else {
+                *reinterpret_cast<float4*>(static_cast<char*>(h_out) + c * 32) = make_float4(v[0], v[1], v[2], v[3]);
+                *reinterpret_cast<float4*>(static_cast<char*>(h_out) + c * 32 + 16) = make_float4(v[4], v[5], v[6], v[7]);
+            }
+        }
+        u32 w[4];
+#pragma unroll
+        for (int i = 0; i < E / 4; ++i)
+            w[i] = cvt4_e4m3(v[4 * i] * r, v[4 * i + 1] * r, v[4 * i + 2] * r, v[4 * i + 3] * r);
+        if constexpr (E == 16) *reinterpret_cast<uint4*>(dst + c * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+        else *reinterpret_cast<uint2*>(dst + c * 8) = make_uint2(w[0], w[1]);
+    }
+    if (blockIdx.x == 0) {
+        size_t i = nchunks * E + threadIdx.x;
+        if (i < n) {
+            const float h = round_through<Tag>(gelu_fast(load_one<Tag>(src, i)));
+            if constexpr (WANT_H) {
+                if constexpr (Elem<Tag>::bytes == 2) static_cast<unsigned short*>(h_out)[i] = (unsigned short)Elem<Tag>::store(h);
+                else static_cast<float*>(h_out)[i] = h;
+            }
+            dst[i] = (uint8_t)cvt1_e4m3(h * r);
+        }
+    }
+}
+
 // The same cast for a matrix whose rows are `src_ld` elements apart, written with rows `dst_ld` bytes apart: a block of
 // columns of a wider destination (the concatenated input of FLUX's single-block output projection).  cols % E == 0.
 template <typename Tag>
@@ -658,6 +719,35 @@ extern "C" int lq_fp8_scale_cast(uint8_t* dst, const void* src, lq_dtype_t dtype
         case LQ_BF16: return launch_cast<BF16Tag>(dst, src, scale, invert, n, as_stream(stream));
         case LQ_F32: return launch_cast<F32Tag>(dst, src, scale, invert, n, as_stream(stream));
         default: set_error("lq_fp8_scale_cast: unsupported dtype %d", (int)dtype); return LQ_ERR_UNSUPPORTED;
+    }
+}
+
+template <typename Tag>
+static int launch_gelu_cast(uint8_t* dst, float* scale_out, void* h_out, const void* src, const float* src_max, size_t n, hipStream_t st) {
+    const dim3 grid(stream_grid(n, Chunk16<Tag>::elems)), block(256);
+    const bool nt = n * Elem<Tag>::bytes >= kStreamBytes;
+    if (h_out != nullptr) {
+        hipLaunchKernelGGL((fp8_gelu_cast_kernel<Tag, false, true>), grid, block, 0, st, dst, scale_out, h_out, src, src_max, n);
+    } else if (nt) {
+        hipLaunchKernelGGL((fp8_gelu_cast_kernel<Tag, true, false>), grid, block, 0, st, dst, scale_out, h_out, src, src_max, n);
+    } else {
+        hipLaunchKernelGGL((fp8_gelu_cast_kernel<Tag, false, false>), grid, block, 0, st, dst, scale_out, h_out, src, src_max, n);
+    }
+    return check_launch("fp8_gelu_cast");
+}
+
+extern "C" int lq_fp8_gelu_cast(uint8_t* dst, float* scale_out, void* h_out, const void* src, lq_dtype_t dtype, size_t n,
+                                const float* src_max, lq_stream_t stream) {
+    LQ_REQUIRE(scale_out && src_max && ((dst && src) || n == 0), LQ_ERR_ARG, "lq_fp8_gelu_cast: null pointer");
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(h_out) % 16 == 0,
+               LQ_ERR_ARG, "lq_fp8_gelu_cast: src, dst and h_out must be 16-byte aligned");
+    if (n == 0) return LQ_OK;
+    switch (dtype) {
+        case LQ_F16: return launch_gelu_cast<F16Tag>(dst, scale_out, h_out, src, src_max, n, as_stream(stream));
+        case LQ_BF16: return launch_gelu_cast<BF16Tag>(dst, scale_out, h_out, src, src_max, n, as_stream(stream));
+        case LQ_F32: return launch_gelu_cast<F32Tag>(dst, scale_out, h_out, src, src_max, n, as_stream(stream));
+        default: set_error("lq_fp8_gelu_cast: unsupported dtype %d", (int)dtype); return LQ_ERR_UNSUPPORTED;
     }
 }
 

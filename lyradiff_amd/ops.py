@@ -449,6 +449,39 @@ def fp8_linear(a_q, w_rows32, a_scale, b_scale, bias=None, gelu: bool = False, r
     return (c, c8) if want_output else c8
 
 
+def fp8_linear_max(a_q, w_rows32, a_scale, b_scale, bias, out_max, out_dtype=torch.bfloat16):
+    """fp8_linear without activation that also joins its largest output into out_max (fp32 [1], zeroed by the caller; stays
+    >= 0): what fp8_gelu_quant needs to quantise gelu(C) in one pass."""
+    _chk(a_q, "a_q", (torch.uint8,))
+    _chk(w_rows32, "w_rows32", (torch.uint8,))
+    _chk(a_scale, "a_scale", (torch.float32,))
+    _chk(b_scale, "b_scale", (torch.float32,))
+    _chk(out_max, "out_max", (torch.float32,))
+    m, k = a_q.shape
+    n = w_rows32.shape[0]
+    if w_rows32.shape[1] != k:
+        raise ValueError("K mismatch between activation and weight")
+    if bias is not None:
+        _chk(bias, "bias", (out_dtype,))
+    c = torch.empty((m, n), dtype=out_dtype, device=a_q.device)
+    _l.check(_l.load().lq_gemm_fp8_max(_ptr(c), _DT[out_dtype], _ptr(a_q), _ptr(w_rows32), _ptr(a_scale), _ptr(b_scale),
+                                       _ptr(bias), m, n, k, _ptr(out_max), _stream()), "lq_gemm_fp8_max")
+    return c
+
+
+def fp8_gelu_quant(y, y_max, want_h: bool = False):
+    """h = T(gelu_tanh(y)), codes = e4m3(h / scale), scale = max|h| / 448 in one pass over y; y_max (fp32 [1]) >= max(y, 0) as
+    fp8_linear_max leaves it.  Returns (codes uint8, scale fp32 [1]) and h when want_h."""
+    _chk(y, "y", _FLOATS)
+    _chk(y_max, "y_max", (torch.float32,))
+    q = torch.empty(y.shape, dtype=torch.uint8, device=y.device)
+    s = torch.empty(1, dtype=torch.float32, device=y.device)
+    h = torch.empty_like(y) if want_h else None
+    _l.check(_l.load().lq_fp8_gelu_cast(_ptr(q), _ptr(s), _ptr(h), _ptr(y), _DT[y.dtype], y.numel(), _ptr(y_max), _stream()),
+             "lq_fp8_gelu_cast")
+    return (q, s, h) if want_h else (q, s)
+
+
 def fp8_linear_gated(a_q, w_rows32, a_scale, b_scale, bias, gate, residual, rows_per_gate: int, out=None):
     """FP8 GEMM + invokeFusedGateAndResidual: out = residual + gate[row // rows_per_gate] * (A.W^T*sa*sb + bias), with
     the roundings of the unfused sequence.  gate [ceil(M/rows_per_gate), N], residual [M, N]; out may be residual."""

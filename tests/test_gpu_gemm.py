@@ -488,6 +488,67 @@ def test_random_shapes_all_gemms(ops, dev):
                        f"fp8 {m}x{n}x{k4}", max_share_outside=2e-2)  # tiny K: a larger share of sums cancels
 
 
+# ---- GEMM that leaves its largest output, then activation + dynamic quantisation in one pass -----------------------------
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+def test_gelu_of_a_stored_tensor_is_monotone_from_zero_up_and_bounded_below_it(ops, dev, dt):
+    """What fp8_gelu_quant's scale rests on, value by value over every finite number of T: h = T(gelu(y)) never decreases as y
+    grows from 0, and no negative y gives |h| above the bound the kernel falls back to.  h itself against the oracle's GELU."""
+    t = TORCH_DT[dt]
+    bits = torch.arange(0, 1 << 16, dtype=torch.int32).to(torch.int16)
+    y = bits.view(t)
+    y = y[torch.isfinite(y.float())]
+    big = torch.full((1,), 1e30, dtype=torch.float32, device=dev)
+    _, _, h = ops.fp8_gelu_quant(y.to(dev), big, want_h=True)
+    yf, hf = y.float().numpy(), h.float().cpu().numpy()
+    order = np.argsort(yf, kind="stable")
+    yf, hf = yf[order], hf[order]
+    pos = yf >= 0
+    assert np.all(np.diff(hf[pos]) >= 0), "T(gelu(y)) decreases somewhere on y >= 0"
+    assert np.abs(hf[~pos]).max() <= 0.171875 < hf[pos][np.searchsorted(yf[pos], 0.5)]
+    ref = O.round_to(O.gelu_tanh_f32(yf), dt)
+    fin = np.abs(yf) < 1e4  # beyond that the oracle's x^3 overflows to inf - inf
+    assert_close_tol(hf[fin], ref[fin], "gelu of a stored tensor")
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+# the first three run the persistent kernel (whole 256x256 tiles, k % 128 == 0), with and without a round of half tiles; the
+# last two the two-workgroups-per-CU kernels, ragged edges included
+@pytest.mark.parametrize("m,n,k", [(512, 1024, 256), (4608, 12288, 128), (6912, 9216, 256), (333, 416, 704), (1024, 3072, 192)])
+def test_fp8_linear_max_then_gelu_quant(ops, dev, m, n, k, dt):
+    """C and its running maximum, then h = T(gelu(C)) quantised with the scale derived from that maximum: the same codes
+    and scale as the amax + cast kernels give on h (checked against the oracle in test_gpu_quant.py)."""
+    g = rng_t(m + n + k + 3)
+    t = TORCH_DT[dt]
+    qa, sa = ops.fp8_quant(torch.randn(m, k, generator=g).to(t).to(dev))
+    qw, sw = ops.fp8_quant((torch.randn(n, k, generator=g) * 0.05).to(t).to(dev))
+    wp = ops.repack_weight(qw)
+    bias = (torch.randn(n, generator=g) * 0.1).to(t).to(dev)
+    ymax = torch.zeros(1, dtype=torch.float32, device=dev)
+    c = ops.fp8_linear_max(qa, wp, sa, sw, bias, ymax, t)
+    ref = O.fp8_gemm(qa.cpu().numpy(), qw.cpu().numpy(), sa.item(), sw.item(), to_np_f32(bias.cpu()), False, None, 0.0, dt)
+    check_fp8_gemm(to_np_f32(c.cpu()), ref, qa.cpu().numpy(), qw.cpu().numpy(), sa.item(), sw.item(), dt, "fp8 gemm with running maximum")
+    assert ymax.item() == max(c.float().max().item(), 0.0) and ymax.item() >= 0.5
+    # accumulation semantics: a larger value already in the slot wins
+    big = torch.full((1,), 1e6, dtype=torch.float32, device=dev)
+    assert torch.equal(ops.fp8_linear_max(qa, wp, sa, sw, bias, big, t), c) and big.item() == 1e6
+    q, s, h = ops.fp8_gelu_quant(c, ymax, want_h=True)
+    q_ref, s_ref = ops.fp8_quant(h)
+    assert torch.equal(s, s_ref) and torch.equal(q, q_ref)
+    q2, s2 = ops.fp8_gelu_quant(c, ymax)
+    assert torch.equal(q2, q) and torch.equal(s2, s)
+    assert_close_tol(to_np_f32(h.cpu()), O.round_to(O.gelu_tanh_f32(to_np_f32(c.cpu())), dt), "gelu of the stored output")
+
+
+def test_fp8_gelu_quant_without_a_large_value_takes_the_bound(ops, dev):
+    g = rng_t(9)
+    y = (torch.rand(5000, generator=g) - 0.7).clamp(max=0.4).bfloat16().to(dev)
+    ymax = y.float().max().clamp(min=0).reshape(1)
+    q, s, h = ops.fp8_gelu_quant(y, ymax, want_h=True)
+    assert s.item() == np.float32(max(h.float().max().item(), 0.171875)) / np.float32(448.0)
+    assert torch.equal(q, ops.fp8_scale_cast(h, s))
+    assert h.float().abs().max().item() <= s.item() * 448.0 * (1 + 1e-6)  # nothing saturates
+
+
 # ---- FP8 GEMM epilogue outputs for the next FP8 linear -----------------------------------------------------------------
 @pytest.mark.parametrize("m,n,k,gelu", [(333, 416, 704, True), (1024, 3072, 3072, False), (4608, 12288, 3072, True)])
 @pytest.mark.parametrize("dt", ["bf16", "f16"])
