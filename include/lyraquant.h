@@ -252,9 +252,11 @@ int lq_gemm_fp8_max(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8
  * src_max[0] >= max(y, 0) exactly (lq_gemm_fp8_max leaves it): T(gelu(.)) is non-decreasing from 0 up, so max|h| =
  * h(src_max) whenever src_max >= 0.5 -- the result is then bit for bit that of lq_fp8_amax_cast on h.  A tensor without a
  * single value of 0.5 or more takes max(h(src_max), 0.171875) for max|h|: an upper bound (no |gelu| of a negative number
- * exceeds 0.17), not the exact maximum. */
+ * exceeds 0.17), not the exact maximum.
+ * clear_max (optional, != src_max): set to 0 by this launch -- the slot the NEXT lq_gemm_fp8_max will accumulate into, so that a
+ * chain that alternates two slots needs no fill launch between its steps. */
 int lq_fp8_gelu_cast(uint8_t* dst, float* scale_out, void* h_out, const void* src, lq_dtype_t dtype, size_t n,
-                     const float* src_max, lq_stream_t stream);
+                     const float* src_max, float* clear_max, lq_stream_t stream);
 
 /* lq_gemm_fp8 (no activation) whose epilogue applies FLUX's gate and second residual:
  *   C[m,n] = T( T( T(y[m,n]) * gate[m / rows_per_gate, n] ) + residual[m,n] ),  y = (sa*sb)*acc + bias[n]

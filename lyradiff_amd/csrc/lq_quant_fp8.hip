@@ -136,8 +136,9 @@ constexpr float kGeluNegBound = 0.171875f;  // >= |gelu(y)| for every y < 0; a v
 template <typename Tag, bool NT, bool WANT_H>
 __global__ __launch_bounds__(256) void fp8_gelu_cast_kernel(uint8_t* __restrict__ dst, float* __restrict__ scale_out,
                                                             void* __restrict__ h_out, const void* __restrict__ src,
-                                                            const float* __restrict__ src_max, size_t n) {
+                                                            const float* __restrict__ src_max, float* __restrict__ clear, size_t n) {
     constexpr int E = Chunk16<Tag>::elems;
+    if (clear != nullptr && blockIdx.x == 0 && threadIdx.x == 0) clear[0] = 0.0f;  // the next call's slot for a running maximum
     const float ym = round_through<Tag>(fmaxf(src_max[0], 0.0f));
     float amax = round_through<Tag>(gelu_fast(ym));
     if (!(ym >= 0.5f)) amax = fmaxf(amax, kGeluNegBound);
@@ -723,30 +724,33 @@ extern "C" int lq_fp8_scale_cast(uint8_t* dst, const void* src, lq_dtype_t dtype
 }
 
 template <typename Tag>
-static int launch_gelu_cast(uint8_t* dst, float* scale_out, void* h_out, const void* src, const float* src_max, size_t n, hipStream_t st) {
+static int launch_gelu_cast(uint8_t* dst, float* scale_out, void* h_out, const void* src, const float* src_max, float* clear, size_t n,
+                            hipStream_t st) {
     const dim3 grid(stream_grid(n, Chunk16<Tag>::elems)), block(256);
     const bool nt = n * Elem<Tag>::bytes >= kStreamBytes;
     if (h_out != nullptr) {
-        hipLaunchKernelGGL((fp8_gelu_cast_kernel<Tag, false, true>), grid, block, 0, st, dst, scale_out, h_out, src, src_max, n);
+        hipLaunchKernelGGL((fp8_gelu_cast_kernel<Tag, false, true>), grid, block, 0, st, dst, scale_out, h_out, src, src_max, clear, n);
     } else if (nt) {
-        hipLaunchKernelGGL((fp8_gelu_cast_kernel<Tag, true, false>), grid, block, 0, st, dst, scale_out, h_out, src, src_max, n);
+        hipLaunchKernelGGL((fp8_gelu_cast_kernel<Tag, true, false>), grid, block, 0, st, dst, scale_out, h_out, src, src_max, clear, n);
     } else {
-        hipLaunchKernelGGL((fp8_gelu_cast_kernel<Tag, false, false>), grid, block, 0, st, dst, scale_out, h_out, src, src_max, n);
+        hipLaunchKernelGGL((fp8_gelu_cast_kernel<Tag, false, false>), grid, block, 0, st, dst, scale_out, h_out, src, src_max, clear, n);
     }
     return check_launch("fp8_gelu_cast");
 }
 
 extern "C" int lq_fp8_gelu_cast(uint8_t* dst, float* scale_out, void* h_out, const void* src, lq_dtype_t dtype, size_t n,
-                                const float* src_max, lq_stream_t stream) {
+                                const float* src_max, float* clear_max, lq_stream_t stream) {
     LQ_REQUIRE(scale_out && src_max && ((dst && src) || n == 0), LQ_ERR_ARG, "lq_fp8_gelu_cast: null pointer");
+    LQ_REQUIRE(clear_max != src_max && clear_max != scale_out, LQ_ERR_ARG,
+               "lq_fp8_gelu_cast: clear_max must not be the slot this call reads or the scale it writes");
     LQ_REQUIRE(reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(h_out) % 16 == 0,
                LQ_ERR_ARG, "lq_fp8_gelu_cast: src, dst and h_out must be 16-byte aligned");
     if (n == 0) return LQ_OK;
     switch (dtype) {
-        case LQ_F16: return launch_gelu_cast<F16Tag>(dst, scale_out, h_out, src, src_max, n, as_stream(stream));
-        case LQ_BF16: return launch_gelu_cast<BF16Tag>(dst, scale_out, h_out, src, src_max, n, as_stream(stream));
-        case LQ_F32: return launch_gelu_cast<F32Tag>(dst, scale_out, h_out, src, src_max, n, as_stream(stream));
+        case LQ_F16: return launch_gelu_cast<F16Tag>(dst, scale_out, h_out, src, src_max, clear_max, n, as_stream(stream));
+        case LQ_BF16: return launch_gelu_cast<BF16Tag>(dst, scale_out, h_out, src, src_max, clear_max, n, as_stream(stream));
+        case LQ_F32: return launch_gelu_cast<F32Tag>(dst, scale_out, h_out, src, src_max, clear_max, n, as_stream(stream));
         default: set_error("lq_fp8_gelu_cast: unsupported dtype %d", (int)dtype); return LQ_ERR_UNSUPPORTED;
     }
 }

@@ -469,15 +469,18 @@ def fp8_linear_max(a_q, w_rows32, a_scale, b_scale, bias, out_max, out_dtype=tor
     return c
 
 
-def fp8_gelu_quant(y, y_max, want_h: bool = False):
+def fp8_gelu_quant(y, y_max, want_h: bool = False, clear_max=None):
     """h = T(gelu_tanh(y)), codes = e4m3(h / scale), scale = max|h| / 448 in one pass over y; y_max (fp32 [1]) >= max(y, 0) as
-    fp8_linear_max leaves it.  Returns (codes uint8, scale fp32 [1]) and h when want_h."""
+    fp8_linear_max leaves it.  Returns (codes uint8, scale fp32 [1]) and h when want_h.  clear_max (fp32 [1], another tensor
+    than y_max) is set to 0 by the same launch: the slot of the next fp8_linear_max."""
     _chk(y, "y", _FLOATS)
     _chk(y_max, "y_max", (torch.float32,))
+    if clear_max is not None:
+        _chk(clear_max, "clear_max", (torch.float32,))
     q = torch.empty(y.shape, dtype=torch.uint8, device=y.device)
     s = torch.empty(1, dtype=torch.float32, device=y.device)
     h = torch.empty_like(y) if want_h else None
-    _l.check(_l.load().lq_fp8_gelu_cast(_ptr(q), _ptr(s), _ptr(h), _ptr(y), _DT[y.dtype], y.numel(), _ptr(y_max), _stream()),
+    _l.check(_l.load().lq_fp8_gelu_cast(_ptr(q), _ptr(s), _ptr(h), _ptr(y), _DT[y.dtype], y.numel(), _ptr(y_max), _ptr(clear_max), _stream()),
              "lq_fp8_gelu_cast")
     return (q, s, h) if want_h else (q, s)
 

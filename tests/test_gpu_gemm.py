@@ -534,8 +534,11 @@ def test_fp8_linear_max_then_gelu_quant(ops, dev, m, n, k, dt):
     q, s, h = ops.fp8_gelu_quant(c, ymax, want_h=True)
     q_ref, s_ref = ops.fp8_quant(h)
     assert torch.equal(s, s_ref) and torch.equal(q, q_ref)
-    q2, s2 = ops.fp8_gelu_quant(c, ymax)
-    assert torch.equal(q2, q) and torch.equal(s2, s)
+    nxt = torch.full((1,), 7.0, dtype=torch.float32, device=dev)
+    q2, s2 = ops.fp8_gelu_quant(c, ymax, clear_max=nxt)
+    assert torch.equal(q2, q) and torch.equal(s2, s) and nxt.item() == 0.0
+    with pytest.raises(RuntimeError):
+        ops.fp8_gelu_quant(c, ymax, clear_max=ymax)
     assert_close_tol(to_np_f32(h.cpu()), O.round_to(O.gelu_tanh_f32(to_np_f32(c.cpu())), dt), "gelu of the stored output")
 
 
