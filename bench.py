@@ -500,6 +500,13 @@ def extra_kernels(torch, ops, dev):
     sm = (torch.rand(k, generator=g) + 0.5).to(dev)
     us = timeit(lambda: ops.w4a4_quant(xr(), sm))
     res[f"w4a4_quant_{m}x{k}"] = {"us": round(us, 2), "GB/s": round((2.5 * m * k + 4.0 * m * k / 64) / us / 1e3, 1)}
+    us = timeit(lambda: ops.w4a4_quant_lora_down(xr(), sm, dn))  # both of the above from one read of x
+    res[f"w4a4_quant_and_lora_down_rank32_{m}x{k}"] = {"us": round(us, 2), "GB/s": round((2.5 * m * k + 4.0 * m * k / 64 + 64.0 * m) / us / 1e3, 1)}
+    y16 = torch.randn(m, 4 * k, generator=g).bfloat16().to(dev)
+    ymx = y16.float().max().clamp(min=0).reshape(1)
+    us = timeit(lambda: ops.fp8_gelu_quant(y16, ymx))
+    res[f"fp8_gelu_cast_{m}x{4 * k}"] = {"us": round(us, 2), "GB/s": round(3.0 * m * 4 * k / us / 1e3, 1)}
+    del y16
     for (m, k) in [(4608, 3072), (4608, 12288)]:
         xr = rotating(torch.randn(m, k, generator=g).bfloat16().to(dev))
         us = timeit(lambda: ops.fp8_quant(xr()))
