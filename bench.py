@@ -507,6 +507,20 @@ def extra_kernels(torch, ops, dev):
     us = timeit(lambda: ops.fp8_gelu_quant(y16, ymx))
     res[f"fp8_gelu_cast_{m}x{4 * k}"] = {"us": round(us, 2), "GB/s": round(3.0 * m * 4 * k / us / 1e3, 1)}
     del y16
+    for (m, k) in [(4608, 3072), (6912, 3072)]:
+        # where the one-launch quantiser's time goes: device time stamps of every workgroup, medians over 20 launches (us from the
+        # first workgroup's start)
+        xr = rotating(torch.randn(m, k, generator=g).bfloat16().to(dev))
+        rows = []
+        for _ in range(25):
+            q, s_, st = ops.fp8_quant_timeline(xr())
+            t = (st - st[:, 0].min()).double().cpu() * 0.01
+            rows.append([t[:, 0].max().item(), t[:, 1].max().item(), t[:, 2].max().item(), t[:, 3].max().item(),
+                         (t[:, 1] - t[:, 0]).mean().item(), (t[:, 2] - t[:, 1]).mean().item(), (t[:, 3] - t[:, 2]).mean().item()])
+        med = torch.tensor(rows[5:]).median(dim=0).values.tolist()
+        res[f"fp8_amax_cast_timeline_{m}x{k}"] = dict(zip(
+            ["last_workgroup_started_us", "last_loads_back_us", "last_released_from_exchange_us", "last_stores_acknowledged_us",
+             "mean_load_phase_us", "mean_exchange_us", "mean_cast_and_store_us"], [round(v, 2) for v in med]))
     for (m, k) in [(4608, 3072), (4608, 12288)]:
         xr = rotating(torch.randn(m, k, generator=g).bfloat16().to(dev))
         us = timeit(lambda: ops.fp8_quant(xr()))

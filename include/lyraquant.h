@@ -149,6 +149,13 @@ int lq_fp8_amax_cast_release_slot(lq_stream_t stream);
  * zero -- run it once the overlapping calls have finished. */
 int lq_fp8_amax_cast_static(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t n,
                             lq_stream_t stream);
+/* Measurement aid, no counterpart in the reference: lq_fp8_amax_cast's one launch with four readings of the device's constant
+ * 100 MHz clock per workgroup, stamps[4*w + 0..3] = workgroup w started, its partial maximum is formed (all its loads are back),
+ * it is released from the grid-wide exchange, its stores are acknowledged.  stamps: device memory, 4 * 512 entries, zeroed by
+ * the caller (entries of workgroups beyond the launch's grid stay zero).  LQ_ERR_UNSUPPORTED when the call would not take the
+ * one-launch route (fewer than 4096 elements, unaligned buffers, no free exchange slot, stream capture). */
+int lq_fp8_amax_cast_timeline(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t n,
+                              unsigned long long* stamps, lq_stream_t stream);
 size_t lq_fp8_amax_cast_static_max_elems(void);
 int lq_fp8_amax_cast_static_reset(lq_stream_t stream);
 

@@ -388,7 +388,11 @@ __device__ __forceinline__ unsigned long long poll_tagged(const unsigned long lo
 template <typename Tag, int KEEP>
 __global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_t* __restrict__ dst, float* __restrict__ scale_out,
                                                                           const void* __restrict__ src, size_t n, CoopSlot* slot,
-                                                                          unsigned launch, unsigned* timeout) {
+                                                                          unsigned launch, unsigned* timeout,
+                                                                          unsigned long long* __restrict__ stamps) {
+    // stamps (NULL in every product launch): four readings of the constant 100 MHz clock per workgroup -- started, partial
+    // maximum formed (its loads are back), released from the exchange, stores acknowledged (lq_fp8_amax_cast_timeline)
+    if (stamps != nullptr && threadIdx.x == 0) stamps[blockIdx.x * 4] = wall_clock64();
     constexpr int E2 = Elem<Tag>::bytes == 2 ? 8 : 4;  // elements per 16-byte piece
     constexpr int BLK = 128 * E2;                      // elements per 2 KiB block
     typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
@@ -435,6 +439,7 @@ __global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_
     amax = wave_max(amax);
     if (lane == 0) red[threadIdx.x >> 6] = amax;
     __syncthreads();
+    if (stamps != nullptr && threadIdx.x == 0) stamps[blockIdx.x * 4 + 1] = wall_clock64();
     if (threadIdx.x == 0) {
         float wg_max = 0.0f;
 #pragma unroll
@@ -466,6 +471,7 @@ __global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_
         tensor_max = ok ? __uint_as_float((unsigned)v) : __builtin_nanf("");
     }
     __syncthreads();
+    if (stamps != nullptr && threadIdx.x == 0) stamps[blockIdx.x * 4 + 2] = wall_clock64();
     const float s = tensor_max / 448.0f;  // NaN after a time-out
     if (threadIdx.x == 0 && s != s) {
         __hip_atomic_store(timeout, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -509,6 +515,11 @@ __global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_
     }
     if (blockIdx.x == 0)
         for (size_t i = nblocks * BLK + threadIdx.x; i < n; i += kCoopThreads) dst[i] = (uint8_t)cvt1_e4m3(load_one<Tag>(src, i) * r);
+    if (stamps != nullptr) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's stores are acknowledged
+        __syncthreads();
+        if (threadIdx.x == 0) stamps[blockIdx.x * 4 + 3] = wall_clock64();
+    }
 }
 
 // Returns LQ_OK when the fused launch was issued, 1 when the caller should fall back to the scratch-free
@@ -537,7 +548,7 @@ template <typename Tag, int KEEP> struct CoopCapacity {
 
 template <typename Tag, int KEEP>
 static int launch_coop_keep(uint8_t* dst, float* scale_out, const void* src, size_t n, hipStream_t st, int dev, FusedScratch* ws,
-                            size_t waves_needed) {
+                            size_t waves_needed, unsigned long long* stamps) {
     const int num_cu = CoopCapacity<Tag, KEEP>::get(dev).num_cu;
     if (num_cu == 0) return 1;
     unsigned launch = 0;
@@ -548,12 +559,13 @@ static int launch_coop_keep(uint8_t* dst, float* scale_out, const void* src, siz
     if (grid > kCoopMaxBlocks) grid = kCoopMaxBlocks;
     if (grid == 0) grid = 1;
     hipLaunchKernelGGL((fp8_amax_cast_coop_kernel<Tag, KEEP>), dim3((unsigned)grid), dim3(kCoopThreads), 0, st, dst, scale_out, src, n,
-                       &ws->coop[slot], launch, &ws->timeout);
+                       &ws->coop[slot], launch, &ws->timeout, stamps);
     return check_launch("fp8_amax_cast_fused");
 }
 
 template <typename Tag>
-static int launch_amax_cast_coop(uint8_t* dst, float* scale_out, const void* src, size_t n, hipStream_t st) {
+static int launch_amax_cast_coop(uint8_t* dst, float* scale_out, const void* src, size_t n, hipStream_t st,
+                                 unsigned long long* stamps = nullptr) {
     if (reinterpret_cast<uintptr_t>(src) % 16 != 0 || reinterpret_cast<uintptr_t>(dst) % 16 != 0) return 1;
     if (st == hipStreamPerThread) return 1;  // one handle for every thread's own stream: its launches can overlap
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
@@ -569,9 +581,9 @@ static int launch_amax_cast_coop(uint8_t* dst, float* scale_out, const void* src
     if (num_cu == 0) return 1;
     const size_t waves = (size_t)num_cu * (kCoopThreads / 64);
     const size_t per_wave = (blocks + waves - 1) / waves;
-    if (per_wave <= 4) return launch_coop_keep<Tag, 4>(dst, scale_out, src, n, st, dev, ws, blocks);
-    if (per_wave <= 8) return launch_coop_keep<Tag, 8>(dst, scale_out, src, n, st, dev, ws, blocks);
-    return launch_coop_keep<Tag, 10>(dst, scale_out, src, n, st, dev, ws, blocks);
+    if (per_wave <= 4) return launch_coop_keep<Tag, 4>(dst, scale_out, src, n, st, dev, ws, blocks, stamps);
+    if (per_wave <= 8) return launch_coop_keep<Tag, 8>(dst, scale_out, src, n, st, dev, ws, blocks, stamps);
+    return launch_coop_keep<Tag, 10>(dst, scale_out, src, n, st, dev, ws, blocks, stamps);
 }
 
 // ---- two launches, no barrier: partial maxima + ticket, then the cast ------------------------------------------------
@@ -793,6 +805,25 @@ extern "C" int lq_fp8_amax_cast(uint8_t* dst, float* scale_out, const void* src,
     rc = lq_fp8_amax_scale(scale_out, src, dtype, n, stream);
     if (rc != LQ_OK) return rc;
     return lq_fp8_scale_cast(dst, src, dtype, scale_out, 1, n, stream);
+}
+
+extern "C" int lq_fp8_amax_cast_timeline(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t n,
+                                         unsigned long long* stamps, lq_stream_t stream) {
+    LQ_REQUIRE(dst && scale_out && src && stamps, LQ_ERR_ARG, "lq_fp8_amax_cast_timeline: null pointer");
+    int rc = 1;
+    if (n >= 4096) {
+        switch (dtype) {
+            case LQ_F16: rc = launch_amax_cast_coop<F16Tag>(dst, scale_out, src, n, as_stream(stream), stamps); break;
+            case LQ_BF16: rc = launch_amax_cast_coop<BF16Tag>(dst, scale_out, src, n, as_stream(stream), stamps); break;
+            case LQ_F32: rc = launch_amax_cast_coop<F32Tag>(dst, scale_out, src, n, as_stream(stream), stamps); break;
+            default: set_error("lq_fp8_amax_cast_timeline: unsupported dtype %d", (int)dtype); return LQ_ERR_UNSUPPORTED;
+        }
+    }
+    if (rc == 1) {
+        set_error("lq_fp8_amax_cast_timeline: the one-launch form does not apply to this call (size, alignment, stream or capture)");
+        return LQ_ERR_UNSUPPORTED;
+    }
+    return rc;
 }
 
 extern "C" int lq_fp8_amax_cast_static(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t n,

@@ -93,6 +93,7 @@ SYMBOLS = {
     "lq_gate_residual_layernorm_mod": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _Z, _Z, _Z, _F, _P]),
     "lq_gemm_w4a4_ex": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P]),
     "lq_gemm_w4a4_lora": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
+    "lq_fp8_amax_cast_timeline": (_I, [_P, _P, _P, _I, _Z, _P, _P]),
     "lq_gemm_fp8_max": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _P, _P]),
     "lq_fp8_gelu_cast": (_I, [_P, _P, _P, _P, _I, _Z, _P, _P, _P]),
     "lq_lora_down": (_I, [_P, _I, _P, _P, _I, _I, _I, _I, _P]),

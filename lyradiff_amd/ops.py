@@ -337,6 +337,18 @@ def fp8_quant_static_reset() -> None:
     _l.check(_l.load().lq_fp8_amax_cast_static_reset(_stream()), "lq_fp8_amax_cast_static_reset")
 
 
+def fp8_quant_timeline(x):
+    """fp8_quant's one launch with device time stamps: returns (codes, scale, stamps int64 [workgroups, 4] in units of 10 ns:
+    started, loads back, released from the exchange, stores acknowledged)."""
+    _chk(x, "x", _FLOATS)
+    q = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    s = torch.empty(1, dtype=torch.float32, device=x.device)
+    stamps = torch.zeros((512, 4), dtype=torch.int64, device=x.device)
+    _l.check(_l.load().lq_fp8_amax_cast_timeline(_ptr(q), _ptr(s), _ptr(x), _DT[x.dtype], x.numel(), _ptr(stamps), _stream()),
+             "lq_fp8_amax_cast_timeline")
+    return q, s, stamps[stamps[:, 0] != 0]
+
+
 def fp8_quant_static(x, q_out, scale_out):
     """fp8_quant into caller-owned outputs through lq_fp8_amax_cast_static: two launches, no barrier, no allocation
     (scratch in a static device array shared by every call on the GPU: do not overlap calls)."""

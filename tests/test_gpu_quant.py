@@ -338,6 +338,19 @@ def test_fp8_amax_cast_one_launch_sizes(ops, dev, dt, n):
     assert ops.fp8_amax_cast_status() is False
 
 
+def test_fp8_amax_cast_timeline_gives_the_same_bits_and_ordered_stamps(ops, dev):
+    x = (torch.randn(4608 * 3072, generator=rng_t(3)) * 2).bfloat16().to(dev)
+    q0, s0 = ops.fp8_quant(x)
+    q, s, st = ops.fp8_quant_timeline(x)
+    assert torch.equal(q, q0) and torch.equal(s, s0)
+    st = st.cpu().numpy()
+    assert 1 <= st.shape[0] <= 512 and np.all(np.diff(st, axis=1) >= 0), "started <= loads back <= released <= stores acknowledged"
+    assert st[:, 2].min() >= st[:, 1].max(), "nobody is released from the exchange before the last partial maximum is formed"
+    assert (st[:, 3].max() - st[:, 0].min()) * 0.01 < 1000.0  # microseconds
+    with pytest.raises(RuntimeError):
+        ops.fp8_quant_timeline(x[:100])
+
+
 def test_fp8_quant_static_reset(ops, dev):
     """The repair call of the allocation-free quantiser: after it the status is clean and the quantiser works."""
     x = (torch.randn(70000, generator=rng_t(9)) * 3).bfloat16().to(dev)
