@@ -188,6 +188,38 @@ def test_config3_flux_mlp_fp8(ops, dev):
     check_fp8_linear(ops, dev, qh, sh, wq_dn, ws_dn, wp_dn, ws_dn_d, b_dn, False, 34, "config 3 down")
 
 
+def test_config3_flux_mlp_fp8_as_benchmarked(ops, dev):
+    """The chain bench.py times: the up projection leaves its largest output (persistent kernel at this shape), the GELU and the
+    dynamic quantisation of the hidden tensor are one pass that derives its scale from that maximum, then the down projection."""
+    m, d, hdim = 4608, 3072, 12288
+    g = rng_t(1003)
+    x = torch.randn(m, d, generator=g).bfloat16().to(dev)
+    b_up = (torch.randn(hdim, generator=g) * 0.1).bfloat16()
+    b_dn = (torch.randn(d, generator=g) * 0.1).bfloat16()
+    wq_up, ws_up, wp_up, ws_up_d = fp8_weight(ops, dev, hdim, d, g)
+    wq_dn, ws_dn, wp_dn, ws_dn_d = fp8_weight(ops, dev, d, hdim, g)
+    qa, sa = ops.fp8_quant(x)
+    umax = torch.zeros(1, dtype=torch.float32, device=dev)
+    u = ops.fp8_linear_max(qa, wp_up, sa, ws_up_d, b_up.to(dev), umax, torch.bfloat16)
+    rows = band_rows(m, 41)
+    qa_rows = qa[torch.from_numpy(rows).to(dev)].cpu().numpy()
+    ref = O.fp8_gemm(qa_rows, wq_up, float(sa.cpu()), ws_up, to_np_f32(b_up), False, None, 0.0, "bf16")
+    got = to_np_f32(u[torch.from_numpy(rows).to(dev)])
+    check_fp8_gemm(got, ref, qa_rows, wq_up, float(sa.cpu()), ws_up, "bf16", "config 3 up, running maximum")
+    check_fp8_against_instruction_model(got[::16], qa_rows[::16], wq_up, float(sa.cpu()), ws_up, to_np_f32(b_up), "bf16", "config 3 up")
+    assert umax.item() == u.float().max().item() >= 0.5
+    nxt = torch.ones(1, dtype=torch.float32, device=dev)
+    qh, sh, h = ops.fp8_gelu_quant(u, umax, want_h=True)
+    qh2, sh2 = ops.fp8_gelu_quant(u, umax, clear_max=nxt)
+    assert torch.equal(qh2, qh) and torch.equal(sh2, sh) and nxt.item() == 0.0
+    hn = to_np_f32(h)
+    assert_close_tol(hn[rows], O.round_to(O.gelu_tanh_f32(to_np_f32(u)[rows]), "bf16"), "config 3 GELU of the stored output")
+    s_ref = O.fp8_scale(hn)  # scale and codes: exactly the amax and cast of the activated tensor
+    assert float(sh.cpu()) == float(s_ref)
+    assert np.array_equal(qh.cpu().numpy()[rows], O.fp8_scale_cast(hn[rows], s_ref, True))
+    check_fp8_linear(ops, dev, qh, sh, wq_dn, ws_dn, wp_dn, ws_dn_d, b_dn, False, 44, "config 3 down")
+
+
 # ---- config 4: FLUX attention projection, W4A4 group 64, fp16 scales ----------------------------------------------
 @pytest.mark.parametrize("sdt", ["f16", "f32"])
 def test_config4_flux_attn_proj_w4a4(ops, dev, sdt):
