@@ -563,6 +563,7 @@ def extra_kernels(torch, ops, dev):
                 res[f"gemm_weight_only_{kind}_g128_zeros_{name}_{m}x{n}x{k}"] = {"us": round(us, 2), "TFLOP/s": round(2.0 * m * n * k / us / 1e6, 1)}
     res.update(flux_block_times(torch, ops, dev, timeit))
     res.update(flux_linear_chain_1280(torch, ops, dev, timeit))
+    res.update(flux_mlp_chain_graph(torch, ops, dev, timeit))
     res.update(sdxl_geglu_ffn_chain(torch, ops, dev, timeit))
     res.update(flux_whole_blocks(torch, dev, timeit))
     return res
@@ -697,6 +698,48 @@ def sdxl_geglu_ffn_chain(torch, ops, dev, timeit):
         raise RuntimeError("graph replay of the SDXL INT8 chain differs from the eager result")
     res["sdxl_geglu_ffn_int8_chain_4096_graph_replay"] = {"us": round(us_g, 2), "TOP/s": round(ops_total / us_g / 1e6, 1)}
     return res
+
+
+def flux_mlp_chain_graph(torch, ops, dev, timeit):
+    """The headline chain (BASELINE.json configs[2]) replayed from a HIP graph, next to the same chain launched eagerly: what the
+    four launch gaps of a step cost.  Under capture the input quantiser takes its exchange-free three-kernel route."""
+    m, d, h = 4608, 3072, 12288
+    g = torch.Generator().manual_seed(1003)
+    x = torch.randn(m, d, generator=g).bfloat16().to(dev)
+    wu, su = ops.fp8_quant((torch.randn(h, d, generator=g) * 0.02).bfloat16().to(dev))
+    wd, sd = ops.fp8_quant((torch.randn(d, h, generator=g) * 0.02).bfloat16().to(dev))
+    wu, wd = ops.repack_weight(wu), ops.repack_weight(wd)
+    bu = (torch.randn(h, generator=g) * 0.1).bfloat16().to(dev)
+    bd = (torch.randn(d, generator=g) * 0.1).bfloat16().to(dev)
+    um = torch.zeros(1, dtype=torch.float32, device=dev)
+
+    def chain():
+        qx, sx = ops.fp8_quant(x)
+        um.zero_()
+        u = ops.fp8_linear_max(qx, wu, sx, su, bu, um, torch.bfloat16)
+        qh, sh = ops.fp8_gelu_quant(u, um)
+        return ops.fp8_linear(qh, wd, sh, sd, bd, False, None, 0.0, torch.bfloat16)
+
+    us = timeit(chain, iters=30, warm=20)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        chain()
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        y_static = chain()
+    torch.cuda.synchronize()
+    for _ in range(3):  # every replay against the eager result, with eager work and synchronisations between the replays
+        ref = chain()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        if not torch.equal(y_static, ref):
+            raise RuntimeError("graph replay of the FLUX MLP chain differs from the eager result")
+    us_g = timeit(graph.replay, iters=30, warm=20)
+    flop = 2.0 * m * (d * h + h * d)
+    return {"flux_mlp_fp8_chain_eager_same_input": {"us": round(us, 2), "TFLOP/s": round(flop / us / 1e6, 1)},
+            "flux_mlp_fp8_chain_graph_replay": {"us": round(us_g, 2), "TFLOP/s": round(flop / us_g / 1e6, 1)}}
 
 
 def flux_linear_chain_1280(torch, ops, dev, timeit):
