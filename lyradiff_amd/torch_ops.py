@@ -19,7 +19,8 @@ from . import ops as _ops
 _lib_op = torch.library.custom_op
 NAMES = ("sq_quant", "sq_quant_dynamic", "geglu_int8_dynamic", "int8_linear", "fp8_quant", "fp8_scale_cast", "fp8_linear",
          "w4a4_quant", "w4a4_linear", "repack_weight", "lora_down", "layernorm_mod_fp8", "gate_residual_layernorm_mod_fp8",
-         "fp8_linear_codes", "fp8_linear_gated", "flux_attn_post_fp8", "flux_single_mlp_fp8", "rmsnorm_rope")
+         "fp8_linear_codes", "fp8_linear_gated", "flux_attn_post_fp8", "flux_single_mlp_fp8", "rmsnorm_rope",
+         "fp8_linear_max", "fp8_gelu_quant", "w4a4_quant_lora_down")
 
 
 @_lib_op("lyradiff::sq_quant", mutates_args=())
@@ -97,6 +98,40 @@ def fp8_linear(a_q: Tensor, w_rows32: Tensor, a_scale: Tensor, b_scale: Tensor, 
 @fp8_linear.register_fake
 def _(a_q, w_rows32, a_scale, b_scale, bias=None, gelu=False, residual=None, beta=0.0, out_dtype=torch.bfloat16):
     return a_q.new_empty((a_q.shape[0], w_rows32.shape[0]), dtype=out_dtype)
+
+
+@_lib_op("lyradiff::fp8_linear_max", mutates_args=("out_max",))
+def fp8_linear_max(a_q: Tensor, w_rows32: Tensor, a_scale: Tensor, b_scale: Tensor, bias: Optional[Tensor], out_max: Tensor,
+                   out_dtype: torch.dtype = torch.bfloat16) -> Tensor:
+    return _ops.fp8_linear_max(a_q, w_rows32, a_scale, b_scale, bias, out_max, out_dtype)
+
+
+@fp8_linear_max.register_fake
+def _(a_q, w_rows32, a_scale, b_scale, bias, out_max, out_dtype=torch.bfloat16):
+    return a_q.new_empty((a_q.shape[0], w_rows32.shape[0]), dtype=out_dtype)
+
+
+@_lib_op("lyradiff::fp8_gelu_quant", mutates_args=())
+def fp8_gelu_quant(y: Tensor, y_max: Tensor) -> Tuple[Tensor, Tensor]:
+    return _ops.fp8_gelu_quant(y, y_max)
+
+
+@fp8_gelu_quant.register_fake
+def _(y, y_max):
+    return y.new_empty(y.shape, dtype=torch.uint8), y.new_empty((1,), dtype=torch.float32)
+
+
+@_lib_op("lyradiff::w4a4_quant_lora_down", mutates_args=())
+def w4a4_quant_lora_down(x: Tensor, smooth: Optional[Tensor], lora_down_w: Tensor,
+                         scale_dtype: torch.dtype = torch.float32) -> Tuple[Tensor, Tensor, Tensor]:
+    return _ops.w4a4_quant_lora_down(x, smooth, lora_down_w, scale_dtype)
+
+
+@w4a4_quant_lora_down.register_fake
+def _(x, smooth, lora_down_w, scale_dtype=torch.float32):
+    m, k = x.shape
+    return (x.new_empty((m, k // 8), dtype=torch.int32), x.new_empty((m, k // 64), dtype=scale_dtype),
+            x.new_empty((m, lora_down_w.shape[0])))
 
 
 @_lib_op("lyradiff::w4a4_quant", mutates_args=())

@@ -60,6 +60,13 @@ def test_shape_inference_without_a_gpu(tops):
         out = torch.ops.lyradiff.flux_attn_post_fp8(xs, xs, msa, wf, one, one, b1, wd, one, one, b2)
         assert out.shape == xs.shape and out.dtype == xs.dtype
         assert torch.ops.lyradiff.lora_down(xb, torch.empty(32, 3072, dtype=torch.bfloat16, device=dev)).shape == (4608, 32)
+        # the running-maximum chain and the one-pass W4A4 quantiser
+        u = torch.ops.lyradiff.fp8_linear_max(qf, wf, sf, sf, None, one)
+        assert u.shape == (4608, 12288) and u.dtype == torch.bfloat16
+        qh, sh = torch.ops.lyradiff.fp8_gelu_quant(u, one)
+        assert qh.shape == u.shape and qh.dtype == torch.uint8 and sh.shape == (1,) and sh.dtype == torch.float32
+        w_, s_, a_ = torch.ops.lyradiff.w4a4_quant_lora_down(xb, None, torch.empty(32, 3072, dtype=torch.bfloat16, device=dev))
+        assert w_.shape == (4608, 384) and s_.shape == (4608, 48) and a_.shape == (4608, 32) and a_.dtype == torch.bfloat16
 
 
 def test_host_tensors_are_rejected(tops):
@@ -94,6 +101,16 @@ def test_operators_match_direct_wrappers(tops, dev):
     assert torch.equal(torch.ops.lyradiff.w4a4_linear(qa, w4, sa, sa[:128].contiguous(), None),
                        ops.w4a4_linear(qa, w4, sa, sa[:128].contiguous(), None))
     assert np.isfinite(torch.ops.lyradiff.fp8_scale_cast(xb, sf).float().cpu().numpy()).all()
+    um, um0 = torch.zeros(1, device=dev), torch.zeros(1, device=dev)
+    u = torch.ops.lyradiff.fp8_linear_max(qf, wf, sf, sf, None, um)
+    assert torch.equal(u, ops.fp8_linear_max(qf, wf, sf, sf, None, um0)) and torch.equal(um, um0) and um.item() > 0
+    qh, sh = torch.ops.lyradiff.fp8_gelu_quant(u, um)
+    qh0, sh0 = ops.fp8_gelu_quant(u, um)
+    assert torch.equal(qh, qh0) and torch.equal(sh, sh0)
+    dn = (torch.randn(32, 512, generator=g) * 0.05).bfloat16().to(dev)
+    sm = (torch.rand(512, generator=g) + 0.5).to(dev)
+    got3, ref3 = torch.ops.lyradiff.w4a4_quant_lora_down(xb, sm, dn), ops.w4a4_quant_lora_down(xb, sm, dn)
+    assert all(torch.equal(a, b) for a, b in zip(got3, ref3))
 
 
 @pytest.mark.gpu
