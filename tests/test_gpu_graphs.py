@@ -54,6 +54,49 @@ def test_flux_mlp_fp8_chain_replays_exactly(ops, dev):
         torch.cuda.synchronize()
 
 
+def test_flux_mlp_fp8_running_maximum_chain_replays_exactly(ops, dev):
+    """The chain bench.py times -- persistent GEMM that leaves its largest output, GELU + quantisation in one pass that also
+    clears the other maximum slot -- captured as two steps (so both slots take both roles) and replayed."""
+    m, d, h = 1024, 3072, 12288  # 192 tiles of 256x256: the up projection runs tactic 6/4; the persistent kernel is forced below
+    g = torch.Generator().manual_seed(8)
+    w_up, s_up = ops.fp8_quant((torch.randn(h, d, generator=g) * 0.02).bfloat16().to(dev))
+    w_dn, s_dn = ops.fp8_quant((torch.randn(d, h, generator=g) * 0.02).bfloat16().to(dev))
+    wp_up, wp_dn = ops.repack_weight(w_up), ops.repack_weight(w_dn)
+    b_up = (torch.randn(h, generator=g) * 0.02).bfloat16().to(dev)
+    b_dn = (torch.randn(d, generator=g) * 0.02).bfloat16().to(dev)
+    x = torch.randn(m, d, generator=g).bfloat16().to(dev)
+    slots = [torch.zeros(1, dtype=torch.float32, device=dev) for _ in range(2)]
+
+    def step(inp, k):
+        q, s = ops.fp8_quant(inp)
+        with ops.gemm_thread_tactic(7):
+            u = ops.fp8_linear_max(q, wp_up, s, s_up, b_up, slots[k % 2])
+        q2, s2 = ops.fp8_gelu_quant(u, slots[k % 2], clear_max=slots[(k + 1) % 2])
+        return ops.fp8_linear(q2, wp_dn, s2, s_dn, b_dn, False)
+
+    def two_steps(inp):
+        return step(inp, 0), step(inp * 2, 1)
+
+    side = torch.cuda.Stream()
+    static_x = x.clone()
+    with torch.cuda.stream(side):
+        two_steps(static_x)  # warm-up on the capture stream; leaves slot 0 cleared for the next step 0
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        static_y = two_steps(static_x)
+    for i in range(3):
+        xi = (x * (1.0 + 0.25 * i)).bfloat16()
+        eager = two_steps(xi)
+        torch.cuda.synchronize()
+        static_x.copy_(xi)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y[0], eager[0]) and torch.equal(static_y[1], eager[1]), f"replay {i} differs from the eager result"
+        ops.sq_quant_dynamic(x.half(), None)  # unrelated eager work between replays
+        torch.cuda.synchronize()
+
+
 def test_sdxl_int8_ffn_chain_replays_exactly(ops, dev):
     m, d, inner = 4096, 640, 2560
     g = torch.Generator().manual_seed(6)
