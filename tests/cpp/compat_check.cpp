@@ -211,6 +211,49 @@ int main() {
             }
     }
     std::printf("weight-only path (lq_repack_weight_only + CutlassFpAIntBGemmRunner, group scales and zeros): %d mismatches\n", badwo);
+    // ---------------- W4A4: invokeFusedQuantizeAndLoraDownSimple = one pass over A for words, scales and the rank-32 projection ----
+    int bad4 = 0;
+    {
+        const int qm = 70, qk = 384, rank = 32;
+        std::vector<hip_bfloat16> ha(qm * qk), hd(rank * qk);
+        std::vector<float> hsm(qk);
+        for (auto& v : ha) v = hip_bfloat16(6.0f * lcg(seed));
+        for (auto& v : hd) v = hip_bfloat16(0.2f * lcg(seed));
+        for (auto& v : hsm) v = 0.75f + lcg(seed);
+        hip_bfloat16 *da, *dd; float *dsm, *dC, *dC2, *dsc, *dsc2; uint32_t *dwords, *dwords2;
+        CK(hipMalloc(&da, ha.size() * 2)); CK(hipMalloc(&dd, hd.size() * 2)); CK(hipMalloc(&dsm, qk * 4));
+        CK(hipMalloc(&dC, qm * rank * 4)); CK(hipMalloc(&dC2, qm * rank * 4)); CK(hipMalloc(&dsc, qm * (qk / 64) * 4)); CK(hipMalloc(&dsc2, qm * (qk / 64) * 4));
+        CK(hipMalloc(&dwords, qm * (qk / 8) * 4)); CK(hipMalloc(&dwords2, qm * (qk / 8) * 4));
+        CK(hipMemcpy(da, ha.data(), ha.size() * 2, hipMemcpyHostToDevice)); CK(hipMemcpy(dd, hd.data(), hd.size() * 2, hipMemcpyHostToDevice));
+        CK(hipMemcpy(dsm, hsm.data(), qk * 4, hipMemcpyHostToDevice));
+        try {
+            invokeFusedQuantizeAndLoraDownSimple(dC, dwords, dsc, da, dd, dsm, qm, rank, qk, qk / 64, st);
+            detail::check(lq_w4a4_quantize(dwords2, dsc2, LQ_F32, da, LQ_BF16, dsm, qm, qk, 64, st), "lq_w4a4_quantize");
+            detail::check(lq_lora_down(dC2, LQ_F32, da, dd, LQ_BF16, qm, qk, rank, st), "lq_lora_down");
+        } catch (const std::exception& e) {
+            std::printf("exception: %s\n", e.what());
+            return 5;
+        }
+        CK(hipStreamSynchronize(st));
+        std::vector<uint32_t> w1(qm * (qk / 8)), w2(w1.size());
+        std::vector<float> s1(qm * (qk / 64)), s2(s1.size()), c1(qm * rank);
+        CK(hipMemcpy(w1.data(), dwords, w1.size() * 4, hipMemcpyDeviceToHost)); CK(hipMemcpy(w2.data(), dwords2, w2.size() * 4, hipMemcpyDeviceToHost));
+        CK(hipMemcpy(s1.data(), dsc, s1.size() * 4, hipMemcpyDeviceToHost)); CK(hipMemcpy(s2.data(), dsc2, s2.size() * 4, hipMemcpyDeviceToHost));
+        CK(hipMemcpy(c1.data(), dC, c1.size() * 4, hipMemcpyDeviceToHost));
+        for (size_t i = 0; i < w1.size(); ++i) bad4 += w1[i] != w2[i];
+        for (size_t i = 0; i < s1.size(); ++i) bad4 += s1[i] != s2[i];
+        for (int i = 0; i < qm; ++i)
+            for (int r = 0; r < rank; ++r) {
+                double ref = 0, mag = 0;
+                for (int p = 0; p < qk; ++p) {
+                    const double t = (double)(float)ha[i * qk + p] * (double)(float)hd[r * qk + p];
+                    ref += t;
+                    mag += std::fabs(t);
+                }
+                if (std::fabs((double)c1[i * rank + r] - ref) > 1e-6 * mag + 1e-30) ++bad4;
+            }
+    }
+    std::printf("w4a4 quantise + low-rank down in one pass (invokeFusedQuantizeAndLoraDownSimple): %d mismatches\n", bad4);
     // error convention: exception with the reference's prefix
     bool threw = false;
     try {
@@ -220,5 +263,5 @@ int main() {
         threw = std::string(e.what()).find("[lyradiff Error]") == 0;
     }
     std::printf("bad shape raises std::runtime_error with the reference's prefix: %s\n", threw ? "yes" : "no");
-    return (bad == 0 && badw == 0 && bad8 == 0 && badwo == 0 && threw) ? 0 : 1;
+    return (bad == 0 && badw == 0 && bad8 == 0 && badwo == 0 && bad4 == 0 && threw) ? 0 : 1;
 }

@@ -14,7 +14,7 @@ def test_cpp_reference_style_call_sites(dev):
     r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count(": 0 mismatches") == 3 and "0 outliers" in r.stdout and "prefix: yes" in r.stdout
+    assert r.stdout.count(": 0 mismatches") == 4 and "0 outliers" in r.stdout and "prefix: yes" in r.stdout
 
 
 def test_cpp_layer_types(dev):
