@@ -226,10 +226,11 @@ def main():
     # ---- after the timed region: each kernel alone, launched back to back between ONE pair of events (no marker
     # between launches, so no launch gap inside the figure), on the same rotating inputs
     def batched(fn, n=20):
-        # first until two groups of ten launches agree to 1.5 %: after any pause the device needs some 30 ms of load
-        # before its power management settles, and a figure taken during that ramp is up to 20 % too slow
-        prev = None
-        for _ in range(40):
+        # first at least 40 ms of this kernel's own load, and on until two groups of ten launches agree to 1.5 %: after
+        # any pause the device needs some 30 ms of load before its power management settles, a figure taken during that
+        # ramp is up to 20 % too slow, and two neighbouring groups can agree to 1.5 % half way up the ramp
+        prev, busy_ms = None, 0.0
+        for _ in range(120):
             a, b = ev(), ev()
             a.record()
             for i in range(10):
@@ -237,7 +238,8 @@ def main():
             b.record()
             torch.cuda.synchronize()
             cur = a.elapsed_time(b)
-            if prev is not None and abs(cur - prev) <= 0.015 * prev:
+            busy_ms += cur
+            if busy_ms >= 40.0 and prev is not None and abs(cur - prev) <= 0.015 * prev:
                 break
             prev = cur
         a, b = ev(), ev()
@@ -430,10 +432,10 @@ def extra_kernels(torch, ops, dev):
         for _ in range(warm):
             fn()
         torch.cuda.synchronize()
-        # a kernel of 50 us and more is power limited: run it until two groups of ten launches agree to 1.5 % (the device
-        # needs about 30 ms of load to settle from idle), as the headline benchmark does before its warm-up
-        prev = None
-        for _ in range(30):
+        # a kernel of 50 us and more is power limited: give it at least 40 ms of its own load and run it on until two
+        # groups of ten launches agree to 1.5 % (the device needs about 30 ms of load to settle from idle)
+        prev, busy_ms = None, 0.0
+        for _ in range(120):
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             a.record()
             for _ in range(10):
@@ -441,7 +443,8 @@ def extra_kernels(torch, ops, dev):
             b.record()
             torch.cuda.synchronize()
             cur = a.elapsed_time(b)
-            if cur < 0.5 or (prev is not None and abs(cur - prev) <= 0.015 * prev):
+            busy_ms += cur
+            if cur < 0.5 or (busy_ms >= 40.0 and prev is not None and abs(cur - prev) <= 0.015 * prev):
                 break
             prev = cur
         es = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
