@@ -108,6 +108,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=M)
     ap.add_argument("--extra", action="store_true", help="also time the INT8 / W4A4 / SDXL-shape kernels")
+    ap.add_argument("--row-major", action="store_true",
+                    help="run the chain on row-major quantised activations (the reference's layout) instead of k-panels")
     ap.add_argument("--event-every", type=int, default=2,
                     help="on every N-th timed step ONE kernel is bracketed by a pair of HIP events (the up GEMM on every other "
                          "such step, the three others in turn); markers are not free -- five of them in one step cost the "
@@ -151,13 +153,27 @@ def main():
 
     calls = [0]
 
+    # The four kernels of a step.  Quantised activations travel between them as k-panels [K/64, M, 64] (written by the
+    # quantisers in the same pass, read by the GEMMs in whole cache lines; codes, scales and outputs are bit for bit those
+    # of the row-major calls, which --row-major times instead).
+    if args.row_major:
+        quant_x = ops.fp8_quant
+        gemm_up = lambda q, s, um: ops.fp8_linear_max(q, wp_up, s, s_up, bu, um, torch.bfloat16)
+        quant_h = lambda u, um, nxt: ops.fp8_gelu_quant(u, um, clear_max=nxt)
+        gemm_down = lambda q, s: ops.fp8_linear(q, wp_dn, s, s_dn, bd, False, None, 0.0, torch.bfloat16)
+    else:
+        quant_x = ops.fp8_quant_panels
+        gemm_up = lambda q, s, um: ops.fp8_linear_panels(q, wp_up, s, s_up, bu, um, torch.bfloat16)
+        quant_h = lambda u, um, nxt: ops.fp8_gelu_quant_panels(u, um, clear_max=nxt)
+        gemm_down = lambda q, s: ops.fp8_linear_panels(q, wp_dn, s, s_dn, bd, None, torch.bfloat16)
+
     def step(i, record=None):
         """One pass of the chain; record = index into `names` of the one kernel to bracket with a pair of events."""
         xi = xs[i % n_rot]
         e = (ev(), ev()) if record is not None else None
         if record == 0:
             e[0].record()
-        qx, sx = ops.fp8_quant(xi)
+        qx, sx = quant_x(xi)
         if record == 0:
             e[1].record()
         # the up projection's epilogue also leaves its largest output, from which the next pass derives max|gelu(u)|/448,
@@ -168,17 +184,17 @@ def main():
         calls[0] += 1
         if record == 1:
             e[0].record()
-        u = ops.fp8_linear_max(qx, wp_up, sx, s_up, bu, um, torch.bfloat16)
+        u = gemm_up(qx, sx, um)
         if record == 1:
             e[1].record()
         if record == 2:
             e[0].record()
-        qh, sh = ops.fp8_gelu_quant(u, um, clear_max=um_next)
+        qh, sh = quant_h(u, um, um_next)
         if record == 2:
             e[1].record()
         if record == 3:
             e[0].record()
-        y = ops.fp8_linear(qh, wp_dn, sh, s_dn, bd, False, None, 0.0, torch.bfloat16)
+        y = gemm_down(qh, sh)
         if record == 3:
             e[1].record()
         if record is not None:
@@ -250,24 +266,36 @@ def main():
         torch.cuda.synchronize()
         return a.elapsed_time(b) / n * 1e3
 
-    qx0, sx0 = ops.fp8_quant(xs[0])
+    qx0, sx0 = ops.fp8_quant(xs[0])  # row-major codes for the comparison kernels below
     um0 = torch.zeros(1, dtype=torch.float32, device=dev)
-    u0 = ops.fp8_linear_max(qx0, wp_up, sx0, s_up, bu, um0, torch.bfloat16)
-    qh0, sh0 = ops.fp8_gelu_quant(u0, um0)
+    qxc, sxc = quant_x(xs[0])
+    u0 = gemm_up(qxc, sxc, um0)
+    qh0, sh0 = quant_h(u0, um0, None)
     alone = {
-        "quant_x": batched(lambda i: ops.fp8_quant(xs[i % n_rot])),
-        "gemm_up": batched(lambda i: ops.fp8_linear_max(qx0, wp_up, sx0, s_up, bu, um0, torch.bfloat16)),
-        "quant_h": batched(lambda i: ops.fp8_gelu_quant(u0, um0)),
-        "gemm_down": batched(lambda i: ops.fp8_linear(qh0, wp_dn, sh0, s_dn, bd, False, None, 0.0, torch.bfloat16)),
+        "quant_x": batched(lambda i: quant_x(xs[i % n_rot])),
+        "gemm_up": batched(lambda i: gemm_up(qxc, sxc, um0)),
+        "quant_h": batched(lambda i: quant_h(u0, um0, None)),
+        "gemm_down": batched(lambda i: gemm_down(qh0, sh0)),
     }
+    # the same two GEMMs on row-major activations (every line of the activation is then requested from L2 twice)
+    rows_cmp = None
+    if not args.row_major:
+        qhr, shr = ops.fp8_gelu_quant(u0, um0)
+        rows_cmp = {"gemm_up_us_back_to_back": round(batched(lambda i: ops.fp8_linear_max(qx0, wp_up, sx0, s_up, bu, um0, torch.bfloat16)), 2),
+                    "gemm_down_us_back_to_back": round(batched(lambda i: ops.fp8_linear(qhr, wp_dn, shr, s_dn, bd, False, None, 0.0, torch.bfloat16)), 2)}
+        del qhr
     # the up projection with the activation and the output maximum in its epilogue (not part of the timed chain)
     sg0 = torch.zeros(1, dtype=torch.float32, device=dev)
     up_gelu_us = batched(lambda i: ops.fp8_linear(qx0, wp_up, sx0, s_up, bu, True, None, 0.0, torch.bfloat16, out_scale=sg0))
     # the power argument, checkable from this line: the SAME up-projection kernel on all-zero operands (no switching in
     # the matrix pipe, so the clock is not pulled down), and the shader clock a probe on a second stream sees while the
     # kernel runs on random and on zero operands (idle clock for reference)
-    zq, zw = torch.zeros_like(qx0), torch.zeros_like(wp_up)
-    zeros_us = batched(lambda i: ops.fp8_linear_max(zq, zw, sx0, s_up, bu, um0, torch.bfloat16))
+    zq, zw = torch.zeros_like(qxc), torch.zeros_like(wp_up)
+    if args.row_major:
+        gemm_up_on = lambda q, w: ops.fp8_linear_max(q, w, sx0, s_up, bu, um0, torch.bfloat16)
+    else:
+        gemm_up_on = lambda q, w: ops.fp8_linear_panels(q, w, sx0, s_up, bu, um0, torch.bfloat16)
+    zeros_us = batched(lambda i: gemm_up_on(zq, zw))
 
     def clock_under(fn, per_launch_us=None, n=6):
         side = torch.cuda.Stream()
@@ -288,7 +316,8 @@ def main():
         w8 = ops.unpack_weight(wp_up).view(torch.float8_e4m3fn)
         vendor = {"up_4608x12288x3072": round(batched(lambda i: torch._scaled_mm(a8, w8.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)), 2)}
         del w8
-        h8, wd8 = qh0.view(torch.float8_e4m3fn), ops.unpack_weight(wp_dn).view(torch.float8_e4m3fn)
+        h8 = (qh0 if args.row_major else ops.fp8_panels_to_rows(qh0)).view(torch.float8_e4m3fn)
+        wd8 = ops.unpack_weight(wp_dn).view(torch.float8_e4m3fn)
         vendor["down_4608x3072x12288"] = round(batched(lambda i: torch._scaled_mm(h8, wd8.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)), 2)
         del wd8
     except Exception:  # not every PyTorch build exposes it
@@ -308,8 +337,8 @@ def main():
     pipe_only["zero_operands"]["shader_clock_ghz"] = clock_under(lambda i: ops.mfma_fp8_probe(None, 1000), pipe_only["zero_operands"]["us"])
     clocks = {
         "idle": clock_under(lambda i: None),
-        "up_gemm_random_operands": clock_under(lambda i: ops.fp8_linear_max(qx0, wp_up, sx0, s_up, bu, um0, torch.bfloat16)),
-        "up_gemm_zero_operands": clock_under(lambda i: ops.fp8_linear_max(zq, zw, sx0, s_up, bu, um0, torch.bfloat16)),
+        "up_gemm_random_operands": clock_under(lambda i: gemm_up_on(qxc, wp_up)),
+        "up_gemm_zero_operands": clock_under(lambda i: gemm_up_on(zq, zw)),
     }
     if vendor is not None:
         w8 = ops.unpack_weight(wp_up).view(torch.float8_e4m3fn)
@@ -339,6 +368,8 @@ def main():
                                                                     "TFLOP/s": round(gemm_flops / up_gelu_us / 1e6, 1),
                                                                     "note": "not in the timed chain: the activation in the GEMM's epilogue"},
     }
+    if rows_cmp is not None:
+        kernels["same_gemms_on_row_major_activations"] = rows_cmp
     kernels.update(other)
     achieved = gemm_flops / per["gemm_up"] / 1e6
     traffic, traffic_src = profiled_traffic()
@@ -371,6 +402,7 @@ def main():
         "dtype": "fp8_e4m3", "data": "synthetic",
         "config": {"workload": "FLUX DiT MLP FP8 e4m3 per-tensor, M=4608: act-quant -> GEMM 3072->12288 (+bias) "
                                "-> GELU + act-quant -> GEMM 12288->3072 (+bias), bf16 in/out (BASELINE.json configs[2])",
+                   "quantised_activation_layout": "row-major [M, K]" if args.row_major else "k-panels [K/64, M, 64] written by the quantisers",
                    "tokens": M, "d_model": D, "d_ff": H, "profiled_tactics": tactics,
                    "settle_steps_before_warmup": settled_after, "settle_ms": round(settle_ms, 1)},
         "roofline": roofline, "kernels": kernels,
@@ -716,12 +748,12 @@ def flux_mlp_chain_graph(torch, ops, dev, timeit):
     bd = (torch.randn(d, generator=g) * 0.1).bfloat16().to(dev)
     um = torch.zeros(1, dtype=torch.float32, device=dev)
 
-    def chain():
-        qx, sx = ops.fp8_quant(x)
+    def chain():  # quantised activations as k-panels, as in the headline step
+        qx, sx = ops.fp8_quant_panels(x)
         um.zero_()
-        u = ops.fp8_linear_max(qx, wu, sx, su, bu, um, torch.bfloat16)
-        qh, sh = ops.fp8_gelu_quant(u, um)
-        return ops.fp8_linear(qh, wd, sh, sd, bd, False, None, 0.0, torch.bfloat16)
+        u = ops.fp8_linear_panels(qx, wu, sx, su, bu, um, torch.bfloat16)
+        qh, sh = ops.fp8_gelu_quant_panels(u, um)
+        return ops.fp8_linear_panels(qh, wd, sh, sd, bd, None, torch.bfloat16)
 
     us = timeit(chain, iters=30, warm=20)
     side = torch.cuda.Stream()
@@ -762,13 +794,13 @@ def flux_linear_chain_1280(torch, ops, dev, timeit):
 
     def chain():
         for name, x in (("qkv", xs[0]), ("out", xs[1])):
-            q, s = ops.fp8_quant(x)
-            ops.fp8_linear(q, lin[name][0], s, lin[name][1], lin[name][2])
-        q, s = ops.fp8_quant(xs[2])
+            q, s = ops.fp8_quant_panels(x)
+            ops.fp8_linear_panels(q, lin[name][0], s, lin[name][1], lin[name][2])
+        q, s = ops.fp8_quant_panels(xs[2])
         sh.zero_()
-        u = ops.fp8_linear_max(q, lin["up"][0], s, lin["up"][1], lin["up"][2], sh, torch.bfloat16)
-        qh, s2 = ops.fp8_gelu_quant(u, sh)
-        return ops.fp8_linear(qh, lin["down"][0], s2, lin["down"][1], lin["down"][2])
+        u = ops.fp8_linear_panels(q, lin["up"][0], s, lin["up"][1], lin["up"][2], sh, torch.bfloat16)
+        qh, s2 = ops.fp8_gelu_quant_panels(u, sh)
+        return ops.fp8_linear_panels(qh, lin["down"][0], s2, lin["down"][1], lin["down"][2])
 
     us = timeit(chain, iters=20, warm=3)
     flop = 2.0 * m * d * (3 * d + d + 4 * d + 4 * d)

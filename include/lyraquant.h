@@ -265,6 +265,25 @@ int lq_gemm_fp8_max(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8
 int lq_fp8_gelu_cast(uint8_t* dst, float* scale_out, void* h_out, const void* src, lq_dtype_t dtype, size_t n,
                      const float* src_max, float* clear_max, lq_stream_t stream);
 
+/* ---- FP8 activations in k-panels -------------------------------------------------------------------------------------
+ * A quantised activation [rows, k] stored as [k / 64][rows][64] instead of row-major: element (r, j) lies at byte
+ * ((j / 64) * rows + r) * 64 + j % 64.  The 64 bytes a GEMM k-tile takes from each activation row are then contiguous over
+ * the rows (256 rows = 16 KiB of whole 128-byte cache lines); from a row-major operand a 64-byte k-tile takes half a line
+ * per row and every line is requested from L2 twice, one k-tile apart.  This is to the activation what rows32 is to the
+ * weight: a layout made by the producer (here the quantiser, in the same pass) for the GEMM's transfers.  k % 64 == 0 and
+ * rows * k < 2^32.  The reference has no counterpart (its FP8 activations are row-major, utils/memory_utils.cu:431-446);
+ * codes, scale and GEMM outputs are bit for bit those of the row-major entry points.
+ *   lq_fp8_amax_cast_panels   = lq_fp8_amax_cast (same one-launch form, same fall-back sequence) writing k-panels
+ *   lq_fp8_gelu_cast_panels   = lq_fp8_gelu_cast without h_out, writing k-panels
+ *   lq_gemm_fp8_panels        = lq_gemm_fp8 without activation or residual on such an activation; with out_max also
+ *                               lq_gemm_fp8_max (out_max may be NULL) */
+int lq_fp8_amax_cast_panels(uint8_t* dst_panels, float* scale_out, const void* src, lq_dtype_t dtype, size_t rows, size_t k,
+                            lq_stream_t stream);
+int lq_fp8_gelu_cast_panels(uint8_t* dst_panels, float* scale_out, const void* src, lq_dtype_t dtype, size_t rows, size_t k,
+                            const float* src_max, float* clear_max, lq_stream_t stream);
+int lq_gemm_fp8_panels(void* C, lq_dtype_t out_dtype, const uint8_t* A_panels, const uint8_t* B_rows32, const float* a_scale,
+                       const float* b_scale, const void* bias, int m, int n, int k, float* out_max, lq_stream_t stream);
+
 /* lq_gemm_fp8 (no activation) whose epilogue applies FLUX's gate and second residual:
  *   C[m,n] = T( T( T(y[m,n]) * gate[m / rows_per_gate, n] ) + residual[m,n] ),  y = (sa*sb)*acc + bias[n]
  * with every rounding of the reference's sequence "GEMM stores T, then multiply and add in T": it replaces

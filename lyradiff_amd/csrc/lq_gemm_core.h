@@ -57,6 +57,11 @@ struct GemmParams {
     // the GEMM after it.  Measured on the FLUX MLP chain (113 MB hidden tensor): up + cast + down 340-353 -> 319-330 us
     // together with the nontemporal loads of the cast.
     int stream_c;
+    // A is stored as k-panels [kb / 64][m][64] instead of row-major [m][kb]: the 64 bytes a k-tile takes from each of a
+    // tile's rows are then contiguous (256 rows = 16 KiB, whole 128-byte cache lines), where a row-major operand gives half
+    // a line per row and every line is requested from L2 twice, one k-tile apart (TCP_TCC_READ_REQ per launch at
+    // 4608x3072x12288: 16.2 M row-major, 10.6 M = the operand bytes / 128 in panels).  Kernels with 64-byte k-tiles only.
+    int a_panel;
     // gelu: 0 none, 1 on the fp32 value, 2 on the value rounded to T first (the activation applied by a separate
     // kernel to a stored T tensor)
     // gate: C = T( T( T(y) * gate[m / gate_rows, n] ) + residual[m, n] ), the roundings of a GEMM that stores T
@@ -242,7 +247,9 @@ struct GemmKernel {
         const u32 smem_base = (u32)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
 
         // ---- global -> LDS transfer plan (per lane offsets are fixed; the bases advance with k) ----
-        const uint8_t* a_base = p.A + (size_t)m0 * kb;
+        const u32 a_pitch = p.a_panel ? (u32)BKB : (u32)kb;                      // bytes between two rows of A
+        const size_t a_kstep = p.a_panel ? (size_t)p.m * BKB : (size_t)BKB;  // bytes between two k-tiles of a row
+        const uint8_t* a_base = p.A + (size_t)m0 * a_pitch;
         const uint8_t* b_base = p.B + (size_t)(n0 / 32) * b_block_stride;
         u32 a_voff[A_DMA], b_voff[B_DMA];
         const int row_last = p.m - 1 - m0, blk_last = p.n / 32 - 1 - n0 / 32;
@@ -250,7 +257,7 @@ struct GemmKernel {
         for (int i = 0; i < A_DMA; ++i) {
             int slot = (wave * A_DMA + i) * 64 + lane;  // 16-byte slot inside the A stage
             int row = slot / CH, c = (slot % CH) ^ chunk_swizzle<CH>(row);
-            a_voff[i] = (u32)min(row, row_last) * (u32)kb + c * 16;
+            a_voff[i] = (u32)min(row, row_last) * a_pitch + c * 16;
         }
 #pragma unroll
         for (int i = 0; i < B_DMA; ++i) {
@@ -307,7 +314,7 @@ struct GemmKernel {
         };
 
         auto issue_tile = [&](int kt, int stage) {
-            const uint8_t* ga = a_base + (size_t)kt * BKB;
+            const uint8_t* ga = a_base + (size_t)kt * a_kstep;
             const uint8_t* gb = b_base + (size_t)kt * (BKB * 32);
             const u32 sa = smem_base + stage * STAGE_BYTES + wave * (A_DMA * 1024);
             const u32 sb = smem_base + stage * STAGE_BYTES + A_BYTES + wave * (B_DMA * 1024);
@@ -320,7 +327,7 @@ struct GemmKernel {
         // Transfers lo..hi-1 of a tile (A first, then B), for main loops that spread a tile's transfers
         // between their MFMAs; lo and hi are compile-time values after unrolling.
         auto issue_range = [&](int kt, int stage, int lo, int hi) {
-            const uint8_t* ga = a_base + (size_t)kt * BKB;
+            const uint8_t* ga = a_base + (size_t)kt * a_kstep;
             const uint8_t* gb = b_base + (size_t)kt * (BKB * 32);
             const u32 sa = smem_base + stage * STAGE_BYTES + wave * (A_DMA * 1024);
             const u32 sb = smem_base + stage * STAGE_BYTES + A_BYTES + wave * (B_DMA * 1024);
@@ -885,6 +892,10 @@ static int launch_gemm(GemmParams p, hipStream_t st) {
     if (p.kb % BKB != 0) {
         set_error("gemm: row length %d bytes is not a multiple of the %d-byte k-tile", p.kb, BKB);
         return LQ_ERR_SHAPE;
+    }
+    if (p.a_panel && BKB != 64) {
+        set_error("gemm: an activation in 64-byte k-panels needs a configuration with 64-byte k-tiles");
+        return LQ_ERR_ARG;
     }
     p.tiles_m = (p.m + BM - 1) / BM;
     p.tiles_n = (p.n + BN - 1) / BN;

@@ -32,7 +32,7 @@ template <typename OutTag> static int run_fp8(GemmParams p, hipStream_t st) {
             out_enum<OutTag>() != LQ_F32)
             t = 7;
     }
-    if (t == 1 && p.kb % 128 != 0) t = 0;  // the 128-byte k-tile needs k % 128 == 0
+    if (t == 1 && (p.kb % 128 != 0 || p.a_panel)) t = 0;  // the 128-byte k-tile needs k % 128 == 0 and a row-major activation
     // The per-shape cache is filled by timing the plain epilogue.  With one wavefront per SIMD nothing runs beside tactic 6's
     // epilogue: one that does more than scale and bias (activation, output maximum, codes, gate, residual) costs 13-18 us
     // per 256x256 tile there (transcendentals, or one exposed memory round trip per group of rows) and next to nothing with
@@ -121,6 +121,21 @@ extern "C" int lq_gemm_fp8_max(void* C, lq_dtype_t out_dtype, const uint8_t* A, 
     // two-workgroups-per-CU kernels only: the persistent kernel's counted waits do not get along with such stores)
     p.stream_c = (size_t)m * (size_t)n * (out_dtype == LQ_F32 ? 4 : 2) >= kStreamBytes;
     return fp8_dispatch("lq_gemm_fp8_max", p, out_dtype, stream);
+}
+
+extern "C" int lq_gemm_fp8_panels(void* C, lq_dtype_t out_dtype, const uint8_t* A_panels, const uint8_t* B_rows32,
+                                  const float* a_scale, const float* b_scale, const void* bias, int m, int n, int k,
+                                  float* out_max, lq_stream_t stream) {
+    int rc = fp8_check("lq_gemm_fp8_panels", C, A_panels, B_rows32, a_scale, b_scale, bias, nullptr, m, n, k);
+    if (rc != LQ_OK) return rc > 0 ? LQ_OK : rc;
+    LQ_REQUIRE(C, LQ_ERR_ARG, "lq_gemm_fp8_panels: null pointer");
+    GemmParams p = {};
+    p.C = C; p.A = A_panels; p.B = B_rows32; p.bias = bias; p.a_scale = a_scale; p.b_scale = b_scale;
+    p.out_max = out_max; p.ldc8 = (size_t)n;
+    p.m = m; p.n = n; p.k = k; p.kb = k;
+    p.a_panel = 1;
+    p.stream_c = out_max != nullptr && (size_t)m * (size_t)n * (out_dtype == LQ_F32 ? 4 : 2) >= kStreamBytes;  // as lq_gemm_fp8_max
+    return fp8_dispatch("lq_gemm_fp8_panels", p, out_dtype, stream);
 }
 
 extern "C" int lq_gemm_fp8(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32,

@@ -74,13 +74,15 @@ struct GemmPersist {
         const size_t b_block_stride = (size_t)(kb / 16) * 512;
         const u32 smem_base = (u32)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
 
+        const u32 a_pitch = p.a_panel ? (u32)BKB : (u32)kb;                      // row-major A or k-panels [kb / 64][m][64]
+        const size_t a_kstep = p.a_panel ? (size_t)p.m * BKB : (size_t)BKB;
         // per-lane transfer offsets: every tile is full, so they do not depend on the tile
         u32 a_voff[A_DMA], b_voff[B_DMA];
 #pragma unroll
         for (int i = 0; i < A_DMA; ++i) {
             const int slot = (wave * A_DMA + i) * 64 + lane;
             const int row = slot / CH, c = (slot % CH) ^ chunk_swizzle<CH>(row);
-            a_voff[i] = (u32)row * (u32)kb + c * 16;
+            a_voff[i] = (u32)row * a_pitch + c * 16;
         }
 #pragma unroll
         for (int i = 0; i < B_DMA; ++i) {
@@ -105,12 +107,12 @@ struct GemmPersist {
         auto cursor_at = [&](int tj) -> Cursor {
             int m0, n0;
             tile_origin(tj, m0, n0);
-            return Cursor{p.A + (size_t)m0 * kb, p.B + (size_t)(n0 / 32) * b_block_stride, 0, tj};
+            return Cursor{p.A + (size_t)m0 * a_pitch, p.B + (size_t)(n0 / 32) * b_block_stride, 0, tj};
         };
         auto advance = [&](Cursor& c) {
             if (c.kt + 1 < ktiles) {
                 ++c.kt;
-                c.ga += BKB;
+                c.ga += a_kstep;
                 c.gb += BKB * 32;
             } else if (c.tj + 1 < my_tiles) {
                 c = cursor_at(c.tj + 1);

@@ -43,6 +43,38 @@ template <typename Tag> __device__ __forceinline__ float load_one(const void* ba
     else return static_cast<const float*>(base)[idx];
 }
 
+// Codes written as k-panels [k / 64][rows][64] instead of row-major [rows][k]: the layout in which the 64 bytes a GEMM
+// k-tile takes from each activation row are contiguous over the rows (lq_gemm_fp8_panels).  PanelMap{k = 0} is row-major.
+// A kernel that writes panels walks the tensor in blocks of RB rows x KC 64-element chunks, one block per wavefront and
+// step, every lane taking E consecutive elements of one row (E = 8 or 16: a 16- or 32-byte read, an 8- or 16-byte
+// write): (64 / E) * KC lanes share a row and RB = E / KC rows make a block, so a wavefront reads KC * 64 * sizeof(T)
+// contiguous bytes of each of its rows (whole 128-byte lines) and writes RB x 64 contiguous bytes into each of KC panels.
+// Blocks are numbered along k first; a wavefront's next block is a fixed number of blocks on (quotient and remainder by
+// the blocks per row block come from the host), so the walk costs one 32-bit division per thread.
+struct PanelMap {
+    unsigned k, rows;
+};
+struct PanelStep {  // a fixed advance in blocks, as whole row blocks + remainder along k
+    unsigned dq, dr;
+};
+static PanelStep panel_step(size_t blocks, unsigned kcs) { return PanelStep{(unsigned)(blocks / kcs), (unsigned)(blocks % kcs)}; }
+template <int E, int KC = 1> struct PanelWalk {  // blocks of RB rows x KC 64-element chunks
+    static constexpr int LPR = (64 / E) * KC;  // lanes per row of a block
+    static constexpr int RB = 64 / LPR;        // rows per block
+    unsigned rb, kc;                           // row block and first 64-element chunk of the wavefront's current block
+    unsigned lr, sub, part;                    // this lane's row inside the block, its chunk inside the block's KC, its piece of that chunk
+    __device__ __forceinline__ PanelWalk(unsigned wave, unsigned lane, unsigned kcs)
+        : rb(wave / (kcs / KC)), kc((wave % (kcs / KC)) * KC), lr(lane / LPR), sub((lane % LPR) / (64 / E)), part(lane % (64 / E)) {}
+    __device__ __forceinline__ void step(const PanelStep& d, unsigned kcs) {  // d counts blocks: d.dr blocks along k = d.dr * KC chunks
+        kc += d.dr * KC;
+        rb += d.dq;
+        if (kc >= kcs) { kc -= kcs; ++rb; }
+    }
+    __device__ __forceinline__ unsigned row() const { return rb * RB + lr; }
+    __device__ __forceinline__ size_t src_elem(const PanelMap& pm) const { return (size_t)row() * pm.k + (kc + sub) * 64 + part * E; }
+    __device__ __forceinline__ size_t dst_byte(const PanelMap& pm) const { return ((size_t)(kc + sub) * pm.rows + row()) * 64 + part * E; }
+};
+
 // saturate-to-finite RNE conversion of two floats into the low or high half of a dword
 // (finite inputs and infinities; NaN lanes are patched by the caller)
 __device__ __forceinline__ u32 cvt2_e4m3(float a, float b, u32 old, bool hi) {
@@ -102,23 +134,31 @@ __global__ __launch_bounds__(256) void fp8_amax_kernel(float* __restrict__ scale
     }
 }
 
-template <typename Tag, bool NT>
+template <typename Tag, bool NT, bool PANEL = false>
 __global__ __launch_bounds__(256) void fp8_cast_kernel(uint8_t* __restrict__ dst, const void* __restrict__ src,
-                                                       const float* __restrict__ scale, int invert, size_t n) {
+                                                       const float* __restrict__ scale, int invert, size_t n, PanelMap pm = PanelMap{0, 0},
+                                                       PanelStep stride = PanelStep{0, 0}) {
     constexpr int E = Chunk16<Tag>::elems;
     const float s = scale[0];
     const float r = invert ? 1.0f / s : s;
-    const size_t nchunks = n / E;
-    for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < nchunks; c += (size_t)gridDim.x * blockDim.x) {
+    auto chunk = [&](size_t e, uint8_t* o) {  // E elements from element e on -> E codes at o
         float v[16];
-        load_elems<Tag, NT>(src, c * E, v);
+        load_elems<Tag, NT>(src, e, v);
         u32 w[4];
 #pragma unroll
         for (int i = 0; i < E / 4; ++i)
             w[i] = cvt4_e4m3(v[4 * i] * r, v[4 * i + 1] * r, v[4 * i + 2] * r, v[4 * i + 3] * r);
-        if constexpr (E == 16) *reinterpret_cast<uint4*>(dst + c * 16) = make_uint4(w[0], w[1], w[2], w[3]);
-        else *reinterpret_cast<uint2*>(dst + c * 8) = make_uint2(w[0], w[1]);
+        if constexpr (E == 16) *reinterpret_cast<uint4*>(o) = make_uint4(w[0], w[1], w[2], w[3]);
+        else *reinterpret_cast<uint2*>(o) = make_uint2(w[0], w[1]);
+    };
+    if constexpr (PANEL) {
+        const unsigned kcs = pm.k / 64, nrb = (pm.rows + E - 1) / E;
+        for (PanelWalk<E> pw((blockIdx.x * blockDim.x + threadIdx.x) >> 6, threadIdx.x & 63, kcs); pw.rb < nrb; pw.step(stride, kcs))
+            if (pw.row() < pm.rows) chunk(pw.src_elem(pm), dst + pw.dst_byte(pm));
+        return;
     }
+    const size_t nchunks = n / E;
+    for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < nchunks; c += (size_t)gridDim.x * blockDim.x) chunk(c * E, dst + c * E);
     if (blockIdx.x == 0) {
         size_t i = nchunks * E + threadIdx.x;
         if (i < n) dst[i] = (uint8_t)cvt1_e4m3(load_one<Tag>(src, i) * r);
@@ -133,10 +173,12 @@ __global__ __launch_bounds__(256) void fp8_cast_kernel(uint8_t* __restrict__ dst
 // the kernel takes that route from ymax >= 0.5 (h = 0.345).  Below that -- a tensor without a single output of 0.5 or more --
 // the scale comes from the bound max(h(ymax), kGeluNegBound) instead of the exact maximum.
 constexpr float kGeluNegBound = 0.171875f;  // >= |gelu(y)| for every y < 0; a value of fp16 and bf16
-template <typename Tag, bool NT, bool WANT_H>
+// PANEL: 0 = row-major codes; 1 or 4 = k-panels, walked in blocks of PANEL 64-element chunks per row (PanelWalk)
+template <typename Tag, bool NT, bool WANT_H, int PANEL = 0>
 __global__ __launch_bounds__(256) void fp8_gelu_cast_kernel(uint8_t* __restrict__ dst, float* __restrict__ scale_out,
                                                             void* __restrict__ h_out, const void* __restrict__ src,
-                                                            const float* __restrict__ src_max, float* __restrict__ clear, size_t n) {
+                                                            const float* __restrict__ src_max, float* __restrict__ clear, size_t n,
+                                                            PanelMap pm = PanelMap{0, 0}, PanelStep stride = PanelStep{0, 0}) {
     constexpr int E = Chunk16<Tag>::elems;
     if (clear != nullptr && blockIdx.x == 0 && threadIdx.x == 0) clear[0] = 0.0f;  // the next call's slot for a running maximum
     const float ym = round_through<Tag>(fmaxf(src_max[0], 0.0f));
@@ -145,10 +187,9 @@ __global__ __launch_bounds__(256) void fp8_gelu_cast_kernel(uint8_t* __restrict_
     const float s = amax / 448.0f;
     const float r = 1.0f / s;
     if (blockIdx.x == 0 && threadIdx.x == 0) scale_out[0] = s;
-    const size_t nchunks = n / E;
-    for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < nchunks; c += (size_t)gridDim.x * blockDim.x) {
+    auto chunk = [&](size_t e, uint8_t* o) {  // E elements from element e on -> h (row-major, optional) and E codes at o
         float v[16];
-        load_elems<Tag, NT>(src, c * E, v);
+        load_elems<Tag, NT>(src, e, v);
 #pragma unroll
         for (int i = 0; i < E; i += 2) {
             v[i] = gelu_fast(v[i]);
@@ -156,24 +197,34 @@ __global__ __launch_bounds__(256) void fp8_gelu_cast_kernel(uint8_t* __restrict_
             round_through2<Tag>(v[i], v[i + 1]);
         }
         if constexpr (WANT_H) {
+            char* ho = static_cast<char*>(h_out) + (e / E) * 32;
             if constexpr (Elem<Tag>::bytes == 2) {
                 u32 hw[E / 2];
 #pragma unroll
                 for (int i = 0; i < E / 2; ++i) hw[i] = Elem<Tag>::store(v[2 * i]) | (Elem<Tag>::store(v[2 * i + 1]) << 16);
-                *reinterpret_cast<uint4*>(static_cast<char*>(h_out) + c * 32) = make_uint4(hw[0], hw[1], hw[2], hw[3]);
-                *reinterpret_cast<uint4*>(static_cast<char*>(h_out) + c * 32 + 16) = make_uint4(hw[4], hw[5], hw[6], hw[7]);
+                *reinterpret_cast<uint4*>(ho) = make_uint4(hw[0], hw[1], hw[2], hw[3]);
+                *reinterpret_cast<uint4*>(ho + 16) = make_uint4(hw[4], hw[5], hw[6], hw[7]);
             } else {
-                *reinterpret_cast<float4*>(static_cast<char*>(h_out) + c * 32) = make_float4(v[0], v[1], v[2], v[3]);
-                *reinterpret_cast<float4*>(static_cast<char*>(h_out) + c * 32 + 16) = make_float4(v[4], v[5], v[6], v[7]);
+                *reinterpret_cast<float4*>(ho) = make_float4(v[0], v[1], v[2], v[3]);
+                *reinterpret_cast<float4*>(ho + 16) = make_float4(v[4], v[5], v[6], v[7]);
             }
         }
         u32 w[4];
 #pragma unroll
         for (int i = 0; i < E / 4; ++i)
             w[i] = cvt4_e4m3(v[4 * i] * r, v[4 * i + 1] * r, v[4 * i + 2] * r, v[4 * i + 3] * r);
-        if constexpr (E == 16) *reinterpret_cast<uint4*>(dst + c * 16) = make_uint4(w[0], w[1], w[2], w[3]);
-        else *reinterpret_cast<uint2*>(dst + c * 8) = make_uint2(w[0], w[1]);
+        if constexpr (E == 16) *reinterpret_cast<uint4*>(o) = make_uint4(w[0], w[1], w[2], w[3]);
+        else *reinterpret_cast<uint2*>(o) = make_uint2(w[0], w[1]);
+    };
+    if constexpr (PANEL != 0) {
+        using Walk = PanelWalk<E, PANEL>;
+        const unsigned kcs = pm.k / 64, nrb = (pm.rows + Walk::RB - 1) / Walk::RB;
+        for (Walk pw((blockIdx.x * blockDim.x + threadIdx.x) >> 6, threadIdx.x & 63, kcs); pw.rb < nrb; pw.step(stride, kcs))
+            if (pw.row() < pm.rows) chunk(pw.src_elem(pm), dst + pw.dst_byte(pm));
+        return;
     }
+    const size_t nchunks = n / E;
+    for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < nchunks; c += (size_t)gridDim.x * blockDim.x) chunk(c * E, dst + c * E);
     if (blockIdx.x == 0) {
         size_t i = nchunks * E + threadIdx.x;
         if (i < n) {
@@ -385,11 +436,12 @@ __device__ __forceinline__ unsigned long long poll_tagged(const unsigned long lo
     return v;
 }
 
-template <typename Tag, int KEEP>
+template <typename Tag, int KEEP, bool PANEL = false>
 __global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_t* __restrict__ dst, float* __restrict__ scale_out,
                                                                           const void* __restrict__ src, size_t n, CoopSlot* slot,
                                                                           unsigned launch, unsigned* timeout,
-                                                                          unsigned long long* __restrict__ stamps) {
+                                                                          unsigned long long* __restrict__ stamps,
+                                                                          PanelMap pm = PanelMap{0, 0}, PanelStep round_step = PanelStep{0, 0}) {
     // stamps (NULL in every product launch): four readings of the constant 100 MHz clock per workgroup -- started, partial
     // maximum formed (its loads are back), released from the exchange, stores acknowledged (lq_fp8_amax_cast_timeline)
     if (stamps != nullptr && threadIdx.x == 0) stamps[blockIdx.x * 4] = wall_clock64();
@@ -402,6 +454,32 @@ __global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_
     const size_t wave = ((size_t)blockIdx.x * kCoopThreads + threadIdx.x) >> 6;
     const size_t nwaves = (size_t)gridDim.x * (kCoopThreads / 64);
     const char* in = static_cast<const char*>(src) + lane * 16;
+    uint8_t* out = dst + lane * E2;
+    // Where this lane's 16-byte piece number j of the wavefront comes from and where its codes go.  Row-major: pieces 2i and
+    // 2i + 1 are pieces `lane` and `lane + 64` of the wavefront's block i (2 KiB of consecutive elements; blocks wave,
+    // wave + nwaves, ...).  k-panels: piece j lies in the wavefront's j-th block of E2 rows x 64 elements (PanelWalk: 64 / E2
+    // lanes share a row, so one load instruction reads whole 128-byte lines and one store writes E2 x 64 contiguous bytes).
+    struct Place {
+        const char* p;
+        uint8_t* o;
+        bool ok;
+    };
+    const unsigned kcs = PANEL ? pm.k / 64 : 1, nrb = PANEL ? (pm.rows + E2 - 1) / E2 : 0;
+    PanelWalk<E2> pw((unsigned)wave, (unsigned)lane, kcs);
+    auto rewind = [&]() { pw = PanelWalk<E2>((unsigned)wave, (unsigned)lane, kcs); };
+    auto place = [&](size_t j) -> Place {  // k-panels: of the walk's current block, which the caller steps once per piece
+        if constexpr (PANEL) {
+            return Place{static_cast<const char*>(src) + pw.src_elem(pm) * Elem<Tag>::bytes, dst + pw.dst_byte(pm),
+                         pw.rb < nrb && pw.row() < pm.rows};
+        } else {
+            const size_t b = wave + (j >> 1) * nwaves;
+            return Place{in + b * 2048 + (j & 1) * 1024, out + b * BLK + (j & 1) * (64 * E2), b < nblocks};
+        }
+    };
+    auto more = [&](size_t j) -> bool {  // pieces left for this wavefront
+        if constexpr (PANEL) return pw.rb < nrb;
+        else return wave + (j >> 1) * nwaves < nblocks;
+    };
     uint4 keep[KEEP][2];
     float amax = 0.0f;
     auto piece_amax = [&](const uint4& v) {
@@ -412,27 +490,26 @@ __global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_
         for (int i = 0; i < E2; ++i) amax = fmaxf(amax, fabsf(f[i]));
     };
 #pragma unroll
-    for (int it = 0; it < KEEP; ++it) {
-        const size_t b = wave + it * nwaves;
-        keep[it][0] = make_uint4(0, 0, 0, 0);
-        keep[it][1] = make_uint4(0, 0, 0, 0);
-        if (b < nblocks) {
-            const u32x4_t a = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(in + b * 2048));
-            const u32x4_t c = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(in + b * 2048 + 1024));
-            keep[it][0] = make_uint4(a.x, a.y, a.z, a.w);
-            keep[it][1] = make_uint4(c.x, c.y, c.z, c.w);
+    for (int j = 0; j < 2 * KEEP; ++j) {
+        const Place pl = place(j);
+        keep[j >> 1][j & 1] = make_uint4(0, 0, 0, 0);
+        if (pl.ok) {
+            const u32x4_t a = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(pl.p));
+            keep[j >> 1][j & 1] = make_uint4(a.x, a.y, a.z, a.w);
         }
+        if constexpr (PANEL) pw.step(round_step, kcs);
     }
 #pragma unroll
     for (int it = 0; it < KEEP; ++it) {
         piece_amax(keep[it][0]);
         piece_amax(keep[it][1]);
     }
-    for (size_t b = wave + KEEP * nwaves; b < nblocks; b += nwaves) {  // what the registers cannot hold is read twice
-        piece_amax(*reinterpret_cast<const uint4*>(in + b * 2048));
-        piece_amax(*reinterpret_cast<const uint4*>(in + b * 2048 + 1024));
+    for (size_t j = 2 * KEEP; more(j); ++j) {  // what the registers cannot hold is read twice
+        const Place pl = place(j);
+        if (pl.ok) piece_amax(*reinterpret_cast<const uint4*>(pl.p));
+        if constexpr (PANEL) pw.step(round_step, kcs);
     }
-    if (blockIdx.x == 0)  // fewer than BLK trailing elements
+    if (!PANEL && blockIdx.x == 0)  // fewer than BLK trailing elements (the blocks of the k-panel walk cover every element)
         for (size_t i = nblocks * BLK + threadIdx.x; i < n; i += kCoopThreads) amax = fmaxf(amax, fabsf(load_one<Tag>(src, i)));
     __shared__ float red[kCoopThreads / 64];
     __shared__ float tensor_max;
@@ -486,7 +563,6 @@ __global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_
         for (int u = 0; u < 2; ++u)
             asm volatile("" : "+v"(keep[it][u].x), "+v"(keep[it][u].y), "+v"(keep[it][u].z), "+v"(keep[it][u].w));
     const float r = 1.0f / s;
-    uint8_t* out = dst + lane * E2;
     auto piece_cast = [&](const uint4& v, uint8_t* o, bool stream_out) {
         float f[8];
         if constexpr (E2 == 8) unpack8<Tag>(v, f);
@@ -501,19 +577,19 @@ __global__ __launch_bounds__(kCoopThreads) void fp8_amax_cast_coop_kernel(uint8_
             else *reinterpret_cast<u32*>(o) = w0;
         }
     };
+    rewind();
 #pragma unroll
-    for (int it = 0; it < KEEP; ++it) {
-        const size_t b = wave + it * nwaves;
-        if (b < nblocks) {
-            piece_cast(keep[it][0], out + b * BLK, true);
-            piece_cast(keep[it][1], out + b * BLK + 64 * E2, true);
-        }
+    for (int j = 0; j < 2 * KEEP; ++j) {
+        const Place pl = place(j);
+        if (pl.ok) piece_cast(keep[j >> 1][j & 1], pl.o, true);
+        if constexpr (PANEL) pw.step(round_step, kcs);
     }
-    for (size_t b = wave + KEEP * nwaves; b < nblocks; b += nwaves) {
-        piece_cast(*reinterpret_cast<const uint4*>(in + b * 2048), out + b * BLK, true);
-        piece_cast(*reinterpret_cast<const uint4*>(in + b * 2048 + 1024), out + b * BLK + 64 * E2, true);
+    for (size_t j = 2 * KEEP; more(j); ++j) {
+        const Place pl = place(j);
+        if (pl.ok) piece_cast(*reinterpret_cast<const uint4*>(pl.p), pl.o, true);
+        if constexpr (PANEL) pw.step(round_step, kcs);
     }
-    if (blockIdx.x == 0)
+    if (!PANEL && blockIdx.x == 0)
         for (size_t i = nblocks * BLK + threadIdx.x; i < n; i += kCoopThreads) dst[i] = (uint8_t)cvt1_e4m3(load_one<Tag>(src, i) * r);
     if (stamps != nullptr) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's stores are acknowledged
@@ -548,7 +624,7 @@ template <typename Tag, int KEEP> struct CoopCapacity {
 
 template <typename Tag, int KEEP>
 static int launch_coop_keep(uint8_t* dst, float* scale_out, const void* src, size_t n, hipStream_t st, int dev, FusedScratch* ws,
-                            size_t waves_needed, unsigned long long* stamps) {
+                            size_t waves_needed, unsigned long long* stamps, PanelMap pm) {
     const int num_cu = CoopCapacity<Tag, KEEP>::get(dev).num_cu;
     if (num_cu == 0) return 1;
     unsigned launch = 0;
@@ -558,14 +634,24 @@ static int launch_coop_keep(uint8_t* dst, float* scale_out, const void* src, siz
     if (grid > (size_t)num_cu) grid = num_cu;
     if (grid > kCoopMaxBlocks) grid = kCoopMaxBlocks;
     if (grid == 0) grid = 1;
-    hipLaunchKernelGGL((fp8_amax_cast_coop_kernel<Tag, KEEP>), dim3((unsigned)grid), dim3(kCoopThreads), 0, st, dst, scale_out, src, n,
-                       &ws->coop[slot], launch, &ws->timeout, stamps);
+    if (pm.k != 0) {
+        if constexpr (KEEP > 8) {  // the k-panel walk's addresses do not fit beside ten kept chunks (53 registers spilled):
+            return 1;              // the caller keeps eight and reads the rest twice
+        } else {
+            const size_t nwaves = grid * (kCoopThreads / 64);
+            hipLaunchKernelGGL((fp8_amax_cast_coop_kernel<Tag, KEEP, true>), dim3((unsigned)grid), dim3(kCoopThreads), 0, st, dst,
+                               scale_out, src, n, &ws->coop[slot], launch, &ws->timeout, stamps, pm, panel_step(nwaves, pm.k / 64));
+        }
+    } else {
+        hipLaunchKernelGGL((fp8_amax_cast_coop_kernel<Tag, KEEP>), dim3((unsigned)grid), dim3(kCoopThreads), 0, st, dst, scale_out, src,
+                           n, &ws->coop[slot], launch, &ws->timeout, stamps);
+    }
     return check_launch("fp8_amax_cast_fused");
 }
 
 template <typename Tag>
 static int launch_amax_cast_coop(uint8_t* dst, float* scale_out, const void* src, size_t n, hipStream_t st,
-                                 unsigned long long* stamps = nullptr) {
+                                 unsigned long long* stamps = nullptr, PanelMap pm = PanelMap{0, 0}) {
     if (reinterpret_cast<uintptr_t>(src) % 16 != 0 || reinterpret_cast<uintptr_t>(dst) % 16 != 0) return 1;
     if (st == hipStreamPerThread) return 1;  // one handle for every thread's own stream: its launches can overlap
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
@@ -576,14 +662,18 @@ static int launch_amax_cast_coop(uint8_t* dst, float* scale_out, const void* src
     int dev = 0;
     FusedScratch* ws = device_scratch(&dev);
     if (ws == nullptr) return LQ_ERR_HIP;
-    const size_t blocks = n / (Elem<Tag>::bytes == 2 ? 1024 : 512);  // 2 KiB blocks, one per wavefront and kept chunk
+    size_t blocks = n / (Elem<Tag>::bytes == 2 ? 1024 : 512);  // 2 KiB blocks, one per wavefront and kept chunk
+    if (pm.k != 0) {  // k-panels: two blocks of 8 (4 for fp32) rows x 64 elements per kept chunk, the last row block may be partial
+        const size_t rb = Elem<Tag>::bytes == 2 ? 8 : 4;
+        blocks = (((pm.rows + rb - 1) / rb) * (pm.k / 64) + 1) / 2;
+    }
     const int num_cu = CoopCapacity<Tag, 4>::get(dev).num_cu;
     if (num_cu == 0) return 1;
     const size_t waves = (size_t)num_cu * (kCoopThreads / 64);
     const size_t per_wave = (blocks + waves - 1) / waves;
-    if (per_wave <= 4) return launch_coop_keep<Tag, 4>(dst, scale_out, src, n, st, dev, ws, blocks, stamps);
-    if (per_wave <= 8) return launch_coop_keep<Tag, 8>(dst, scale_out, src, n, st, dev, ws, blocks, stamps);
-    return launch_coop_keep<Tag, 10>(dst, scale_out, src, n, st, dev, ws, blocks, stamps);
+    if (per_wave <= 4) return launch_coop_keep<Tag, 4>(dst, scale_out, src, n, st, dev, ws, blocks, stamps, pm);
+    if (per_wave <= 8 || pm.k != 0) return launch_coop_keep<Tag, 8>(dst, scale_out, src, n, st, dev, ws, blocks, stamps, pm);
+    return launch_coop_keep<Tag, 10>(dst, scale_out, src, n, st, dev, ws, blocks, stamps, pm);
 }
 
 // ---- two launches, no barrier: partial maxima + ticket, then the cast ------------------------------------------------
@@ -687,7 +777,14 @@ template <typename Tag> static int launch_amax(float* scale, const void* x, size
     return check_launch("fp8_amax");
 }
 template <typename Tag>
-static int launch_cast(uint8_t* dst, const void* src, const float* scale, int invert, size_t n, hipStream_t st) {
+static int launch_cast(uint8_t* dst, const void* src, const float* scale, int invert, size_t n, hipStream_t st,
+                       PanelMap pm = PanelMap{0, 0}) {
+    if (pm.k != 0) {  // k-panels: the caller has checked the alignment (every piece of 8 or 16 elements stays inside a 64-element chunk)
+        const unsigned grid = stream_grid(n, Chunk16<Tag>::elems);
+        hipLaunchKernelGGL((fp8_cast_kernel<Tag, false, true>), dim3(grid), dim3(256), 0, st, dst, src, scale, invert, n, pm,
+                           panel_step((size_t)grid * 4, pm.k / 64));
+        return check_launch("fp8_cast");
+    }
     if (reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0) {
         if (n * Elem<Tag>::bytes >= kStreamBytes)
             hipLaunchKernelGGL((fp8_cast_kernel<Tag, true>), dim3(stream_grid(n, Chunk16<Tag>::elems)), dim3(256), 0, st, dst, src, scale, invert, n);
@@ -737,10 +834,19 @@ extern "C" int lq_fp8_scale_cast(uint8_t* dst, const void* src, lq_dtype_t dtype
 
 template <typename Tag>
 static int launch_gelu_cast(uint8_t* dst, float* scale_out, void* h_out, const void* src, const float* src_max, float* clear, size_t n,
-                            hipStream_t st) {
+                            hipStream_t st, PanelMap pm = PanelMap{0, 0}) {
     const dim3 grid(stream_grid(n, Chunk16<Tag>::elems)), block(256);
     const bool nt = n * Elem<Tag>::bytes >= kStreamBytes;
-    if (h_out != nullptr) {
+    if (pm.k != 0) {
+        // blocks of 4 rows x 256 elements where k allows it (512 contiguous bytes per source row; 4608x12288 bf16: 34.3 us against
+        // 35.9 with 16 rows x 64 elements and 33.6 row-major), else 16 rows x 64 elements
+        const bool wide = (pm.k / 64) % 4 == 0;
+        const PanelStep stride = panel_step((size_t)grid.x * 4, pm.k / 64 / (wide ? 4 : 1));  // a wavefront's next block: one per wavefront of the grid on
+        if (wide && nt) hipLaunchKernelGGL((fp8_gelu_cast_kernel<Tag, true, false, 4>), grid, block, 0, st, dst, scale_out, h_out, src, src_max, clear, n, pm, stride);
+        else if (wide) hipLaunchKernelGGL((fp8_gelu_cast_kernel<Tag, false, false, 4>), grid, block, 0, st, dst, scale_out, h_out, src, src_max, clear, n, pm, stride);
+        else if (nt) hipLaunchKernelGGL((fp8_gelu_cast_kernel<Tag, true, false, 1>), grid, block, 0, st, dst, scale_out, h_out, src, src_max, clear, n, pm, stride);
+        else hipLaunchKernelGGL((fp8_gelu_cast_kernel<Tag, false, false, 1>), grid, block, 0, st, dst, scale_out, h_out, src, src_max, clear, n, pm, stride);
+    } else if (h_out != nullptr) {
         hipLaunchKernelGGL((fp8_gelu_cast_kernel<Tag, false, true>), grid, block, 0, st, dst, scale_out, h_out, src, src_max, clear, n);
     } else if (nt) {
         hipLaunchKernelGGL((fp8_gelu_cast_kernel<Tag, true, false>), grid, block, 0, st, dst, scale_out, h_out, src, src_max, clear, n);
@@ -765,6 +871,61 @@ extern "C" int lq_fp8_gelu_cast(uint8_t* dst, float* scale_out, void* h_out, con
         case LQ_F32: return launch_gelu_cast<F32Tag>(dst, scale_out, h_out, src, src_max, clear_max, n, as_stream(stream));
         default: set_error("lq_fp8_gelu_cast: unsupported dtype %d", (int)dtype); return LQ_ERR_UNSUPPORTED;
     }
+}
+
+// LQ_OK, or the error for a shape the k-panel layout does not take
+static int panels_check(const char* what, const void* dst, const void* src, size_t rows, size_t k) {
+    LQ_REQUIRE(k % 64 == 0 && rows * k <= 0xFFFFFFFFull, LQ_ERR_SHAPE,
+               "%s: k-panels need k %% 64 == 0 and fewer than 2^32 elements (rows=%zu k=%zu)", what, rows, k);
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0, LQ_ERR_ARG,
+               "%s: src and dst must be 16-byte aligned", what);
+    return LQ_OK;
+}
+
+extern "C" int lq_fp8_amax_cast_panels(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t rows, size_t k,
+                                       lq_stream_t stream) {
+    const size_t n = rows * k;
+    LQ_REQUIRE(scale_out && ((dst && src) || n == 0), LQ_ERR_ARG, "lq_fp8_amax_cast_panels: null pointer");
+    LQ_REQUIRE(dtype == LQ_F16 || dtype == LQ_BF16 || dtype == LQ_F32, LQ_ERR_UNSUPPORTED, "lq_fp8_amax_cast_panels: unsupported dtype %d",
+               (int)dtype);
+    if (n == 0) return lq_fp8_amax_cast(dst, scale_out, src, dtype, 0, stream);
+    int rc = panels_check("lq_fp8_amax_cast_panels", dst, src, rows, k);
+    if (rc != LQ_OK) return rc;
+    const PanelMap pm{(unsigned)k, (unsigned)rows};
+    hipStream_t st = as_stream(stream);
+    if (n >= 4096) {
+        rc = dtype == LQ_F16    ? launch_amax_cast_coop<F16Tag>(dst, scale_out, src, n, st, nullptr, pm)
+             : dtype == LQ_BF16 ? launch_amax_cast_coop<BF16Tag>(dst, scale_out, src, n, st, nullptr, pm)
+                                : launch_amax_cast_coop<F32Tag>(dst, scale_out, src, n, st, nullptr, pm);
+        if (rc <= 0) return rc;
+    }
+    // scratch-free sequence, as in lq_fp8_amax_cast
+    hipLaunchKernelGGL(fill_f32_kernel, dim3(1), dim3(1), 0, st, scale_out, 0.0f);
+    rc = check_launch("fp8_amax_cast_panels(fill)");
+    if (rc != LQ_OK) return rc;
+    rc = lq_fp8_amax_scale(scale_out, src, dtype, n, stream);
+    if (rc != LQ_OK) return rc;
+    return dtype == LQ_F16    ? launch_cast<F16Tag>(dst, src, scale_out, 1, n, st, pm)
+           : dtype == LQ_BF16 ? launch_cast<BF16Tag>(dst, src, scale_out, 1, n, st, pm)
+                              : launch_cast<F32Tag>(dst, src, scale_out, 1, n, st, pm);
+}
+
+extern "C" int lq_fp8_gelu_cast_panels(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t rows, size_t k,
+                                       const float* src_max, float* clear_max, lq_stream_t stream) {
+    const size_t n = rows * k;
+    LQ_REQUIRE(scale_out && src_max && ((dst && src) || n == 0), LQ_ERR_ARG, "lq_fp8_gelu_cast_panels: null pointer");
+    LQ_REQUIRE(clear_max != src_max && clear_max != scale_out, LQ_ERR_ARG,
+               "lq_fp8_gelu_cast_panels: clear_max must not be the slot this call reads or the scale it writes");
+    LQ_REQUIRE(dtype == LQ_F16 || dtype == LQ_BF16 || dtype == LQ_F32, LQ_ERR_UNSUPPORTED, "lq_fp8_gelu_cast_panels: unsupported dtype %d",
+               (int)dtype);
+    if (n == 0) return LQ_OK;
+    int rc = panels_check("lq_fp8_gelu_cast_panels", dst, src, rows, k);
+    if (rc != LQ_OK) return rc;
+    const PanelMap pm{(unsigned)k, (unsigned)rows};
+    hipStream_t st = as_stream(stream);
+    return dtype == LQ_F16    ? launch_gelu_cast<F16Tag>(dst, scale_out, nullptr, src, src_max, clear_max, n, st, pm)
+           : dtype == LQ_BF16 ? launch_gelu_cast<BF16Tag>(dst, scale_out, nullptr, src, src_max, clear_max, n, st, pm)
+                              : launch_gelu_cast<F32Tag>(dst, scale_out, nullptr, src, src_max, clear_max, n, st, pm);
 }
 
 extern "C" int lq_fp8_scale_cast_2d(uint8_t* dst, size_t dst_ld, const void* src, size_t src_ld, lq_dtype_t dtype,

@@ -497,6 +497,70 @@ def fp8_gelu_quant(y, y_max, want_h: bool = False, clear_max=None):
     return (q, s, h) if want_h else (q, s)
 
 
+# ---- activations in k-panels ------------------------------------------------------------------------------------------
+# A quantised activation [M, K] stored as [K/64, M, 64] (k-panels): the 64 bytes a GEMM k-tile takes from each row are then
+# contiguous over the rows, so the GEMM's transfers fetch whole 128-byte cache lines (a row-major operand gives half a line
+# per row and every line is requested from L2 twice).  The quantisers write the layout directly; the GEMM results are the
+# bits of the row-major calls.  K % 64 == 0.
+
+def fp8_panels_to_rows(q_panels):
+    """[K/64, M, 64] k-panels -> the row-major [M, K] tensor (a copy; for checks and for consumers of the plain layout)."""
+    kp, m, w = q_panels.shape
+    return q_panels.permute(1, 0, 2).reshape(m, kp * w).contiguous()
+
+
+def fp8_quant_panels(x):
+    """fp8_quant of a 2-D x [M, K] with the codes written as k-panels: returns (uint8 [K/64, M, 64], scale fp32 [1])."""
+    _chk(x, "x", _FLOATS)
+    if x.dim() != 2 or x.shape[1] % 64 != 0:
+        raise ValueError("fp8_quant_panels: x must be [M, K] with K % 64 == 0")
+    m, k = x.shape
+    q = torch.empty((k // 64, m, 64), dtype=torch.uint8, device=x.device)
+    s = torch.empty(1, dtype=torch.float32, device=x.device)
+    _l.check(_l.load().lq_fp8_amax_cast_panels(_ptr(q), _ptr(s), _ptr(x), _DT[x.dtype], m, k, _stream()), "lq_fp8_amax_cast_panels")
+    return q, s
+
+
+def fp8_gelu_quant_panels(y, y_max, clear_max=None):
+    """fp8_gelu_quant of a 2-D y [M, K] with the codes written as k-panels [K/64, M, 64]."""
+    _chk(y, "y", _FLOATS)
+    _chk(y_max, "y_max", (torch.float32,))
+    if clear_max is not None:
+        _chk(clear_max, "clear_max", (torch.float32,))
+    if y.dim() != 2 or y.shape[1] % 64 != 0:
+        raise ValueError("fp8_gelu_quant_panels: y must be [M, K] with K % 64 == 0")
+    m, k = y.shape
+    q = torch.empty((k // 64, m, 64), dtype=torch.uint8, device=y.device)
+    s = torch.empty(1, dtype=torch.float32, device=y.device)
+    _l.check(_l.load().lq_fp8_gelu_cast_panels(_ptr(q), _ptr(s), _ptr(y), _DT[y.dtype], m, k, _ptr(y_max), _ptr(clear_max), _stream()),
+             "lq_fp8_gelu_cast_panels")
+    return q, s
+
+
+def fp8_linear_panels(a_panels, w_rows32, a_scale, b_scale, bias, out_max=None, out_dtype=torch.bfloat16):
+    """fp8_linear (scales and bias, no activation) on an activation in k-panels [K/64, M, 64]; with out_max (fp32 [1]) also
+    fp8_linear_max.  Same bits as the row-major calls."""
+    _chk(a_panels, "a_panels", (torch.uint8,))
+    _chk(w_rows32, "w_rows32", (torch.uint8,))
+    _chk(a_scale, "a_scale", (torch.float32,))
+    _chk(b_scale, "b_scale", (torch.float32,))
+    if out_max is not None:
+        _chk(out_max, "out_max", (torch.float32,))
+    if a_panels.dim() != 3 or a_panels.shape[2] != 64:
+        raise ValueError("fp8_linear_panels: a_panels must be [K/64, M, 64]")
+    kp, m, _ = a_panels.shape
+    k = kp * 64
+    n = w_rows32.shape[0]
+    if w_rows32.shape[1] != k:
+        raise ValueError("K mismatch between activation and weight")
+    if bias is not None:
+        _chk(bias, "bias", (out_dtype,))
+    c = torch.empty((m, n), dtype=out_dtype, device=a_panels.device)
+    _l.check(_l.load().lq_gemm_fp8_panels(_ptr(c), _DT[out_dtype], _ptr(a_panels), _ptr(w_rows32), _ptr(a_scale), _ptr(b_scale),
+                                          _ptr(bias), m, n, k, _ptr(out_max), _stream()), "lq_gemm_fp8_panels")
+    return c
+
+
 def fp8_linear_gated(a_q, w_rows32, a_scale, b_scale, bias, gate, residual, rows_per_gate: int, out=None):
     """FP8 GEMM + invokeFusedGateAndResidual: out = residual + gate[row // rows_per_gate] * (A.W^T*sa*sb + bias), with
     the roundings of the unfused sequence.  gate [ceil(M/rows_per_gate), N], residual [M, N]; out may be residual."""

@@ -20,7 +20,8 @@ _lib_op = torch.library.custom_op
 NAMES = ("sq_quant", "sq_quant_dynamic", "geglu_int8_dynamic", "int8_linear", "fp8_quant", "fp8_scale_cast", "fp8_linear",
          "w4a4_quant", "w4a4_linear", "repack_weight", "lora_down", "layernorm_mod_fp8", "gate_residual_layernorm_mod_fp8",
          "fp8_linear_codes", "fp8_linear_gated", "flux_attn_post_fp8", "flux_single_mlp_fp8", "rmsnorm_rope",
-         "fp8_linear_max", "fp8_gelu_quant", "w4a4_quant_lora_down")
+         "fp8_linear_max", "fp8_gelu_quant", "w4a4_quant_lora_down", "fp8_quant_panels", "fp8_gelu_quant_panels",
+         "fp8_linear_panels")
 
 
 @_lib_op("lyradiff::sq_quant", mutates_args=())
@@ -119,6 +120,37 @@ def fp8_gelu_quant(y: Tensor, y_max: Tensor) -> Tuple[Tensor, Tensor]:
 @fp8_gelu_quant.register_fake
 def _(y, y_max):
     return y.new_empty(y.shape, dtype=torch.uint8), y.new_empty((1,), dtype=torch.float32)
+
+
+@_lib_op("lyradiff::fp8_quant_panels", mutates_args=())
+def fp8_quant_panels(x: Tensor) -> Tuple[Tensor, Tensor]:
+    return _ops.fp8_quant_panels(x)
+
+
+@fp8_quant_panels.register_fake
+def _(x):
+    return x.new_empty((x.shape[1] // 64, x.shape[0], 64), dtype=torch.uint8), x.new_empty((1,), dtype=torch.float32)
+
+
+@_lib_op("lyradiff::fp8_gelu_quant_panels", mutates_args=())
+def fp8_gelu_quant_panels(y: Tensor, y_max: Tensor) -> Tuple[Tensor, Tensor]:
+    return _ops.fp8_gelu_quant_panels(y, y_max)
+
+
+@fp8_gelu_quant_panels.register_fake
+def _(y, y_max):
+    return y.new_empty((y.shape[1] // 64, y.shape[0], 64), dtype=torch.uint8), y.new_empty((1,), dtype=torch.float32)
+
+
+@_lib_op("lyradiff::fp8_linear_panels", mutates_args=("out_max",))
+def fp8_linear_panels(a_panels: Tensor, w_rows32: Tensor, a_scale: Tensor, b_scale: Tensor, bias: Optional[Tensor],
+                      out_max: Optional[Tensor] = None, out_dtype: torch.dtype = torch.bfloat16) -> Tensor:
+    return _ops.fp8_linear_panels(a_panels, w_rows32, a_scale, b_scale, bias, out_max, out_dtype)
+
+
+@fp8_linear_panels.register_fake
+def _(a_panels, w_rows32, a_scale, b_scale, bias, out_max=None, out_dtype=torch.bfloat16):
+    return a_panels.new_empty((a_panels.shape[1], w_rows32.shape[0]), dtype=out_dtype)
 
 
 @_lib_op("lyradiff::w4a4_quant_lora_down", mutates_args=())

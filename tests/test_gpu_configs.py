@@ -217,7 +217,15 @@ def test_config3_flux_mlp_fp8_as_benchmarked(ops, dev):
     s_ref = O.fp8_scale(hn)  # scale and codes: exactly the amax and cast of the activated tensor
     assert float(sh.cpu()) == float(s_ref)
     assert np.array_equal(qh.cpu().numpy()[rows], O.fp8_scale_cast(hn[rows], s_ref, True))
-    check_fp8_linear(ops, dev, qh, sh, wq_dn, ws_dn, wp_dn, ws_dn_d, b_dn, False, 44, "config 3 down")
+    y = check_fp8_linear(ops, dev, qh, sh, wq_dn, ws_dn, wp_dn, ws_dn_d, b_dn, False, 44, "config 3 down")
+    # bench.py passes the quantised activations between these kernels as k-panels [K/64, M, 64]: the same bits at every step
+    qa_p, sa_p = ops.fp8_quant_panels(x)
+    assert torch.equal(sa_p, sa) and torch.equal(ops.fp8_panels_to_rows(qa_p), qa)
+    umax_p = torch.zeros(1, dtype=torch.float32, device=dev)
+    assert torch.equal(ops.fp8_linear_panels(qa_p, wp_up, sa_p, ws_up_d, b_up.to(dev), umax_p, torch.bfloat16), u) and torch.equal(umax_p, umax)
+    qh_p, sh_p = ops.fp8_gelu_quant_panels(u, umax, clear_max=nxt)
+    assert torch.equal(sh_p, sh) and torch.equal(ops.fp8_panels_to_rows(qh_p), qh)
+    assert torch.equal(ops.fp8_linear_panels(qh_p, wp_dn, sh_p, ws_dn_d, b_dn.to(dev), None, torch.bfloat16), y)
 
 
 # ---- config 4: FLUX attention projection, W4A4 group 64, fp16 scales ----------------------------------------------

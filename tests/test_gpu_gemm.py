@@ -542,6 +542,72 @@ def test_fp8_linear_max_then_gelu_quant(ops, dev, m, n, k, dt):
     assert_close_tol(to_np_f32(h.cpu()), O.round_to(O.gelu_tanh_f32(to_np_f32(c.cpu())), dt), "gelu of the stored output")
 
 
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32"])
+# the persistent kernel with and without a round of half tiles, the one-wavefront-per-SIMD and two-workgroups-per-CU kernels
+# with ragged edges, a tensor below the one-launch quantiser's size, one whose element count is not a multiple of 1024
+@pytest.mark.parametrize("m,n,k", [(512, 1024, 256), (4608, 12288, 128), (2304, 1536, 3072), (333, 416, 704), (1024, 3072, 192), (7, 64, 64),
+                                   (70, 96, 64)])
+def test_fp8_chain_on_activations_in_k_panels(ops, dev, m, n, k, dt):
+    """Quantisers that write [K/64, M, 64] k-panels and the GEMM that reads them give the bits of the row-major calls."""
+    g = rng_t(m + 2 * n + 3 * k)
+    t = TORCH_DT[dt]
+    tout = torch.bfloat16 if dt == "f32" else t
+    x = torch.randn(m, k, generator=g).to(t).to(dev)
+    qa, sa = ops.fp8_quant(x)
+    qp, sp = ops.fp8_quant_panels(x)
+    assert qp.shape == (k // 64, m, 64) and torch.equal(sp, sa) and torch.equal(ops.fp8_panels_to_rows(qp), qa)
+    qw, sw = ops.fp8_quant((torch.randn(n, k, generator=g) * 0.05).to(tout).to(dev))
+    wp = ops.repack_weight(qw)
+    bias = (torch.randn(n, generator=g) * 0.1).to(tout).to(dev)
+    ymax, ymax_p = torch.zeros(1, dtype=torch.float32, device=dev), torch.zeros(1, dtype=torch.float32, device=dev)
+    c = ops.fp8_linear_max(qa, wp, sa, sw, bias, ymax, tout)
+    c_p = ops.fp8_linear_panels(qp, wp, sp, sw, bias, ymax_p, tout)
+    assert torch.equal(c_p, c) and torch.equal(ymax_p, ymax)
+    assert torch.equal(ops.fp8_linear_panels(qp, wp, sp, sw, bias, None, tout), c)
+    for tactic in range(ops.gemm_tactic_count("fp8")):
+        with ops.gemm_thread_tactic(tactic):
+            assert torch.equal(ops.fp8_linear_panels(qp, wp, sp, sw, None, None, tout),
+                               ops.fp8_linear(qa, wp, sa, sw, None, False, None, 0.0, tout)), f"tactic {tactic}"
+    if n % 64 == 0:
+        y = c.to(t)
+        q, s = ops.fp8_gelu_quant(y, ymax)
+        nxt = torch.full((1,), 7.0, dtype=torch.float32, device=dev)
+        q_p, s_p = ops.fp8_gelu_quant_panels(y, ymax, clear_max=nxt)
+        assert q_p.shape == (n // 64, m, 64) and torch.equal(s_p, s) and torch.equal(ops.fp8_panels_to_rows(q_p), q) and nxt.item() == 0.0
+
+
+def test_fp8_panel_ops_under_stream_capture_and_argument_checks(ops, dev):
+    g = rng_t(77)
+    x = torch.randn(300, 192, generator=g).bfloat16().to(dev)
+    qa, sa = ops.fp8_quant(x)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # a capturing stream takes the exchange-free kernel sequence
+        warm = ops.fp8_quant_panels(x)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            qp, sp = ops.fp8_quant_panels(x)
+        for _ in range(3):
+            qp.zero_()
+            graph.replay()
+            side.synchronize()
+            assert torch.equal(ops.fp8_panels_to_rows(qp), qa) and torch.equal(sp, sa)
+    torch.cuda.current_stream().wait_stream(side)
+    assert torch.equal(ops.fp8_panels_to_rows(warm[0]), qa)
+    with pytest.raises(ValueError):
+        ops.fp8_quant_panels(torch.zeros(8, 96, dtype=torch.bfloat16, device=dev))
+    lib = ops._l.load()
+    buf = torch.zeros(4096, dtype=torch.uint8, device=dev)
+    sc = torch.zeros(1, dtype=torch.float32, device=dev)
+    assert lib.lq_fp8_amax_cast_panels(buf.data_ptr(), sc.data_ptr(), x.data_ptr(), 2, 8, 96, 0) < 0  # k % 64 != 0
+    assert lib.lq_fp8_gelu_cast_panels(buf.data_ptr(), sc.data_ptr(), x.data_ptr(), 2, 8, 96, sc.data_ptr(), None, 0) < 0
+    assert lib.lq_fp8_amax_cast_panels(buf.data_ptr(), sc.data_ptr(), x.data_ptr(), 2, 0, 64, 0) == 0  # empty
+    with ops.gemm_thread_tactic(1):  # the 128-byte k-tile configuration reads row-major activations only: another one runs
+        w = ops.repack_weight(ops.fp8_quant((torch.randn(256, 192, generator=g) * 0.05).bfloat16().to(dev))[0])
+        qp, sp = ops.fp8_quant_panels(x)
+        assert torch.equal(ops.fp8_linear_panels(qp, w, sp, sp, None), ops.fp8_linear(qa, w, sa, sa, None, False, None, 0.0, torch.bfloat16))
+
+
 def test_fp8_gelu_quant_without_a_large_value_takes_the_bound(ops, dev):
     g = rng_t(9)
     y = (torch.rand(5000, generator=g) - 0.7).clamp(max=0.4).bfloat16().to(dev)

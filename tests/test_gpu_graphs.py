@@ -54,7 +54,8 @@ def test_flux_mlp_fp8_chain_replays_exactly(ops, dev):
         torch.cuda.synchronize()
 
 
-def test_flux_mlp_fp8_running_maximum_chain_replays_exactly(ops, dev):
+@pytest.mark.parametrize("panels", [False, True])
+def test_flux_mlp_fp8_running_maximum_chain_replays_exactly(ops, dev, panels):
     """The chain bench.py times -- persistent GEMM that leaves its largest output, GELU + quantisation in one pass that also
     clears the other maximum slot -- captured as two steps (so both slots take both roles) and replayed."""
     m, d, h = 1024, 3072, 12288  # 192 tiles of 256x256: the up projection runs tactic 6/4; the persistent kernel is forced below
@@ -68,6 +69,12 @@ def test_flux_mlp_fp8_running_maximum_chain_replays_exactly(ops, dev):
     slots = [torch.zeros(1, dtype=torch.float32, device=dev) for _ in range(2)]
 
     def step(inp, k):
+        if panels:  # quantised activations as k-panels, as bench.py passes them
+            q, s = ops.fp8_quant_panels(inp)
+            with ops.gemm_thread_tactic(7):
+                u = ops.fp8_linear_panels(q, wp_up, s, s_up, b_up, slots[k % 2])
+            q2, s2 = ops.fp8_gelu_quant_panels(u, slots[k % 2], clear_max=slots[(k + 1) % 2])
+            return ops.fp8_linear_panels(q2, wp_dn, s2, s_dn, b_dn)
         q, s = ops.fp8_quant(inp)
         with ops.gemm_thread_tactic(7):
             u = ops.fp8_linear_max(q, wp_up, s, s_up, b_up, slots[k % 2])

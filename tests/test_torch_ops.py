@@ -65,6 +65,12 @@ def test_shape_inference_without_a_gpu(tops):
         assert u.shape == (4608, 12288) and u.dtype == torch.bfloat16
         qh, sh = torch.ops.lyradiff.fp8_gelu_quant(u, one)
         assert qh.shape == u.shape and qh.dtype == torch.uint8 and sh.shape == (1,) and sh.dtype == torch.float32
+        qp, sp = torch.ops.lyradiff.fp8_quant_panels(xb)
+        assert qp.shape == (48, 4608, 64) and qp.dtype == torch.uint8 and sp.shape == (1,)
+        up = torch.ops.lyradiff.fp8_linear_panels(qp, wf, sp, sf, None, one)
+        assert up.shape == (4608, 12288) and up.dtype == torch.bfloat16
+        qhp, shp = torch.ops.lyradiff.fp8_gelu_quant_panels(up, one)
+        assert qhp.shape == (192, 4608, 64) and qhp.dtype == torch.uint8 and shp.shape == (1,)
         w_, s_, a_ = torch.ops.lyradiff.w4a4_quant_lora_down(xb, None, torch.empty(32, 3072, dtype=torch.bfloat16, device=dev))
         assert w_.shape == (4608, 384) and s_.shape == (4608, 48) and a_.shape == (4608, 32) and a_.dtype == torch.bfloat16
 
@@ -107,6 +113,12 @@ def test_operators_match_direct_wrappers(tops, dev):
     qh, sh = torch.ops.lyradiff.fp8_gelu_quant(u, um)
     qh0, sh0 = ops.fp8_gelu_quant(u, um)
     assert torch.equal(qh, qh0) and torch.equal(sh, sh0)
+    qp, sp = torch.ops.lyradiff.fp8_quant_panels(xb)
+    assert torch.equal(ops.fp8_panels_to_rows(qp), qf) and torch.equal(sp, sf)
+    um2 = torch.zeros(1, device=dev)
+    assert torch.equal(torch.ops.lyradiff.fp8_linear_panels(qp, wf, sp, sf, None, um2), u) and torch.equal(um2, um)
+    qhp, shp = torch.ops.lyradiff.fp8_gelu_quant_panels(u, um)
+    assert torch.equal(ops.fp8_panels_to_rows(qhp), qh) and torch.equal(shp, sh)
     dn = (torch.randn(32, 512, generator=g) * 0.05).bfloat16().to(dev)
     sm = (torch.rand(512, generator=g) + 0.5).to(dev)
     got3, ref3 = torch.ops.lyradiff.w4a4_quant_lora_down(xb, sm, dn), ops.w4a4_quant_lora_down(xb, sm, dn)
