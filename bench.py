@@ -447,10 +447,16 @@ def other_metric_gemms(torch, ops, dev, batched):
     ac = (torch.rand(n, generator=g) * 9e-3 + 1e-3).to(dev)
     ar = (torch.rand(m, generator=g) * 0.05).to(dev)
     b = (torch.randn(n, generator=g) * 0.02).half().to(dev)
-    us = batched(lambda i: ops.int8_linear(a, w, ac, ar, b, torch.float16))
+    # the activation as k-panels [K/64, M, 64], the layout lq_sq_dynamic_quant_panels writes (random codes: any arrangement of
+    # them is a valid activation); the row-major time beside it
+    a_p = a.view(k // 64, m, 64)
+    us = batched(lambda i: ops.int8_linear_panels(a_p, w, ac, ar, b, torch.float16))
+    us_rows = batched(lambda i: ops.int8_linear(a, w, ac, ar, b, torch.float16))
     tops = 2.0 * m * n * k / us / 1e6
     out[f"gemm_int8_w8a8_{m}x{n}x{k}"] = {"us_back_to_back": round(us, 2), "TOP/s": round(tops, 1),
-                                          "frac_of_int8_peak": round(tops / INT8_PEAK_TOPS, 4)}
+                                          "frac_of_int8_peak": round(tops / INT8_PEAK_TOPS, 4),
+                                          "activation_layout": "k-panels [K/64, M, 64]",
+                                          "us_back_to_back_row_major_activation": round(us_rows, 2)}
     del a, w
     m, n, k = M, D, D
     aw = torch.randint(-2 ** 31, 2 ** 31 - 1, (m, k // 8), generator=g, dtype=torch.int32).to(dev)
@@ -568,6 +574,8 @@ def extra_kernels(torch, ops, dev):
         xr = rotating(torch.randn(m, k, generator=g).bfloat16().to(dev))
         us = timeit(lambda: ops.fp8_quant(xr()))
         res[f"fp8_amax_cast_{m}x{k}"] = {"us": round(us, 2), "GB/s": round(3.0 * m * k / us / 1e3, 1)}
+        us = timeit(lambda: ops.fp8_quant_panels(xr()))
+        res[f"fp8_amax_cast_panels_{m}x{k}"] = {"us": round(us, 2), "GB/s": round(3.0 * m * k / us / 1e3, 1)}
         us = timeit(lambda: ops.fp8_scale_cast(xr(), one))
         res[f"fp8_scale_cast_{m}x{k}"] = {"us": round(us, 2), "GB/s": round(3.0 * m * k / us / 1e3, 1)}
     for (m, k) in [(1024, 1280), (4096, 640), (4608, 3072), (4608, 12288)]:
@@ -576,6 +584,9 @@ def extra_kernels(torch, ops, dev):
         xr = rotating(x)
         us = timeit(lambda: ops.sq_quant_dynamic(xr(), pre))
         res[f"sq_dynamic_quant_{m}x{k}"] = {"us": round(us, 2), "GB/s": round((3.0 * m * k + 4 * m + 4 * k) / us / 1e3, 1)}
+        if k >= 3072:  # the same quantiser writing k-panels [K/64, M, 64]
+            us = timeit(lambda: ops.sq_quant_dynamic_panels(xr(), pre))
+            res[f"sq_dynamic_quant_panels_{m}x{k}"] = {"us": round(us, 2), "GB/s": round((3.0 * m * k + 4 * m + 4 * k) / us / 1e3, 1)}
     for (m, k) in [(4096, 1280), (4096, 640), (4608, 3072)]:
         x = torch.randn(m, k, generator=g).half().to(dev)
         gb = torch.randn(k, generator=g).half().to(dev)

@@ -277,6 +277,12 @@ int lq_fp8_gelu_cast(uint8_t* dst, float* scale_out, void* h_out, const void* sr
  *   lq_fp8_gelu_cast_panels   = lq_fp8_gelu_cast without h_out, writing k-panels
  *   lq_gemm_fp8_panels        = lq_gemm_fp8 without activation or residual on such an activation; with out_max also
  *                               lq_gemm_fp8_max (out_max may be NULL) */
+/* The same layout for the INT8 path: lq_sq_dynamic_quant writing its codes as k-panels (scale_out as there; dim % 64 == 0,
+ * dim <= 16384, 16-byte aligned buffers) and lq_gemm_int8 reading them.  Bit-identical codes, scales and outputs. */
+int lq_sq_dynamic_quant_panels(int8_t* dst_panels, float* scale_out, const void* src, lq_dtype_t src_dtype,
+                               const float* pre_quant_scale, size_t rows, size_t dim, lq_stream_t stream);
+int lq_gemm_int8_panels(void* C, lq_dtype_t out_dtype, const int8_t* A_panels, const int8_t* B_rows32, const float* alpha_col,
+                        const float* alpha_row, int per_token, const void* bias, int m, int n, int k, lq_stream_t stream);
 int lq_fp8_amax_cast_panels(uint8_t* dst_panels, float* scale_out, const void* src, lq_dtype_t dtype, size_t rows, size_t k,
                             lq_stream_t stream);
 int lq_fp8_gelu_cast_panels(uint8_t* dst_panels, float* scale_out, const void* src, lq_dtype_t dtype, size_t rows, size_t k,

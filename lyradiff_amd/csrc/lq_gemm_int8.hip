@@ -31,7 +31,7 @@ template <typename OutTag> static int run_int8(GemmParams p, hipStream_t st) {
             (out_enum<OutTag>() == LQ_F16 || out_enum<OutTag>() == LQ_BF16))
             t = 7;
     }
-    if (t == 1 && p.kb % 128 != 0) t = 0;  // the 128-byte k-tile needs k % 128 == 0
+    if (t == 1 && (p.kb % 128 != 0 || p.a_panel)) t = 0;  // the 128-byte k-tile needs k % 128 == 0 and a row-major activation
     if (t == 7) {  // the persistent form of tactic 6 where it applies, tactic 6 itself elsewhere
         const int rc = launch_persist_int8(p, out_enum<OutTag>(), st);
         if (rc != 1) return rc;
@@ -53,9 +53,23 @@ template <typename OutTag> static int run_int8(GemmParams p, hipStream_t st) {
 
 using namespace lq;
 
+static int gemm_int8(void* C, lq_dtype_t out_dtype, const int8_t* A, const int8_t* B_rows32, const float* alpha_col,
+                     const float* alpha_row, int per_token, const void* bias, int m, int n, int k, int a_panel, lq_stream_t stream);
+
 extern "C" int lq_gemm_int8(void* C, lq_dtype_t out_dtype, const int8_t* A, const int8_t* B_rows32,
                             const float* alpha_col, const float* alpha_row, int per_token, const void* bias, int m,
                             int n, int k, lq_stream_t stream) {
+    return gemm_int8(C, out_dtype, A, B_rows32, alpha_col, alpha_row, per_token, bias, m, n, k, 0, stream);
+}
+
+extern "C" int lq_gemm_int8_panels(void* C, lq_dtype_t out_dtype, const int8_t* A_panels, const int8_t* B_rows32,
+                                   const float* alpha_col, const float* alpha_row, int per_token, const void* bias, int m,
+                                   int n, int k, lq_stream_t stream) {
+    return gemm_int8(C, out_dtype, A_panels, B_rows32, alpha_col, alpha_row, per_token, bias, m, n, k, 1, stream);
+}
+
+static int gemm_int8(void* C, lq_dtype_t out_dtype, const int8_t* A, const int8_t* B_rows32, const float* alpha_col,
+                     const float* alpha_row, int per_token, const void* bias, int m, int n, int k, int a_panel, lq_stream_t stream) {
     LQ_REQUIRE(C && A && B_rows32, LQ_ERR_ARG, "lq_gemm_int8: null pointer");
     LQ_REQUIRE(out_dtype == LQ_I32 || (alpha_col && alpha_row), LQ_ERR_ARG, "lq_gemm_int8: scale pointers are required");
     LQ_REQUIRE(m >= 0 && n > 0 && k > 0 && n % 32 == 0 && k % 64 == 0, LQ_ERR_SHAPE,
@@ -69,6 +83,7 @@ extern "C" int lq_gemm_int8(void* C, lq_dtype_t out_dtype, const int8_t* A, cons
     p.C = C; p.A = reinterpret_cast<const uint8_t*>(A); p.B = reinterpret_cast<const uint8_t*>(B_rows32);
     p.bias = bias; p.alpha_col = alpha_col; p.alpha_row = alpha_row; p.per_token = per_token;
     p.m = m; p.n = n; p.k = k; p.kb = k;
+    p.a_panel = a_panel;
     hipStream_t st = as_stream(stream);
     switch (out_dtype) {
         case LQ_F16: return run_int8<F16Tag>(p, st);

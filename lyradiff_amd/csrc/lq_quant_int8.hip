@@ -146,7 +146,10 @@ __global__ __launch_bounds__(256) void sq_quant_rows_kernel(int8_t* __restrict__
 // registers whatever the row length, so eight of them share a SIMD and the loads of one overlap the
 // arithmetic of the others; the dynamic variant exchanges the span maxima through LDS (one barrier).
 // A lane outside the row re-reads a valid octet (harmless for the maximum) and stores nothing.
-template <typename Tag, int MODE, bool HAS_PRE, int R, bool STREAM = false>
+// PANEL: the codes are written as k-panels [dim / 64][rows][64] (byte ((c / 64) * rows + row) * 64 + c % 64) for
+// lq_gemm_int8_panels instead of row-major: a lane's eight codes stay inside one 64-byte segment, eight lanes fill it, and
+// with two rows per workgroup the two segments of a 128-byte line are written by the same wavefront.
+template <typename Tag, int MODE, bool HAS_PRE, int R, bool STREAM = false, bool PANEL = false>
 __global__ __launch_bounds__(1024) void sq_quant_split_kernel(int8_t* __restrict__ dst, float* __restrict__ scale_out,
                                                               const void* __restrict__ src,
                                                               const float* __restrict__ pre,
@@ -243,7 +246,12 @@ __global__ __launch_bounds__(1024) void sq_quant_split_kernel(int8_t* __restrict
                 o.x = pack4_s8(q[0], q[1], q[2], q[3]);
                 o.y = pack4_s8(q[4], q[5], q[6], q[7]);
             }
-            if (valid[p] && live[rr]) st8<STREAM>(ob + col[p], o);
+            if constexpr (PANEL) {
+                if (valid[p] && live[rr])
+                    st8<STREAM>(dst + ((size_t)(col[p] >> 6) * rows + (row0 + rr)) * 64 + (col[p] & 63), o);
+            } else {
+                if (valid[p] && live[rr]) st8<STREAM>(ob + col[p], o);
+            }
         }
     }
 }
@@ -663,6 +671,44 @@ extern "C" int lq_sq_dynamic_quant(int8_t* dst, float* scale_out, const void* sr
     if (rows == 0) return LQ_OK;
     LQ_REQUIRE(dim > 0, LQ_ERR_SHAPE, "lq_sq_dynamic_quant: dim must be positive");
     return dispatch_sq_quant<2>(dst, scale_out, src, src_dtype, pre_quant_scale, nullptr, rows, dim, as_stream(stream));
+}
+
+// Dynamic per-token quantisation with the codes written as k-panels: the split kernel for every row length (a wavefront per
+// 1024 columns), two rows per workgroup when a smoothing vector is given.
+template <typename Tag>
+static int launch_sq_dynamic_panels(int8_t* dst, float* scale_out, const void* src, const float* pre, size_t rows, size_t dim,
+                                    hipStream_t st) {
+    const int np = (int)((dim + 511) / 512), d = (int)dim;
+    const dim3 block(64 * ((np + 1) / 2));
+    const bool stream_io = rows * dim * Elem<Tag>::bytes >= kStreamQuantBytes;
+    if (pre) {
+        const dim3 grid((unsigned)((rows + 1) / 2));
+        if (stream_io) hipLaunchKernelGGL((sq_quant_split_kernel<Tag, 2, true, 2, true, true>), grid, block, 0, st, dst, scale_out, src, pre, nullptr, rows, d);
+        else hipLaunchKernelGGL((sq_quant_split_kernel<Tag, 2, true, 2, false, true>), grid, block, 0, st, dst, scale_out, src, pre, nullptr, rows, d);
+    } else {
+        const dim3 grid((unsigned)rows);
+        if (stream_io) hipLaunchKernelGGL((sq_quant_split_kernel<Tag, 2, false, 1, true, true>), grid, block, 0, st, dst, scale_out, src, pre, nullptr, rows, d);
+        else hipLaunchKernelGGL((sq_quant_split_kernel<Tag, 2, false, 1, false, true>), grid, block, 0, st, dst, scale_out, src, pre, nullptr, rows, d);
+    }
+    return check_launch("sq_quant_split(panels)");
+}
+
+extern "C" int lq_sq_dynamic_quant_panels(int8_t* dst_panels, float* scale_out, const void* src, lq_dtype_t src_dtype,
+                                          const float* pre_quant_scale, size_t rows, size_t dim, lq_stream_t stream) {
+    LQ_REQUIRE(dst_panels && src && scale_out, LQ_ERR_ARG, "lq_sq_dynamic_quant_panels: null pointer");
+    if (rows == 0) return LQ_OK;
+    LQ_REQUIRE(dim > 0 && dim % 64 == 0 && dim <= 16384 && rows <= 0x7fffffffu, LQ_ERR_SHAPE,
+               "lq_sq_dynamic_quant_panels: k-panels need dim %% 64 == 0 and dim <= 16384 (rows=%zu dim=%zu)", rows, dim);
+    LQ_REQUIRE(reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst_panels) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(pre_quant_scale) % 16 == 0,
+               LQ_ERR_ARG, "lq_sq_dynamic_quant_panels: src, dst and pre_quant_scale must be 16-byte aligned");
+    hipStream_t st = as_stream(stream);
+    switch (src_dtype) {
+        case LQ_F16: return launch_sq_dynamic_panels<F16Tag>(dst_panels, scale_out, src, pre_quant_scale, rows, dim, st);
+        case LQ_BF16: return launch_sq_dynamic_panels<BF16Tag>(dst_panels, scale_out, src, pre_quant_scale, rows, dim, st);
+        case LQ_F32: return launch_sq_dynamic_panels<F32Tag>(dst_panels, scale_out, src, pre_quant_scale, rows, dim, st);
+        default: set_error("lq_sq_dynamic_quant_panels: unsupported source dtype %d", (int)src_dtype); return LQ_ERR_UNSUPPORTED;
+    }
 }
 
 extern "C" int lq_sq_output_dequant(void* dst, lq_dtype_t dst_dtype, const int32_t* src, const float* input_quant_scale,

@@ -561,6 +561,51 @@ def fp8_linear_panels(a_panels, w_rows32, a_scale, b_scale, bias, out_max=None, 
     return c
 
 
+def sq_quant_dynamic_panels(x, pre_quant_scale=None):
+    """sq_quant_dynamic of a 2-D x [M, K] with the codes written as k-panels: returns (int8 [K/64, M, 64], scale fp32 [M])."""
+    _chk(x, "x", _FLOATS)
+    if x.dim() != 2 or x.shape[1] % 64 != 0:
+        raise ValueError("sq_quant_dynamic_panels: x must be [M, K] with K % 64 == 0")
+    m, k = x.shape
+    if pre_quant_scale is not None:
+        _chk(pre_quant_scale, "pre_quant_scale", (torch.float32,))
+        if pre_quant_scale.numel() != k:
+            raise ValueError("pre_quant_scale must have K elements")
+    q = torch.empty((k // 64, m, 64), dtype=torch.int8, device=x.device)
+    s = torch.empty(m, dtype=torch.float32, device=x.device)
+    _l.check(_l.load().lq_sq_dynamic_quant_panels(_ptr(q), _ptr(s), _ptr(x), _DT[x.dtype], _ptr(pre_quant_scale), m, k, _stream()),
+             "lq_sq_dynamic_quant_panels")
+    return q, s
+
+
+def int8_linear_panels(a_panels, w_rows32, alpha_col, alpha_row, bias=None, out_dtype=torch.float16):
+    """int8_linear on an activation in k-panels [K/64, M, 64].  Same bits as the row-major call."""
+    _chk(a_panels, "a_panels", (torch.int8,))
+    _chk(w_rows32, "w_rows32", (torch.int8,))
+    if a_panels.dim() != 3 or a_panels.shape[2] != 64:
+        raise ValueError("int8_linear_panels: a_panels must be [K/64, M, 64]")
+    kp, m, _ = a_panels.shape
+    k = kp * 64
+    n = w_rows32.shape[0]
+    if w_rows32.shape[1] != k:
+        raise ValueError("K mismatch between activation and weight")
+    per_token = 0
+    if out_dtype != torch.int32:
+        _chk(alpha_col, "alpha_col", (torch.float32,))
+        _chk(alpha_row, "alpha_row", (torch.float32,))
+        if alpha_col.numel() != n:
+            raise ValueError("alpha_col must have N elements")
+        if alpha_row.numel() not in (1, m):
+            raise ValueError("alpha_row must have 1 or M elements")
+        per_token = int(alpha_row.numel() == m and m != 1)
+    if bias is not None:
+        _chk(bias, "bias", (out_dtype,))
+    c = torch.empty((m, n), dtype=out_dtype, device=a_panels.device)
+    _l.check(_l.load().lq_gemm_int8_panels(_ptr(c), _DT[out_dtype], _ptr(a_panels), _ptr(w_rows32), _ptr(alpha_col),
+                                           _ptr(alpha_row), per_token, _ptr(bias), m, n, k, _stream()), "lq_gemm_int8_panels")
+    return c
+
+
 def fp8_linear_gated(a_q, w_rows32, a_scale, b_scale, bias, gate, residual, rows_per_gate: int, out=None):
     """FP8 GEMM + invokeFusedGateAndResidual: out = residual + gate[row // rows_per_gate] * (A.W^T*sa*sb + bias), with
     the roundings of the unfused sequence.  gate [ceil(M/rows_per_gate), N], residual [M, N]; out may be residual."""

@@ -576,6 +576,31 @@ def test_fp8_chain_on_activations_in_k_panels(ops, dev, m, n, k, dt):
         assert q_p.shape == (n // 64, m, 64) and torch.equal(s_p, s) and torch.equal(ops.fp8_panels_to_rows(q_p), q) and nxt.item() == 0.0
 
 
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("m,n,k,pre", [(512, 1024, 256, True), (4608, 1536, 3072, True), (333, 416, 704, False), (71, 96, 64, True),
+                                       (1024, 768, 12288, False)])
+def test_int8_chain_on_activations_in_k_panels(ops, dev, m, n, k, pre, dt):
+    """The per-token quantiser writing k-panels and the INT8 GEMM reading them give the bits of the row-major calls."""
+    g = rng_t(5 * m + n + k)
+    t = TORCH_DT[dt]
+    x = (torch.randn(m, k, generator=g) * 3).to(t).to(dev)
+    ps = (torch.rand(k, generator=g) + 0.5).to(dev) if pre else None
+    q, s = ops.sq_quant_dynamic(x, ps)
+    qp, sp = ops.sq_quant_dynamic_panels(x, ps)
+    assert qp.shape == (k // 64, m, 64) and torch.equal(sp, s) and torch.equal(ops.fp8_panels_to_rows(qp), q)
+    w = ops.repack_weight(torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8).to(dev))
+    ac = (torch.rand(n, generator=g) * 1e-2 + 1e-3).to(dev)
+    bias = (torch.randn(n, generator=g) * 0.1).half().to(dev)
+    assert torch.equal(ops.int8_linear_panels(qp, w, ac, sp, bias, torch.float16), ops.int8_linear(q, w, ac, s, bias, torch.float16))
+    assert torch.equal(ops.int8_linear_panels(qp, w, None, None, None, torch.int32), ops.int8_linear(q, w, None, None, None, torch.int32))
+    for tactic in range(ops.gemm_tactic_count("int8")):
+        with ops.gemm_thread_tactic(tactic):
+            assert torch.equal(ops.int8_linear_panels(qp, w, ac, sp, None, torch.bfloat16),
+                               ops.int8_linear(q, w, ac, s, None, torch.bfloat16)), f"tactic {tactic}"
+    with pytest.raises(ValueError):
+        ops.sq_quant_dynamic_panels(torch.zeros(8, 96, dtype=torch.float16, device=dev))
+
+
 def test_fp8_panel_ops_under_stream_capture_and_argument_checks(ops, dev):
     g = rng_t(77)
     x = torch.randn(300, 192, generator=g).bfloat16().to(dev)
