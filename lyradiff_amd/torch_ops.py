@@ -21,7 +21,7 @@ NAMES = ("sq_quant", "sq_quant_dynamic", "geglu_int8_dynamic", "int8_linear", "f
          "w4a4_quant", "w4a4_linear", "repack_weight", "lora_down", "layernorm_mod_fp8", "gate_residual_layernorm_mod_fp8",
          "fp8_linear_codes", "fp8_linear_gated", "flux_attn_post_fp8", "flux_single_mlp_fp8", "rmsnorm_rope",
          "fp8_linear_max", "fp8_gelu_quant", "w4a4_quant_lora_down", "fp8_quant_panels", "fp8_gelu_quant_panels",
-         "fp8_linear_panels")
+         "fp8_linear_panels", "sq_quant_dynamic_panels", "int8_linear_panels")
 
 
 @_lib_op("lyradiff::sq_quant", mutates_args=())
@@ -67,6 +67,27 @@ def int8_linear(a_q: Tensor, w_rows32: Tensor, alpha_col: Optional[Tensor], alph
 @int8_linear.register_fake
 def _(a_q, w_rows32, alpha_col, alpha_row, bias=None, out_dtype=torch.float16):
     return a_q.new_empty((a_q.shape[0], w_rows32.shape[0]), dtype=out_dtype)
+
+
+@_lib_op("lyradiff::sq_quant_dynamic_panels", mutates_args=())
+def sq_quant_dynamic_panels(x: Tensor, pre_quant_scale: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
+    return _ops.sq_quant_dynamic_panels(x, pre_quant_scale)
+
+
+@sq_quant_dynamic_panels.register_fake
+def _(x, pre_quant_scale=None):
+    return x.new_empty((x.shape[1] // 64, x.shape[0], 64), dtype=torch.int8), x.new_empty((x.shape[0],), dtype=torch.float32)
+
+
+@_lib_op("lyradiff::int8_linear_panels", mutates_args=())
+def int8_linear_panels(a_panels: Tensor, w_rows32: Tensor, alpha_col: Optional[Tensor], alpha_row: Optional[Tensor],
+                       bias: Optional[Tensor] = None, out_dtype: torch.dtype = torch.float16) -> Tensor:
+    return _ops.int8_linear_panels(a_panels, w_rows32, alpha_col, alpha_row, bias, out_dtype)
+
+
+@int8_linear_panels.register_fake
+def _(a_panels, w_rows32, alpha_col, alpha_row, bias=None, out_dtype=torch.float16):
+    return a_panels.new_empty((a_panels.shape[1], w_rows32.shape[0]), dtype=out_dtype)
 
 
 @_lib_op("lyradiff::fp8_quant", mutates_args=())

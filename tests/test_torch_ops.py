@@ -94,6 +94,10 @@ def test_operators_match_direct_wrappers(tops, dev):
     q, s = torch.ops.lyradiff.sq_quant_dynamic(x, None)
     q0, s0 = ops.sq_quant_dynamic(x, None)
     assert torch.equal(q, q0) and torch.equal(s, s0)
+    qp, sp = torch.ops.lyradiff.sq_quant_dynamic_panels(x, None)
+    assert torch.equal(ops.fp8_panels_to_rows(qp), q0) and torch.equal(sp, s0)
+    assert torch.equal(torch.ops.lyradiff.int8_linear_panels(qp, ops.repack_weight(w), ws, sp, None),
+                       ops.int8_linear(q0, ops.repack_weight(w), ws, s0, None))
     wp = torch.ops.lyradiff.repack_weight(w)
     assert torch.equal(torch.ops.lyradiff.int8_linear(q, wp, ws, s, None, torch.float16), ops.int8_linear(q0, wp, ws, s0))
     xb = torch.randn(256, 512, generator=g).bfloat16().to(dev)
