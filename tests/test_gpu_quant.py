@@ -338,6 +338,18 @@ def test_fp8_amax_cast_one_launch_sizes(ops, dev, dt, n):
     assert ops.fp8_amax_cast_status() is False
 
 
+@pytest.mark.parametrize("dt,m,k", [("bf16", 4608, 12288), ("f32", 4608, 12288), ("f16", 6912, 3072), ("bf16", 5000, 8256)])
+def test_fp8_quant_panels_of_tensors_beyond_the_kept_chunks(ops, dev, dt, m, k):
+    """The one-launch quantiser writing k-panels keeps eight chunks per lane and reads the rest of a larger tensor twice (the
+    second loop of its walk); 5000 x 8256 also ends in a partial row block."""
+    g = torch.Generator(device=dev).manual_seed(m + k)
+    x = (torch.randn(m, k, generator=g, device=dev) * 2).to(TORCH_DT[dt])
+    q, s = ops.fp8_quant(x)
+    qp, sp = ops.fp8_quant_panels(x)
+    assert torch.equal(sp, s) and torch.equal(ops.fp8_panels_to_rows(qp), q)
+    assert ops.fp8_amax_cast_status() is False
+
+
 def test_fp8_amax_cast_timeline_gives_the_same_bits_and_ordered_stamps(ops, dev):
     x = (torch.randn(4608 * 3072, generator=rng_t(3)) * 2).bfloat16().to(dev)
     q0, s0 = ops.fp8_quant(x)
