@@ -274,6 +274,7 @@ int lq_fp8_gelu_cast(uint8_t* dst, float* scale_out, void* h_out, const void* sr
  * rows * k < 2^32.  The reference has no counterpart (its FP8 activations are row-major, utils/memory_utils.cu:431-446);
  * codes, scale and GEMM outputs are bit for bit those of the row-major entry points.
  *   lq_fp8_amax_cast_panels   = lq_fp8_amax_cast (same one-launch form, same fall-back sequence) writing k-panels
+ *   lq_fp8_scale_cast_panels  = lq_fp8_scale_cast (given scale: the reference's static _input_scale flow) writing k-panels
  *   lq_fp8_gelu_cast_panels   = lq_fp8_gelu_cast without h_out, writing k-panels
  *   lq_gemm_fp8_panels        = lq_gemm_fp8 without activation or residual on such an activation; with out_max also
  *                               lq_gemm_fp8_max (out_max may be NULL) */
@@ -285,6 +286,8 @@ int lq_gemm_int8_panels(void* C, lq_dtype_t out_dtype, const int8_t* A_panels, c
                         const float* alpha_row, int per_token, const void* bias, int m, int n, int k, lq_stream_t stream);
 int lq_fp8_amax_cast_panels(uint8_t* dst_panels, float* scale_out, const void* src, lq_dtype_t dtype, size_t rows, size_t k,
                             lq_stream_t stream);
+int lq_fp8_scale_cast_panels(uint8_t* dst_panels, const void* src, lq_dtype_t dtype, const float* scale, int invert, size_t rows,
+                             size_t k, lq_stream_t stream);
 int lq_fp8_gelu_cast_panels(uint8_t* dst_panels, float* scale_out, const void* src, lq_dtype_t dtype, size_t rows, size_t k,
                             const float* src_max, float* clear_max, lq_stream_t stream);
 int lq_gemm_fp8_panels(void* C, lq_dtype_t out_dtype, const uint8_t* A_panels, const uint8_t* B_rows32, const float* a_scale,

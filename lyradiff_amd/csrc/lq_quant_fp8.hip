@@ -134,7 +134,8 @@ __global__ __launch_bounds__(256) void fp8_amax_kernel(float* __restrict__ scale
     }
 }
 
-template <typename Tag, bool NT, bool PANEL = false>
+// PANEL: 0 = row-major codes; 1 or 4 = k-panels, walked in blocks of PANEL 64-element chunks per row (PanelWalk)
+template <typename Tag, bool NT, int PANEL = 0>
 __global__ __launch_bounds__(256) void fp8_cast_kernel(uint8_t* __restrict__ dst, const void* __restrict__ src,
                                                        const float* __restrict__ scale, int invert, size_t n, PanelMap pm = PanelMap{0, 0},
                                                        PanelStep stride = PanelStep{0, 0}) {
@@ -151,9 +152,10 @@ __global__ __launch_bounds__(256) void fp8_cast_kernel(uint8_t* __restrict__ dst
         if constexpr (E == 16) *reinterpret_cast<uint4*>(o) = make_uint4(w[0], w[1], w[2], w[3]);
         else *reinterpret_cast<uint2*>(o) = make_uint2(w[0], w[1]);
     };
-    if constexpr (PANEL) {
-        const unsigned kcs = pm.k / 64, nrb = (pm.rows + E - 1) / E;
-        for (PanelWalk<E> pw((blockIdx.x * blockDim.x + threadIdx.x) >> 6, threadIdx.x & 63, kcs); pw.rb < nrb; pw.step(stride, kcs))
+    if constexpr (PANEL != 0) {
+        using Walk = PanelWalk<E, PANEL>;
+        const unsigned kcs = pm.k / 64, nrb = (pm.rows + Walk::RB - 1) / Walk::RB;
+        for (Walk pw((blockIdx.x * blockDim.x + threadIdx.x) >> 6, threadIdx.x & 63, kcs); pw.rb < nrb; pw.step(stride, kcs))
             if (pw.row() < pm.rows) chunk(pw.src_elem(pm), dst + pw.dst_byte(pm));
         return;
     }
@@ -781,8 +783,12 @@ static int launch_cast(uint8_t* dst, const void* src, const float* scale, int in
                        PanelMap pm = PanelMap{0, 0}) {
     if (pm.k != 0) {  // k-panels: the caller has checked the alignment (every piece of 8 or 16 elements stays inside a 64-element chunk)
         const unsigned grid = stream_grid(n, Chunk16<Tag>::elems);
-        hipLaunchKernelGGL((fp8_cast_kernel<Tag, false, true>), dim3(grid), dim3(256), 0, st, dst, src, scale, invert, n, pm,
-                           panel_step((size_t)grid * 4, pm.k / 64));
+        const bool wide = (pm.k / 64) % 4 == 0, nt = n * Elem<Tag>::bytes >= kStreamBytes;  // block shapes as in launch_gelu_cast
+        const PanelStep stride = panel_step((size_t)grid * 4, pm.k / 64 / (wide ? 4 : 1));
+        if (wide && nt) hipLaunchKernelGGL((fp8_cast_kernel<Tag, true, 4>), dim3(grid), dim3(256), 0, st, dst, src, scale, invert, n, pm, stride);
+        else if (wide) hipLaunchKernelGGL((fp8_cast_kernel<Tag, false, 4>), dim3(grid), dim3(256), 0, st, dst, src, scale, invert, n, pm, stride);
+        else if (nt) hipLaunchKernelGGL((fp8_cast_kernel<Tag, true, 1>), dim3(grid), dim3(256), 0, st, dst, src, scale, invert, n, pm, stride);
+        else hipLaunchKernelGGL((fp8_cast_kernel<Tag, false, 1>), dim3(grid), dim3(256), 0, st, dst, src, scale, invert, n, pm, stride);
         return check_launch("fp8_cast");
     }
     if (reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0) {
@@ -908,6 +914,22 @@ extern "C" int lq_fp8_amax_cast_panels(uint8_t* dst, float* scale_out, const voi
     return dtype == LQ_F16    ? launch_cast<F16Tag>(dst, src, scale_out, 1, n, st, pm)
            : dtype == LQ_BF16 ? launch_cast<BF16Tag>(dst, src, scale_out, 1, n, st, pm)
                               : launch_cast<F32Tag>(dst, src, scale_out, 1, n, st, pm);
+}
+
+extern "C" int lq_fp8_scale_cast_panels(uint8_t* dst, const void* src, lq_dtype_t dtype, const float* scale, int invert, size_t rows,
+                                        size_t k, lq_stream_t stream) {
+    const size_t n = rows * k;
+    LQ_REQUIRE(scale && ((dst && src) || n == 0), LQ_ERR_ARG, "lq_fp8_scale_cast_panels: null pointer");
+    LQ_REQUIRE(dtype == LQ_F16 || dtype == LQ_BF16 || dtype == LQ_F32, LQ_ERR_UNSUPPORTED, "lq_fp8_scale_cast_panels: unsupported dtype %d",
+               (int)dtype);
+    if (n == 0) return LQ_OK;
+    int rc = panels_check("lq_fp8_scale_cast_panels", dst, src, rows, k);
+    if (rc != LQ_OK) return rc;
+    const PanelMap pm{(unsigned)k, (unsigned)rows};
+    hipStream_t st = as_stream(stream);
+    return dtype == LQ_F16    ? launch_cast<F16Tag>(dst, src, scale, invert, n, st, pm)
+           : dtype == LQ_BF16 ? launch_cast<BF16Tag>(dst, src, scale, invert, n, st, pm)
+                              : launch_cast<F32Tag>(dst, src, scale, invert, n, st, pm);
 }
 
 extern "C" int lq_fp8_gelu_cast_panels(uint8_t* dst, float* scale_out, const void* src, lq_dtype_t dtype, size_t rows, size_t k,

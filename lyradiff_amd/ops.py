@@ -509,6 +509,19 @@ def fp8_panels_to_rows(q_panels):
     return q_panels.permute(1, 0, 2).reshape(m, kp * w).contiguous()
 
 
+def fp8_scale_cast_panels(x, scale, invert: bool = True):
+    """fp8_scale_cast (a given scale: the reference's static input scale) of a 2-D x [M, K] into k-panels uint8 [K/64, M, 64]."""
+    _chk(x, "x", _FLOATS)
+    _chk(scale, "scale", (torch.float32,))
+    if x.dim() != 2 or x.shape[1] % 64 != 0:
+        raise ValueError("fp8_scale_cast_panels: x must be [M, K] with K % 64 == 0")
+    m, k = x.shape
+    q = torch.empty((k // 64, m, 64), dtype=torch.uint8, device=x.device)
+    _l.check(_l.load().lq_fp8_scale_cast_panels(_ptr(q), _ptr(x), _DT[x.dtype], _ptr(scale), int(invert), m, k, _stream()),
+             "lq_fp8_scale_cast_panels")
+    return q
+
+
 def fp8_quant_panels(x):
     """fp8_quant of a 2-D x [M, K] with the codes written as k-panels: returns (uint8 [K/64, M, 64], scale fp32 [1])."""
     _chk(x, "x", _FLOATS)

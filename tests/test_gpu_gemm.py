@@ -556,6 +556,8 @@ def test_fp8_chain_on_activations_in_k_panels(ops, dev, m, n, k, dt):
     qa, sa = ops.fp8_quant(x)
     qp, sp = ops.fp8_quant_panels(x)
     assert qp.shape == (k // 64, m, 64) and torch.equal(sp, sa) and torch.equal(ops.fp8_panels_to_rows(qp), qa)
+    static = torch.full((1,), 0.03125, dtype=torch.float32, device=dev)  # a given scale, as the reference's static input scale
+    assert torch.equal(ops.fp8_panels_to_rows(ops.fp8_scale_cast_panels(x, static)), ops.fp8_scale_cast(x, static))
     qw, sw = ops.fp8_quant((torch.randn(n, k, generator=g) * 0.05).to(tout).to(dev))
     wp = ops.repack_weight(qw)
     bias = (torch.randn(n, generator=g) * 0.1).to(tout).to(dev)

@@ -348,6 +348,7 @@ def test_fp8_quant_panels_of_tensors_beyond_the_kept_chunks(ops, dev, dt, m, k):
     qp, sp = ops.fp8_quant_panels(x)
     assert torch.equal(sp, s) and torch.equal(ops.fp8_panels_to_rows(qp), q)
     assert ops.fp8_amax_cast_status() is False
+    assert torch.equal(ops.fp8_panels_to_rows(ops.fp8_scale_cast_panels(x, s)), q)  # the cast with a given scale, same walk
 
 
 def test_fp8_amax_cast_timeline_gives_the_same_bits_and_ordered_stamps(ops, dev):
