@@ -277,7 +277,13 @@ int lq_fp8_gelu_cast(uint8_t* dst, float* scale_out, void* h_out, const void* sr
  *   lq_fp8_scale_cast_panels  = lq_fp8_scale_cast (given scale: the reference's static _input_scale flow) writing k-panels
  *   lq_fp8_gelu_cast_panels   = lq_fp8_gelu_cast without h_out, writing k-panels
  *   lq_gemm_fp8_panels        = lq_gemm_fp8 without activation or residual on such an activation; with out_max also
- *                               lq_gemm_fp8_max (out_max may be NULL) */
+ *                               lq_gemm_fp8_max (out_max may be NULL)
+ * and for the static-scale sequences of the FLUX blocks (the row-major forms are documented further down):
+ *   lq_layernorm_mod_fp8_panels, lq_layernorm_mod_fp8_dual_panels, lq_gate_residual_layernorm_mod_fp8_panels
+ *                             = the LayerNorm + cast kernels writing their codes as k-panels [dim / 64][batch * rows][64]
+ *   lq_gemm_fp8_codes_panels  = lq_gemm_fp8_codes reading its activation AND writing its codes as k-panels ([n / 64][m][64]; a
+ *                               block of columns of a wider tensor of panels is the pointer C + (first column / 64) * m * 64)
+ *   lq_gemm_fp8_gated_panels  = lq_gemm_fp8_gated reading its activation as k-panels */
 /* The same layout for the INT8 path: lq_sq_dynamic_quant writing its codes as k-panels (scale_out as there; dim % 64 == 0,
  * dim <= 16384, 16-byte aligned buffers) and lq_gemm_int8 reading them.  Bit-identical codes, scales and outputs. */
 int lq_sq_dynamic_quant_panels(int8_t* dst_panels, float* scale_out, const void* src, lq_dtype_t src_dtype,
@@ -292,6 +298,23 @@ int lq_fp8_gelu_cast_panels(uint8_t* dst_panels, float* scale_out, const void* s
                             const float* src_max, float* clear_max, lq_stream_t stream);
 int lq_gemm_fp8_panels(void* C, lq_dtype_t out_dtype, const uint8_t* A_panels, const uint8_t* B_rows32, const float* a_scale,
                        const float* b_scale, const void* bias, int m, int n, int k, float* out_max, lq_stream_t stream);
+int lq_gemm_fp8_codes_panels(uint8_t* C_fp8_panels, const float* C_fp8_scale, lq_dtype_t round_dtype, const uint8_t* A_panels,
+                             const uint8_t* B_rows32, const float* a_scale, const float* b_scale, const void* bias, int gelu, int m,
+                             int n, int k, lq_stream_t stream);
+int lq_gemm_fp8_gated_panels(void* C, lq_dtype_t out_dtype, const uint8_t* A_panels, const uint8_t* B_rows32, const float* a_scale,
+                             const float* b_scale, const void* bias, const void* gate, size_t rows_per_gate, const void* residual,
+                             int m, int n, int k, lq_stream_t stream);
+int lq_layernorm_mod_fp8_panels(uint8_t* dst_panels, const void* src, const void* scale, const void* shift, lq_dtype_t dtype,
+                                const float* input_scale, size_t batch, size_t rows_per_batch, size_t dim, float eps,
+                                lq_stream_t stream);
+int lq_layernorm_mod_fp8_dual_panels(uint8_t* dst_a_panels, const float* input_scale_a, uint8_t* dst_b_panels,
+                                     const float* input_scale_b, const void* src, const void* scale, const void* shift,
+                                     lq_dtype_t dtype, size_t batch, size_t rows_per_batch, size_t dim, float eps,
+                                     lq_stream_t stream);
+int lq_gate_residual_layernorm_mod_fp8_panels(uint8_t* dst_panels, void* hidden_out, const void* attn, const void* gate,
+                                              const void* input, const void* scale, const void* shift, lq_dtype_t dtype,
+                                              const float* input_scale, size_t batch, size_t rows_per_batch, size_t dim,
+                                              float eps, lq_stream_t stream);
 
 /* lq_gemm_fp8 (no activation) whose epilogue applies FLUX's gate and second residual:
  *   C[m,n] = T( T( T(y[m,n]) * gate[m / rows_per_gate, n] ) + residual[m,n] ),  y = (sa*sb)*acc + bias[n]

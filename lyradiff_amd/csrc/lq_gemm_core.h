@@ -52,6 +52,7 @@ struct GemmParams {
     uint8_t* C8;            // optional: e4m3 codes of C with a given (static) scale, written next to or instead of C
     const float* c8_scale;  // scale of C8: C8 = e4m3(f32(T(y)) * (1 / c8_scale[0]))
     size_t ldc8;            // row pitch of C8 in bytes (n when the codes are dense)
+    int c8_panel;           // C8 is written as k-panels [n / 64][m][64] (the next GEMM's activation layout, see a_panel); ldc8 unused
     // C is written with nontemporal stores: set for an output that is read once, by one streaming pass (the cast of a
     // dynamic-scale chain: out_scale given), and is too large to share the 256 MB last-level cache with the operands of
     // the GEMM after it.  Measured on the FLUX MLP chain (113 MB hidden tensor): up + cast + down 340-353 -> 319-330 us
@@ -778,7 +779,8 @@ struct GemmKernel {
                                 float tq[4];
 #pragma unroll
                                 for (int e = 0; e < 4; ++e) tq[e] = round_through<OutTag>(y[e]) * c8_inv;
-                                *reinterpret_cast<u32*>(p.C8 + (size_t)mo * p.ldc8 + out_n) = e4m3x4(tq[0], tq[1], tq[2], tq[3]);
+                                *reinterpret_cast<u32*>(p.C8 + (p.c8_panel ? ((size_t)(out_n >> 6) * p.m + mo) * 64 + (out_n & 63) : (size_t)mo * p.ldc8 + out_n)) =
+                                    e4m3x4(tq[0], tq[1], tq[2], tq[3]);
                             }
                         }
                         if constexpr (GEN) {

@@ -146,9 +146,9 @@ extern "C" int lq_gemm_fp8(void* C, lq_dtype_t out_dtype, const uint8_t* A, cons
                           nullptr, stream);
 }
 
-extern "C" int lq_gemm_fp8_gated(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32,
+static int gemm_fp8_gated(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32,
                                  const float* a_scale, const float* b_scale, const void* bias, const void* gate,
-                                 size_t rows_per_gate, const void* residual, int m, int n, int k, lq_stream_t stream) {
+                                 size_t rows_per_gate, const void* residual, int m, int n, int k, int a_panel, lq_stream_t stream) {
     int rc = fp8_check("lq_gemm_fp8_gated", C, A, B_rows32, a_scale, b_scale, bias, residual, m, n, k);
     if (rc != LQ_OK) return rc > 0 ? LQ_OK : rc;
     LQ_REQUIRE(C && gate && residual, LQ_ERR_ARG, "lq_gemm_fp8_gated: null pointer");
@@ -159,12 +159,25 @@ extern "C" int lq_gemm_fp8_gated(void* C, lq_dtype_t out_dtype, const uint8_t* A
     p.C = C; p.A = A; p.B = B_rows32; p.bias = bias; p.a_scale = a_scale; p.b_scale = b_scale;
     p.residual = residual; p.beta = 1.0f; p.gate = gate; p.gate_rows = rows_per_gate; p.ldc8 = (size_t)n;
     p.m = m; p.n = n; p.k = k; p.kb = k;
+    p.a_panel = a_panel;
     return fp8_dispatch("lq_gemm_fp8_gated", p, out_dtype, stream);
 }
 
-extern "C" int lq_gemm_fp8_codes(uint8_t* C_fp8, size_t ldc, const float* C_fp8_scale, lq_dtype_t round_dtype,
+extern "C" int lq_gemm_fp8_gated(void* C, lq_dtype_t out_dtype, const uint8_t* A, const uint8_t* B_rows32, const float* a_scale,
+                                 const float* b_scale, const void* bias, const void* gate, size_t rows_per_gate, const void* residual,
+                                 int m, int n, int k, lq_stream_t stream) {
+    return gemm_fp8_gated(C, out_dtype, A, B_rows32, a_scale, b_scale, bias, gate, rows_per_gate, residual, m, n, k, 0, stream);
+}
+
+extern "C" int lq_gemm_fp8_gated_panels(void* C, lq_dtype_t out_dtype, const uint8_t* A_panels, const uint8_t* B_rows32,
+                                        const float* a_scale, const float* b_scale, const void* bias, const void* gate,
+                                        size_t rows_per_gate, const void* residual, int m, int n, int k, lq_stream_t stream) {
+    return gemm_fp8_gated(C, out_dtype, A_panels, B_rows32, a_scale, b_scale, bias, gate, rows_per_gate, residual, m, n, k, 1, stream);
+}
+
+static int gemm_fp8_codes(uint8_t* C_fp8, size_t ldc, const float* C_fp8_scale, lq_dtype_t round_dtype,
                                  const uint8_t* A, const uint8_t* B_rows32, const float* a_scale, const float* b_scale,
-                                 const void* bias, int gelu, int m, int n, int k, lq_stream_t stream) {
+                                 const void* bias, int gelu, int m, int n, int k, int panels, lq_stream_t stream) {
     LQ_REQUIRE(gelu >= 0 && gelu <= 2, LQ_ERR_ARG, "lq_gemm_fp8_codes: gelu must be 0, 1 or 2");
     LQ_REQUIRE(ldc >= (size_t)(n > 0 ? n : 0) && ldc % 4 == 0, LQ_ERR_SHAPE, "lq_gemm_fp8_codes: need ldc >= n and ldc %% 4 == 0 (ldc=%zu n=%d)", ldc, n);
     int rc = fp8_check("lq_gemm_fp8_codes", nullptr, A, B_rows32, a_scale, b_scale, bias, nullptr, m, n, k);
@@ -176,5 +189,21 @@ extern "C" int lq_gemm_fp8_codes(uint8_t* C_fp8, size_t ldc, const float* C_fp8_
     p.A = A; p.B = B_rows32; p.bias = bias; p.a_scale = a_scale; p.b_scale = b_scale; p.gelu = gelu;
     p.C8 = C_fp8; p.c8_scale = C_fp8_scale; p.ldc8 = ldc;
     p.m = m; p.n = n; p.k = k; p.kb = k;
+    p.a_panel = panels;   // both the activation read and the codes written, or neither
+    p.c8_panel = panels;
+    LQ_REQUIRE(!panels || n % 64 == 0, LQ_ERR_SHAPE, "lq_gemm_fp8_codes_panels: codes in k-panels need n %% 64 == 0 (n=%d)", n);
     return fp8_dispatch("lq_gemm_fp8_codes", p, round_dtype, stream);
+}
+
+extern "C" int lq_gemm_fp8_codes(uint8_t* C_fp8, size_t ldc, const float* C_fp8_scale, lq_dtype_t round_dtype, const uint8_t* A,
+                                 const uint8_t* B_rows32, const float* a_scale, const float* b_scale, const void* bias, int gelu,
+                                 int m, int n, int k, lq_stream_t stream) {
+    return gemm_fp8_codes(C_fp8, ldc, C_fp8_scale, round_dtype, A, B_rows32, a_scale, b_scale, bias, gelu, m, n, k, 0, stream);
+}
+
+extern "C" int lq_gemm_fp8_codes_panels(uint8_t* C_fp8_panels, const float* C_fp8_scale, lq_dtype_t round_dtype,
+                                        const uint8_t* A_panels, const uint8_t* B_rows32, const float* a_scale, const float* b_scale,
+                                        const void* bias, int gelu, int m, int n, int k, lq_stream_t stream) {
+    return gemm_fp8_codes(C_fp8_panels, (size_t)(n > 0 ? n : 0), C_fp8_scale, round_dtype, A_panels, B_rows32, a_scale, b_scale, bias, gelu,
+                          m, n, k, 1, stream);
 }

@@ -76,7 +76,9 @@ __global__ __launch_bounds__(SPLIT ? 384 : 256) void ln_quant_rows_kernel(uint8_
                                                             const void* __restrict__ gamma, const void* __restrict__ beta,
                                                             const float* __restrict__ pre, const float* __restrict__ in_scale,
                                                             uint8_t* __restrict__ dst_b, const float* __restrict__ in_scale_b,
-                                                            size_t rows, int dim, size_t rows_per_batch, float eps, float rdim) {
+                                                            size_t rows, int dim, size_t rows_per_batch, float eps, float rdim, int codes_panel) {
+    // codes_panel (fp8 codes only): dst / dst_b are k-panels [dim / 64][rows][64] instead of row-major (a lane's eight codes
+    // stay inside one 64-byte segment), the activation layout of lq_gemm_fp8_panels
     __shared__ __attribute__((aligned(16))) float red[3][8];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const size_t row = SPLIT ? (size_t)blockIdx.x : (size_t)blockIdx.x * 4 + wave;
@@ -268,7 +270,7 @@ __global__ __launch_bounds__(SPLIT ? 384 : 256) void ln_quant_rows_kernel(uint8_
                     o.x = ln_nan_fix(o.x, v);
                     o.y = ln_nan_fix(o.y, v + 4);
                 }
-                st8<STREAM>(out + row_off + col, o);
+                st8<STREAM>(out + (codes_panel ? ((size_t)(col >> 6) * rows + row) * 64 + (col & 63) : row_off + col), o);
             }
         }
         }
@@ -296,7 +298,7 @@ __global__ __launch_bounds__(SPLIT ? 384 : 256) void ln_quant_rows_kernel(uint8_
 struct LnArgs {
     uint8_t* dst; void* dst2; float* scale_out; const void* src; const void* residual; const void* bias;
     const void* gamma; const void* beta; const float* pre; const float* in_scale; uint8_t* dst_b; const float* in_scale_b;
-    size_t rows; int dim; size_t rows_per_batch; float eps;
+    size_t rows; int dim; size_t rows_per_batch; float eps; int codes_panel;
 };
 
 template <typename Tag, int QMODE, int RESID, bool MOD> static int launch_ln(const LnArgs& a, hipStream_t st) {
@@ -308,19 +310,19 @@ template <typename Tag, int QMODE, int RESID, bool MOD> static int launch_ln(con
         const bool stream_io = QMODE != 3 && a.rows * (size_t)a.dim * 2 >= kStreamQuantBytes;
         if (a.dim % 1024 == 0 && stream_io)
             hipLaunchKernelGGL((ln_quant_rows_kernel<Tag, 2, QMODE, RESID, MOD, true, true, true>), grid, block, 0, st, a.dst, a.dst2, a.scale_out,
-                               a.src, a.residual, a.bias, a.gamma, a.beta, a.pre, a.in_scale, a.dst_b, a.in_scale_b, a.rows, a.dim, a.rows_per_batch, a.eps, 1.0f / (float)a.dim);
+                               a.src, a.residual, a.bias, a.gamma, a.beta, a.pre, a.in_scale, a.dst_b, a.in_scale_b, a.rows, a.dim, a.rows_per_batch, a.eps, 1.0f / (float)a.dim, a.codes_panel);
         else if (a.dim % 1024 == 0)
             hipLaunchKernelGGL((ln_quant_rows_kernel<Tag, 2, QMODE, RESID, MOD, true, true>), grid, block, 0, st, a.dst, a.dst2, a.scale_out,
-                               a.src, a.residual, a.bias, a.gamma, a.beta, a.pre, a.in_scale, a.dst_b, a.in_scale_b, a.rows, a.dim, a.rows_per_batch, a.eps, 1.0f / (float)a.dim);
+                               a.src, a.residual, a.bias, a.gamma, a.beta, a.pre, a.in_scale, a.dst_b, a.in_scale_b, a.rows, a.dim, a.rows_per_batch, a.eps, 1.0f / (float)a.dim, a.codes_panel);
         else
             hipLaunchKernelGGL((ln_quant_rows_kernel<Tag, 2, QMODE, RESID, MOD, true, false>), grid, block, 0, st, a.dst, a.dst2, a.scale_out,
-                               a.src, a.residual, a.bias, a.gamma, a.beta, a.pre, a.in_scale, a.dst_b, a.in_scale_b, a.rows, a.dim, a.rows_per_batch, a.eps, 1.0f / (float)a.dim);
+                               a.src, a.residual, a.bias, a.gamma, a.beta, a.pre, a.in_scale, a.dst_b, a.in_scale_b, a.rows, a.dim, a.rows_per_batch, a.eps, 1.0f / (float)a.dim, a.codes_panel);
         return check_launch("layernorm_quant");
     }
     dim3 grid((unsigned)((a.rows + 3) / 4)), block(256);
 #define LQ_LN_CASE(NPV)                                                                                              \
     hipLaunchKernelGGL((ln_quant_rows_kernel<Tag, NPV, QMODE, RESID, MOD, false>), grid, block, 0, st, a.dst, a.dst2, a.scale_out, \
-                       a.src, a.residual, a.bias, a.gamma, a.beta, a.pre, a.in_scale, a.dst_b, a.in_scale_b, a.rows, a.dim, a.rows_per_batch, a.eps, 1.0f / (float)a.dim)
+                       a.src, a.residual, a.bias, a.gamma, a.beta, a.pre, a.in_scale, a.dst_b, a.in_scale_b, a.rows, a.dim, a.rows_per_batch, a.eps, 1.0f / (float)a.dim, a.codes_panel)
     if (np <= 1) LQ_LN_CASE(1);
     else if (np <= 2) LQ_LN_CASE(2);
     else LQ_LN_CASE(3);
@@ -358,7 +360,7 @@ extern "C" int lq_layernorm_int8(int8_t* dst, float* scale_out, void* dst2, cons
                LQ_ERR_ARG, "lq_layernorm_int8: vectors must be 16-byte aligned");
     if (rows == 0) return LQ_OK;
     LnArgs a = {reinterpret_cast<uint8_t*>(dst), dst2, scale_out, src, residual, bias, gamma, beta, pre_quant_scale,
-                input_quant_scale, nullptr, nullptr, rows, (int)dim, 1, eps};
+                input_quant_scale, nullptr, nullptr, rows, (int)dim, 1, eps, 0};
     hipStream_t st = as_stream(stream);
     const bool dyn = scale_out != nullptr, res = residual != nullptr, f16 = dtype == LQ_F16;
 #define LQ_LN_GO(Tag)                                                                                   \
@@ -368,24 +370,37 @@ extern "C" int lq_layernorm_int8(int8_t* dst, float* scale_out, void* dst2, cons
 #undef LQ_LN_GO
 }
 
-extern "C" int lq_layernorm_mod_fp8(uint8_t* dst, const void* src, const void* scale, const void* shift, lq_dtype_t dtype,
+static int lq_layernorm_mod_fp8_impl(uint8_t* dst, const void* src, const void* scale, const void* shift, lq_dtype_t dtype,
                                     const float* input_scale, size_t batch, size_t rows_per_batch, size_t dim, float eps,
-                                    lq_stream_t stream) {
+                                    lq_stream_t stream, int panels) {
     int rc = check_ln_common("lq_layernorm_mod_fp8", dst, src, dtype, batch * rows_per_batch, dim);
     if (rc != LQ_OK) return rc;
     LQ_REQUIRE(scale && shift && input_scale, LQ_ERR_ARG, "lq_layernorm_mod_fp8: scale, shift and input_scale are required");
     LQ_REQUIRE(reinterpret_cast<uintptr_t>(scale) % 16 == 0 && reinterpret_cast<uintptr_t>(shift) % 16 == 0, LQ_ERR_ARG,
                "lq_layernorm_mod_fp8: scale and shift must be 16-byte aligned");
     if (batch * rows_per_batch == 0) return LQ_OK;
+    LQ_REQUIRE(!panels || dim % 64 == 0, LQ_ERR_SHAPE, "layernorm: codes in k-panels need dim %% 64 == 0 (dim=%zu)", dim);
     LnArgs a = {dst, nullptr, nullptr, src, nullptr, nullptr, scale, shift, nullptr, input_scale, nullptr, nullptr,
-                batch * rows_per_batch, (int)dim, rows_per_batch, eps};
+                batch * rows_per_batch, (int)dim, rows_per_batch, eps, panels};
     hipStream_t st = as_stream(stream);
     return dtype == LQ_F16 ? launch_ln<F16Tag, 2, 0, true>(a, st) : launch_ln<BF16Tag, 2, 0, true>(a, st);
 }
 
-extern "C" int lq_layernorm_mod_fp8_dual(uint8_t* dst_a, const float* input_scale_a, uint8_t* dst_b, const float* input_scale_b,
+extern "C" int lq_layernorm_mod_fp8(uint8_t* dst, const void* src, const void* scale, const void* shift, lq_dtype_t dtype,
+                                    const float* input_scale, size_t batch, size_t rows_per_batch, size_t dim, float eps,
+                                    lq_stream_t stream) {
+    return lq_layernorm_mod_fp8_impl(dst, src, scale, shift, dtype, input_scale, batch, rows_per_batch, dim, eps, stream, 0);
+}
+
+extern "C" int lq_layernorm_mod_fp8_panels(uint8_t* dst, const void* src, const void* scale, const void* shift, lq_dtype_t dtype,
+                                    const float* input_scale, size_t batch, size_t rows_per_batch, size_t dim, float eps,
+                                    lq_stream_t stream) {
+    return lq_layernorm_mod_fp8_impl(dst, src, scale, shift, dtype, input_scale, batch, rows_per_batch, dim, eps, stream, 1);
+}
+
+static int lq_layernorm_mod_fp8_dual_impl(uint8_t* dst_a, const float* input_scale_a, uint8_t* dst_b, const float* input_scale_b,
                                          const void* src, const void* scale, const void* shift, lq_dtype_t dtype, size_t batch,
-                                         size_t rows_per_batch, size_t dim, float eps, lq_stream_t stream) {
+                                         size_t rows_per_batch, size_t dim, float eps, lq_stream_t stream, int panels) {
     int rc = check_ln_common("lq_layernorm_mod_fp8_dual", dst_a, src, dtype, batch * rows_per_batch, dim);
     if (rc != LQ_OK) return rc;
     if (batch * rows_per_batch == 0) return LQ_OK;
@@ -394,10 +409,23 @@ extern "C" int lq_layernorm_mod_fp8_dual(uint8_t* dst_a, const float* input_scal
                    reinterpret_cast<uintptr_t>(dst_b) % 8 == 0,
                LQ_ERR_ARG, "lq_layernorm_mod_fp8_dual: scale and shift must be 16-byte, dst_b 8-byte aligned");
     if (batch * rows_per_batch == 0) return LQ_OK;
+    LQ_REQUIRE(!panels || dim % 64 == 0, LQ_ERR_SHAPE, "layernorm: codes in k-panels need dim %% 64 == 0 (dim=%zu)", dim);
     LnArgs a = {dst_a, nullptr, nullptr, src, nullptr, nullptr, scale, shift, nullptr, input_scale_a, dst_b, input_scale_b,
-                batch * rows_per_batch, (int)dim, rows_per_batch, eps};
+                batch * rows_per_batch, (int)dim, rows_per_batch, eps, panels};
     hipStream_t st = as_stream(stream);
     return dtype == LQ_F16 ? launch_ln<F16Tag, 2, 0, true>(a, st) : launch_ln<BF16Tag, 2, 0, true>(a, st);
+}
+
+extern "C" int lq_layernorm_mod_fp8_dual(uint8_t* dst_a, const float* input_scale_a, uint8_t* dst_b, const float* input_scale_b,
+                                         const void* src, const void* scale, const void* shift, lq_dtype_t dtype, size_t batch,
+                                         size_t rows_per_batch, size_t dim, float eps, lq_stream_t stream) {
+    return lq_layernorm_mod_fp8_dual_impl(dst_a, input_scale_a, dst_b, input_scale_b, src, scale, shift, dtype, batch, rows_per_batch, dim, eps, stream, 0);
+}
+
+extern "C" int lq_layernorm_mod_fp8_dual_panels(uint8_t* dst_a, const float* input_scale_a, uint8_t* dst_b, const float* input_scale_b,
+                                         const void* src, const void* scale, const void* shift, lq_dtype_t dtype, size_t batch,
+                                         size_t rows_per_batch, size_t dim, float eps, lq_stream_t stream) {
+    return lq_layernorm_mod_fp8_dual_impl(dst_a, input_scale_a, dst_b, input_scale_b, src, scale, shift, dtype, batch, rows_per_batch, dim, eps, stream, 1);
 }
 
 extern "C" int lq_gate_residual_layernorm_mod(void* dst, void* hidden_out, const void* attn, const void* gate, const void* input,
@@ -418,18 +446,18 @@ extern "C" int lq_gate_residual_layernorm_mod(void* dst, void* hidden_out, const
     hipStream_t st = as_stream(stream);
     if (gated) {
         LnArgs a = {static_cast<uint8_t*>(dst), hidden_out, nullptr, attn, input, gate, scale, shift, nullptr, nullptr, nullptr, nullptr,
-                    batch * rows_per_batch, (int)dim, rows_per_batch, eps};
+                    batch * rows_per_batch, (int)dim, rows_per_batch, eps, 0};
         return dtype == LQ_F16 ? launch_ln<F16Tag, 3, 2, true>(a, st) : launch_ln<BF16Tag, 3, 2, true>(a, st);
     }
     LnArgs a = {static_cast<uint8_t*>(dst), nullptr, nullptr, input, nullptr, nullptr, scale, shift, nullptr, nullptr, nullptr, nullptr,
-                batch * rows_per_batch, (int)dim, rows_per_batch, eps};
+                batch * rows_per_batch, (int)dim, rows_per_batch, eps, 0};
     return dtype == LQ_F16 ? launch_ln<F16Tag, 3, 0, true>(a, st) : launch_ln<BF16Tag, 3, 0, true>(a, st);
 }
 
-extern "C" int lq_gate_residual_layernorm_mod_fp8(uint8_t* dst, void* hidden_out, const void* attn, const void* gate,
+static int lq_gate_residual_layernorm_mod_fp8_impl(uint8_t* dst, void* hidden_out, const void* attn, const void* gate,
                                                   const void* input, const void* scale, const void* shift, lq_dtype_t dtype,
                                                   const float* input_scale, size_t batch, size_t rows_per_batch, size_t dim,
-                                                  float eps, lq_stream_t stream) {
+                                                  float eps, lq_stream_t stream, int panels) {
     int rc = check_ln_common("lq_gate_residual_layernorm_mod_fp8", dst, attn, dtype, batch * rows_per_batch, dim);
     if (rc != LQ_OK) return rc;
     if (batch * rows_per_batch == 0) return LQ_OK;
@@ -440,8 +468,23 @@ extern "C" int lq_gate_residual_layernorm_mod_fp8(uint8_t* dst, void* hidden_out
                    reinterpret_cast<uintptr_t>(hidden_out) % 16 == 0,
                LQ_ERR_ARG, "lq_gate_residual_layernorm_mod_fp8: all tensors must be 16-byte aligned");
     if (batch * rows_per_batch == 0) return LQ_OK;
+    LQ_REQUIRE(!panels || dim % 64 == 0, LQ_ERR_SHAPE, "layernorm: codes in k-panels need dim %% 64 == 0 (dim=%zu)", dim);
     LnArgs a = {dst, hidden_out, nullptr, attn, input, gate, scale, shift, nullptr, input_scale, nullptr, nullptr,
-                batch * rows_per_batch, (int)dim, rows_per_batch, eps};
+                batch * rows_per_batch, (int)dim, rows_per_batch, eps, panels};
     hipStream_t st = as_stream(stream);
     return dtype == LQ_F16 ? launch_ln<F16Tag, 2, 2, true>(a, st) : launch_ln<BF16Tag, 2, 2, true>(a, st);
+}
+
+extern "C" int lq_gate_residual_layernorm_mod_fp8(uint8_t* dst, void* hidden_out, const void* attn, const void* gate,
+                                                  const void* input, const void* scale, const void* shift, lq_dtype_t dtype,
+                                                  const float* input_scale, size_t batch, size_t rows_per_batch, size_t dim,
+                                                  float eps, lq_stream_t stream) {
+    return lq_gate_residual_layernorm_mod_fp8_impl(dst, hidden_out, attn, gate, input, scale, shift, dtype, input_scale, batch, rows_per_batch, dim, eps, stream, 0);
+}
+
+extern "C" int lq_gate_residual_layernorm_mod_fp8_panels(uint8_t* dst, void* hidden_out, const void* attn, const void* gate,
+                                                  const void* input, const void* scale, const void* shift, lq_dtype_t dtype,
+                                                  const float* input_scale, size_t batch, size_t rows_per_batch, size_t dim,
+                                                  float eps, lq_stream_t stream) {
+    return lq_gate_residual_layernorm_mod_fp8_impl(dst, hidden_out, attn, gate, input, scale, shift, dtype, input_scale, batch, rows_per_batch, dim, eps, stream, 1);
 }

@@ -97,6 +97,11 @@ SYMBOLS = {
     "lq_gemm_fp8_max": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _P, _P]),
     "lq_fp8_gelu_cast": (_I, [_P, _P, _P, _P, _I, _Z, _P, _P, _P]),
     "lq_fp8_amax_cast_panels": (_I, [_P, _P, _P, _I, _Z, _Z, _P]),
+    "lq_layernorm_mod_fp8_panels": (_I, [_P, _P, _P, _P, _I, _P, _Z, _Z, _Z, _F, _P]),
+    "lq_layernorm_mod_fp8_dual_panels": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _Z, _Z, _Z, _F, _P]),
+    "lq_gate_residual_layernorm_mod_fp8_panels": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _P, _Z, _Z, _Z, _F, _P]),
+    "lq_gemm_fp8_gated_panels": (_I, [_P, _I, _P, _P, _P, _P, _P, _P, _Z, _P, _I, _I, _I, _P]),
+    "lq_gemm_fp8_codes_panels": (_I, [_P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "lq_fp8_scale_cast_panels": (_I, [_P, _P, _I, _P, _I, _Z, _Z, _P]),
     "lq_sq_dynamic_quant_panels": (_I, [_P, _P, _P, _I, _P, _Z, _Z, _P]),
     "lq_gemm_int8_panels": (_I, [_P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _P]),

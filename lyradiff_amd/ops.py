@@ -202,22 +202,32 @@ def layernorm_int8(x, gamma, beta, pre_quant_scale=None, input_quant_scale=None,
     return q, s, h
 
 
-def layernorm_mod_fp8(x, scale, shift, input_scale, eps: float = 1e-6):
+def _codes_like(x, panels: bool):
+    """Destination of the e4m3 codes of x [B, S, D]: the same shape, or k-panels [D/64, B*S, 64] (see fp8_quant_panels)."""
+    if not panels:
+        return torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    if x.shape[-1] % 64 != 0:
+        raise ValueError("codes in k-panels need a last dimension that is a multiple of 64")
+    return torch.empty((x.shape[-1] // 64, x.numel() // x.shape[-1], 64), dtype=torch.uint8, device=x.device)
+
+
+def layernorm_mod_fp8(x, scale, shift, input_scale, eps: float = 1e-6, panels: bool = False):
     """invokeLayerNormWithShiftAndScale + FP8 cast: x [B, S, D], scale/shift [B, D], static input_scale [1];
-    returns e4m3 codes (uint8) of shape x."""
+    returns e4m3 codes (uint8) of shape x, or with panels=True as k-panels [D/64, B*S, 64]."""
     _chk(x, "x", (torch.float16, torch.bfloat16))
     _chk(scale, "scale", (x.dtype,))
     _chk(shift, "shift", (x.dtype,))
     _chk(input_scale, "input_scale", (torch.float32,))
     if x.dim() != 3 or tuple(scale.shape) != (x.shape[0], x.shape[2]) or scale.shape != shift.shape:
         raise ValueError("x must be [B,S,D] and scale, shift [B,D]")
-    q = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
-    _l.check(_l.load().lq_layernorm_mod_fp8(_ptr(q), _ptr(x), _ptr(scale), _ptr(shift), _DT[x.dtype], _ptr(input_scale),
-                                            x.shape[0], x.shape[1], x.shape[2], float(eps), _stream()), "lq_layernorm_mod_fp8")
+    q = _codes_like(x, panels)
+    fn = _l.load().lq_layernorm_mod_fp8_panels if panels else _l.load().lq_layernorm_mod_fp8
+    _l.check(fn(_ptr(q), _ptr(x), _ptr(scale), _ptr(shift), _DT[x.dtype], _ptr(input_scale),
+                x.shape[0], x.shape[1], x.shape[2], float(eps), _stream()), "lq_layernorm_mod_fp8")
     return q
 
 
-def layernorm_mod_fp8_dual(x, scale, shift, input_scale_a, input_scale_b, eps: float = 1e-6):
+def layernorm_mod_fp8_dual(x, scale, shift, input_scale_a, input_scale_b, eps: float = 1e-6, panels: bool = False):
     """layernorm_mod_fp8 for two consumers of the normalised tensor: returns (codes_a, codes_b)."""
     _chk(x, "x", (torch.float16, torch.bfloat16))
     _chk(scale, "scale", (x.dtype,))
@@ -226,15 +236,15 @@ def layernorm_mod_fp8_dual(x, scale, shift, input_scale_a, input_scale_b, eps: f
     _chk(input_scale_b, "input_scale_b", (torch.float32,))
     if x.dim() != 3 or tuple(scale.shape) != (x.shape[0], x.shape[2]) or scale.shape != shift.shape:
         raise ValueError("x must be [B,S,D] and scale, shift [B,D]")
-    qa = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
-    qb = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
-    _l.check(_l.load().lq_layernorm_mod_fp8_dual(_ptr(qa), _ptr(input_scale_a), _ptr(qb), _ptr(input_scale_b), _ptr(x),
-                                                 _ptr(scale), _ptr(shift), _DT[x.dtype], x.shape[0], x.shape[1], x.shape[2],
-                                                 float(eps), _stream()), "lq_layernorm_mod_fp8_dual")
+    qa, qb = _codes_like(x, panels), _codes_like(x, panels)
+    fn = _l.load().lq_layernorm_mod_fp8_dual_panels if panels else _l.load().lq_layernorm_mod_fp8_dual
+    _l.check(fn(_ptr(qa), _ptr(input_scale_a), _ptr(qb), _ptr(input_scale_b), _ptr(x), _ptr(scale), _ptr(shift), _DT[x.dtype],
+                x.shape[0], x.shape[1], x.shape[2], float(eps), _stream()), "lq_layernorm_mod_fp8_dual")
     return qa, qb
 
 
-def gate_residual_layernorm_mod_fp8(attn, gate, x, scale, shift, input_scale, eps: float = 1e-6, hidden_out=None):
+def gate_residual_layernorm_mod_fp8(attn, gate, x, scale, shift, input_scale, eps: float = 1e-6, hidden_out=None,
+                                    panels: bool = False):
     """invokeFusedGateAndResidual + invokeLayerNormWithShiftAndScale + FP8 cast in one pass:
     hidden = x + gate*attn (each op rounded to the tensor dtype), codes = e4m3(adaLN(hidden) / input_scale).
     attn, x [B,S,D]; gate, scale, shift [B,D].  Returns (codes, hidden); hidden_out may be x itself."""
@@ -247,10 +257,10 @@ def gate_residual_layernorm_mod_fp8(attn, gate, x, scale, shift, input_scale, ep
     if hidden_out is None:
         hidden_out = torch.empty_like(x)
     _chk(hidden_out, "hidden_out", (x.dtype,))
-    q = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
-    _l.check(_l.load().lq_gate_residual_layernorm_mod_fp8(_ptr(q), _ptr(hidden_out), _ptr(attn), _ptr(gate), _ptr(x), _ptr(scale),
-                                                          _ptr(shift), _DT[x.dtype], _ptr(input_scale), x.shape[0], x.shape[1],
-                                                          x.shape[2], float(eps), _stream()),
+    q = _codes_like(x, panels)
+    fn = _l.load().lq_gate_residual_layernorm_mod_fp8_panels if panels else _l.load().lq_gate_residual_layernorm_mod_fp8
+    _l.check(fn(_ptr(q), _ptr(hidden_out), _ptr(attn), _ptr(gate), _ptr(x), _ptr(scale), _ptr(shift), _DT[x.dtype],
+                _ptr(input_scale), x.shape[0], x.shape[1], x.shape[2], float(eps), _stream()),
              "lq_gate_residual_layernorm_mod_fp8")
     return q, hidden_out
 
@@ -509,17 +519,29 @@ def fp8_panels_to_rows(q_panels):
     return q_panels.permute(1, 0, 2).reshape(m, kp * w).contiguous()
 
 
-def fp8_scale_cast_panels(x, scale, invert: bool = True):
-    """fp8_scale_cast (a given scale: the reference's static input scale) of a 2-D x [M, K] into k-panels uint8 [K/64, M, 64]."""
+def _panel_block(out, m: int, n: int, col_offset: int) -> int:
+    """Address of columns [col_offset, col_offset + n) inside k-panels out [W/64, M, 64]: a block of columns is a run of whole
+    panels, so writing into a wider destination is a pointer offset."""
+    _chk(out, "out", (torch.uint8,))
+    if out.dim() != 3 or out.shape[1] != m or out.shape[2] != 64 or col_offset < 0 or col_offset % 64 != 0 or n % 64 != 0 or \
+            col_offset + n > out.shape[0] * 64:
+        raise ValueError("out must be k-panels [W/64, M, 64] with col_offset and N multiples of 64 and col_offset + N <= W")
+    return out.data_ptr() + (col_offset // 64) * m * 64
+
+
+def fp8_scale_cast_panels(x, scale, invert: bool = True, out=None, col_offset: int = 0):
+    """fp8_scale_cast (a given scale: the reference's static input scale) of a 2-D x [M, K] into k-panels uint8 [K/64, M, 64],
+    or into columns [col_offset, col_offset + K) of wider k-panels `out` [W/64, M, 64]."""
     _chk(x, "x", _FLOATS)
     _chk(scale, "scale", (torch.float32,))
     if x.dim() != 2 or x.shape[1] % 64 != 0:
         raise ValueError("fp8_scale_cast_panels: x must be [M, K] with K % 64 == 0")
     m, k = x.shape
-    q = torch.empty((k // 64, m, 64), dtype=torch.uint8, device=x.device)
-    _l.check(_l.load().lq_fp8_scale_cast_panels(_ptr(q), _ptr(x), _DT[x.dtype], _ptr(scale), int(invert), m, k, _stream()),
-             "lq_fp8_scale_cast_panels")
-    return q
+    if out is None:
+        out = torch.empty((k // 64, m, 64), dtype=torch.uint8, device=x.device)
+    _l.check(_l.load().lq_fp8_scale_cast_panels(_panel_block(out, m, k, col_offset), _ptr(x), _DT[x.dtype], _ptr(scale), int(invert), m, k,
+                                                _stream()), "lq_fp8_scale_cast_panels")
+    return out
 
 
 def fp8_quant_panels(x):
@@ -669,6 +691,61 @@ def fp8_linear_codes(a_q, w_rows32, a_scale, b_scale, bias, out_fp8_scale, gelu:
     _l.check(_l.load().lq_gemm_fp8_codes(out.data_ptr() + col_offset, out.shape[1], _ptr(out_fp8_scale), _DT[round_dtype],
                                          _ptr(a_q), _ptr(w_rows32), _ptr(a_scale), _ptr(b_scale), _ptr(bias), int(gelu), m, n, k,
                                          _stream()), "lq_gemm_fp8_codes")
+    return out
+
+
+def fp8_linear_gated_panels(a_panels, w_rows32, a_scale, b_scale, bias, gate, residual, rows_per_gate: int, out=None):
+    """fp8_linear_gated on an activation in k-panels [K/64, M, 64].  Same bits as the row-major call."""
+    _chk(a_panels, "a_panels", (torch.uint8,))
+    _chk(w_rows32, "w_rows32", (torch.uint8,))
+    _chk(a_scale, "a_scale", (torch.float32,))
+    _chk(b_scale, "b_scale", (torch.float32,))
+    _chk(residual, "residual", _FLOATS)
+    _chk(gate, "gate", (residual.dtype,))
+    if bias is not None:
+        _chk(bias, "bias", (residual.dtype,))
+    if a_panels.dim() != 3 or a_panels.shape[2] != 64:
+        raise ValueError("a_panels must be [K/64, M, 64]")
+    kp, m, _ = a_panels.shape
+    k, n = kp * 64, w_rows32.shape[0]
+    if w_rows32.shape[1] != k:
+        raise ValueError("K mismatch between activation and weight")
+    if residual.numel() != m * n or rows_per_gate <= 0 or gate.numel() != ((m + rows_per_gate - 1) // rows_per_gate) * n:
+        raise ValueError("residual must be [M,N] and gate [ceil(M/rows_per_gate), N]")
+    if out is None:
+        out = torch.empty((m, n), dtype=residual.dtype, device=a_panels.device)
+    _chk(out, "out", (residual.dtype,))
+    _l.check(_l.load().lq_gemm_fp8_gated_panels(_ptr(out), _DT[residual.dtype], _ptr(a_panels), _ptr(w_rows32), _ptr(a_scale),
+                                                _ptr(b_scale), _ptr(bias), _ptr(gate), int(rows_per_gate), _ptr(residual), m, n, k,
+                                                _stream()), "lq_gemm_fp8_gated_panels")
+    return out
+
+
+def fp8_linear_codes_panels(a_panels, w_rows32, a_scale, b_scale, bias, out_fp8_scale, gelu: int = 0, round_dtype=torch.bfloat16,
+                            out=None, col_offset: int = 0):
+    """fp8_linear_codes with both the activation and the codes it writes as k-panels: a_panels [K/64, M, 64] -> codes
+    [N/64, M, 64], or columns [col_offset, col_offset + N) of wider k-panels `out` [W/64, M, 64].  Same codes as the row-major
+    call."""
+    _chk(a_panels, "a_panels", (torch.uint8,))
+    _chk(w_rows32, "w_rows32", (torch.uint8,))
+    _chk(a_scale, "a_scale", (torch.float32,))
+    _chk(b_scale, "b_scale", (torch.float32,))
+    _chk(out_fp8_scale, "out_fp8_scale", (torch.float32,))
+    if bias is not None:
+        _chk(bias, "bias", (round_dtype,))
+    if a_panels.dim() != 3 or a_panels.shape[2] != 64:
+        raise ValueError("a_panels must be [K/64, M, 64]")
+    kp, m, _ = a_panels.shape
+    k, n = kp * 64, w_rows32.shape[0]
+    if w_rows32.shape[1] != k:
+        raise ValueError("K mismatch between activation and weight")
+    if n % 64 != 0:
+        raise ValueError("codes in k-panels need N % 64 == 0")
+    if out is None:
+        out = torch.empty((n // 64, m, 64), dtype=torch.uint8, device=a_panels.device)
+    _l.check(_l.load().lq_gemm_fp8_codes_panels(_panel_block(out, m, n, col_offset), _ptr(out_fp8_scale), _DT[round_dtype], _ptr(a_panels),
+                                                _ptr(w_rows32), _ptr(a_scale), _ptr(b_scale), _ptr(bias), int(gelu), m, n, k, _stream()),
+             "lq_gemm_fp8_codes_panels")
     return out
 
 

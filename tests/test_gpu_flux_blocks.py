@@ -67,6 +67,63 @@ def test_gemm_fp8_gated_matches_unfused_bit_for_bit(ops, dev, dt, m, n, k, rpg):
     assert out.data_ptr() == res2.data_ptr() and np.array_equal(to_np_f32(res2), want)
 
 
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("m,n,k,rpg", [(4608, 3072, 1024, 4608), (600, 256, 128, 77), (37, 64, 64, 5)])
+def test_static_scale_ops_on_k_panels_give_the_row_major_bits(ops, dev, dt, m, n, k, rpg):
+    """The FLUX blocks' static-scale sequence with its FP8 activations as k-panels [K/64, M, 64]: LayerNorm + cast kernels
+    that write them, the GEMM that reads them and writes the next activation's codes as panels (also into a block of
+    columns of a wider tensor), the gated GEMM that reads those."""
+    t = TORCH_DT[dt]
+    g = rng_t(m + 7 * n + k)
+    qa, sa, wr, _, sw, bias = _fp8_operands(ops, dev, m, n, k, 300 + m + n, dt)
+    qa_p = qa.view(m, k // 64, 64).permute(1, 0, 2).contiguous()
+    nb = (m + rpg - 1) // rpg
+    gate = torch.randn(nb, n, generator=g).to(t).to(dev)
+    res = (2 * torch.randn(m, n, generator=g)).to(t).to(dev)
+    assert torch.equal(ops.fp8_linear_gated_panels(qa_p, wr, sa, sw, bias, gate, res, rpg), ops.fp8_linear_gated(qa, wr, sa, sw, bias, gate, res, rpg))
+    s_out = torch.tensor([0.013], dtype=torch.float32, device=dev)
+    for gelu in (0, 2):
+        dense = ops.fp8_linear_codes(qa, wr, sa, sw, bias, s_out, gelu=gelu, round_dtype=t)
+        assert torch.equal(ops.fp8_panels_to_rows(ops.fp8_linear_codes_panels(qa_p, wr, sa, sw, bias, s_out, gelu=gelu, round_dtype=t)), dense)
+        wide = torch.full(((128 + n + 64) // 64, m, 64), 0xAB, dtype=torch.uint8, device=dev)
+        ops.fp8_linear_codes_panels(qa_p, wr, sa, sw, bias, s_out, gelu=gelu, round_dtype=t, out=wide, col_offset=128)
+        rows = ops.fp8_panels_to_rows(wide)
+        assert torch.equal(rows[:, 128:128 + n], dense) and (rows[:, :128] == 0xAB).all() and (rows[:, 128 + n:] == 0xAB).all()
+    for tac in range(ops.gemm_tactic_count("fp8")):
+        with ops.gemm_thread_tactic(tac):
+            assert torch.equal(ops.fp8_panels_to_rows(ops.fp8_linear_codes_panels(qa_p, wr, sa, sw, bias, s_out, gelu=1, round_dtype=t)),
+                               ops.fp8_linear_codes(qa, wr, sa, sw, bias, s_out, gelu=1, round_dtype=t)), tac
+    # the static cast into a block of columns of wider panels
+    xs = torch.randn(m, 128, generator=g).to(t).to(dev)
+    wide = torch.full((5, m, 64), 0xAB, dtype=torch.uint8, device=dev)
+    ops.fp8_scale_cast_panels(xs, s_out, out=wide, col_offset=64)
+    rows = ops.fp8_panels_to_rows(wide)
+    assert torch.equal(rows[:, 64:192], ops.fp8_scale_cast(xs, s_out)) and (rows[:, :64] == 0xAB).all() and (rows[:, 192:] == 0xAB).all()
+    with pytest.raises(ValueError):
+        ops.fp8_linear_codes_panels(qa_p, wr, sa, sw, bias, s_out, round_dtype=t, out=wide, col_offset=32)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("batch,seq,dim", [(2, 2304, 3072), (3, 50, 768), (1, 37, 2560)])
+def test_layernorm_fp8_kernels_writing_k_panels(ops, dev, dt, batch, seq, dim):
+    t = TORCH_DT[dt]
+    g = rng_t(batch + seq + dim)
+    x = (torch.randn(batch, seq, dim, generator=g) * 1.5).to(t).to(dev)
+    attn = torch.randn(batch, seq, dim, generator=g).to(t).to(dev)
+    gate, scale, shift = [(0.3 * torch.randn(batch, dim, generator=g)).to(t).to(dev) for _ in range(3)]
+    s_a = torch.tensor([0.011], dtype=torch.float32, device=dev)
+    s_b = torch.tensor([0.017], dtype=torch.float32, device=dev)
+    rows = lambda q: ops.fp8_panels_to_rows(q).view(batch, seq, dim)
+    q_p = ops.layernorm_mod_fp8(x, scale, shift, s_a, panels=True)
+    assert q_p.shape == (dim // 64, batch * seq, 64) and torch.equal(rows(q_p), ops.layernorm_mod_fp8(x, scale, shift, s_a))
+    qa_p, qb_p = ops.layernorm_mod_fp8_dual(x, scale, shift, s_a, s_b, panels=True)
+    qa, qb = ops.layernorm_mod_fp8_dual(x, scale, shift, s_a, s_b)
+    assert torch.equal(rows(qa_p), qa) and torch.equal(rows(qb_p), qb)
+    q2_p, h_p = ops.gate_residual_layernorm_mod_fp8(attn, gate, x, scale, shift, s_a, panels=True)
+    q2, h = ops.gate_residual_layernorm_mod_fp8(attn, gate, x, scale, shift, s_a)
+    assert torch.equal(rows(q2_p), q2) and torch.equal(h_p, h)
+
+
 def test_gemm_fp8_gated_every_tactic(ops, dev):
     m, n, k, rpg = 700, 512, 256, 300
     qa, sa, wr, _, sw, bias = _fp8_operands(ops, dev, m, n, k, 7, "bf16")
