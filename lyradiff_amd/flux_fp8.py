@@ -95,12 +95,13 @@ def load_ada_layernorm(src, prefix: str, dim: int, n_chunks: int, full: bool, dt
 
 
 def ada_fp8_layernorm(x: torch.Tensor, temb: torch.Tensor, linear: Union[FP8Linear, AdaLinear16], n_chunks: int, code_scales=(),
-                      switch_scale: bool = False, eps: float = 1e-6):
+                      switch_scale: bool = False, eps: float = 1e-6, panels: bool = False):
     """AdaFP8LayerNorm<T>::forward (layers/ada_layer_norm/AdaFP8LayerNorm.cc:93-205): msa = FP8 linear of the
     (already SiLU'd) time embedding, stored [n_chunks, B, D]; output = (1 + msa[1]) * LayerNorm(x) + msa[0]
     (msa[0]/msa[1] swapped with switch_scale).  x [B, S, D], temb [B, D].
     code_scales: () -> the 16-bit normalised tensor as the reference writes it; one or two fp32 [1] input scales ->
-    the e4m3 codes for the FP8 linears that consume it instead (cast fused, no 16-bit tensor).
+    the e4m3 codes for the FP8 linears that consume it instead (cast fused, no 16-bit tensor); with panels=True the codes
+    are k-panels [D/64, B*S, 64] (ops.fp8_quant_panels) instead of [B, S, D].
     Returns (norm | codes | (codes_a, codes_b), msa)."""
     b, s, d = x.shape
     if isinstance(linear, AdaLinear16):  # not a quantized linear: a plain 16-bit matmul (AdaLayerNorm.cc)
@@ -113,8 +114,8 @@ def ada_fp8_layernorm(x: torch.Tensor, temb: torch.Tensor, linear: Union[FP8Line
     if len(code_scales) == 0:
         return ops.gate_residual_layernorm_mod(x, scale, shift, eps=eps), msa
     if len(code_scales) == 1:
-        return ops.layernorm_mod_fp8(x, scale, shift, code_scales[0], eps), msa
-    return ops.layernorm_mod_fp8_dual(x, scale, shift, code_scales[0], code_scales[1], eps), msa
+        return ops.layernorm_mod_fp8(x, scale, shift, code_scales[0], eps, panels=panels), msa
+    return ops.layernorm_mod_fp8_dual(x, scale, shift, code_scales[0], code_scales[1], eps, panels=panels), msa
 
 
 def flux_attn_post_fp8(x: torch.Tensor, attn_output: torch.Tensor, msa: torch.Tensor, w: FluxAttnPostFP8Weights,
@@ -124,29 +125,42 @@ def flux_attn_post_fp8(x: torch.Tensor, attn_output: torch.Tensor, msa: torch.Te
     if tuple(msa.shape) != (6, b, d):
         raise ValueError("msa must be [6, B, D]")
     gate_msa, shift_mlp, scale_mlp, gate_mlp = msa[2], msa[3], msa[4], msa[5]
-    q1, hidden = ops.gate_residual_layernorm_mod_fp8(attn_output, gate_msa, x, scale_mlp, shift_mlp, w.gelu_proj.input_scale, eps)
-    q2 = ops.fp8_linear_codes(q1.view(b * s, d), w.gelu_proj.weight_rows32, w.gelu_proj.input_scale, w.gelu_proj.weight_scale,
-                              w.gelu_proj.bias, w.ff_linear.input_scale, gelu=1, round_dtype=x.dtype)
-    out = ops.fp8_linear_gated(q2, w.ff_linear.weight_rows32, w.ff_linear.input_scale, w.ff_linear.weight_scale,
-                               w.ff_linear.bias, gate_mlp, hidden.view(b * s, d), rows_per_gate=s)
+    # the two FP8 activations of the sequence travel as k-panels [K/64, B*S, 64] (whole cache lines for the GEMMs' transfers)
+    q1, hidden = ops.gate_residual_layernorm_mod_fp8(attn_output, gate_msa, x, scale_mlp, shift_mlp, w.gelu_proj.input_scale, eps,
+                                                     panels=True)
+    q2 = ops.fp8_linear_codes_panels(q1, w.gelu_proj.weight_rows32, w.gelu_proj.input_scale, w.gelu_proj.weight_scale,
+                                     w.gelu_proj.bias, w.ff_linear.input_scale, gelu=1, round_dtype=x.dtype)
+    out = ops.fp8_linear_gated_panels(q2, w.ff_linear.weight_rows32, w.ff_linear.input_scale, w.ff_linear.weight_scale,
+                                      w.ff_linear.bias, gate_mlp, hidden.view(b * s, d), rows_per_gate=s)
     return out.view(b, s, d)
 
 
 def flux_single_mlp_fp8(x: torch.Tensor, norm_hidden, attn_output: torch.Tensor, gate: torch.Tensor,
-                        w: FluxSingleMlpFP8Weights) -> torch.Tensor:
+                        w: FluxSingleMlpFP8Weights, norm_in_panels: bool = False) -> torch.Tensor:
     """x, attn_output [B, S, D]; gate [B, D] (chunk 2 of the single block's msa) -> output [B, S, D].
     norm_hidden is either the 16-bit adaLN output [B, S, D] (cast here with proj_mlp's input scale) or its e4m3
-    codes for proj_mlp (uint8 [B, S, D], e.g. the second output of ops.layernorm_mod_fp8_dual)."""
+    codes for proj_mlp: uint8 [B, S, D], or with norm_in_panels uint8 k-panels [D/64, B*S, 64] (the second output of
+    ops.layernorm_mod_fp8_dual)."""
     b, s, d = x.shape
     m = b * s
     f = w.proj_mlp.weight_rows32.shape[0]
-    q1 = norm_hidden if norm_hidden.dtype == torch.uint8 else ops.fp8_scale_cast(norm_hidden, w.proj_mlp.input_scale)
-    q2 = torch.empty((m, d + f), dtype=torch.uint8, device=x.device)
-    ops.fp8_scale_cast_into(attn_output.view(m, d), w.proj_out.input_scale, q2, 0)
-    ops.fp8_linear_codes(q1.view(m, d), w.proj_mlp.weight_rows32, w.proj_mlp.input_scale, w.proj_mlp.weight_scale,
-                         w.proj_mlp.bias, w.proj_out.input_scale, gelu=2, round_dtype=x.dtype, out=q2, col_offset=d)
-    out = ops.fp8_linear_gated(q2, w.proj_out.weight_rows32, w.proj_out.input_scale, w.proj_out.weight_scale,
-                               w.proj_out.bias, gate, x.view(m, d), rows_per_gate=s)
+    if norm_hidden.dtype == torch.uint8 and not norm_in_panels:  # row-major codes from the caller: the row-major sequence
+        q2 = torch.empty((m, d + f), dtype=torch.uint8, device=x.device)
+        ops.fp8_scale_cast_into(attn_output.view(m, d), w.proj_out.input_scale, q2, 0)
+        ops.fp8_linear_codes(norm_hidden.view(m, d), w.proj_mlp.weight_rows32, w.proj_mlp.input_scale, w.proj_mlp.weight_scale,
+                             w.proj_mlp.bias, w.proj_out.input_scale, gelu=2, round_dtype=x.dtype, out=q2, col_offset=d)
+        out = ops.fp8_linear_gated(q2, w.proj_out.weight_rows32, w.proj_out.input_scale, w.proj_out.weight_scale,
+                                   w.proj_out.bias, gate, x.view(m, d), rows_per_gate=s)
+        return out.view(b, s, d)
+    # every FP8 activation as k-panels: the concatenated input of proj_out is [ (D + F)/64, M, 64 ], its two column blocks
+    # (attention output, GELU of proj_mlp) are runs of whole panels
+    q1 = norm_hidden if norm_hidden.dtype == torch.uint8 else ops.fp8_scale_cast_panels(norm_hidden.view(m, d), w.proj_mlp.input_scale)
+    q2 = torch.empty(((d + f) // 64, m, 64), dtype=torch.uint8, device=x.device)
+    ops.fp8_scale_cast_panels(attn_output.view(m, d), w.proj_out.input_scale, out=q2, col_offset=0)
+    ops.fp8_linear_codes_panels(q1, w.proj_mlp.weight_rows32, w.proj_mlp.input_scale, w.proj_mlp.weight_scale,
+                                w.proj_mlp.bias, w.proj_out.input_scale, gelu=2, round_dtype=x.dtype, out=q2, col_offset=d)
+    out = ops.fp8_linear_gated_panels(q2, w.proj_out.weight_rows32, w.proj_out.input_scale, w.proj_out.weight_scale,
+                                      w.proj_out.bias, gate, x.view(m, d), rows_per_gate=s)
     return out.view(b, s, d)
 
 
@@ -195,28 +209,29 @@ def load_flux_double_block_fp8(src, prefix: str, dim: int, dtype=torch.bfloat16,
                                      load_flux_attn_post_fp8(src, prefix + "ff_context.", dim, dtype, device, keep_master))
 
 
-def _linear_from_codes(lin: FP8Linear, codes: torch.Tensor, dtype) -> torch.Tensor:
-    m = codes.numel() // codes.shape[-1]
-    y = ops.fp8_linear(codes.view(m, codes.shape[-1]), lin.weight_rows32, lin.input_scale, lin.weight_scale, lin.bias, out_dtype=dtype)
-    return y.view(*codes.shape[:-1], y.shape[-1])
+def _linear_from_panels(lin: FP8Linear, panels: torch.Tensor, batch: int, dtype) -> torch.Tensor:
+    """FP8 linear on codes in k-panels [K/64, B*S, 64] -> [B, S, N]."""
+    y = ops.fp8_linear_panels(panels, lin.weight_rows32, lin.input_scale, lin.weight_scale, lin.bias, None, dtype)
+    return y.view(batch, y.shape[0] // batch, y.shape[1])
 
 
 def flux_single_block_fp8(x: torch.Tensor, temb: torch.Tensor, w: FluxSingleBlockFP8Weights, attention) -> torch.Tensor:
     """FluxSingleTransformerFP8Block<T>::forward (FluxSingleTransformerFP8Block.cc:163-291).  x [B, S, D], temb [B, D]
     (SiLU already applied); attention(qkv [B, S, 3D]) -> [B, S, D].  One adaLN read yields the codes for to_qkv and for
     proj_mlp; five launches besides the attention."""
-    (c_qkv, c_mlp), msa = ada_fp8_layernorm(x, temb, w.norm, 3, (w.to_qkv.input_scale, w.mlp.proj_mlp.input_scale))
-    attn_out = attention(_linear_from_codes(w.to_qkv, c_qkv, x.dtype))
-    return flux_single_mlp_fp8(x, c_mlp, attn_out.contiguous(), msa[2].contiguous(), w.mlp)
+    (c_qkv, c_mlp), msa = ada_fp8_layernorm(x, temb, w.norm, 3, (w.to_qkv.input_scale, w.mlp.proj_mlp.input_scale), panels=True)
+    attn_out = attention(_linear_from_panels(w.to_qkv, c_qkv, x.shape[0], x.dtype))
+    return flux_single_mlp_fp8(x, c_mlp, attn_out.contiguous(), msa[2].contiguous(), w.mlp, norm_in_panels=True)
 
 
 def flux_double_block_fp8(x: torch.Tensor, context: torch.Tensor, temb: torch.Tensor, w: FluxDoubleBlockFP8Weights, attention):
     """FluxTransformerFP8Block<T>::forward (FluxTransformerFP8Block.cc:159-262) with FluxAttentionFP8Processor
     (FluxAttentionFP8Processor.cc:165-360).  attention(qkv [B, S, 3D], context_qkv [B, Sc, 3D]) -> (attn [B, S, D],
     context_attn [B, Sc, D]).  Returns (output, context_output)."""
-    c, msa = ada_fp8_layernorm(x, temb, w.norm1, 6, (w.to_qkv.input_scale,))
-    cc, cmsa = ada_fp8_layernorm(context, temb, w.norm1_context, 6, (w.to_added_qkv.input_scale,))
-    attn, cattn = attention(_linear_from_codes(w.to_qkv, c, x.dtype), _linear_from_codes(w.to_added_qkv, cc, x.dtype))
+    c, msa = ada_fp8_layernorm(x, temb, w.norm1, 6, (w.to_qkv.input_scale,), panels=True)
+    cc, cmsa = ada_fp8_layernorm(context, temb, w.norm1_context, 6, (w.to_added_qkv.input_scale,), panels=True)
+    attn, cattn = attention(_linear_from_panels(w.to_qkv, c, x.shape[0], x.dtype),
+                            _linear_from_panels(w.to_added_qkv, cc, context.shape[0], x.dtype))
     a_out = w.to_out.forward(attn.contiguous())
     c_out = w.to_add_out.forward(cattn.contiguous())
     return flux_attn_post_fp8(x, a_out, msa, w.ff), flux_attn_post_fp8(context, c_out, cmsa, w.ff_context)
