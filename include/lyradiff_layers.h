@@ -682,19 +682,22 @@ public:
         const T* scale_mlp = msa + 4 * batch_size * d;
         const T* gate_mlp = msa + 5 * batch_size * d;
         const lq_dtype_t dt = detail::DType<T>::value;
-        detail::check(lq_gate_residual_layernorm_mod_fp8(reinterpret_cast<uint8_t*>(fp8_buffer), hidden_buffer, attn_tensor.getPtr<T>(),
-                                                         gate_msa, input_tensor.getPtr<T>(), scale_mlp, shift_mlp, dt,
-                                                         weights->gelu_proj_input_scale, batch_size, seq_len, d, 1e-6f, stream_),
+        // the two FP8 activations (fp8_buffer [D/64][M][64], fp8_buffer2 [4D/64][M][64]) are k-panels: same bytes, whole
+        // cache lines for the GEMMs' transfers (lyraquant.h)
+        detail::check(lq_gate_residual_layernorm_mod_fp8_panels(reinterpret_cast<uint8_t*>(fp8_buffer), hidden_buffer, attn_tensor.getPtr<T>(),
+                                                                gate_msa, input_tensor.getPtr<T>(), scale_mlp, shift_mlp, dt,
+                                                                weights->gelu_proj_input_scale, batch_size, seq_len, d, 1e-6f, stream_),
                       "FluxAttnPostFP8Processor norm");
-        detail::check(lq_gemm_fp8_codes(reinterpret_cast<uint8_t*>(fp8_buffer2), 4 * d, weights->ff_linear_input_scale, dt,
-                                        reinterpret_cast<const uint8_t*>(fp8_buffer), reinterpret_cast<const uint8_t*>(weights->gelu_proj_weight),
-                                        weights->gelu_proj_input_scale, weights->gelu_proj_weight_scale, weights->gelu_proj_bias,
-                                        /*gelu=*/1, (int)m, (int)(4 * d), (int)d, stream_),
+        detail::check(lq_gemm_fp8_codes_panels(reinterpret_cast<uint8_t*>(fp8_buffer2), weights->ff_linear_input_scale, dt,
+                                               reinterpret_cast<const uint8_t*>(fp8_buffer),
+                                               reinterpret_cast<const uint8_t*>(weights->gelu_proj_weight), weights->gelu_proj_input_scale,
+                                               weights->gelu_proj_weight_scale, weights->gelu_proj_bias,
+                                               /*gelu=*/1, (int)m, (int)(4 * d), (int)d, stream_),
                       "FluxAttnPostFP8Processor gelu_proj");
-        detail::check(lq_gemm_fp8_gated(output_tensor.getPtr<T>(), dt, reinterpret_cast<const uint8_t*>(fp8_buffer2),
-                                        reinterpret_cast<const uint8_t*>(weights->ff_linear_weight), weights->ff_linear_input_scale,
-                                        weights->ff_linear_weight_scale, weights->ff_linear_bias, gate_mlp, seq_len, hidden_buffer,
-                                        (int)m, (int)d, (int)(4 * d), stream_),
+        detail::check(lq_gemm_fp8_gated_panels(output_tensor.getPtr<T>(), dt, reinterpret_cast<const uint8_t*>(fp8_buffer2),
+                                               reinterpret_cast<const uint8_t*>(weights->ff_linear_weight), weights->ff_linear_input_scale,
+                                               weights->ff_linear_weight_scale, weights->ff_linear_bias, gate_mlp, seq_len, hidden_buffer,
+                                               (int)m, (int)d, (int)(4 * d), stream_),
                       "FluxAttnPostFP8Processor ff_linear");
         if (is_free_buffer_after_forward_) freeBuffer();
     }
@@ -813,17 +816,20 @@ public:
         fp8_buffer2 = static_cast<fp8_e4m3_t*>(allocator_->reMallocWithName("fp8_input_buffer2", m * d, false));
         const lq_dtype_t dt = detail::DType<T>::value;
         uint8_t* cat = reinterpret_cast<uint8_t*>(fp8_buffer1);
-        detail::check(lq_fp8_scale_cast(reinterpret_cast<uint8_t*>(fp8_buffer2), norm_tensor.getPtr<T>(), dt, weights->proj_mlp_input_scale, 1,
-                                        m * d, stream_), "FluxSingleTransformerFP8Mlp cast");
-        detail::check(lq_fp8_scale_cast_2d(cat, d + f, attn_tensor.getPtr<T>(), d, dt, weights->proj_out_input_scale, 1, m, d, stream_),
+        // FP8 activations as k-panels (lyraquant.h): fp8_buffer2 [D/64][M][64]; proj_out's concatenated input `cat`
+        // [(D + F)/64][M][64], whose two column blocks (attention output, GELU of proj_mlp) are runs of whole panels
+        detail::check(lq_fp8_scale_cast_panels(reinterpret_cast<uint8_t*>(fp8_buffer2), norm_tensor.getPtr<T>(), dt, weights->proj_mlp_input_scale,
+                                               1, m, d, stream_), "FluxSingleTransformerFP8Mlp cast");
+        detail::check(lq_fp8_scale_cast_panels(cat, attn_tensor.getPtr<T>(), dt, weights->proj_out_input_scale, 1, m, d, stream_),
                       "FluxSingleTransformerFP8Mlp attn cast");
-        detail::check(lq_gemm_fp8_codes(cat + d, d + f, weights->proj_out_input_scale, dt, reinterpret_cast<const uint8_t*>(fp8_buffer2),
-                                        reinterpret_cast<const uint8_t*>(weights->proj_mlp_weight), weights->proj_mlp_input_scale,
-                                        weights->proj_mlp_weight_scale, weights->proj_mlp_bias, /*gelu=*/2, (int)m, (int)f, (int)d, stream_),
+        detail::check(lq_gemm_fp8_codes_panels(cat + (d / 64) * m * 64, weights->proj_out_input_scale, dt,
+                                               reinterpret_cast<const uint8_t*>(fp8_buffer2),
+                                               reinterpret_cast<const uint8_t*>(weights->proj_mlp_weight), weights->proj_mlp_input_scale,
+                                               weights->proj_mlp_weight_scale, weights->proj_mlp_bias, /*gelu=*/2, (int)m, (int)f, (int)d, stream_),
                       "FluxSingleTransformerFP8Mlp proj_mlp");
-        detail::check(lq_gemm_fp8_gated(output_tensor.getPtr<T>(), dt, cat, reinterpret_cast<const uint8_t*>(weights->proj_out_weight),
-                                        weights->proj_out_input_scale, weights->proj_out_weight_scale, weights->proj_out_bias,
-                                        gate_tensor.getPtr<T>(), seq_len, input_tensor.getPtr<T>(), (int)m, (int)d, (int)(d + f), stream_),
+        detail::check(lq_gemm_fp8_gated_panels(output_tensor.getPtr<T>(), dt, cat, reinterpret_cast<const uint8_t*>(weights->proj_out_weight),
+                                               weights->proj_out_input_scale, weights->proj_out_weight_scale, weights->proj_out_bias,
+                                               gate_tensor.getPtr<T>(), seq_len, input_tensor.getPtr<T>(), (int)m, (int)d, (int)(d + f), stream_),
                       "FluxSingleTransformerFP8Mlp proj_out");
         (void)is_free_buffer_after_forward_;
     }

@@ -133,20 +133,32 @@ struct FP8Linear {
     }
     void clear_lora() { requantise(master_h.to(at::kCUDA)); }
 
-    at::Tensor cast_input(const at::Tensor& x2) const {  // e4m3 codes of x with the calibrated static scale
-        at::Tensor q = at::empty(x2.sizes(), on_gpu(at::kByte));
-        ok(lq_fp8_scale_cast(P8(q), P(x2), lq_dt(x2.scalar_type()), PF(in_scale), 1, (size_t)x2.numel(), cur_stream()),
-           "lq_fp8_scale_cast");
+    // FP8 activations inside this file travel as k-panels [K/64][M][64] (lyraquant.h): the quantising kernels write them,
+    // the GEMMs fetch them in whole cache lines; codes and outputs are those of the row-major calls.
+    at::Tensor cast_input(const at::Tensor& x2) const {  // e4m3 codes of x [M, K] with the calibrated static scale, as k-panels
+        at::Tensor q = at::empty({x2.size(1) / 64, x2.size(0), 64}, on_gpu(at::kByte));
+        ok(lq_fp8_scale_cast_panels(P8(q), P(x2), lq_dt(x2.scalar_type()), PF(in_scale), 1, (size_t)x2.size(0), (size_t)x2.size(1),
+                                    cur_stream()),
+           "lq_fp8_scale_cast_panels");
         return q;
     }
-    at::Tensor from_codes(const at::Tensor& q, int64_t m, at::ScalarType T) const {
+    at::Tensor from_panels(const at::Tensor& q, int64_t m, at::ScalarType T) const {
         at::Tensor y = at::empty({m, n}, on_gpu(T));
-        ok(lq_gemm_fp8(P(y), lq_dt(T), P8(q), P8(w_rows32), PF(in_scale), PF(w_scale), P(bias), 0, nullptr, 0.0f, (int)m, (int)n,
-                       (int)k, cur_stream()),
-           "lq_gemm_fp8");
+        ok(lq_gemm_fp8_panels(P(y), lq_dt(T), P8(q), P8(w_rows32), PF(in_scale), PF(w_scale), P(bias), (int)m, (int)n, (int)k, nullptr,
+                              cur_stream()),
+           "lq_gemm_fp8_panels");
         return y;
     }
-    // `gate` [B, n] and `residual` [m, n]:  T(T(T(y) * gate) + residual) in the epilogue
+    at::Tensor from_panels_gated(const at::Tensor& q, int64_t m, const at::Tensor& gate, int64_t rows_per_gate,
+                                 const at::Tensor& residual) const {
+        at::Tensor y = at::empty({m, n}, residual.options());
+        ok(lq_gemm_fp8_gated_panels(P(y), lq_dt(residual.scalar_type()), P8(q), P8(w_rows32), PF(in_scale), PF(w_scale), P(bias), P(gate),
+                                    (size_t)rows_per_gate, P(residual), (int)m, (int)n, (int)k, cur_stream()),
+           "lq_gemm_fp8_gated_panels");
+        return y;
+    }
+    // `gate` [B, n] and `residual` [m, n]:  T(T(T(y) * gate) + residual) in the epilogue; row-major codes (written by the W4A4
+    // GEMM's epilogue in the INT4 blocks)
     at::Tensor from_codes_gated(const at::Tensor& q, int64_t m, const at::Tensor& gate, int64_t rows_per_gate,
                                 const at::Tensor& residual) const {
         at::Tensor y = at::empty({m, n}, residual.options());
@@ -206,17 +218,17 @@ struct AdaLinear {
     // msa [chunks, B, D] from the (already SiLU'd) time embedding [B, D]  (AdaFP8LayerNorm.cc:100-175, invokeTranspose102)
     at::Tensor msa(const at::Tensor& temb, int64_t chunks) const {
         const int64_t b = temb.size(0), d = temb.size(1);
-        at::Tensor flat = fp8 ? q.from_codes(q.cast_input(temb), b, temb.scalar_type()) : at::linear(temb, weight, bias);
+        at::Tensor flat = fp8 ? q.from_panels(q.cast_input(temb), b, temb.scalar_type()) : at::linear(temb, weight, bias);
         return b > 1 ? flat.view({b, chunks, d}).transpose(0, 1).contiguous() : flat.view({chunks, 1, d});
     }
 };
 
 // (1 + msa[1]) * LayerNorm(x) + msa[0] with the FP8 cast(s) of the consumers fused; x [B, S, D]
-at::Tensor adaln_codes(const at::Tensor& x, const at::Tensor& msa, const at::Tensor& in_scale) {
-    at::Tensor c = at::empty(x.sizes(), on_gpu(at::kByte));
-    ok(lq_layernorm_mod_fp8(P8(c), P(x), P(msa[1]), P(msa[0]), lq_dt(x.scalar_type()), PF(in_scale), (size_t)x.size(0),
-                            (size_t)x.size(1), (size_t)x.size(2), 1e-6f, cur_stream()),
-       "lq_layernorm_mod_fp8");
+at::Tensor adaln_codes(const at::Tensor& x, const at::Tensor& msa, const at::Tensor& in_scale) {  // k-panels [D/64, B*S, 64]
+    at::Tensor c = at::empty({x.size(2) / 64, x.size(0) * x.size(1), 64}, on_gpu(at::kByte));
+    ok(lq_layernorm_mod_fp8_panels(P8(c), P(x), P(msa[1]), P(msa[0]), lq_dt(x.scalar_type()), PF(in_scale), (size_t)x.size(0),
+                                   (size_t)x.size(1), (size_t)x.size(2), 1e-6f, cur_stream()),
+       "lq_layernorm_mod_fp8_panels");
     return c;
 }
 at::Tensor adaln_16(const at::Tensor& x, const at::Tensor& msa) {
@@ -255,15 +267,15 @@ struct AttnPostFP8 {
     at::Tensor forward(const at::Tensor& x, const at::Tensor& attn, const at::Tensor& msa) const {
         const int64_t b = x.size(0), s = x.size(1), d = x.size(2), m = b * s;
         const lq_dtype_t dt = lq_dt(x.scalar_type());
-        at::Tensor q1 = at::empty(x.sizes(), on_gpu(at::kByte)), hidden = at::empty_like(x);
-        ok(lq_gate_residual_layernorm_mod_fp8(P8(q1), P(hidden), P(attn), P(msa[2]), P(x), P(msa[4]), P(msa[3]), dt, PF(gelu_proj.in_scale),
-                                              (size_t)b, (size_t)s, (size_t)d, 1e-6f, cur_stream()),
-           "lq_gate_residual_layernorm_mod_fp8");
-        at::Tensor q2 = at::empty({m, 4 * d}, on_gpu(at::kByte));
-        ok(lq_gemm_fp8_codes(P8(q2), (size_t)(4 * d), PF(ff_linear.in_scale), dt, P8(q1), P8(gelu_proj.w_rows32), PF(gelu_proj.in_scale),
-                             PF(gelu_proj.w_scale), P(gelu_proj.bias), 1, (int)m, (int)(4 * d), (int)d, cur_stream()),
-           "lq_gemm_fp8_codes");
-        return ff_linear.from_codes_gated(q2, m, msa[5], s, hidden).view({b, s, d});
+        at::Tensor q1 = at::empty({d / 64, m, 64}, on_gpu(at::kByte)), hidden = at::empty_like(x);
+        ok(lq_gate_residual_layernorm_mod_fp8_panels(P8(q1), P(hidden), P(attn), P(msa[2]), P(x), P(msa[4]), P(msa[3]), dt,
+                                                     PF(gelu_proj.in_scale), (size_t)b, (size_t)s, (size_t)d, 1e-6f, cur_stream()),
+           "lq_gate_residual_layernorm_mod_fp8_panels");
+        at::Tensor q2 = at::empty({4 * d / 64, m, 64}, on_gpu(at::kByte));
+        ok(lq_gemm_fp8_codes_panels(P8(q2), PF(ff_linear.in_scale), dt, P8(q1), P8(gelu_proj.w_rows32), PF(gelu_proj.in_scale),
+                                    PF(gelu_proj.w_scale), P(gelu_proj.bias), 1, (int)m, (int)(4 * d), (int)d, cur_stream()),
+           "lq_gemm_fp8_codes_panels");
+        return ff_linear.from_panels_gated(q2, m, msa[5], s, hidden).view({b, s, d});
     }
 };
 
@@ -417,8 +429,8 @@ struct FluxTransformerBlockOp : th::CustomClassHolder {
             qkv = to_qkv4.run(adaln_16(x, msa).view({b * s, d}), nullptr, true).view({b, s, 3 * d});
             cqkv = to_added_qkv4.run(adaln_16(c, cmsa).view({b * sc, d}), nullptr, true).view({b, sc, 3 * d});
         } else {
-            qkv = to_qkv.from_codes(adaln_codes(x, msa, to_qkv.in_scale), b * s, cfg.T).view({b, s, 3 * d});
-            cqkv = to_added_qkv.from_codes(adaln_codes(c, cmsa, to_added_qkv.in_scale), b * sc, cfg.T).view({b, sc, 3 * d});
+            qkv = to_qkv.from_panels(adaln_codes(x, msa, to_qkv.in_scale), b * s, cfg.T).view({b, s, 3 * d});
+            cqkv = to_added_qkv.from_panels(adaln_codes(c, cmsa, to_added_qkv.in_scale), b * sc, cfg.T).view({b, sc, 3 * d});
         }
         at::Tensor o = attention_core(qkv, cqkv, norm_qk, norm_added_qk, rope_emb, cfg.heads);
         at::Tensor attn = o.slice(1, sc, sc + s).contiguous().view({b * s, d}), cattn = o.slice(1, 0, sc).contiguous().view({b * sc, d});
@@ -426,8 +438,8 @@ struct FluxTransformerBlockOp : th::CustomClassHolder {
             at::Tensor a_out = to_out4.run(attn, nullptr, true).view({b, s, d}), c_out = to_add_out4.run(cattn, nullptr, true).view({b, sc, d});
             return {ff4.forward(x, a_out, msa), ff_context4.forward(c, c_out, cmsa)};
         }
-        at::Tensor a_out = to_out.from_codes(to_out.cast_input(attn), b * s, cfg.T).view({b, s, d});
-        at::Tensor c_out = to_add_out.from_codes(to_add_out.cast_input(cattn), b * sc, cfg.T).view({b, sc, d});
+        at::Tensor a_out = to_out.from_panels(to_out.cast_input(attn), b * s, cfg.T).view({b, s, d});
+        at::Tensor c_out = to_add_out.from_panels(to_add_out.cast_input(cattn), b * sc, cfg.T).view({b, sc, d});
         return {ff.forward(x, a_out, msa), ff_context.forward(c, c_out, cmsa)};
     }
 };
@@ -516,21 +528,22 @@ struct FluxSingleTransformerBlockOp : th::CustomClassHolder {
             return proj_out_2.run(mlp, &tail, true).view({b, s, d});
         }
         // one adaLN read yields the codes for to_qkv and for proj_mlp
-        at::Tensor c_qkv = at::empty(x.sizes(), on_gpu(at::kByte)), c_mlp = at::empty(x.sizes(), on_gpu(at::kByte));
-        ok(lq_layernorm_mod_fp8_dual(P8(c_qkv), PF(to_qkv.in_scale), P8(c_mlp), PF(proj_mlp.in_scale), P(x), P(msa[1]), P(msa[0]), dt,
-                                     (size_t)b, (size_t)s, (size_t)d, 1e-6f, cur_stream()),
-           "lq_layernorm_mod_fp8_dual");
-        at::Tensor attn = attention_core(to_qkv.from_codes(c_qkv, m, cfg.T).view({b, s, 3 * d}), none, norm_qk, none, rope_emb, cfg.heads)
+        at::Tensor c_qkv = at::empty({d / 64, m, 64}, on_gpu(at::kByte)), c_mlp = at::empty({d / 64, m, 64}, on_gpu(at::kByte));
+        ok(lq_layernorm_mod_fp8_dual_panels(P8(c_qkv), PF(to_qkv.in_scale), P8(c_mlp), PF(proj_mlp.in_scale), P(x), P(msa[1]), P(msa[0]),
+                                            dt, (size_t)b, (size_t)s, (size_t)d, 1e-6f, cur_stream()),
+           "lq_layernorm_mod_fp8_dual_panels");
+        at::Tensor attn = attention_core(to_qkv.from_panels(c_qkv, m, cfg.T).view({b, s, 3 * d}), none, norm_qk, none, rope_emb, cfg.heads)
                               .contiguous();
-        // proj_out's input [attn | gelu(mlp)] as e4m3 codes: the attention columns by a strided cast, the mlp columns
-        // straight from the proj_mlp GEMM's epilogue (FluxSingleTransformerFP8Block.cc:216-253)
-        at::Tensor q2 = at::empty({m, d + f}, on_gpu(at::kByte));
-        ok(lq_fp8_scale_cast_2d(P8(q2), (size_t)(d + f), P(attn), (size_t)d, dt, PF(proj_out.in_scale), 1, (size_t)m, (size_t)d, cur_stream()),
-           "lq_fp8_scale_cast_2d");
-        ok(lq_gemm_fp8_codes(P8(q2) + d, (size_t)(d + f), PF(proj_out.in_scale), dt, P8(c_mlp), P8(proj_mlp.w_rows32), PF(proj_mlp.in_scale),
-                             PF(proj_mlp.w_scale), P(proj_mlp.bias), 2, (int)m, (int)f, (int)d, cur_stream()),
-           "lq_gemm_fp8_codes");
-        return proj_out.from_codes_gated(q2, m, gate, s, x.view({m, d})).view({b, s, d});
+        // proj_out's input [attn | gelu(mlp)] as e4m3 codes in k-panels [(D + F)/64, M, 64]: a block of columns is a run of whole
+        // panels, so the attention columns are a cast into the first D/64 panels and the mlp columns come straight from the
+        // proj_mlp GEMM's epilogue into the rest (FluxSingleTransformerFP8Block.cc:216-253)
+        at::Tensor q2 = at::empty({(d + f) / 64, m, 64}, on_gpu(at::kByte));
+        ok(lq_fp8_scale_cast_panels(P8(q2), P(attn), dt, PF(proj_out.in_scale), 1, (size_t)m, (size_t)d, cur_stream()),
+           "lq_fp8_scale_cast_panels");
+        ok(lq_gemm_fp8_codes_panels(P8(q2) + (size_t)(d / 64) * (size_t)m * 64, PF(proj_out.in_scale), dt, P8(c_mlp), P8(proj_mlp.w_rows32),
+                                    PF(proj_mlp.in_scale), PF(proj_mlp.w_scale), P(proj_mlp.bias), 2, (int)m, (int)f, (int)d, cur_stream()),
+           "lq_gemm_fp8_codes_panels");
+        return proj_out.from_panels_gated(q2, m, gate, s, x.view({m, d})).view({b, s, d});
     }
 };
 
