@@ -355,7 +355,7 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 __device__ __forceinline__ float gelu_fast(float x) {
     // 0.5 x (1 + tanh(u)) = x / (1 + exp(-2u)),  u = sqrt(2/pi) (x + 0.044715 x^3);  -2u log2(e) = x (A + B x^2)
     constexpr float A = -2.0f * 0.7978845608028654f * 1.4426950408889634f, B = A * 0.044715f;
-    const float t = x * (A + B * (x * x));
+    const float t = x * __builtin_fmaf(B, x * x, A);  // one rounding fewer than the separate multiply and add; the result is compared by tolerance
     const float e = __builtin_amdgcn_exp2f(t);             // exp(-2u): 0 for large x, inf for very negative x
     return x * __builtin_amdgcn_rcpf(1.0f + e);            // x, resp. -0
 }
